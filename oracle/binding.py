@@ -1,0 +1,274 @@
+"""ctypes binding to the C oracle (liboracle.so / liboracle_simd.so).
+
+TEST INFRASTRUCTURE ONLY -- see oracle/__init__.py.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+ORDER_HWY, ORDER_AVX2, ORDER_SCALAR, ORDER_DOTPROD = 0, 1, 2, 3
+ORDERS = {"hwy": 0, "avx2": 1, "scalar": 2, "dotprod": 3}
+SILU_EXACT, SILU_FAST, SILU_FAST_FMA = 0, 1, 2
+
+Q4K = 144
+Q8K = 292
+
+
+def build() -> None:
+    subprocess.run(["make", "-C", _HERE, "all"], check=True, capture_output=True)
+
+
+def _load(name: str) -> C.CDLL:
+    path = os.path.join(_HERE, name)
+    if not os.path.exists(path):
+        build()
+    return C.CDLL(path)
+
+
+_lib = None
+_simd = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        L = _load("liboracle.so")
+        L.orc_fp16_to_fp32.restype = C.c_float
+        L.orc_fp16_to_fp32.argtypes = [C.c_uint16]
+        L.orc_fp32_to_fp16.restype = C.c_uint16
+        L.orc_fp32_to_fp16.argtypes = [C.c_float]
+        L.orc_nearest_int.restype = C.c_int
+        L.orc_nearest_int.argtypes = [C.c_float]
+        L.orc_fast_exp.restype = C.c_float
+        L.orc_fast_exp.argtypes = [C.c_float]
+        L.orc_fast_exp_fma.restype = C.c_float
+        L.orc_fast_exp_fma.argtypes = [C.c_float]
+        L.orc_silu_mul.restype = C.c_float
+        L.orc_silu_mul.argtypes = [C.c_float, C.c_float, C.c_int]
+        L.orc_dot_q4k_q8k.restype = C.c_float
+        L.orc_dot_q4k_q8k.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+        L.orc_dot_dequant_f64.restype = C.c_double
+        L.orc_dot_dequant_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.orc_dot_magnitude_f64.restype = C.c_double
+        L.orc_dot_magnitude_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.orc_build_assignments.restype = C.c_int64
+        _lib = L
+    return _lib
+
+
+def simd() -> C.CDLL:
+    global _simd
+    if _simd is None:
+        _simd = _load("liboracle_simd.so")
+    return _simd
+
+
+def _p(a: np.ndarray) -> C.c_void_p:
+    return C.c_void_p(a.ctypes.data)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+# ---------------------------------------------------------------- scalars
+def fp16_to_fp32(h: int) -> float:
+    return lib().orc_fp16_to_fp32(h)
+
+
+def fp32_to_fp16(f: float) -> int:
+    return lib().orc_fp32_to_fp16(f)
+
+
+def nearest_int(v: float) -> int:
+    return lib().orc_nearest_int(v)
+
+
+def scales_kmask(packed12: np.ndarray):
+    p = _c(packed12, np.uint8)
+    s = np.zeros(8, np.uint8)
+    m = np.zeros(8, np.uint8)
+    lib().orc_q4k_scales_kmask(_p(p), _p(s), _p(m))
+    return s, m
+
+
+def scales_indexed(packed12: np.ndarray):
+    p = _c(packed12, np.uint8)
+    s = np.zeros(8, np.uint8)
+    m = np.zeros(8, np.uint8)
+    lib().orc_q4k_scales_indexed(_p(p), _p(s), _p(m))
+    return s, m
+
+
+# ---------------------------------------------------------------- quantizer
+def quantize_rows_q8k(x: np.ndarray) -> np.ndarray:
+    """fp32 [n, k] -> uint8 [n, k/256*292] (block_q8_K bytes)."""
+    x = _c(x, np.float32)
+    if x.ndim == 1:
+        x = x[None, :]
+    n, k = x.shape
+    out = np.zeros((n, k // 256 * Q8K), np.uint8)
+    rc = lib().orc_quantize_rows_q8k(_p(x), C.c_int64(n), C.c_int64(k), _p(out), C.c_int64(k))
+    if rc:
+        raise ValueError(f"orc_quantize_rows_q8k rc={rc}")
+    return out
+
+
+def split_q8k(q8: np.ndarray):
+    """uint8 [n, nb*292] -> (d [n,nb] f32, qs [n,nb,256] i8, bsums [n,nb,16] i16)."""
+    n = q8.shape[0]
+    b = q8.reshape(n, -1, Q8K)
+    d = b[:, :, 0:4].copy().view(np.float32).reshape(n, -1)
+    qs = b[:, :, 4:260].copy().view(np.int8)
+    bs = b[:, :, 260:292].copy().view(np.int16)
+    return d, qs, bs
+
+
+# ---------------------------------------------------------------- sums / dots
+def matrix_block_sums(w: np.ndarray, cols: int, q8: np.ndarray):
+    """w uint8 [rows, nb*144], q8 uint8 [n, nb*292] -> two int32 [rows, n, nb]."""
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    rows, n, nb = w.shape[0], q8.shape[0], cols // 256
+    ds = np.zeros((rows, n, nb), np.int32)
+    md = np.zeros((rows, n, nb), np.int32)
+    rc = lib().orc_matrix_block_sums(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+                                     C.c_int64(n), C.c_size_t(q8.shape[1]), _p(ds), _p(md))
+    if rc:
+        raise ValueError(f"orc_matrix_block_sums rc={rc}")
+    return ds, md
+
+
+def mul_mat_q4k_q8k(w: np.ndarray, cols: int, q8: np.ndarray, order: int = ORDER_DOTPROD) -> np.ndarray:
+    """-> fp32 [n, rows]"""
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    rows, n = w.shape[0], q8.shape[0]
+    out = np.zeros((n, rows), np.float32)
+    rc = lib().orc_mul_mat_q4k_q8k(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+                                   C.c_int64(n), C.c_size_t(q8.shape[1]), _p(out), C.c_int64(rows), C.c_int(order))
+    if rc:
+        raise ValueError(f"orc_mul_mat_q4k_q8k rc={rc}")
+    return out
+
+
+def mul_mat_q4k_f32(w: np.ndarray, cols: int, x: np.ndarray, order: int = ORDER_DOTPROD) -> np.ndarray:
+    return mul_mat_q4k_q8k(w, cols, quantize_rows_q8k(x), order)
+
+
+def dot_dequant_f64(w: np.ndarray, cols: int, q8: np.ndarray) -> np.ndarray:
+    """double-precision dequantize-then-dot, [n, rows]."""
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    L = lib()
+    out = np.zeros((q8.shape[0], w.shape[0]), np.float64)
+    for m in range(q8.shape[0]):
+        for r in range(w.shape[0]):
+            out[m, r] = L.orc_dot_dequant_f64(C.c_void_p(w[r].ctypes.data), C.c_void_p(q8[m].ctypes.data),
+                                              C.c_int64(cols))
+    return out
+
+
+def dot_magnitude_f64(w: np.ndarray, cols: int, q8: np.ndarray) -> np.ndarray:
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    L = lib()
+    out = np.zeros((q8.shape[0], w.shape[0]), np.float64)
+    for m in range(q8.shape[0]):
+        for r in range(w.shape[0]):
+            out[m, r] = L.orc_dot_magnitude_f64(C.c_void_p(w[r].ctypes.data), C.c_void_p(q8[m].ctypes.data),
+                                                C.c_int64(cols))
+    return out
+
+
+# ---------------------------------------------------------------- FFN / router / MoE
+def ffn_swiglu(gate, up, down, hidden: int, inter: int, x, order=ORDER_DOTPROD, silu=SILU_FAST_FMA,
+               want_inter=False):
+    gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+    x = _c(x, np.float32)
+    n = x.shape[0]
+    y = np.zeros((n, hidden), np.float32)
+    mid = np.zeros((n, inter), np.float32)
+    rc = lib().orc_ffn_swiglu_q4k(_p(gate), _p(up), _p(down), C.c_int64(hidden), C.c_int64(inter), _p(x),
+                                  C.c_int64(n), _p(y), C.c_int(order), C.c_int(silu), _p(mid))
+    if rc:
+        raise ValueError(f"orc_ffn_swiglu_q4k rc={rc}")
+    return (y, mid) if want_inter else y
+
+
+def route_topk(logits, top_k: int, weights_mode: int = 0):
+    logits = _c(logits, np.float32)
+    n, e = logits.shape
+    ids = np.zeros((n, top_k), np.int32)
+    w = np.zeros((n, top_k), np.float32)
+    rc = lib().orc_route_topk(_p(logits), C.c_int64(e), C.c_int64(n), C.c_int(top_k), C.c_int(weights_mode), _p(ids),
+                              _p(w))
+    if rc:
+        raise ValueError(f"orc_route_topk rc={rc}")
+    return ids, w
+
+
+def build_assignments(ids, n_experts: int) -> np.ndarray:
+    ids = _c(ids, np.int32)
+    n, k = ids.shape
+    out = np.zeros((n * k, 3), np.int32)
+    cnt = lib().orc_build_assignments(_p(ids), C.c_int64(n), C.c_int(k), C.c_int64(n_experts), _p(out))
+    return out[:cnt]
+
+
+class _MoEWeights(C.Structure):
+    _fields_ = [("hidden", C.c_int64), ("inter", C.c_int64), ("n_experts", C.c_int64), ("top_k", C.c_int),
+                ("gate_exps", C.c_void_p), ("up_exps", C.c_void_p), ("down_exps", C.c_void_p),
+                ("sh_gate", C.c_void_p), ("sh_up", C.c_void_p), ("sh_down", C.c_void_p),
+                ("sh_gate_inp", C.c_void_p)]
+
+
+def moe_layer(gate_exps, up_exps, down_exps, hidden, inter, top_k, x, logits, shared=None, order=ORDER_DOTPROD,
+              silu=SILU_EXACT, weights_mode=0, accumulate_mode=0):
+    """gate_exps/up_exps: uint8 [E, inter, hidden/256*144]; down_exps: uint8 [E, hidden, inter/256*144].
+    shared: None or (gate, up, down, gate_inp[hidden] or None).
+    Returns dict(y, ids, weights, hidden)."""
+    ge, ue, de = _c(gate_exps, np.uint8), _c(up_exps, np.uint8), _c(down_exps, np.uint8)
+    x = _c(x, np.float32)
+    logits = _c(logits, np.float32)
+    n = x.shape[0]
+    keep = [ge, ue, de, x, logits]
+    W = _MoEWeights(hidden, inter, ge.shape[0], top_k, ge.ctypes.data, ue.ctypes.data, de.ctypes.data, None, None,
+                    None, None)
+    if shared is not None:
+        sg, su, sd = (_c(a, np.uint8) for a in shared[:3])
+        keep += [sg, su, sd]
+        W.sh_gate, W.sh_up, W.sh_down = sg.ctypes.data, su.ctypes.data, sd.ctypes.data
+        if shared[3] is not None:
+            gi = _c(shared[3], np.float32)
+            keep.append(gi)
+            W.sh_gate_inp = gi.ctypes.data
+    y = np.zeros((n, hidden), np.float32)
+    ids = np.zeros((n, top_k), np.int32)
+    wts = np.zeros((n, top_k), np.float32)
+    hid = np.zeros((n, top_k, inter), np.float32)
+    rc = lib().orc_moe_layer(C.byref(W), _p(x), _p(logits), C.c_int64(n), _p(y), C.c_int(order), C.c_int(silu),
+                             C.c_int(weights_mode), C.c_int(accumulate_mode), _p(ids), _p(wts), _p(hid))
+    if rc:
+        raise ValueError(f"orc_moe_layer rc={rc}")
+    return {"y": y, "ids": ids, "weights": wts, "hidden": hid}
+
+
+# ---------------------------------------------------------------- timed SIMD baseline
+def simd_mul_mat_q4k_q8k(w, cols: int, q8, threads: int) -> np.ndarray:
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    rows, n = w.shape[0], q8.shape[0]
+    out = np.zeros((n, rows), np.float32)
+    rc = simd().orc_simd_mul_mat_q4k_q8k(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+                                         C.c_int64(n), C.c_size_t(q8.shape[1]), _p(out), C.c_int64(rows),
+                                         C.c_int(threads))
+    if rc:
+        raise ValueError(f"orc_simd_mul_mat_q4k_q8k rc={rc}")
+    return out
