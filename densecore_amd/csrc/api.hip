@@ -1,0 +1,637 @@
+// C ABI of libmi355q4k.so (declared in include/mi355_q4k.h): argument checks, weight handles,
+// a grow-only device workspace and the sequencing of kernel launches.  No arithmetic lives here.
+#include "../../include/mi355_q4k.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "common.h"
+#include "kernels.h"
+
+using namespace mq;
+
+struct mq_weight {
+    uint8_t* data = nullptr;     // tiled layout, experts back to back
+    int64_t rows = 0, cols = 0, n_experts = 0;
+    int64_t nb = 0, rowtiles = 0;
+    size_t expert_bytes = 0;     // tiled bytes per expert
+    size_t total_bytes = 0;
+};
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(MQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define MQ_HIP(call)                                     \
+    do {                                                 \
+        hipError_t e_ = (call);                          \
+        if (e_ != hipSuccess) return hip_fail(e_, #call); \
+    } while (0)
+
+// A device buffer that only grows.  Growing frees the old allocation, which synchronises the
+// device, so kernels already queued on any stream have finished with it.
+struct Buffer {
+    void* ptr = nullptr;
+    size_t cap = 0;
+    hipError_t reserve(size_t bytes) {
+        if (bytes <= cap) return hipSuccess;
+        if (ptr) {
+            hipError_t e = hipFree(ptr);
+            ptr = nullptr;
+            cap = 0;
+            if (e != hipSuccess) return e;
+        }
+        const size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        hipError_t e = hipMalloc(&ptr, want);
+        if (e == hipSuccess) cap = want;
+        return e;
+    }
+    void release() {
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+    }
+};
+
+struct State {
+    bool ready = false;
+    int device = -1;
+    std::mutex mu;
+    Buffer aq, ad;        // A-major activations of the op input
+    Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
+    Buffer aq2, ad2;      // A-major activations of the intermediate
+    Buffer part;          // MoE per-(token,k) down results
+    Buffer route;         // ids / weights / groups / entries
+    Buffer stage_in, stage_out;  // host-pointer entry points
+} g;
+
+int check_ready() {
+    if (!g.ready) return fail(MQ_ERR_STATE, "mq_init has not been called (or no GPU is present)");
+    return MQ_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_weight(const mq_weight* w, const char* name) {
+    if (!w || !w->data) return fail(MQ_ERR_INVALID, "%s: null weight handle", name);
+    return MQ_OK;
+}
+
+int check_x(const float* x, int64_t n, int64_t ldx, int64_t cols, const char* name) {
+    if (!x) return fail(MQ_ERR_INVALID, "%s: null activation pointer", name);
+    if (n < 0) return fail(MQ_ERR_INVALID, "%s: negative row count", name);
+    if (ldx < cols) return fail(MQ_ERR_INVALID, "%s: ldx %lld < cols %lld", name, (long long)ldx, (long long)cols);
+    if (!aligned16(x) || (ldx & 3)) return fail(MQ_ERR_INVALID, "%s: activations must be 16-byte aligned with ldx %% 4 == 0", name);
+    return MQ_OK;
+}
+
+// Quantize x into the A-major workspace pair (aq, ad).
+int quantize_into(Buffer& aq, Buffer& ad, const float* x, int64_t n, int64_t ldx, int64_t cols, hipStream_t s) {
+    const int64_t nb = cols / kQK;
+    MQ_HIP(aq.reserve(aq_bytes(n, nb)));
+    MQ_HIP(ad.reserve(ad_count(n, nb) * sizeof(float)));
+    MQ_HIP(launch_quantize_q8k(x, n, ldx, cols, nullptr, 0, (uint8_t*)aq.ptr, (float*)ad.ptr, s));
+    return MQ_OK;
+}
+
+int alloc_weight(int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
+    if (!out) return fail(MQ_ERR_INVALID, "null output handle");
+    *out = nullptr;
+    if (rows <= 0 || cols <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "rows, cols and n_experts must be positive");
+    if (cols % kQK) return fail(MQ_ERR_INVALID, "cols %lld is not a multiple of 256", (long long)cols);
+    mq_weight* w = new mq_weight;
+    w->rows = rows;
+    w->cols = cols;
+    w->n_experts = n_experts;
+    w->nb = cols / kQK;
+    w->rowtiles = (rows + 15) / 16;
+    w->expert_bytes = (size_t)w->rowtiles * (size_t)w->nb * kTileBytes;
+    w->total_bytes = w->expert_bytes * (size_t)n_experts;
+    hipError_t e = hipMalloc((void**)&w->data, w->total_bytes);
+    if (e != hipSuccess) {
+        delete w;
+        return hip_fail(e, "hipMalloc(weights)");
+    }
+    if (rows % 16) {  // padding rows of the last tile must read as zero blocks
+        e = hipMemset(w->data, 0, w->total_bytes);
+        if (e != hipSuccess) {
+            (void)hipFree(w->data);
+            delete w;
+            return hip_fail(e, "hipMemset(weights)");
+        }
+    }
+    *out = w;
+    return MQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mq_last_error(void) { return g_error.c_str(); }
+
+int mq_init(int device) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) return fail(MQ_ERR_STATE, "no HIP device available (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= count) return fail(MQ_ERR_INVALID, "device %d out of range [0, %d)", device, count);
+    MQ_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    MQ_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(MQ_ERR_UNSUPPORTED, "built for gfx950, device is %s", prop.gcnArchName);
+    g.device = device;
+    g.ready = true;
+    return MQ_OK;
+}
+
+int mq_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (!g.ready) return MQ_OK;
+    (void)hipDeviceSynchronize();
+    for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    g.ready = false;
+    return MQ_OK;
+}
+
+int mq_device_info(char* name_out, size_t name_cap, int* cu_count, size_t* hbm_bytes) {
+    if (int rc = check_ready()) return rc;
+    hipDeviceProp_t prop;
+    MQ_HIP(hipGetDeviceProperties(&prop, g.device));
+    if (name_out && name_cap) snprintf(name_out, name_cap, "%s (%s)", prop.name, prop.gcnArchName);
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- weights
+int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts, size_t row_bytes,
+                     size_t expert_bytes, mq_weight** out) {
+    if (int rc = check_ready()) return rc;
+    if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_upload: null host pointer");
+    if (cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_weight_upload: cols %lld is not a positive multiple of 256", (long long)cols);
+    const size_t min_row = (size_t)(cols / kQK) * kQ4Block;
+    if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_upload: row_bytes %zu < %zu or odd", row_bytes, min_row);
+    if (n_experts > 1 && expert_bytes < row_bytes * (size_t)rows) return fail(MQ_ERR_INVALID, "mq_weight_upload: expert_bytes too small");
+    mq_weight* w = nullptr;
+    if (int rc = alloc_weight(rows, cols, n_experts, &w)) return rc;
+    const size_t raw_total = n_experts > 1 ? expert_bytes * (size_t)(n_experts - 1) + row_bytes * (size_t)rows
+                                           : row_bytes * (size_t)(rows - 1) + min_row;
+    void* raw = nullptr;
+    hipError_t e = hipMalloc(&raw, raw_total);
+    if (e == hipSuccess) e = hipMemcpy(raw, q4k_host, raw_total, hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+        e = launch_tile_weights((const uint8_t*)raw, rows, w->nb, row_bytes, expert_bytes, n_experts, w->data,
+                                w->expert_bytes, nullptr);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (raw) (void)hipFree(raw);
+    if (e != hipSuccess) {
+        mq_weight_free(w);
+        return hip_fail(e, "mq_weight_upload");
+    }
+    *out = w;
+    return MQ_OK;
+}
+
+int mq_weight_synthetic(uint64_t seed, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
+    if (int rc = check_ready()) return rc;
+    mq_weight* w = nullptr;
+    if (int rc = alloc_weight(rows, cols, n_experts, &w)) return rc;
+    hipError_t e = launch_synth_weights(seed, rows, w->nb, n_experts, w->data, w->expert_bytes, nullptr);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        mq_weight_free(w);
+        return hip_fail(e, "mq_weight_synthetic");
+    }
+    *out = w;
+    return MQ_OK;
+}
+
+int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, size_t expert_bytes) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_weight_download")) return rc;
+    if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_download: null host pointer");
+    const size_t min_row = (size_t)w->nb * kQ4Block;
+    if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_download: bad row_bytes");
+    if (w->n_experts > 1 && expert_bytes < row_bytes * (size_t)w->rows) return fail(MQ_ERR_INVALID, "mq_weight_download: bad expert_bytes");
+    const size_t raw_total = w->n_experts > 1 ? expert_bytes * (size_t)(w->n_experts - 1) + row_bytes * (size_t)w->rows
+                                              : row_bytes * (size_t)(w->rows - 1) + min_row;
+    void* raw = nullptr;
+    hipError_t e = hipMalloc(&raw, raw_total);
+    if (e == hipSuccess) e = hipMemcpy(raw, q4k_host, raw_total, hipMemcpyHostToDevice);  // keep caller's padding bytes
+    if (e == hipSuccess)
+        e = launch_untile_weights(w->data, w->rows, w->nb, row_bytes, expert_bytes, w->n_experts, (uint8_t*)raw,
+                                  w->expert_bytes, nullptr);
+    if (e == hipSuccess) e = hipMemcpy(q4k_host, raw, raw_total, hipMemcpyDeviceToHost);
+    if (raw) (void)hipFree(raw);
+    if (e != hipSuccess) return hip_fail(e, "mq_weight_download");
+    return MQ_OK;
+}
+
+int mq_weight_shape(const mq_weight* w, int64_t* rows, int64_t* cols, int64_t* n_experts, size_t* device_bytes) {
+    if (int rc = check_weight(w, "mq_weight_shape")) return rc;
+    if (rows) *rows = w->rows;
+    if (cols) *cols = w->cols;
+    if (n_experts) *n_experts = w->n_experts;
+    if (device_bytes) *device_bytes = w->total_bytes;
+    return MQ_OK;
+}
+
+int mq_weight_free(mq_weight* w) {
+    if (!w) return MQ_OK;
+    if (w->data) (void)hipFree(w->data);
+    delete w;
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- quantizer
+int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void* q8_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (k <= 0 || k % kQK) return fail(MQ_ERR_INVALID, "mq_quantize_q8k: k %lld is not a positive multiple of 256", (long long)k);
+    if (int rc = check_x(x_dev, n, ldx, k, "mq_quantize_q8k")) return rc;
+    if (!q8_dev || (reinterpret_cast<uintptr_t>(q8_dev) & 3u)) return fail(MQ_ERR_INVALID, "mq_quantize_q8k: output must be non-null and 4-byte aligned");
+    MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, k, q8_dev, (size_t)(k / kQK) * kQ8Block, nullptr, nullptr, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- dense matmul
+static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, int32_t* dbg_dot, int32_t* dbg_min,
+                          hipStream_t s) {
+    if (n == 0) return MQ_OK;
+    MatmulArgs a;
+    a.w0 = w->data;
+    a.rows = w->rows;
+    a.nb = w->nb;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ad = (const float*)g.ad.ptr;
+    a.n = n;
+    a.y = y;
+    a.ldy = ldy;
+    a.dbg_dot = dbg_dot;
+    a.dbg_min = dbg_min;
+    MQ_HIP(launch_matmul(a, s));
+    return MQ_OK;
+}
+
+int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                   void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: weight is an expert stack; use mq_mul_mat_id_q4k");
+    if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_mul_mat_q4k")) return rc;
+    if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
+    return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
+}
+
+int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t q8_row_bytes, float* y_dev,
+                       int64_t ldy, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k_q8k")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: weight is an expert stack");
+    if (!q8_dev || !y_dev || n < 0 || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: bad arguments");
+    if (q8_row_bytes < (size_t)w->nb * kQ8Block || (q8_row_bytes & 3) || (reinterpret_cast<uintptr_t>(q8_dev) & 3u))
+        return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: q8 rows too short or not 4-byte aligned");
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    MQ_HIP(g.aq.reserve(aq_bytes(n, w->nb)));
+    MQ_HIP(g.ad.reserve(ad_count(n, w->nb) * sizeof(float)));
+    MQ_HIP(launch_q8k_to_amajor(q8_dev, n, q8_row_bytes, w->cols, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
+    return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
+}
+
+int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int64_t ldx, float* y_host, int64_t ldy) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k_host")) return rc;
+    if (!x_host || !y_host || n < 0 || ldx < w->cols || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_host: bad arguments");
+    if (n == 0) return MQ_OK;
+    float* xin = nullptr;
+    float* yout = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g.mu);
+        MQ_HIP(g.stage_in.reserve((size_t)n * (size_t)w->cols * sizeof(float)));
+        MQ_HIP(g.stage_out.reserve((size_t)n * (size_t)w->rows * sizeof(float)));
+        xin = (float*)g.stage_in.ptr;
+        yout = (float*)g.stage_out.ptr;
+    }
+    MQ_HIP(hipMemcpy2D(xin, (size_t)w->cols * 4, x_host, (size_t)ldx * 4, (size_t)w->cols * 4, (size_t)n, hipMemcpyHostToDevice));
+    if (int rc = mq_mul_mat_q4k(w, xin, n, w->cols, yout, w->rows, nullptr)) return rc;
+    MQ_HIP(hipMemcpy2D(y_host, (size_t)ldy * 4, yout, (size_t)w->rows * 4, (size_t)w->rows * 4, (size_t)n, hipMemcpyDeviceToHost));
+    return MQ_OK;
+}
+
+int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, int32_t* dot_scaled_dev,
+                        int32_t* min_dot_dev, float* y_dev, int64_t ldy, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_debug_block_sums")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: dense weights only");
+    if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_debug_block_sums")) return rc;
+    if (!dot_scaled_dev || !min_dot_dev || !y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: null output");
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
+    return matmul_from_ws(w, n, y_dev, ldy, dot_scaled_dev, min_dot_dev, s);
+}
+
+// ---------------------------------------------------------------------------------- dense FFN
+int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev,
+                      int64_t n, float* y_dev, int silu_mode, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(gate, "mq_ffn_swiglu_q4k(gate)")) return rc;
+    if (int rc = check_weight(up, "mq_ffn_swiglu_q4k(up)")) return rc;
+    if (int rc = check_weight(down, "mq_ffn_swiglu_q4k(down)")) return rc;
+    const int64_t hidden = gate->cols, inter = gate->rows;
+    if (up->cols != hidden || up->rows != inter || down->cols != inter || down->rows != hidden || gate->n_experts != 1 ||
+        up->n_experts != 1 || down->n_experts != 1)
+        return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: gate/up must be [inter][hidden] and down [hidden][inter]");
+    if (inter % kQK) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: inter %lld is not a multiple of 256", (long long)inter);
+    if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: silu_mode %d", silu_mode);
+    if (int rc = check_x(x_dev, n, hidden, hidden, "mq_ffn_swiglu_q4k")) return rc;
+    if (!y_dev) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: null output");
+    if (n == 0) return MQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+    MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
+    MatmulArgs a;
+    a.w0 = gate->data;
+    a.w1 = up->data;
+    a.rows = inter;
+    a.nb = gate->nb;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ad = (const float*)g.ad.ptr;
+    a.n = n;
+    a.y = (float*)g.mid.ptr;
+    a.ldy = inter;
+    a.swiglu = 1;
+    a.silu_mode = silu_mode;
+    MQ_HIP(launch_matmul(a, s));
+    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    MatmulArgs d;
+    d.w0 = down->data;
+    d.rows = hidden;
+    d.nb = down->nb;
+    d.aq = (const uint8_t*)g.aq2.ptr;
+    d.ad = (const float*)g.ad2.ptr;
+    d.n = n;
+    d.y = y_dev;
+    d.ldy = hidden;
+    MQ_HIP(launch_matmul(d, s));
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- router / MoE
+namespace {
+struct RouteWs {  // carved out of g.route
+    int32_t* ids;
+    float* weights;
+    int32_t* group_expert;
+    int32_t* group_begin;
+    int32_t* n_groups;
+    int32_t* entry_token;
+    int32_t* entry_k;
+};
+int carve_route(int64_t n, int top_k, int64_t n_experts, RouteWs& r) {
+    const size_t entries = (size_t)n * (size_t)top_k;
+    const size_t groups = (size_t)n_experts + 2;
+    const size_t ints = entries * 4 + groups * 2 + 16;
+    MQ_HIP(g.route.reserve(ints * 4));
+    int32_t* p = (int32_t*)g.route.ptr;
+    r.ids = p;
+    p += entries;
+    r.weights = (float*)p;
+    p += entries;
+    r.entry_token = p;
+    p += entries;
+    r.entry_k = p;
+    p += entries;
+    r.group_expert = p;
+    p += groups;
+    r.group_begin = p;
+    p += groups;
+    r.n_groups = p;
+    return MQ_OK;
+}
+}  // namespace
+
+int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int top_k, int weights_mode,
+                      int32_t* ids_dev, float* weights_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!logits_dev || !ids_dev || !weights_dev) return fail(MQ_ERR_INVALID, "mq_moe_route_topk: null pointer");
+    if (n < 0 || n_experts <= 0 || top_k <= 0 || top_k > n_experts || top_k > 8)
+        return fail(MQ_ERR_INVALID, "mq_moe_route_topk: need 0 < top_k <= min(8, n_experts)");
+    if (weights_mode < 0 || weights_mode > 2) return fail(MQ_ERR_INVALID, "mq_moe_route_topk: weights_mode %d", weights_mode);
+    if (n == 0) return MQ_OK;
+    MQ_HIP(launch_route_topk(logits_dev, n_experts, n, top_k, weights_mode, ids_dev, weights_dev, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
+                      int top_k, float* y_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_id_q4k")) return rc;
+    if (!ids_dev || !y_dev || top_k <= 0) return fail(MQ_ERR_INVALID, "mq_mul_mat_id_q4k: null pointer or top_k <= 0");
+    if (x_slots != 1 && x_slots != top_k) return fail(MQ_ERR_INVALID, "mq_mul_mat_id_q4k: x_slots must be 1 or top_k");
+    if (int rc = check_x(x_dev, n * x_slots, w->cols, w->cols, "mq_mul_mat_id_q4k")) return rc;
+    if (n == 0) return MQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n * x_slots, w->cols, w->cols, s)) return rc;
+    RouteWs r;
+    if (int rc = carve_route(n, top_k, w->n_experts, r)) return rc;
+    // entries with ids outside [0, n_experts) are dropped by the grouping, so clear y first
+    MQ_HIP(launch_fill_zero(y_dev, (size_t)n * top_k * (size_t)w->rows, s));
+    MQ_HIP(launch_build_groups(ids_dev, n, top_k, w->n_experts, r.group_expert, r.group_begin, r.n_groups,
+                               r.entry_token, r.entry_k, s));
+    MatmulArgs a;
+    a.w0 = w->data;
+    a.rows = w->rows;
+    a.nb = w->nb;
+    a.expert_bytes = w->expert_bytes;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ad = (const float*)g.ad.ptr;
+    a.n = n;  // widest possible group
+    a.y = y_dev;
+    a.ldy = w->rows;
+    a.grouped = 1;
+    a.group_expert = r.group_expert;
+    a.group_begin = r.group_begin;
+    a.n_groups = r.n_groups;
+    a.entry_token = r.entry_token;
+    a.entry_k = r.entry_k;
+    a.a_tok_stride = x_slots == 1 ? 1 : top_k;  // activation row: token, or token*top_k + k
+    a.a_k_stride = x_slots == 1 ? 0 : 1;
+    a.y_tok_stride = top_k;                     // output row: token*top_k + k
+    a.y_k_stride = 1;
+    const int64_t pairs = n * (int64_t)top_k;
+    a.max_groups = (int)(pairs < w->n_experts ? pairs : w->n_experts);
+    MQ_HIP(launch_matmul(a, s));
+    return MQ_OK;
+}
+
+int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float* logits_dev, int64_t n, float* y_dev,
+                     int32_t* ids_out_dev, float* weights_out_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!L) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null layer");
+    if (int rc = check_weight(L->gate_exps, "mq_moe_layer_q4k(gate_exps)")) return rc;
+    if (int rc = check_weight(L->up_exps, "mq_moe_layer_q4k(up_exps)")) return rc;
+    if (int rc = check_weight(L->down_exps, "mq_moe_layer_q4k(down_exps)")) return rc;
+    const int64_t hidden = L->gate_exps->cols, inter = L->gate_exps->rows, E = L->gate_exps->n_experts;
+    const int K = L->top_k;
+    if (L->up_exps->cols != hidden || L->up_exps->rows != inter || L->up_exps->n_experts != E ||
+        L->down_exps->cols != inter || L->down_exps->rows != hidden || L->down_exps->n_experts != E)
+        return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: expert tensor shapes disagree");
+    if (inter % kQK) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: inter must be a multiple of 256");
+    if (K <= 0 || K > 8 || K > E) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: need 0 < top_k <= min(8, n_experts)");
+    const bool has_shared = L->shared_gate || L->shared_up || L->shared_down;
+    if (has_shared) {
+        if (int rc = check_weight(L->shared_gate, "mq_moe_layer_q4k(shared_gate)")) return rc;
+        if (int rc = check_weight(L->shared_up, "mq_moe_layer_q4k(shared_up)")) return rc;
+        if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)")) return rc;
+        if (L->shared_gate->cols != hidden || L->shared_gate->rows != inter || L->shared_up->cols != hidden ||
+            L->shared_up->rows != inter || L->shared_down->cols != inter || L->shared_down->rows != hidden)
+            return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: shared expert must have the routed experts' shape");
+    }
+    if (int rc = check_x(x_dev, n, hidden, hidden, "mq_moe_layer_q4k")) return rc;
+    if (!logits_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null logits or output");
+    if (n == 0) return MQ_OK;
+
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    const int slots = K + (has_shared ? 1 : 0);  // rows per token in the hidden / partial buffers
+    RouteWs r;
+    if (int rc = carve_route(n, K, E, r)) return rc;
+    MQ_HIP(launch_route_topk(logits_dev, E, n, K, L->route_mode, r.ids, r.weights, s));
+    MQ_HIP(launch_build_groups(r.ids, n, K, E, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+
+    const int64_t mid_rows = n * slots;
+    MQ_HIP(g.mid.reserve((size_t)mid_rows * (size_t)inter * sizeof(float)));
+    MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden * sizeof(float)));
+    const int64_t pairs = n * (int64_t)K;
+    const int max_groups = (int)(pairs < E ? pairs : E);
+
+    // gate/up + SwiGLU: activation row = token, output row = token*slots + k
+    MatmulArgs a;
+    a.w0 = L->gate_exps->data;
+    a.w1 = L->up_exps->data;
+    a.rows = inter;
+    a.nb = L->gate_exps->nb;
+    a.expert_bytes = L->gate_exps->expert_bytes;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ad = (const float*)g.ad.ptr;
+    a.n = n;
+    a.y = (float*)g.mid.ptr;
+    a.ldy = inter;
+    a.swiglu = 1;
+    a.silu_mode = L->silu_mode;
+    a.grouped = 1;
+    a.group_expert = r.group_expert;
+    a.group_begin = r.group_begin;
+    a.n_groups = r.n_groups;
+    a.entry_token = r.entry_token;
+    a.entry_k = r.entry_k;
+    a.a_tok_stride = 1;
+    a.a_k_stride = 0;
+    a.y_tok_stride = slots;
+    a.y_k_stride = 1;
+    a.max_groups = max_groups;
+    if (has_shared) {
+        a.sh_w0 = L->shared_gate->data;
+        a.sh_w1 = L->shared_up->data;
+        a.sh_tokens = (int)n;
+        a.sh_arow_stride = 1;
+        a.sh_arow_offset = 0;
+        a.sh_yrow_stride = slots;
+        a.sh_yrow_offset = K;
+        a.sh_silu_mode = MQ_SILU_FAST_FMA;
+    }
+    MQ_HIP(launch_matmul(a, s));
+
+    // Q8_K of every hidden row (rows of dropped entries hold stale data and are never read)
+    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, mid_rows, inter, inter, s)) return rc;
+
+    // down: activation row = output row = token*slots + k
+    MatmulArgs d;
+    d.w0 = L->down_exps->data;
+    d.rows = hidden;
+    d.nb = L->down_exps->nb;
+    d.expert_bytes = L->down_exps->expert_bytes;
+    d.aq = (const uint8_t*)g.aq2.ptr;
+    d.ad = (const float*)g.ad2.ptr;
+    d.n = n;
+    d.y = (float*)g.part.ptr;
+    d.ldy = hidden;
+    d.grouped = 1;
+    d.group_expert = r.group_expert;
+    d.group_begin = r.group_begin;
+    d.n_groups = r.n_groups;
+    d.entry_token = r.entry_token;
+    d.entry_k = r.entry_k;
+    d.a_tok_stride = slots;
+    d.a_k_stride = 1;
+    d.y_tok_stride = slots;
+    d.y_k_stride = 1;
+    d.max_groups = max_groups;
+    if (has_shared) {
+        d.sh_w0 = L->shared_down->data;
+        d.sh_tokens = (int)n;
+        d.sh_arow_stride = slots;
+        d.sh_arow_offset = K;
+        d.sh_yrow_stride = slots;
+        d.sh_yrow_offset = K;
+    }
+    MQ_HIP(launch_matmul(d, s));
+
+    MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, K, slots, hidden, r.weights, r.ids, E,
+                              has_shared ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
+    if (ids_out_dev) MQ_HIP(hipMemcpyAsync(ids_out_dev, r.ids, (size_t)pairs * 4, hipMemcpyDeviceToDevice, s));
+    if (weights_out_dev) MQ_HIP(hipMemcpyAsync(weights_out_dev, r.weights, (size_t)pairs * 4, hipMemcpyDeviceToDevice, s));
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- memory helpers
+int mq_device_malloc(void** ptr, size_t bytes) {
+    if (int rc = check_ready()) return rc;
+    if (!ptr) return fail(MQ_ERR_INVALID, "mq_device_malloc: null out pointer");
+    MQ_HIP(hipMalloc(ptr, bytes ? bytes : 1));
+    return MQ_OK;
+}
+int mq_device_free(void* ptr) {
+    if (ptr) MQ_HIP(hipFree(ptr));
+    return MQ_OK;
+}
+int mq_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes) {
+    MQ_HIP(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+    return MQ_OK;
+}
+int mq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes) {
+    MQ_HIP(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+    return MQ_OK;
+}
+int mq_stream_synchronize(void* stream) {
+    MQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return MQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+// Shared constants, layouts and small device helpers for the gfx950 Q4_K x Q8_K kernels.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mq {
+
+constexpr int kQK = 256;             // weights per super-block
+constexpr int kQ4Block = 144;        // bytes of block_q4_K
+constexpr int kQ8Block = 292;        // bytes of block_q8_K
+constexpr int kTileRows = 16;        // weight rows per tile (the N side of a 16x16 MFMA)
+constexpr int kTileBytes = kTileRows * kQ4Block;  // 2304
+constexpr int kTileQBytes = kTileRows * 128;      // 2048: nibble part
+constexpr int kTokTile = 16;         // activation rows per MFMA (the M side)
+
+// ---------------------------------------------------------------------------------------------
+// Weight layout in HBM ("row-tile major"): a matrix of `rows` x `cols` is cut into tiles of 16
+// rows x one super-block.  Tile (rt, b) sits at ((rt * nb + b) * 2304) bytes; a wave reads it
+// with three fully coalesced 16-byte-per-lane loads and gets its MFMA B operand without any
+// shuffle:
+//   bytes [i*1024 + lane*16, +16), i = 0,1   lane = kq*16 + r  (r = row in tile, kq = 0..3)
+//        [0..7]  = qs[r][32*(2i)   + 8*kq .. +7]   -> low nibbles: sub-block 4i,   elements 8kq..8kq+7
+//                                                     high nibbles: sub-block 4i+1
+//        [8..15] = qs[r][32*(2i+1) + 8*kq .. +7]   -> sub-blocks 4i+2 (low) and 4i+3 (high)
+//   bytes [2048 + r*16, +16)                 = {fp16 d, fp16 dmin, scales[12]} of row r
+// Same 144 bytes per 256 weights as ggml's block_q4_K; only the order differs.
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ inline size_t tile_offset(int64_t rt, int64_t b, int64_t nb) {
+    return (size_t)(rt * nb + b) * kTileBytes;
+}
+
+// Offset inside a tile of the 8-byte word `word` (0..17) of row r's block_q4_K.
+__host__ __device__ inline int tile_word_offset(int r, int word) {
+    if (word < 2) return kTileQBytes + r * 16 + word * 8;
+    const int j = word - 2;        // qs[8j .. 8j+7]
+    const int chunk = j >> 2;      // 32-byte chunk of qs
+    const int kq = j & 3;
+    return (chunk >> 1) * 1024 + (kq * 16 + r) * 16 + (chunk & 1) * 8;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Activation layout consumed by the matmul kernels ("A-major Q8_K"): the same int8 codes and fp32
+// scales as block_q8_K, ordered so that a wave reads its MFMA A operand with coalesced 16-byte
+// loads.  Activation row m (a token, or a (token, k) pair) lives in row-tile m/16, slot m%16:
+//   codes : [m/16][b][gp 0..3][kq 0..3][slot 0..15][16 B]
+//           16 B = {qs[64gp + 8kq .. +7], qs[64gp + 32 + 8kq .. +7]}  (sub-blocks 2gp and 2gp+1)
+//   scale : [m/16][b][slot] fp32
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ inline size_t aq_offset(int64_t m, int64_t b, int gp, int kq, int64_t nb) {
+    return ((((size_t)(m >> 4) * nb + b) * 4 + gp) * 4 + kq) * 256 + (size_t)(m & 15) * 16;
+}
+__host__ __device__ inline size_t ad_index(int64_t m, int64_t b, int64_t nb) {
+    return ((size_t)(m >> 4) * nb + b) * 16 + (size_t)(m & 15);
+}
+__host__ __device__ inline size_t aq_bytes(int64_t n_rows, int64_t nb) {
+    return (size_t)((n_rows + 15) >> 4) * nb * 4096;
+}
+__host__ __device__ inline size_t ad_count(int64_t n_rows, int64_t nb) {
+    return (size_t)((n_rows + 15) >> 4) * nb * 16;
+}
+
+// SplitMix64 finaliser: the synthetic-weight recipe shared with densecore_amd/synth.py.
+__host__ __device__ inline uint64_t mix64(uint64_t z) {
+    z ^= z >> 30;
+    z *= 0xBF58476D1CE4E5B9ull;
+    z ^= z >> 27;
+    z *= 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return z;
+}
+constexpr uint64_t kGamma = 0x9E3779B97F4A7C15ull;
+constexpr uint64_t kScaleStream = 0x5CA1E5CA1E5CA1E5ull;
+
+#if defined(__HIPCC__)
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h16) {
+    return __half2float(__ushort_as_half((unsigned short)h16));
+}
+
+// Streaming 16-byte load for weights that are read exactly once.
+__device__ __forceinline__ v4u load_stream16(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const v4u*>(p));
+}
+__device__ __forceinline__ v4u load16(const void* p) { return *reinterpret_cast<const v4u*>(p); }
+
+// The reference's fast exp (core/src/backend/cpu_backend_internal.h:99-114): unfused Horner.
+__device__ __forceinline__ float fast_exp_plain(float x) {
+    x = x < -50.0f ? -50.0f : x;
+    x = x > 50.0f ? 50.0f : x;
+    const float y = __fmul_rn(x, 1.4426950408889634f);
+    const float fl = floorf(y);
+    const float f = __fsub_rn(y, fl);
+    const float inner = __fadd_rn(0.224494337302845f, __fmul_rn(f, 0.07944023841053369f));
+    const float mid = __fadd_rn(0.6960656421638072f, __fmul_rn(f, inner));
+    const float p = __fadd_rn(1.0f, __fmul_rn(f, mid));
+    const int ebits = ((int)fl + 127) << 23;
+    return __fmul_rn(__int_as_float(ebits), p);
+}
+// core/src/kernels/hwy/hwy_fastexp.h:13-47: the same cubic with fused multiply-adds.
+__device__ __forceinline__ float fast_exp_fma(float x) {
+    x = fmaxf(fminf(x, 50.0f), -50.0f);
+    const float y = __fmul_rn(x, 1.4426950408889634f);
+    const float fl = floorf(y);
+    const float f = __fsub_rn(y, fl);
+    float p = __fmaf_rn(f, 0.07944023841053369f, 0.224494337302845f);
+    p = __fmaf_rn(f, p, 0.6960656421638072f);
+    p = __fmaf_rn(f, p, 1.0f);
+    const int ebits = ((int)fl + 127) << 23;
+    return __fmul_rn(__int_as_float(ebits), p);
+}
+// silu(gate) * up in the three orders the reference uses (see include/mi355_q4k.h MQ_SILU_*).
+__device__ __forceinline__ float silu_mul(float g, float u, int mode) {
+    if (mode == 1) return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, fast_exp_plain(-g))), u);
+    if (mode == 2) {
+        const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, fast_exp_fma(__fmul_rn(g, -1.0f))));
+        return __fmul_rn(__fmul_rn(g, sig), u);
+    }
+    return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
+}
+#endif
+
+}  // namespace mq

@@ -1,0 +1,79 @@
+// Host-callable launchers of the gfx950 kernels (internal to libmi355q4k.so).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mq {
+
+// ---- quantize.hip ----------------------------------------------------------------------------
+// fp32 rows -> Q8_K.  q8_std (block_q8_K rows, may be null) and/or the A-major pair (aq, ad; may be
+// null) are written from the same registers.
+hipError_t launch_quantize_q8k(const float* x, int64_t n, int64_t ldx, int64_t k, void* q8_std, size_t q8_row_bytes,
+                               uint8_t* aq, float* ad, hipStream_t stream);
+// block_q8_K rows -> A-major layout.
+hipError_t launch_q8k_to_amajor(const void* q8_std, int64_t n, size_t q8_row_bytes, int64_t k, uint8_t* aq, float* ad,
+                                hipStream_t stream);
+
+// ---- weights.hip -----------------------------------------------------------------------------
+// ggml row layout (rows x nb blocks, row_bytes apart) -> tiled layout, one expert per grid.y.
+hipError_t launch_tile_weights(const uint8_t* raw, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
+                               int64_t n_experts, uint8_t* tiled, size_t tiled_expert_bytes, hipStream_t stream);
+hipError_t launch_untile_weights(const uint8_t* tiled, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
+                                 int64_t n_experts, uint8_t* raw, size_t tiled_expert_bytes, hipStream_t stream);
+hipError_t launch_synth_weights(uint64_t seed, int64_t rows, int64_t nb, int64_t n_experts, uint8_t* tiled,
+                                size_t tiled_expert_bytes, hipStream_t stream);
+
+// ---- matmul.hip ------------------------------------------------------------------------------
+struct MatmulArgs {
+    const uint8_t* w0 = nullptr;   // tiled weights (expert 0); gate when swiglu
+    const uint8_t* w1 = nullptr;   // up weights when swiglu, else unused
+    int64_t rows = 0;              // output rows of one matrix
+    int64_t nb = 0;                // super-blocks per row (cols / 256)
+    size_t expert_bytes = 0;       // tiled bytes per expert (grouped mode)
+    const uint8_t* aq = nullptr;   // A-major activations
+    const float* ad = nullptr;
+    int64_t n = 0;                 // activation rows (dense mode)
+    float* y = nullptr;            // dense: [n][ldy]; grouped: [entry][ldy]
+    int64_t ldy = 0;
+    int swiglu = 0;                // 1: y = silu(w0 x) * (w1 x)
+    int silu_mode = 0;
+    int32_t* dbg_dot = nullptr;    // optional [rows][n][nb]
+    int32_t* dbg_min = nullptr;
+    // grouped (expert-routed) mode: work list built on the device
+    int grouped = 0;
+    const int32_t* group_expert = nullptr;  // [max_groups] expert id per group
+    const int32_t* group_begin = nullptr;   // [max_groups + 1] offsets into entries
+    const int32_t* n_groups = nullptr;      // [1]
+    const int32_t* entry_token = nullptr;   // [n_entries] token of each entry, sorted by (expert, token, k)
+    const int32_t* entry_k = nullptr;       // [n_entries] routing slot of each entry
+    int a_tok_stride = 1, a_k_stride = 0;   // activation row of an entry = token * a_tok_stride + k * a_k_stride
+    int y_tok_stride = 1, y_k_stride = 0;   // output row of an entry
+    int max_groups = 0;
+    // optional second family of groups with their own weights (the shared expert): group ids >= n_groups
+    const uint8_t* sh_w0 = nullptr;
+    const uint8_t* sh_w1 = nullptr;
+    int sh_tokens = 0;             // number of activation rows the shared expert sees (0 = none)
+    int sh_arow_stride = 1;        // activation row of token t = t * sh_arow_stride + sh_arow_offset
+    int sh_arow_offset = 0;
+    int sh_yrow_stride = 1;        // output row of token t
+    int sh_yrow_offset = 0;
+    int sh_silu_mode = 2;
+};
+hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream);
+
+// ---- router.hip ------------------------------------------------------------------------------
+hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
+                             float* weights, hipStream_t stream);
+// Expert-grouped work list from ids [n][top_k]: entries sorted by (expert, token, k).
+//   group_expert[g], group_begin[g..g+1], n_groups[0], entry_token[e], entry_k[e]
+hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t n_experts, int32_t* group_expert,
+                               int32_t* group_begin, int32_t* n_groups, int32_t* entry_token, int32_t* entry_k,
+                               hipStream_t stream);
+// y[t][r] = sum_k w[t][k] * part[t*slots + k][r]  (k in order) + gate[t] * part[t*slots + top_k][r]
+hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots, int64_t rows, const float* weights,
+                              const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,
+                              const float* x, float* y, hipStream_t stream);
+hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
+
+}  // namespace mq

@@ -1,0 +1,169 @@
+/*
+ * mi355_q4k.h -- C ABI of libmi355q4k.so: DenseCore's Q4_K-weight x
+ * Q8_K-activation matmul path on one MI355X (gfx950).
+ *
+ * Every entry point is plain C: pointers, sizes, int status (0 = ok, negative
+ * = error, text via mq_last_error()).  Pointers named *_dev are device
+ * pointers (HBM), *_host are host pointers.  `stream` is a hipStream_t passed
+ * as void* (NULL = the default stream).  All launches are stream-ordered and
+ * return without synchronising unless the name ends in _host.
+ *
+ * Each declaration cites the DenseCore interface it stands in for
+ * (paths relative to the DenseCore tree).
+ */
+#ifndef MI355_Q4K_H
+#define MI355_Q4K_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MQ_OK 0
+#define MQ_ERR_INVALID (-1)   /* bad argument (null, shape, alignment)          */
+#define MQ_ERR_HIP (-2)       /* a HIP call failed                              */
+#define MQ_ERR_STATE (-3)     /* library not initialised / no GPU               */
+#define MQ_ERR_UNSUPPORTED (-4)
+
+/* SiLU-gate flavours; which one the reference runs depends on the branch
+ * (exact: core/src/kernels/hwy/hwy_moe_quant.cc:377; fast:
+ * core/src/backend/cpu_backend_moe_raw_batched.inl:1673 with
+ * cpu_backend_internal.h:99-114; fast_fma: core/src/kernels/hwy/hwy_activation.cc:153-167). */
+#define MQ_SILU_EXACT 0
+#define MQ_SILU_FAST 1
+#define MQ_SILU_FAST_FMA 2
+
+/* Router weight flavours (core/src/llm/moe/native.cpp:650-675, :2321-2355, :822-866). */
+#define MQ_ROUTE_FUSED 0
+#define MQ_ROUTE_FLOOR 1
+#define MQ_ROUTE_FLOOR_FINITE 2
+
+typedef struct mq_weight mq_weight; /* device-resident Q4_K matrix (or expert stack) */
+
+/* ---- library state ---------------------------------------------------------
+ * Mirrors the engine-level init/teardown and error string of the C API
+ * (core/include/densecore.h:163 DenseCoreGetLastError, :296 InitEngine). */
+int mq_init(int device);
+int mq_shutdown(void);
+const char* mq_last_error(void);
+/* HIP runtime version, device name, CU count: what a host would log at load. */
+int mq_device_info(char* name_out, size_t name_cap, int* cu_count, size_t* hbm_bytes);
+
+/* ---- weights ----------------------------------------------------------------
+ * Takes ggml-layout Q4_K bytes exactly as a GGUF tensor holds them: rows of
+ * cols/256 block_q4_K (144 B each), `row_bytes` apart (ggml nb[1]); expert
+ * matrices `expert_bytes` apart (ggml nb[2], core/src/llm/moe/native.cpp:4091-4094).
+ * n_experts = 1 for a dense matrix.  The data is copied to HBM once and
+ * re-tiled for the GPU (same 144 B per 256 weights); the host buffer is not
+ * referenced afterwards.  Stands in for the weight side of
+ * GgmlQuantizedMatrixView (core/include/densecore/backend/cpu_backend.h:91-99)
+ * and for the repack cache GetOrCreateQ4KRepackedGemvWeight
+ * (core/src/kernels/q4k_repacked_gemv.cpp:403). */
+int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts, size_t row_bytes,
+                     size_t expert_bytes, mq_weight** out);
+/* Same tensor filled on the device from a 64-bit seed with the synthetic
+ * recipe of densecore_amd/synth.py (byte-identical to uploading
+ * synth.q4k_matrix(seed, rows*n_experts, cols)); for multi-GB benchmark sets. */
+int mq_weight_synthetic(uint64_t seed, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out);
+/* Copies the tensor back in ggml row layout (inverse of the re-tiling). */
+int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, size_t expert_bytes);
+int mq_weight_shape(const mq_weight* w, int64_t* rows, int64_t* cols, int64_t* n_experts, size_t* device_bytes);
+int mq_weight_free(mq_weight* w);
+
+/* ---- Q8_K activation quantizer ----------------------------------------------
+ * x_dev fp32 [n][ldx] (first k of each row used) -> q8_dev [n][k/256] block_q8_K
+ * (292 B: fp32 d, 256 int8, 16 int16 bsums), bit-exact with
+ * QuantizeRowQ8K_Hwy (core/include/densecore/simd/hwy_ops.h:255,
+ * core/src/kernels/hwy/hwy_moe_quant.cc:103-143) and ggml's from_float at
+ * core/src/llm/matmul/gemv_exec.cpp:298-332. */
+int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void* q8_dev, void* stream);
+
+/* ---- dense matmul: ggml_mul_mat on GGML_TYPE_Q4_K ---------------------------
+ * y[m][r] = W[r] . q8k(x[m]),  m < n, r < rows.  x_dev fp32 [n][ldx], y_dev
+ * fp32 [n][ldy] (token-major, i.e. ggml dst ne = [rows, n]).  Replaces
+ * cb_gemv_custom (core/src/llm/matmul/gemv_exec.cpp:99, n == 1),
+ * cb_gemv_batched_custom (core/src/llm/matmul/batched_exec.cpp:55, 2 <= n <= 16)
+ * and CpuBackend::MatMulGgmlQuantizedTransB
+ * (core/include/densecore/backend/cpu_backend.h:293-300, any n). */
+int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                   void* stream);
+/* Same with already-quantized activations: q8_dev [n][q8_row_bytes] block_q8_K rows
+ * (RunMoEQ4KRawBatchedProjectionImpl, core/src/backend/cpu_backend_moe_raw_batched.inl:1352). */
+int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t q8_row_bytes, float* y_dev,
+                       int64_t ldy, void* stream);
+/* Host-pointer convenience for a CPU graph executor: copies x in, y out, and
+ * synchronises.  What a GGML_OP_CUSTOM callback calls when ith == 0. */
+int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int64_t ldx, float* y_host, int64_t ldy);
+
+/* ---- dense SwiGLU FFN --------------------------------------------------------
+ * y = down( silu(gate x) * (up x) ), x_dev [n][hidden], y_dev [n][hidden].
+ * gate/up: rows = inter, cols = hidden; down: rows = hidden, cols = inter.
+ * The three smart_mul_mat calls plus cb_silu_mul_fused of a dense FFN block
+ * (core/src/llm/graph/decoder.cpp:2662-2730, core/src/llm/graph/fused_ops.cpp:317-366). */
+int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev,
+                      int64_t n, float* y_dev, int silu_mode, void* stream);
+
+/* ---- MoE router ---------------------------------------------------------------
+ * logits_dev fp32 [n][n_experts] -> ids_dev int32 [n][top_k], weights_dev fp32
+ * [n][top_k]: stable top-k (ties -> lower id, NaN last) and softmax over the
+ * selected logits.  ComputeQwenNativeMoEStableTopK
+ * (core/src/llm/moe/native.cpp:621-676) / cb_moe_topk_weights_from_logits (:800-868). */
+int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int top_k, int weights_mode,
+                      int32_t* ids_dev, float* weights_dev, void* stream);
+
+/* ---- expert-routed matmul: ggml_mul_mat_id on GGML_TYPE_Q4_K -----------------
+ * y[t][k][r] = W[ids[t][k]][r] . q8k(x[t][k or 0]).  x_dev fp32 [n][x_slots][cols]
+ * with x_slots == 1 (one row per token, broadcast over k: the gate/up case) or
+ * x_slots == top_k (one row per (token, k): the down case).  ids_dev int32
+ * [n][top_k]; entries outside [0, n_experts) produce zeros.  Tokens are grouped
+ * by expert on the device; nothing returns to the host.  y_dev fp32
+ * [n][top_k][rows].  (ggml_mul_mat_id as emitted at
+ * core/src/llm/moe/native_gemma.cpp:1509-1559.) */
+int mq_mul_mat_id_q4k(const mq_weight* w_exps, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
+                      int top_k, float* y_dev, void* stream);
+
+/* ---- fused MoE layer -------------------------------------------------------------
+ * The four custom nodes of TryBuildQwen35NativeMoEGraph
+ * (core/src/llm/moe/native.cpp:4691, :4831-4911) plus the shared-expert branch
+ * (core/src/llm/graph/decoder.cpp:2426-2600):
+ *   route top_k -> gate/up + SwiGLU per (token, k) -> Q8_K -> down ->
+ *   y[t] = sum_k w[t][k] * down_k (k in routing order) + sigmoid(sh_gate_inp . x[t]) * shared_ffn(x[t]).
+ * shared_* may all be NULL (no shared expert); sh_gate_inp_dev fp32 [hidden] or NULL (gate = 1). */
+typedef struct {
+    const mq_weight* gate_exps; /* n_experts x [inter][hidden]  */
+    const mq_weight* up_exps;
+    const mq_weight* down_exps; /* n_experts x [hidden][inter]  */
+    const mq_weight* shared_gate;
+    const mq_weight* shared_up;
+    const mq_weight* shared_down;
+    const float* sh_gate_inp_dev;
+    int top_k;
+    int silu_mode;        /* routed experts; the shared expert always uses MQ_SILU_FAST_FMA */
+    int route_mode;
+} mq_moe_layer_desc;
+int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const float* logits_dev, int64_t n,
+                     float* y_dev, int32_t* ids_out_dev /* may be NULL */, float* weights_out_dev /* may be NULL */,
+                     void* stream);
+
+/* ---- verification hook -------------------------------------------------------------
+ * Runs the production matmul kernel with its per-super-block integer sums
+ * written out: dot_scaled_dev / min_dot_dev int32 [rows][n][cols/256], the two
+ * integers every reference kernel forms before touching floating point
+ * (core/src/llm/matmul/kquant_batched_kernels.h:285-297).  Mirrors the
+ * reference's ...ForTest hooks (core/src/llm/moe/native.cpp:5107-5636). */
+int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, int32_t* dot_scaled_dev,
+                        int32_t* min_dot_dev, float* y_dev, int64_t ldy, void* stream);
+
+/* ---- device memory helpers (so a C host needs no HIP headers) -------------------- */
+int mq_device_malloc(void** ptr, size_t bytes);
+int mq_device_free(void* ptr);
+int mq_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes);
+int mq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes);
+int mq_stream_synchronize(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

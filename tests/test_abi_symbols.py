@@ -1,0 +1,35 @@
+"""CPU-side checks of the C ABI: the library loads without a GPU, exports every symbol the public
+header declares, and refuses work loudly when no device is present."""
+import os
+import re
+
+import pytest
+
+from densecore_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mi355_q4k.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_loader_agree():
+    assert declared_symbols() == sorted(_lib.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.load()
+    for name in declared_symbols():
+        assert hasattr(L, name), name
+
+
+@pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="a GPU is present")
+def test_no_gpu_is_a_loud_error_not_a_fallback():
+    L = _lib.load()
+    assert L.mq_init(0) != 0
+    assert b"no HIP device" in L.mq_last_error()
+    with pytest.raises(_lib.MqError):
+        _lib.lib()
