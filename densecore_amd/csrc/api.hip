@@ -489,62 +489,32 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     return MQ_OK;
 }
 
-int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float* logits_dev, int64_t n, float* y_dev,
-                     int32_t* ids_out_dev, float* weights_out_dev, void* stream) {
-    if (int rc = check_ready()) return rc;
-    if (!L) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null layer");
-    if (int rc = check_weight(L->gate_exps, "mq_moe_layer_q4k(gate_exps)")) return rc;
-    if (int rc = check_weight(L->up_exps, "mq_moe_layer_q4k(up_exps)")) return rc;
-    if (int rc = check_weight(L->down_exps, "mq_moe_layer_q4k(down_exps)")) return rc;
-    const int64_t hidden = L->gate_exps->cols, inter = L->gate_exps->rows, E = L->gate_exps->n_experts;
-    const int K = L->top_k;
-    if (L->up_exps->cols != hidden || L->up_exps->rows != inter || L->up_exps->n_experts != E ||
-        L->down_exps->cols != inter || L->down_exps->rows != hidden || L->down_exps->n_experts != E)
-        return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: expert tensor shapes disagree");
-    if (inter % kQK) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: inter must be a multiple of 256");
-    if (K <= 0 || K > 8 || K > E) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: need 0 < top_k <= min(8, n_experts)");
-    const bool has_shared = L->shared_gate || L->shared_up || L->shared_down;
-    if (has_shared) {
-        if (int rc = check_weight(L->shared_gate, "mq_moe_layer_q4k(shared_gate)")) return rc;
-        if (int rc = check_weight(L->shared_up, "mq_moe_layer_q4k(shared_up)")) return rc;
-        if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)")) return rc;
-        if (L->shared_gate->cols != hidden || L->shared_gate->rows != inter || L->shared_up->cols != hidden ||
-            L->shared_up->rows != inter || L->shared_down->cols != inter || L->shared_down->rows != hidden)
-            return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: shared expert must have the routed experts' shape");
-    }
-    if (int rc = check_x(x_dev, n, hidden, hidden, "mq_moe_layer_q4k")) return rc;
-    if (!logits_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null logits or output");
-    if (n == 0) return MQ_OK;
+namespace {
 
-    std::lock_guard<std::mutex> lock(g.mu);
-    hipStream_t s = (hipStream_t)stream;
-    const int slots = K + (has_shared ? 1 : 0);  // rows per token in the hidden / partial buffers
-    RouteWs r;
-    if (int rc = carve_route(n, K, E, r)) return rc;
-    MQ_HIP(launch_route_topk(logits_dev, E, n, K, L->route_mode, r.ids, r.weights, s));
-    MQ_HIP(launch_build_groups(r.ids, n, K, E, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
-    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+struct SharedExpert {
+    const mq_weight* gate = nullptr;
+    const mq_weight* up = nullptr;
+    const mq_weight* down = nullptr;
+};
 
-    const int64_t mid_rows = n * slots;
-    MQ_HIP(g.mid.reserve((size_t)mid_rows * (size_t)inter * sizeof(float)));
-    MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden * sizeof(float)));
-    const int64_t pairs = n * (int64_t)K;
-    const int max_groups = (int)(pairs < E ? pairs : E);
-
-    // gate/up + SwiGLU: activation row = token, output row = token*slots + k
+// gate/up + SwiGLU for every routed (token, k) pair (and the shared expert as slot top_k):
+// hidden row = token * slots + k.  Caller holds g.mu; groups are already built in r.
+int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExpert& sh, int64_t n, int top_k, int slots,
+                   int silu_mode, const RouteWs& r, float* hidden, hipStream_t s) {
+    const int64_t pairs = n * (int64_t)top_k;
     MatmulArgs a;
-    a.w0 = L->gate_exps->data;
-    a.w1 = L->up_exps->data;
-    a.rows = inter;
-    a.nb = L->gate_exps->nb;
-    a.expert_bytes = L->gate_exps->expert_bytes;
+    a.w0 = gate->data;
+    a.w1 = up->data;
+    a.rows = gate->rows;
+    a.nb = gate->nb;
+    a.expert_bytes = gate->expert_bytes;
     a.aq = (const uint8_t*)g.aq.ptr;
     a.ad = (const float*)g.ad.ptr;
     a.n = n;
-    a.y = (float*)g.mid.ptr;
-    a.ldy = inter;
+    a.y = hidden;
+    a.ldy = gate->rows;
     a.swiglu = 1;
-    a.silu_mode = L->silu_mode;
+    a.silu_mode = silu_mode;
     a.grouped = 1;
     a.group_expert = r.group_expert;
     a.group_begin = r.group_begin;
@@ -555,33 +525,41 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     a.a_k_stride = 0;
     a.y_tok_stride = slots;
     a.y_k_stride = 1;
-    a.max_groups = max_groups;
-    if (has_shared) {
-        a.sh_w0 = L->shared_gate->data;
-        a.sh_w1 = L->shared_up->data;
+    a.max_groups = (int)(pairs < gate->n_experts ? pairs : gate->n_experts);
+    if (sh.gate) {
+        a.sh_w0 = sh.gate->data;
+        a.sh_w1 = sh.up->data;
         a.sh_tokens = (int)n;
         a.sh_arow_stride = 1;
         a.sh_arow_offset = 0;
         a.sh_yrow_stride = slots;
-        a.sh_yrow_offset = K;
+        a.sh_yrow_offset = top_k;
         a.sh_silu_mode = MQ_SILU_FAST_FMA;
     }
     MQ_HIP(launch_matmul(a, s));
+    return MQ_OK;
+}
 
-    // Q8_K of every hidden row (rows of dropped entries hold stale data and are never read)
-    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, mid_rows, inter, inter, s)) return rc;
-
-    // down: activation row = output row = token*slots + k
+// Q8_K of the hidden rows, down projection per (token, k) into g.part, then the weighted combine.
+int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hidden, int64_t n, int top_k, int slots,
+                 const RouteWs& r, const int32_t* ids, const float* weights, const float* sh_gate_inp,
+                 const float* x, float* y, hipStream_t s) {
+    const int64_t pairs = n * (int64_t)top_k;
+    const int64_t mid_rows = n * slots;
+    const int64_t inter = down->cols, hidden_dim = down->rows;
+    // rows of dropped entries may hold anything; they are quantized but never read
+    if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
+    MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden_dim * sizeof(float)));
     MatmulArgs d;
-    d.w0 = L->down_exps->data;
-    d.rows = hidden;
-    d.nb = L->down_exps->nb;
-    d.expert_bytes = L->down_exps->expert_bytes;
+    d.w0 = down->data;
+    d.rows = hidden_dim;
+    d.nb = down->nb;
+    d.expert_bytes = down->expert_bytes;
     d.aq = (const uint8_t*)g.aq2.ptr;
     d.ad = (const float*)g.ad2.ptr;
     d.n = n;
     d.y = (float*)g.part.ptr;
-    d.ldy = hidden;
+    d.ldy = hidden_dim;
     d.grouped = 1;
     d.group_expert = r.group_expert;
     d.group_begin = r.group_begin;
@@ -592,21 +570,153 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     d.a_k_stride = 1;
     d.y_tok_stride = slots;
     d.y_k_stride = 1;
-    d.max_groups = max_groups;
-    if (has_shared) {
-        d.sh_w0 = L->shared_down->data;
+    d.max_groups = (int)(pairs < down->n_experts ? pairs : down->n_experts);
+    if (sh.down) {
+        d.sh_w0 = sh.down->data;
         d.sh_tokens = (int)n;
         d.sh_arow_stride = slots;
-        d.sh_arow_offset = K;
+        d.sh_arow_offset = top_k;
         d.sh_yrow_stride = slots;
-        d.sh_yrow_offset = K;
+        d.sh_yrow_offset = top_k;
     }
     MQ_HIP(launch_matmul(d, s));
+    MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, slots, hidden_dim, weights, ids, down->n_experts,
+                              sh.down ? 1 : 0, sh_gate_inp, x, y, s));
+    return MQ_OK;
+}
 
-    MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, K, slots, hidden, r.weights, r.ids, E,
-                              has_shared ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
-    if (ids_out_dev) MQ_HIP(hipMemcpyAsync(ids_out_dev, r.ids, (size_t)pairs * 4, hipMemcpyDeviceToDevice, s));
-    if (weights_out_dev) MQ_HIP(hipMemcpyAsync(weights_out_dev, r.weights, (size_t)pairs * 4, hipMemcpyDeviceToDevice, s));
+int check_experts(const mq_weight* gate, const mq_weight* up, const mq_weight* down, int top_k, const char* name) {
+    if (gate && up) {
+        if (up->cols != gate->cols || up->rows != gate->rows || up->n_experts != gate->n_experts)
+            return fail(MQ_ERR_INVALID, "%s: gate and up expert tensors disagree", name);
+        if (gate->rows % kQK) return fail(MQ_ERR_INVALID, "%s: inter must be a multiple of 256", name);
+    }
+    if (gate && down) {
+        if (down->cols != gate->rows || down->rows != gate->cols || down->n_experts != gate->n_experts)
+            return fail(MQ_ERR_INVALID, "%s: down expert tensor does not match gate/up", name);
+    }
+    const mq_weight* any = gate ? gate : down;
+    if (top_k <= 0 || top_k > 8 || top_k > any->n_experts)
+        return fail(MQ_ERR_INVALID, "%s: need 0 < top_k <= min(8, n_experts)", name);
+    return MQ_OK;
+}
+
+}  // namespace
+
+int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const float* x_dev, int64_t n, int64_t ldx,
+                          float* h_dev, int64_t ldh, int silu_mode, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(gate, "mq_swiglu_mul_mat_q4k(gate)")) return rc;
+    if (int rc = check_weight(up, "mq_swiglu_mul_mat_q4k(up)")) return rc;
+    if (up->cols != gate->cols || up->rows != gate->rows || gate->n_experts != 1 || up->n_experts != 1)
+        return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: gate and up must be dense matrices of one shape");
+    if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: silu_mode %d", silu_mode);
+    if (int rc = check_x(x_dev, n, ldx, gate->cols, "mq_swiglu_mul_mat_q4k")) return rc;
+    if (!h_dev || ldh < gate->rows) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: null output or ldh < rows");
+    if (n == 0) return MQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
+    MatmulArgs a;
+    a.w0 = gate->data;
+    a.w1 = up->data;
+    a.rows = gate->rows;
+    a.nb = gate->nb;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ad = (const float*)g.ad.ptr;
+    a.n = n;
+    a.y = h_dev;
+    a.ldy = ldh;
+    a.swiglu = 1;
+    a.silu_mode = silu_mode;
+    MQ_HIP(launch_matmul(a, s));
+    return MQ_OK;
+}
+
+int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exps, const float* x_dev, int64_t n,
+                             const int32_t* ids_dev, int top_k, int silu_mode, float* hidden_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(gate_exps, "mq_moe_gateup_swiglu_q4k(gate_exps)")) return rc;
+    if (int rc = check_weight(up_exps, "mq_moe_gateup_swiglu_q4k(up_exps)")) return rc;
+    if (int rc = check_experts(gate_exps, up_exps, nullptr, top_k, "mq_moe_gateup_swiglu_q4k")) return rc;
+    if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_moe_gateup_swiglu_q4k: silu_mode %d", silu_mode);
+    if (int rc = check_x(x_dev, n, gate_exps->cols, gate_exps->cols, "mq_moe_gateup_swiglu_q4k")) return rc;
+    if (!ids_dev || !hidden_dev) return fail(MQ_ERR_INVALID, "mq_moe_gateup_swiglu_q4k: null ids or output");
+    if (n == 0) return MQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    RouteWs r;
+    if (int rc = carve_route(n, top_k, gate_exps->n_experts, r)) return rc;
+    MQ_HIP(launch_fill_zero(hidden_dev, (size_t)n * top_k * (size_t)gate_exps->rows, s));
+    MQ_HIP(launch_build_groups(ids_dev, n, top_k, gate_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
+                               r.entry_token, r.entry_k, s));
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, gate_exps->cols, gate_exps->cols, s)) return rc;
+    return run_moe_gateup(gate_exps, up_exps, SharedExpert{}, n, top_k, top_k, silu_mode, r, hidden_dev, s);
+}
+
+int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev, int64_t n, const int32_t* ids_dev,
+                             const float* weights_dev, int top_k, float* y_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(down_exps, "mq_moe_down_weighted_q4k(down_exps)")) return rc;
+    if (int rc = check_experts(nullptr, nullptr, down_exps, top_k, "mq_moe_down_weighted_q4k")) return rc;
+    if (int rc = check_x(hidden_dev, n * top_k, down_exps->cols, down_exps->cols, "mq_moe_down_weighted_q4k")) return rc;
+    if (!ids_dev || !weights_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_down_weighted_q4k: null pointer");
+    if (n == 0) return MQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    RouteWs r;
+    if (int rc = carve_route(n, top_k, down_exps->n_experts, r)) return rc;
+    MQ_HIP(launch_build_groups(ids_dev, n, top_k, down_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
+                               r.entry_token, r.entry_k, s));
+    return run_moe_down(down_exps, SharedExpert{}, hidden_dev, n, top_k, top_k, r, ids_dev, weights_dev, nullptr,
+                        nullptr, y_dev, s);
+}
+
+int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float* logits_dev, int64_t n, float* y_dev,
+                     int32_t* ids_out_dev, float* weights_out_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!L) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null layer");
+    if (int rc = check_weight(L->gate_exps, "mq_moe_layer_q4k(gate_exps)")) return rc;
+    if (int rc = check_weight(L->up_exps, "mq_moe_layer_q4k(up_exps)")) return rc;
+    if (int rc = check_weight(L->down_exps, "mq_moe_layer_q4k(down_exps)")) return rc;
+    if (int rc = check_experts(L->gate_exps, L->up_exps, L->down_exps, L->top_k, "mq_moe_layer_q4k")) return rc;
+    const int64_t hidden = L->gate_exps->cols, inter = L->gate_exps->rows, E = L->gate_exps->n_experts;
+    const int K = L->top_k;
+    if (L->silu_mode < 0 || L->silu_mode > 2 || L->route_mode < 0 || L->route_mode > 2)
+        return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: bad silu_mode or route_mode");
+    SharedExpert sh;
+    if (L->shared_gate || L->shared_up || L->shared_down) {
+        if (int rc = check_weight(L->shared_gate, "mq_moe_layer_q4k(shared_gate)")) return rc;
+        if (int rc = check_weight(L->shared_up, "mq_moe_layer_q4k(shared_up)")) return rc;
+        if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)")) return rc;
+        if (L->shared_gate->cols != hidden || L->shared_gate->rows != inter || L->shared_up->cols != hidden ||
+            L->shared_up->rows != inter || L->shared_down->cols != inter || L->shared_down->rows != hidden ||
+            L->shared_gate->n_experts != 1 || L->shared_up->n_experts != 1 || L->shared_down->n_experts != 1)
+            return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: shared expert must have the routed experts' shape");
+        sh.gate = L->shared_gate;
+        sh.up = L->shared_up;
+        sh.down = L->shared_down;
+    }
+    if (int rc = check_x(x_dev, n, hidden, hidden, "mq_moe_layer_q4k")) return rc;
+    if (!logits_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null logits or output");
+    if (n == 0) return MQ_OK;
+
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    const int slots = K + (sh.gate ? 1 : 0);  // hidden / partial rows per token
+    RouteWs r;
+    if (int rc = carve_route(n, K, E, r)) return rc;
+    MQ_HIP(launch_route_topk(logits_dev, E, n, K, L->route_mode, r.ids, r.weights, s));
+    MQ_HIP(launch_build_groups(r.ids, n, K, E, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
+    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+    MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
+    if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, s)) return rc;
+    if (int rc = run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, n, K, slots, r, r.ids, r.weights,
+                              L->sh_gate_inp_dev, x_dev, y_dev, s))
+        return rc;
+    const size_t pair_bytes = (size_t)n * K * 4;
+    if (ids_out_dev) MQ_HIP(hipMemcpyAsync(ids_out_dev, r.ids, pair_bytes, hipMemcpyDeviceToDevice, s));
+    if (weights_out_dev) MQ_HIP(hipMemcpyAsync(weights_out_dev, r.weights, pair_bytes, hipMemcpyDeviceToDevice, s));
     return MQ_OK;
 }
 

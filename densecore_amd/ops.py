@@ -139,6 +139,16 @@ def debug_block_sums(w: Q4KWeight, x: torch.Tensor):
     return ds, md, y
 
 
+def swiglu_mul_mat(gate: Q4KWeight, up: Q4KWeight, x: torch.Tensor, silu: int = SILU_EXACT) -> torch.Tensor:
+    """FusedSwiGLUQ4KQ8KRows_Hwy (core/src/kernels/hwy/hwy_moe_quant.cc:359-380): silu(gate x) * (up x)."""
+    x = _f32(x)
+    n = x.shape[0]
+    h = torch.empty((n, gate.rows), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().mq_swiglu_mul_mat_q4k(gate._h, up._h, _ptr(x), n, x.stride(0), _ptr(h), gate.rows, silu,
+                                                _stream()), "mq_swiglu_mul_mat_q4k")
+    return h
+
+
 def ffn_swiglu(gate: Q4KWeight, up: Q4KWeight, down: Q4KWeight, x: torch.Tensor, silu: int = SILU_FAST_FMA):
     """down( silu(gate x) * (up x) ): the dense FFN block of core/src/llm/graph/decoder.cpp:2662-2730."""
     x = _f32(x)
@@ -168,6 +178,30 @@ def mul_mat_id(w: Q4KWeight, x: torch.Tensor, ids: torch.Tensor) -> torch.Tensor
     y = torch.empty((n, top_k, w.rows), dtype=torch.float32, device=x.device)
     _lib.check(_lib.lib().mq_mul_mat_id_q4k(w._h, _ptr(x), n, slots, _ptr(ids), top_k, _ptr(y), _stream()),
                "mq_mul_mat_id_q4k")
+    return y
+
+
+def moe_gateup_swiglu(gate_exps: Q4KWeight, up_exps: Q4KWeight, x: torch.Tensor, ids: torch.Tensor,
+                      silu: int = SILU_EXACT) -> torch.Tensor:
+    """cb_qwen35_native_moe_gateup_raw_qxk_swiglu (core/src/llm/moe/native.cpp:3929): -> hidden [n, top_k, inter]."""
+    x = _f32(x)
+    ids = ids.contiguous()
+    n, top_k = ids.shape
+    h = torch.empty((n, top_k, gate_exps.rows), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().mq_moe_gateup_swiglu_q4k(gate_exps._h, up_exps._h, _ptr(x), n, _ptr(ids), top_k, silu,
+                                                   _ptr(h), _stream()), "mq_moe_gateup_swiglu_q4k")
+    return h
+
+
+def moe_down_weighted(down_exps: Q4KWeight, hidden: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor):
+    """cb_qwen35_native_moe_down_q5k_weighted_logits (core/src/llm/moe/native.cpp:3051): -> y [n, hidden]."""
+    hidden = _f32(hidden)
+    ids = ids.contiguous()
+    weights = _f32(weights)
+    n, top_k = ids.shape
+    y = torch.empty((n, down_exps.rows), dtype=torch.float32, device=hidden.device)
+    _lib.check(_lib.lib().mq_moe_down_weighted_q4k(down_exps._h, _ptr(hidden), n, _ptr(ids), _ptr(weights), top_k,
+                                                   _ptr(y), _stream()), "mq_moe_down_weighted_q4k")
     return y
 
 

@@ -97,6 +97,14 @@ int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t
  * synchronises.  What a GGML_OP_CUSTOM callback calls when ith == 0. */
 int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int64_t ldx, float* y_host, int64_t ldy);
 
+/* ---- fused gate/up + SwiGLU ----------------------------------------------------
+ * h[m][r] = silu(gate[r] . q8k(x[m])) * (up[r] . q8k(x[m])), one pass over both matrices.
+ * FusedSwiGLUQ4KQ8KRows_Hwy (core/include/densecore/simd/hwy_ops.h:275-281,
+ * core/src/kernels/hwy/hwy_moe_quant.cc:359-380) and RunMoEQ4KRawBatchedFusedSwiGLUImpl
+ * (core/src/backend/cpu_backend_moe_raw_batched.inl:1629-1698). */
+int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const float* x_dev, int64_t n, int64_t ldx,
+                          float* h_dev, int64_t ldh, int silu_mode, void* stream);
+
 /* ---- dense SwiGLU FFN --------------------------------------------------------
  * y = down( silu(gate x) * (up x) ), x_dev [n][hidden], y_dev [n][hidden].
  * gate/up: rows = inter, cols = hidden; down: rows = hidden, cols = inter.
@@ -123,6 +131,21 @@ int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int
  * core/src/llm/moe/native_gemma.cpp:1509-1559.) */
 int mq_mul_mat_id_q4k(const mq_weight* w_exps, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
                       int top_k, float* y_dev, void* stream);
+
+/* ---- the two expert nodes of the native MoE graph --------------------------------
+ * gate/up node: hidden[t][k][r] = silu(gate_e[r] . q8k(x[t])) * (up_e[r] . q8k(x[t])), e = ids[t][k];
+ * hidden_dev fp32 [n][top_k][inter].  cb_qwen35_native_moe_gateup_raw_qxk_swiglu
+ * (core/src/llm/moe/native.cpp:3929-4345, built at :4871-4874).  Rows whose id is outside
+ * [0, n_experts) are set to zero. */
+int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exps, const float* x_dev, int64_t n,
+                             const int32_t* ids_dev, int top_k, int silu_mode, float* hidden_dev, void* stream);
+/* down node: y[t][r] = sum_k weights[t][k] * (down_e[r] . q8k(hidden[t][k])), k in routing order,
+ * zero weights and invalid ids skipped.  cb_qwen35_native_moe_down_q5k_weighted_logits
+ * (core/src/llm/moe/native.cpp:3051-3295, built at :4906-4911) with the weights already resolved
+ * by mq_moe_route_topk; also RunMoEQ4KRawBatchedWeightedScatterProjectionImpl
+ * (core/src/backend/cpu_backend_moe_raw_batched.inl:1437-1492). */
+int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev, int64_t n, const int32_t* ids_dev,
+                             const float* weights_dev, int top_k, float* y_dev, void* stream);
 
 /* ---- fused MoE layer -------------------------------------------------------------
  * The four custom nodes of TryBuildQwen35NativeMoEGraph

@@ -202,6 +202,17 @@ def ffn_swiglu(gate, up, down, hidden: int, inter: int, x, order=ORDER_DOTPROD, 
     return (y, mid) if want_inter else y
 
 
+def swiglu_mul_mat(gate, up, hidden: int, inter: int, x, order=ORDER_DOTPROD, silu=SILU_EXACT):
+    gate, up = _c(gate, np.uint8), _c(up, np.uint8)
+    x = _c(x, np.float32)
+    out = np.zeros((x.shape[0], inter), np.float32)
+    rc = lib().orc_swiglu_mul_mat_q4k_f32(_p(gate), _p(up), C.c_int64(inter), C.c_int64(hidden), _p(x),
+                                          C.c_int64(x.shape[0]), _p(out), C.c_int(order), C.c_int(silu))
+    if rc:
+        raise ValueError(f"orc_swiglu_mul_mat_q4k_f32 rc={rc}")
+    return out
+
+
 def route_topk(logits, top_k: int, weights_mode: int = 0):
     logits = _c(logits, np.float32)
     n, e = logits.shape
@@ -227,6 +238,44 @@ class _MoEWeights(C.Structure):
                 ("gate_exps", C.c_void_p), ("up_exps", C.c_void_p), ("down_exps", C.c_void_p),
                 ("sh_gate", C.c_void_p), ("sh_up", C.c_void_p), ("sh_down", C.c_void_p),
                 ("sh_gate_inp", C.c_void_p)]
+
+
+def _moe_w(gate_exps, up_exps, down_exps, hidden, inter, top_k, keep):
+    n_exp = (gate_exps if gate_exps is not None else down_exps).shape[0]
+    W = _MoEWeights(hidden, inter, n_exp, top_k, None, None, None, None, None, None, None)
+    for name, arr in (("gate_exps", gate_exps), ("up_exps", up_exps), ("down_exps", down_exps)):
+        if arr is not None:
+            a = _c(arr, np.uint8)
+            keep.append(a)
+            setattr(W, name, a.ctypes.data)
+    return W
+
+
+def moe_gateup_swiglu(gate_exps, up_exps, hidden, inter, x, ids, order=ORDER_DOTPROD, silu=SILU_EXACT):
+    keep = []
+    ids = _c(ids, np.int32)
+    x = _c(x, np.float32)
+    W = _moe_w(gate_exps, up_exps, None, hidden, inter, ids.shape[1], keep)
+    out = np.zeros((x.shape[0], ids.shape[1], inter), np.float32)
+    rc = lib().orc_moe_gateup_swiglu(C.byref(W), _p(x), _p(ids), C.c_int64(x.shape[0]), C.c_int(order), C.c_int(silu),
+                                     _p(out))
+    if rc:
+        raise ValueError(f"orc_moe_gateup_swiglu rc={rc}")
+    return out
+
+
+def moe_down_weighted(down_exps, hidden, inter, hid, ids, weights, order=ORDER_DOTPROD, accumulate_mode=0):
+    keep = []
+    ids = _c(ids, np.int32)
+    hid = _c(hid, np.float32)
+    weights = _c(weights, np.float32)
+    W = _moe_w(None, None, down_exps, hidden, inter, ids.shape[1], keep)
+    y = np.zeros((ids.shape[0], hidden), np.float32)
+    rc = lib().orc_moe_down_weighted(C.byref(W), _p(hid), _p(ids), _p(weights), C.c_int64(ids.shape[0]),
+                                     C.c_int(order), C.c_int(accumulate_mode), _p(y))
+    if rc:
+        raise ValueError(f"orc_moe_down_weighted rc={rc}")
+    return y
 
 
 def moe_layer(gate_exps, up_exps, down_exps, hidden, inter, top_k, x, logits, shared=None, order=ORDER_DOTPROD,

@@ -432,6 +432,22 @@ int orc_mul_mat_q4k_f32(const void* w, int64_t rows, int64_t cols, size_t row_by
 }
 
 /* ------------------------------------------------------------------ */
+/* fused gate/up + SwiGLU on one activation set (hwy_moe_quant.cc:359-380) */
+/* ------------------------------------------------------------------ */
+int orc_swiglu_mul_mat_q4k_f32(const void* gate, const void* up, int64_t inter, int64_t hidden, const float* x,
+                               int64_t n, float* out, int order, int silu_mode) {
+    if (!gate || !up || !x || !out || hidden <= 0 || hidden % ORC_QK_K || inter <= 0) return -1;
+    const size_t wrow = (size_t)(hidden / ORC_QK_K) * sizeof(orc_block_q4k);
+    float* u = (float*)malloc(sizeof(float) * (size_t)n * (size_t)inter);
+    if (!u) return -2;
+    int rc = orc_mul_mat_q4k_f32(gate, inter, hidden, wrow, x, n, hidden, out, inter, order);
+    if (rc == 0) rc = orc_mul_mat_q4k_f32(up, inter, hidden, wrow, x, n, hidden, u, inter, order);
+    for (int64_t i = 0; rc == 0 && i < n * inter; ++i) out[i] = orc_silu_mul(out[i], u[i], silu_mode);
+    free(u);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ */
 /* dense SwiGLU FFN                                                     */
 /* ------------------------------------------------------------------ */
 int orc_ffn_swiglu_q4k(const void* gate, const void* up, const void* down, int64_t hidden, int64_t inter,
@@ -592,106 +608,129 @@ static float stable_sigmoid(float x) { /* fused_ops.cpp:451-458 */
     return z / (1.0f + z);
 }
 
+/* hidden[t][k][r] = silu(gate_e[r] . q8(x[t])) * (up_e[r] . q8(x[t])), e = ids[t][k]
+ * (native.cpp:4306-4342 / hwy_moe_quant.cc:359-380; raw_batched.inl:1629-1698 for n > 4).
+ * Entries whose id is outside [0, n_experts) are left untouched. */
+int orc_moe_gateup_swiglu(const orc_moe_weights* w, const float* x, const int32_t* ids, int64_t n_tokens, int order,
+                          int silu_mode, float* hidden) {
+    if (!w || !x || !ids || !hidden || w->hidden % ORC_QK_K) return -1;
+    const int64_t H = w->hidden, I = w->inter;
+    const int K = w->top_k;
+    const size_t row_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t exp_in = row_in * (size_t)I;
+    const size_t q8_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q8k);
+    uint8_t* xq = (uint8_t*)malloc(q8_in * (size_t)n_tokens);
+    if (!xq) return -2;
+    int rc = orc_quantize_rows_q8k(x, n_tokens, H, xq, H);
+    for (int64_t t = 0; rc == 0 && t < n_tokens; ++t) {
+        for (int k = 0; k < K; ++k) {
+            const int32_t e = ids[t * K + k];
+            if (e < 0 || e >= w->n_experts) continue;
+            const uint8_t* ge = (const uint8_t*)w->gate_exps + (size_t)e * exp_in;
+            const uint8_t* ue = (const uint8_t*)w->up_exps + (size_t)e * exp_in;
+            float* h = hidden + ((size_t)t * K + k) * (size_t)I;
+            for (int64_t r = 0; r < I; ++r) {
+                const float g = orc_dot_q4k_q8k(ge + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
+                const float u = orc_dot_q4k_q8k(ue + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
+                h[r] = orc_silu_mul(g, u, silu_mode);
+            }
+        }
+    }
+    free(xq);
+    return rc;
+}
+
+/* y[t][r] = sum over routed experts of weights[t][k] * (down_e[r] . q8(hidden[t][k])).
+ * accumulate_mode 0: per token, k = 0..top_k-1 in routing order (native.cpp:3233-3285);
+ * accumulate_mode 1: expert-sorted assignment order (native.cpp:3152-3194). */
+int orc_moe_down_weighted(const orc_moe_weights* w, const float* hidden, const int32_t* ids, const float* weights,
+                          int64_t n_tokens, int order, int accumulate_mode, float* y) {
+    if (!w || !hidden || !ids || !weights || !y || w->inter % ORC_QK_K) return -1;
+    const int64_t H = w->hidden, I = w->inter, E = w->n_experts;
+    const int K = w->top_k;
+    const size_t row_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t exp_mid = row_mid * (size_t)H;
+    const size_t q8_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q8k);
+    uint8_t* hq = (uint8_t*)malloc(q8_mid * (size_t)n_tokens * K);
+    orc_assignment* asg = (orc_assignment*)malloc(sizeof(orc_assignment) * (size_t)n_tokens * K);
+    if (!hq || !asg) {
+        free(hq);
+        free(asg);
+        return -2;
+    }
+    orc_quantize_rows_q8k(hidden, n_tokens * K, I, hq, I);
+    memset(y, 0, sizeof(float) * (size_t)n_tokens * (size_t)H);
+    const int64_t cnt = orc_build_assignments(ids, n_tokens, K, E, asg);
+    if (accumulate_mode == 0) { /* re-sort the valid entries into (token, k) order */
+        int64_t c = 0;
+        for (int64_t t = 0; t < n_tokens; ++t)
+            for (int k = 0; k < K; ++k) {
+                const int32_t e = ids[t * K + k];
+                if (e < 0 || e >= E) continue;
+                asg[c].expert = e;
+                asg[c].token = (int32_t)t;
+                asg[c].k = k;
+                ++c;
+            }
+    }
+    for (int64_t a = 0; a < cnt; ++a) {
+        const float gw = weights[(size_t)asg[a].token * K + asg[a].k];
+        if (gw == 0.0f) continue; /* native.cpp:3237 */
+        const uint8_t* de = (const uint8_t*)w->down_exps + (size_t)asg[a].expert * exp_mid;
+        const uint8_t* q = hq + ((size_t)asg[a].token * K + asg[a].k) * q8_mid;
+        for (int64_t r = 0; r < H; ++r) {
+            const float v = orc_dot_q4k_q8k(de + (size_t)r * row_mid, q, I, order);
+            y[(size_t)asg[a].token * H + r] += v * gw;
+        }
+    }
+    free(hq);
+    free(asg);
+    return 0;
+}
+
+/* Shared expert: dense FFN (fast-exp SiLU on the contiguous dense path, fused_ops.cpp:342-343),
+ * scaled by sigmoid(sh_gate_inp . x) (fused_ops.cpp:437-475), added to y (decoder.cpp:2600). */
+int orc_moe_add_shared(const orc_moe_weights* w, const float* x, int64_t n_tokens, int order, float* y) {
+    if (!w->sh_gate || !w->sh_up || !w->sh_down) return 0;
+    const int64_t H = w->hidden, I = w->inter;
+    float* sh = (float*)malloc(sizeof(float) * (size_t)n_tokens * (size_t)H);
+    if (!sh) return -2;
+    int rc = orc_ffn_swiglu_q4k(w->sh_gate, w->sh_up, w->sh_down, H, I, x, n_tokens, sh, order, ORC_SILU_FAST_FMA, NULL);
+    for (int64_t t = 0; rc == 0 && t < n_tokens; ++t) {
+        float scale = 1.0f;
+        if (w->sh_gate_inp) {
+            double acc = 0.0;
+            for (int64_t c = 0; c < H; ++c) acc += (double)w->sh_gate_inp[c] * (double)x[t * H + c];
+            scale = stable_sigmoid((float)acc);
+        }
+        for (int64_t r = 0; r < H; ++r) {
+            const float s = sh[t * H + r] * scale;
+            y[t * H + r] = y[t * H + r] + s;
+        }
+    }
+    free(sh);
+    return rc;
+}
+
 int orc_moe_layer(const orc_moe_weights* w, const float* x, const float* logits, int64_t n_tokens, float* y,
                   int order, int silu_mode, int weights_mode, int accumulate_mode, int32_t* ids_out,
                   float* weights_out, float* hidden_out) {
     if (!w || !x || !logits || !y || n_tokens <= 0 || w->hidden % ORC_QK_K || w->inter % ORC_QK_K || w->top_k <= 0)
         return -1;
-    const int64_t H = w->hidden, I = w->inter, E = w->n_experts;
     const int K = w->top_k;
-    const size_t row_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q4k);  /* gate/up row */
-    const size_t row_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q4k); /* down row   */
-    const size_t exp_in = row_in * (size_t)I, exp_mid = row_mid * (size_t)H;
-    const size_t q8_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q8k);
-    const size_t q8_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q8k);
-
     int32_t* ids = (int32_t*)malloc(sizeof(int32_t) * (size_t)n_tokens * K);
     float* wts = (float*)malloc(sizeof(float) * (size_t)n_tokens * K);
-    float* hid = (float*)malloc(sizeof(float) * (size_t)n_tokens * K * (size_t)I);
-    uint8_t* xq = (uint8_t*)malloc(q8_in * (size_t)n_tokens);
-    uint8_t* hq = (uint8_t*)malloc(q8_mid * (size_t)n_tokens * K);
-    orc_assignment* asg = (orc_assignment*)malloc(sizeof(orc_assignment) * (size_t)n_tokens * K);
-    int rc = (ids && wts && hid && xq && hq && asg) ? 0 : -2;
-
-    if (rc == 0) rc = orc_route_topk(logits, E, n_tokens, K, weights_mode, ids, wts);
-    if (rc == 0) rc = orc_quantize_rows_q8k(x, n_tokens, H, xq, H);
-    if (rc == 0) {
-        /* gate/up + SwiGLU: hidden[t][k][r] (native.cpp:4306-4342 / hwy_moe_quant.cc:359-380) */
-        for (int64_t t = 0; t < n_tokens; ++t) {
-            for (int k = 0; k < K; ++k) {
-                const int32_t e = ids[t * K + k];
-                const uint8_t* ge = (const uint8_t*)w->gate_exps + (size_t)e * exp_in;
-                const uint8_t* ue = (const uint8_t*)w->up_exps + (size_t)e * exp_in;
-                float* h = hid + ((size_t)t * K + k) * (size_t)I;
-                for (int64_t r = 0; r < I; ++r) {
-                    const float g = orc_dot_q4k_q8k(ge + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
-                    const float u = orc_dot_q4k_q8k(ue + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
-                    h[r] = orc_silu_mul(g, u, silu_mode);
-                }
-                orc_quantize_row_q8k(h, hq + ((size_t)t * K + k) * q8_mid, I);
-            }
-        }
-        memset(y, 0, sizeof(float) * (size_t)n_tokens * (size_t)H);
-        if (accumulate_mode == 0) {
-            for (int64_t t = 0; t < n_tokens; ++t) {
-                for (int k = 0; k < K; ++k) {
-                    const float gw = wts[t * K + k];
-                    if (gw == 0.0f) continue; /* native.cpp:3237 */
-                    const uint8_t* de = (const uint8_t*)w->down_exps + (size_t)ids[t * K + k] * exp_mid;
-                    const uint8_t* q = hq + ((size_t)t * K + k) * q8_mid;
-                    for (int64_t r = 0; r < H; ++r) {
-                        const float v = orc_dot_q4k_q8k(de + (size_t)r * row_mid, q, I, order);
-                        y[t * H + r] += v * gw;
-                    }
-                }
-            }
-        } else {
-            const int64_t cnt = orc_build_assignments(ids, n_tokens, K, E, asg);
-            for (int64_t a = 0; a < cnt; ++a) {
-                const float gw = wts[(size_t)asg[a].token * K + asg[a].k];
-                if (gw == 0.0f) continue;
-                const uint8_t* de = (const uint8_t*)w->down_exps + (size_t)asg[a].expert * exp_mid;
-                const uint8_t* q = hq + ((size_t)asg[a].token * K + asg[a].k) * q8_mid;
-                for (int64_t r = 0; r < H; ++r) {
-                    const float v = orc_dot_q4k_q8k(de + (size_t)r * row_mid, q, I, order);
-                    y[(size_t)asg[a].token * H + r] += v * gw;
-                }
-            }
-        }
-        /* shared expert: dense FFN (fast-exp SiLU on the contiguous dense path,
-         * fused_ops.cpp:342-343), scaled by sigmoid(sh_gate_inp . x), added
-         * (decoder.cpp:2470-2600). */
-        if (w->sh_gate && w->sh_up && w->sh_down) {
-            float* sh = (float*)malloc(sizeof(float) * (size_t)n_tokens * (size_t)H);
-            if (!sh) {
-                rc = -2;
-            } else {
-                rc = orc_ffn_swiglu_q4k(w->sh_gate, w->sh_up, w->sh_down, H, I, x, n_tokens, sh, order,
-                                        ORC_SILU_FAST_FMA, NULL);
-                for (int64_t t = 0; rc == 0 && t < n_tokens; ++t) {
-                    float scale = 1.0f;
-                    if (w->sh_gate_inp) {
-                        double acc = 0.0;
-                        for (int64_t c = 0; c < H; ++c) acc += (double)w->sh_gate_inp[c] * (double)x[t * H + c];
-                        scale = stable_sigmoid((float)acc);
-                    }
-                    for (int64_t r = 0; r < H; ++r) {
-                        const float s = sh[t * H + r] * scale;
-                        y[t * H + r] = y[t * H + r] + s;
-                    }
-                }
-                free(sh);
-            }
-        }
-    }
+    float* hid = (float*)calloc((size_t)n_tokens * K * (size_t)w->inter, sizeof(float));
+    int rc = (ids && wts && hid) ? 0 : -2;
+    if (rc == 0) rc = orc_route_topk(logits, w->n_experts, n_tokens, K, weights_mode, ids, wts);
+    if (rc == 0) rc = orc_moe_gateup_swiglu(w, x, ids, n_tokens, order, silu_mode, hid);
+    if (rc == 0) rc = orc_moe_down_weighted(w, hid, ids, wts, n_tokens, order, accumulate_mode, y);
+    if (rc == 0) rc = orc_moe_add_shared(w, x, n_tokens, order, y);
     if (rc == 0 && ids_out) memcpy(ids_out, ids, sizeof(int32_t) * (size_t)n_tokens * K);
     if (rc == 0 && weights_out) memcpy(weights_out, wts, sizeof(float) * (size_t)n_tokens * K);
-    if (rc == 0 && hidden_out) memcpy(hidden_out, hid, sizeof(float) * (size_t)n_tokens * K * (size_t)I);
+    if (rc == 0 && hidden_out) memcpy(hidden_out, hid, sizeof(float) * (size_t)n_tokens * K * (size_t)w->inter);
     free(ids);
     free(wts);
     free(hid);
-    free(xq);
-    free(hq);
-    free(asg);
     return rc;
 }

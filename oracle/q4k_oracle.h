@@ -117,6 +117,10 @@ int orc_mul_mat_q4k_q8k(const void* w, int64_t rows, int64_t cols, size_t row_by
 int orc_mul_mat_q4k_f32(const void* w, int64_t rows, int64_t cols, size_t row_bytes, const float* x, int64_t n,
                         int64_t ldx, float* out, int64_t ldo, int order);
 
+/* out[m][r] = silu(gate[r] . q8(x[m])) * (up[r] . q8(x[m])) */
+int orc_swiglu_mul_mat_q4k_f32(const void* gate, const void* up, int64_t inter, int64_t hidden, const float* x,
+                               int64_t n, float* out, int order, int silu_mode);
+
 /* ---- dense SwiGLU FFN: y = down( silu(gate x) * (up x) ) --------------- */
 int orc_ffn_swiglu_q4k(const void* gate, const void* up, const void* down, int64_t hidden, int64_t inter,
                        const float* x, int64_t n, float* y, int order, int silu_mode, float* inter_out);
@@ -150,6 +154,12 @@ typedef struct {
     const void* sh_down;
     const float* sh_gate_inp; /* [hidden] fp32 scalar-gate vector, may be NULL */
 } orc_moe_weights;
+
+int orc_moe_gateup_swiglu(const orc_moe_weights* w, const float* x, const int32_t* ids, int64_t n_tokens, int order,
+                          int silu_mode, float* hidden /* [n][top_k][inter] */);
+int orc_moe_down_weighted(const orc_moe_weights* w, const float* hidden, const int32_t* ids, const float* weights,
+                          int64_t n_tokens, int order, int accumulate_mode, float* y);
+int orc_moe_add_shared(const orc_moe_weights* w, const float* x, int64_t n_tokens, int order, float* y);
 
 /* accumulate_mode 0: per token, k = 0..top_k-1 in routing order (native.cpp:3233-3285)
  * accumulate_mode 1: expert-sorted assignment order (native.cpp:3152-3194) */

@@ -1,0 +1,245 @@
+"""GPU parity: fused gate/up SwiGLU, the dense FFN, the router, expert grouping and the MoE layer.
+
+Chained operators are checked stage by stage with the GPU's own intermediate fed to the oracle
+("teacher forcing"): a Q8_K re-quantization sits between gate/up and down, so an intermediate that
+differs by one fp32 ulp can flip an int8 code, and an end-to-end comparison would measure that
+discontinuity instead of the kernels.  The end-to-end checks use a looser, stated bound.
+"""
+import numpy as np
+import pytest
+
+from densecore_amd import synth
+from oracle import binding as orc
+from tests._parity import assert_fp32_parity
+
+pytestmark = pytest.mark.gpu
+
+SILU_REL = 1e-4      # on top of a small absolute floor: silu(g)*u is a product of two 1e-4-accurate dots
+END_TO_END_REL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    from densecore_amd import ops as o
+    assert torch.cuda.is_available()
+    return o
+
+
+def cu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close_prod(got, ref, what):
+    """Elementwise product outputs: 1e-4 relative plus 1e-5 of the row's rms as the absolute floor."""
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    floor = 1e-5 * np.sqrt(np.mean(ref ** 2, axis=-1, keepdims=True))
+    assert np.all(np.abs(got - ref) <= SILU_REL * np.abs(ref) + floor), what
+
+
+def down_mag(w, cols, x):
+    q8 = orc.quantize_rows_q8k(x)
+    return orc.dot_magnitude_f64(w, cols, q8)
+
+
+@pytest.mark.parametrize("n", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("silu", [0, 1, 2])
+def test_swiglu_and_ffn_stagewise(ops, n, silu):
+    H, I = 1024, 1792
+    g, u, d = (synth.q4k_matrix(synth.tensor_seed("ffn", nm), r, c) for nm, r, c in
+               (("g", I, H), ("u", I, H), ("d", H, I)))
+    x = synth.normal_f32(synth.tensor_seed("ffn-x", n), (n, H))
+    G, U, D = ops.Q4KWeight.from_ggml(g, H), ops.Q4KWeight.from_ggml(u, H), ops.Q4KWeight.from_ggml(d, I)
+    h_gpu = ops.swiglu_mul_mat(G, U, cu(x), silu).cpu().numpy()
+    for order in orc.ORDERS.values():
+        assert_close_prod(h_gpu, orc.swiglu_mul_mat(g, u, H, I, x, order, silu), f"swiglu order={order}")
+    y_gpu = ops.ffn_swiglu(G, U, D, cu(x), silu).cpu().numpy()
+    # the fused FFN is exactly swiglu -> mul_mat
+    y_comp = ops.mul_mat(D, cu(h_gpu)).cpu().numpy()
+    assert np.array_equal(y_gpu.view(np.uint32), y_comp.view(np.uint32))
+    # down stage against the oracle on the GPU's own intermediate
+    mag = down_mag(d, I, h_gpu)
+    for name, order in orc.ORDERS.items():
+        assert_fp32_parity(y_gpu, orc.mul_mat_q4k_f32(d, I, h_gpu, order), mag, f"ffn-down order={name}")
+    # end to end against the oracle
+    y_ref = orc.ffn_swiglu(g, u, d, H, I, x, orc.ORDER_DOTPROD, silu)
+    assert np.max(np.abs(y_gpu - y_ref)) <= END_TO_END_REL * np.max(np.abs(y_ref))
+    for w in (G, U, D):
+        w.free()
+
+
+def test_ffn_full_size_single_token(ops):
+    """The dense FFN shape of the benchmark (4096 -> 14336 -> 4096) at one token."""
+    H, I = 4096, 14336
+    seeds = [synth.tensor_seed("cfg2", nm) for nm in "gud"]
+    G, U, D = (ops.Q4KWeight.synthetic(s, r, c) for s, (r, c) in zip(seeds, ((I, H), (I, H), (H, I))))
+    g, u, d = G.to_ggml(), U.to_ggml(), D.to_ggml()
+    x = synth.normal_f32(synth.tensor_seed("cfg2-x"), (1, H))
+    h_gpu = ops.swiglu_mul_mat(G, U, cu(x), 2).cpu().numpy()
+    assert_close_prod(h_gpu, orc.swiglu_mul_mat(g, u, H, I, x, orc.ORDER_DOTPROD, 2), "swiglu")
+    y_gpu = ops.ffn_swiglu(G, U, D, cu(x), 2).cpu().numpy()
+    assert_fp32_parity(y_gpu, orc.mul_mat_q4k_f32(d, I, h_gpu, orc.ORDER_DOTPROD), down_mag(d, I, h_gpu), "down")
+    for w in (G, U, D):
+        w.free()
+
+
+def reference_patterned_floats(rows, cols, scale):
+    """Input recipe of the reference's MoE tests (core/tests/moe/test_moe_ops.cpp:119-129)."""
+    r = np.arange(rows)[:, None]
+    c = np.arange(cols)[None, :]
+    return (((r * 17 + c * 29 + 7) % 41) - 20).astype(np.float32) * np.float32(scale)
+
+
+def test_matmul_on_the_references_patterned_inputs(ops):
+    rows, cols, n = 64, 512, 3
+    w = synth.q4k_matrix(3, rows, cols)
+    x = reference_patterned_floats(n, cols, 0.03125)
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    y = ops.mul_mat(W, cu(x)).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    assert np.array_equal(ops.quantize_row_q8_k(cu(x)).cpu().numpy(), q8)
+    assert_fp32_parity(y, orc.mul_mat_q4k_q8k(w, cols, q8, orc.ORDER_HWY), orc.dot_magnitude_f64(w, cols, q8), "pattern")
+    # the reference's own acceptance bound for this kernel family is 1e-4 absolute on such inputs
+    # (core/tests/moe/test_moe_ops.cpp:327)
+    assert np.max(np.abs(y - orc.dot_dequant_f64(w, cols, q8))) < 1e-4 * max(1.0, np.max(np.abs(y)))
+    W.free()
+
+
+# ----------------------------------------------------------------------------- router
+@pytest.mark.parametrize("n,e,k", [(1, 256, 8), (4, 256, 8), (16, 256, 8), (64, 256, 8), (7, 60, 4), (3, 8, 8),
+                                   (5, 1000, 6)])
+def test_router_ids_exact_weights_close(ops, n, e, k):
+    logits = synth.normal_f32(synth.tensor_seed("route", n, e, k), (n, e))
+    if n > 2:
+        logits[1, 3] = logits[1, e - 1] = logits[1].max() + 1.0   # tie at the top
+        logits[2, :] = 0.5                                         # all equal
+    for mode in (0, 1, 2):
+        ids, w = ops.moe_route_topk(cu(logits), k, mode)
+        oi, ow = orc.route_topk(logits, k, mode)
+        assert np.array_equal(ids.cpu().numpy(), oi), f"mode {mode}"
+        assert np.allclose(w.cpu().numpy(), ow, rtol=3e-6, atol=1e-9), f"mode {mode}"
+
+
+def test_router_nan_and_inf_rows(ops):
+    logits = synth.normal_f32(5, (4, 64))
+    logits[0, 10] = np.nan
+    logits[1, :] = -np.inf
+    logits[2, 7] = np.inf
+    logits[3, :32] = np.nan
+    for mode in (0, 1, 2):
+        ids, w = ops.moe_route_topk(cu(logits), 8, mode)
+        oi, ow = orc.route_topk(logits, 8, mode)
+        assert np.array_equal(ids.cpu().numpy(), oi), f"mode {mode}"
+        assert np.allclose(w.cpu().numpy(), ow, rtol=3e-6, atol=1e-9, equal_nan=True), f"mode {mode}"
+
+
+# ----------------------------------------------------------------------------- expert-routed matmul
+def make_experts(tag, E, H, I):
+    ge = np.stack([synth.q4k_matrix(synth.tensor_seed(tag, "g", e), I, H) for e in range(E)])
+    ue = np.stack([synth.q4k_matrix(synth.tensor_seed(tag, "u", e), I, H) for e in range(E)])
+    de = np.stack([synth.q4k_matrix(synth.tensor_seed(tag, "d", e), H, I) for e in range(E)])
+    return ge, ue, de
+
+
+@pytest.mark.parametrize("n", [1, 4, 16, 40])
+def test_mul_mat_id_matches_per_pair_dense_results(ops, n):
+    E, H, I, K = 12, 512, 256, 4
+    ge, _, de = make_experts("mmid", E, H, I)
+    GE, DE = ops.Q4KWeight.from_ggml(ge, H), ops.Q4KWeight.from_ggml(de, I)
+    x = synth.normal_f32(synth.tensor_seed("mmid-x", n), (n, H))
+    ids, _ = orc.route_topk(synth.normal_f32(synth.tensor_seed("mmid-l", n), (n, E)), K, 0)
+    if n >= 4:
+        ids[1, 2] = -1        # invalid ids produce zero rows
+        ids[2, 0] = E + 3
+    y = ops.mul_mat_id(GE, cu(x), cu(ids)).cpu().numpy()                      # x broadcast over k
+    xk = synth.normal_f32(synth.tensor_seed("mmid-xk", n), (n, K, I))
+    yk = ops.mul_mat_id(DE, cu(xk), cu(ids)).cpu().numpy()                    # one row per (token, k)
+    for t in range(n):
+        for k in range(K):
+            e = ids[t, k]
+            if e < 0 or e >= E:
+                assert not y[t, k].any() and not yk[t, k].any()
+                continue
+            q8 = orc.quantize_rows_q8k(x[t:t + 1])
+            assert_fp32_parity(y[t, k][None], orc.mul_mat_q4k_q8k(ge[e], H, q8), orc.dot_magnitude_f64(ge[e], H, q8),
+                               f"t{t}k{k}")
+            q8 = orc.quantize_rows_q8k(xk[t, k][None])
+            assert_fp32_parity(yk[t, k][None], orc.mul_mat_q4k_q8k(de[e], I, q8), orc.dot_magnitude_f64(de[e], I, q8),
+                               f"down t{t}k{k}")
+    GE.free()
+    DE.free()
+
+
+# ----------------------------------------------------------------------------- MoE layer
+@pytest.mark.parametrize("n,silu", [(1, 0), (4, 0), (16, 1), (64, 1)])
+def test_moe_layer_stagewise(ops, n, silu):
+    """Benchmark MoE layer shape (hidden 2048, inter 512, top-8, shared expert) with 24 experts so
+    the scalar oracle finishes in seconds."""
+    E, H, I, K = 24, 2048, 512, 8
+    ge, ue, de = make_experts("moe", E, H, I)
+    sg, su, sd = (synth.q4k_matrix(synth.tensor_seed("moe-sh", nm), r, c) for nm, r, c in
+                  (("g", I, H), ("u", I, H), ("d", H, I)))
+    gate_inp = synth.normal_f32(synth.tensor_seed("moe-gi"), (H,)) * np.float32(0.02)
+    x = synth.normal_f32(synth.tensor_seed("moe-x", n), (n, H))
+    logits = synth.normal_f32(synth.tensor_seed("moe-l", n), (n, E))
+    GE, UE, DE = ops.Q4KWeight.from_ggml(ge, H), ops.Q4KWeight.from_ggml(ue, H), ops.Q4KWeight.from_ggml(de, I)
+    SG, SU, SD = ops.Q4KWeight.from_ggml(sg, H), ops.Q4KWeight.from_ggml(su, H), ops.Q4KWeight.from_ggml(sd, I)
+
+    ids_t, w_t = ops.moe_route_topk(cu(logits), K, 0)
+    ids, wts = ids_t.cpu().numpy(), w_t.cpu().numpy()
+    oi, ow = orc.route_topk(logits, K, 0)
+    assert np.array_equal(ids, oi) and np.allclose(wts, ow, rtol=3e-6)
+
+    # stage 1: gate/up + SwiGLU per (token, k)
+    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids_t, silu).cpu().numpy()
+    assert_close_prod(hid, orc.moe_gateup_swiglu(ge, ue, H, I, x, ids, orc.ORDER_DOTPROD, silu), "gate/up")
+
+    # stage 2: down + weighted sum in routing order, on the GPU's own hidden and weights
+    y_routed = ops.moe_down_weighted(DE, cu(hid), ids_t, w_t).cpu().numpy()
+    y_ref = orc.moe_down_weighted(de, H, I, hid, ids, wts, orc.ORDER_DOTPROD, 0)
+    # magnitude: weighted sum of the per-expert magnitudes
+    mag = np.zeros((n, H))
+    for t in range(n):
+        for k in range(K):
+            q8 = orc.quantize_rows_q8k(hid[t, k][None])
+            mag[t] += abs(wts[t, k]) * orc.dot_magnitude_f64(de[ids[t, k]], I, q8)[0]
+    assert_fp32_parity(y_routed, y_ref, mag, "down routing-order")
+    assert_fp32_parity(y_routed, orc.moe_down_weighted(de, H, I, hid, ids, wts, orc.ORDER_AVX2, 1), mag,
+                       "down expert-order")
+
+    # whole layer: equals its own stages plus the shared expert; end to end against the oracle
+    y, ids2, w2 = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=(SG, SU, SD, cu(gate_inp)), silu=silu)
+    assert np.array_equal(ids2.cpu().numpy(), ids) and np.array_equal(w2.cpu().numpy().view(np.uint32), wts.view(np.uint32))
+    y_nosh, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=silu)
+    assert np.array_equal(y_nosh.cpu().numpy().view(np.uint32), y_routed.view(np.uint32))
+    ref = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=(sg, su, sd, gate_inp), silu=silu)
+    y = y.cpu().numpy()
+    assert np.max(np.abs(y - ref["y"])) <= END_TO_END_REL * np.max(np.abs(ref["y"]))
+    # shared expert alone = layer - routed part, against the dense FFN path scaled by the sigmoid gate
+    sh_gpu = ops.ffn_swiglu(SG, SU, SD, cu(x), 2).cpu().numpy()
+    gate = 1.0 / (1.0 + np.exp(-(x.astype(np.float64) @ gate_inp.astype(np.float64))))
+    want = y_routed.astype(np.float64) + sh_gpu.astype(np.float64) * gate[:, None]
+    assert np.max(np.abs(y - want)) <= 2e-6 * np.max(np.abs(want))
+    for w in (GE, UE, DE, SG, SU, SD):
+        w.free()
+
+
+def test_moe_layer_zero_weight_and_duplicate_free_paths(ops):
+    """One token whose logits make a single expert take all the weight: the others' weights underflow
+    to exactly zero in fp32 and are skipped (core/src/llm/moe/native.cpp:3237)."""
+    E, H, I, K = 8, 256, 256, 8
+    ge, ue, de = make_experts("moe0", E, H, I)
+    GE, UE, DE = ops.Q4KWeight.from_ggml(ge, H), ops.Q4KWeight.from_ggml(ue, H), ops.Q4KWeight.from_ggml(de, I)
+    x = synth.normal_f32(91, (2, H))
+    logits = np.zeros((2, E), np.float32)
+    logits[0, 5] = 200.0
+    logits[1] = np.linspace(-1, 1, E)
+    y, ids, w = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, silu=0)
+    w = w.cpu().numpy()
+    assert w[0, 0] == 1.0 and not w[0, 1:].any()
+    ref = orc.moe_layer(ge, ue, de, H, I, K, x, logits, silu=0)
+    assert np.array_equal(ids.cpu().numpy(), ref["ids"])
+    assert np.max(np.abs(y.cpu().numpy() - ref["y"])) <= END_TO_END_REL * np.max(np.abs(ref["y"]))
+    for t in (GE, UE, DE):
+        t.free()
