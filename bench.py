@@ -1,0 +1,287 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q4_K x Q8_K hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[1]): the dense FFN-shaped skinny GEMM -- Q4_K gate/up
+4096->14336 (fused with the SiLU gate) and down 14336->4096 -- at the decode widths
+n = 1, 2, 4, 8, 16.  One step = one FFN pass at each of the five widths, each pass on the next
+weight set of a ring of distinct sets (792 MB, larger than every cache level), so the weights
+always come from HBM.  Activations and weights are resident in HBM before the timed region; the
+steps are replayed as HIP graphs (what a serving loop does) unless --eager is given.
+
+Prints one JSON line: whole-job GB/s over the algorithmic bytes (weights once, fp32 activations in,
+fp32 outputs out), the roofline of the dominant kernel (fused gate/up), and the CPU baseline (the
+oracle's AVX2 + threads build on this box's host cores, bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HIDDEN, INTER = 4096, 14336
+WIDTHS = (1, 2, 4, 8, 16)
+RING = 8
+HBM_PEAK_GBPS = 8000.0
+Q4K_MATRIX_BYTES = INTER * (HIDDEN // 256) * 144          # 33,030,144: the same for gate, up and down
+
+
+def ffn_bytes(n: int) -> int:
+    """Algorithmic bytes of one FFN pass: three weight matrices once, fp32 x in, fp32 y out."""
+    return 3 * Q4K_MATRIX_BYTES + n * (HIDDEN * 4 + HIDDEN * 4)
+
+
+def gateup_bytes(n: int) -> int:
+    """Algorithmic bytes of one fused gate/up launch: two matrices, fp32 x in, fp32 hidden out."""
+    return 2 * Q4K_MATRIX_BYTES + n * (HIDDEN * 4 + INTER * 4)
+
+
+def moe_bytes(n: int, distinct: int) -> int:
+    """One MoE layer (hidden 2048, inter 512): distinct routed experts + the shared one, x in, y out."""
+    return (distinct + 1) * 3 * 512 * 8 * 144 + n * (2048 * 4 * 2)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--eager", action="store_true", help="launch from Python every step instead of replaying HIP graphs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the GEMV / MoE side measurements")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU (one MI355X per box); --gpus N with N > 1 is not run. "
+              "How the path would shard over more GPUs is described in DESIGN.md.", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from densecore_amd import ops, synth
+
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    # ---------------------------------------------------------------- resident data
+    sets = []
+    for r in range(RING):
+        sets.append(tuple(ops.Q4KWeight.synthetic(synth.tensor_seed("cfg2", r, nm), rows, cols)
+                          for nm, rows, cols in (("gate", INTER, HIDDEN), ("up", INTER, HIDDEN), ("down", HIDDEN, INTER))))
+    xs = {n: torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg2-x", n), (n, HIDDEN))).to(dev) for n in WIDTHS}
+    torch.cuda.synchronize()
+
+    def run_step(i: int):
+        for j, n in enumerate(WIDTHS):
+            g, u, d = sets[(i * len(WIDTHS) + j) % RING]
+            ops.ffn_swiglu(g, u, d, xs[n], ops.SILU_FAST_FMA)
+
+    for i in range(RING):          # sizes the library workspace before anything is captured
+        run_step(i)
+    torch.cuda.synchronize()
+
+    graphs = None
+    if not args.eager:
+        graphs = []
+        side = torch.cuda.Stream()
+        for i in range(RING):       # step i and step i + RING touch the same weight sets
+            gph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gph, stream=side):
+                run_step(i)
+            graphs.append(gph)
+        torch.cuda.synchronize()
+
+    def step(i: int):
+        if graphs is None:
+            run_step(i)
+        else:
+            graphs[i % RING].replay()
+
+    # ---------------------------------------------------------------- timed region
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    step_bytes = sum(ffn_bytes(n) for n in WIDTHS)
+    value = step_bytes * args.steps / elapsed / 1e9
+
+    # ---------------------------------------------------------------- dominant kernel, live
+    # HIP event pairs recorded by the library on the launch stream around every fused gate/up launch
+    ops.census_reset()
+    ops.census_enable(True)
+    launches = 0
+    for i in range(max(RING, min(args.steps, 48))):
+        run_step(i)
+        launches += len(WIDTHS)
+    torch.cuda.synchronize()
+    ops.census_enable(False)
+    gu = ops.census_read(ops.KIND_DENSE_SWIGLU)
+    dn = ops.census_read(ops.KIND_DENSE)
+    ops.census_reset()
+    gu_bytes = sum(gateup_bytes(n) for n in WIDTHS) / len(WIDTHS)
+    achieved = gu_bytes / (gu["avg_us"] * 1e-6) / 1e9 if gu["avg_us"] > 0 else 0.0
+    roofline = {
+        "bound": "hbm", "kernel": "matmul_kernel<2,1> (fused gate/up + SwiGLU, 14336x4096 x2, n=1..16)",
+        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None, "bytes_per_launch": int(gu_bytes), "avg_us": round(gu["avg_us"], 3),
+        "min_us": round(gu["min_us"], 3), "launches": gu["count"],
+        "down_kernel": {"avg_us": round(dn["avg_us"], 3), "min_us": round(dn["min_us"], 3),
+                        "achieved": round((Q4K_MATRIX_BYTES + 6.2 * (INTER * 4 + HIDDEN * 4)) / (dn["avg_us"] * 1e-6) / 1e9, 1)
+                        if dn["avg_us"] > 0 else 0.0},
+    }
+
+    # ---------------------------------------------------------------- per-width detail
+    per_width = {}
+    for n in WIDTHS:
+        for i in range(RING):
+            ops.ffn_swiglu(*sets[i], xs[n], ops.SILU_FAST_FMA)
+        torch.cuda.synchronize()
+        reps = 64
+        t1 = time.perf_counter()
+        if graphs is None:
+            for i in range(reps):
+                ops.ffn_swiglu(*sets[i % RING], xs[n], ops.SILU_FAST_FMA)
+        else:
+            gph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gph, stream=side):
+                for i in range(RING):
+                    ops.ffn_swiglu(*sets[i], xs[n], ops.SILU_FAST_FMA)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(reps // RING):
+                gph.replay()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t1) / reps
+        per_width[str(n)] = {"us": round(dt * 1e6, 2), "GBps": round(ffn_bytes(n) / dt / 1e9, 1),
+                             "pct_hbm_peak": round(ffn_bytes(n) / dt / 1e9 / HBM_PEAK_GBPS * 100, 1),
+                             "tokens_per_s": round(n / dt, 1)}
+
+    extras = {}
+    if not args.no_extras:
+        extras = side_measurements(ops, synth, torch, np, dev)
+
+    # ---------------------------------------------------------------- CPU baseline (rank 0, N = 1)
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(sets[0], xs, args.cpu_seconds, np)
+
+    out = {
+        "metric": "Q4_K GEMV + MoE mul_mat_id GB/s (% HBM peak); MoE decode tok/s, 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 x int4 -> int32, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "cfg2: dense FFN skinny GEMM, Q4_K gate/up 4096->14336 + SiLU gate + down 14336->4096, "
+                               "widths n=1,2,4,8,16 per step, cold ring of 8 weight sets (792 MB)",
+                   "launch": "eager" if graphs is None else "hip-graph replay",
+                   "bytes_per_step": step_bytes},
+        "pct_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 1),
+        "per_width": per_width,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    out.update(extras)
+    print(json.dumps(out))
+    return 0
+
+
+def side_measurements(ops, synth, torch, np, dev):
+    """cfg1 GEMV and the cfg3 MoE layer, each on a cold ring, replayed as HIP graphs."""
+    res = {}
+    side = torch.cuda.Stream()
+
+    def time_graph(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        gph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gph, stream=side):
+            fn()
+        torch.cuda.synchronize()
+        gph.replay()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(reps):
+            gph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / reps
+
+    # cfg1: 4096 x 4096 GEMV, ring of 64 matrices (604 MB)
+    ring = [ops.Q4KWeight.synthetic(synth.tensor_seed("cfg1", r), 4096, 4096) for r in range(64)]
+    x1 = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg1-x"), (1, 4096))).to(dev)
+    dt = time_graph(lambda: [ops.mul_mat(w, x1) for w in ring], 20) / len(ring)
+    b = 4096 * 16 * 144 + 2 * 4096 * 4
+    res["gemv_4096x4096_n1"] = {"us": round(dt * 1e6, 2), "GBps": round(b / dt / 1e9, 1),
+                                "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+    for w in ring:
+        w.free()
+
+    # cfg3: MoE layer, hidden 2048, 256 + 1 experts, inter 512, top-8; ring of 4 layers (1.8 GB)
+    E, H, I, K = 256, 2048, 512, 8
+    layers = []
+    for r in range(4):
+        ge = ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "gate"), I, H, E)
+        ue = ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "up"), I, H, E)
+        de = ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "down"), H, I, E)
+        sh = (ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "sg"), I, H),
+              ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "su"), I, H),
+              ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "sd"), H, I),
+              torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3", r, "gi"), (H,)) * np.float32(0.02)).to(dev))
+        layers.append((ge, ue, de, sh))
+    moe = {}
+    for n in (1, 4, 16, 64):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))).to(dev)
+        lg = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))).to(dev)
+        silu = ops.SILU_EXACT if n <= 4 else ops.SILU_FAST
+        _, ids, _ = ops.moe_layer(*layers[0][:3], x, lg, K, shared=layers[0][3], silu=silu)
+        distinct = int(torch.unique(ids).numel())
+        dt = time_graph(lambda: [ops.moe_layer(ge, ue, de, x, lg, K, shared=sh, silu=silu)
+                                 for ge, ue, de, sh in layers], 20) / len(layers)
+        b = moe_bytes(n, distinct)
+        moe[str(n)] = {"us": round(dt * 1e6, 2), "distinct_experts": distinct, "GBps": round(b / dt / 1e9, 1),
+                       "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1), "tokens_per_s": round(n / dt, 1)}
+    res["moe_layer_mul_mat_id"] = moe
+    return res
+
+
+def cpu_baseline(weight_set, xs, seconds, np):
+    """The oracle's AVX2 + pthreads build on this box's host cores: the same FFN passes (all five
+    widths) on weight set 0, repeated for about `seconds` of CPU work."""
+    from oracle import binding as orc
+    g, u, d = (w.to_ggml() for w in weight_set)
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+    x_host = {n: xs[n].cpu().numpy() for n in WIDTHS}
+    orc.simd_ffn_swiglu(g, u, d, HIDDEN, INTER, x_host[1], threads)   # page everything in
+    done, t0 = 0, time.perf_counter()
+    while True:
+        for n in WIDTHS:
+            orc.simd_ffn_swiglu(g, u, d, HIDDEN, INTER, x_host[n], threads)
+        done += 1
+        if time.perf_counter() - t0 >= seconds or done >= 200:
+            break
+    dt = time.perf_counter() - t0
+    total = done * sum(ffn_bytes(n) for n in WIDTHS)
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": round(total / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{done} passes over the five FFN widths (n=1,2,4,8,16) on weight set 0, {dt:.1f} s, "
+                      f"AVX2 + {threads} pthreads, rows split as ith*ceil(N/nth)",
+            "cpu": model}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

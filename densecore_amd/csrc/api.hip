@@ -7,6 +7,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "common.h"
 #include "kernels.h"
@@ -81,6 +82,37 @@ struct State {
     Buffer route;         // ids / weights / groups / entries
     Buffer stage_in, stage_out;  // host-pointer entry points
 } g;
+
+// Launch census: event pairs around matmul-kernel launches (see mq_census_* in the public header).
+struct Census {
+    bool on = false;
+    struct Rec {
+        hipEvent_t start, stop;
+        int kind;
+    };
+    std::vector<Rec> pool;   // created once, reused after reset
+    size_t used = 0;
+    static constexpr size_t kMax = 8192;
+} census;
+
+hipError_t census_launch(const MatmulArgs& a, hipStream_t s) {
+    if (!census.on || census.used >= Census::kMax) return launch_matmul(a, s);
+    if (census.used == census.pool.size()) {
+        Census::Rec r;
+        hipError_t e = hipEventCreate(&r.start);
+        if (e != hipSuccess) return e;
+        e = hipEventCreate(&r.stop);
+        if (e != hipSuccess) return e;
+        census.pool.push_back(r);
+    }
+    Census::Rec& r = census.pool[census.used++];
+    r.kind = (a.grouped ? 2 : 0) + (a.swiglu ? 1 : 0);
+    hipError_t e = hipEventRecord(r.start, s);
+    if (e != hipSuccess) return e;
+    e = launch_matmul(a, s);
+    if (e != hipSuccess) return e;
+    return hipEventRecord(r.stop, s);
+}
 
 int check_ready() {
     if (!g.ready) return fail(MQ_ERR_STATE, "mq_init has not been called (or no GPU is present)");
@@ -287,7 +319,7 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
     a.ldy = ldy;
     a.dbg_dot = dbg_dot;
     a.dbg_min = dbg_min;
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(census_launch(a, s));
     return MQ_OK;
 }
 
@@ -385,7 +417,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.ldy = inter;
     a.swiglu = 1;
     a.silu_mode = silu_mode;
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(census_launch(a, s));
     if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
@@ -396,7 +428,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     d.n = n;
     d.y = y_dev;
     d.ldy = hidden;
-    MQ_HIP(launch_matmul(d, s));
+    MQ_HIP(census_launch(d, s));
     return MQ_OK;
 }
 
@@ -485,7 +517,7 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     a.y_k_stride = 1;
     const int64_t pairs = n * (int64_t)top_k;
     a.max_groups = (int)(pairs < w->n_experts ? pairs : w->n_experts);
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(census_launch(a, s));
     return MQ_OK;
 }
 
@@ -536,7 +568,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
         a.sh_yrow_offset = top_k;
         a.sh_silu_mode = MQ_SILU_FAST_FMA;
     }
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(census_launch(a, s));
     return MQ_OK;
 }
 
@@ -579,7 +611,7 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
         d.sh_yrow_stride = slots;
         d.sh_yrow_offset = top_k;
     }
-    MQ_HIP(launch_matmul(d, s));
+    MQ_HIP(census_launch(d, s));
     MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, slots, hidden_dim, weights, ids, down->n_experts,
                               sh.down ? 1 : 0, sh_gate_inp, x, y, s));
     return MQ_OK;
@@ -629,7 +661,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     a.ldy = ldh;
     a.swiglu = 1;
     a.silu_mode = silu_mode;
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(census_launch(a, s));
     return MQ_OK;
 }
 
@@ -717,6 +749,42 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     const size_t pair_bytes = (size_t)n * K * 4;
     if (ids_out_dev) MQ_HIP(hipMemcpyAsync(ids_out_dev, r.ids, pair_bytes, hipMemcpyDeviceToDevice, s));
     if (weights_out_dev) MQ_HIP(hipMemcpyAsync(weights_out_dev, r.weights, pair_bytes, hipMemcpyDeviceToDevice, s));
+    return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- census
+int mq_census_enable(int on) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    census.on = on != 0;
+    return MQ_OK;
+}
+int mq_census_reset(void) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (census.used) (void)hipDeviceSynchronize();
+    census.used = 0;
+    return MQ_OK;
+}
+int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int64_t* count) {
+    if (int rc = check_ready()) return rc;
+    if (kind < 0 || kind >= MQ_KIND_COUNT) return fail(MQ_ERR_INVALID, "mq_census_read: kind %d", kind);
+    std::lock_guard<std::mutex> lock(g.mu);
+    MQ_HIP(hipDeviceSynchronize());
+    double sum = 0.0, lo = 1e30, hi = 0.0;
+    int64_t n = 0;
+    for (size_t i = 0; i < census.used; ++i) {
+        if (census.pool[i].kind != kind) continue;
+        float ms = 0.0f;
+        MQ_HIP(hipEventElapsedTime(&ms, census.pool[i].start, census.pool[i].stop));
+        const double us = (double)ms * 1000.0;
+        sum += us;
+        lo = us < lo ? us : lo;
+        hi = us > hi ? us : hi;
+        ++n;
+    }
+    if (avg_us) *avg_us = n ? sum / (double)n : 0.0;
+    if (min_us) *min_us = n ? lo : 0.0;
+    if (max_us) *max_us = hi;
+    if (count) *count = n;
     return MQ_OK;
 }
 

@@ -225,3 +225,23 @@ def moe_layer(gate_exps: Q4KWeight, up_exps: Q4KWeight, down_exps: Q4KWeight, x:
     _lib.check(_lib.lib().mq_moe_layer_q4k(C.byref(d), _ptr(x), _ptr(logits), n, _ptr(y), _ptr(ids), _ptr(wts),
                                            _stream()), "mq_moe_layer_q4k")
     return y, ids, wts
+
+
+KIND_DENSE, KIND_DENSE_SWIGLU, KIND_GROUPED, KIND_GROUPED_SWIGLU = 0, 1, 2, 3
+
+
+def census_enable(on: bool) -> None:
+    """Record a HIP event pair around every matmul-kernel launch (the GPU analogue of the reference's
+    matmul dispatch census, core/src/llm/matmul/gemv_exec.cpp:203-276)."""
+    _lib.check(_lib.lib().mq_census_enable(1 if on else 0), "mq_census_enable")
+
+
+def census_reset() -> None:
+    _lib.check(_lib.lib().mq_census_reset(), "mq_census_reset")
+
+
+def census_read(kind: int) -> dict:
+    avg, lo, hi, cnt = C.c_double(), C.c_double(), C.c_double(), C.c_int64()
+    _lib.check(_lib.lib().mq_census_read(kind, C.byref(avg), C.byref(lo), C.byref(hi), C.byref(cnt)),
+               "mq_census_read")
+    return {"avg_us": avg.value, "min_us": lo.value, "max_us": hi.value, "count": cnt.value}

@@ -179,6 +179,20 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const f
 int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, int32_t* dot_scaled_dev,
                         int32_t* min_dot_dev, float* y_dev, int64_t ldy, void* stream);
 
+/* ---- launch census -------------------------------------------------------------------
+ * When enabled, a HIP event pair is recorded on the launch stream around every matmul-kernel
+ * launch; mq_census_read synchronises and returns the device time between the pairs.  The GPU
+ * counterpart of the reference's matmul dispatch census of (path, shape, wall ns)
+ * (core/src/llm/matmul/gemv_exec.cpp:203-276).  Off by default: the extra events serialise launches. */
+#define MQ_KIND_DENSE 0          /* one dense matrix                     */
+#define MQ_KIND_DENSE_SWIGLU 1   /* gate + up fused, dense               */
+#define MQ_KIND_GROUPED 2        /* expert-routed                        */
+#define MQ_KIND_GROUPED_SWIGLU 3 /* expert-routed gate + up fused        */
+#define MQ_KIND_COUNT 4
+int mq_census_enable(int on);
+int mq_census_reset(void);
+int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int64_t* count);
+
 /* ---- device memory helpers (so a C host needs no HIP headers) -------------------- */
 int mq_device_malloc(void** ptr, size_t bytes);
 int mq_device_free(void* ptr);

@@ -321,3 +321,14 @@ def simd_mul_mat_q4k_q8k(w, cols: int, q8, threads: int) -> np.ndarray:
     if rc:
         raise ValueError(f"orc_simd_mul_mat_q4k_q8k rc={rc}")
     return out
+
+
+def simd_ffn_swiglu(gate, up, down, hidden: int, inter: int, x, threads: int, silu=SILU_FAST_FMA) -> np.ndarray:
+    gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+    x = _c(x, np.float32)
+    y = np.zeros((x.shape[0], hidden), np.float32)
+    rc = simd().orc_simd_ffn_swiglu_q4k(_p(gate), _p(up), _p(down), C.c_int64(hidden), C.c_int64(inter), _p(x),
+                                        C.c_int64(x.shape[0]), _p(y), C.c_int(threads), C.c_int(silu))
+    if rc:
+        raise ValueError(f"orc_simd_ffn_swiglu_q4k rc={rc}")
+    return y

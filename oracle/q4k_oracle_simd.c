@@ -139,3 +139,34 @@ int orc_simd_mul_mat_id_q4k_q8k(const void* const* w_list, const void* const* q8
     }
     return 0;
 }
+
+/* Dense SwiGLU FFN on host cores: quantize (scalar oracle), gate and up rows split over the
+ * threads, SiLU-gate, re-quantize, down rows split over the threads.  Timed as the CPU baseline of
+ * the FFN-shaped workload; equals orc_ffn_swiglu_q4k(..., ORC_ORDER_AVX2, ...) bit for bit. */
+int orc_simd_ffn_swiglu_q4k(const void* gate, const void* up, const void* down, int64_t hidden, int64_t inter,
+                            const float* x, int64_t n, float* y, int threads, int silu_mode) {
+    if (!gate || !up || !down || !x || !y || hidden % ORC_QK_K || inter % ORC_QK_K || n <= 0) return -1;
+    const size_t wrow_in = (size_t)(hidden / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t wrow_mid = (size_t)(inter / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t q8_in = (size_t)(hidden / ORC_QK_K) * sizeof(orc_block_q8k);
+    const size_t q8_mid = (size_t)(inter / ORC_QK_K) * sizeof(orc_block_q8k);
+    uint8_t* xq = (uint8_t*)malloc(q8_in * (size_t)n);
+    uint8_t* hq = (uint8_t*)malloc(q8_mid * (size_t)n);
+    float* g = (float*)malloc(sizeof(float) * (size_t)n * (size_t)inter * 2);
+    int rc = (xq && hq && g) ? 0 : -2;
+    if (rc == 0) {
+        float* u = g + (size_t)n * (size_t)inter;
+        orc_quantize_rows_q8k(x, n, hidden, xq, hidden);
+        rc = orc_simd_mul_mat_q4k_q8k(gate, inter, hidden, wrow_in, xq, n, q8_in, g, inter, threads);
+        if (rc == 0) rc = orc_simd_mul_mat_q4k_q8k(up, inter, hidden, wrow_in, xq, n, q8_in, u, inter, threads);
+        if (rc == 0) {
+            for (int64_t i = 0; i < n * inter; ++i) g[i] = orc_silu_mul(g[i], u[i], silu_mode);
+            orc_quantize_rows_q8k(g, n, inter, hq, inter);
+            rc = orc_simd_mul_mat_q4k_q8k(down, hidden, inter, wrow_mid, hq, n, q8_mid, y, hidden, threads);
+        }
+    }
+    free(xq);
+    free(hq);
+    free(g);
+    return rc;
+}

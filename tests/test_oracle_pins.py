@@ -272,6 +272,15 @@ def test_simd_baseline_is_bitwise_the_avx2_order():
         assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
 
 
+def test_simd_ffn_baseline_matches_scalar_oracle():
+    H, I, n = 512, 768, 3
+    g, u, d = synth.q4k_matrix(55, I, H), synth.q4k_matrix(56, I, H), synth.q4k_matrix(57, H, I)
+    x = synth.normal_f32(58, (n, H))
+    want = orc.ffn_swiglu(g, u, d, H, I, x, orc.ORDER_AVX2, orc.SILU_FAST_FMA)
+    got = orc.simd_ffn_swiglu(g, u, d, H, I, x, threads=4)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 # ----------------------------------------------------------------- activation
 def test_fast_exp_error_class_and_silu_flavours():
     xs = np.linspace(-20, 20, 4001, dtype=np.float32)
