@@ -47,6 +47,7 @@ def moe_bytes(n: int, distinct: int) -> int:
 
 
 def main() -> int:
+    global RING
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -55,6 +56,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the GEMV / MoE side measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (one MI355X per box); --gpus N with N > 1 is not run. "
@@ -65,6 +67,8 @@ def main() -> int:
     import torch
 
     from densecore_amd import ops, synth
+
+    RING = max(1, args.ring)
 
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")

@@ -20,6 +20,8 @@
 //
 // MFMA operand roles: A (M side) = 16 activation rows, B (N side) = 16 weight rows, so each lane's
 // four accumulators belong to ONE weight row (lane%16) and it needs only that row's scales.
+#include <cstdlib>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -47,6 +49,9 @@ struct ARegs {
     float yd[TT][4]; // Q8_K scale of the four activation rows this lane accumulates
 };
 
+// All loads are unconditional: the caller clamps the row of a dead slot to a live row of the same
+// group, whose result is simply never stored.  Branch-free loads let the compiler count the
+// outstanding requests exactly, which is what keeps the next tile in flight during the MFMAs.
 template <int TT>
 __device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__ aq, const float* __restrict__ ad,
                                        const int (&arow)[TT], const int (&drow)[TT][4], int64_t b, int64_t nb,
@@ -54,12 +59,9 @@ __device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
-        for (int gp = 0; gp < 4; ++gp) {
-            v4u z = {0u, 0u, 0u, 0u};
-            a.q[tt][gp] = arow[tt] >= 0 ? load16(aq + aq_offset(arow[tt], b, gp, kq, nb)) : z;
-        }
+        for (int gp = 0; gp < 4; ++gp) a.q[tt][gp] = load16(aq + aq_offset(arow[tt], b, gp, kq, nb));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a.yd[tt][i] = drow[tt][i] >= 0 ? ad[ad_index(drow[tt][i], b, nb)] : 0.0f;
+        for (int i = 0; i < 4; ++i) a.yd[tt][i] = ad[ad_index(drow[tt][i], b, nb)];
     }
 }
 
@@ -164,11 +166,10 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
             auto map = [&](int s, int& ar, int& yr) {
-                const int e = chunk + 16 * tt + s;
-                if (e >= count) {
-                    ar = -1;
-                    yr = -1;
-                } else if (!GROUPED) {
+                const int e_raw = chunk + 16 * tt + s;
+                const bool live = e_raw < count;
+                const int e = live ? e_raw : count - 1;  // dead slot: read a live row, store nothing
+                if (!GROUPED) {
                     ar = e;
                     yr = e;
                 } else if (shared_group) {
@@ -179,6 +180,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                     ar = tok * p.a_tok_stride + kk * p.a_k_stride;
                     yr = tok * p.y_tok_stride + kk * p.y_k_stride;
                 }
+                if (!live) yr = -1;
             };
             int unused;
             map(slot, arow[tt], unused);
@@ -194,50 +196,55 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[m][tt][i] = 0.0f;
 
-        int64_t b = wave;
-        if (b < nb) {
-            TileRegs cur[NMAT];
-            ARegs<TT> acur;
+        // Two register stages, ping-pong: while one tile's MFMAs run, the next tile's loads are in
+        // flight.  The steady-state loop has no conditionals, so every wait counts exactly the
+        // loads issued after the data it needs.
+        if (wave < nb) {
+            const int64_t cnt = (nb - wave + n_waves - 1) / n_waves;  // super-blocks of this wave
+            TileRegs t0[NMAT], t1[NMAT];
+            ARegs<TT> a0, a1;
+            auto issue = [&](TileRegs(&t)[NMAT], ARegs<TT>& a, int64_t i) {
+                const int64_t b = wave + i * n_waves;
 #pragma unroll
-            for (int m = 0; m < NMAT; ++m) load_tile(cur[m], tiles[m] + (size_t)b * kTileBytes, lane);
-            load_a<TT>(acur, p.aq, p.ad, arow, drow, b, nb, kq);
-            while (true) {
-                const int64_t bn = b + n_waves;
-                const bool more = bn < nb;
-                TileRegs nxt[NMAT];
-                ARegs<TT> anxt;
-                if (more) {
-#pragma unroll
-                    for (int m = 0; m < NMAT; ++m) load_tile(nxt[m], tiles[m] + (size_t)bn * kTileBytes, lane);
-                    if (TT == 1) load_a<TT>(anxt, p.aq, p.ad, arow, drow, bn, nb, kq);
-                }
+                for (int m = 0; m < NMAT; ++m) load_tile(t[m], tiles[m] + (size_t)b * kTileBytes, lane);
+                load_a<TT>(a, p.aq, p.ad, arow, drow, b, nb, kq);
+            };
+            auto consume = [&](const TileRegs(&t)[NMAT], const ARegs<TT>& a, int64_t i) {
+                const int64_t b = wave + i * n_waves;
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][4], msum[TT][4];
-                    compute_tile<TT>(cur[m], acur, acc[m], dsum, msum);
+                    compute_tile<TT>(t[m], a, acc[m], dsum, msum);
                     if (DEBUG && p.dbg_dot) {
                         const int64_t row = rt * 16 + slot;
 #pragma unroll
                         for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) {
-                                if (yrow[tt][i] >= 0 && row < p.rows) {
-                                    const size_t idx = ((size_t)row * (size_t)p.n + (size_t)yrow[tt][i]) * nb + b;
-                                    p.dbg_dot[idx] = dsum[tt][i];
-                                    p.dbg_min[idx] = msum[tt][i];
+                            for (int i2 = 0; i2 < 4; ++i2) {
+                                if (yrow[tt][i2] >= 0 && row < p.rows) {
+                                    const size_t idx = ((size_t)row * (size_t)p.n + (size_t)yrow[tt][i2]) * nb + b;
+                                    p.dbg_dot[idx] = dsum[tt][i2];
+                                    p.dbg_min[idx] = msum[tt][i2];
                                 }
                             }
                     }
                 }
-                if (!more) break;
-#pragma unroll
-                for (int m = 0; m < NMAT; ++m) cur[m] = nxt[m];
-                if (TT == 1) {
-                    acur = anxt;
-                } else {  // wide token tiles: too many registers to hold two blocks of activations
-                    load_a<TT>(acur, p.aq, p.ad, arow, drow, bn, nb, kq);
-                }
-                b = bn;
+            };
+            issue(t0, a0, 0);
+            int64_t i = 0;
+            while (i + 2 < cnt) {
+                issue(t1, a1, i + 1);
+                consume(t0, a0, i);
+                issue(t0, a0, i + 2);
+                consume(t1, a1, i + 1);
+                i += 2;
+            }
+            if (cnt - i == 2) {
+                issue(t1, a1, i + 1);
+                consume(t0, a0, i);
+                consume(t1, a1, i + 1);
+            } else {
+                consume(t0, a0, i);
             }
         }
 
@@ -318,6 +325,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
     // expected live groups: at most one per routed (token, k) pair
     int64_t live = a.grouped ? groups : 1;
     int waves = pick_waves(a.nb, rowtiles * live);
+    if (const char* ev = getenv("MQ_WAVES")) waves = atoi(ev) > 0 ? atoi(ev) : waves;  // tuning knob
     while (waves > 1 && ((size_t)(waves - 1) * nmat * tt * 1024 > 64 * 1024 || a.nb % waves != 0)) --waves;
     const dim3 grid((unsigned)rowtiles, (unsigned)groups);
 
