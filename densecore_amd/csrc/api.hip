@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -79,6 +80,7 @@ struct State {
     Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
     Buffer aq2, ad2;      // A-major activations of the intermediate
     Buffer part;          // MoE per-(token,k) down results
+    Buffer counters;      // arrival counters of the fused output quantization (kept zero between launches)
     Buffer route;         // ids / weights / groups / entries
     Buffer stage_in, stage_out;  // host-pointer entry points
 } g;
@@ -143,6 +145,15 @@ int quantize_into(Buffer& aq, Buffer& ad, const float* x, int64_t n, int64_t ldx
     return MQ_OK;
 }
 
+// Arrival counters for the fused output quantization: zeroed when (re)allocated, and every launch
+// leaves them zero again.
+int reserve_counters(size_t count) {
+    const size_t before = g.counters.cap;
+    MQ_HIP(g.counters.reserve(count * sizeof(uint32_t)));
+    if (g.counters.cap != before) MQ_HIP(hipMemset(g.counters.ptr, 0, g.counters.cap));
+    return MQ_OK;
+}
+
 int alloc_weight(int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
     if (!out) return fail(MQ_ERR_INVALID, "null output handle");
     *out = nullptr;
@@ -199,7 +210,7 @@ int mq_shutdown(void) {
     std::lock_guard<std::mutex> lock(g.mu);
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
-    for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
     g.ready = false;
     return MQ_OK;
 }
@@ -417,8 +428,20 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.ldy = inter;
     a.swiglu = 1;
     a.silu_mode = silu_mode;
+    // the SwiGLU output is re-quantized by the gate/up kernel itself (last workgroup per 256-row block)
+    MQ_HIP(g.aq2.reserve(aq_bytes(n, inter / kQK)));
+    MQ_HIP(g.ad2.reserve(ad_count(n, inter / kQK) * sizeof(float)));
+    if (int rc = reserve_counters((size_t)(inter / kQK))) return rc;
+    const bool fuse_q = getenv("MQ_NOFUSEQ") == nullptr;  // tuning knob
+    if (fuse_q) {
+        a.out_aq = (uint8_t*)g.aq2.ptr;
+        a.out_ad = (float*)g.ad2.ptr;
+        a.out_counters = (uint32_t*)g.counters.ptr;
+    }
     MQ_HIP(census_launch(a, s));
-    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    if (!fuse_q) {
+        if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    }
     MatmulArgs d;
     d.w0 = down->data;
     d.rows = hidden;
@@ -532,9 +555,19 @@ struct SharedExpert {
 // gate/up + SwiGLU for every routed (token, k) pair (and the shared expert as slot top_k):
 // hidden row = token * slots + k.  Caller holds g.mu; groups are already built in r.
 int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExpert& sh, int64_t n, int top_k, int slots,
-                   int silu_mode, const RouteWs& r, float* hidden, hipStream_t s) {
+                   int silu_mode, const RouteWs& r, float* hidden, bool quantize_hidden, hipStream_t s) {
     const int64_t pairs = n * (int64_t)top_k;
     MatmulArgs a;
+    if (quantize_hidden) {  // hidden rows leave the kernel already in Q8_K (A-major), ready for the down projection
+        const int64_t out_nb = gate->rows / kQK;
+        const int64_t groups = (pairs < gate->n_experts ? pairs : gate->n_experts) + 1;
+        MQ_HIP(g.aq2.reserve(aq_bytes(n * slots, out_nb)));
+        MQ_HIP(g.ad2.reserve(ad_count(n * slots, out_nb) * sizeof(float)));
+        if (int rc = reserve_counters((size_t)(groups * out_nb))) return rc;
+        a.out_aq = (uint8_t*)g.aq2.ptr;
+        a.out_ad = (float*)g.ad2.ptr;
+        a.out_counters = (uint32_t*)g.counters.ptr;
+    }
     a.w0 = gate->data;
     a.w1 = up->data;
     a.rows = gate->rows;
@@ -573,14 +606,16 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
 }
 
 // Q8_K of the hidden rows, down projection per (token, k) into g.part, then the weighted combine.
-int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hidden, int64_t n, int top_k, int slots,
-                 const RouteWs& r, const int32_t* ids, const float* weights, const float* sh_gate_inp,
-                 const float* x, float* y, hipStream_t s) {
+int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hidden, bool hidden_is_quantized, int64_t n,
+                 int top_k, int slots, const RouteWs& r, const int32_t* ids, const float* weights,
+                 const float* sh_gate_inp, const float* x, float* y, hipStream_t s) {
     const int64_t pairs = n * (int64_t)top_k;
     const int64_t mid_rows = n * slots;
     const int64_t inter = down->cols, hidden_dim = down->rows;
-    // rows of dropped entries may hold anything; they are quantized but never read
-    if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
+    // rows of dropped entries may hold anything; they are never read
+    if (!hidden_is_quantized) {
+        if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
+    }
     MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden_dim * sizeof(float)));
     MatmulArgs d;
     d.w0 = down->data;
@@ -683,7 +718,7 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, gate_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, gate_exps->cols, gate_exps->cols, s)) return rc;
-    return run_moe_gateup(gate_exps, up_exps, SharedExpert{}, n, top_k, top_k, silu_mode, r, hidden_dev, s);
+    return run_moe_gateup(gate_exps, up_exps, SharedExpert{}, n, top_k, top_k, silu_mode, r, hidden_dev, false, s);
 }
 
 int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev, int64_t n, const int32_t* ids_dev,
@@ -700,7 +735,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
     if (int rc = carve_route(n, top_k, down_exps->n_experts, r)) return rc;
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, down_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
-    return run_moe_down(down_exps, SharedExpert{}, hidden_dev, n, top_k, top_k, r, ids_dev, weights_dev, nullptr,
+    return run_moe_down(down_exps, SharedExpert{}, hidden_dev, false, n, top_k, top_k, r, ids_dev, weights_dev, nullptr,
                         nullptr, y_dev, s);
 }
 
@@ -742,8 +777,8 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     MQ_HIP(launch_build_groups(r.ids, n, K, E, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
-    if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, s)) return rc;
-    if (int rc = run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, n, K, slots, r, r.ids, r.weights,
+    if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
+    if (int rc = run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, r.ids, r.weights,
                               L->sh_gate_inp_dev, x_dev, y_dev, s))
         return rc;
     const size_t pair_bytes = (size_t)n * K * 4;

@@ -13,7 +13,6 @@ constexpr int kQ8Block = 292;        // bytes of block_q8_K
 constexpr int kTileRows = 16;        // weight rows per tile (the N side of a 16x16 MFMA)
 constexpr int kTileBytes = kTileRows * kQ4Block;  // 2304
 constexpr int kTileQBytes = kTileRows * 128;      // 2048: nibble part
-constexpr int kTokTile = 16;         // activation rows per MFMA (the M side)
 
 // ---------------------------------------------------------------------------------------------
 // Weight layout in HBM ("row-tile major"): a matrix of `rows` x `cols` is cut into tiles of 16
@@ -42,23 +41,33 @@ __host__ __device__ inline int tile_word_offset(int r, int word) {
 
 // ---------------------------------------------------------------------------------------------
 // Activation layout consumed by the matmul kernels ("A-major Q8_K"): the same int8 codes and fp32
-// scales as block_q8_K, ordered so that a wave reads its MFMA A operand with coalesced 16-byte
-// loads.  Activation row m (a token, or a (token, k) pair) lives in row-tile m/16, slot m%16:
-//   codes : [m/16][b][gp 0..3][kq 0..3][slot 0..15][16 B]
-//           16 B = {qs[64gp + 8kq .. +7], qs[64gp + 32 + 8kq .. +7]}  (sub-blocks 2gp and 2gp+1)
-//   scale : [m/16][b][slot] fp32
+// scales as block_q8_K, ordered so that a wave reads the A operand of v_mfma_i32_16x16x64_i8 with
+// coalesced 16-byte loads.  One MFMA covers a 64-weight chunk, i.e. two 32-wide sub-blocks with
+// different scales; to keep their partial sums apart every activation row owns TWO of the 16
+// M-side slots: slot 2t holds the codes of the even sub-block in bytes 0..7 and zeros in bytes
+// 8..15, slot 2t+1 the reverse.  The products against the zero halves vanish, so output slot 2t is
+// the dot over sub-block 2c alone and slot 2t+1 the dot over sub-block 2c+1.  A tile is therefore
+// 8 activation rows.  Row m lives in tile m/8, position t = m%8:
+//   codes : [m/8][b][c 0..3][kq 0..3][slot 0..15][16 B]      (4096 B per tile and super-block)
+//           slot 2t   = {qs[64c + 8kq .. +7], 0 x 8}
+//           slot 2t+1 = {0 x 8, qs[64c + 32 + 8kq .. +7]}
+//   scale : [m/8][b][t] fp32
 // ---------------------------------------------------------------------------------------------
-__host__ __device__ inline size_t aq_offset(int64_t m, int64_t b, int gp, int kq, int64_t nb) {
-    return ((((size_t)(m >> 4) * nb + b) * 4 + gp) * 4 + kq) * 256 + (size_t)(m & 15) * 16;
+constexpr int kTokTile = 8;  // activation rows per MFMA (two M-side slots each)
+__host__ __device__ inline size_t aq_row_offset(int64_t m, int64_t nb) {  // row part of the address
+    return (size_t)(m >> 3) * (size_t)nb * 4096 + (size_t)(m & 7) * 32;
+}
+__host__ __device__ inline size_t aq_offset(int64_t m, int64_t b, int c, int kq, int h, int64_t nb) {
+    return aq_row_offset(m, nb) + (size_t)b * 4096 + (size_t)(c * 4 + kq) * 256 + (size_t)h * 16;
 }
 __host__ __device__ inline size_t ad_index(int64_t m, int64_t b, int64_t nb) {
-    return ((size_t)(m >> 4) * nb + b) * 16 + (size_t)(m & 15);
+    return ((size_t)(m >> 3) * nb + b) * 8 + (size_t)(m & 7);
 }
 __host__ __device__ inline size_t aq_bytes(int64_t n_rows, int64_t nb) {
-    return (size_t)((n_rows + 15) >> 4) * nb * 4096;
+    return (size_t)((n_rows + 7) >> 3) * nb * 4096;
 }
 __host__ __device__ inline size_t ad_count(int64_t n_rows, int64_t nb) {
-    return (size_t)((n_rows + 15) >> 4) * nb * 16;
+    return (size_t)((n_rows + 7) >> 3) * nb * 8;
 }
 
 // SplitMix64 finaliser: the synthetic-weight recipe shared with densecore_amd/synth.py.

@@ -40,6 +40,12 @@ struct MatmulArgs {
     int silu_mode = 0;
     int32_t* dbg_dot = nullptr;    // optional [rows][n][nb]
     int32_t* dbg_min = nullptr;
+    // optional fused re-quantization of the output: the workgroup that completes a 256-row block of
+    // y (the last of its 16 row tiles to finish) quantizes that block of every live activation row
+    // to Q8_K in the A-major layout, ready to be the next matmul's input.  rows % 256 == 0.
+    uint8_t* out_aq = nullptr;
+    float* out_ad = nullptr;
+    uint32_t* out_counters = nullptr;  // [groups][rows/256], zero before the launch, zero again after it
     // grouped (expert-routed) mode: work list built on the device
     int grouped = 0;
     const int32_t* group_expert = nullptr;  // [max_groups] expert id per group

@@ -6,24 +6,36 @@
 //               workgroup as a whole streams one contiguous run of tiles.
 //   wavefront = per super-block: three coalesced 16-byte-per-lane loads bring one 2304-byte tile
 //               (16 rows x 256 weights) straight into MFMA operand order; the next tile is
-//               requested before the current one is consumed.
-//   arithmetic (per tile, up to 16 activation rows at once, independent of how many are live):
-//       8 x v_mfma_i32_16x16x32_i8   one per 32-wide sub-block: sum q4*q8            (int32)
-//       v_mad_i32_i24 with the 6-bit sub-block scale                 -> dot_scaled   (int32)
-//       4 x v_mfma_i32_16x16x64_i8   6-bit mins broadcast as the B operand: sum min*q8 -> min_dot
-//       fp32: acc += (d*yd)*dot_scaled - (dmin*yd)*min_dot   (core/src/llm/matmul/kquant_batched_kernels.h:299-301)
+//               requested before the current one is consumed (two register stages, ping-pong).
+//   arithmetic, per tile and per group of 8 activation rows (independent of how many are live):
+//       4 x v_mfma_i32_16x16x64_i8   one per 64-weight chunk.  Each activation row owns two M-side
+//                                    slots with complementary zero halves (see common.h), so the
+//                                    two 32-wide sub-blocks of the chunk come out as separate
+//                                    int32 sums: sum q4*q8 per sub-block.
+//       v_mad_i32_i24 with the 6-bit sub-block scales                       -> dot_scaled (int32)
+//       4 x v_mfma_i32_16x16x64_i8   the 6-bit mins broadcast as the B operand: sum min*q8
+//                                                                           -> min_dot   (int32)
+//       fp32: acc += (d*yd)*dot_scaled - (dmin*yd)*min_dot  (core/src/llm/matmul/kquant_batched_kernels.h:299-301)
 //   The two integers are exactly the reference's per-super-block sums; min_dot is formed from the
 //   int8 codes instead of the 16 bsums, which is the same number because bsums[j] is by
 //   construction the sum of codes 16j..16j+15 (core/src/kernels/hwy/hwy_moe_quant.cc:133-139).
 //   epilogue: wave partials are added in wave order through LDS (deterministic), optional
 //   silu(gate)*up, one store per (activation row, weight row).
 //
-// MFMA operand roles: A (M side) = 16 activation rows, B (N side) = 16 weight rows, so each lane's
-// four accumulators belong to ONE weight row (lane%16) and it needs only that row's scales.
+// MFMA operand roles: A (M side) = 8 activation rows x 2 slots, B (N side) = 16 weight rows, so a
+// lane's four accumulators belong to ONE weight row (lane%16) and to two activation rows
+// (2*(lane/16) and 2*(lane/16)+1): it needs only that row's scales and writes two outputs.
 #include <cstdlib>
 
 #include "common.h"
 #include "kernels.h"
+#include "q8k_block.h"
+
+// Ablation switches for microbenchmarks only (the library is always built with 0):
+// 1 = replace the tile arithmetic by a cheap reduction, 2 = do not load activations.
+#ifndef MQ_ABLATE
+#define MQ_ABLATE 0
+#endif
 
 namespace mq {
 
@@ -39,52 +51,65 @@ __device__ __forceinline__ void load_tile(TileRegs& t, const uint8_t* tile, int 
     t.hdr = load_stream16(tile + kTileQBytes + (lane & 15) * 16);
 }
 
-__device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) {
-    return (long)(((uint64_t)hi << 32) | (uint64_t)lo);
-}
-
 template <int TT>
 struct ARegs {
-    v4u q[TT][4];    // [token tile][sub-block pair]: 16 B = 8 codes of sub-block 2gp, 8 of 2gp+1
-    float yd[TT][4]; // Q8_K scale of the four activation rows this lane accumulates
+    v4u q[TT][4];    // [token tile][64-weight chunk]: this lane's 16 B of the split-slot A operand
+    float yd[TT][2]; // Q8_K scales of the two activation rows this lane accumulates
 };
 
 // All loads are unconditional: the caller clamps the row of a dead slot to a live row of the same
 // group, whose result is simply never stored.  Branch-free loads let the compiler count the
 // outstanding requests exactly, which is what keeps the next tile in flight during the MFMAs.
 template <int TT>
-__device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__ aq, const float* __restrict__ ad,
-                                       const int (&arow)[TT], const int (&drow)[TT][4], int64_t b, int64_t nb,
-                                       int kq) {
+__device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__ aq_blk, const float* __restrict__ ad_blk,
+                                       const size_t (&a_off)[TT], const int (&d_idx)[TT][2]) {
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
+#if MQ_ABLATE & 2
+        for (int c = 0; c < 4; ++c) a.q[tt][c] = v4u{(unsigned)a_off[tt], 1u, 2u, (unsigned)c};
+        for (int j = 0; j < 2; ++j) a.yd[tt][j] = (float)d_idx[tt][j];
+#else
 #pragma unroll
-        for (int gp = 0; gp < 4; ++gp) a.q[tt][gp] = load16(aq + aq_offset(arow[tt], b, gp, kq, nb));
+        for (int c = 0; c < 4; ++c) a.q[tt][c] = load16(aq_blk + a_off[tt] + c * 1024);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a.yd[tt][i] = ad[ad_index(drow[tt][i], b, nb)];
+        for (int j = 0; j < 2; ++j) a.yd[tt][j] = ad_blk[d_idx[tt][j]];
+#endif
     }
 }
 
 template <int TT>
-__device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>& a, float (&acc)[TT][4],
-                                             int32_t (&dot_out)[TT][4], int32_t (&min_out)[TT][4]) {
+__device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>& a, float (&acc)[TT][2],
+                                             int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2]) {
+#if MQ_ABLATE & 1
+    {
+        unsigned x = t.q0.x ^ t.q0.y ^ t.q0.z ^ t.q0.w ^ t.q1.x ^ t.q1.y ^ t.q1.z ^ t.q1.w ^ t.hdr.x ^ t.hdr.y ^ t.hdr.z ^ t.hdr.w;
+        for (int tt = 0; tt < TT; ++tt) {
+            for (int c = 0; c < 4; ++c) x ^= a.q[tt][c].x ^ a.q[tt][c].y ^ a.q[tt][c].z ^ a.q[tt][c].w;
+            acc[tt][0] += (float)x * a.yd[tt][0];
+            acc[tt][1] += (float)x * a.yd[tt][1];
+            dot_out[tt][0] = dot_out[tt][1] = min_out[tt][0] = min_out[tt][1] = 0;
+        }
+        return;
+    }
+#endif
     // 6-bit scale / min unpack, word-parallel (core/src/kernels/hwy/hwy_moe_quant.cc:90-101)
     const uint32_t w0 = t.hdr.y, w1 = t.hdr.z, w2 = t.hdr.w;
     const uint32_t sc[2] = {w0 & 0x3f3f3f3fu, (w2 & 0x0f0f0f0fu) | (((w0 >> 6) & 0x03030303u) << 4)};
     const uint32_t mn[2] = {w1 & 0x3f3f3f3fu, ((w2 >> 4) & 0x0f0f0f0fu) | (((w1 >> 6) & 0x03030303u) << 4)};
     const uint32_t qw[8] = {t.q0.x, t.q0.y, t.q0.z, t.q0.w, t.q1.x, t.q1.y, t.q1.z, t.q1.w};
 
-    v4i dot[TT], mnd[TT];
+    int32_t dot[TT][2];
+    v4i mnd[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        dot[tt] = v4i{0, 0, 0, 0};
+        dot[tt][0] = dot[tt][1] = 0;
         mnd[tt] = v4i{0, 0, 0, 0};
     }
 #pragma unroll
     for (int c = 0; c < 4; ++c) {  // 64-weight chunk: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
         const uint32_t qa = qw[2 * c], qb = qw[2 * c + 1];
-        const long b_lo = pack64(qa & 0x0f0f0f0fu, qb & 0x0f0f0f0fu);
-        const long b_hi = pack64((qa >> 4) & 0x0f0f0f0fu, (qb >> 4) & 0x0f0f0f0fu);
+        const v4i b_q = {(int)(qa & 0x0f0f0f0fu), (int)(qb & 0x0f0f0f0fu), (int)((qa >> 4) & 0x0f0f0f0fu),
+                         (int)((qb >> 4) & 0x0f0f0f0fu)};
         const int s_lo = (int)((sc[c >> 1] >> (16 * (c & 1))) & 0xffu);
         const int s_hi = (int)((sc[c >> 1] >> (16 * (c & 1) + 8)) & 0xffu);
         // v_perm_b32 replicates one byte of the unpacked mins into all four bytes of the operand
@@ -94,12 +119,12 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
             const v4u av = a.q[tt][c];
-            const v4i zero = {0, 0, 0, 0};
-            const v4i p_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(av.x, av.y), b_lo, zero, 0, 0, 0);
-            const v4i p_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(av.z, av.w), b_hi, zero, 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) dot[tt][i] += __mul24(p_lo[i], s_lo) + __mul24(p_hi[i], s_hi);
             const v4i a16 = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i zero = {0, 0, 0, 0};
+            // p[0], p[2]: sub-block 2c of rows 2kq and 2kq+1;  p[1], p[3]: sub-block 2c+1
+            const v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(a16, b_q, zero, 0, 0, 0);
+            dot[tt][0] += __mul24(p[0], s_lo) + __mul24(p[1], s_hi);
+            dot[tt][1] += __mul24(p[2], s_lo) + __mul24(p[3], s_hi);
             mnd[tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a16, b_min, mnd[tt], 0, 0, 0);
         }
     }
@@ -108,25 +133,54 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float d = __fmul_rn(wd, a.yd[tt][i]);
-            const float dm = __fmul_rn(wm, a.yd[tt][i]);
-            const float term = __fsub_rn(__fmul_rn(d, (float)dot[tt][i]), __fmul_rn(dm, (float)mnd[tt][i]));
-            acc[tt][i] = __fadd_rn(acc[tt][i], term);
-            dot_out[tt][i] = dot[tt][i];
-            min_out[tt][i] = mnd[tt][i];
+        for (int j = 0; j < 2; ++j) {
+            const int32_t md = mnd[tt][2 * j] + mnd[tt][2 * j + 1];
+            const float d = __fmul_rn(wd, a.yd[tt][j]);
+            const float dm = __fmul_rn(wm, a.yd[tt][j]);
+            const float term = __fsub_rn(__fmul_rn(d, (float)dot[tt][j]), __fmul_rn(dm, (float)md));
+            acc[tt][j] = __fadd_rn(acc[tt][j], term);
+            dot_out[tt][j] = dot[tt][j];
+            min_out[tt][j] = md;
         }
     }
 }
 
-// One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group).
+// Activation row and output row of entry e of the current group.
+template <bool GROUPED>
+__device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_group, int begin, int e, int& ar, int& yr) {
+    if (!GROUPED) {
+        ar = e;
+        yr = e;
+    } else if (shared_group) {
+        ar = e * p.sh_arow_stride + p.sh_arow_offset;
+        yr = e * p.sh_yrow_stride + p.sh_yrow_offset;
+    } else {
+        const int tok = p.entry_token[begin + e], kk = p.entry_k[begin + e];
+        ar = tok * p.a_tok_stride + kk * p.a_k_stride;
+        yr = tok * p.y_tok_stride + kk * p.y_k_stride;
+    }
+}
+
+// Register stages a wave keeps in flight.  The kernel is bound by bytes in flight, not by
+// arithmetic: HBM latency under load is 1.5-2.5 us, so a CU needs on the order of 100 KB of
+// outstanding tile loads.  A stage is one super-block's activations (A operand) plus the NMAT
+// weight tiles that share them; at 2 waves per SIMD the register file holds four such stages.
+template <int NMAT, int TT>
+struct Depth {
+    static constexpr int kStages = TT == 1 ? (NMAT == 2 ? 3 : 4) : 2;
+};
+
+// One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
+// waves split the super-blocks of the row.  NMAT == 2: gate and up tiles of the same rows share
+// the activations in registers and meet in silu(gate)*up.
 template <int NMAT, int TT, bool GROUPED, bool DEBUG>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
-    extern __shared__ float red[];  // [W][NMAT][TT][4][64]
+    constexpr int S = Depth<NMAT, TT>::kStages;
+    extern __shared__ float red[];  // [W-1][NMAT][TT][2][64]
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps tile addresses scalar
     const int n_waves = blockDim.x >> 6;
-    const int slot = lane & 15;  // activation row within a token tile (A side), weight row (B side)
+    const int slot = lane & 15;  // A side: M slot (activation row slot/2, half slot%2); B side: weight row
     const int kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const int64_t nb = p.nb;
@@ -159,94 +213,94 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     const uint8_t* tiles[NMAT];
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) tiles[m] = w[m] + tile_offset(rt, 0, nb);
+#if MQ_ABLATE & 4
+    long long stamp[3];
+    stamp[0] = wall_clock64();
+#endif
 
-    for (int chunk = 0; chunk < count; chunk += 16 * TT) {
-        // activation-row / output-row indices of this lane's A slot and of its four D slots
-        int arow[TT], drow[TT][4], yrow[TT][4];
+    for (int chunk = 0; chunk < count; chunk += kTokTile * TT) {
+        // activation row behind this lane's A slot, and activation / output rows of its two outputs
+        size_t a_off[TT];
+        int d_idx[TT][2], yrow[TT][2];
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
-            auto map = [&](int s, int& ar, int& yr) {
-                const int e_raw = chunk + 16 * tt + s;
+            auto map = [&](int pos, int& ar, int& yr) {
+                const int e_raw = chunk + kTokTile * tt + pos;
                 const bool live = e_raw < count;
-                const int e = live ? e_raw : count - 1;  // dead slot: read a live row, store nothing
-                if (!GROUPED) {
-                    ar = e;
-                    yr = e;
-                } else if (shared_group) {
-                    ar = e * p.sh_arow_stride + p.sh_arow_offset;
-                    yr = e * p.sh_yrow_stride + p.sh_yrow_offset;
-                } else {
-                    const int tok = p.entry_token[begin + e], kk = p.entry_k[begin + e];
-                    ar = tok * p.a_tok_stride + kk * p.a_k_stride;
-                    yr = tok * p.y_tok_stride + kk * p.y_k_stride;
-                }
+                // dead slot: read a live row, store nothing
+                entry_rows<GROUPED>(p, shared_group, begin, live ? e_raw : count - 1, ar, yr);
                 if (!live) yr = -1;
             };
-            int unused;
-            map(slot, arow[tt], unused);
+            int ar, yr;
+            map(slot >> 1, ar, yr);
+            a_off[tt] = aq_row_offset(ar, nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) map(4 * kq + i, drow[tt][i], yrow[tt][i]);
+            for (int j = 0; j < 2; ++j) {
+                map(2 * kq + j, ar, yrow[tt][j]);
+                d_idx[tt][j] = (int)((size_t)(ar >> 3) * (size_t)nb * 8 + (size_t)(ar & 7));
+            }
         }
 
-        float acc[NMAT][TT][4];
+        float acc[NMAT][TT][2];
 #pragma unroll
         for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-            for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[m][tt][i] = 0.0f;
+            for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = acc[m][tt][1] = 0.0f;
 
-        // Two register stages, ping-pong: while one tile's MFMAs run, the next tile's loads are in
-        // flight.  The steady-state loop has no conditionals, so every wait counts exactly the
-        // loads issued after the data it needs.
+        // Ring of S register stages.  Stage i of this wave is super-block wave + i*W.  S-1 stages are
+        // requested before the first is consumed, and every consume is preceded by the request for
+        // the stage S-1 ahead, so S-1 stages are in flight while the MFMAs of one run.  All branches
+        // are wave-uniform and the loads themselves unconditional.
         if (wave < nb) {
-            const int64_t cnt = (nb - wave + n_waves - 1) / n_waves;  // super-blocks of this wave
-            TileRegs t0[NMAT], t1[NMAT];
-            ARegs<TT> a0, a1;
-            auto issue = [&](TileRegs(&t)[NMAT], ARegs<TT>& a, int64_t i) {
-                const int64_t b = wave + i * n_waves;
+            const int cnt = (int)((nb - wave + n_waves - 1) / n_waves);  // super-blocks of this wave
+            TileRegs ring_t[S][NMAT];
+            ARegs<TT> ring_a[S];
+            // Requests past the wave's last super-block are pointed at the (cache-resident)
+            // activation buffer instead of being skipped: the number of loads per stage stays
+            // fixed, so every wait below can count exactly.
+            auto issue = [&](int st, int i) {
+                const bool valid = i < cnt;
+                const int b = valid ? wave + i * n_waves : wave;
 #pragma unroll
-                for (int m = 0; m < NMAT; ++m) load_tile(t[m], tiles[m] + (size_t)b * kTileBytes, lane);
-                load_a<TT>(a, p.aq, p.ad, arow, drow, b, nb, kq);
+                for (int m = 0; m < NMAT; ++m)
+                    load_tile(ring_t[st][m], valid ? tiles[m] + (size_t)b * kTileBytes : p.aq, lane);
+                load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             };
-            auto consume = [&](const TileRegs(&t)[NMAT], const ARegs<TT>& a, int64_t i) {
-                const int64_t b = wave + i * n_waves;
+            auto consume = [&](int st, int i) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
-                    int32_t dsum[TT][4], msum[TT][4];
-                    compute_tile<TT>(t[m], a, acc[m], dsum, msum);
+                    int32_t dsum[TT][2], msum[TT][2];
+                    compute_tile<TT>(ring_t[st][m], ring_a[st], acc[m], dsum, msum);
                     if (DEBUG && p.dbg_dot) {
+                        const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;
 #pragma unroll
                         for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                            for (int i2 = 0; i2 < 4; ++i2) {
-                                if (yrow[tt][i2] >= 0 && row < p.rows) {
-                                    const size_t idx = ((size_t)row * (size_t)p.n + (size_t)yrow[tt][i2]) * nb + b;
-                                    p.dbg_dot[idx] = dsum[tt][i2];
-                                    p.dbg_min[idx] = msum[tt][i2];
+                            for (int j = 0; j < 2; ++j) {
+                                if (yrow[tt][j] >= 0 && row < p.rows) {
+                                    const size_t idx = ((size_t)row * (size_t)p.n + (size_t)yrow[tt][j]) * nb + b;
+                                    p.dbg_dot[idx] = dsum[tt][j];
+                                    p.dbg_min[idx] = msum[tt][j];
                                 }
                             }
                     }
                 }
             };
-            issue(t0, a0, 0);
-            int64_t i = 0;
-            while (i + 2 < cnt) {
-                issue(t1, a1, i + 1);
-                consume(t0, a0, i);
-                issue(t0, a0, i + 2);
-                consume(t1, a1, i + 1);
-                i += 2;
-            }
-            if (cnt - i == 2) {
-                issue(t1, a1, i + 1);
-                consume(t0, a0, i);
-                consume(t1, a1, i + 1);
-            } else {
-                consume(t0, a0, i);
+#pragma unroll
+            for (int st = 0; st < S - 1; ++st) issue(st, st);
+            for (int base = 0; base < cnt; base += S) {
+#pragma unroll
+                for (int st = 0; st < S; ++st) {
+                    const int i = base + st;
+                    issue((st + S - 1) % S, i + S - 1);
+                    if (i < cnt) consume(st, i);
+                }
             }
         }
+#if MQ_ABLATE & 4
+        stamp[1] = wall_clock64();
+#endif
 
         // ---- cross-wave reduction in wave order, then the epilogue on wave 0 ----
         if (n_waves > 1) {
@@ -256,8 +310,8 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            red[((((wave - 1) * NMAT + m) * TT + tt) * 4 + i) * 64 + lane] = acc[m][tt][i];
+                        for (int j = 0; j < 2; ++j)
+                            red[((((wave - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane] = acc[m][tt][j];
             }
             __syncthreads();
         }
@@ -268,32 +322,80 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            acc[m][tt][i] =
-                                __fadd_rn(acc[m][tt][i], red[((((wv - 1) * NMAT + m) * TT + tt) * 4 + i) * 64 + lane]);
+                        for (int j = 0; j < 2; ++j)
+                            acc[m][tt][j] =
+                                __fadd_rn(acc[m][tt][j], red[((((wv - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane]);
             }
             const int64_t row = rt * 16 + slot;
             if (row < p.rows) {
 #pragma unroll
                 for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        if (yrow[tt][i] >= 0) {
-                            float v = acc[0][tt][i];
-                            if (NMAT == 2) v = silu_mul(v, acc[1][tt][i], silu_mode);
-                            p.y[(size_t)yrow[tt][i] * (size_t)p.ldy + (size_t)row] = v;
+                    for (int j = 0; j < 2; ++j) {
+                        if (yrow[tt][j] >= 0) {
+                            float v = acc[0][tt][j];
+                            if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][tt][j], silu_mode);
+                            float* dst = p.y + (size_t)yrow[tt][j] * (size_t)p.ldy + (size_t)row;
+                            if (p.out_aq) {  // another workgroup re-reads this value: store it device-coherently
+                                __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            } else {
+                                *dst = v;
+                            }
                         }
                     }
             }
         }
-        if (n_waves > 1 && chunk + 16 * TT < count) __syncthreads();  // red[] is reused by the next chunk
+        if (n_waves > 1 && chunk + kTokTile * TT < count) __syncthreads();  // red[] is reused by the next chunk
+#if MQ_ABLATE & 4
+        stamp[2] = wall_clock64();
+        if (lane == 0 && p.dbg_min) {
+            long long* o = reinterpret_cast<long long*>(p.dbg_min) + ((size_t)blockIdx.x * n_waves + wave) * 4;
+            o[0] = stamp[0];
+            o[1] = stamp[1];
+            o[2] = stamp[2];
+            o[3] = 0;
+        }
+#endif
+    }
+
+    // ---- optional: the last workgroup to finish a 256-row block of y re-quantizes it to Q8_K ----
+    if (p.out_aq) {
+        __shared__ int is_last;
+        const int out_nb = (int)(p.rows >> 8);
+        const int hb = (int)(rt >> 4);
+        // The y stores above are device-scope write-through stores.  A workgroup barrier does not
+        // wait for global stores, so wait for their acknowledgement explicitly: after this they are
+        // visible device-wide and the workgroup may be counted.  (A full release fence would write
+        // back the whole L2 of this XCD on every workgroup.)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t* c = p.out_counters + (size_t)blockIdx.y * out_nb + hb;
+            const uint32_t prev = atomicAdd(c, 1u);
+            is_last = prev == 15u;
+            if (prev == 15u) atomicExch(c, 0u);  // leave the counters zero for the next launch
+        }
+        __syncthreads();
+        if (is_last) {
+            for (int e = wave; e < count; e += n_waves) {
+                int ar, yr;
+                entry_rows<GROUPED>(p, shared_group, begin, e, ar, yr);
+                const float* src = p.y + (size_t)yr * (size_t)p.ldy + (size_t)hb * 256 + lane * 4;
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)  // device-scope loads: other workgroups wrote these values
+                    v[j] = __hip_atomic_load(src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const Q8Lane r = quantize_block_q8k(v, lane);
+                store_amajor(p.out_aq, p.out_ad, yr, hb, out_nb, lane, r);
+            }
+        }
     }
 }
 
+// Waves per workgroup: the chip holds 2 waves per SIMD of this kernel (2048 in all); aim at filling
+// that once, with a count that divides the super-blocks of a row evenly and at most 8.
 int pick_waves(int64_t nb, int64_t workgroups) {
-    // Aim at ~4 waves per SIMD over the whole chip (256 CUs x 4 SIMDs), with waves that divide
-    // the super-blocks of a row evenly where possible.
-    const int64_t target = 4096;
+    const int64_t target = 2048;
     int64_t ideal = (target + workgroups - 1) / (workgroups > 0 ? workgroups : 1);
     if (ideal < 1) ideal = 1;
     if (ideal > 8) ideal = 8;
@@ -306,7 +408,7 @@ int pick_waves(int64_t nb, int64_t workgroups) {
 
 template <int NMAT, int TT, bool GROUPED, bool DEBUG>
 hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream) {
-    const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 4 * 64 * sizeof(float) : 0;
+    const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
     hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, a);
     return hipGetLastError();
 }
@@ -315,18 +417,19 @@ hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t str
 
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
     if (a.rows <= 0 || a.nb <= 0) return hipErrorInvalidValue;
+    if (a.out_aq && (a.rows & 255)) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
     const int nmat = a.swiglu ? 2 : 1;
     const bool debug = a.dbg_dot != nullptr;
-    // widest activation group this launch can see decides the token-tile count
+    // widest activation group this launch can see decides how many 8-row token tiles a pass holds
     const int64_t widest = a.grouped ? (a.n > a.sh_tokens ? a.n : a.sh_tokens) : a.n;
-    const int tt = widest <= 16 ? 1 : (widest <= 32 ? 2 : 4);
+    const int tt = widest <= 8 ? 1 : 2;
     const int groups = a.grouped ? a.max_groups + (a.sh_tokens > 0 ? 1 : 0) : 1;
-    // expected live groups: at most one per routed (token, k) pair
-    int64_t live = a.grouped ? groups : 1;
-    int waves = pick_waves(a.nb, rowtiles * live);
-    if (const char* ev = getenv("MQ_WAVES")) waves = atoi(ev) > 0 ? atoi(ev) : waves;  // tuning knob
-    while (waves > 1 && ((size_t)(waves - 1) * nmat * tt * 1024 > 64 * 1024 || a.nb % waves != 0)) --waves;
+    int waves = pick_waves(a.nb, rowtiles * groups);
+    if (const char* ev = getenv("MQ_WAVES")) {  // tuning knob
+        const int v = atoi(ev);
+        if (v > 0 && v <= 8 && a.nb % v == 0) waves = v;
+    }
     const dim3 grid((unsigned)rowtiles, (unsigned)groups);
 
 #define MQ_LAUNCH(NM, T)                                                              \
@@ -338,12 +441,10 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
 
     if (nmat == 1) {
         if (tt == 1) MQ_LAUNCH(1, 1);
-        if (tt == 2) MQ_LAUNCH(1, 2);
-        MQ_LAUNCH(1, 4);
+        MQ_LAUNCH(1, 2);
     } else {
         if (tt == 1) MQ_LAUNCH(2, 1);
-        if (tt == 2) MQ_LAUNCH(2, 2);
-        MQ_LAUNCH(2, 4);
+        MQ_LAUNCH(2, 2);
     }
 #undef MQ_LAUNCH
     return hipSuccess;

@@ -1,0 +1,87 @@
+// Wave-level Q8_K quantization of one 256-value super-block, shared by the stand-alone quantizer
+// and by the matmul epilogue that re-quantizes its own output.
+//
+// Bit-exact with the reference quantizer (core/src/kernels/hwy/hwy_moe_quant.cc:103-143):
+//   * the extreme element is the FIRST one of largest magnitude and keeps its sign, so the
+//     cross-lane arg-max breaks ties towards the lower index;
+//   * iscale = -127/max and d = 1/iscale are correctly rounded divisions;
+//   * iscale*x is rounded before the +1.5*2^23 add (no FMA contraction), which then yields
+//     round-half-even in the low mantissa bits.
+#pragma once
+
+#include "common.h"
+
+namespace mq {
+
+#if defined(__HIPCC__)
+__device__ __forceinline__ int nearest_int_rne(float v) {
+    const float biased = __fadd_rn(v, 12582912.0f);
+    return (__float_as_int(biased) & 0x007fffff) - 0x00400000;
+}
+
+struct Q8Lane {
+    uint32_t packed;  // this lane's four int8 codes (elements 4*lane .. 4*lane+3)
+    float d;          // block scale (same in every lane)
+    int bsum;         // lanes 4j..4j+3: sum of codes 16j..16j+15
+};
+
+// Every lane of the wave passes elements 4*lane .. 4*lane+3 of the block.
+__device__ __forceinline__ Q8Lane quantize_block_q8k(const float (&e)[4], int lane) {
+    float best_abs = 0.0f, best = 0.0f;
+    int best_idx = lane * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a = fabsf(e[j]);
+        if (a > best_abs) {
+            best_abs = a;
+            best = e[j];
+            best_idx = lane * 4 + j;
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float o_abs = __shfl_xor(best_abs, off, 64);
+        const float o_val = __shfl_xor(best, off, 64);
+        const int o_idx = __shfl_xor(best_idx, off, 64);
+        if (o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx)) {
+            best_abs = o_abs;
+            best = o_val;
+            best_idx = o_idx;
+        }
+    }
+    int q[4] = {0, 0, 0, 0};
+    Q8Lane r;
+    r.d = 0.0f;
+    if (best_abs != 0.0f) {
+        const float iscale = __fdiv_rn(-127.0f, best);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int v = nearest_int_rne(__fmul_rn(iscale, e[j]));
+            q[j] = v > 127 ? 127 : v;
+        }
+        r.d = __fdiv_rn(1.0f, iscale);
+    }
+    r.packed = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) | ((uint32_t)(q[2] & 0xff) << 16) |
+               ((uint32_t)(q[3] & 0xff) << 24);
+    int s = q[0] + q[1] + q[2] + q[3];
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    r.bsum = s;
+    return r;
+}
+
+// Writes the lane's codes of activation row m, super-block b into the A-major layout (common.h).
+__device__ __forceinline__ void store_amajor(uint8_t* aq, float* ad, int64_t m, int64_t b, int64_t nb, int lane,
+                                             const Q8Lane& r) {
+    // element 4*lane+j: sub-block g = lane/8, index in sub-block 4*(lane%8)+j.  The codes go to the
+    // half of the row's slot that belongs to the sub-block's parity, zeros to the other half.
+    const int g = lane >> 3, h = g & 1;
+    const int kq = (lane & 7) >> 1;
+    const size_t off = aq_offset(m, b, g >> 1, kq, h, nb) + (size_t)(lane & 1) * 4;
+    *reinterpret_cast<uint32_t*>(aq + off + h * 8) = r.packed;
+    *reinterpret_cast<uint32_t*>(aq + off + (1 - h) * 8) = 0u;
+    if (lane == 0) ad[ad_index(m, b, nb)] = r.d;
+}
+#endif
+
+}  // namespace mq

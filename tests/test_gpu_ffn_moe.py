@@ -220,7 +220,11 @@ def test_moe_layer_stagewise(ops, n, silu):
     sh_gpu = ops.ffn_swiglu(SG, SU, SD, cu(x), 2).cpu().numpy()
     gate = 1.0 / (1.0 + np.exp(-(x.astype(np.float64) @ gate_inp.astype(np.float64))))
     want = y_routed.astype(np.float64) + sh_gpu.astype(np.float64) * gate[:, None]
-    assert np.max(np.abs(y - want)) <= 2e-6 * np.max(np.abs(want))
+    # the shared expert runs as one more group of the expert-routed launch, whose wave split (and so
+    # its fp32 summation order) may differ from the dense launch: an ulp in the hidden state can flip
+    # a Q8_K code, hence the end-to-end bound here and the tight bound on the typical token
+    rel = np.max(np.abs(y - want), axis=1) / np.max(np.abs(want), axis=1)
+    assert np.max(rel) <= END_TO_END_REL and np.median(rel) <= 2e-6
     for w in (GE, UE, DE, SG, SU, SD):
         w.free()
 
