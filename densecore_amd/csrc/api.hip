@@ -493,8 +493,8 @@ int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int
                       int32_t* ids_dev, float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;
     if (!logits_dev || !ids_dev || !weights_dev) return fail(MQ_ERR_INVALID, "mq_moe_route_topk: null pointer");
-    if (n < 0 || n_experts <= 0 || top_k <= 0 || top_k > n_experts || top_k > 8)
-        return fail(MQ_ERR_INVALID, "mq_moe_route_topk: need 0 < top_k <= min(8, n_experts)");
+    if (n < 0 || n_experts <= 0 || n_experts > 2048 || top_k <= 0 || top_k > n_experts || top_k > 8)
+        return fail(MQ_ERR_INVALID, "mq_moe_route_topk: need 0 < top_k <= min(8, n_experts) and n_experts <= 2048");
     if (weights_mode < 0 || weights_mode > 2) return fail(MQ_ERR_INVALID, "mq_moe_route_topk: weights_mode %d", weights_mode);
     if (n == 0) return MQ_OK;
     MQ_HIP(launch_route_topk(logits_dev, n_experts, n, top_k, weights_mode, ids_dev, weights_dev, (hipStream_t)stream));
@@ -773,18 +773,18 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     const int slots = K + (sh.gate ? 1 : 0);  // hidden / partial rows per token
     RouteWs r;
     if (int rc = carve_route(n, K, E, r)) return rc;
-    MQ_HIP(launch_route_topk(logits_dev, E, n, K, L->route_mode, r.ids, r.weights, s));
-    MQ_HIP(launch_build_groups(r.ids, n, K, E, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
+    // ids and weights go straight to the caller's buffers when it wants them
+    int32_t* ids = ids_out_dev ? ids_out_dev : r.ids;
+    float* wts = weights_out_dev ? weights_out_dev : r.weights;
+    // one arrival counter, kept apart from the quantization counters (last slot of that buffer)
+    if (int rc = reserve_counters(4096)) return rc;
+    MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
+                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
     if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
-    if (int rc = run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, r.ids, r.weights,
-                              L->sh_gate_inp_dev, x_dev, y_dev, s))
-        return rc;
-    const size_t pair_bytes = (size_t)n * K * 4;
-    if (ids_out_dev) MQ_HIP(hipMemcpyAsync(ids_out_dev, r.ids, pair_bytes, hipMemcpyDeviceToDevice, s));
-    if (weights_out_dev) MQ_HIP(hipMemcpyAsync(weights_out_dev, r.weights, pair_bytes, hipMemcpyDeviceToDevice, s));
-    return MQ_OK;
+    return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
+                        x_dev, y_dev, s);
 }
 
 // ---------------------------------------------------------------------------------- census

@@ -76,6 +76,10 @@ hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, 
 hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t n_experts, int32_t* group_expert,
                                int32_t* group_begin, int32_t* n_groups, int32_t* entry_token, int32_t* entry_k,
                                hipStream_t stream);
+// Router and grouping in one launch at decode widths (falls back to the two kernels above for n > 256).
+hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
+                                  float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, hipStream_t stream);
 // y[t][r] = sum_k w[t][k] * part[t*slots + k][r]  (k in order) + gate[t] * part[t*slots + top_k][r]
 hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots, int64_t rows, const float* weights,
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,

@@ -192,14 +192,18 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     bool shared_group = false;
     int silu_mode = p.silu_mode;
     if (GROUPED) {
-        const int ng = *p.n_groups;
+        // the three list reads are independent of each other (the lists are sized for every
+        // possible group), so they cost one memory round trip, not three
         const int g = blockIdx.y;
+        const int ng = *p.n_groups;
+        const int g_expert = p.group_expert[g];
+        const int g_begin = p.group_begin[g], g_end = p.group_begin[g + 1];
         if (g < ng) {
-            const size_t eoff = (size_t)p.group_expert[g] * p.expert_bytes;
+            const size_t eoff = (size_t)g_expert * p.expert_bytes;
             w[0] += eoff;
             if (NMAT == 2) w[1] += eoff;
-            begin = p.group_begin[g];
-            count = p.group_begin[g + 1] - begin;
+            begin = g_begin;
+            count = g_end - g_begin;
         } else if (g == ng && p.sh_tokens > 0) {
             shared_group = true;
             w[0] = p.sh_w0;
@@ -423,7 +427,9 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
     const bool debug = a.dbg_dot != nullptr;
     // widest activation group this launch can see decides how many 8-row token tiles a pass holds
     const int64_t widest = a.grouped ? (a.n > a.sh_tokens ? a.n : a.sh_tokens) : a.n;
-    const int tt = widest <= 8 ? 1 : 2;
+    // Expert groups rarely hold more than 8 rows at decode widths; the few that do (and the shared
+    // expert) take a second pass over their 16 rows of weights, which then come from cache.
+    const int tt = (a.grouped || widest <= 8) ? 1 : 2;
     const int groups = a.grouped ? a.max_groups + (a.sh_tokens > 0 ? 1 : 0) : 1;
     int waves = pick_waves(a.nb, rowtiles * groups);
     if (const char* ev = getenv("MQ_WAVES")) {  // tuning knob

@@ -17,71 +17,23 @@ __device__ __forceinline__ bool precedes(float a, int ia, float b, int ib) {
     return ia < ib;
 }
 
-constexpr int kMaxPerLane = 16;  // up to 1024 experts per token
-
-// One wavefront per token.  Lane l owns experts l, l+64, ...; each of the top_k rounds takes the
-// best remaining candidate of the wave.
-__global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict__ logits, int n_experts, int64_t n,
-                                                         int top_k, int mode, int32_t* __restrict__ ids,
-                                                         float* __restrict__ weights) {
-    const int lane = threadIdx.x & 63;
-    const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (tok >= n) return;
-    const float* row = logits + tok * n_experts;
-    float v[kMaxPerLane];
-    uint32_t live = 0;
-#pragma unroll
-    for (int j = 0; j < kMaxPerLane; ++j) {
-        const int e = lane + 64 * j;
-        v[j] = 0.0f;
-        if (e < n_experts) {
-            v[j] = row[e];
-            live |= 1u << j;
-        }
+// 64-bit sort key of a router candidate: larger key = earlier in the routing order.  High word:
+// the logit mapped to an unsigned integer of the same order (NaN lowest, -0 folded into +0 because
+// the reference compares with < and >); low word: ~id, so that equal logits order by lower id.
+__device__ __forceinline__ unsigned long long route_key(float v, int id) {
+    uint32_t hi;
+    if (isnan(v)) {
+        hi = 0u;
+    } else {
+        const uint32_t bits = __float_as_uint(v == 0.0f ? 0.0f : v);
+        hi = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
     }
-    float sel_logit = 0.0f;  // lane k keeps the k-th selected logit
-    int sel_id = -1;
-    for (int k = 0; k < top_k; ++k) {
-        float best = 0.0f;
-        int best_id = 0x7fffffff;  // "none": loses to every real candidate below
-        bool have = false;
-#pragma unroll
-        for (int j = 0; j < kMaxPerLane; ++j) {
-            if (live & (1u << j)) {
-                const int e = lane + 64 * j;
-                if (!have || precedes(v[j], e, best, best_id)) {
-                    best = v[j];
-                    best_id = e;
-                    have = true;
-                }
-            }
-        }
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const float ob = __shfl_xor(best, off, 64);
-            const int oid = __shfl_xor(best_id, off, 64);
-            const bool ohave = oid != 0x7fffffff;
-            if (ohave && (!have || precedes(ob, oid, best, best_id))) {
-                best = ob;
-                best_id = oid;
-                have = true;
-            }
-        }
-        if ((best_id & 63) == lane) live &= ~(1u << (best_id >> 6));
-        if (lane == k) {
-            sel_logit = best;
-            sel_id = best_id;
-        }
-    }
-    if (lane < top_k) ids[tok * top_k + lane] = sel_id;
+    return ((unsigned long long)hi << 32) | (unsigned long long)(uint32_t)(~(uint32_t)id);
+}
 
-    // softmax over the selected logits, summed in routing order on one lane
-    float l[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) l[k] = __shfl(sel_logit, k < top_k ? k : 0, 64);
-    if (lane != 0) return;
+// softmax over the selected logits, summed in routing order (three reference variants)
+__device__ __forceinline__ void route_weights(const float* l, int top_k, int mode, float* __restrict__ out) {
     float w[8];
-    float* out = weights + tok * top_k;
     if (mode == 0) {  // core/src/llm/moe/native.cpp:650-675
         float mx = -INFINITY;
         bool all_finite = true;
@@ -98,9 +50,9 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
         }
         if (!(den > 0.0f) || !isfinite(den)) {
             for (int k = 0; k < top_k; ++k) out[k] = __fdiv_rn(1.0f, (float)top_k);
-            return;
+        } else {
+            for (int k = 0; k < top_k; ++k) out[k] = __fdiv_rn(w[k], den);
         }
-        for (int k = 0; k < top_k; ++k) out[k] = __fdiv_rn(w[k], den);
     } else if (mode == 1) {  // core/src/llm/moe/native.cpp:2321-2355
         float mx = -INFINITY;
         for (int k = 0; k < top_k; ++k) mx = fmaxf(mx, l[k]);
@@ -127,18 +79,70 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
     }
 }
 
-// Single workgroup.  Counting sort of the (token, k) pairs by expert; pairs keep their natural
+constexpr int kMaxExperts = 2048;
+
+// Routing of one token by one workgroup of 256 threads: every expert's rank is the number of
+// candidates that precede it (ComputeQwenNativeMoEStableTopK's order, core/src/llm/moe/native.cpp:610-645);
+// the experts of rank < top_k are the selection, already in routing order.
+// keys: n_experts 64-bit words of LDS; sel: 8 floats + 8 ints of LDS.
+__device__ __forceinline__ void route_token_block(const float* __restrict__ row, int n_experts, int top_k, int mode,
+                                                  unsigned long long* keys, float* sel_logit, int32_t* sel_id,
+                                                  int32_t* __restrict__ ids_out, float* __restrict__ w_out,
+                                                  bool coherent_ids) {
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_experts; e += 256) keys[e] = route_key(row[e], e);
+    __syncthreads();
+    for (int e = tid; e < n_experts; e += 256) {
+        const unsigned long long mine = keys[e];
+        int rank = 0;
+        int j = 0;
+        for (; j + 16 <= n_experts; j += 16) {  // batches of 16 keep the LDS reads pipelined
+            unsigned long long k16[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) k16[u] = keys[j + u];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) rank += k16[u] > mine;
+        }
+        for (; j < n_experts; ++j) rank += keys[j] > mine;
+        if (rank < top_k) {
+            sel_logit[rank] = row[e];
+            sel_id[rank] = e;
+        }
+    }
+    __syncthreads();
+    if (tid < top_k) {
+        if (coherent_ids) {
+            __hip_atomic_store(ids_out + tid, sel_id[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            ids_out[tid] = sel_id[tid];
+        }
+    }
+    if (tid == 0) {
+        float l[8];
+        for (int k = 0; k < top_k; ++k) l[k] = sel_logit[k];
+        route_weights(l, top_k, mode, w_out);
+    }
+}
+
+__global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict__ logits, int n_experts, int top_k,
+                                                         int mode, int32_t* __restrict__ ids,
+                                                         float* __restrict__ weights) {
+    extern __shared__ unsigned long long route_sh[];  // [n_experts] keys, then 8 floats, 8 ints
+    float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
+    int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
+    const int64_t tok = blockIdx.x;
+    route_token_block(logits + tok * n_experts, n_experts, top_k, mode, route_sh, sel_logit, sel_id, ids + tok * top_k,
+                      weights + tok * top_k, false);
+}
+
+// Counting sort of the (token, k) pairs by expert, by one workgroup.  Pairs keep their natural
 // (token, k) order inside an expert, which is the (expert, token, k) order of
 // core/src/llm/moe/native.cpp:1726-1730.  Experts nobody selected produce no group.
-__global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __restrict__ ids, int n_entries,
-                                                            int top_k, int n_experts, int32_t* __restrict__ group_expert,
-                                                            int32_t* __restrict__ group_begin,
-                                                            int32_t* __restrict__ n_groups,
-                                                            int32_t* __restrict__ entry_token,
-                                                            int32_t* __restrict__ entry_k) {
-    extern __shared__ int32_t sh[];  // [n_experts] counts -> offsets, [n_experts] group index
-    int32_t* count = sh;
-    int32_t* gidx = sh + n_experts;
+// ids may live in LDS or in global memory; count[] is n_experts ints of LDS.
+__device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries, int top_k, int n_experts,
+                                              int32_t* count, int32_t* __restrict__ group_expert,
+                                              int32_t* __restrict__ group_begin, int32_t* __restrict__ n_groups,
+                                              int32_t* __restrict__ entry_token, int32_t* __restrict__ entry_k) {
     const int tid = threadIdx.x, nt = blockDim.x;
     for (int e = tid; e < n_experts; e += nt) count[e] = 0;
     __syncthreads();
@@ -147,32 +151,127 @@ __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __res
         if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
     }
     __syncthreads();
-    if (tid == 0) {  // n_experts is a few hundred: a serial scan costs less than a barrier tree here
-        int off = 0, g = 0;
-        for (int e = 0; e < n_experts; ++e) {
-            const int c = count[e];
-            count[e] = off;
-            if (c > 0) {
-                group_expert[g] = e;
-                group_begin[g] = off;
-                gidx[e] = g;
-                ++g;
+    if (tid < 64) {  // wave 0: exclusive scan over the experts, lane l covers a run of consecutive experts
+        const int per = (n_experts + 63) / 64;
+        const int e0 = tid * per;
+        int sum = 0, active = 0;
+        for (int j = 0; j < per; ++j) {
+            const int e = e0 + j;
+            if (e < n_experts) {
+                sum += count[e];
+                active += count[e] > 0;
             }
-            off += c;
         }
-        group_begin[g] = off;
-        *n_groups = g;
+        int off = sum, g = active;  // inclusive scans across lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int o = __shfl_up(off, d, 64);
+            const int og = __shfl_up(g, d, 64);
+            if (tid >= d) {
+                off += o;
+                g += og;
+            }
+        }
+        const int total = __shfl(off, 63, 64), groups = __shfl(g, 63, 64);
+        off -= sum;
+        g -= active;
+        for (int j = 0; j < per; ++j) {
+            const int e = e0 + j;
+            if (e < n_experts) {
+                const int c = count[e];
+                count[e] = off;
+                if (c > 0) {
+                    group_expert[g] = e;
+                    group_begin[g] = off;
+                    ++g;
+                }
+                off += c;
+            }
+        }
+        if (tid == 0) {
+            group_begin[groups] = total;
+            *n_groups = groups;
+        }
     }
     __syncthreads();
     for (int i = tid; i < n_entries; i += nt) {
         const int e = ids[i];
         if (e < 0 || e >= n_experts) continue;
         int rank = 0;  // earlier pairs routed to the same expert
-        for (int j = 0; j < i; ++j) rank += ids[j] == e;
+        int j = 0;
+        for (; j + 16 <= i; j += 16) {
+            int v16[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v16[u] = ids[j + u];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) rank += v16[u] == e;
+        }
+        for (; j < i; ++j) rank += ids[j] == e;
         const int pos = count[e] + rank;
         entry_token[pos] = i / top_k;
         entry_k[pos] = i - (i / top_k) * top_k;
     }
+}
+
+__global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __restrict__ ids, int n_entries,
+                                                            int top_k, int n_experts, int use_lds,
+                                                            int32_t* __restrict__ group_expert,
+                                                            int32_t* __restrict__ group_begin,
+                                                            int32_t* __restrict__ n_groups,
+                                                            int32_t* __restrict__ entry_token,
+                                                            int32_t* __restrict__ entry_k) {
+    extern __shared__ int32_t sh[];  // [n_experts] counts -> offsets, then [n_entries] ids when they fit
+    int32_t* count = sh;
+    const int32_t* src = ids;
+    if (use_lds) {
+        int32_t* ids_s = sh + n_experts;
+        for (int i = threadIdx.x; i < n_entries; i += blockDim.x) ids_s[i] = ids[i];
+        src = ids_s;  // the barrier inside group_entries orders these stores
+    }
+    group_entries(src, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k);
+}
+
+// Router and grouping in one launch (decode widths): a workgroup per token routes it; the last
+// workgroup to finish gathers all ids and builds the expert groups.  `arrivals` is one zeroed
+// uint32 in device memory that the kernel leaves zero again.
+__global__ void __launch_bounds__(256) route_and_group_kernel(const float* __restrict__ logits, int n_experts, int n,
+                                                              int top_k, int mode, int32_t* __restrict__ ids,
+                                                              float* __restrict__ weights, uint32_t* arrivals,
+                                                              int32_t* __restrict__ group_expert,
+                                                              int32_t* __restrict__ group_begin,
+                                                              int32_t* __restrict__ n_groups,
+                                                              int32_t* __restrict__ entry_token,
+                                                              int32_t* __restrict__ entry_k) {
+    extern __shared__ unsigned long long route_sh[];  // keys | sel | then reused: counts, ids
+    __shared__ int is_last;
+    float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
+    int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
+    const bool solo = gridDim.x == 1;  // up to four tokens: one workgroup does everything, no handshake
+    const int per_block = solo ? n : 1;
+    for (int t = 0; t < per_block; ++t) {
+        const int tok = blockIdx.x * per_block + t;
+        route_token_block(logits + (size_t)tok * n_experts, n_experts, top_k, mode, route_sh, sel_logit, sel_id,
+                          ids + (size_t)tok * top_k, weights + (size_t)tok * top_k, !solo);
+        __syncthreads();  // keys / sel are reused by the next token and by the grouping below
+    }
+    if (!solo) {
+        // the ids were stored device-coherently; wait for their acknowledgement before being counted
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t prev = atomicAdd(arrivals, 1u);
+            is_last = prev == (uint32_t)(n - 1);
+            if (is_last) atomicExch(arrivals, 0u);
+        }
+        __syncthreads();
+        if (!is_last) return;
+    }
+    int32_t* count = reinterpret_cast<int32_t*>(route_sh);
+    int32_t* ids_s = count + n_experts;
+    const int n_entries = n * top_k;
+    for (int i = threadIdx.x; i < n_entries; i += 256)
+        ids_s[i] = solo ? ids[i] : __hip_atomic_load(ids + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    group_entries(ids_s, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k);
 }
 
 __device__ __forceinline__ float stable_sigmoid(float x) {  // core/src/llm/graph/fused_ops.cpp:451-458
@@ -227,9 +326,10 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, s
 
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                              float* weights, hipStream_t stream) {
-    if (n_experts > 64 * kMaxPerLane || top_k > 8) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, logits, (int)n_experts, n,
-                       top_k, mode, ids, weights);
+    if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
+    const size_t lds = (size_t)n_experts * 8 + 64;
+    hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)n), dim3(256), lds, stream, logits, (int)n_experts, top_k, mode,
+                       ids, weights);
     return hipGetLastError();
 }
 
@@ -239,8 +339,29 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     const int64_t entries = n * top_k;
     if (entries > (int64_t)1 << 30 || n_experts > 8192) return hipErrorInvalidValue;
     const int threads = entries >= 1024 ? 1024 : (entries > 256 ? 512 : 256);
-    hipLaunchKernelGGL(build_groups_kernel, dim3(1), dim3(threads), (size_t)n_experts * 8, stream, ids, (int)entries,
-                       top_k, (int)n_experts, group_expert, group_begin, n_groups, entry_token, entry_k);
+    const int use_lds = entries <= 8192;
+    const size_t lds = (size_t)n_experts * 4 + (use_lds ? (size_t)entries * 4 : 0);
+    hipLaunchKernelGGL(build_groups_kernel, dim3(1), dim3(threads), lds, stream, ids, (int)entries, top_k,
+                       (int)n_experts, use_lds, group_expert, group_begin, n_groups, entry_token, entry_k);
+    return hipGetLastError();
+}
+
+hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
+                                  float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, hipStream_t stream) {
+    if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
+    const size_t lds_route = (size_t)n_experts * 8 + 64;
+    const size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
+    if (lds_group > 60 * 1024) {  // prefill widths: route, then group from global memory
+        hipError_t e = launch_route_topk(logits, n_experts, n, top_k, mode, ids, weights, stream);
+        if (e != hipSuccess) return e;
+        return launch_build_groups(ids, n, top_k, n_experts, group_expert, group_begin, n_groups, entry_token, entry_k,
+                                   stream);
+    }
+    hipLaunchKernelGGL(route_and_group_kernel, dim3(n <= 4 ? 1u : (unsigned)n), dim3(256),
+                       lds_route > lds_group ? lds_route : lds_group,
+                       stream, logits, (int)n_experts, (int)n, top_k, mode, ids, weights, arrivals, group_expert,
+                       group_begin, n_groups, entry_token, entry_k);
     return hipGetLastError();
 }
 
