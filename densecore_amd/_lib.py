@@ -16,7 +16,7 @@ EXPORTS = [
     "mq_weight_upload", "mq_weight_synthetic", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
     "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
-    "mq_moe_route_topk", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums",
+    "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums",
     "mq_census_enable", "mq_census_reset", "mq_census_read",
     "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_stream_synchronize",
 ]
@@ -66,6 +66,7 @@ def load() -> C.CDLL:
     L.mq_moe_gateup_swiglu_q4k.argtypes = [vp, vp, vp, i64, vp, ci, ci, vp, vp]
     L.mq_moe_down_weighted_q4k.argtypes = [vp, vp, i64, vp, vp, ci, vp, vp]
     L.mq_moe_route_topk.argtypes = [vp, i64, i64, ci, ci, vp, vp, vp]
+    L.mq_moe_weights_from_logits.argtypes = [vp, i64, i64, vp, ci, vp, vp]
     L.mq_mul_mat_id_q4k.argtypes = [vp, vp, i64, ci, vp, ci, vp, vp]
     L.mq_moe_layer_q4k.argtypes = [C.POINTER(MoELayerDesc), vp, vp, i64, vp, vp, vp, vp]
     L.mq_debug_block_sums.argtypes = [vp, vp, i64, i64, vp, vp, vp, i64, vp]

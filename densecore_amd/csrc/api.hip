@@ -501,6 +501,17 @@ int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int
     return MQ_OK;
 }
 
+int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev, int top_k,
+                               float* weights_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!logits_dev || !ids_dev || !weights_dev) return fail(MQ_ERR_INVALID, "mq_moe_weights_from_logits: null pointer");
+    if (n < 0 || n_experts <= 0 || top_k <= 0 || top_k > 8)
+        return fail(MQ_ERR_INVALID, "mq_moe_weights_from_logits: need n_experts > 0 and 0 < top_k <= 8");
+    if (n == 0) return MQ_OK;
+    MQ_HIP(launch_weights_from_ids(logits_dev, n_experts, n, ids_dev, top_k, weights_dev, (hipStream_t)stream));
+    return MQ_OK;
+}
+
 int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
                       int top_k, float* y_dev, void* stream) {
     if (int rc = check_ready()) return rc;

@@ -73,6 +73,8 @@ hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, 
                              float* weights, hipStream_t stream);
 // Expert-grouped work list from ids [n][top_k]: entries sorted by (expert, token, k).
 //   group_expert[g], group_begin[g..g+1], n_groups[0], entry_token[e], entry_k[e]
+hipError_t launch_weights_from_ids(const float* logits, int64_t n_experts, int64_t n, const int32_t* ids, int top_k,
+                                   float* weights, hipStream_t stream);
 hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t n_experts, int32_t* group_expert,
                                int32_t* group_begin, int32_t* n_groups, int32_t* entry_token, int32_t* entry_k,
                                hipStream_t stream);

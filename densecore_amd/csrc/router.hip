@@ -135,6 +135,33 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
                       weights + tok * top_k, false);
 }
 
+// Weights of already-selected experts from the raw logits (core/src/llm/moe/native.cpp:2305-2357):
+// invalid ids weigh 0 and take no part in the max; one thread per token.
+__global__ void __launch_bounds__(64) weights_from_ids_kernel(const float* __restrict__ logits, int n_experts, int n,
+                                                              const int32_t* __restrict__ ids, int top_k,
+                                                              float* __restrict__ weights) {
+    const int tok = blockIdx.x * 64 + threadIdx.x;
+    if (tok >= n) return;
+    const float* row = logits + (size_t)tok * n_experts;
+    float l[8];
+    bool ok[8];
+    float mx = -INFINITY;
+    for (int k = 0; k < top_k; ++k) {
+        const int e = ids[(size_t)tok * top_k + k];
+        ok[k] = e >= 0 && e < n_experts;
+        l[k] = ok[k] ? row[e] : 0.0f;
+        if (ok[k] && l[k] > mx) mx = l[k];
+    }
+    if (!isfinite(mx)) mx = 0.0f;
+    float den = 0.0f;
+    for (int k = 0; k < top_k; ++k) {
+        l[k] = ok[k] ? expf(__fsub_rn(l[k], mx)) : 0.0f;
+        if (ok[k]) den = __fadd_rn(den, l[k]);
+    }
+    den = den < 6.103515625e-5f ? 6.103515625e-5f : den;  // std::max(den, floor): a NaN den is replaced too
+    for (int k = 0; k < top_k; ++k) weights[(size_t)tok * top_k + k] = __fdiv_rn(l[k], den);
+}
+
 // Counting sort of the (token, k) pairs by expert, by one workgroup.  Pairs keep their natural
 // (token, k) order inside an expert, which is the (expert, token, k) order of
 // core/src/llm/moe/native.cpp:1726-1730.  Experts nobody selected produce no group.
@@ -330,6 +357,14 @@ hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, 
     const size_t lds = (size_t)n_experts * 8 + 64;
     hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)n), dim3(256), lds, stream, logits, (int)n_experts, top_k, mode,
                        ids, weights);
+    return hipGetLastError();
+}
+
+hipError_t launch_weights_from_ids(const float* logits, int64_t n_experts, int64_t n, const int32_t* ids, int top_k,
+                                   float* weights, hipStream_t stream) {
+    if (top_k > 8 || top_k <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(weights_from_ids_kernel, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, stream, logits,
+                       (int)n_experts, (int)n, ids, top_k, weights);
     return hipGetLastError();
 }
 

@@ -169,6 +169,17 @@ def moe_route_topk(logits: torch.Tensor, top_k: int, mode: int = ROUTE_FUSED):
     return ids, w
 
 
+def moe_weights_from_logits(logits: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """Qwen35NativeMoEComputeTopKWeightsFromLogits (core/src/llm/moe/native.cpp:2305-2357): weights of given ids."""
+    logits = _f32(logits)
+    ids = ids.contiguous()
+    n, e = logits.shape
+    w = torch.empty(ids.shape, dtype=torch.float32, device=logits.device)
+    _lib.check(_lib.lib().mq_moe_weights_from_logits(_ptr(logits), e, n, _ptr(ids), ids.shape[1], _ptr(w), _stream()),
+               "mq_moe_weights_from_logits")
+    return w
+
+
 def mul_mat_id(w: Q4KWeight, x: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     """ggml_mul_mat_id: x fp32 [n, cols] or [n, top_k, cols]; ids int32 [n, top_k] -> y [n, top_k, rows]."""
     x = _f32(x)

@@ -121,6 +121,13 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
 int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int top_k, int weights_mode,
                       int32_t* ids_dev, float* weights_dev, void* stream);
 
+/* Weights of ALREADY selected experts from the raw logits, as the down node resolves them itself:
+ * softmax over the valid selected logits (a non-finite max counts as 0, denominator floored at 2^-14),
+ * ids outside [0, n_experts) weigh 0.  Qwen35NativeMoEComputeTopKWeightsFromLogits
+ * (core/src/llm/moe/native.cpp:2305-2357). */
+int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev,
+                               int top_k, float* weights_dev, void* stream);
+
 /* ---- expert-routed matmul: ggml_mul_mat_id on GGML_TYPE_Q4_K -----------------
  * y[t][k][r] = W[ids[t][k]][r] . q8k(x[t][k or 0]).  x_dev fp32 [n][x_slots][cols]
  * with x_slots == 1 (one row per token, broadcast over k: the gate/up case) or

@@ -1,0 +1,85 @@
+/*
+ * mi355_q4k_ggml.h -- GGML_OP_CUSTOM adapters over the mi355_q4k C ABI.
+ *
+ * DenseCore replaces ggml_mul_mat / ggml_mul_mat_id by writing a
+ * {ggml_custom_op_t fn, n_tasks, userdata} triple into dst->op_params with
+ * dst->op = GGML_OP_CUSTOM (core/src/llm/matmul/graph_ops.cpp:212-227,297-308)
+ * or through ggml_custom_4d (core/src/llm/moe/native.cpp:4872-4873,4907-4909).
+ * The functions below have exactly that callback shape,
+ *     void fn(struct ggml_tensor* dst, int ith, int nth, void* userdata),
+ * read their operands from dst->src[] the way the callbacks they replace do,
+ * run the whole node on the GPU when ith == 0, return at once for ith > 0
+ * (the convention of cb_matmul_hal_custom, core/src/llm/matmul/exec.cpp:36),
+ * and synchronise before returning because the next graph node reads dst->data
+ * on the host.  Like the reference's callbacks they return void; an invalid
+ * node leaves dst untouched (core/src/llm/matmul/gemv_exec.cpp:102-143) and
+ * the reason is kept for mq_ggml_last_status() / mq_last_error().
+ *
+ * All tensor memory is host memory borrowed from the graph.  Weight tensors
+ * are uploaded to HBM the first time their data pointer is seen and kept in a
+ * process-wide cache keyed by (data, ne, nb) -- the counterpart of
+ * GetOrCreateQ4KRepackedGemvWeight's cache
+ * (core/src/kernels/q4k_repacked_gemv.cpp:403-470) -- until
+ * mq_ggml_weight_cache_clear().
+ *
+ * `struct ggml_tensor` is ggml's.  When no ggml header is on the include path
+ * the implementation is compiled against a field-for-field mirror of the
+ * members it reads (densecore_amd/host/ggml_tensor_mirror.h).
+ */
+#ifndef MI355_Q4K_GGML_H
+#define MI355_Q4K_GGML_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+struct ggml_tensor;
+
+/* Optional userdata of every adapter (NULL = defaults).  The graph owns it, as it owns
+ * GemvUserData / Qwen35SharedQ8RowsUserData (core/src/llm/runtime/work_context.h:10-11,
+ * core/src/llm/moe/native.cpp:1027-1038). */
+typedef struct {
+    int silu_mode;    /* MQ_SILU_*  (gate/up node); default MQ_SILU_EXACT for n <= 4, MQ_SILU_FAST above,
+                         as core/src/llm/moe/native.cpp:3614-3616 and cpu_backend_moe_raw_batched.inl:1673 choose */
+    int route_mode;   /* MQ_ROUTE_* (down node: weights from logits); default MQ_ROUTE_FLOOR_FINITE */
+    int use_defaults; /* non-zero: ignore the two fields above */
+    int last_status;  /* written by the adapter: MQ_OK or MQ_ERR_* */
+} mq_ggml_userdata;
+
+/* dst F32 ne=[N_out, M]; src[0] = input F32 ne=[K_in, M] (column stride nb[1]); src[1] = weight
+ * Q4_K ne=[K_in, N_out], nb[1] = row bytes.  cb_gemv_custom (core/src/llm/matmul/gemv_exec.cpp:99-143). */
+void mq_cb_gemv_custom(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+/* Same operands with 2 <= M; cb_gemv_batched_custom (core/src/llm/matmul/batched_exec.cpp:55-74). */
+void mq_cb_gemv_batched_custom(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+/* dst F32 ne=[n_ff, top_k, n_tokens]; src = {gate_exps Q4_K ne=[n_embd, n_ff, n_expert], up_exps,
+ * input F32 ne=[n_embd, n_tokens], selected_experts I32 ne=[top_k, n_tokens]}.
+ * cb_qwen35_native_moe_gateup_raw_qxk_swiglu (core/src/llm/moe/native.cpp:3929-4345, :4871-4874). */
+void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+/* dst F32 ne=[n_embd, n_tokens]; src = {down_exps Q4_K ne=[n_ff, n_embd, n_expert], hidden F32
+ * ne=[n_ff, top_k, n_tokens], selected_experts I32 ne=[top_k, n_tokens], gate_logits F32
+ * ne=[n_expert, n_tokens]}.  cb_qwen35_native_moe_down_q5k_weighted_logits
+ * (core/src/llm/moe/native.cpp:3051-3295, :4906-4909). */
+void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+
+/* Status of the calling thread's last adapter call (MQ_OK / MQ_ERR_*). */
+int mq_ggml_last_status(void);
+/* Frees every cached device weight (call when the model is unloaded). */
+int mq_ggml_weight_cache_clear(void);
+int64_t mq_ggml_weight_cache_size(void);
+
+/* Library-level boundary without a graph: C[M][N] = A[M][K] . W[N][K]^T with W raw ggml Q4_K rows.
+ * CpuBackend::MatMulGgmlQuantizedTransB(const Tensor& A, const GgmlQuantizedMatrixView& W, Tensor* C, int)
+ * (core/include/densecore/backend/cpu_backend.h:91-99,293-300) flattened to plain pointers: a/c are host
+ * fp32 with row strides lda/ldc in elements (Tensor::stride[0]); w_type_id must be 12 (GGML_TYPE_Q4_K).
+ * Returns 1 when the product was computed and 0 when the call is rejected, like the bool it replaces. */
+int mq_matmul_ggml_quantized_transb(const float* a, int64_t m, int64_t k, int64_t lda, const void* w_data,
+                                    int32_t w_type_id, int64_t w_rows, int64_t w_cols, size_t w_row_bytes, float* c,
+                                    int64_t ldc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_Q4K_GGML_H */

@@ -225,6 +225,17 @@ def route_topk(logits, top_k: int, weights_mode: int = 0):
     return ids, w
 
 
+def route_weights_from_ids(logits, ids) -> np.ndarray:
+    logits = _c(logits, np.float32)
+    ids = _c(ids, np.int32)
+    n, e = logits.shape
+    w = np.zeros(ids.shape, np.float32)
+    rc = lib().orc_route_weights_from_ids(_p(logits), C.c_int64(e), C.c_int64(n), _p(ids), C.c_int(ids.shape[1]), _p(w))
+    if rc:
+        raise ValueError(f"orc_route_weights_from_ids rc={rc}")
+    return w
+
+
 def build_assignments(ids, n_experts: int) -> np.ndarray:
     ids = _c(ids, np.int32)
     n, k = ids.shape

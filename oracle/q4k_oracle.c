@@ -570,6 +570,34 @@ int orc_route_topk(const float* logits, int64_t n_experts, int64_t n_tokens, int
     return 0;
 }
 
+/* Routing weights of GIVEN ids (the down node resolves them from the raw logits itself):
+ * native.cpp:2305-2357.  Ids outside [0, n_experts) get weight 0 and take no part in the max. */
+int orc_route_weights_from_ids(const float* logits, int64_t n_experts, int64_t n_tokens, const int32_t* ids, int top_k,
+                               float* weights) {
+    if (!logits || !ids || !weights || n_experts <= 0 || top_k <= 0 || n_tokens < 0) return -1;
+    for (int64_t t = 0; t < n_tokens; ++t) {
+        const float* row = logits + t * n_experts;
+        const int32_t* sel = ids + t * top_k;
+        float* w = weights + t * top_k;
+        float mx = -INFINITY;
+        for (int k = 0; k < top_k; ++k)
+            if (sel[k] >= 0 && sel[k] < n_experts && row[sel[k]] > mx) mx = row[sel[k]];
+        if (!isfinite(mx)) mx = 0.0f;
+        float den = 0.0f;
+        for (int k = 0; k < top_k; ++k) {
+            float v = 0.0f;
+            if (sel[k] >= 0 && sel[k] < n_experts) {
+                v = expf(row[sel[k]] - mx);
+                den += v;
+            }
+            w[k] = v;
+        }
+        if (den < 6.103515625e-5f) den = 6.103515625e-5f;
+        for (int k = 0; k < top_k; ++k) w[k] /= den;
+    }
+    return 0;
+}
+
 static int cmp_assignment(const void* pa, const void* pb) {
     const orc_assignment* a = (const orc_assignment*)pa;
     const orc_assignment* b = (const orc_assignment*)pb;

@@ -131,6 +131,10 @@ int orc_ffn_swiglu_q4k(const void* gate, const void* up, const void* down, int64
  * 1 = multi-token variant with the 6.1035e-5 floor (native.cpp:2305-2357). */
 int orc_route_topk(const float* logits, int64_t n_experts, int64_t n_tokens, int top_k, int weights_mode,
                    int32_t* ids, float* weights);
+/* Weights of given ids from raw logits (core/src/llm/moe/native.cpp:2305-2357): softmax over the valid
+ * selected logits, max replaced by 0 when not finite, denominator floored at 2^-14, invalid ids -> 0. */
+int orc_route_weights_from_ids(const float* logits, int64_t n_experts, int64_t n_tokens, const int32_t* ids, int top_k,
+                               float* weights);
 
 typedef struct {
     int32_t expert;

@@ -10,8 +10,8 @@ from densecore_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "mi355_q4k.h")).read()
+def declared_symbols(header="mi355_q4k.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mq_[a-z0-9_]+)\s*\(", text)))
 
@@ -24,6 +24,20 @@ def test_library_exports_every_declared_symbol():
     L = _lib.load()
     for name in declared_symbols():
         assert hasattr(L, name), name
+
+
+def test_ggml_adapter_library_exports_every_declared_symbol():
+    import ctypes
+
+    from densecore_amd import ggml_adapter
+    _lib.load()
+    L = ctypes.CDLL(ggml_adapter.LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    declared = declared_symbols("mi355_q4k_ggml.h")
+    assert declared == sorted(ggml_adapter.EXPORTS)
+    for name in declared:
+        assert hasattr(L, name), name
+    # the ctypes mirror must have ggml's layout: data at 248, name at 256, 336 bytes in all
+    assert ggml_adapter.GgmlTensor.data.offset == 248 and ctypes.sizeof(ggml_adapter.GgmlTensor) == 336
 
 
 @pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="a GPU is present")

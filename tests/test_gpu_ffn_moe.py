@@ -247,3 +247,19 @@ def test_moe_layer_zero_weight_and_duplicate_free_paths(ops):
     assert np.max(np.abs(y.cpu().numpy() - ref["y"])) <= END_TO_END_REL * np.max(np.abs(ref["y"]))
     for t in (GE, UE, DE):
         t.free()
+
+
+@pytest.mark.parametrize("n", [1, 37])
+def test_weights_from_logits_match_oracle(ops, n):
+    import torch
+    """mq_moe_weights_from_logits vs orc_route_weights_from_ids, incl. invalid ids and an all-(-inf) row."""
+    rng = np.random.default_rng(5 + n)
+    logits = rng.normal(size=(n, 256)).astype(np.float32)
+    ids = np.stack([rng.permutation(256)[:8] for _ in range(n)]).astype(np.int32)
+    ids[0, 2] = -1
+    ids[n - 1, 7] = 256
+    logits[0, ids[0, 0]] = -np.inf
+    got = ops.moe_weights_from_logits(torch.from_numpy(logits).cuda(), torch.from_numpy(ids).cuda()).cpu().numpy()
+    ref = orc.route_weights_from_ids(logits, ids)
+    np.testing.assert_allclose(got, ref, rtol=3e-7, atol=0)  # expf differs from the host's by at most an ulp
+    assert got[0, 2] == 0 and got[n - 1, 7] == 0 and got[0, 0] == 0

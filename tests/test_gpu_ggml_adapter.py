@@ -1,0 +1,120 @@
+"""The GGML_OP_CUSTOM adapters, driven as a ggml CPU graph would drive them (host tensors, strides,
+ith/nth), checked against the oracle.  Mirrors the callback-level tests of the reference
+(core/tests/... inference_test_hooks.inl:177-256: batched callback vs the reference dot <= 1e-4)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from densecore_amd import synth
+from oracle import binding as orc
+from tests._parity import assert_fp32_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ga():
+    from densecore_amd import ggml_adapter
+    ggml_adapter.lib()
+    yield ggml_adapter
+    ggml_adapter.lib().mq_ggml_weight_cache_clear()
+
+
+def _dense_ref(w, cols, x):
+    return orc.mul_mat_q4k_q8k(w, cols, orc.quantize_rows_q8k(x), orc.ORDER_AVX2)
+
+
+@pytest.mark.parametrize("m,pad", [(1, 0), (5, 0), (3, 64)])
+def test_dense_node(ga, m, pad):
+    rows, cols = 512, 1024
+    w = synth.q4k_matrix(101, rows, cols)
+    xbuf = np.zeros((m, cols + pad), np.float32)
+    xbuf[:, :cols] = synth.normal_f32(102, (m, cols))
+    ybuf = np.full((m, rows + pad), 7.0, np.float32)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q4_K, [cols, rows], name=b"blk.0.ffn_gate.weight")
+    tx = ga.tensor(xbuf, ga.GGML_TYPE_F32, [cols, m], nb=[4, 4 * (cols + pad)])
+    ty = ga.tensor(ybuf, ga.GGML_TYPE_F32, [rows, m], nb=[4, 4 * (rows + pad)])
+    ga.set_src(ty, tx, tw)
+    fn = ga.lib().mq_cb_gemv_custom if m == 1 else ga.lib().mq_cb_gemv_batched_custom
+    fn(C.byref(ty), 1, 4, None)  # a worker other than 0 does nothing
+    assert np.all(ybuf == 7.0)
+    fn(C.byref(ty), 0, 4, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    x = np.ascontiguousarray(xbuf[:, :cols])
+    ref = _dense_ref(w, cols, x)
+    mag = orc.dot_magnitude_f64(w, cols, orc.quantize_rows_q8k(x))
+    assert_fp32_parity(ybuf[:, :rows], ref, mag)
+    assert np.all(ybuf[:, rows:] == 7.0)  # padding of a strided dst is not written
+    before = ga.lib().mq_ggml_weight_cache_size()
+    fn(C.byref(ty), 0, 4, None)  # second call reuses the uploaded weight
+    assert ga.lib().mq_ggml_weight_cache_size() == before
+
+
+def test_dense_node_rejects_mismatch(ga):
+    rows, cols = 256, 512
+    w = synth.q4k_matrix(111, rows, cols)
+    x = synth.normal_f32(112, (1, cols))
+    y = np.full((1, rows + 16), 3.0, np.float32)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q4_K, [cols, rows])
+    tx = ga.tensor(x, ga.GGML_TYPE_F32, [cols, 1])
+    ty = ga.tensor(y, ga.GGML_TYPE_F32, [rows + 16, 1])  # dst->ne[0] != weight->ne[1]
+    ga.set_src(ty, tx, tw)
+    ud = ga.UserData(0, 0, 1, 0)
+    ga.lib().mq_cb_gemv_custom(C.byref(ty), 0, 1, C.byref(ud))
+    assert ud.last_status != 0 and np.all(y == 3.0)
+    tf = ga.tensor(np.zeros((rows, cols), np.float32), ga.GGML_TYPE_F32, [cols, rows])  # F32 weight: not this path
+    ty2 = ga.tensor(np.full((1, rows), 3.0, np.float32), ga.GGML_TYPE_F32, [rows, 1])
+    ga.set_src(ty2, tx, tf)
+    ga.lib().mq_cb_gemv_custom(C.byref(ty2), 0, 1, C.byref(ud))
+    assert ud.last_status != 0 and np.all(ty2._keep == 3.0)
+
+
+@pytest.mark.parametrize("n", [1, 6])
+def test_moe_nodes(ga, n):
+    hidden, inter, n_exp, top_k = 512, 256, 8, 2
+    gate = np.stack([synth.q4k_matrix(2010 + e, inter, hidden) for e in range(n_exp)])
+    up = np.stack([synth.q4k_matrix(2020 + e, inter, hidden) for e in range(n_exp)])
+    down = np.stack([synth.q4k_matrix(2030 + e, hidden, inter) for e in range(n_exp)])
+    x = synth.normal_f32(204, (n, hidden))
+    logits = synth.normal_f32(205, (n, n_exp))
+    ids, _ = orc.route_topk(logits, top_k, 1)
+    silu = orc.SILU_EXACT if n <= 4 else orc.SILU_FAST
+    # gate/up node
+    hid = np.zeros((n, top_k, inter), np.float32)
+    tg = ga.tensor(gate, ga.GGML_TYPE_Q4_K, [hidden, inter, n_exp])
+    tu = ga.tensor(up, ga.GGML_TYPE_Q4_K, [hidden, inter, n_exp])
+    tx = ga.tensor(x, ga.GGML_TYPE_F32, [hidden, n])
+    ts = ga.tensor(ids, ga.GGML_TYPE_I32, [top_k, n])
+    th = ga.tensor(hid, ga.GGML_TYPE_F32, [inter, top_k, n])
+    ga.set_src(th, tg, tu, tx, ts)
+    ga.lib().mq_cb_moe_gateup_swiglu(C.byref(th), 0, 8, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    ref_hid = orc.moe_gateup_swiglu(gate, up, hidden, inter, x, ids, orc.ORDER_AVX2, silu)
+    np.testing.assert_allclose(hid, ref_hid, rtol=2e-4, atol=2e-4 * np.abs(ref_hid).max())
+    # down node, fed the oracle's hidden so that the stage is checked on identical inputs
+    y = np.zeros((n, hidden), np.float32)
+    td = ga.tensor(down, ga.GGML_TYPE_Q4_K, [inter, hidden, n_exp])
+    th2 = ga.tensor(ref_hid, ga.GGML_TYPE_F32, [inter, top_k, n])
+    tl = ga.tensor(logits, ga.GGML_TYPE_F32, [n_exp, n])
+    ty = ga.tensor(y, ga.GGML_TYPE_F32, [hidden, n])
+    ga.set_src(ty, td, th2, ts, tl)
+    ga.lib().mq_cb_moe_down_weighted_logits(C.byref(ty), 0, 8, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    w_ref = orc.route_weights_from_ids(logits, ids)
+    ref_y = orc.moe_down_weighted(down, hidden, inter, ref_hid, ids, w_ref, orc.ORDER_AVX2, 0)
+    np.testing.assert_allclose(y, ref_y, rtol=2e-4, atol=2e-4 * np.abs(ref_y).max())
+
+
+def test_library_level_matmul(ga):
+    m, rows, cols = 7, 384, 768
+    w = synth.q4k_matrix(301, rows, cols)
+    a = synth.normal_f32(302, (m, cols))
+    c = np.zeros((m, rows), np.float32)
+    ok = ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, ga.GGML_TYPE_Q4_K, rows,
+                                                  cols, 144 * (cols // 256), c.ctypes.data, rows)
+    assert ok == 1
+    assert_fp32_parity(c, _dense_ref(w, cols, a), orc.dot_magnitude_f64(w, cols, orc.quantize_rows_q8k(a)))
+    # a type other than Q4_K is rejected like an unsupported ggml type
+    assert ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, 2, rows, cols,
+                                                    144 * (cols // 256), c.ctypes.data, rows) == 0

@@ -409,3 +409,27 @@ def test_ffn_against_double_brute_force():
     assert np.allclose(mid, h, rtol=2e-4, atol=1e-5 * np.abs(h).max())
     want = np_q8_dequant(mid) @ np_dequant(d, I).T
     assert np.max(np.abs(y - want)) < 1e-5 * np.abs(want).max()
+
+
+def test_weights_from_ids_agree_with_router_and_double_softmax():
+    """orc_route_weights_from_ids: on the router's own selection it must reproduce the router's FLOOR-mode
+    weights bit for bit (two restatements of one formula in the reference, native.cpp:822-866 vs :2305-2357,
+    on finite logits) and equal a double-precision softmax restricted to the selected set; invalid ids weigh 0."""
+    rng = np.random.default_rng(77)
+    logits = rng.normal(size=(33, 64)).astype(np.float32)
+    ids, w_router = orc.route_topk(logits, 8, 1)
+    w = orc.route_weights_from_ids(logits, ids)
+    assert np.array_equal(w, w_router)
+    sel = np.take_along_axis(logits.astype(np.float64), ids.astype(np.int64), axis=1)
+    ref = np.exp(sel - sel.max(axis=1, keepdims=True))
+    ref /= ref.sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(w, ref, rtol=2e-6)
+    bad = ids.copy()
+    bad[:, 3] = -1
+    bad[:, 5] = 64
+    wb = orc.route_weights_from_ids(logits, bad)
+    assert np.all(wb[:, 3] == 0) and np.all(wb[:, 5] == 0)
+    np.testing.assert_allclose(wb.sum(axis=1), 1.0, rtol=1e-6)
+    # arbitrary (unsorted) ids: any permutation of the selection gives the permuted weights up to summation order
+    perm = rng.permutation(8)
+    np.testing.assert_allclose(orc.route_weights_from_ids(logits, ids[:, perm]), w[:, perm], rtol=1e-6)
