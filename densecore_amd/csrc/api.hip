@@ -77,6 +77,7 @@ struct State {
     int device = -1;
     std::mutex mu;
     Buffer aq, ad;        // A-major activations of the op input
+    Buffer ap;            // P-major activations of the prefill GEMM
     Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
     Buffer aq2, ad2;      // A-major activations of the intermediate
     Buffer part;          // MoE per-(token,k) down results
@@ -334,6 +335,29 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
     return MQ_OK;
 }
 
+// Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk.
+constexpr int64_t kPrefillMinRows = 48;
+
+static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                       hipStream_t s) {
+    if (n == 0) return MQ_OK;
+    MQ_HIP(g.ap.reserve(pmajor_bytes(n, w->nb)));
+    MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, w->cols, (uint8_t*)g.ap.ptr, s));
+    MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy, s));
+    return MQ_OK;
+}
+
+int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_gemm_q4k")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: weight is an expert stack");
+    if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
+    if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");
+    std::lock_guard<std::mutex> lock(g.mu);
+    return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, (hipStream_t)stream);
+}
+
 int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                    void* stream) {
     if (int rc = check_ready()) return rc;
@@ -343,6 +367,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    if (n >= kPrefillMinRows) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }

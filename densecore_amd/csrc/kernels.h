@@ -68,6 +68,15 @@ struct MatmulArgs {
 };
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream);
 
+// ---- prefill.hip -----------------------------------------------------------------------------
+// fp32 rows -> Q8_K in the P-major layout of the prefill GEMM (pmajor_bytes(n, nb) bytes).
+size_t pmajor_bytes(int64_t n, int64_t nb);
+hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
+                                      hipStream_t stream);
+// y[n][ldy] = P-major activations . tiled weights^T on the int8 matrix cores.
+hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
+                               int64_t ldy, hipStream_t stream);
+
 // ---- router.hip ------------------------------------------------------------------------------
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                              float* weights, hipStream_t stream);

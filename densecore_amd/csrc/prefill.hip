@@ -1,0 +1,257 @@
+// Prefill GEMM for gfx950: C[M][N] = q8k(A[M][K]) . W_q4k[N][K]^T for M in the hundreds and above,
+// where the work is arithmetic on the int8 matrix cores rather than weight streaming
+// (RunQ4KRawBatchedDenseGemm, core/src/backend/cpu_backend_q4k_dense.cpp:57-101, behind
+// CpuBackend::MatMulGgmlQuantizedTransB, core/src/backend/cpu_backend_quantized_matmul.cpp:150-175).
+//
+// The per-sub-block 6-bit scales are what keeps Q4_K off a plain int8 GEMM.  Here they are folded
+// into the weight operand so that v_mfma_i32_16x16x64_i8 accumulates over the whole super-block:
+//     scale = 8*s1 + s0  (two 3-bit digits)   ->   (s1*q4) and (s0*q4) both fit a signed byte (<= 105)
+//     dot_scaled = 8 * sum_k (s1*q4)_k q8_k  +  sum_k (s0*q4)_k q8_k                  (exact, int32)
+// and the min term runs on the matrix cores as well, from the sub-block sums of the codes
+// bs_g = bsums[2g] + bsums[2g+1] = 128*h_g + l_g (h in [-32, 31], l in [0, 127], both bytes):
+//     min_dot = 128 * sum_g min_g h_g  +  sum_g min_g l_g                               (exact, int32)
+// which is the reference's sum_j bsums[j] * min[j/2] (core/src/llm/matmul/kquant_batched_kernels.h:285-297).
+// Ten MFMAs per 16x16 output tile and super-block, no per-sub-block vector work; the fp32 update
+//     acc += (d*yd) * dot_scaled - (dmin*yd) * min_dot
+// is done once per super-block, as every reference kernel does.
+//
+//   grid      = (ceil(rowtiles / 8), ceil(m_tiles / 8)); workgroup = 4 wavefronts
+//   workgroup = 128 weight rows x 128 activation rows; per super-block it stages the 128 activation
+//               rows (35 KB in the P-major layout below) in LDS
+//   wavefront = 2 weight tiles (32 rows) x the 8 activation tiles; it reads its weight tiles
+//               straight from HBM in MFMA lane order and expands them in registers
+//
+// P-major activations (written by quantize_q8k_pmajor_kernel): [b][mt][4416 B], mt = m / 16:
+//   [j 0..3][kq 0..3][tok 0..15][16 B]   codes: bytes 0..7 = sub-block ga(j), elements 8kq..8kq+7,
+//                                        bytes 8..15 = sub-block gb(j), same elements, with
+//                                        (ga, gb) = (0,2) (1,3) (4,6) (5,7) for j = 0..3 -- the pairs
+//                                        that one 16-byte word of a weight tile holds per nibble half
+//   [tok][16 B] at 4096                  l_0..l_7, h_0..h_7
+//   [tok] fp32 at 4352                   block scale d
+#include "common.h"
+#include "kernels.h"
+#include "q8k_block.h"
+
+namespace mq {
+
+namespace {
+
+constexpr int kPTileBytes = 4416;
+constexpr int kPTileWords = kPTileBytes / 16;  // 276
+constexpr int kMTilesPerGroup = 8;             // activation tiles (of 16 rows) per workgroup
+constexpr int kWTilesPerWave = 2;
+
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+
+// four bytes (each <= 15) times a 3-bit digit, bytewise; the digit comes replicated in both halves
+__device__ __forceinline__ uint32_t scale_bytes(uint32_t nibbles, uint32_t digit_pk) {
+    const v2us a = __builtin_bit_cast(v2us, nibbles);
+    const v2us d = __builtin_bit_cast(v2us, digit_pk);
+    return __builtin_bit_cast(uint32_t, (v2us)(a * d));
+}
+
+// byte `i` of `word` replicated into bits 0..7 and 16..23
+__device__ __forceinline__ uint32_t digit_pair(uint32_t word, int i) {
+    const uint32_t v = (word >> (8 * i)) & 0xffu;
+    return v | (v << 16);
+}
+
+struct WTile {
+    v4i hi[4], lo[4];  // B operands of the four chunk pairs, scaled by the high / low scale digit
+    v4i mins;          // B operand of the min MFMAs (k-group 0 only)
+    float d, dmin;
+};
+
+__device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, const v4u hdr, int kq, WTile& t) {
+    // 6-bit scales and mins (core/src/kernels/hwy/hwy_moe_quant.cc:90-101), four to a word
+    const uint32_t sc03 = hdr.y & 0x3f3f3f3fu, mn03 = hdr.z & 0x3f3f3f3fu;
+    const uint32_t sc47 = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+    const uint32_t mn47 = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+    const uint32_t s1_03 = (sc03 >> 3) & 0x07070707u, s0_03 = sc03 & 0x07070707u;
+    const uint32_t s1_47 = (sc47 >> 3) & 0x07070707u, s0_47 = sc47 & 0x07070707u;
+    const v4u seg[2] = {seg0, seg1};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t s1w = i ? s1_47 : s1_03, s0w = i ? s0_47 : s0_03;
+        // sub-blocks 4i .. 4i+3 are bytes 0..3 of the digit words
+        const uint32_t l0 = seg[i].x & 0x0f0f0f0fu, l1 = seg[i].y & 0x0f0f0f0fu;  // sub-block 4i
+        const uint32_t l2 = seg[i].z & 0x0f0f0f0fu, l3 = seg[i].w & 0x0f0f0f0fu;  // sub-block 4i+2
+        const uint32_t h0 = (seg[i].x >> 4) & 0x0f0f0f0fu, h1 = (seg[i].y >> 4) & 0x0f0f0f0fu;  // 4i+1
+        const uint32_t h2 = (seg[i].z >> 4) & 0x0f0f0f0fu, h3 = (seg[i].w >> 4) & 0x0f0f0f0fu;  // 4i+3
+        const uint32_t a1 = digit_pair(s1w, 0), a0 = digit_pair(s0w, 0);
+        const uint32_t b1 = digit_pair(s1w, 1), b0 = digit_pair(s0w, 1);
+        const uint32_t c1 = digit_pair(s1w, 2), c0 = digit_pair(s0w, 2);
+        const uint32_t e1 = digit_pair(s1w, 3), e0 = digit_pair(s0w, 3);
+        t.hi[2 * i] = v4i{(int)scale_bytes(l0, a1), (int)scale_bytes(l1, a1), (int)scale_bytes(l2, c1),
+                          (int)scale_bytes(l3, c1)};
+        t.lo[2 * i] = v4i{(int)scale_bytes(l0, a0), (int)scale_bytes(l1, a0), (int)scale_bytes(l2, c0),
+                          (int)scale_bytes(l3, c0)};
+        t.hi[2 * i + 1] = v4i{(int)scale_bytes(h0, b1), (int)scale_bytes(h1, b1), (int)scale_bytes(h2, e1),
+                              (int)scale_bytes(h3, e1)};
+        t.lo[2 * i + 1] = v4i{(int)scale_bytes(h0, b0), (int)scale_bytes(h1, b0), (int)scale_bytes(h2, e0),
+                              (int)scale_bytes(h3, e0)};
+    }
+    t.mins = kq == 0 ? v4i{(int)mn03, (int)mn47, 0, 0} : v4i{0, 0, 0, 0};
+    t.d = half_bits_to_float(hdr.x & 0xffffu);
+    t.dmin = half_bits_to_float(hdr.x >> 16);
+}
+
+__global__ void __launch_bounds__(256) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
+                                                           int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
+                                                           int64_t n_tokens, float* __restrict__ y, int64_t ldy) {
+    extern __shared__ __align__(16) uint8_t a_lds[];  // kMTilesPerGroup * 4416 bytes
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, kq = lane >> 4;
+    const int64_t mt0 = (int64_t)blockIdx.y * kMTilesPerGroup;
+    const int mt_count = (int)(m_tiles - mt0 < kMTilesPerGroup ? m_tiles - mt0 : kMTilesPerGroup);
+    const int64_t rt0 = ((int64_t)blockIdx.x * 4 + wave) * kWTilesPerWave;
+    // weight tiles past the end are replaced by the last valid one and simply not stored
+    int64_t rt[kWTilesPerWave];
+#pragma unroll
+    for (int t = 0; t < kWTilesPerWave; ++t) rt[t] = rt0 + t < rowtiles ? rt0 + t : rowtiles - 1;
+
+    float acc[kWTilesPerWave][kMTilesPerGroup][4];
+#pragma unroll
+    for (int t = 0; t < kWTilesPerWave; ++t)
+#pragma unroll
+        for (int m = 0; m < kMTilesPerGroup; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][m][i] = 0.0f;
+
+    const int copy_words = mt_count * kPTileWords;
+    for (int64_t b = 0; b < nb; ++b) {
+        // this wave's weight tiles, requested first so that they travel during the LDS staging
+        v4u seg0[kWTilesPerWave], seg1[kWTilesPerWave], hdr[kWTilesPerWave];
+#pragma unroll
+        for (int t = 0; t < kWTilesPerWave; ++t) {
+            const uint8_t* tile = w + tile_offset(rt[t], b, nb);
+            seg0[t] = load16(tile + lane * 16);
+            seg1[t] = load16(tile + 1024 + lane * 16);
+            hdr[t] = load16(tile + kTileQBytes + r * 16);
+        }
+        __syncthreads();  // every wave is done reading the previous super-block's activations
+        const uint8_t* src = ap + ((size_t)b * (size_t)m_tiles + (size_t)mt0) * kPTileBytes;
+        for (int i = tid; i < copy_words; i += 256)
+            *reinterpret_cast<v4u*>(a_lds + (size_t)i * 16) = load16(src + (size_t)i * 16);
+        WTile wt[kWTilesPerWave];
+#pragma unroll
+        for (int t = 0; t < kWTilesPerWave; ++t) expand_tile(seg0[t], seg1[t], hdr[t], kq, wt[t]);
+        __syncthreads();
+
+#pragma unroll
+        for (int m = 0; m < kMTilesPerGroup; ++m) {
+            if (m < mt_count) {  // uniform over the workgroup
+                const uint8_t* at = a_lds + m * kPTileBytes;
+                v4i a[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
+                const v4i dg = *reinterpret_cast<const v4i*>(at + 4096 + r * 16);
+                const float4 yd = *reinterpret_cast<const float4*>(at + 4352 + kq * 16);
+                const v4i a_l = kq == 0 ? v4i{dg.x, dg.y, 0, 0} : v4i{0, 0, 0, 0};
+                const v4i a_h = kq == 0 ? v4i{dg.z, dg.w, 0, 0} : v4i{0, 0, 0, 0};
+                const v4i zero = {0, 0, 0, 0};
+                v4i hi[kWTilesPerWave], lo[kWTilesPerWave], mh[kWTilesPerWave], ml[kWTilesPerWave];
+#pragma unroll
+                for (int t = 0; t < kWTilesPerWave; ++t) {
+                    hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].hi[0], zero, 0, 0, 0);
+                    lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].lo[0], zero, 0, 0, 0);
+                    mh[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_h, wt[t].mins, zero, 0, 0, 0);
+                    ml[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_l, wt[t].mins, zero, 0, 0, 0);
+                }
+#pragma unroll
+                for (int j = 1; j < 4; ++j)
+#pragma unroll
+                    for (int t = 0; t < kWTilesPerWave; ++t) {
+                        hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].hi[j], hi[t], 0, 0, 0);
+                        lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].lo[j], lo[t], 0, 0, 0);
+                    }
+                const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+#pragma unroll
+                for (int t = 0; t < kWTilesPerWave; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int dot = hi[t][i] * 8 + lo[t][i];
+                        const int mnd = mh[t][i] * 128 + ml[t][i];
+                        const float s = __fmul_rn(wt[t].d, ydv[i]);
+                        const float ms = __fmul_rn(wt[t].dmin, ydv[i]);
+                        float v = __fmaf_rn(s, (float)dot, acc[t][m][i]);
+                        acc[t][m][i] = __fmaf_rn(-ms, (float)mnd, v);
+                    }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < kWTilesPerWave; ++t) {
+        const int64_t row = (rt0 + t) * kTileRows + r;
+        if (rt0 + t >= rowtiles || row >= rows) continue;
+#pragma unroll
+        for (int m = 0; m < kMTilesPerGroup; ++m) {
+            if (m >= mt_count) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t tok = (mt0 + m) * 16 + kq * 4 + i;
+                if (tok < n_tokens) y[tok * ldy + row] = acc[t][m][i];
+            }
+        }
+    }
+}
+
+// One wavefront per (activation row, super-block); rows in [n, 16*m_tiles) are written as zeros.
+__global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* __restrict__ x, int64_t n, int64_t ldx,
+                                                                  int64_t nb, int64_t m_tiles,
+                                                                  uint8_t* __restrict__ ap) {
+    const int lane = threadIdx.x & 63;
+    const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (unit >= m_tiles * 16 * nb) return;
+    const int64_t m = unit / nb;
+    const int64_t b = unit - m * nb;
+    float e[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (m < n) {
+        const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
+        e[0] = v.x, e[1] = v.y, e[2] = v.z, e[3] = v.w;
+    }
+    const Q8Lane q = quantize_block_q8k(e, lane);
+    uint8_t* tile = ap + ((size_t)b * (size_t)m_tiles + (size_t)(m >> 4)) * kPTileBytes;
+    const int tok = (int)(m & 15);
+    // elements 4*lane..4*lane+3: sub-block g = lane/8, elements 4*(lane%8).. of it
+    const int g = lane >> 3;
+    const int j = 2 * (g >> 2) + (g & 1), half = (g >> 1) & 1;
+    const int kq = (lane & 7) >> 1;
+    *reinterpret_cast<uint32_t*>(tile + j * 1024 + (kq * 16 + tok) * 16 + half * 8 + (lane & 1) * 4) = q.packed;
+    const int bs = q.bsum + __shfl_xor(q.bsum, 4, 64);  // codes 32g .. 32g+31
+    if ((lane & 7) == 0) {
+        tile[4096 + tok * 16 + g] = (uint8_t)(bs & 127);
+        tile[4096 + tok * 16 + 8 + g] = (uint8_t)(bs >> 7);
+    }
+    if (lane == 0) *reinterpret_cast<float*>(tile + 4352 + tok * 4) = q.d;
+}
+
+}  // namespace
+
+size_t pmajor_bytes(int64_t n, int64_t nb) { return (size_t)((n + 15) / 16) * (size_t)nb * kPTileBytes; }
+
+hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
+                                      hipStream_t stream) {
+    const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
+    const int64_t units = m_tiles * 16 * nb;
+    if (units == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx,
+                       nb, m_tiles, ap);
+    return hipGetLastError();
+}
+
+hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
+                               int64_t ldy, hipStream_t stream) {
+    const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
+    if (rowtiles == 0 || m_tiles == 0) return hipSuccess;
+    const dim3 grid((unsigned)((rowtiles + 4 * kWTilesPerWave - 1) / (4 * kWTilesPerWave)),
+                    (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup));
+    if (grid.y > 65535u) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(prefill_gemm_kernel, grid, dim3(256), kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+                       ap, m_tiles, n, y, ldy);
+    return hipGetLastError();
+}
+
+}  // namespace mq

@@ -106,6 +106,16 @@ def mul_mat(w: Q4KWeight, x: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def gemm(w: Q4KWeight, x: torch.Tensor) -> torch.Tensor:
+    """The same product through the int8 matrix-core GEMM kernel at any n (RunQ4KRawBatchedDenseGemm,
+    core/src/backend/cpu_backend_q4k_dense.cpp:57-101)."""
+    x = _f32(x)
+    n = x.shape[0]
+    y = torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().mq_gemm_q4k(w._h, _ptr(x), n, x.stride(0), _ptr(y), w.rows, _stream()), "mq_gemm_q4k")
+    return y
+
+
 def mul_mat_q8k(w: Q4KWeight, q8: torch.Tensor) -> torch.Tensor:
     """RunMoEQ4KRawBatchedProjectionImpl (core/src/backend/cpu_backend_moe_raw_batched.inl:1352): Q8_K rows in."""
     n = q8.shape[0]

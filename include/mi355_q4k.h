@@ -89,6 +89,14 @@ int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void*
  * (core/include/densecore/backend/cpu_backend.h:293-300, any n). */
 int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                    void* stream);
+/* The same product computed by the matrix-core GEMM kernel whatever n is (mq_mul_mat_q4k switches to it
+ * by itself from a few dozen rows up): weights are read once per 128 activation rows and the int8 MFMA
+ * units do the arithmetic.  RunQ4KRawBatchedDenseGemm (core/src/backend/cpu_backend_q4k_dense.cpp:57-101),
+ * the A.shape[0] >= 4 branch of MatMulGgmlQuantizedTransBWithPath
+ * (core/src/backend/cpu_backend_quantized_matmul.cpp:164-170).  Same integers per super-block as
+ * mq_mul_mat_q4k; the fp32 update uses fused multiply-adds, so results agree to rounding, not bitwise. */
+int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                void* stream);
 /* Same with already-quantized activations: q8_dev [n][q8_row_bytes] block_q8_K rows
  * (RunMoEQ4KRawBatchedProjectionImpl, core/src/backend/cpu_backend_moe_raw_batched.inl:1352). */
 int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t q8_row_bytes, float* y_dev,

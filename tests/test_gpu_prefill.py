@@ -1,0 +1,127 @@
+"""The matrix-core prefill GEMM (mq_gemm_q4k) against the oracle and against the decode kernel.
+
+Reference counterpart: RunQ4KRawBatchedDenseGemm behind MatMulGgmlQuantizedTransB
+(core/src/backend/cpu_backend_q4k_dense.cpp:57-101); its own test compares with the dequantized
+double-precision dot at 1e-4 (core/tests/test_moe_ops.cpp:170-201,428-430), as assert_fp32_parity does."""
+import numpy as np
+import pytest
+
+from densecore_amd import synth
+from oracle import binding as orc
+from tests._parity import assert_fp32_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    from densecore_amd import ops as o
+    assert torch.cuda.is_available()
+    return o
+
+
+def cu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("n", [1, 5, 16, 17, 130, 200])
+@pytest.mark.parametrize("rows,cols", [(48, 256), (272, 1024), (40, 512)])
+def test_gemm_matches_oracle(ops, n, rows, cols):
+    w = synth.q4k_matrix(synth.tensor_seed("pf-w", rows, cols), rows, cols)
+    x = synth.normal_f32(synth.tensor_seed("pf-x", n, cols), (n, cols))
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    mag = orc.dot_magnitude_f64(w, cols, q8)
+    for name, order in orc.ORDERS.items():
+        assert_fp32_parity(got, orc.mul_mat_q4k_q8k(w, cols, q8, order), mag, f"order={name}")
+    assert_fp32_parity(got, orc.dot_dequant_f64(w, cols, q8), mag, "dequantized double")
+    W.free()
+
+
+def test_gemm_extreme_codes_do_not_overflow_the_byte_digits(ops):
+    """All nibbles 15, scales and mins 63, activations +-max: the largest (s1*q4) and (s0*q4) bytes
+    (105), the largest sub-block code sums (+-4064 -> digits h = +-32, l = 0..127) and the largest
+    int32 sums of a super-block."""
+    rows, cols, n = 32, 512, 40
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.float16(0.005).tobytes(), np.uint8)
+    blk[4:16] = 0xFF
+    blk[16:] = 0xFF
+    w = np.tile(blk, (rows, cols // 256))
+    x = np.ones((n, cols), np.float32)
+    x[1::2] *= -1.0            # every code -127 / +127
+    x[2, ::2] *= -1.0          # alternating signs: sub-block sums of 0
+    x[3, :300] = 0.0
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    ref = orc.mul_mat_q4k_q8k(w, cols, q8, orc.ORDER_SCALAR)
+    assert_fp32_parity(got, ref, orc.dot_magnitude_f64(w, cols, q8), "extremes")
+    W.free()
+
+
+@pytest.mark.parametrize("n", [3, 64, 150])
+def test_gemm_integer_sums_are_exact(ops, n):
+    """With d = dmin = 1 and integer activations whose largest magnitude per block is 127, the Q8_K codes
+    are the activations themselves (scale +-1) and every fp32 operation of the kernel is exact, so the
+    output must EQUAL sum_b yd_b * (dot_scaled_b - min_dot_b) built from the oracle's integers: a single
+    wrong unit in either integer sum of any super-block shows up."""
+    rows, cols = 80, 768
+    nb = cols // 256
+    w = synth.q4k_matrix(synth.tensor_seed("pf-int", rows), rows, cols).reshape(rows, nb, 144).copy()
+    w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[:, :, 2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w = w.reshape(rows, nb * 144)
+    rng = np.random.default_rng(n)
+    x = rng.integers(-127, 128, size=(n, cols)).astype(np.float32)
+    x.reshape(n, nb, 256)[:, :, 7] = rng.choice([-127.0, 127.0], size=(n, nb))
+    q8 = orc.quantize_rows_q8k(x)
+    d, qs, _ = orc.split_q8k(q8)
+    assert np.all(np.abs(d) == 1.0) and np.array_equal(qs.reshape(n, cols) * d.repeat(256, axis=1), x)
+    ds, md = orc.matrix_block_sums(w, cols, q8)            # [rows, n, nb]
+    want = ((ds.astype(np.int64) - md.astype(np.int64)) * d.astype(np.int64)[None]).sum(axis=2).T
+    assert np.abs(want).max() < 2 ** 24
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, want.astype(np.float32))
+    W.free()
+
+
+def test_gemm_agrees_with_decode_kernel_and_dispatch(ops):
+    import torch
+    rows, cols, n = 512, 2048, 96
+    W = ops.Q4KWeight.synthetic(77, rows, cols)
+    x = cu(synth.normal_f32(78, (n, cols)))
+    big = ops.gemm(W, x)
+    assert torch.equal(ops.mul_mat(W, x), big)          # n >= 48 is routed to the GEMM kernel
+    small = torch.cat([ops.mul_mat(W, x[i:i + 16]) for i in range(0, n, 16)])
+    scale = small.abs().max().item()
+    assert (big - small).abs().max().item() <= 1e-5 * scale   # same integers, fp32 rounding only
+    # strided input rows and a padded output are honoured
+    xp = torch.zeros((n, cols + 256), device="cuda")
+    xp[:, :cols] = x
+    assert torch.equal(ops.gemm(W, xp[:, :cols]), big)
+    W.free()
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+def test_gemm_full_size_rows_against_decode_kernel(ops, m):
+    """W 4096 -> 14336 at M = 512 / 2048: every 37th activation row is recomputed by the decode kernel,
+    whose integer sums are pinned bit-exactly elsewhere; plus linearity in the activations' sign."""
+    import torch
+    rows, cols = 14336, 4096
+    W = ops.Q4KWeight.synthetic(4, rows, cols)
+    g = torch.Generator(device="cuda").manual_seed(m)
+    x = torch.randn((m, cols), device="cuda", generator=g)
+    y = ops.gemm(W, x)
+    pick = torch.arange(0, m, 37, device="cuda")
+    ref = torch.cat([ops.mul_mat(W, x[pick[i:i + 16]]) for i in range(0, len(pick), 16)])
+    scale = ref.abs().max().item()
+    assert (y[pick] - ref).abs().max().item() <= 1e-5 * scale
+    # Q8_K quantization is odd (codes and scale flip sign together), so the product is too, exactly
+    assert torch.equal(ops.gemm(W, -x), -y)
+    W.free()
