@@ -526,6 +526,24 @@ int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int
     return MQ_OK;
 }
 
+int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                       float eps, float* sum_out_dev, float* normed_out_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!x_dev || !normed_out_dev || n < 0 || cols <= 0) return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_f32: bad arguments");
+    MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_router_logits_f32(const float* w_dev, int64_t n_experts, int64_t cols, const float* x_dev, int64_t n, int64_t ldx,
+                         float* logits_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!w_dev || !x_dev || !logits_dev || n < 0 || n > 65535 || n_experts <= 0 || cols <= 0 || (cols & 255) || ldx < cols ||
+        (ldx & 3) || (reinterpret_cast<uintptr_t>(x_dev) & 15u) || (reinterpret_cast<uintptr_t>(w_dev) & 15u))
+        return fail(MQ_ERR_INVALID, "mq_router_logits_f32: need cols %% 256 == 0, 16-byte aligned rows, n <= 65535");
+    MQ_HIP(launch_router_logits(w_dev, n_experts, cols, x_dev, n, ldx, logits_dev, (hipStream_t)stream));
+    return MQ_OK;
+}
+
 int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev, int top_k,
                                float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;

@@ -1,0 +1,86 @@
+// The two small fp32 operators that sit between the quantized matmuls of a decoder layer: the
+// fused residual add + RMSNorm that feeds every projection, and the F32 router projection that
+// produces the MoE logits.  Both are bandwidth-trivial; they exist so that a decode step stays on
+// the device between the Q4_K kernels.
+#include "common.h"
+#include "kernels.h"
+
+namespace mq {
+
+namespace {
+
+// sum[t] = x[t] + delta[t] (delta may be null); normed[t] = sum[t] * (rsqrt(mean(sum^2) + eps) * weight)
+// AddRMSNorm (core/src/kernels/hwy/hwy_normalization.cc:102-153; plain form in
+// core/tests/kernels/test_normalization.cpp:57-68).  One workgroup per token; the squares are
+// summed per thread in column order, then across lanes and waves in a fixed order.
+__global__ void __launch_bounds__(256) add_rmsnorm_kernel(const float* x, const float* __restrict__ delta,
+                                                          const float* __restrict__ weight, int64_t cols, float eps,
+                                                          float* sum_out,
+                                                          float* __restrict__ normed_out) {
+    __shared__ float wave_sum[4];
+    const int64_t base = (int64_t)blockIdx.x * cols;
+    float ssq = 0.0f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        const float v = delta ? __fadd_rn(x[base + c], delta[base + c]) : x[base + c];
+        if (sum_out) sum_out[base + c] = v;
+        ssq = __fmaf_rn(v, v, ssq);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = ssq;
+    __syncthreads();
+    const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+    const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        // sum_out may alias x: a thread re-reads what it stored itself rather than adding delta twice
+        const float v = sum_out ? sum_out[base + c] : (delta ? __fadd_rn(x[base + c], delta[base + c]) : x[base + c]);
+        const float sw = weight ? __fmul_rn(scale, weight[c]) : scale;
+        normed_out[base + c] = __fmul_rn(v, sw);
+    }
+}
+
+// logits[t][e] = w[e] . x[t], fp32 (the ffn_gate_inp projection, core/src/llm/graph/decoder.cpp:2265).
+// One wavefront per (expert, token): lanes stride the columns, fixed-order butterfly at the end.
+__global__ void __launch_bounds__(256) router_logits_kernel(const float* __restrict__ w, int64_t n_experts,
+                                                            int64_t cols, const float* __restrict__ x, int64_t ldx,
+                                                            float* __restrict__ logits) {
+    const int lane = threadIdx.x & 63;
+    const int64_t e = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t t = blockIdx.y;
+    if (e >= n_experts) return;
+    const float* wr = w + e * cols;
+    const float* xr = x + t * ldx;
+    float acc = 0.0f;
+    for (int64_t c = (int64_t)lane * 4; c + 3 < cols; c += 256) {
+        const float4 a = *reinterpret_cast<const float4*>(wr + c);
+        const float4 b = *reinterpret_cast<const float4*>(xr + c);
+        acc = __fmaf_rn(a.x, b.x, acc);
+        acc = __fmaf_rn(a.y, b.y, acc);
+        acc = __fmaf_rn(a.z, b.z, acc);
+        acc = __fmaf_rn(a.w, b.w, acc);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) logits[t * n_experts + e] = acc;
+}
+
+}  // namespace
+
+hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
+                              float eps, float* sum_out, float* normed_out, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
+                       normed_out);
+    return hipGetLastError();
+}
+
+hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols, const float* x, int64_t n, int64_t ldx,
+                                float* logits, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    if (n > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(router_logits_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256), 0, stream, w,
+                       n_experts, cols, x, ldx, logits);
+    return hipGetLastError();
+}
+
+}  // namespace mq

@@ -77,6 +77,12 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
 hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
                                int64_t ldy, hipStream_t stream);
 
+// ---- elementwise.hip -------------------------------------------------------------------------
+hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
+                              float eps, float* sum_out, float* normed_out, hipStream_t stream);
+hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols, const float* x, int64_t n, int64_t ldx,
+                                float* logits, hipStream_t stream);
+
 // ---- router.hip ------------------------------------------------------------------------------
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                              float* weights, hipStream_t stream);

@@ -185,6 +185,19 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const f
                      float* y_dev, int32_t* ids_out_dev /* may be NULL */, float* weights_out_dev /* may be NULL */,
                      void* stream);
 
+/* ---- the fp32 operators either side of the path --------------------------------------------
+ * sum = x + delta (delta_dev may be NULL: sum = x), normed = sum * (weight / sqrt(mean(sum^2) + eps));
+ * x/delta/sum/normed fp32 [n][cols] dense, weight_dev fp32 [cols] or NULL (ones), sum_out_dev may be NULL
+ * or alias x_dev.  AddRMSNorm (core/src/kernels/hwy/hwy_normalization.cc:102-153) as wired by
+ * cb_add_rms_norm (core/src/llm/graph/fused_ops.cpp:138-169); the input of every projection above. */
+int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                       float eps, float* sum_out_dev, float* normed_out_dev, void* stream);
+/* logits[t][e] = w[e] . x[t] in fp32: the ffn_gate_inp router projection
+ * (core/src/llm/graph/decoder.cpp:2265) whose output mq_moe_layer_q4k consumes.  w_dev fp32
+ * [n_experts][cols], x_dev fp32 [n][ldx], logits_dev fp32 [n][n_experts]; cols % 256 == 0. */
+int mq_router_logits_f32(const float* w_dev, int64_t n_experts, int64_t cols, const float* x_dev, int64_t n,
+                         int64_t ldx, float* logits_dev, void* stream);
+
 /* ---- verification hook -------------------------------------------------------------
  * Runs the production matmul kernel with its per-super-block integer sums
  * written out: dot_scaled_dev / min_dot_dev int32 [rows][n][cols/256], the two

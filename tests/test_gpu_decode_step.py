@@ -1,0 +1,100 @@
+"""The synthetic MoE decoder step (densecore_amd/decode_step.py) against its CPU restatement
+(oracle/decode_step.py): single layers on identical inputs, a multi-layer chain end to end, the
+full-size layer shape, and HIP-graph replays against eager launches."""
+import numpy as np
+import pytest
+
+from oracle import binding as orc
+from oracle import decode_step as ref_step
+
+pytestmark = pytest.mark.gpu
+
+STAGE_REL = 3e-4     # one matmul stage fed by a 1-ulp-different normalised input (a Q8_K code may flip)
+CHAIN_REL = 5e-3     # several layers end to end
+
+
+@pytest.fixture(scope="module")
+def ds():
+    import torch
+    from densecore_amd import decode_step
+    assert torch.cuda.is_available()
+    return decode_step
+
+
+def host_weights(ly):
+    lw = {"wqkv": ly.wqkv.to_ggml(), "wo": ly.wo.to_ggml(), "gate_exps": ly.gate_exps.to_ggml(),
+          "up_exps": ly.up_exps.to_ggml(), "down_exps": ly.down_exps.to_ggml(), "router": ly.router.cpu().numpy()}
+    if ly.shared:
+        lw.update(sh_gate=ly.shared[0].to_ggml(), sh_up=ly.shared[1].to_ggml(), sh_down=ly.shared[2].to_ggml(),
+                  sh_gate_inp=ly.sh_gate_inp.cpu().numpy())
+    return lw
+
+
+def close(got, ref, rel, what):
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    err = np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30)
+    assert err <= rel, f"{what}: {err:.3e} > {rel}"
+
+
+def small_cfg(ds, n_layers):
+    return ds.StepConfig(n_layers=n_layers, hidden=512, n_experts=16, inter=256, top_k=4, n_q=512, n_kv=128, seed=7)
+
+
+@pytest.mark.parametrize("n", [1, 4, 8])
+def test_single_layer_stagewise(ds, n):
+    import torch
+    cfg = small_cfg(ds, 1)
+    step = ds.DecodeStep(cfg, n)
+    x = torch.randn((n, cfg.hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(n))
+    out = step.run(x).cpu().numpy()
+    r = ref_step.layer_forward(host_weights(step.layers[0]), x.cpu().numpy(), None, cfg, step.silu_mode())
+    close(step.qkv.cpu().numpy(), r["qkv"], STAGE_REL, "qkv")
+    close(step.o.cpu().numpy(), r["o"], STAGE_REL, "wo")
+    close(step.logits.cpu().numpy(), r["logits"], 1e-5, "router logits")
+    assert np.array_equal(step.ids[0].cpu().numpy(), r["ids"])
+    close(step.wts[0].cpu().numpy(), r["weights"], 1e-5, "routing weights")
+    close(step.y.cpu().numpy(), r["y"], 2e-3, "moe layer")
+    close(out, r["x"] + r["y"], 2e-3, "layer output")
+    step.free()
+
+
+def test_chain_of_layers_and_graph_replay(ds):
+    import torch
+    cfg = small_cfg(ds, 4)
+    n = 4
+    step = ds.DecodeStep(cfg, n)
+    x = torch.randn((n, cfg.hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(99))
+    eager = step.run(x).clone()
+    xs, delta = x.cpu().numpy(), None
+    for i, ly in enumerate(step.layers):
+        r = ref_step.layer_forward(host_weights(ly), xs, delta, cfg, step.silu_mode())
+        assert np.array_equal(step.ids[i].cpu().numpy(), r["ids"]), f"layer {i}: routing differs"
+        xs, delta = r["x"], r["y"]
+    close(eager.cpu().numpy(), xs + delta, CHAIN_REL, "4-layer chain")
+    # graph replays, with eager work and synchronisations in between, reproduce the eager result bit for bit
+    step.x.copy_(x)
+    step.capture()
+    for rep in range(3):
+        step.x.copy_(x)
+        got = step.replay().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep}"
+        assert torch.equal(step.run(x), eager)
+        torch.cuda.synchronize()
+    step.free()
+
+
+@pytest.mark.parametrize("n", [1, 8])
+def test_full_size_layer(ds, n):
+    """hidden 2048, 256 experts + shared, inter 512, top-8, 16 query / 2 KV heads of 128: one layer."""
+    import torch
+    cfg = ds.StepConfig(n_layers=1, seed=11)
+    step = ds.DecodeStep(cfg, n)
+    x = torch.randn((n, cfg.hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(5 + n))
+    out = step.run(x).cpu().numpy()
+    r = ref_step.layer_forward(host_weights(step.layers[0]), x.cpu().numpy(), None, cfg, step.silu_mode())
+    assert np.array_equal(step.ids[0].cpu().numpy(), r["ids"])
+    close(step.qkv.cpu().numpy(), r["qkv"], STAGE_REL, "qkv")
+    close(step.y.cpu().numpy(), r["y"], 2e-3, "moe layer")
+    close(out, r["x"] + r["y"], 2e-3, "layer output")
+    step.free()

@@ -1,0 +1,50 @@
+"""add + RMSNorm and the fp32 router projection against plain numpy (float64 accumulation)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import decode_step as ref_step
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n,cols", [(1, 2048), (5, 512), (3, 768)])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_add_rmsnorm(n, cols, with_delta):
+    import torch
+    from densecore_amd import _lib
+    rng = np.random.default_rng(n * cols)
+    x = rng.normal(size=(n, cols)).astype(np.float32) * 3
+    d = rng.normal(size=(n, cols)).astype(np.float32) if with_delta else None
+    xs, hs = ref_step.add_rmsnorm(x, d, 1e-6)
+    xt = torch.from_numpy(x).cuda()
+    dt = torch.from_numpy(d).cuda() if with_delta else None
+    h = torch.empty_like(xt)
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    # the sum is written in place over x, as the decoder step does
+    _lib.check(_lib.lib().mq_add_rmsnorm_f32(p(xt), p(dt), None, n, cols, C.c_float(1e-6), p(xt), p(h), None), "rms")
+    torch.cuda.synchronize()
+    assert np.array_equal(xt.cpu().numpy(), xs)
+    np.testing.assert_allclose(h.cpu().numpy(), hs, rtol=2e-6, atol=1e-7)
+    # with a weight vector
+    w = rng.normal(size=cols).astype(np.float32)
+    xt2 = torch.from_numpy(x).cuda()
+    _lib.check(_lib.lib().mq_add_rmsnorm_f32(p(xt2), p(dt), p(torch.from_numpy(w).cuda()), n, cols, C.c_float(1e-6),
+                                             None, p(h), None), "rms")
+    np.testing.assert_allclose(h.cpu().numpy(), hs * w, rtol=3e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("n", [1, 9])
+def test_router_logits(n):
+    import torch
+    from densecore_amd import _lib
+    rng = np.random.default_rng(n)
+    w = rng.normal(size=(256, 2048)).astype(np.float32)
+    x = rng.normal(size=(n, 2048)).astype(np.float32)
+    out = torch.empty((n, 256), device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    wt, xt = torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda()
+    _lib.check(_lib.lib().mq_router_logits_f32(p(wt), 256, 2048, p(xt), n, 2048, p(out), None), "router")
+    ref = ref_step.router_logits(w, x)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=0, atol=2e-5 * np.abs(ref).max())
