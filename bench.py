@@ -28,6 +28,10 @@ HIDDEN, INTER = 4096, 14336
 WIDTHS = (1, 2, 4, 8, 16)
 RING = 8
 HBM_PEAK_GBPS = 8000.0
+INT8_PEAK_TOPS = 5000.0          # dense int8 MFMA, MI355X
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# command, scaled by the same counters' reading on a copy kernel of known size; None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = None
 Q4K_MATRIX_BYTES = INTER * (HIDDEN // 256) * 144          # 33,030,144: the same for gate, up and down
 
 
@@ -59,8 +63,8 @@ def main() -> int:
     ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path is measured on ONE GPU (one MI355X per box); --gpus N with N > 1 is not run. "
-              "How the path would shard over more GPUs is described in DESIGN.md.", file=sys.stderr)
+        print("bench.py: this path is measured on ONE GPU (one MI355X per box); --gpus N with N > 1 is not run "
+              "(the design notes say how the path would shard over more GPUs).", file=sys.stderr)
         return 2
 
     import numpy as np
@@ -120,29 +124,56 @@ def main() -> int:
     value = step_bytes * args.steps / elapsed / 1e9
 
     # ---------------------------------------------------------------- dominant kernel, live
-    # HIP event pairs recorded by the library on the launch stream around every fused gate/up launch
-    ops.census_reset()
-    ops.census_enable(True)
-    launches = 0
-    for i in range(max(RING, min(args.steps, 48))):
-        run_step(i)
-        launches += len(WIDTHS)
-    torch.cuda.synchronize()
-    ops.census_enable(False)
-    gu = ops.census_read(ops.KIND_DENSE_SWIGLU)
-    dn = ops.census_read(ops.KIND_DENSE)
-    ops.census_reset()
-    gu_bytes = sum(gateup_bytes(n) for n in WIDTHS) / len(WIDTHS)
-    achieved = gu_bytes / (gu["avg_us"] * 1e-6) / 1e9 if gu["avg_us"] > 0 else 0.0
+    # The fused gate/up kernel alone, back to back on the cold ring, from pre-quantized activations:
+    # HIP events on the replay stream around a graph of launches, divided by the launch count.
+    def kernel_leg(widths, reps):
+        acts = {n: ops.Q8KActs(n, HIDDEN).quantize(xs[n]) for n in widths}
+        outs = {n: torch.empty((n, INTER), dtype=torch.float32, device=dev) for n in widths}
+
+        def launches():
+            k = 0
+            for i in range(RING):
+                for n in widths:
+                    g, u, _ = sets[(i * len(widths) + k) % RING]
+                    acts[n].swiglu_mul_mat(g, u, ops.SILU_FAST_FMA, out=outs[n])
+                    k += 1
+            return RING * len(widths)
+
+        count = launches()
+        torch.cuda.synchronize()
+        gph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gph, stream=side_stream):
+            launches()
+        torch.cuda.synchronize()
+        gph.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            gph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        for a in acts.values():
+            a.free()
+        return e0.elapsed_time(e1) * 1e3 / (reps * count)     # us per launch
+
+    side_stream = torch.cuda.Stream()
+    narrow = tuple(n for n in WIDTHS if n <= 8)      # one activation tile:  matmul_kernel<2,1,...>
+    wide = tuple(n for n in WIDTHS if n > 8)         # two activation tiles: matmul_kernel<2,2,...>
+    us_narrow = kernel_leg(narrow, 25)
+    us_wide = kernel_leg(wide, 25) if wide else 0.0
+    b_narrow = sum(gateup_bytes(n) for n in narrow) / len(narrow)
+    achieved = b_narrow / (us_narrow * 1e-6) / 1e9
     roofline = {
-        "bound": "hbm", "kernel": "matmul_kernel<2,1> (fused gate/up + SwiGLU, 14336x4096 x2, n=1..16)",
+        "bound": "hbm", "kernel": "matmul_kernel<2,1,false,false> (fused gate/up + SwiGLU, 2 x 14336x4096 Q4_K, n=1,2,4,8)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": None, "bytes_per_launch": int(gu_bytes), "avg_us": round(gu["avg_us"], 3),
-        "min_us": round(gu["min_us"], 3), "launches": gu["count"],
-        "down_kernel": {"avg_us": round(dn["avg_us"], 3), "min_us": round(dn["min_us"], 3),
-                        "achieved": round((Q4K_MATRIX_BYTES + 6.2 * (INTER * 4 + HIDDEN * 4)) / (dn["avg_us"] * 1e-6) / 1e9, 1)
-                        if dn["avg_us"] > 0 else 0.0},
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": int(b_narrow), "avg_us": round(us_narrow, 3),
+        "how": "HIP events around graph replays of back-to-back launches on the cold ring, per launch",
     }
+    if wide:
+        b_wide = sum(gateup_bytes(n) for n in wide) / len(wide)
+        roofline["n16_kernel"] = {"kernel": "matmul_kernel<2,2,false,false> (n=16)", "avg_us": round(us_wide, 3),
+                                  "achieved": round(b_wide / (us_wide * 1e-6) / 1e9, 1),
+                                  "frac": round(b_wide / (us_wide * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
 
     # ---------------------------------------------------------------- per-width detail
     per_width = {}
@@ -157,7 +188,7 @@ def main() -> int:
                 ops.ffn_swiglu(*sets[i % RING], xs[n], ops.SILU_FAST_FMA)
         else:
             gph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gph, stream=side):
+            with torch.cuda.graph(gph, stream=side_stream):
                 for i in range(RING):
                     ops.ffn_swiglu(*sets[i], xs[n], ops.SILU_FAST_FMA)
             torch.cuda.synchronize()
@@ -253,6 +284,60 @@ def side_measurements(ops, synth, torch, np, dev):
         moe[str(n)] = {"us": round(dt * 1e6, 2), "distinct_experts": distinct, "GBps": round(b / dt / 1e9, 1),
                        "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1), "tokens_per_s": round(n / dt, 1)}
     res["moe_layer_mul_mat_id"] = moe
+    for ge, ue, de, sh in layers:
+        for w in (ge, ue, de) + sh[:3]:
+            w.free()
+
+    # cfg4: prefill GEMM 4096 -> 14336 on the int8 matrix cores, quantizer included
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("cfg4"), 14336, 4096)
+    pre = {}
+    for m in (512, 2048):
+        x = torch.randn((m, 4096), device=dev, generator=torch.Generator(device=dev).manual_seed(m))
+        y = torch.empty((m, 14336), dtype=torch.float32, device=dev)
+        dt = time_graph(lambda: [ops.gemm(W, x, out=y) for _ in range(4)], 10) / 4
+        tops = 2.0 * m * 4096 * 14336 / dt / 1e12
+        pre[str(m)] = {"us": round(dt * 1e6, 1), "TOPs": round(tops, 1),
+                       "pct_int8_mfma_peak": round(tops / INT8_PEAK_TOPS * 100, 2),
+                       "pct_int8_mfma_peak_issued": round(tops * 2.5 / INT8_PEAK_TOPS * 100, 2),
+                       "tokens_per_s": round(m / dt, 1)}
+    pre["note"] = ("useful ops 2*M*N*K over quantize + GEMM time; 'issued' counts the 10 MFMAs the kernel issues "
+                   "per 4 a plain int8 GEMM would (two scale digits + two min digits)")
+    res["prefill_gemm_4096x14336"] = pre
+    W.free()
+
+    # cfg5: 40-layer synthetic MoE decoder step, one HIP graph per width
+    from densecore_amd import decode_step
+    cfg = decode_step.StepConfig(synthetic_logits=True)   # router logits N(0,1), as the MoE block is specified
+    base = decode_step.DecodeStep(cfg, 1)
+    steps = {}
+    for n in (1, 4, 8):
+        st = base if n == 1 else decode_step.DecodeStep(cfg, n, layers=base.layers)
+        x = torch.randn((n, cfg.hidden), device=dev, generator=torch.Generator(device=dev).manual_seed(100 + n))
+        st.run(x)
+        torch.cuda.synchronize()
+        distinct = [int(torch.unique(st.ids[i]).numel()) for i in range(cfg.n_layers)]
+        st.x.copy_(x)
+        st.capture()
+        st.replay()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        reps = 10
+        for _ in range(reps):
+            st.replay()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t) / reps
+        q4 = lambda r, c: r * c // 256 * 144
+        per_expert = 2 * q4(cfg.inter, cfg.hidden) + q4(cfg.hidden, cfg.inter)
+        fixed = per_expert + q4(cfg.n_q + 2 * cfg.n_kv, cfg.hidden) + q4(cfg.hidden, cfg.n_q) + cfg.n_experts * cfg.hidden * 4
+        step_bytes = sum(d * per_expert + fixed + n * cfg.hidden * 8 for d in distinct)
+        steps[str(n)] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(n / dt, 1),
+                         "us_per_layer": round(dt * 1e6 / cfg.n_layers, 2),
+                         "distinct_experts_per_layer": round(sum(distinct) / len(distinct), 1),
+                         "per_layer_GBps": round(step_bytes / cfg.n_layers / (dt / cfg.n_layers) / 1e9, 1),
+                         "pct_hbm_peak": round(step_bytes / dt / 1e9 / HBM_PEAK_GBPS * 100, 2)}
+    steps["weights_GB"] = round(cfg.layer_weight_bytes() * cfg.n_layers / 1e9, 2)
+    res["moe_decode_step_40_layers"] = steps
+    base.free()
     return res
 
 
@@ -269,7 +354,7 @@ def cpu_baseline(weight_set, xs, seconds, np):
         for n in WIDTHS:
             orc.simd_ffn_swiglu(g, u, d, HIDDEN, INTER, x_host[n], threads)
         done += 1
-        if time.perf_counter() - t0 >= seconds or done >= 200:
+        if time.perf_counter() - t0 >= seconds:
             break
     dt = time.perf_counter() - t0
     total = done * sum(ffn_bytes(n) for n in WIDTHS)

@@ -23,6 +23,13 @@ struct mq_weight {
     size_t total_bytes = 0;
 };
 
+struct mq_acts {
+    void* aq = nullptr;   // A-major codes
+    void* ad = nullptr;   // A-major scales
+    int64_t max_rows = 0, cols = 0, nb = 0;
+    int64_t n = 0;        // rows quantized by the last mq_acts_quantize
+};
+
 namespace {
 
 thread_local std::string g_error;
@@ -752,6 +759,80 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     a.silu_mode = silu_mode;
     MQ_HIP(census_launch(a, s));
     return MQ_OK;
+}
+
+// ---------------------------------------------------------------------------------- shared Q8_K rows
+int mq_acts_create(int64_t max_rows, int64_t cols, mq_acts** out) {
+    if (int rc = check_ready()) return rc;
+    if (!out || max_rows <= 0 || cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_acts_create: need max_rows > 0 and cols a positive multiple of 256");
+    mq_acts* a = new mq_acts;
+    a->max_rows = max_rows, a->cols = cols, a->nb = cols / kQK;
+    hipError_t e = hipMalloc(&a->aq, aq_bytes(max_rows, a->nb));
+    if (e == hipSuccess) e = hipMalloc(&a->ad, ad_count(max_rows, a->nb) * sizeof(float));
+    if (e != hipSuccess) {
+        if (a->aq) (void)hipFree(a->aq);
+        delete a;
+        return fail(MQ_ERR_HIP, "mq_acts_create: %s", hipGetErrorString(e));
+    }
+    *out = a;
+    return MQ_OK;
+}
+
+int mq_acts_free(mq_acts* a) {
+    if (!a) return MQ_OK;
+    if (a->aq) (void)hipFree(a->aq);
+    if (a->ad) (void)hipFree(a->ad);
+    delete a;
+    return MQ_OK;
+}
+
+int mq_acts_quantize(mq_acts* a, const float* x_dev, int64_t n, int64_t ldx, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!a) return fail(MQ_ERR_INVALID, "mq_acts_quantize: null handle");
+    if (n > a->max_rows) return fail(MQ_ERR_INVALID, "mq_acts_quantize: %lld rows exceed the handle's %lld", (long long)n, (long long)a->max_rows);
+    if (int rc = check_x(x_dev, n, ldx, a->cols, "mq_acts_quantize")) return rc;
+    a->n = n;
+    if (n == 0) return MQ_OK;
+    MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, a->cols, nullptr, 0, (uint8_t*)a->aq, (float*)a->ad, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+static int acts_matmul(const mq_weight* w0, const mq_weight* w1, const mq_acts* a, float* y_dev, int64_t ldy, int swiglu,
+                       int silu_mode, void* stream, const char* who) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w0, who)) return rc;
+    if (w1) {
+        if (int rc = check_weight(w1, who)) return rc;
+        if (w1->cols != w0->cols || w1->rows != w0->rows || w1->n_experts != 1) return fail(MQ_ERR_INVALID, "%s: gate and up must be dense matrices of one shape", who);
+    }
+    if (!a || !y_dev || w0->n_experts != 1 || a->cols != w0->cols || ldy < w0->rows) return fail(MQ_ERR_INVALID, "%s: null argument, expert stack, column mismatch or ldy < rows", who);
+    if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "%s: silu_mode %d", who, silu_mode);
+    if (a->n == 0) return MQ_OK;
+    MatmulArgs m;
+    m.w0 = w0->data;
+    m.w1 = w1 ? w1->data : nullptr;
+    m.rows = w0->rows;
+    m.nb = w0->nb;
+    m.aq = (const uint8_t*)a->aq;
+    m.ad = (const float*)a->ad;
+    m.n = a->n;
+    m.y = y_dev;
+    m.ldy = ldy;
+    m.swiglu = swiglu;
+    m.silu_mode = silu_mode;
+    std::lock_guard<std::mutex> lock(g.mu);
+    MQ_HIP(census_launch(m, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_mul_mat_q4k_acts(const mq_weight* w, const mq_acts* a, float* y_dev, int64_t ldy, void* stream) {
+    return acts_matmul(w, nullptr, a, y_dev, ldy, 0, 0, stream, "mq_mul_mat_q4k_acts");
+}
+
+int mq_swiglu_mul_mat_q4k_acts(const mq_weight* gate, const mq_weight* up, const mq_acts* a, float* h_dev, int64_t ldh,
+                               int silu_mode, void* stream) {
+    if (!up) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k_acts: null up matrix");
+    return acts_matmul(gate, up, a, h_dev, ldh, 1, silu_mode, stream, "mq_swiglu_mul_mat_q4k_acts");
 }
 
 int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exps, const float* x_dev, int64_t n,

@@ -34,6 +34,9 @@ class StepConfig:
     shared_expert: bool = True
     eps: float = 1e-6
     seed: int = 2026
+    # True: every layer routes on resident N(0,1) logits (the MoE block as the benchmark config states it),
+    # the router projection still runs but its output is not used.  False: logits = W_router . rmsnorm(x).
+    synthetic_logits: bool = False
 
     def layer_weight_bytes(self) -> int:
         """ggml bytes of one layer's weights (Q4_K: 144 B per 256 weights; router fp32)."""
@@ -76,9 +79,10 @@ class Layer:
 class DecodeStep:
     """Owns the weights of `cfg.n_layers` layers and the activation buffers of one batch width."""
 
-    def __init__(self, cfg: StepConfig, n_tokens: int):
+    def __init__(self, cfg: StepConfig, n_tokens: int, layers=None):
         self.cfg, self.n = cfg, n_tokens
-        self.layers = [Layer(cfg, i) for i in range(cfg.n_layers)]
+        self._owns_layers = layers is None
+        self.layers = layers if layers is not None else [Layer(cfg, i) for i in range(cfg.n_layers)]
         f = lambda *shape: torch.empty(shape, dtype=torch.float32, device="cuda")
         H = cfg.hidden
         self.x, self.h, self.o, self.y = f(n_tokens, H), f(n_tokens, H), f(n_tokens, H), f(n_tokens, H)
@@ -87,6 +91,10 @@ class DecodeStep:
         self.ids = torch.empty((cfg.n_layers, n_tokens, cfg.top_k), dtype=torch.int32, device="cuda")
         self.wts = f(cfg.n_layers, n_tokens, cfg.top_k)
         self.out = f(n_tokens, H)
+        self.fixed_logits = None
+        if cfg.synthetic_logits:
+            g = torch.Generator(device="cuda").manual_seed(synth.tensor_seed("decode-step-logits", cfg.seed, n_tokens) & 0x7FFFFFFF)
+            self.fixed_logits = torch.randn((cfg.n_layers, n_tokens, cfg.n_experts), device="cuda", generator=g)
         self._graph = None
 
     def silu_mode(self) -> int:
@@ -115,7 +123,8 @@ class DecodeStep:
                                      p(self.h), st), "mq_add_rmsnorm_f32")
             chk(L.mq_router_logits_f32(p(ly.router), cfg.n_experts, cfg.hidden, p(self.h), n, cfg.hidden,
                                        p(self.logits), st), "mq_router_logits_f32")
-            chk(L.mq_moe_layer_q4k(C.byref(ly.desc), p(self.h), p(self.logits), n, p(self.y), p(self.ids[i]),
+            lg = self.fixed_logits[i] if self.fixed_logits is not None else self.logits
+            chk(L.mq_moe_layer_q4k(C.byref(ly.desc), p(self.h), p(lg), n, p(self.y), p(self.ids[i]),
                                    p(self.wts[i]), st), "mq_moe_layer_q4k")
             delta = self.y
         # final residual add; the normalised copy lands in self.h and is not used
@@ -137,6 +146,7 @@ class DecodeStep:
 
     def free(self):
         self._graph = None
-        for ly in self.layers:
-            ly.free()
+        if self._owns_layers:
+            for ly in self.layers:
+                ly.free()
         self.layers = []

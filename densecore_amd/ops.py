@@ -106,14 +106,46 @@ def mul_mat(w: Q4KWeight, x: torch.Tensor) -> torch.Tensor:
     return y
 
 
-def gemm(w: Q4KWeight, x: torch.Tensor) -> torch.Tensor:
+def gemm(w: Q4KWeight, x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     """The same product through the int8 matrix-core GEMM kernel at any n (RunQ4KRawBatchedDenseGemm,
     core/src/backend/cpu_backend_q4k_dense.cpp:57-101)."""
     x = _f32(x)
     n = x.shape[0]
-    y = torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
+    y = out if out is not None else torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
     _lib.check(_lib.lib().mq_gemm_q4k(w._h, _ptr(x), n, x.stride(0), _ptr(y), w.rows, _stream()), "mq_gemm_q4k")
     return y
+
+
+class Q8KActs:
+    """Device-resident Q8_K rows shared by several products (the reference's shared Q8 scratch,
+    core/src/llm/matmul/gemv_exec.cpp:298-341)."""
+
+    def __init__(self, max_rows: int, cols: int):
+        h = C.c_void_p()
+        _lib.check(_lib.lib().mq_acts_create(max_rows, cols, C.byref(h)), "mq_acts_create")
+        self._h, self.max_rows, self.cols, self.n = h.value, max_rows, cols, 0
+
+    def quantize(self, x: torch.Tensor) -> "Q8KActs":
+        x = _f32(x)
+        _lib.check(_lib.lib().mq_acts_quantize(self._h, _ptr(x), x.shape[0], x.stride(0), _stream()), "mq_acts_quantize")
+        self.n = x.shape[0]
+        return self
+
+    def mul_mat(self, w: Q4KWeight, out: torch.Tensor = None) -> torch.Tensor:
+        y = out if out is not None else torch.empty((self.n, w.rows), dtype=torch.float32, device="cuda")
+        _lib.check(_lib.lib().mq_mul_mat_q4k_acts(w._h, self._h, _ptr(y), y.stride(0), _stream()), "mq_mul_mat_q4k_acts")
+        return y
+
+    def swiglu_mul_mat(self, gate: Q4KWeight, up: Q4KWeight, silu: int = 0, out: torch.Tensor = None) -> torch.Tensor:
+        h = out if out is not None else torch.empty((self.n, gate.rows), dtype=torch.float32, device="cuda")
+        _lib.check(_lib.lib().mq_swiglu_mul_mat_q4k_acts(gate._h, up._h, self._h, _ptr(h), h.stride(0), silu, _stream()),
+                   "mq_swiglu_mul_mat_q4k_acts")
+        return h
+
+    def free(self) -> None:
+        if self._h:
+            _lib.lib().mq_acts_free(self._h)
+            self._h = None
 
 
 def mul_mat_q8k(w: Q4KWeight, q8: torch.Tensor) -> torch.Tensor:

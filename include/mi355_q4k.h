@@ -105,6 +105,22 @@ int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t
  * synchronises.  What a GGML_OP_CUSTOM callback calls when ith == 0. */
 int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int64_t ldx, float* y_host, int64_t ldy);
 
+/* ---- quantize once, multiply many times -----------------------------------------------------
+ * A handle to Q8_K activation rows kept on the device in the layout the matmul kernels read, so that
+ * several projections of one input (q/k/v, gate/up) pay for one quantization.  The reference does
+ * the same with the Q8_K scratch that one thread fills and every row-partition thread reads
+ * (core/src/llm/matmul/gemv_exec.cpp:298-341, MatmulWorkState core/src/llm/runtime/work_state.h:86-89)
+ * and with Qwen35SharedQ8RowsUserData (core/src/llm/moe/native.cpp:1027-1038).
+ * create/free allocate and must stay outside a HIP-graph capture; quantize and the two products
+ * only launch kernels.  n of the products is the n of the handle's last mq_acts_quantize. */
+typedef struct mq_acts mq_acts;
+int mq_acts_create(int64_t max_rows, int64_t cols, mq_acts** out);
+int mq_acts_free(mq_acts* a);
+int mq_acts_quantize(mq_acts* a, const float* x_dev, int64_t n, int64_t ldx, void* stream);
+int mq_mul_mat_q4k_acts(const mq_weight* w, const mq_acts* a, float* y_dev, int64_t ldy, void* stream);
+int mq_swiglu_mul_mat_q4k_acts(const mq_weight* gate, const mq_weight* up, const mq_acts* a, float* h_dev,
+                               int64_t ldh, int silu_mode, void* stream);
+
 /* ---- fused gate/up + SwiGLU ----------------------------------------------------
  * h[m][r] = silu(gate[r] . q8k(x[m])) * (up[r] . q8k(x[m])), one pass over both matrices.
  * FusedSwiGLUQ4KQ8KRows_Hwy (core/include/densecore/simd/hwy_ops.h:275-281,

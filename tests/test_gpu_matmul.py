@@ -125,3 +125,22 @@ def test_matmul_is_deterministic(ops):
     for _ in range(3):
         assert np.array_equal(ops.mul_mat(w, x).cpu().numpy().view(np.uint32), a.view(np.uint32))
     w.free()
+
+
+def test_shared_activation_handle_matches_the_one_shot_entry_points():
+    """mq_acts_*: quantize once, then mq_mul_mat_q4k_acts / mq_swiglu_mul_mat_q4k_acts must equal
+    mq_mul_mat_q4k / mq_swiglu_mul_mat_q4k bit for bit (same kernels, same quantized rows)."""
+    import torch
+    from densecore_amd import ops
+    rows, cols = 768, 1024
+    g = ops.Q4KWeight.synthetic(501, rows, cols)
+    u = ops.Q4KWeight.synthetic(502, rows, cols)
+    acts = ops.Q8KActs(16, cols)
+    for n in (16, 3):       # the second, smaller batch reuses the handle
+        x = torch.from_numpy(synth.normal_f32(503 + n, (n, cols))).cuda()
+        acts.quantize(x)
+        assert torch.equal(acts.mul_mat(g), ops.mul_mat(g, x))
+        assert torch.equal(acts.swiglu_mul_mat(g, u, 1), ops.swiglu_mul_mat(g, u, x, 1))
+    with pytest.raises(Exception):
+        acts.quantize(torch.zeros((17, cols), device="cuda"))
+    acts.free(), g.free(), u.free()
