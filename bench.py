@@ -29,9 +29,11 @@ WIDTHS = (1, 2, 4, 8, 16)
 RING = 8
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0          # dense int8 MFMA, MI355X
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# command, scaled by the same counters' reading on a copy kernel of known size; None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
+# `bench.py --kernel-only`: 32,507.8 KiB fetched and 210.0 KiB written per dispatch on average, each scaled by what
+# the same counter reads for the 256 MiB copy of `bench.py --copy-calibration` (FETCH_SIZE 131,083.8 KiB -> x2.000,
+# WRITE_SIZE 262,144.0 KiB -> x1.000): 66,570,000 B read + 215,000 B written.
+TRAFFIC_BYTES_PER_LAUNCH = 66785000
 Q4K_MATRIX_BYTES = INTER * (HIDDEN // 256) * 144          # 33,030,144: the same for gate, up and down
 
 
@@ -60,6 +62,11 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the GEMV / MoE side measurements")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a 256 MiB device-to-device copy kernel 20 times (the known-size reference for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
+    ap.add_argument("--kernel-only", action="store_true",
+                    help="only run the back-to-back launches of the dominant kernel (for counter passes) and exit")
     ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -77,6 +84,15 @@ def main() -> int:
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": src.numel(), "bytes_written": dst.numel(), "launches": 20}))
+        return 0
+
     # ---------------------------------------------------------------- resident data
     sets = []
     for r in range(RING):
@@ -84,6 +100,45 @@ def main() -> int:
                           for nm, rows, cols in (("gate", INTER, HIDDEN), ("up", INTER, HIDDEN), ("down", HIDDEN, INTER))))
     xs = {n: torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg2-x", n), (n, HIDDEN))).to(dev) for n in WIDTHS}
     torch.cuda.synchronize()
+
+    side_stream = torch.cuda.Stream()
+    # The fused gate/up kernel alone, back to back on the cold ring, from pre-quantized activations:
+    # HIP events on the replay stream around a graph of launches, divided by the launch count.
+    def kernel_leg(widths, reps):
+        acts = {n: ops.Q8KActs(n, HIDDEN).quantize(xs[n]) for n in widths}
+        outs = {n: torch.empty((n, INTER), dtype=torch.float32, device=dev) for n in widths}
+
+        def launches():
+            k = 0
+            for i in range(RING):
+                for n in widths:
+                    g, u, _ = sets[k % RING]
+                    acts[n].swiglu_mul_mat(g, u, ops.SILU_FAST_FMA, out=outs[n])
+                    k += 1
+            return RING * len(widths)
+
+        count = launches()
+        torch.cuda.synchronize()
+        gph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gph, stream=side_stream):
+            launches()
+        torch.cuda.synchronize()
+        gph.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            gph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        for a in acts.values():
+            a.free()
+        return e0.elapsed_time(e1) * 1e3 / (reps * count)     # us per launch
+
+    if args.kernel_only:
+        narrow = tuple(n for n in WIDTHS if n <= 8)
+        us = kernel_leg(narrow, 5)
+        print(json.dumps({"kernel_only": "matmul_kernel<2,1,false,false>", "avg_us": round(us, 3), "widths": narrow}))
+        return 0
 
     def run_step(i: int):
         for j, n in enumerate(WIDTHS):
@@ -124,57 +179,52 @@ def main() -> int:
     value = step_bytes * args.steps / elapsed / 1e9
 
     # ---------------------------------------------------------------- dominant kernel, live
-    # The fused gate/up kernel alone, back to back on the cold ring, from pre-quantized activations:
-    # HIP events on the replay stream around a graph of launches, divided by the launch count.
-    def kernel_leg(widths, reps):
-        acts = {n: ops.Q8KActs(n, HIDDEN).quantize(xs[n]) for n in widths}
-        outs = {n: torch.empty((n, INTER), dtype=torch.float32, device=dev) for n in widths}
-
-        def launches():
-            k = 0
-            for i in range(RING):
-                for n in widths:
-                    g, u, _ = sets[(i * len(widths) + k) % RING]
-                    acts[n].swiglu_mul_mat(g, u, ops.SILU_FAST_FMA, out=outs[n])
-                    k += 1
-            return RING * len(widths)
-
-        count = launches()
-        torch.cuda.synchronize()
-        gph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gph, stream=side_stream):
-            launches()
-        torch.cuda.synchronize()
-        gph.replay()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            gph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        for a in acts.values():
-            a.free()
-        return e0.elapsed_time(e1) * 1e3 / (reps * count)     # us per launch
-
-    side_stream = torch.cuda.Stream()
     narrow = tuple(n for n in WIDTHS if n <= 8)      # one activation tile:  matmul_kernel<2,1,...>
     wide = tuple(n for n in WIDTHS if n > 8)         # two activation tiles: matmul_kernel<2,2,...>
+    # (1) the kernel's own duration: start/stop HIP events that the library binds to every gate/up dispatch
+    #     of the same FFN passes the timed region runs (the begin/end timestamps a profiler reports); (2) the same kernel launched back to back from pre-quantized
+    #     activations, events around the whole graph replay, per launch (what a pipelined loop pays).
+    blocker = [torch.empty(1 << 30, dtype=torch.float32, device=dev) for _ in range(2)]
+
+    def census_leg(widths, passes):
+        ops.census_reset()
+        ops.census_enable(True)
+        for _ in range(6):      # ~10 ms of queued copies: the launches below are all submitted while the GPU is
+            blocker[1].copy_(blocker[0])   # still busy, so no event interval contains host submission time
+        for i in range(passes):
+            for n in widths:
+                g, u, d = sets[i % RING]
+                ops.ffn_swiglu(g, u, d, xs[n], ops.SILU_FAST_FMA)
+        torch.cuda.synchronize()
+        ops.census_enable(False)
+        r = ops.census_read(ops.KIND_DENSE_SWIGLU)
+        ops.census_reset()
+        return r
+
+    c_narrow = census_leg(narrow, 32)
     us_narrow = kernel_leg(narrow, 25)
-    us_wide = kernel_leg(wide, 25) if wide else 0.0
     b_narrow = sum(gateup_bytes(n) for n in narrow) / len(narrow)
-    achieved = b_narrow / (us_narrow * 1e-6) / 1e9
+    achieved = b_narrow / (c_narrow["avg_us"] * 1e-6) / 1e9
     roofline = {
         "bound": "hbm", "kernel": "matmul_kernel<2,1,false,false> (fused gate/up + SwiGLU, 2 x 14336x4096 Q4_K, n=1,2,4,8)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": int(b_narrow), "avg_us": round(us_narrow, 3),
-        "how": "HIP events around graph replays of back-to-back launches on the cold ring, per launch",
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH, "bytes_per_launch": int(b_narrow), "avg_us": round(c_narrow["avg_us"], 3),
+        "min_us": round(c_narrow["min_us"], 3), "launches": c_narrow["count"],
+        "how": "start/stop HIP events bound to each dispatch of the kernel (hipExtLaunchKernelGGL), cold ring",
+        "back_to_back": {"avg_us": round(us_narrow, 3), "achieved": round(b_narrow / (us_narrow * 1e-6) / 1e9, 1),
+                         "frac": round(b_narrow / (us_narrow * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                         "how": "events around graph replays of 32 launches from pre-quantized activations, per launch"},
     }
     if wide:
+        c_wide = census_leg(wide, 128)
+        us_wide = kernel_leg(wide, 25)
         b_wide = sum(gateup_bytes(n) for n in wide) / len(wide)
-        roofline["n16_kernel"] = {"kernel": "matmul_kernel<2,2,false,false> (n=16)", "avg_us": round(us_wide, 3),
-                                  "achieved": round(b_wide / (us_wide * 1e-6) / 1e9, 1),
-                                  "frac": round(b_wide / (us_wide * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        roofline["n16_kernel"] = {"kernel": "matmul_kernel<2,2,false,false> (n=16)", "avg_us": round(c_wide["avg_us"], 3),
+                                  "achieved": round(b_wide / (c_wide["avg_us"] * 1e-6) / 1e9, 1),
+                                  "frac": round(b_wide / (c_wide["avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                                  "back_to_back_us": round(us_wide, 3)}
 
+    del blocker
     # ---------------------------------------------------------------- per-width detail
     per_width = {}
     for n in WIDTHS:

@@ -93,7 +93,7 @@ struct State {
     Buffer stage_in, stage_out;  // host-pointer entry points
 } g;
 
-// Launch census: event pairs around matmul-kernel launches (see mq_census_* in the public header).
+// Launch census: a start/stop event pair bound to each matmul-kernel dispatch (see mq_census_* in the public header).
 struct Census {
     bool on = false;
     struct Rec {
@@ -117,11 +117,7 @@ hipError_t census_launch(const MatmulArgs& a, hipStream_t s) {
     }
     Census::Rec& r = census.pool[census.used++];
     r.kind = (a.grouped ? 2 : 0) + (a.swiglu ? 1 : 0);
-    hipError_t e = hipEventRecord(r.start, s);
-    if (e != hipSuccess) return e;
-    e = launch_matmul(a, s);
-    if (e != hipSuccess) return e;
-    return hipEventRecord(r.stop, s);
+    return launch_matmul(a, s, r.start, r.stop);
 }
 
 int check_ready() {
@@ -464,16 +460,10 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     MQ_HIP(g.aq2.reserve(aq_bytes(n, inter / kQK)));
     MQ_HIP(g.ad2.reserve(ad_count(n, inter / kQK) * sizeof(float)));
     if (int rc = reserve_counters((size_t)(inter / kQK))) return rc;
-    const bool fuse_q = getenv("MQ_NOFUSEQ") == nullptr;  // tuning knob
-    if (fuse_q) {
-        a.out_aq = (uint8_t*)g.aq2.ptr;
-        a.out_ad = (float*)g.ad2.ptr;
-        a.out_counters = (uint32_t*)g.counters.ptr;
-    }
+    a.out_aq = (uint8_t*)g.aq2.ptr;
+    a.out_ad = (float*)g.ad2.ptr;
+    a.out_counters = (uint32_t*)g.counters.ptr;
     MQ_HIP(census_launch(a, s));
-    if (!fuse_q) {
-        if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
-    }
     MatmulArgs d;
     d.w0 = down->data;
     d.rows = hidden;

@@ -66,7 +66,8 @@ struct MatmulArgs {
     int sh_yrow_offset = 0;
     int sh_silu_mode = 2;
 };
-hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream);
+// start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
+hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 // ---- prefill.hip -----------------------------------------------------------------------------
 // fp32 rows -> Q8_K in the P-major layout of the prefill GEMM (pmajor_bytes(n, nb) bytes).

@@ -27,15 +27,11 @@
 // (2*(lane/16) and 2*(lane/16)+1): it needs only that row's scales and writes two outputs.
 #include <cstdlib>
 
+#include <hip/hip_ext.h>
+
 #include "common.h"
 #include "kernels.h"
 #include "q8k_block.h"
-
-// Ablation switches for microbenchmarks only (the library is always built with 0):
-// 1 = replace the tile arithmetic by a cheap reduction, 2 = do not load activations.
-#ifndef MQ_ABLATE
-#define MQ_ABLATE 0
-#endif
 
 namespace mq {
 
@@ -65,33 +61,16 @@ __device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__
                                        const size_t (&a_off)[TT], const int (&d_idx)[TT][2]) {
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-#if MQ_ABLATE & 2
-        for (int c = 0; c < 4; ++c) a.q[tt][c] = v4u{(unsigned)a_off[tt], 1u, 2u, (unsigned)c};
-        for (int j = 0; j < 2; ++j) a.yd[tt][j] = (float)d_idx[tt][j];
-#else
 #pragma unroll
         for (int c = 0; c < 4; ++c) a.q[tt][c] = load16(aq_blk + a_off[tt] + c * 1024);
 #pragma unroll
         for (int j = 0; j < 2; ++j) a.yd[tt][j] = ad_blk[d_idx[tt][j]];
-#endif
     }
 }
 
 template <int TT>
 __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>& a, float (&acc)[TT][2],
                                              int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2]) {
-#if MQ_ABLATE & 1
-    {
-        unsigned x = t.q0.x ^ t.q0.y ^ t.q0.z ^ t.q0.w ^ t.q1.x ^ t.q1.y ^ t.q1.z ^ t.q1.w ^ t.hdr.x ^ t.hdr.y ^ t.hdr.z ^ t.hdr.w;
-        for (int tt = 0; tt < TT; ++tt) {
-            for (int c = 0; c < 4; ++c) x ^= a.q[tt][c].x ^ a.q[tt][c].y ^ a.q[tt][c].z ^ a.q[tt][c].w;
-            acc[tt][0] += (float)x * a.yd[tt][0];
-            acc[tt][1] += (float)x * a.yd[tt][1];
-            dot_out[tt][0] = dot_out[tt][1] = min_out[tt][0] = min_out[tt][1] = 0;
-        }
-        return;
-    }
-#endif
     // 6-bit scale / min unpack, word-parallel (core/src/kernels/hwy/hwy_moe_quant.cc:90-101)
     const uint32_t w0 = t.hdr.y, w1 = t.hdr.z, w2 = t.hdr.w;
     const uint32_t sc[2] = {w0 & 0x3f3f3f3fu, (w2 & 0x0f0f0f0fu) | (((w0 >> 6) & 0x03030303u) << 4)};
@@ -217,10 +196,6 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     const uint8_t* tiles[NMAT];
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) tiles[m] = w[m] + tile_offset(rt, 0, nb);
-#if MQ_ABLATE & 4
-    long long stamp[3];
-    stamp[0] = wall_clock64();
-#endif
 
     for (int chunk = 0; chunk < count; chunk += kTokTile * TT) {
         // activation row behind this lane's A slot, and activation / output rows of its two outputs
@@ -302,9 +277,6 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 }
             }
         }
-#if MQ_ABLATE & 4
-        stamp[1] = wall_clock64();
-#endif
 
         // ---- cross-wave reduction in wave order, then the epilogue on wave 0 ----
         if (n_waves > 1) {
@@ -350,16 +322,6 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             }
         }
         if (n_waves > 1 && chunk + kTokTile * TT < count) __syncthreads();  // red[] is reused by the next chunk
-#if MQ_ABLATE & 4
-        stamp[2] = wall_clock64();
-        if (lane == 0 && p.dbg_min) {
-            long long* o = reinterpret_cast<long long*>(p.dbg_min) + ((size_t)blockIdx.x * n_waves + wave) * 4;
-            o[0] = stamp[0];
-            o[1] = stamp[1];
-            o[2] = stamp[2];
-            o[3] = 0;
-        }
-#endif
     }
 
     // ---- optional: the last workgroup to finish a 256-row block of y re-quantizes it to Q8_K ----
@@ -411,15 +373,21 @@ int pick_waves(int64_t nb, int64_t workgroups) {
 }
 
 template <int NMAT, int TT, bool GROUPED, bool DEBUG>
-hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream) {
+hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
-    hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, a);
+    if (start && stop) {
+        // the events take the dispatch's own begin / end timestamps: no extra packets around the kernel
+        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, start, stop,
+                              0, a);
+    } else {
+        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, a);
+    }
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
+hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     if (a.rows <= 0 || a.nb <= 0) return hipErrorInvalidValue;
     if (a.out_aq && (a.rows & 255)) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
@@ -431,18 +399,14 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream) {
     // expert) take a second pass over their 16 rows of weights, which then come from cache.
     const int tt = (a.grouped || widest <= 8) ? 1 : 2;
     const int groups = a.grouped ? a.max_groups + (a.sh_tokens > 0 ? 1 : 0) : 1;
-    int waves = pick_waves(a.nb, rowtiles * groups);
-    if (const char* ev = getenv("MQ_WAVES")) {  // tuning knob
-        const int v = atoi(ev);
-        if (v > 0 && v <= 8 && a.nb % v == 0) waves = v;
-    }
+    const int waves = pick_waves(a.nb, rowtiles * groups);
     const dim3 grid((unsigned)rowtiles, (unsigned)groups);
 
 #define MQ_LAUNCH(NM, T)                                                              \
     do {                                                                              \
-        if (a.grouped) return launch_one<NM, T, true, false>(a, waves, grid, stream); \
-        if (debug) return launch_one<NM, T, false, true>(a, waves, grid, stream);     \
-        return launch_one<NM, T, false, false>(a, waves, grid, stream);               \
+        if (a.grouped) return launch_one<NM, T, true, false>(a, waves, grid, stream, start, stop); \
+        if (debug) return launch_one<NM, T, false, true>(a, waves, grid, stream, start, stop);     \
+        return launch_one<NM, T, false, false>(a, waves, grid, stream, start, stop);               \
     } while (0)
 
     if (nmat == 1) {

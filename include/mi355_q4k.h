@@ -224,10 +224,10 @@ int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64
                         int32_t* min_dot_dev, float* y_dev, int64_t ldy, void* stream);
 
 /* ---- launch census -------------------------------------------------------------------
- * When enabled, a HIP event pair is recorded on the launch stream around every matmul-kernel
- * launch; mq_census_read synchronises and returns the device time between the pairs.  The GPU
+ * When enabled, every matmul-kernel launch carries a start/stop HIP event pair that receives the
+ * dispatch's own begin and end timestamps; mq_census_read synchronises and returns the kernel durations.  The GPU
  * counterpart of the reference's matmul dispatch census of (path, shape, wall ns)
- * (core/src/llm/matmul/gemv_exec.cpp:203-276).  Off by default: the extra events serialise launches. */
+ * (core/src/llm/matmul/gemv_exec.cpp:203-276).  Off by default. */
 #define MQ_KIND_DENSE 0          /* one dense matrix                     */
 #define MQ_KIND_DENSE_SWIGLU 1   /* gate + up fused, dense               */
 #define MQ_KIND_GROUPED 2        /* expert-routed                        */

@@ -48,7 +48,10 @@ def test_matmul_integer_sums_exact_and_fp32_within_tolerance(ops, rows, cols, n)
     ods, omd = orc.matrix_block_sums(w, cols, q8)
     assert np.array_equal(ds, ods), "dot_scaled differs"
     assert np.array_equal(md, omd), "min_dot differs"
-    assert np.array_equal(y_dbg.view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    if n < 48:
+        assert np.array_equal(y_dbg.view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    else:   # from 48 rows up mq_mul_mat_q4k runs the matrix-core GEMM, whose fp32 update uses fused multiply-adds
+        assert np.abs(y_dbg - y).max() <= 1e-5 * np.abs(y).max(), "decode and GEMM kernels disagree"
     mag = orc.dot_magnitude_f64(w, cols, q8)
     for name, ref in oracle_all_orders(w, cols, q8).items():
         assert_fp32_parity(y, ref, mag, f"order={name}")
