@@ -611,7 +611,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     MatmulArgs a;
     if (quantize_hidden) {  // hidden rows leave the kernel already in Q8_K (A-major), ready for the down projection
         const int64_t out_nb = gate->rows / kQK;
-        const int64_t groups = (pairs < gate->n_experts ? pairs : gate->n_experts) + 1;
+        const int64_t groups = (pairs < gate->n_experts ? pairs : gate->n_experts) + (n + 7) / 8;  // + shared-expert passes
         MQ_HIP(g.aq2.reserve(aq_bytes(n * slots, out_nb)));
         MQ_HIP(g.ad2.reserve(ad_count(n * slots, out_nb) * sizeof(float)));
         if (int rc = reserve_counters((size_t)(groups * out_nb))) return rc;

@@ -131,8 +131,8 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
         ar = e;
         yr = e;
     } else if (shared_group) {
-        ar = e * p.sh_arow_stride + p.sh_arow_offset;
-        yr = e * p.sh_yrow_stride + p.sh_yrow_offset;
+        ar = (begin + e) * p.sh_arow_stride + p.sh_arow_offset;
+        yr = (begin + e) * p.sh_yrow_stride + p.sh_yrow_offset;
     } else {
         const int tok = p.entry_token[begin + e], kk = p.entry_k[begin + e];
         ar = tok * p.a_tok_stride + kk * p.a_k_stride;
@@ -183,11 +183,14 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             if (NMAT == 2) w[1] += eoff;
             begin = g_begin;
             count = g_end - g_begin;
-        } else if (g == ng && p.sh_tokens > 0) {
+        } else if (g - ng < (p.sh_tokens + kTokTile * TT - 1) / (kTokTile * TT)) {
+            // the shared expert sees every token: one group per pass of rows, so that its passes run
+            // side by side instead of one after the other in a single workgroup
             shared_group = true;
             w[0] = p.sh_w0;
             w[1] = p.sh_w1;
-            count = p.sh_tokens;
+            begin = (g - ng) * kTokTile * TT;
+            count = p.sh_tokens - begin < kTokTile * TT ? p.sh_tokens - begin : kTokTile * TT;
             silu_mode = p.sh_silu_mode;
         } else {
             return;  // whole workgroup leaves together, before any barrier
@@ -398,7 +401,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     // Expert groups rarely hold more than 8 rows at decode widths; the few that do (and the shared
     // expert) take a second pass over their 16 rows of weights, which then come from cache.
     const int tt = (a.grouped || widest <= 8) ? 1 : 2;
-    const int groups = a.grouped ? a.max_groups + (a.sh_tokens > 0 ? 1 : 0) : 1;
+    const int groups = a.grouped ? a.max_groups + (a.sh_tokens + 8 * tt - 1) / (8 * tt) : 1;
     const int waves = pick_waves(a.nb, rowtiles * groups);
     const dim3 grid((unsigned)rowtiles, (unsigned)groups);
 

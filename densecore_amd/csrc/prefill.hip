@@ -50,10 +50,9 @@ __device__ __forceinline__ uint32_t scale_bytes(uint32_t nibbles, uint32_t digit
     return __builtin_bit_cast(uint32_t, (v2us)(a * d));
 }
 
-// byte `i` of `word` replicated into bits 0..7 and 16..23
+// byte `i` of `word` replicated into bits 0..7 and 16..23 (one v_perm_b32: selector 0x0c yields a zero byte)
 __device__ __forceinline__ uint32_t digit_pair(uint32_t word, int i) {
-    const uint32_t v = (word >> (8 * i)) & 0xffu;
-    return v | (v << 16);
+    return __builtin_amdgcn_perm(0u, word, 0x0c000c00u | (uint32_t)i | ((uint32_t)i << 16));
 }
 
 struct WTile {
