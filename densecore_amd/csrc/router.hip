@@ -81,10 +81,19 @@ __device__ __forceinline__ void route_weights(const float* l, int top_k, int mod
 
 constexpr int kMaxExperts = 2048;
 
-// Routing of one token by one workgroup of 256 threads: every expert's rank is the number of
-// candidates that precede it (ComputeQwenNativeMoEStableTopK's order, core/src/llm/moe/native.cpp:610-645);
-// the experts of rank < top_k are the selection, already in routing order.
-// keys: n_experts 64-bit words of LDS; sel: 8 floats + 8 ints of LDS.
+// The logit behind a route_key (NaN comes back as a canonical NaN, -0 as +0: neither changes a weight).
+__device__ __forceinline__ float route_key_logit(unsigned long long key) {
+    const uint32_t hi = (uint32_t)(key >> 32);
+    if (hi == 0u) return __int_as_float(0x7fc00000);
+    return __uint_as_float((hi & 0x80000000u) ? (hi & 0x7fffffffu) : ~hi);
+}
+
+// Routing of one token by one workgroup of 256 threads.  All threads turn the logits into sort keys in
+// LDS; wavefront 0 then extracts the top_k largest keys one after the other (lane l owns the experts
+// e = l mod 64: a local maximum over its keys, a 6-step butterfly across the lanes, and the owner of
+// the winner clears it).  The keys are unique and totally ordered exactly like
+// ComputeQwenNativeMoEStableTopK (core/src/llm/moe/native.cpp:610-645), so the k-th extraction is the
+// k-th expert of the routing order.  keys: n_experts 64-bit words of LDS; sel: 8 floats + 8 ints of LDS.
 __device__ __forceinline__ void route_token_block(const float* __restrict__ row, int n_experts, int top_k, int mode,
                                                   unsigned long long* keys, float* sel_logit, int32_t* sel_id,
                                                   int32_t* __restrict__ ids_out, float* __restrict__ w_out,
@@ -92,21 +101,29 @@ __device__ __forceinline__ void route_token_block(const float* __restrict__ row,
     const int tid = threadIdx.x;
     for (int e = tid; e < n_experts; e += 256) keys[e] = route_key(row[e], e);
     __syncthreads();
-    for (int e = tid; e < n_experts; e += 256) {
-        const unsigned long long mine = keys[e];
-        int rank = 0;
-        int j = 0;
-        for (; j + 16 <= n_experts; j += 16) {  // batches of 16 keep the LDS reads pipelined
-            unsigned long long k16[16];
+    if (tid < 64) {
+        for (int r = 0; r < top_k; ++r) {
+            unsigned long long best = 0ull;  // below every key
+            for (int e = tid; e < n_experts; e += 64) {
+                const unsigned long long k = keys[e];
+                best = k > best ? k : best;
+            }
 #pragma unroll
-            for (int u = 0; u < 16; ++u) k16[u] = keys[j + u];
-#pragma unroll
-            for (int u = 0; u < 16; ++u) rank += k16[u] > mine;
+            for (int off = 32; off > 0; off >>= 1) {
+                const unsigned long long o = __shfl_xor(best, off, 64);
+                best = o > best ? o : best;
+            }
+            const int id = (int)~(uint32_t)best;
+            if (tid == (id & 63)) keys[id] = 0ull;  // the owning lane is the only one that reads this key again
+            if (tid == 0) {
+                sel_id[r] = id;
+                sel_logit[r] = route_key_logit(best);
+            }
         }
-        for (; j < n_experts; ++j) rank += keys[j] > mine;
-        if (rank < top_k) {
-            sel_logit[rank] = row[e];
-            sel_id[rank] = e;
+        if (tid == 0) {
+            float l[8];
+            for (int k = 0; k < top_k; ++k) l[k] = sel_logit[k];
+            route_weights(l, top_k, mode, w_out);
         }
     }
     __syncthreads();
@@ -116,11 +133,6 @@ __device__ __forceinline__ void route_token_block(const float* __restrict__ row,
         } else {
             ids_out[tid] = sel_id[tid];
         }
-    }
-    if (tid == 0) {
-        float l[8];
-        for (int k = 0; k < top_k; ++k) l[k] = sel_logit[k];
-        route_weights(l, top_k, mode, w_out);
     }
 }
 
@@ -273,7 +285,7 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
     __shared__ int is_last;
     float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
     int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
-    const bool solo = gridDim.x == 1;  // up to four tokens: one workgroup does everything, no handshake
+    const bool solo = gridDim.x == 1;  // one or two tokens: one workgroup does everything, no handshake
     const int per_block = solo ? n : 1;
     for (int t = 0; t < per_block; ++t) {
         const int tok = blockIdx.x * per_block + t;
@@ -393,7 +405,7 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
         return launch_build_groups(ids, n, top_k, n_experts, group_expert, group_begin, n_groups, entry_token, entry_k,
                                    stream);
     }
-    hipLaunchKernelGGL(route_and_group_kernel, dim3(n <= 4 ? 1u : (unsigned)n), dim3(256),
+    hipLaunchKernelGGL(route_and_group_kernel, dim3(n <= 2 ? 1u : (unsigned)n), dim3(256),
                        lds_route > lds_group ? lds_route : lds_group,
                        stream, logits, (int)n_experts, (int)n, top_k, mode, ids, weights, arrivals, group_expert,
                        group_begin, n_groups, entry_token, entry_k);
