@@ -456,14 +456,10 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.ldy = inter;
     a.swiglu = 1;
     a.silu_mode = silu_mode;
-    // the SwiGLU output is re-quantized by the gate/up kernel itself (last workgroup per 256-row block)
-    MQ_HIP(g.aq2.reserve(aq_bytes(n, inter / kQK)));
-    MQ_HIP(g.ad2.reserve(ad_count(n, inter / kQK) * sizeof(float)));
-    if (int rc = reserve_counters((size_t)(inter / kQK))) return rc;
-    a.out_aq = (uint8_t*)g.aq2.ptr;
-    a.out_ad = (float*)g.ad2.ptr;
-    a.out_counters = (uint32_t*)g.counters.ptr;
     MQ_HIP(census_launch(a, s));
+    // The SwiGLU output is re-quantized by a launch of its own: the kernel's fused re-quantization (last
+    // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
+    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
     d.rows = hidden;
