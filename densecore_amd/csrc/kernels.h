@@ -36,6 +36,7 @@ struct MatmulArgs {
     int64_t n = 0;                 // activation rows (dense mode)
     float* y = nullptr;            // dense: [n][ldy]; grouped: [entry][ldy]
     int64_t ldy = 0;
+    int rt_per_wg = 1;             // row tiles per workgroup (set by launch_matmul)
     int swiglu = 0;                // 1: y = silu(w0 x) * (w1 x)
     int silu_mode = 0;
     int32_t* dbg_dot = nullptr;    // optional [rows][n][nb]

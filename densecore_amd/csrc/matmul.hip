@@ -161,7 +161,11 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     const int n_waves = blockDim.x >> 6;
     const int slot = lane & 15;  // A side: M slot (activation row slot/2, half slot%2); B side: weight row
     const int kq = lane >> 4;
-    const int64_t rt = blockIdx.x;
+    // A one-wave workgroup may own several consecutive row tiles (rt_per_wg): it streams them as one run of
+    // tiles and finishes a row tile every nb stages.  Workgroups whose waves split K own exactly one.
+    const int rt_per_wg = p.rt_per_wg > 1 ? p.rt_per_wg : 1;
+    const int64_t rt = (int64_t)blockIdx.x * rt_per_wg;
+    const int rt_count = (int)(((p.rows + 15) >> 4) - rt < rt_per_wg ? ((p.rows + 15) >> 4) - rt : rt_per_wg);
     const int64_t nb = p.nb;
 
     // ---- which activation rows does this workgroup see, and which weights ----
@@ -229,12 +233,34 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = acc[m][tt][1] = 0.0f;
 
+        // silu(gate)*up if fused, then one store per (activation row, weight row) of row tile `tile_rt`
+        auto store_rows = [&](int64_t tile_rt) {
+            const int64_t row = tile_rt * 16 + slot;
+            if (row >= p.rows) return;
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if (yrow[tt][j] >= 0) {
+                        float v = acc[0][tt][j];
+                        if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][tt][j], silu_mode);
+                        float* dst = p.y + (size_t)yrow[tt][j] * (size_t)p.ldy + (size_t)row;
+                        if (p.out_aq) {  // another workgroup re-reads this value: store it device-coherently
+                            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        } else {
+                            *dst = v;
+                        }
+                    }
+                }
+        };
+
         // Ring of S register stages.  Stage i of this wave is super-block wave + i*W.  S-1 stages are
         // requested before the first is consumed, and every consume is preceded by the request for
         // the stage S-1 ahead, so S-1 stages are in flight while the MFMAs of one run.  All branches
         // are wave-uniform and the loads themselves unconditional.
         if (wave < nb) {
-            const int cnt = (int)((nb - wave + n_waves - 1) / n_waves);  // super-blocks of this wave
+            const int per_rt = (int)((nb - wave + n_waves - 1) / n_waves);  // super-blocks of this wave per row tile
+            const int cnt = per_rt * rt_count;                              // stages of this wave
             TileRegs ring_t[S][NMAT];
             ARegs<TT> ring_a[S];
             // Requests past the wave's last super-block are pointed at the (cache-resident)
@@ -242,10 +268,13 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             // fixed, so every wait below can count exactly.
             auto issue = [&](int st, int i) {
                 const bool valid = i < cnt;
-                const int b = valid ? wave + i * n_waves : wave;
+                // several row tiles (one wave, per_rt == nb): stage i is tile i of the contiguous run,
+                // super-block i % nb; one row tile: super-block wave + i*W
+                const int t = valid ? (rt_per_wg > 1 ? i : wave + i * n_waves) : wave;
+                const int b = rt_per_wg > 1 ? t % per_rt : t;
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    load_tile(ring_t[st][m], valid ? tiles[m] + (size_t)b * kTileBytes : p.aq, lane);
+                    load_tile(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileBytes : p.aq, lane);
                 load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             };
             auto consume = [&](int st, int i) {
@@ -253,7 +282,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][2], msum[TT][2];
                     compute_tile<TT>(ring_t[st][m], ring_a[st], acc[m], dsum, msum);
-                    if (DEBUG && p.dbg_dot) {
+                    if (DEBUG && p.dbg_dot) {  // debug launches own one row tile per workgroup
                         const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;
 #pragma unroll
@@ -276,7 +305,16 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 for (int st = 0; st < S; ++st) {
                     const int i = base + st;
                     issue((st + S - 1) % S, i + S - 1);
-                    if (i < cnt) consume(st, i);
+                    if (i < cnt) {
+                        consume(st, i);
+                        if (rt_per_wg > 1 && (i + 1) % per_rt == 0) {  // a row tile is complete: store it, start the next
+                            store_rows(rt + i / per_rt);
+#pragma unroll
+                            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                                for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = acc[m][tt][1] = 0.0f;
+                        }
+                    }
                 }
             }
         }
@@ -294,7 +332,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             }
             __syncthreads();
         }
-        if (wave == 0) {
+        if (wave == 0 && rt_per_wg == 1) {
             for (int wv = 1; wv < n_waves; ++wv) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
@@ -305,24 +343,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                             acc[m][tt][j] =
                                 __fadd_rn(acc[m][tt][j], red[((((wv - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane]);
             }
-            const int64_t row = rt * 16 + slot;
-            if (row < p.rows) {
-#pragma unroll
-                for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        if (yrow[tt][j] >= 0) {
-                            float v = acc[0][tt][j];
-                            if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][tt][j], silu_mode);
-                            float* dst = p.y + (size_t)yrow[tt][j] * (size_t)p.ldy + (size_t)row;
-                            if (p.out_aq) {  // another workgroup re-reads this value: store it device-coherently
-                                __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            } else {
-                                *dst = v;
-                            }
-                        }
-                    }
-            }
+            store_rows(rt);
         }
         if (n_waves > 1 && chunk + kTokTile * TT < count) __syncthreads();  // red[] is reused by the next chunk
     }
@@ -403,13 +424,22 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int tt = (a.grouped || widest <= 8) ? 1 : 2;
     const int groups = a.grouped ? a.max_groups + (a.sh_tokens + 8 * tt - 1) / (8 * tt) : 1;
     const int waves = pick_waves(a.nb, rowtiles * groups);
-    const dim3 grid((unsigned)rowtiles, (unsigned)groups);
+    // Short rows (few super-blocks) in one-wave workgroups: let a workgroup stream several row tiles, so that
+    // its look-ups and activation addressing are paid once per ~16 tiles rather than once per row tile.
+    MatmulArgs b = a;
+    b.rt_per_wg = 1;
+    if (waves == 1 && !debug && !a.out_aq) {
+        int64_t want = 16 / (a.nb * nmat);
+        while (want > 1 && rowtiles % want) --want;  // an even split keeps the last workgroup full
+        b.rt_per_wg = (int)(want > 1 ? want : 1);
+    }
+    const dim3 grid((unsigned)(rowtiles / b.rt_per_wg), (unsigned)groups);
 
 #define MQ_LAUNCH(NM, T)                                                              \
     do {                                                                              \
-        if (a.grouped) return launch_one<NM, T, true, false>(a, waves, grid, stream, start, stop); \
-        if (debug) return launch_one<NM, T, false, true>(a, waves, grid, stream, start, stop);     \
-        return launch_one<NM, T, false, false>(a, waves, grid, stream, start, stop);               \
+        if (a.grouped) return launch_one<NM, T, true, false>(b, waves, grid, stream, start, stop); \
+        if (debug) return launch_one<NM, T, false, true>(b, waves, grid, stream, start, stop);     \
+        return launch_one<NM, T, false, false>(b, waves, grid, stream, start, stop);               \
     } while (0)
 
     if (nmat == 1) {
