@@ -523,7 +523,21 @@ int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* 
                        float eps, float* sum_out_dev, float* normed_out_dev, void* stream) {
     if (int rc = check_ready()) return rc;
     if (!x_dev || !normed_out_dev || n < 0 || cols <= 0) return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_f32: bad arguments");
-    MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, (hipStream_t)stream));
+    MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, nullptr, nullptr,
+                              (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                       float eps, float* sum_out_dev, float* normed_out_dev, mq_acts* acts, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!x_dev || !acts || n < 0 || cols <= 0) return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_q8k: bad arguments");
+    if (acts->cols != cols || n > acts->max_rows) return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_q8k: the handle holds %lld x %lld, asked for %lld x %lld", (long long)acts->max_rows, (long long)acts->cols, (long long)n, (long long)cols);
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15u) || (normed_out_dev && (reinterpret_cast<uintptr_t>(normed_out_dev) & 15u)))
+        return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_q8k: rows must be 16-byte aligned");
+    acts->n = n;
+    MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, (uint8_t*)acts->aq,
+                              (float*)acts->ad, (hipStream_t)stream));
     return MQ_OK;
 }
 
@@ -899,9 +913,12 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     float* wts = weights_out_dev ? weights_out_dev : r.weights;
     // one arrival counter, kept apart from the quantization counters (last slot of that buffer)
     if (int rc = reserve_counters(4096)) return rc;
+    // the same launch quantizes x: extra workgroups next to the routing ones
+    MQ_HIP(g.aq.reserve(aq_bytes(n, hidden / kQK)));
+    MQ_HIP(g.ad.reserve(ad_count(n, hidden / kQK) * sizeof(float)));
     MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
-                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
-    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, x_dev, hidden,
+                                  hidden, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
     if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
     return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,

@@ -4,6 +4,7 @@
 // the device between the Q4_K kernels.
 #include "common.h"
 #include "kernels.h"
+#include "q8k_block.h"
 
 namespace mq {
 
@@ -13,10 +14,12 @@ namespace {
 // AddRMSNorm (core/src/kernels/hwy/hwy_normalization.cc:102-153; plain form in
 // core/tests/kernels/test_normalization.cpp:57-68).  One workgroup per token; the squares are
 // summed per thread in column order, then across lanes and waves in a fixed order.
+// When q_aq is given (cols % 256 == 0) the normalised row also leaves as Q8_K in the layout the matmul
+// kernels read, quantized from the very floats that normed_out receives.
 __global__ void __launch_bounds__(256) add_rmsnorm_kernel(const float* x, const float* __restrict__ delta,
                                                           const float* __restrict__ weight, int64_t cols, float eps,
-                                                          float* sum_out,
-                                                          float* __restrict__ normed_out) {
+                                                          float* sum_out, float* __restrict__ normed_out,
+                                                          uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
     __shared__ float wave_sum[4];
     const int64_t base = (int64_t)blockIdx.x * cols;
     float ssq = 0.0f;
@@ -31,11 +34,25 @@ __global__ void __launch_bounds__(256) add_rmsnorm_kernel(const float* x, const 
     __syncthreads();
     const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
     const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
-    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+    auto normed = [&](int64_t c) {
         // sum_out may alias x: a thread re-reads what it stored itself rather than adding delta twice
         const float v = sum_out ? sum_out[base + c] : (delta ? __fadd_rn(x[base + c], delta[base + c]) : x[base + c]);
         const float sw = weight ? __fmul_rn(scale, weight[c]) : scale;
-        normed_out[base + c] = __fmul_rn(v, sw);
+        return __fmul_rn(v, sw);
+    };
+    if (!q_aq) {
+        for (int64_t c = threadIdx.x; c < cols; c += 256) normed_out[base + c] = normed(c);
+        return;
+    }
+    // one wavefront per super-block, lane l holds its elements 4l .. 4l+3
+    __syncthreads();  // pass 1 stored sum_out with another thread-to-column mapping
+    const int lane = threadIdx.x & 63;
+    const int64_t nb = cols / kQK;
+    for (int64_t b = threadIdx.x >> 6; b < nb; b += 4) {
+        const int64_t c0 = b * kQK + lane * 4;
+        const float e[4] = {normed(c0), normed(c0 + 1), normed(c0 + 2), normed(c0 + 3)};
+        if (normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = make_float4(e[0], e[1], e[2], e[3]);
+        store_amajor(q_aq, q_ad, blockIdx.x, b, nb, lane, quantize_block_q8k(e, lane));
     }
 }
 
@@ -67,10 +84,12 @@ __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restr
 }  // namespace
 
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
-                              float eps, float* sum_out, float* normed_out, hipStream_t stream) {
+                              float eps, float* sum_out, float* normed_out, uint8_t* q_aq, float* q_ad,
+                              hipStream_t stream) {
     if (n == 0) return hipSuccess;
+    if (q_aq && (cols % kQK)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
-                       normed_out);
+                       normed_out, q_aq, q_ad);
     return hipGetLastError();
 }
 

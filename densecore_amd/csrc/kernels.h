@@ -81,7 +81,8 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
 
 // ---- elementwise.hip -------------------------------------------------------------------------
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
-                              float eps, float* sum_out, float* normed_out, hipStream_t stream);
+                              float eps, float* sum_out, float* normed_out, uint8_t* q_aq, float* q_ad,
+                              hipStream_t stream);
 hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols, const float* x, int64_t n, int64_t ldx,
                                 float* logits, hipStream_t stream);
 
@@ -98,7 +99,8 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
 // Router and grouping in one launch at decode widths (falls back to the two kernels above for n > 256).
 hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                                   float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
-                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, hipStream_t stream);
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, const float* qx,
+                                  int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream);
 // y[t][r] = sum_k w[t][k] * part[t*slots + k][r]  (k in order) + gate[t] * part[t*slots + top_k][r]
 hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots, int64_t rows, const float* weights,
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,

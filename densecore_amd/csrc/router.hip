@@ -3,6 +3,7 @@
 // returns to the host; the matmul kernels read the lists these kernels write.
 #include "common.h"
 #include "kernels.h"
+#include "q8k_block.h"
 
 namespace mq {
 
@@ -272,7 +273,9 @@ __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __res
 
 // Router and grouping in one launch (decode widths): a workgroup per token routes it; the last
 // workgroup to finish gathers all ids and builds the expert groups.  `arrivals` is one zeroed
-// uint32 in device memory that the kernel leaves zero again.
+// uint32 in device memory that the kernel leaves zero again.  Workgroups past `route_blocks` do an
+// unrelated job that needs nothing from the router and would otherwise cost a launch of its own: they
+// quantize the layer input to Q8_K (four (row, super-block) units each, as quantize_q8k_kernel does).
 __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __restrict__ logits, int n_experts, int n,
                                                               int top_k, int mode, int32_t* __restrict__ ids,
                                                               float* __restrict__ weights, uint32_t* arrivals,
@@ -280,12 +283,24 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
                                                               int32_t* __restrict__ group_begin,
                                                               int32_t* __restrict__ n_groups,
                                                               int32_t* __restrict__ entry_token,
-                                                              int32_t* __restrict__ entry_k) {
+                                                              int32_t* __restrict__ entry_k, int route_blocks,
+                                                              const float* __restrict__ qx, int64_t q_ldx, int64_t q_nb,
+                                                              uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
+    if ((int)blockIdx.x >= route_blocks) {
+        const int lane = threadIdx.x & 63;
+        const int64_t unit = (int64_t)(blockIdx.x - route_blocks) * 4 + (threadIdx.x >> 6);
+        if (unit >= (int64_t)n * q_nb) return;
+        const int64_t m = unit / q_nb, b = unit - m * q_nb;
+        const float4 v = *reinterpret_cast<const float4*>(qx + m * q_ldx + b * kQK + lane * 4);
+        const float e[4] = {v.x, v.y, v.z, v.w};
+        store_amajor(q_aq, q_ad, m, b, q_nb, lane, quantize_block_q8k(e, lane));
+        return;
+    }
     extern __shared__ unsigned long long route_sh[];  // keys | sel | then reused: counts, ids
     __shared__ int is_last;
     float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
     int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
-    const bool solo = gridDim.x == 1;  // one or two tokens: one workgroup does everything, no handshake
+    const bool solo = route_blocks == 1;  // one or two tokens: one workgroup does everything, no handshake
     const int per_block = solo ? n : 1;
     for (int t = 0; t < per_block; ++t) {
         const int tok = blockIdx.x * per_block + t;
@@ -395,20 +410,26 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
 
 hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                                   float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
-                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, hipStream_t stream) {
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, const float* qx,
+                                  int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
     const size_t lds_route = (size_t)n_experts * 8 + 64;
     const size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
-    if (lds_group > 60 * 1024) {  // prefill widths: route, then group from global memory
+    if (lds_group > 60 * 1024) {  // prefill widths: route, then group from global memory, quantize on its own
         hipError_t e = launch_route_topk(logits, n_experts, n, top_k, mode, ids, weights, stream);
         if (e != hipSuccess) return e;
-        return launch_build_groups(ids, n, top_k, n_experts, group_expert, group_begin, n_groups, entry_token, entry_k,
-                                   stream);
+        e = launch_build_groups(ids, n, top_k, n_experts, group_expert, group_begin, n_groups, entry_token, entry_k,
+                                stream);
+        if (e != hipSuccess || !qx) return e;
+        return launch_quantize_q8k(qx, n, q_ldx, q_cols, nullptr, 0, q_aq, q_ad, stream);
     }
-    hipLaunchKernelGGL(route_and_group_kernel, dim3(n <= 2 ? 1u : (unsigned)n), dim3(256),
-                       lds_route > lds_group ? lds_route : lds_group,
-                       stream, logits, (int)n_experts, (int)n, top_k, mode, ids, weights, arrivals, group_expert,
-                       group_begin, n_groups, entry_token, entry_k);
+    const int route_blocks = n <= 2 ? 1 : (int)n;
+    const int64_t q_nb = q_cols / kQK;
+    const int64_t quant_blocks = qx ? (n * q_nb + 3) / 4 : 0;
+    hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(256),
+                       lds_route > lds_group ? lds_route : lds_group, stream, logits, (int)n_experts, (int)n, top_k, mode,
+                       ids, weights, arrivals, group_expert, group_begin, n_groups, entry_token, entry_k, route_blocks, qx,
+                       q_ldx, q_nb, q_aq, q_ad);
     return hipGetLastError();
 }
 

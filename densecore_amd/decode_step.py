@@ -1,7 +1,8 @@
 """A synthetic MoE decoder step built from the C-ABI operators: per layer
 
-    h   = rmsnorm(x)                                   mq_add_rmsnorm_f32 (fused with the previous residual add)
-    qkv = W_qkv . q8k(h)                               mq_mul_mat_q4k     (wq, wk, wv stacked row-wise)
+    h   = q8k(rmsnorm(x))                              mq_add_rmsnorm_q8k (fused with the previous residual add and
+                                                                           with the projection's quantizer)
+    qkv = W_qkv . h                                    mq_mul_mat_q4k_acts (wq, wk, wv stacked row-wise)
     o   = W_o . q8k(qkv[:, :n_q])                      mq_mul_mat_q4k     (the attention core itself is not on
                                                                            this path: q stands in for its output)
     x   = x + o ; h2 = rmsnorm(x)                      mq_add_rmsnorm_f32
@@ -91,6 +92,7 @@ class DecodeStep:
         self.ids = torch.empty((cfg.n_layers, n_tokens, cfg.top_k), dtype=torch.int32, device="cuda")
         self.wts = f(cfg.n_layers, n_tokens, cfg.top_k)
         self.out = f(n_tokens, H)
+        self.h_q8 = ops.Q8KActs(n_tokens, H)
         self.fixed_logits = None
         if cfg.synthetic_logits:
             g = torch.Generator(device="cuda").manual_seed(synth.tensor_seed("decode-step-logits", cfg.seed, n_tokens) & 0x7FFFFFFF)
@@ -115,9 +117,10 @@ class DecodeStep:
         delta = None
         for i, ly in enumerate(self.layers):
             ly.desc.silu_mode = self.silu_mode()
-            chk(L.mq_add_rmsnorm_f32(p(self.x), p(delta) if delta is not None else None, None, n, cfg.hidden,
-                                     C.c_float(cfg.eps), p(self.x), p(self.h), st), "mq_add_rmsnorm_f32")
-            chk(L.mq_mul_mat_q4k(ly.wqkv._h, p(self.h), n, cfg.hidden, p(self.qkv), self.qkv.shape[1], st), "qkv")
+            chk(L.mq_add_rmsnorm_q8k(p(self.x), p(delta) if delta is not None else None, None, n, cfg.hidden,
+                                     C.c_float(cfg.eps), p(self.x), None, C.c_void_p(self.h_q8._h), st),
+                "mq_add_rmsnorm_q8k")
+            chk(L.mq_mul_mat_q4k_acts(ly.wqkv._h, C.c_void_p(self.h_q8._h), p(self.qkv), self.qkv.shape[1], st), "qkv")
             chk(L.mq_mul_mat_q4k(ly.wo._h, p(self.qkv), n, self.qkv.shape[1], p(self.o), cfg.hidden, st), "wo")
             chk(L.mq_add_rmsnorm_f32(p(self.x), p(self.o), None, n, cfg.hidden, C.c_float(cfg.eps), p(self.x),
                                      p(self.h), st), "mq_add_rmsnorm_f32")
@@ -146,6 +149,7 @@ class DecodeStep:
 
     def free(self):
         self._graph = None
+        self.h_q8.free()
         if self._owns_layers:
             for ly in self.layers:
                 ly.free()

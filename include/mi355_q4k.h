@@ -208,6 +208,12 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const f
  * cb_add_rms_norm (core/src/llm/graph/fused_ops.cpp:138-169); the input of every projection above. */
 int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
                        float eps, float* sum_out_dev, float* normed_out_dev, void* stream);
+/* The same with the normalised rows also (or only: normed_out_dev may be NULL) leaving as Q8_K in an
+ * activation handle, ready for mq_mul_mat_q4k_acts: the quantizer that every projection would otherwise
+ * launch first, folded into the operator that produces its input.  cols % 256 == 0, cols = the handle's.
+ * The Q8_K rows are bit-identical to mq_acts_quantize of the fp32 rows this call writes. */
+int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                       float eps, float* sum_out_dev, float* normed_out_dev, mq_acts* acts, void* stream);
 /* logits[t][e] = w[e] . x[t] in fp32: the ffn_gate_inp router projection
  * (core/src/llm/graph/decoder.cpp:2265) whose output mq_moe_layer_q4k consumes.  w_dev fp32
  * [n_experts][cols], x_dev fp32 [n][ldx], logits_dev fp32 [n][n_experts]; cols % 256 == 0. */

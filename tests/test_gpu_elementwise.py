@@ -48,3 +48,31 @@ def test_router_logits(n):
     _lib.check(_lib.lib().mq_router_logits_f32(p(wt), 256, 2048, p(xt), n, 2048, p(out), None), "router")
     ref = ref_step.router_logits(w, x)
     np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=0, atol=2e-5 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("n,cols", [(1, 2048), (6, 512)])
+def test_add_rmsnorm_q8k_equals_norm_then_quantize(n, cols):
+    """mq_add_rmsnorm_q8k: same fp32 rows as mq_add_rmsnorm_f32, and products from its Q8_K handle equal the
+    products from quantizing those fp32 rows separately, bit for bit."""
+    import torch
+    from densecore_amd import _lib, ops
+    rng = np.random.default_rng(n + cols)
+    x = torch.from_numpy(rng.normal(size=(n, cols)).astype(np.float32) * 2).cuda()
+    d = torch.from_numpy(rng.normal(size=(n, cols)).astype(np.float32)).cuda()
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    ref_sum, ref_h = torch.empty_like(x), torch.empty_like(x)
+    _lib.check(_lib.lib().mq_add_rmsnorm_f32(p(x), p(d), None, n, cols, C.c_float(1e-6), p(ref_sum), p(ref_h), None), "f32")
+    acts = ops.Q8KActs(n, cols)
+    got_sum, got_h = torch.empty_like(x), torch.empty_like(x)
+    _lib.check(_lib.lib().mq_add_rmsnorm_q8k(p(x), p(d), None, n, cols, C.c_float(1e-6), p(got_sum), p(got_h),
+                                             C.c_void_p(acts._h), None), "q8k")
+    acts.n = n
+    assert torch.equal(got_sum, ref_sum) and torch.equal(got_h, ref_h)
+    w = ops.Q4KWeight.synthetic(9, 128, cols)
+    assert torch.equal(acts.mul_mat(w), ops.mul_mat(w, ref_h))
+    # without the fp32 copy and with the sum written in place
+    x2 = x.clone()
+    _lib.check(_lib.lib().mq_add_rmsnorm_q8k(p(x2), p(d), None, n, cols, C.c_float(1e-6), p(x2), None,
+                                             C.c_void_p(acts._h), None), "q8k in place")
+    assert torch.equal(x2, ref_sum) and torch.equal(acts.mul_mat(w), ops.mul_mat(w, ref_h))
+    acts.free(), w.free()
