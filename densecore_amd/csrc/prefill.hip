@@ -16,8 +16,9 @@
 // is done once per super-block, as every reference kernel does.
 //
 //   grid      = (ceil(rowtiles / 8), ceil(m_tiles / 8)); workgroup = 4 wavefronts
-//   workgroup = 128 weight rows x 128 activation rows; per super-block it stages the 128 activation
-//               rows (35 KB in the P-major layout below) in LDS
+//   workgroup = 128 weight rows x 128 activation rows; per super-block the 128 activation rows (35 KB
+//               in the P-major layout below) are staged in LDS, double-buffered and requested one
+//               super-block ahead with LDS-direct loads
 //   wavefront = 2 weight tiles (32 rows) x the 8 activation tiles; it reads its weight tiles
 //               straight from HBM in MFMA lane order and expands them in registers
 //
@@ -95,12 +96,32 @@ __device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, cons
     t.dmin = half_bits_to_float(hdr.x >> 16);
 }
 
-__global__ void __launch_bounds__(256) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Requests the activation tiles of super-block b (copy_words 16-byte words, contiguous in HBM) straight
+// into LDS with global_load_lds_dwordx4: lane l of a request writes its 16 bytes at base + 16*l, so a
+// run of 64-word requests is a linear copy that never touches a register.  The instruction offset must
+// stay 0 (the hardware adds it to the global address as well).
+__device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src, uint8_t* buf, int copy_words, int wave,
+                                                int lane) {
+#pragma unroll
+    for (int j = 0; j < 9; ++j) {  // 4 waves x 9 requests x 64 words >= 8 tiles x 276 words
+        const int first = (j * 4 + wave) * 64;
+        if (first + lane < copy_words)
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)(first + lane) * 16), (lds_ptr_t)(buf + first * 16),
+                                             16, 0, 0);
+    }
+}
+
+__global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy) {
-    extern __shared__ __align__(16) uint8_t a_lds[];  // kMTilesPerGroup * 4416 bytes
+    extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * 4416 bytes
+    constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kq = lane >> 4;
     const int64_t mt0 = (int64_t)blockIdx.y * kMTilesPerGroup;
     const int mt_count = (int)(m_tiles - mt0 < kMTilesPerGroup ? m_tiles - mt0 : kMTilesPerGroup);
@@ -119,9 +140,14 @@ __global__ void __launch_bounds__(256) prefill_gemm_kernel(const uint8_t* __rest
             for (int i = 0; i < 4; ++i) acc[t][m][i] = 0.0f;
 
     const int copy_words = mt_count * kPTileWords;
-    for (int64_t b = 0; b < nb; ++b) {
-        // this wave's weight tiles, requested first so that they travel during the LDS staging
-        v4u seg0[kWTilesPerWave], seg1[kWTilesPerWave], hdr[kWTilesPerWave];
+    const uint8_t* a_src = ap + (size_t)mt0 * kPTileBytes;           // + b * a_stride
+    const size_t a_stride = (size_t)m_tiles * kPTileBytes;
+
+    // Software pipeline over the super-blocks: while super-block b is multiplied, the activation tiles
+    // of b+1 travel HBM/L2 -> LDS (other buffer) and this wave's weight tiles of b+1 travel into
+    // registers.  One workgroup barrier per super-block.
+    v4u seg0[kWTilesPerWave], seg1[kWTilesPerWave], hdr[kWTilesPerWave];
+    auto request_w = [&](int64_t b) {
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
             const uint8_t* tile = w + tile_offset(rt[t], b, nb);
@@ -129,19 +155,29 @@ __global__ void __launch_bounds__(256) prefill_gemm_kernel(const uint8_t* __rest
             seg1[t] = load16(tile + 1024 + lane * 16);
             hdr[t] = load16(tile + kTileQBytes + r * 16);
         }
-        __syncthreads();  // every wave is done reading the previous super-block's activations
-        const uint8_t* src = ap + ((size_t)b * (size_t)m_tiles + (size_t)mt0) * kPTileBytes;
-        for (int i = tid; i < copy_words; i += 256)
-            *reinterpret_cast<v4u*>(a_lds + (size_t)i * 16) = load16(src + (size_t)i * 16);
+    };
+    request_a_tiles(a_src, a_lds, copy_words, wave, lane);
+    request_w(0);
+
+    for (int64_t b = 0; b < nb; ++b) {
+        // everything this thread requested for super-block b has landed ...
+        __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4) | (0xF << 8));  // vmcnt(0)
+        // ... and after the barrier so has everybody else's share of the activation tiles; every wave
+        // is also done reading the other buffer (super-block b-1), which the next requests overwrite
+        __syncthreads();
         WTile wt[kWTilesPerWave];
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) expand_tile(seg0[t], seg1[t], hdr[t], kq, wt[t]);
-        __syncthreads();
+        if (b + 1 < nb) {
+            request_a_tiles(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
+            request_w(b + 1);
+        }
+        const uint8_t* a_buf = a_lds + (b & 1) * kBufBytes;
 
 #pragma unroll
         for (int m = 0; m < kMTilesPerGroup; ++m) {
             if (m < mt_count) {  // uniform over the workgroup
-                const uint8_t* at = a_lds + m * kPTileBytes;
+                const uint8_t* at = a_buf + m * kPTileBytes;
                 v4i a[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
@@ -248,8 +284,15 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
     const dim3 grid((unsigned)((rowtiles + 4 * kWTilesPerWave - 1) / (4 * kWTilesPerWave)),
                     (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup));
     if (grid.y > 65535u) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(prefill_gemm_kernel, grid, dim3(256), kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
-                       ap, m_tiles, n, y, ldy);
+    static bool raised = false;  // two activation buffers: more than the default 64 KB of dynamic LDS
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(prefill_gemm_kernel, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows,
+                       nb, ap, m_tiles, n, y, ldy);
     return hipGetLastError();
 }
 
