@@ -105,12 +105,19 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // stay 0 (the hardware adds it to the global address as well).
 __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src, uint8_t* buf, int copy_words, int wave,
                                                 int lane) {
+    // Written as inline assembly on purpose: the compiler then does not know that LDS is written, and so does
+    // not make every later LDS read wait for these requests (they fill the OTHER buffer).  The kernel waits
+    // for them itself, with vmcnt(0) and a barrier, before the buffer is read.  M0 (the LDS base of the request)
+    // is used by nothing else in this kernel.
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)buf;
 #pragma unroll
     for (int j = 0; j < 9; ++j) {  // 4 waves x 9 requests x 64 words >= 8 tiles x 276 words
         const int first = (j * 4 + wave) * 64;
-        if (first + lane < copy_words)
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)(first + lane) * 16), (lds_ptr_t)(buf + first * 16),
-                                             16, 0, 0);
+        if (first + lane < copy_words) {
+            const uint8_t* g = src + (size_t)(first + lane) * 16;
+            const uint32_t dst = lds_base + (uint32_t)first * 16u;  // wave-uniform; lane l lands at dst + 16*l
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory");
+        }
     }
 }
 
