@@ -371,6 +371,13 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
     if (n >= kPrefillMinRows) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
+    if (n == 1 && !census.on) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
+        const int waves = pick_waves(w->nb, w->rowtiles);
+        if (gemv1_fused_applies(w->nb, waves)) {
+            MQ_HIP(launch_gemv1_fused(w->data, w->rows, w->nb, x_dev, y_dev, waves, s));
+            return MQ_OK;
+        }
+    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }

@@ -67,8 +67,16 @@ struct MatmulArgs {
     int sh_yrow_offset = 0;
     int sh_silu_mode = 2;
 };
+// Waves per workgroup that launch_matmul gives `workgroups` workgroups of rows with nb super-blocks.
+int pick_waves(int64_t nb, int64_t workgroups);
 // start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
+
+// ---- gemv1.hip -------------------------------------------------------------------------------
+// One activation row, quantizer inside the kernel; applies when a wave sees at most two super-blocks.
+bool gemv1_fused_applies(int64_t nb, int waves);
+hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, float* y, int waves,
+                              hipStream_t stream);
 
 // ---- prefill.hip -----------------------------------------------------------------------------
 // fp32 rows -> Q8_K in the P-major layout of the prefill GEMM (pmajor_bytes(n, nb) bytes).
