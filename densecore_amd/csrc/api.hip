@@ -490,6 +490,7 @@ struct RouteWs {  // carved out of g.route
     int32_t* n_groups;
     int32_t* entry_token;
     int32_t* entry_k;
+    const int32_t* direct_ids = nullptr;  // one token: the grouped kernels read the ids themselves, no lists
 };
 int carve_route(int64_t n, int top_k, int64_t n_experts, RouteWs& r) {
     const size_t entries = (size_t)n * (size_t)top_k;
@@ -659,6 +660,9 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     a.y_tok_stride = slots;
     a.y_k_stride = 1;
     a.max_groups = (int)(pairs < gate->n_experts ? pairs : gate->n_experts);
+    a.direct_ids = r.direct_ids;
+    a.direct_top_k = top_k;
+    a.n_experts = (int)gate->n_experts;
     if (sh.gate) {
         a.sh_w0 = sh.gate->data;
         a.sh_w1 = sh.up->data;
@@ -706,6 +710,9 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     d.y_tok_stride = slots;
     d.y_k_stride = 1;
     d.max_groups = (int)(pairs < down->n_experts ? pairs : down->n_experts);
+    d.direct_ids = r.direct_ids;
+    d.direct_top_k = top_k;
+    d.n_experts = (int)down->n_experts;
     if (sh.down) {
         d.sh_w0 = sh.down->data;
         d.sh_tokens = (int)n;
@@ -924,8 +931,9 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     MQ_HIP(g.aq.reserve(aq_bytes(n, hidden / kQK)));
     MQ_HIP(g.ad.reserve(ad_count(n, hidden / kQK) * sizeof(float)));
     MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
-                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, x_dev, hidden,
+                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, n > 1, x_dev, hidden,
                                   hidden, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
+    if (n == 1) r.direct_ids = ids;  // the routing slots of the one token are the expert groups
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
     if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
     return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,

@@ -57,6 +57,10 @@ struct MatmulArgs {
     int a_tok_stride = 1, a_k_stride = 0;   // activation row of an entry = token * a_tok_stride + k * a_k_stride
     int y_tok_stride = 1, y_k_stride = 0;   // output row of an entry
     int max_groups = 0;
+    // one-token shortcut: group g is routing slot g of token 0 with expert direct_ids[g]; no lists are read
+    const int32_t* direct_ids = nullptr;
+    int direct_top_k = 0;
+    int n_experts = 0;             // for range-checking direct_ids
     // optional second family of groups with their own weights (the shared expert): group ids >= n_groups
     const uint8_t* sh_w0 = nullptr;
     const uint8_t* sh_w1 = nullptr;
@@ -107,7 +111,7 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
 // Router and grouping in one launch at decode widths (falls back to the two kernels above for n > 256).
 hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                                   float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
-                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, const float* qx,
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, bool build_groups, const float* qx,
                                   int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream);
 // y[t][r] = sum_k w[t][k] * part[t*slots + k][r]  (k in order) + gate[t] * part[t*slots + top_k][r]
 hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots, int64_t rows, const float* weights,

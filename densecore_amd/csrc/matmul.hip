@@ -48,7 +48,11 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
         ar = (begin + e) * p.sh_arow_stride + p.sh_arow_offset;
         yr = (begin + e) * p.sh_yrow_stride + p.sh_yrow_offset;
     } else {
-        const int tok = p.entry_token[begin + e], kk = p.entry_k[begin + e];
+        int tok = 0, kk = begin + e;  // one-token shortcut: entry = (token 0, slot begin)
+        if (!p.direct_ids) {
+            tok = p.entry_token[begin + e];
+            kk = p.entry_k[begin + e];
+        }
         ar = tok * p.a_tok_stride + kk * p.a_k_stride;
         yr = tok * p.y_tok_stride + kk * p.y_k_stride;
     }
@@ -92,9 +96,19 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
         // the three list reads are independent of each other (the lists are sized for every
         // possible group), so they cost one memory round trip, not three
         const int g = blockIdx.y;
-        const int ng = *p.n_groups;
-        const int g_expert = p.group_expert[g];
-        const int g_begin = p.group_begin[g], g_end = p.group_begin[g + 1];
+        int ng, g_expert, g_begin, g_end;
+        if (p.direct_ids) {  // one token: its routing slots are the groups, nothing was sorted
+            ng = p.direct_top_k;
+            g_expert = p.direct_ids[g < ng ? g : 0];
+            g_begin = g;
+            g_end = g + 1;
+            if (g < ng && (g_expert < 0 || g_expert >= p.n_experts)) return;  // dropped entry
+        } else {
+            ng = *p.n_groups;
+            g_expert = p.group_expert[g];
+            g_begin = p.group_begin[g];
+            g_end = p.group_begin[g + 1];
+        }
         if (g < ng) {
             const size_t eoff = (size_t)g_expert * p.expert_bytes;
             w[0] += eoff;

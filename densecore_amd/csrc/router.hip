@@ -283,7 +283,8 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
                                                               int32_t* __restrict__ group_begin,
                                                               int32_t* __restrict__ n_groups,
                                                               int32_t* __restrict__ entry_token,
-                                                              int32_t* __restrict__ entry_k, int route_blocks,
+                                                              int32_t* __restrict__ entry_k, int build_groups,
+                                                              int route_blocks,
                                                               const float* __restrict__ qx, int64_t q_ldx, int64_t q_nb,
                                                               uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
     if ((int)blockIdx.x >= route_blocks) {
@@ -320,6 +321,7 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
         __syncthreads();
         if (!is_last) return;
     }
+    if (!build_groups) return;  // the consumer takes the ids as they are (one token)
     int32_t* count = reinterpret_cast<int32_t*>(route_sh);
     int32_t* ids_s = count + n_experts;
     const int n_entries = n * top_k;
@@ -410,8 +412,8 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
 
 hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                                   float* weights, uint32_t* arrivals, int32_t* group_expert, int32_t* group_begin,
-                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, const float* qx,
-                                  int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream) {
+                                  int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, bool build_groups,
+                                  const float* qx, int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
     const size_t lds_route = (size_t)n_experts * 8 + 64;
     const size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
@@ -428,7 +430,8 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
     const int64_t quant_blocks = qx ? (n * q_nb + 3) / 4 : 0;
     hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(256),
                        lds_route > lds_group ? lds_route : lds_group, stream, logits, (int)n_experts, (int)n, top_k, mode,
-                       ids, weights, arrivals, group_expert, group_begin, n_groups, entry_token, entry_k, route_blocks, qx,
+                       ids, weights, arrivals, group_expert, group_begin, n_groups, entry_token, entry_k, build_groups ? 1 : 0,
+                       route_blocks, qx,
                        q_ldx, q_nb, q_aq, q_ad);
     return hipGetLastError();
 }
