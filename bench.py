@@ -67,6 +67,8 @@ def main() -> int:
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only run the back-to-back launches of the dominant kernel (for counter passes) and exit")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only run the 14336x4096 prefill GEMM at M = 2048 ten times (for counter passes) and exit")
     ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -91,6 +93,16 @@ def main() -> int:
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration_bytes_read": src.numel(), "bytes_written": dst.numel(), "launches": 20}))
+        return 0
+
+    if args.prefill_only:
+        W = ops.Q4KWeight.synthetic(synth.tensor_seed("cfg4"), 14336, 4096)
+        x = torch.randn((2048, 4096), device=dev, generator=torch.Generator(device=dev).manual_seed(2048))
+        y = torch.empty((2048, 14336), dtype=torch.float32, device=dev)
+        for _ in range(10):
+            ops.gemm(W, x, out=y)
+        torch.cuda.synchronize()
+        print(json.dumps({"prefill_only": "prefill_gemm_kernel", "M": 2048, "launches": 10}))
         return 0
 
     # ---------------------------------------------------------------- resident data
