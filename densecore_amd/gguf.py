@@ -1,0 +1,150 @@
+"""ctypes view of the GGUF reader (include/mi355_q4k_gguf.h) and a minimal GGUF writer for tests and tools.
+
+The reader is the C++ one in libmi355q4k_ggml.so; the writer below produces files in the same published
+layout (GGUF v3, little endian) from numpy arrays and is only meant for fixtures and examples.
+"""
+import ctypes as C
+import struct
+
+import numpy as np
+
+from . import _lib, ggml_adapter, ops
+
+EXPORTS = [
+    "mq_gguf_open", "mq_gguf_last_error", "mq_gguf_close", "mq_gguf_tensor_count", "mq_gguf_tensor_at",
+    "mq_gguf_find_tensor", "mq_gguf_get_int", "mq_gguf_get_string", "mq_gguf_load_q4k",
+]
+
+GGML_F32, GGML_F16, GGML_Q4_K, GGML_I32 = 0, 1, 12, 26
+
+
+class TensorInfo(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_int32), ("n_dims", C.c_int32), ("ne", C.c_int64 * 4),
+                ("offset", C.c_uint64), ("nbytes", C.c_uint64), ("data", C.c_void_p)]
+
+
+_handle = None
+
+
+def lib(need_gpu: bool = False):
+    """The host library; the GPU library is only initialised when a tensor is to be uploaded."""
+    global _handle
+    if _handle is None:
+        _lib.load()
+        L = C.CDLL(ggml_adapter.LIB_PATH, mode=C.RTLD_GLOBAL)
+        L.mq_gguf_open.argtypes = [C.c_char_p, C.POINTER(C.c_void_p)]
+        L.mq_gguf_last_error.restype = C.c_char_p
+        L.mq_gguf_close.argtypes = [C.c_void_p]
+        L.mq_gguf_tensor_count.argtypes = [C.c_void_p]
+        L.mq_gguf_tensor_count.restype = C.c_int64
+        L.mq_gguf_tensor_at.argtypes = [C.c_void_p, C.c_int64, C.POINTER(TensorInfo)]
+        L.mq_gguf_find_tensor.argtypes = [C.c_void_p, C.c_char_p]
+        L.mq_gguf_find_tensor.restype = C.c_int64
+        L.mq_gguf_get_int.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64)]
+        L.mq_gguf_get_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t)]
+        L.mq_gguf_load_q4k.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        _handle = L
+    if need_gpu:
+        _lib.lib()
+    return _handle
+
+
+class GgufFile:
+    def __init__(self, path: str):
+        h = C.c_void_p()
+        if lib().mq_gguf_open(path.encode(), C.byref(h)) != 0:
+            raise ValueError(f"{path}: {lib().mq_gguf_last_error().decode()}")
+        self._h = h
+
+    def close(self):
+        if self._h:
+            lib().mq_gguf_close(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def tensors(self):
+        out = []
+        for i in range(lib().mq_gguf_tensor_count(self._h)):
+            t = TensorInfo()
+            lib().mq_gguf_tensor_at(self._h, i, C.byref(t))
+            out.append({"name": t.name.decode(), "type": t.ggml_type, "ne": list(t.ne)[:t.n_dims], "offset": t.offset,
+                        "nbytes": t.nbytes, "data": t.data})
+        return out
+
+    def find(self, name: str) -> int:
+        return lib().mq_gguf_find_tensor(self._h, name.encode())
+
+    def get_int(self, key: str) -> int:
+        v = C.c_int64()
+        if lib().mq_gguf_get_int(self._h, key.encode(), C.byref(v)) != 0:
+            raise KeyError(lib().mq_gguf_last_error().decode())
+        return v.value
+
+    def get_string(self, key: str) -> str:
+        p, n = C.c_char_p(), C.c_size_t()
+        if lib().mq_gguf_get_string(self._h, key.encode(), C.byref(p), C.byref(n)) != 0:
+            raise KeyError(lib().mq_gguf_last_error().decode())
+        return C.string_at(p, n.value).decode()
+
+    def load_q4k(self, name: str) -> "ops.Q4KWeight":
+        """Upload a GGML_TYPE_Q4_K tensor ([K, N] or [K, N, E]) to the GPU."""
+        lib(need_gpu=True)
+        idx = self.find(name)
+        if idx < 0:
+            raise KeyError(name)
+        t = self.tensors()[idx]
+        h = C.c_void_p()
+        rc = lib().mq_gguf_load_q4k(self._h, name.encode(), C.byref(h))
+        if rc != 0:
+            _lib.check(rc, f"mq_gguf_load_q4k({name}): {lib().mq_gguf_last_error().decode()}")
+        ne = t["ne"] + [1] * (3 - len(t["ne"]))
+        return ops.Q4KWeight(h.value, ne[1], ne[0], ne[2])
+
+
+# ------------------------------------------------------------------------------------------ writer
+_SCALAR = {"u8": (0, "<B"), "i8": (1, "<b"), "u16": (2, "<H"), "i16": (3, "<h"), "u32": (4, "<I"), "i32": (5, "<i"),
+           "f32": (6, "<f"), "bool": (7, "<B"), "u64": (10, "<Q"), "i64": (11, "<q"), "f64": (12, "<d")}
+
+
+def _s(b: bytes) -> bytes:
+    return struct.pack("<Q", len(b)) + b
+
+
+def write_gguf(path: str, metadata: dict, tensors: list, alignment: int = 32, version: int = 3) -> None:
+    """metadata: key -> (kind, value) with kind in _SCALAR, "str", or ("arr", kind); tensors: list of
+    (name, ggml_type, ne (innermost first), numpy array holding the raw bytes)."""
+    out = bytearray()
+    md = dict(metadata)
+    if alignment != 32:
+        md["general.alignment"] = ("u32", alignment)
+    out += struct.pack("<IIQQ", 0x46554747, version, len(tensors), len(md))
+    for key, (kind, value) in md.items():
+        out += _s(key.encode())
+        if kind == "str":
+            out += struct.pack("<I", 8) + _s(value.encode())
+        elif isinstance(kind, tuple):
+            ek = kind[1]
+            out += struct.pack("<I", 9)
+            if ek == "str":
+                out += struct.pack("<IQ", 8, len(value)) + b"".join(_s(v.encode()) for v in value)
+            else:
+                out += struct.pack("<IQ", _SCALAR[ek][0], len(value)) + b"".join(struct.pack(_SCALAR[ek][1], v) for v in value)
+        else:
+            out += struct.pack("<I", _SCALAR[kind][0]) + struct.pack(_SCALAR[kind][1], value)
+    offset, blobs = 0, []
+    for name, ggml_type, ne, array in tensors:
+        raw = np.ascontiguousarray(array).tobytes()
+        out += _s(name.encode()) + struct.pack("<I", len(ne)) + b"".join(struct.pack("<Q", d) for d in ne)
+        out += struct.pack("<IQ", ggml_type, offset)
+        blobs.append(raw)
+        offset += (len(raw) + alignment - 1) // alignment * alignment
+    out += b"\0" * ((-len(out)) % alignment)
+    for raw in blobs:
+        out += raw + b"\0" * ((-len(raw)) % alignment)
+    with open(path, "wb") as f:
+        f.write(out)

@@ -1,0 +1,279 @@
+// GGUF container reader for the Q4_K path (host C++, no HIP): see include/mi355_q4k_gguf.h.
+#include "mi355_q4k_gguf.h"
+
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+
+thread_local std::string t_error;
+
+int fail(const std::string& what) {
+    t_error = what;
+    return MQ_ERR_INVALID;
+}
+
+enum ValueType : uint32_t { U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64 };
+
+size_t scalar_size(uint32_t t) {
+    switch (t) {
+        case U8: case I8: case BOOL: return 1;
+        case U16: case I16: return 2;
+        case U32: case I32: case F32: return 4;
+        case U64: case I64: case F64: return 8;
+        default: return 0;
+    }
+}
+
+// bytes per block and elements per block of the ggml types a Q4_K_M file contains
+bool type_layout(int32_t t, size_t* block_bytes, int64_t* block_elems) {
+    switch (t) {
+        case 0: *block_bytes = 4, *block_elems = 1; return true;      // F32
+        case 1: *block_bytes = 2, *block_elems = 1; return true;      // F16
+        case 2: *block_bytes = 18, *block_elems = 32; return true;    // Q4_0
+        case 8: *block_bytes = 34, *block_elems = 32; return true;    // Q8_0
+        case 12: *block_bytes = 144, *block_elems = 256; return true; // Q4_K
+        case 13: *block_bytes = 176, *block_elems = 256; return true; // Q5_K
+        case 14: *block_bytes = 210, *block_elems = 256; return true; // Q6_K
+        case 24: *block_bytes = 1, *block_elems = 1; return true;     // I8
+        case 26: *block_bytes = 4, *block_elems = 1; return true;     // I32
+        case 30: *block_bytes = 2, *block_elems = 1; return true;     // BF16
+        default: return false;
+    }
+}
+
+struct Cursor {
+    const uint8_t* p;
+    const uint8_t* end;
+    bool ok = true;
+    template <typename T>
+    T get() {
+        T v{};
+        if (!ok || (size_t)(end - p) < sizeof(T)) {
+            ok = false;
+            return v;
+        }
+        std::memcpy(&v, p, sizeof(T));
+        p += sizeof(T);
+        return v;
+    }
+    std::string str() {
+        const uint64_t n = get<uint64_t>();
+        if (!ok || (uint64_t)(end - p) < n) {
+            ok = false;
+            return {};
+        }
+        std::string s(reinterpret_cast<const char*>(p), (size_t)n);
+        p += n;
+        return s;
+    }
+    void skip(uint64_t n) {
+        if (!ok || (uint64_t)(end - p) < n) ok = false;
+        else p += n;
+    }
+};
+
+struct Meta {
+    uint32_t type = 0;
+    int64_t ival = 0;
+    std::string sval;
+};
+
+}  // namespace
+
+struct mq_gguf {
+    int fd = -1;
+    const uint8_t* map = nullptr;
+    size_t size = 0;
+    uint32_t version = 0;
+    uint64_t alignment = 32;
+    const uint8_t* data = nullptr;
+    std::vector<std::string> names;
+    std::vector<mq_gguf_tensor> tensors;
+    std::unordered_map<std::string, int64_t> by_name;
+    std::unordered_map<std::string, Meta> meta;
+};
+
+namespace {
+
+bool skip_value(Cursor& c, uint32_t type, int depth = 0) {
+    if (type == STRING) {
+        c.str();
+    } else if (type == ARRAY) {
+        const uint32_t et = c.get<uint32_t>();
+        const uint64_t n = c.get<uint64_t>();
+        if (depth > 2) return false;
+        if (et == STRING || et == ARRAY) {
+            for (uint64_t i = 0; i < n && c.ok; ++i)
+                if (!skip_value(c, et, depth + 1)) return false;
+        } else {
+            const size_t sz = scalar_size(et);
+            if (!sz) return false;
+            c.skip(n * sz);
+        }
+    } else {
+        const size_t sz = scalar_size(type);
+        if (!sz) return false;
+        c.skip(sz);
+    }
+    return c.ok;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mq_gguf_last_error(void) { return t_error.c_str(); }
+
+int mq_gguf_open(const char* path, mq_gguf** out) {
+    if (!path || !out) return fail("null argument");
+    const int fd = ::open(path, O_RDONLY);
+    if (fd < 0) return fail(std::string("cannot open ") + path);
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size < 24) {
+        ::close(fd);
+        return fail("file too short to be GGUF");
+    }
+    void* map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    if (map == MAP_FAILED) {
+        ::close(fd);
+        return fail("mmap failed");
+    }
+    mq_gguf* g = new mq_gguf;
+    g->fd = fd;
+    g->map = static_cast<const uint8_t*>(map);
+    g->size = (size_t)st.st_size;
+    auto bail = [&](const std::string& why) {
+        mq_gguf_close(g);
+        return fail(why);
+    };
+    Cursor c{g->map, g->map + g->size};
+    if (c.get<uint32_t>() != 0x46554747u) return bail("bad magic (not a GGUF file)");
+    g->version = c.get<uint32_t>();
+    if (g->version != 2 && g->version != 3) return bail("unsupported GGUF version " + std::to_string(g->version));
+    const uint64_t n_tensors = c.get<uint64_t>();
+    const uint64_t n_kv = c.get<uint64_t>();
+    if (!c.ok || n_tensors > (1u << 24) || n_kv > (1u << 24)) return bail("implausible header counts");
+    for (uint64_t i = 0; i < n_kv; ++i) {
+        const std::string key = c.str();
+        const uint32_t type = c.get<uint32_t>();
+        if (!c.ok) return bail("truncated metadata");
+        Meta m;
+        m.type = type;
+        switch (type) {
+            case U8: m.ival = c.get<uint8_t>(); break;
+            case I8: m.ival = c.get<int8_t>(); break;
+            case U16: m.ival = c.get<uint16_t>(); break;
+            case I16: m.ival = c.get<int16_t>(); break;
+            case U32: m.ival = c.get<uint32_t>(); break;
+            case I32: m.ival = c.get<int32_t>(); break;
+            case BOOL: m.ival = c.get<uint8_t>() != 0; break;
+            case U64: m.ival = (int64_t)c.get<uint64_t>(); break;
+            case I64: m.ival = c.get<int64_t>(); break;
+            case STRING: m.sval = c.str(); break;
+            default:
+                if (!skip_value(c, type)) return bail("unsupported metadata value for key " + key);
+        }
+        if (!c.ok) return bail("truncated metadata value for key " + key);
+        g->meta.emplace(key, std::move(m));
+    }
+    auto al = g->meta.find("general.alignment");
+    if (al != g->meta.end() && al->second.type == U32 && al->second.ival > 0) g->alignment = (uint64_t)al->second.ival;
+    if (g->alignment & (g->alignment - 1)) return bail("general.alignment is not a power of two");
+    g->names.reserve((size_t)n_tensors);
+    g->tensors.resize((size_t)n_tensors);
+    for (uint64_t i = 0; i < n_tensors; ++i) {
+        g->names.push_back(c.str());
+        mq_gguf_tensor& t = g->tensors[(size_t)i];
+        t.n_dims = (int32_t)c.get<uint32_t>();
+        if (!c.ok || t.n_dims < 1 || t.n_dims > 4) return bail("tensor with unsupported number of dimensions");
+        for (int d = 0; d < 4; ++d) t.ne[d] = 1;
+        for (int d = 0; d < t.n_dims; ++d) t.ne[d] = (int64_t)c.get<uint64_t>();
+        t.ggml_type = (int32_t)c.get<uint32_t>();
+        t.offset = c.get<uint64_t>();
+        if (!c.ok) return bail("truncated tensor table");
+        size_t bb = 0;
+        int64_t be = 1;
+        t.nbytes = 0;
+        if (type_layout(t.ggml_type, &bb, &be)) {
+            if (t.ne[0] <= 0 || t.ne[0] % be) return bail("tensor " + g->names.back() + ": row length is not a whole number of blocks");
+            t.nbytes = (uint64_t)(t.ne[0] / be) * bb * (uint64_t)t.ne[1] * (uint64_t)t.ne[2] * (uint64_t)t.ne[3];
+        }
+    }
+    const uint64_t header = (uint64_t)(c.p - g->map);
+    const uint64_t base = (header + g->alignment - 1) & ~(g->alignment - 1);
+    if (base > g->size) return bail("data section starts past the end of the file");
+    g->data = g->map + base;
+    for (size_t i = 0; i < g->tensors.size(); ++i) {
+        mq_gguf_tensor& t = g->tensors[i];
+        t.name = g->names[i].c_str();
+        if (t.offset % g->alignment) return bail("tensor " + g->names[i] + ": misaligned offset");
+        if (base + t.offset > g->size || t.nbytes > g->size - base - t.offset) return bail("tensor " + g->names[i] + ": data runs past the end of the file");
+        t.data = g->data + t.offset;
+        g->by_name.emplace(g->names[i], (int64_t)i);
+    }
+    *out = g;
+    return MQ_OK;
+}
+
+int mq_gguf_close(mq_gguf* g) {
+    if (!g) return MQ_OK;
+    if (g->map) munmap(const_cast<uint8_t*>(g->map), g->size);
+    if (g->fd >= 0) ::close(g->fd);
+    delete g;
+    return MQ_OK;
+}
+
+int64_t mq_gguf_tensor_count(const mq_gguf* g) { return g ? (int64_t)g->tensors.size() : 0; }
+
+int mq_gguf_tensor_at(const mq_gguf* g, int64_t index, mq_gguf_tensor* out) {
+    if (!g || !out || index < 0 || index >= (int64_t)g->tensors.size()) return fail("tensor index out of range");
+    *out = g->tensors[(size_t)index];
+    return MQ_OK;
+}
+
+int64_t mq_gguf_find_tensor(const mq_gguf* g, const char* name) {
+    if (!g || !name) return -1;
+    auto it = g->by_name.find(name);
+    return it == g->by_name.end() ? -1 : it->second;
+}
+
+int mq_gguf_get_int(const mq_gguf* g, const char* key, int64_t* out) {
+    if (!g || !key || !out) return fail("null argument");
+    auto it = g->meta.find(key);
+    if (it == g->meta.end()) return fail(std::string("no metadata key ") + key);
+    const uint32_t t = it->second.type;
+    if (t == STRING || t == ARRAY || t == F32 || t == F64) return fail(std::string("metadata key ") + key + " is not an integer");
+    *out = it->second.ival;
+    return MQ_OK;
+}
+
+int mq_gguf_get_string(const mq_gguf* g, const char* key, const char** out, size_t* len) {
+    if (!g || !key || !out) return fail("null argument");
+    auto it = g->meta.find(key);
+    if (it == g->meta.end() || it->second.type != STRING) return fail(std::string("no string metadata key ") + key);
+    *out = it->second.sval.c_str();
+    if (len) *len = it->second.sval.size();
+    return MQ_OK;
+}
+
+int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out) {
+    if (!g || !name || !out) return fail("null argument");
+    const int64_t idx = mq_gguf_find_tensor(g, name);
+    if (idx < 0) return fail(std::string("no tensor ") + name);
+    const mq_gguf_tensor& t = g->tensors[(size_t)idx];
+    if (t.ggml_type != 12) return fail(std::string("tensor ") + name + " is not GGML_TYPE_Q4_K");
+    if (t.n_dims > 3 || t.ne[3] != 1) return fail(std::string("tensor ") + name + " has more than three dimensions");
+    const size_t row_bytes = (size_t)(t.ne[0] / 256) * 144;
+    return mq_weight_upload(t.data, t.ne[1], t.ne[0], t.ne[2], row_bytes, row_bytes * (size_t)t.ne[1], out);
+}
+
+}  // extern "C"
