@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libmi355q4k.so")
 # every symbol include/mi355_q4k.h declares
 EXPORTS = [
     "mq_init", "mq_shutdown", "mq_last_error", "mq_device_info",
-    "mq_weight_upload", "mq_weight_synthetic", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
+    "mq_weight_upload", "mq_weight_upload_typed", "mq_weight_synthetic", "mq_weight_synthetic_typed", "mq_weight_type", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
     "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_gemm_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
     "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums",
@@ -56,6 +56,9 @@ def load() -> C.CDLL:
     L.mq_device_info.argtypes = [C.c_char_p, sz, C.POINTER(ci), C.POINTER(sz)]
     L.mq_weight_upload.argtypes = [vp, i64, i64, i64, sz, sz, C.POINTER(vp)]
     L.mq_weight_synthetic.argtypes = [C.c_uint64, i64, i64, i64, C.POINTER(vp)]
+    L.mq_weight_upload_typed.argtypes = [C.c_int, vp, i64, i64, i64, sz, sz, C.POINTER(vp)]
+    L.mq_weight_synthetic_typed.argtypes = [C.c_int, C.c_uint64, i64, i64, i64, C.POINTER(vp)]
+    L.mq_weight_type.argtypes = [vp]
     L.mq_weight_download.argtypes = [vp, vp, sz, sz]
     L.mq_weight_shape.argtypes = [vp, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64), C.POINTER(sz)]
     L.mq_weight_free.argtypes = [vp]

@@ -19,6 +19,7 @@ struct mq_weight {
     uint8_t* data = nullptr;     // tiled layout, experts back to back
     int64_t rows = 0, cols = 0, n_experts = 0;
     int64_t nb = 0, rowtiles = 0;
+    int type = kTypeQ4K;         // ggml_type: 12 (Q4_K) or 13 (Q5_K)
     size_t expert_bytes = 0;     // tiled bytes per expert
     size_t total_bytes = 0;
 };
@@ -158,18 +159,20 @@ int reserve_counters(size_t count) {
     return MQ_OK;
 }
 
-int alloc_weight(int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
+int alloc_weight(int type, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
     if (!out) return fail(MQ_ERR_INVALID, "null output handle");
     *out = nullptr;
+    if (type != kTypeQ4K && type != kTypeQ5K) return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12) and Q5_K (13) weights are supported", type);
     if (rows <= 0 || cols <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "rows, cols and n_experts must be positive");
     if (cols % kQK) return fail(MQ_ERR_INVALID, "cols %lld is not a multiple of 256", (long long)cols);
     mq_weight* w = new mq_weight;
+    w->type = type;
     w->rows = rows;
     w->cols = cols;
     w->n_experts = n_experts;
     w->nb = cols / kQK;
     w->rowtiles = (rows + 15) / 16;
-    w->expert_bytes = (size_t)w->rowtiles * (size_t)w->nb * kTileBytes;
+    w->expert_bytes = (size_t)w->rowtiles * (size_t)w->nb * (size_t)tile_bytes_of(type);
     w->total_bytes = w->expert_bytes * (size_t)n_experts;
     hipError_t e = hipMalloc((void**)&w->data, w->total_bytes);
     if (e != hipSuccess) {
@@ -232,21 +235,27 @@ int mq_device_info(char* name_out, size_t name_cap, int* cu_count, size_t* hbm_b
 // ---------------------------------------------------------------------------------- weights
 int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts, size_t row_bytes,
                      size_t expert_bytes, mq_weight** out) {
+    return mq_weight_upload_typed(kTypeQ4K, q4k_host, rows, cols, n_experts, row_bytes, expert_bytes, out);
+}
+
+int mq_weight_upload_typed(int ggml_type, const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts,
+                           size_t row_bytes, size_t expert_bytes, mq_weight** out) {
     if (int rc = check_ready()) return rc;
+    if (ggml_type != kTypeQ4K && ggml_type != kTypeQ5K) return fail(MQ_ERR_UNSUPPORTED, "mq_weight_upload: ggml type %d (only 12 = Q4_K and 13 = Q5_K)", ggml_type);
     if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_upload: null host pointer");
     if (cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_weight_upload: cols %lld is not a positive multiple of 256", (long long)cols);
-    const size_t min_row = (size_t)(cols / kQK) * kQ4Block;
+    const size_t min_row = (size_t)(cols / kQK) * (size_t)block_bytes_of(ggml_type);
     if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_upload: row_bytes %zu < %zu or odd", row_bytes, min_row);
     if (n_experts > 1 && expert_bytes < row_bytes * (size_t)rows) return fail(MQ_ERR_INVALID, "mq_weight_upload: expert_bytes too small");
     mq_weight* w = nullptr;
-    if (int rc = alloc_weight(rows, cols, n_experts, &w)) return rc;
+    if (int rc = alloc_weight(ggml_type, rows, cols, n_experts, &w)) return rc;
     const size_t raw_total = n_experts > 1 ? expert_bytes * (size_t)(n_experts - 1) + row_bytes * (size_t)rows
                                            : row_bytes * (size_t)(rows - 1) + min_row;
     void* raw = nullptr;
     hipError_t e = hipMalloc(&raw, raw_total);
     if (e == hipSuccess) e = hipMemcpy(raw, q4k_host, raw_total, hipMemcpyHostToDevice);
     if (e == hipSuccess)
-        e = launch_tile_weights((const uint8_t*)raw, rows, w->nb, row_bytes, expert_bytes, n_experts, w->data,
+        e = launch_tile_weights((const uint8_t*)raw, rows, w->nb, ggml_type, row_bytes, expert_bytes, n_experts, w->data,
                                 w->expert_bytes, nullptr);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (raw) (void)hipFree(raw);
@@ -259,10 +268,15 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
 }
 
 int mq_weight_synthetic(uint64_t seed, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
+    return mq_weight_synthetic_typed(kTypeQ4K, seed, rows, cols, n_experts, out);
+}
+
+int mq_weight_synthetic_typed(int ggml_type, uint64_t seed, int64_t rows, int64_t cols, int64_t n_experts,
+                              mq_weight** out) {
     if (int rc = check_ready()) return rc;
     mq_weight* w = nullptr;
-    if (int rc = alloc_weight(rows, cols, n_experts, &w)) return rc;
-    hipError_t e = launch_synth_weights(seed, rows, w->nb, n_experts, w->data, w->expert_bytes, nullptr);
+    if (int rc = alloc_weight(ggml_type, rows, cols, n_experts, &w)) return rc;
+    hipError_t e = launch_synth_weights(seed, rows, w->nb, ggml_type, n_experts, w->data, w->expert_bytes, nullptr);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         mq_weight_free(w);
@@ -276,7 +290,7 @@ int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, siz
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_weight_download")) return rc;
     if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_download: null host pointer");
-    const size_t min_row = (size_t)w->nb * kQ4Block;
+    const size_t min_row = (size_t)w->nb * (size_t)block_bytes_of(w->type);
     if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_download: bad row_bytes");
     if (w->n_experts > 1 && expert_bytes < row_bytes * (size_t)w->rows) return fail(MQ_ERR_INVALID, "mq_weight_download: bad expert_bytes");
     const size_t raw_total = w->n_experts > 1 ? expert_bytes * (size_t)(w->n_experts - 1) + row_bytes * (size_t)w->rows
@@ -285,7 +299,7 @@ int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, siz
     hipError_t e = hipMalloc(&raw, raw_total);
     if (e == hipSuccess) e = hipMemcpy(raw, q4k_host, raw_total, hipMemcpyHostToDevice);  // keep caller's padding bytes
     if (e == hipSuccess)
-        e = launch_untile_weights(w->data, w->rows, w->nb, row_bytes, expert_bytes, w->n_experts, (uint8_t*)raw,
+        e = launch_untile_weights(w->data, w->rows, w->nb, w->type, row_bytes, expert_bytes, w->n_experts, (uint8_t*)raw,
                                   w->expert_bytes, nullptr);
     if (e == hipSuccess) e = hipMemcpy(q4k_host, raw, raw_total, hipMemcpyDeviceToHost);
     if (raw) (void)hipFree(raw);
@@ -301,6 +315,8 @@ int mq_weight_shape(const mq_weight* w, int64_t* rows, int64_t* cols, int64_t* n
     if (device_bytes) *device_bytes = w->total_bytes;
     return MQ_OK;
 }
+
+int mq_weight_type(const mq_weight* w) { return w ? w->type : -1; }
 
 int mq_weight_free(mq_weight* w) {
     if (!w) return MQ_OK;
@@ -325,6 +341,7 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
     if (n == 0) return MQ_OK;
     MatmulArgs a;
     a.w0 = w->data;
+    a.wtype = w->type;
     a.rows = w->rows;
     a.nb = w->nb;
     a.aq = (const uint8_t*)g.aq.ptr;
@@ -355,6 +372,7 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_gemm_q4k")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: weight is an expert stack");
+    if (w->type != kTypeQ4K) return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
@@ -370,8 +388,8 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    if (n >= kPrefillMinRows) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
-    if (n == 1 && !census.on) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
+    if (n >= kPrefillMinRows && w->type == kTypeQ4K) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
+    if (n == 1 && !census.on && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemv1_fused(w->data, w->rows, w->nb, x_dev, y_dev, waves, s));
@@ -442,6 +460,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (up->cols != hidden || up->rows != inter || down->cols != inter || down->rows != hidden || gate->n_experts != 1 ||
         up->n_experts != 1 || down->n_experts != 1)
         return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: gate/up must be [inter][hidden] and down [hidden][inter]");
+    if (up->type != gate->type) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: gate and up must have one quantization type");
     if (inter % kQK) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: inter %lld is not a multiple of 256", (long long)inter);
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: silu_mode %d", silu_mode);
     if (int rc = check_x(x_dev, n, hidden, hidden, "mq_ffn_swiglu_q4k")) return rc;
@@ -453,6 +472,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
     MatmulArgs a;
     a.w0 = gate->data;
+    a.wtype = gate->type;
     a.w1 = up->data;
     a.rows = inter;
     a.nb = gate->nb;
@@ -469,6 +489,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
+    d.wtype = down->type;
     d.rows = hidden;
     d.nb = down->nb;
     d.aq = (const uint8_t*)g.aq2.ptr;
@@ -589,6 +610,7 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
                                r.entry_token, r.entry_k, s));
     MatmulArgs a;
     a.w0 = w->data;
+    a.wtype = w->type;
     a.rows = w->rows;
     a.nb = w->nb;
     a.expert_bytes = w->expert_bytes;
@@ -638,6 +660,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
         a.out_counters = (uint32_t*)g.counters.ptr;
     }
     a.w0 = gate->data;
+    a.wtype = gate->type;
     a.w1 = up->data;
     a.rows = gate->rows;
     a.nb = gate->nb;
@@ -691,6 +714,7 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden_dim * sizeof(float)));
     MatmulArgs d;
     d.w0 = down->data;
+    d.wtype = down->type;
     d.rows = hidden_dim;
     d.nb = down->nb;
     d.expert_bytes = down->expert_bytes;
@@ -729,7 +753,7 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
 
 int check_experts(const mq_weight* gate, const mq_weight* up, const mq_weight* down, int top_k, const char* name) {
     if (gate && up) {
-        if (up->cols != gate->cols || up->rows != gate->rows || up->n_experts != gate->n_experts)
+        if (up->cols != gate->cols || up->rows != gate->rows || up->n_experts != gate->n_experts || up->type != gate->type)
             return fail(MQ_ERR_INVALID, "%s: gate and up expert tensors disagree", name);
         if (gate->rows % kQK) return fail(MQ_ERR_INVALID, "%s: inter must be a multiple of 256", name);
     }
@@ -750,8 +774,8 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(gate, "mq_swiglu_mul_mat_q4k(gate)")) return rc;
     if (int rc = check_weight(up, "mq_swiglu_mul_mat_q4k(up)")) return rc;
-    if (up->cols != gate->cols || up->rows != gate->rows || gate->n_experts != 1 || up->n_experts != 1)
-        return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: gate and up must be dense matrices of one shape");
+    if (up->cols != gate->cols || up->rows != gate->rows || gate->n_experts != 1 || up->n_experts != 1 || up->type != gate->type)
+        return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: gate and up must be dense matrices of one shape and type");
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: silu_mode %d", silu_mode);
     if (int rc = check_x(x_dev, n, ldx, gate->cols, "mq_swiglu_mul_mat_q4k")) return rc;
     if (!h_dev || ldh < gate->rows) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: null output or ldh < rows");
@@ -761,6 +785,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
     MatmulArgs a;
     a.w0 = gate->data;
+    a.wtype = gate->type;
     a.w1 = up->data;
     a.rows = gate->rows;
     a.nb = gate->nb;
@@ -817,13 +842,14 @@ static int acts_matmul(const mq_weight* w0, const mq_weight* w1, const mq_acts* 
     if (int rc = check_weight(w0, who)) return rc;
     if (w1) {
         if (int rc = check_weight(w1, who)) return rc;
-        if (w1->cols != w0->cols || w1->rows != w0->rows || w1->n_experts != 1) return fail(MQ_ERR_INVALID, "%s: gate and up must be dense matrices of one shape", who);
+        if (w1->cols != w0->cols || w1->rows != w0->rows || w1->n_experts != 1 || w1->type != w0->type) return fail(MQ_ERR_INVALID, "%s: gate and up must be dense matrices of one shape", who);
     }
     if (!a || !y_dev || w0->n_experts != 1 || a->cols != w0->cols || ldy < w0->rows) return fail(MQ_ERR_INVALID, "%s: null argument, expert stack, column mismatch or ldy < rows", who);
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "%s: silu_mode %d", who, silu_mode);
     if (a->n == 0) return MQ_OK;
     MatmulArgs m;
     m.w0 = w0->data;
+    m.wtype = w0->type;
     m.w1 = w1 ? w1->data : nullptr;
     m.rows = w0->rows;
     m.nb = w0->nb;
@@ -907,8 +933,10 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)")) return rc;
         if (L->shared_gate->cols != hidden || L->shared_gate->rows != inter || L->shared_up->cols != hidden ||
             L->shared_up->rows != inter || L->shared_down->cols != inter || L->shared_down->rows != hidden ||
-            L->shared_gate->n_experts != 1 || L->shared_up->n_experts != 1 || L->shared_down->n_experts != 1)
-            return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: shared expert must have the routed experts' shape");
+            L->shared_gate->n_experts != 1 || L->shared_up->n_experts != 1 || L->shared_down->n_experts != 1 ||
+            L->shared_gate->type != L->gate_exps->type || L->shared_up->type != L->gate_exps->type ||
+            L->shared_down->type != L->down_exps->type)
+            return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: shared expert must have the routed experts' shape and types");
         sh.gate = L->shared_gate;
         sh.up = L->shared_up;
         sh.down = L->shared_down;

@@ -26,8 +26,8 @@ constexpr int kTileQBytes = kTileRows * 128;      // 2048: nibble part
 //   bytes [2048 + r*16, +16)                 = {fp16 d, fp16 dmin, scales[12]} of row r
 // Same 144 bytes per 256 weights as ggml's block_q4_K; only the order differs.
 // ---------------------------------------------------------------------------------------------
-__host__ __device__ inline size_t tile_offset(int64_t rt, int64_t b, int64_t nb) {
-    return (size_t)(rt * nb + b) * kTileBytes;
+__host__ __device__ inline size_t tile_offset(int64_t rt, int64_t b, int64_t nb, int tile_bytes = kTileBytes) {
+    return (size_t)(rt * nb + b) * (size_t)tile_bytes;
 }
 
 // Offset inside a tile of the 8-byte word `word` (0..17) of row r's block_q4_K.
@@ -37,6 +37,27 @@ __host__ __device__ inline int tile_word_offset(int r, int word) {
     const int chunk = j >> 2;      // 32-byte chunk of qs
     const int kq = j & 3;
     return (chunk >> 1) * 1024 + (kq * 16 + r) * 16 + (chunk & 1) * 8;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q5_K (block_q5_K, 176 bytes: Q4_K plus qh[32], one high bit per weight -- bit s of qh[l] belongs to
+// element l of sub-block s; core/src/kernels/hwy/hwy_moe_quant.cc:36-45,177-200).  Same tile as Q4_K with
+// the high bits appended: 2816 bytes per 16 rows x one super-block,
+//   bytes [0, 2304)                          as above (nibbles, then headers)
+//   bytes [2304 + (kq*16 + r)*8, +8)         = qh[r][8*kq .. 8*kq+7]: all eight sub-block bits of the eight
+//                                              elements whose nibbles lane (kq, r) holds
+// Word w of a block_q5_K (8 bytes each, 22 of them): 0..1 header, 2..5 qh, 6..21 qs.
+// ---------------------------------------------------------------------------------------------
+constexpr int kQ5Block = 176;
+constexpr int kTile5Bytes = kTileRows * kQ5Block;  // 2816
+constexpr int kTileHBytes = kTileBytes;            // offset of the qh part
+constexpr int kTypeQ4K = 12, kTypeQ5K = 13;        // ggml_type values
+__host__ __device__ inline int tile_bytes_of(int type) { return type == kTypeQ5K ? kTile5Bytes : kTileBytes; }
+__host__ __device__ inline int block_bytes_of(int type) { return type == kTypeQ5K ? kQ5Block : kQ4Block; }
+__host__ __device__ inline int tile_word_offset_q5(int r, int word) {
+    if (word < 2) return kTileQBytes + r * 16 + word * 8;
+    if (word < 6) return kTileHBytes + ((word - 2) * 16 + r) * 8;
+    return tile_word_offset(r, word - 4);  // qs words 6..21 map like Q4_K's 2..17
 }
 
 // ---------------------------------------------------------------------------------------------

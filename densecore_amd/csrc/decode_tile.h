@@ -7,14 +7,19 @@
 namespace mq {
 
 #if defined(__HIPCC__)
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
 struct TileRegs {
     v4u q0, q1, hdr;
+    v2u qh;  // Q5_K only: qh[8*kq .. 8*kq+7] of weight row lane%16 (bit s = fifth bit in sub-block s)
 };
 
+template <bool Q5 = false>
 __device__ __forceinline__ void load_tile(TileRegs& t, const uint8_t* tile, int lane) {
     t.q0 = load_stream16(tile + lane * 16);
     t.q1 = load_stream16(tile + 1024 + lane * 16);
     t.hdr = load_stream16(tile + kTileQBytes + (lane & 15) * 16);
+    if (Q5) t.qh = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(tile + kTileHBytes + lane * 8));
 }
 
 template <int TT>
@@ -38,7 +43,12 @@ __device__ __forceinline__ void load_a(ARegs<TT>& a, const uint8_t* __restrict__
     }
 }
 
-template <int TT>
+// bit `s` of every byte of h, moved to bit 4 of that byte
+__device__ __forceinline__ uint32_t fifth_bits(uint32_t h, int s) {
+    return (s <= 4 ? h << (4 - s) : h >> (s - 4)) & 0x10101010u;
+}
+
+template <int TT, bool Q5 = false>
 __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>& a, float (&acc)[TT][2],
                                              int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2]) {
     // 6-bit scale / min unpack, word-parallel (core/src/kernels/hwy/hwy_moe_quant.cc:90-101)
@@ -57,8 +67,14 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
 #pragma unroll
     for (int c = 0; c < 4; ++c) {  // 64-weight chunk: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles)
         const uint32_t qa = qw[2 * c], qb = qw[2 * c + 1];
-        const v4i b_q = {(int)(qa & 0x0f0f0f0fu), (int)(qb & 0x0f0f0f0fu), (int)((qa >> 4) & 0x0f0f0f0fu),
-                         (int)((qb >> 4) & 0x0f0f0f0fu)};
+        v4i b_q = {(int)(qa & 0x0f0f0f0fu), (int)(qb & 0x0f0f0f0fu), (int)((qa >> 4) & 0x0f0f0f0fu),
+                   (int)((qb >> 4) & 0x0f0f0f0fu)};
+        if (Q5) {  // codes 0..31: the fifth bit of sub-blocks 2c and 2c+1 (core/src/kernels/hwy/hwy_moe_quant.cc:177-200)
+            b_q.x |= (int)fifth_bits(t.qh.x, 2 * c);
+            b_q.y |= (int)fifth_bits(t.qh.y, 2 * c);
+            b_q.z |= (int)fifth_bits(t.qh.x, 2 * c + 1);
+            b_q.w |= (int)fifth_bits(t.qh.y, 2 * c + 1);
+        }
         const int s_lo = (int)((sc[c >> 1] >> (16 * (c & 1))) & 0xffu);
         const int s_hi = (int)((sc[c >> 1] >> (16 * (c & 1) + 8)) & 0xffu);
         // v_perm_b32 replicates one byte of the unpacked mins into all four bytes of the operand

@@ -17,11 +17,14 @@ hipError_t launch_q8k_to_amajor(const void* q8_std, int64_t n, size_t q8_row_byt
 
 // ---- weights.hip -----------------------------------------------------------------------------
 // ggml row layout (rows x nb blocks, row_bytes apart) -> tiled layout, one expert per grid.y.
-hipError_t launch_tile_weights(const uint8_t* raw, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
-                               int64_t n_experts, uint8_t* tiled, size_t tiled_expert_bytes, hipStream_t stream);
-hipError_t launch_untile_weights(const uint8_t* tiled, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
-                                 int64_t n_experts, uint8_t* raw, size_t tiled_expert_bytes, hipStream_t stream);
-hipError_t launch_synth_weights(uint64_t seed, int64_t rows, int64_t nb, int64_t n_experts, uint8_t* tiled,
+// type: kTypeQ4K or kTypeQ5K (ggml_type values).
+hipError_t launch_tile_weights(const uint8_t* raw, int64_t rows, int64_t nb, int type, size_t row_bytes,
+                               size_t expert_bytes, int64_t n_experts, uint8_t* tiled, size_t tiled_expert_bytes,
+                               hipStream_t stream);
+hipError_t launch_untile_weights(const uint8_t* tiled, int64_t rows, int64_t nb, int type, size_t row_bytes,
+                                 size_t expert_bytes, int64_t n_experts, uint8_t* raw, size_t tiled_expert_bytes,
+                                 hipStream_t stream);
+hipError_t launch_synth_weights(uint64_t seed, int64_t rows, int64_t nb, int type, int64_t n_experts, uint8_t* tiled,
                                 size_t tiled_expert_bytes, hipStream_t stream);
 
 // ---- matmul.hip ------------------------------------------------------------------------------
@@ -36,6 +39,7 @@ struct MatmulArgs {
     int64_t n = 0;                 // activation rows (dense mode)
     float* y = nullptr;            // dense: [n][ldy]; grouped: [entry][ldy]
     int64_t ldy = 0;
+    int wtype = 12;                // ggml_type of the weights: 12 (Q4_K) or 13 (Q5_K); gate and up share it
     int rt_per_wg = 1;             // row tiles per workgroup (set by launch_matmul)
     int swiglu = 0;                // 1: y = silu(w0 x) * (w1 x)
     int silu_mode = 0;

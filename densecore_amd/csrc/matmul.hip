@@ -70,8 +70,9 @@ struct Depth {
 // One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
 // waves split the super-blocks of the row.  NMAT == 2: gate and up tiles of the same rows share
 // the activations in registers and meet in silu(gate)*up.
-template <int NMAT, int TT, bool GROUPED, bool DEBUG>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, bool Q5>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
+    constexpr int kTileStride = Q5 ? kTile5Bytes : kTileBytes;
     constexpr int S = Depth<NMAT, TT>::kStages;
     extern __shared__ float red[];  // [W-1][NMAT][TT][2][64]
     const int lane = threadIdx.x & 63;
@@ -130,7 +131,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     }
     const uint8_t* tiles[NMAT];
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) tiles[m] = w[m] + tile_offset(rt, 0, nb);
+    for (int m = 0; m < NMAT; ++m) tiles[m] = w[m] + tile_offset(rt, 0, nb, kTileStride);
 
     for (int chunk = 0; chunk < count; chunk += kTokTile * TT) {
         // activation row behind this lane's A slot, and activation / output rows of its two outputs
@@ -202,14 +203,14 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 const int b = rt_per_wg > 1 ? t % per_rt : t;
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    load_tile(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileBytes : p.aq, lane);
+                    load_tile<Q5>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : p.aq, lane);
                 load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             };
             auto consume = [&](int st, int i) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][2], msum[TT][2];
-                    compute_tile<TT>(ring_t[st][m], ring_a[st], acc[m], dsum, msum);
+                    compute_tile<TT, Q5>(ring_t[st][m], ring_a[st], acc[m], dsum, msum);
                     if (DEBUG && p.dbg_dot) {  // debug launches own one row tile per workgroup
                         const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;
@@ -310,15 +311,15 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     }
 }
 
-template <int NMAT, int TT, bool GROUPED, bool DEBUG>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, bool Q5>
 hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
     if (start && stop) {
         // the events take the dispatch's own begin / end timestamps: no extra packets around the kernel
-        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, start, stop,
+        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, Q5>), grid, dim3(64 * waves), lds, stream, start, stop,
                               0, a);
     } else {
-        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG>), grid, dim3(64 * waves), lds, stream, a);
+        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, Q5>), grid, dim3(64 * waves), lds, stream, a);
     }
     return hipGetLastError();
 }
@@ -345,6 +346,8 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int64_t rowtiles = (a.rows + 15) / 16;
     const int nmat = a.swiglu ? 2 : 1;
     const bool debug = a.dbg_dot != nullptr;
+    const bool q5 = a.wtype == kTypeQ5K;
+    if (a.wtype != kTypeQ4K && a.wtype != kTypeQ5K) return hipErrorInvalidValue;
     // widest activation group this launch can see decides how many 8-row token tiles a pass holds
     const int64_t widest = a.grouped ? (a.n > a.sh_tokens ? a.n : a.sh_tokens) : a.n;
     // Expert groups rarely hold more than 8 rows at decode widths; the few that do (and the shared
@@ -365,9 +368,14 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
 
 #define MQ_LAUNCH(NM, T)                                                              \
     do {                                                                              \
-        if (a.grouped) return launch_one<NM, T, true, false>(b, waves, grid, stream, start, stop); \
-        if (debug) return launch_one<NM, T, false, true>(b, waves, grid, stream, start, stop);     \
-        return launch_one<NM, T, false, false>(b, waves, grid, stream, start, stop);               \
+        if (q5) {                                                                                         \
+            if (a.grouped) return launch_one<NM, T, true, false, true>(b, waves, grid, stream, start, stop); \
+            if (debug) return launch_one<NM, T, false, true, true>(b, waves, grid, stream, start, stop);     \
+            return launch_one<NM, T, false, false, true>(b, waves, grid, stream, start, stop);               \
+        }                                                                                                 \
+        if (a.grouped) return launch_one<NM, T, true, false, false>(b, waves, grid, stream, start, stop);    \
+        if (debug) return launch_one<NM, T, false, true, false>(b, waves, grid, stream, start, stop);        \
+        return launch_one<NM, T, false, false, false>(b, waves, grid, stream, start, stop);                  \
     } while (0)
 
     if (nmat == 1) {

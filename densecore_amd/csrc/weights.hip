@@ -1,6 +1,6 @@
-// Weight re-tiling (ggml block_q4_K rows <-> the 16-row tile layout of common.h) and the
-// on-device synthetic fill.  One thread moves one 8-byte word of a block_q4_K; each such word
-// lands in one contiguous 8-byte slot of a tile (tile_word_offset).
+// Weight re-tiling (ggml block_q4_K / block_q5_K rows <-> the 16-row tile layouts of common.h) and the
+// on-device synthetic fill.  One thread moves one 8-byte word of a block; each such word lands in one
+// contiguous 8-byte slot of a tile (tile_word_offset, tile_word_offset_q5).
 #include "common.h"
 #include "kernels.h"
 
@@ -8,48 +8,54 @@ namespace mq {
 
 namespace {
 
-constexpr int kWordsPerBlock = kQ4Block / 8;  // 18
+// 8-byte words per block: 18 (Q4_K) or 22 (Q5_K)
+__host__ __device__ inline int words_per_block(int type) { return block_bytes_of(type) / 8; }
 
-__device__ __forceinline__ bool decode_word(int64_t idx, int64_t rows, int64_t nb, int64_t& row, int64_t& b,
+__device__ __forceinline__ bool decode_word(int64_t idx, int64_t rows, int64_t nb, int type, int64_t& row, int64_t& b,
                                             int& word) {
-    const int64_t per_row = nb * kWordsPerBlock;
+    const int wpb = words_per_block(type);
+    const int64_t per_row = nb * wpb;
     row = idx / per_row;
     if (row >= rows) return false;
     const int64_t rem = idx - row * per_row;
-    b = rem / kWordsPerBlock;
-    word = (int)(rem - b * kWordsPerBlock);
+    b = rem / wpb;
+    word = (int)(rem - b * wpb);
     return true;
 }
 
+// where word `word` of row r's block lives inside its tile
+__device__ __forceinline__ size_t word_in_tiles(int64_t row, int64_t b, int64_t nb, int word, int type) {
+    return tile_offset(row >> 4, b, nb, tile_bytes_of(type)) +
+           (size_t)(type == kTypeQ5K ? tile_word_offset_q5((int)(row & 15), word) : tile_word_offset((int)(row & 15), word));
+}
+
 __global__ void __launch_bounds__(256) tile_weights_kernel(const uint8_t* __restrict__ raw, int64_t rows, int64_t nb,
-                                                           size_t row_bytes, size_t expert_bytes,
+                                                           int type, size_t row_bytes, size_t expert_bytes,
                                                            uint8_t* __restrict__ tiled, size_t tiled_expert_bytes) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t row, b;
     int word;
-    if (!decode_word(idx, rows, nb, row, b, word)) return;
+    if (!decode_word(idx, rows, nb, type, row, b, word)) return;
     const int64_t e = blockIdx.y;
-    const uint8_t* src = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * kQ4Block + word * 8;
-    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + tile_offset(row >> 4, b, nb) +
-                   tile_word_offset((int)(row & 15), word);
-    // block_q4_K is only 2-byte aligned in general; row_bytes is a multiple of 144 = 8*18 in every
-    // ggml tensor, but go through 2-byte loads to stay correct for odd host strides.
+    const uint8_t* src = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + word * 8;
+    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
+    // the blocks are only 2-byte aligned in general: go through 2-byte loads to stay correct for odd host strides
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(src);
     const uint64_t v = (uint64_t)s16[0] | ((uint64_t)s16[1] << 16) | ((uint64_t)s16[2] << 32) | ((uint64_t)s16[3] << 48);
     *reinterpret_cast<uint64_t*>(dst) = v;
 }
 
 __global__ void __launch_bounds__(256) untile_weights_kernel(const uint8_t* __restrict__ tiled, int64_t rows,
-                                                             int64_t nb, size_t row_bytes, size_t expert_bytes,
-                                                             uint8_t* __restrict__ raw, size_t tiled_expert_bytes) {
+                                                             int64_t nb, int type, size_t row_bytes,
+                                                             size_t expert_bytes, uint8_t* __restrict__ raw,
+                                                             size_t tiled_expert_bytes) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t row, b;
     int word;
-    if (!decode_word(idx, rows, nb, row, b, word)) return;
+    if (!decode_word(idx, rows, nb, type, row, b, word)) return;
     const int64_t e = blockIdx.y;
-    const uint8_t* src = tiled + (size_t)e * tiled_expert_bytes + tile_offset(row >> 4, b, nb) +
-                         tile_word_offset((int)(row & 15), word);
-    uint8_t* dst = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * kQ4Block + word * 8;
+    const uint8_t* src = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
+    uint8_t* dst = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + word * 8;
     const uint64_t v = *reinterpret_cast<const uint64_t*>(src);
     uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
     d16[0] = (uint16_t)v;
@@ -65,52 +71,53 @@ __device__ __forceinline__ uint32_t unit_scale_f16(uint64_t w) {
     return (uint32_t)__half_as_ushort(__float2half_rn(v));
 }
 
-__global__ void __launch_bounds__(256) synth_weights_kernel(uint64_t seed, int64_t rows, int64_t nb,
+__global__ void __launch_bounds__(256) synth_weights_kernel(uint64_t seed, int64_t rows, int64_t nb, int type,
                                                             uint8_t* __restrict__ tiled, size_t tiled_expert_bytes) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t row, b;
     int word;
-    if (!decode_word(idx, rows, nb, row, b, word)) return;
+    if (!decode_word(idx, rows, nb, type, row, b, word)) return;
     const int64_t e = blockIdx.y;
-    // stream position of this word in the flat [expert][row][block][18] order
+    // stream position of this word in the flat [expert][row][block][words per block] order
     const uint64_t flat_block = ((uint64_t)e * (uint64_t)rows + (uint64_t)row) * (uint64_t)nb + (uint64_t)b;
-    const uint64_t pos = flat_block * kWordsPerBlock + (uint64_t)word;
+    const uint64_t pos = flat_block * (uint64_t)words_per_block(type) + (uint64_t)word;
     uint64_t v = mix64(seed + (pos + 1) * kGamma);
     if (word == 0) {
         const uint64_t s0 = mix64((seed ^ kScaleStream) + (flat_block * 2 + 1) * kGamma);
         const uint64_t s1 = mix64((seed ^ kScaleStream) + (flat_block * 2 + 2) * kGamma);
         v = (v & 0xffffffff00000000ull) | (uint64_t)unit_scale_f16(s0) | ((uint64_t)unit_scale_f16(s1) << 16);
     }
-    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + tile_offset(row >> 4, b, nb) +
-                   tile_word_offset((int)(row & 15), word);
+    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
     *reinterpret_cast<uint64_t*>(dst) = v;
 }
 
-inline dim3 word_grid(int64_t rows, int64_t nb, int64_t n_experts) {
-    const int64_t words = rows * nb * kWordsPerBlock;
+inline dim3 word_grid(int64_t rows, int64_t nb, int64_t n_experts, int type) {
+    const int64_t words = rows * nb * words_per_block(type);
     return dim3((unsigned)((words + 255) / 256), (unsigned)n_experts);
 }
 
 }  // namespace
 
-hipError_t launch_tile_weights(const uint8_t* raw, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
-                               int64_t n_experts, uint8_t* tiled, size_t tiled_expert_bytes, hipStream_t stream) {
-    hipLaunchKernelGGL(tile_weights_kernel, word_grid(rows, nb, n_experts), dim3(256), 0, stream, raw, rows, nb,
-                       row_bytes, expert_bytes, tiled, tiled_expert_bytes);
+hipError_t launch_tile_weights(const uint8_t* raw, int64_t rows, int64_t nb, int type, size_t row_bytes,
+                               size_t expert_bytes, int64_t n_experts, uint8_t* tiled, size_t tiled_expert_bytes,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(tile_weights_kernel, word_grid(rows, nb, n_experts, type), dim3(256), 0, stream, raw, rows, nb,
+                       type, row_bytes, expert_bytes, tiled, tiled_expert_bytes);
     return hipGetLastError();
 }
 
-hipError_t launch_untile_weights(const uint8_t* tiled, int64_t rows, int64_t nb, size_t row_bytes, size_t expert_bytes,
-                                 int64_t n_experts, uint8_t* raw, size_t tiled_expert_bytes, hipStream_t stream) {
-    hipLaunchKernelGGL(untile_weights_kernel, word_grid(rows, nb, n_experts), dim3(256), 0, stream, tiled, rows, nb,
-                       row_bytes, expert_bytes, raw, tiled_expert_bytes);
+hipError_t launch_untile_weights(const uint8_t* tiled, int64_t rows, int64_t nb, int type, size_t row_bytes,
+                                 size_t expert_bytes, int64_t n_experts, uint8_t* raw, size_t tiled_expert_bytes,
+                                 hipStream_t stream) {
+    hipLaunchKernelGGL(untile_weights_kernel, word_grid(rows, nb, n_experts, type), dim3(256), 0, stream, tiled, rows, nb,
+                       type, row_bytes, expert_bytes, raw, tiled_expert_bytes);
     return hipGetLastError();
 }
 
-hipError_t launch_synth_weights(uint64_t seed, int64_t rows, int64_t nb, int64_t n_experts, uint8_t* tiled,
+hipError_t launch_synth_weights(uint64_t seed, int64_t rows, int64_t nb, int type, int64_t n_experts, uint8_t* tiled,
                                 size_t tiled_expert_bytes, hipStream_t stream) {
-    hipLaunchKernelGGL(synth_weights_kernel, word_grid(rows, nb, n_experts), dim3(256), 0, stream, seed, rows, nb,
-                       tiled, tiled_expert_bytes);
+    hipLaunchKernelGGL(synth_weights_kernel, word_grid(rows, nb, n_experts, type), dim3(256), 0, stream, seed, rows, nb,
+                       type, tiled, tiled_expert_bytes);
     return hipGetLastError();
 }
 

@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .synth import Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
+from .synth import BLOCK_BYTES, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
 
 SILU_EXACT, SILU_FAST, SILU_FAST_FMA = 0, 1, 2
 ROUTE_FUSED, ROUTE_FLOOR, ROUTE_FLOOR_FINITE = 0, 1, 2
@@ -35,31 +35,37 @@ class Q4KWeight:
     """Device-resident Q4_K matrix or expert stack (GgmlQuantizedMatrixView's weight side,
     core/include/densecore/backend/cpu_backend.h:91-99)."""
 
-    def __init__(self, handle: int, rows: int, cols: int, n_experts: int):
+    def __init__(self, handle: int, rows: int, cols: int, n_experts: int, ggml_type: int = GGML_TYPE_Q4_K):
         self._h = C.c_void_p(handle)
-        self.rows, self.cols, self.n_experts = rows, cols, n_experts
+        self.rows, self.cols, self.n_experts, self.ggml_type = rows, cols, n_experts, ggml_type
+
+    @property
+    def block_bytes(self) -> int:
+        return BLOCK_BYTES[self.ggml_type]
 
     @classmethod
-    def from_ggml(cls, data: np.ndarray, cols: int) -> "Q4KWeight":
-        """data: uint8 [rows, row_bytes] or [n_experts, rows, row_bytes] in ggml block_q4_K row layout."""
+    def from_ggml(cls, data: np.ndarray, cols: int, ggml_type: int = GGML_TYPE_Q4_K) -> "Q4KWeight":
+        """data: uint8 [rows, row_bytes] or [n_experts, rows, row_bytes] in ggml block_q4_K (type 12) or
+        block_q5_K (type 13) row layout."""
         a = np.ascontiguousarray(data, dtype=np.uint8)
         if a.ndim == 2:
             a = a[None]
         e, rows, row_bytes = a.shape
         h = C.c_void_p()
-        _lib.check(_lib.lib().mq_weight_upload(C.c_void_p(a.ctypes.data), rows, cols, e, row_bytes, rows * row_bytes,
-                                               C.byref(h)), "mq_weight_upload")
-        return cls(h.value, rows, cols, e)
+        _lib.check(_lib.lib().mq_weight_upload_typed(ggml_type, C.c_void_p(a.ctypes.data), rows, cols, e, row_bytes,
+                                                     rows * row_bytes, C.byref(h)), "mq_weight_upload_typed")
+        return cls(h.value, rows, cols, e, ggml_type)
 
     @classmethod
-    def synthetic(cls, seed: int, rows: int, cols: int, n_experts: int = 1) -> "Q4KWeight":
+    def synthetic(cls, seed: int, rows: int, cols: int, n_experts: int = 1,
+                  ggml_type: int = GGML_TYPE_Q4_K) -> "Q4KWeight":
         h = C.c_void_p()
-        _lib.check(_lib.lib().mq_weight_synthetic(C.c_uint64(seed & 0xFFFFFFFFFFFFFFFF), rows, cols, n_experts,
-                                                  C.byref(h)), "mq_weight_synthetic")
-        return cls(h.value, rows, cols, n_experts)
+        _lib.check(_lib.lib().mq_weight_synthetic_typed(ggml_type, C.c_uint64(seed & 0xFFFFFFFFFFFFFFFF), rows, cols,
+                                                        n_experts, C.byref(h)), "mq_weight_synthetic_typed")
+        return cls(h.value, rows, cols, n_experts, ggml_type)
 
     def to_ggml(self) -> np.ndarray:
-        row_bytes = self.cols // QK_K * Q4K_BLOCK_BYTES
+        row_bytes = self.cols // QK_K * self.block_bytes
         out = np.zeros((self.n_experts, self.rows, row_bytes), np.uint8)
         _lib.check(_lib.lib().mq_weight_download(self._h, C.c_void_p(out.ctypes.data), row_bytes,
                                                  self.rows * row_bytes), "mq_weight_download")
@@ -67,7 +73,7 @@ class Q4KWeight:
 
     @property
     def ggml_bytes(self) -> int:
-        return self.n_experts * self.rows * (self.cols // QK_K) * Q4K_BLOCK_BYTES
+        return self.n_experts * self.rows * (self.cols // QK_K) * self.block_bytes
 
     def free(self) -> None:
         if self._h:

@@ -21,7 +21,11 @@ import numpy as np
 
 QK_K = 256
 Q4K_BLOCK_BYTES = 144
+Q5K_BLOCK_BYTES = 176
 Q8K_BLOCK_BYTES = 292
+GGML_TYPE_Q4_K = 12
+GGML_TYPE_Q5_K = 13
+BLOCK_BYTES = {GGML_TYPE_Q4_K: Q4K_BLOCK_BYTES, GGML_TYPE_Q5_K: Q5K_BLOCK_BYTES}
 
 _GAMMA = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -71,6 +75,25 @@ def q4k_blocks(seed: int, n_blocks: int, first_block: int = 0) -> np.ndarray:
     raw[:, 0:2] = unit_scale_f16(sw[:, 0]).view(np.uint8).reshape(n_blocks, 2)
     raw[:, 2:4] = unit_scale_f16(sw[:, 1]).view(np.uint8).reshape(n_blocks, 2)
     return raw
+
+
+def q5k_blocks(seed: int, n_blocks: int, first_block: int = 0) -> np.ndarray:
+    """``[n_blocks, 176]`` uint8 array of seeded Q5_K super-blocks: the Q4_K recipe over 22 words a block
+    (d, dmin, scales[12], qh[32], qs[128]; core/src/kernels/hwy/hwy_moe_quant.cc:36-45)."""
+    words = stream_u64(seed, first_block * 22, n_blocks * 22).reshape(n_blocks, 22)
+    raw = words.view(np.uint8).reshape(n_blocks, Q5K_BLOCK_BYTES).copy()
+    sw = stream_u64(seed ^ 0x5CA1E5CA1E5CA1E5, first_block * 2, n_blocks * 2).reshape(n_blocks, 2)
+    raw[:, 0:2] = unit_scale_f16(sw[:, 0]).view(np.uint8).reshape(n_blocks, 2)
+    raw[:, 2:4] = unit_scale_f16(sw[:, 1]).view(np.uint8).reshape(n_blocks, 2)
+    return raw
+
+
+def q5k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:
+    """Row-major Q5_K matrix ``[rows, cols/256 * 176]`` uint8 (ggml row layout)."""
+    if cols % QK_K:
+        raise ValueError("cols must be a multiple of 256")
+    nb = cols // QK_K
+    return q5k_blocks(seed, rows * nb).reshape(rows, nb * Q5K_BLOCK_BYTES)
 
 
 def q4k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:

@@ -433,3 +433,82 @@ def test_weights_from_ids_agree_with_router_and_double_softmax():
     # arbitrary (unsorted) ids: any permutation of the selection gives the permuted weights up to summation order
     perm = rng.permutation(8)
     np.testing.assert_allclose(orc.route_weights_from_ids(logits, ids[:, perm]), w[:, perm], rtol=1e-6)
+
+
+# ----------------------------------------------------------------- Q5_K weights
+def np_unpack_q5k(w):
+    """Independent decode of block_q5_K rows, from the published format: the Q4_K fields with 32 qh bytes
+    between the packed scales and the nibbles; bit s of qh[l] is worth 16 in element l of sub-block s."""
+    b = w.reshape(-1, 176)
+    as_q4 = np.concatenate([b[:, 0:16], b[:, 48:176]], axis=1)
+    d, dmin, sc, mn, q = np_unpack_q4k(as_q4)
+    qh = b[:, 16:48].astype(np.int64)                                        # [blk, l]
+    hi = (qh[:, None, :] >> np.arange(8)[None, :, None]) & 1                 # [blk, s, l]
+    return d, dmin, sc, mn, q + 16 * hi.reshape(-1, 256)
+
+
+def test_q5k_layout_and_zero_high_bits_reduce_to_q4k():
+    assert orc.lib().orc_q5k_block_bytes() == 176
+    cols = 1024
+    w4 = synth.q4k_matrix(301, 12, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(302, (3, cols)))
+    w5 = orc.q5k_from_q4k(w4)
+    ds4, md4 = orc.matrix_block_sums(w4, cols, q8)
+    ds5, md5 = orc.q5k_matrix_block_sums(w5, cols, q8)
+    assert np.array_equal(ds4, ds5) and np.array_equal(md4, md5)
+    for order in (orc.ORDER_HWY, orc.ORDER_DOTPROD):
+        assert np.array_equal(orc.mul_mat_q4k_q8k(w4, cols, q8, order), orc.mul_mat_q5k_q8k(w5, cols, q8, order))
+
+
+def test_q5k_all_high_bits_closed_form_and_single_bit_placement():
+    """Every qh bit set adds 16 * scale_s * (sum of sub-block s of the activations), which the Q8_K block
+    carries as bsums; one set bit adds 16 * scale_s * y[32 s + l] and nothing else."""
+    cols = 512
+    w4 = synth.q4k_matrix(311, 6, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(312, (2, cols)))
+    ds4, md4 = orc.matrix_block_sums(w4, cols, q8)
+    full = orc.q5k_from_q4k(w4, np.full((6, 2, 32), 0xFF, np.uint8))
+    ds5, md5 = orc.q5k_matrix_block_sums(full, cols, q8)
+    _, _, sc, _, _ = np_unpack_q4k(w4)
+    _, yq, ybs = orc.split_q8k(q8)
+    sub = ybs.astype(np.int64).reshape(2, 2, 8, 2).sum(axis=3)               # [m, b, s]
+    extra = 16 * np.einsum("rbs,mbs->rmb", sc.reshape(6, 2, 8), sub)
+    assert np.array_equal(ds5, ds4 + extra) and np.array_equal(md5, md4)
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        r, b, s, l = (int(rng.integers(0, n)) for n in (6, 2, 8, 32))
+        qh = np.zeros((6, 2, 32), np.uint8)
+        qh[r, b, l] = 1 << s
+        ds1, _ = orc.q5k_matrix_block_sums(orc.q5k_from_q4k(w4, qh), cols, q8)
+        want = ds4.copy()
+        want[r, :, b] += 16 * sc.reshape(6, 2, 8)[r, b, s] * yq.reshape(2, 2, 256)[:, b, 32 * s + l].astype(np.int64)
+        assert np.array_equal(ds1, want)
+
+
+def test_q5k_sums_brute_force_and_fp32_against_double():
+    cols = 2048
+    w = synth.q5k_matrix(321, 20, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(322, (3, cols)))
+    d, dmin, sc, mn, q = np_unpack_q5k(w)
+    assert q.min() == 0 and q.max() == 31
+    nb = cols // 256
+    _, yq, _ = orc.split_q8k(q8)
+    yq = yq.astype(np.int64).reshape(3, nb, 8, 32)
+    sub = np.einsum("rbgi,mbgi->rmbg", q.reshape(20, nb, 8, 32), yq)
+    bds = np.einsum("rmbg,rbg->rmb", sub, sc.reshape(20, nb, 8))
+    bmd = np.einsum("mbg,rbg->rmb", yq.sum(axis=3), mn.reshape(20, nb, 8))
+    ds, md = orc.q5k_matrix_block_sums(w, cols, q8)
+    assert np.array_equal(ds, bds) and np.array_equal(md, bmd)
+    # dequantize in numpy, dot in double
+    wq = d[:, None, None] * sc[:, :, None] * q.reshape(-1, 8, 32) - dmin[:, None, None] * mn[:, :, None]
+    yd, yq8, _ = orc.split_q8k(q8)
+    act = (yd[..., None].astype(np.float64) * yq8).reshape(3, cols)
+    want = act @ wq.reshape(20, cols).T
+    ref = orc.q5k_dot_dequant_f64(w, cols, q8)
+    assert np.allclose(ref, want, rtol=1e-12, atol=1e-12)
+    mag = orc.q5k_dot_dequant_f64(w, cols, q8, magnitude=True)
+    for order in (orc.ORDER_HWY, orc.ORDER_DOTPROD):
+        got = orc.mul_mat_q5k_q8k(w, cols, q8, order).astype(np.float64)
+        assert np.max(np.abs(got - ref) / mag) < 2e-6
+        ok = np.abs(ref) > 1e-3 * mag
+        assert np.max(np.abs(got - ref)[ok] / np.abs(ref)[ok]) < 1e-4
