@@ -22,7 +22,7 @@ EXPORTS = [
     "mq_matmul_ggml_quantized_transb",
 ]
 
-GGML_TYPE_F32, GGML_TYPE_Q4_K, GGML_TYPE_I32 = 0, 12, 26
+GGML_TYPE_F32, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_I32 = 0, 12, 13, 26
 GGML_OP_CUSTOM_PLACEHOLDER = 0  # the adapters never read dst->op
 
 
@@ -69,8 +69,9 @@ def tensor(array: np.ndarray, ggml_type: int, ne, nb=None, name: bytes = b"") ->
     t.type = ggml_type
     ne = list(ne) + [1] * (4 - len(ne))
     if nb is None:
-        if ggml_type == GGML_TYPE_Q4_K:
-            nb = [144, 144 * (ne[0] // 256)]
+        if ggml_type in (GGML_TYPE_Q4_K, GGML_TYPE_Q5_K):
+            bb = 144 if ggml_type == GGML_TYPE_Q4_K else 176
+            nb = [bb, bb * (ne[0] // 256)]
         else:
             nb = [4, 4 * ne[0]]
         while len(nb) < 4:

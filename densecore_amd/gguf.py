@@ -12,10 +12,10 @@ from . import _lib, ggml_adapter, ops
 
 EXPORTS = [
     "mq_gguf_open", "mq_gguf_last_error", "mq_gguf_close", "mq_gguf_tensor_count", "mq_gguf_tensor_at",
-    "mq_gguf_find_tensor", "mq_gguf_get_int", "mq_gguf_get_string", "mq_gguf_load_q4k",
+    "mq_gguf_find_tensor", "mq_gguf_get_int", "mq_gguf_get_string", "mq_gguf_load_q4k", "mq_gguf_load_weight",
 ]
 
-GGML_F32, GGML_F16, GGML_Q4_K, GGML_I32 = 0, 1, 12, 26
+GGML_F32, GGML_F16, GGML_Q4_K, GGML_Q5_K, GGML_I32 = 0, 1, 12, 13, 26
 
 
 class TensorInfo(C.Structure):
@@ -43,6 +43,7 @@ def lib(need_gpu: bool = False):
         L.mq_gguf_get_int.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64)]
         L.mq_gguf_get_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t)]
         L.mq_gguf_load_q4k.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        L.mq_gguf_load_weight.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
         _handle = L
     if need_gpu:
         _lib.lib()
@@ -93,17 +94,24 @@ class GgufFile:
 
     def load_q4k(self, name: str) -> "ops.Q4KWeight":
         """Upload a GGML_TYPE_Q4_K tensor ([K, N] or [K, N, E]) to the GPU."""
+        return self._load(name, "mq_gguf_load_q4k")
+
+    def load_weight(self, name: str) -> "ops.Q4KWeight":
+        """Upload a GGML_TYPE_Q4_K or GGML_TYPE_Q5_K tensor ([K, N] or [K, N, E]) to the GPU."""
+        return self._load(name, "mq_gguf_load_weight")
+
+    def _load(self, name: str, entry: str) -> "ops.Q4KWeight":
         lib(need_gpu=True)
         idx = self.find(name)
         if idx < 0:
             raise KeyError(name)
         t = self.tensors()[idx]
         h = C.c_void_p()
-        rc = lib().mq_gguf_load_q4k(self._h, name.encode(), C.byref(h))
+        rc = getattr(lib(), entry)(self._h, name.encode(), C.byref(h))
         if rc != 0:
-            _lib.check(rc, f"mq_gguf_load_q4k({name}): {lib().mq_gguf_last_error().decode()}")
+            _lib.check(rc, f"{entry}({name}): {lib().mq_gguf_last_error().decode()}")
         ne = t["ne"] + [1] * (3 - len(t["ne"]))
-        return ops.Q4KWeight(h.value, ne[1], ne[0], ne[2])
+        return ops.Q4KWeight(h.value, ne[1], ne[0], ne[2], t["type"])
 
 
 # ------------------------------------------------------------------------------------------ writer

@@ -18,6 +18,11 @@ namespace {
 
 constexpr int64_t kSuperBlock = 256;
 constexpr size_t kQ4KBlockBytes = 144;
+constexpr size_t kQ5KBlockBytes = 176;
+// block bytes of a weight type this library multiplies, 0 for any other
+constexpr size_t kquant_block_bytes(int type) {
+    return type == (int)GGML_TYPE_Q4_K ? kQ4KBlockBytes : type == (int)GGML_TYPE_Q5_K ? kQ5KBlockBytes : 0;
+}
 
 thread_local int t_status = MQ_OK;
 
@@ -31,40 +36,46 @@ int note(int rc) {
 // arena which reuses an address for another tensor is re-uploaded rather than mis-read.
 struct CachedWeight {
     mq_weight* handle = nullptr;
+    int type = -1;
     int64_t ne[3] = {0, 0, 0};
     size_t nb[3] = {0, 0, 0};
 };
 std::mutex g_cache_mu;
 std::unordered_map<const void*, CachedWeight> g_cache;
 
-bool is_q4k_matrix(const ggml_tensor* w) {
-    return w && w->data && w->type == GGML_TYPE_Q4_K && w->ne[0] > 0 && w->ne[0] % kSuperBlock == 0 && w->ne[1] > 0 &&
-           w->ne[2] > 0 && w->ne[3] == 1 && w->nb[0] == kQ4KBlockBytes &&
-           w->nb[1] >= (size_t)(w->ne[0] / kSuperBlock) * kQ4KBlockBytes;
+// Q4_K or Q5_K rows of whole super-blocks (the two weight types of the callbacks replaced:
+// core/src/llm/moe/native.cpp:2745-2752 accepts exactly these for the expert stacks)
+bool is_kquant_matrix(const ggml_tensor* w) {
+    if (!w || !w->data) return false;
+    const size_t bb = kquant_block_bytes((int)w->type);
+    return bb != 0 && w->ne[0] > 0 && w->ne[0] % kSuperBlock == 0 && w->ne[1] > 0 && w->ne[2] > 0 && w->ne[3] == 1 &&
+           w->nb[0] == bb && w->nb[1] >= (size_t)(w->ne[0] / kSuperBlock) * bb;
 }
 
-const mq_weight* device_weight(const void* data, int64_t cols, int64_t rows, int64_t n_experts, size_t row_bytes,
-                               size_t expert_bytes) {
+const mq_weight* device_weight(const void* data, int type, int64_t cols, int64_t rows, int64_t n_experts,
+                               size_t row_bytes, size_t expert_bytes) {
     std::lock_guard<std::mutex> lock(g_cache_mu);
     CachedWeight& slot = g_cache[data];
-    const bool same = slot.handle && slot.ne[0] == cols && slot.ne[1] == rows && slot.ne[2] == n_experts &&
+    const bool same = slot.handle && slot.type == type && slot.ne[0] == cols && slot.ne[1] == rows && slot.ne[2] == n_experts &&
                       slot.nb[1] == row_bytes && slot.nb[2] == expert_bytes;
     if (same) return slot.handle;
     if (slot.handle) mq_weight_free(slot.handle);
     slot = CachedWeight{};
     mq_weight* h = nullptr;
-    if (note(mq_weight_upload(data, rows, cols, n_experts, row_bytes, expert_bytes, &h)) != MQ_OK) {
+    if (note(mq_weight_upload_typed(type, data, rows, cols, n_experts, row_bytes, expert_bytes, &h)) != MQ_OK) {
         g_cache.erase(data);
         return nullptr;
     }
     slot.handle = h;
+    slot.type = type;
     slot.ne[0] = cols, slot.ne[1] = rows, slot.ne[2] = n_experts;
     slot.nb[1] = row_bytes, slot.nb[2] = expert_bytes;
     return h;
 }
 
 const mq_weight* device_weight(const ggml_tensor* w) {
-    return device_weight(w->data, w->ne[0], w->ne[1], w->ne[2], w->nb[1], w->ne[2] > 1 ? w->nb[2] : w->nb[1] * w->ne[1]);
+    return device_weight(w->data, (int)w->type, w->ne[0], w->ne[1], w->ne[2], w->nb[1],
+                         w->ne[2] > 1 ? w->nb[2] : w->nb[1] * w->ne[1]);
 }
 
 // ---- per-thread staging in HBM -------------------------------------------------------------------
@@ -149,7 +160,7 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
     const ggml_tensor* weight = dst->src[1];
     Options o = options_for(userdata, 1);
     if (!src || !weight || !src->data || !dst->data) return finish(o, MQ_ERR_INVALID);
-    if (!is_q4k_matrix(weight) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
+    if (!is_kquant_matrix(weight) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t k_in = weight->ne[0], n_out = weight->ne[1];
     const int64_t m = src->ne[1] * src->ne[2] * src->ne[3];
     // the reference leaves dst untouched on a shape mismatch (core/src/llm/matmul/gemv_exec.cpp:131-143)
@@ -201,7 +212,7 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
     const ggml_tensor* sel = dst->src[3];
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
     if (!gate || !up || !input || !sel || !input->data || !sel->data || !dst->data) return finish(o, MQ_ERR_INVALID);
-    if (!is_q4k_matrix(gate) || !is_q4k_matrix(up)) return finish(o, MQ_ERR_UNSUPPORTED);
+    if (!is_kquant_matrix(gate) || !is_kquant_matrix(up) || gate->type != up->type) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t n_embd = gate->ne[0], n_ff = gate->ne[1], n_expert = gate->ne[2];
     const int64_t top_k = sel->ne[0], n = sel->ne[1];
     // operand checks of core/src/llm/moe/native.cpp:3935-3990
@@ -243,7 +254,7 @@ void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int /*nth*
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
     if (!down || !hidden || !sel || !logits || !hidden->data || !sel->data || !logits->data || !dst->data)
         return finish(o, MQ_ERR_INVALID);
-    if (!is_q4k_matrix(down)) return finish(o, MQ_ERR_UNSUPPORTED);
+    if (!is_kquant_matrix(down)) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t n_ff = down->ne[0], n_embd = down->ne[1], n_expert = down->ne[2];
     const int64_t top_k = sel->ne[0], n = sel->ne[1];
     // operand checks of core/src/llm/moe/native.cpp:3060-3120 and :2309-2317
@@ -299,14 +310,14 @@ int mq_matmul_ggml_quantized_transb(const float* a, int64_t m, int64_t k, int64_
                                     int32_t w_type_id, int64_t w_rows, int64_t w_cols, size_t w_row_bytes, float* c,
                                     int64_t ldc) {
     // rejection rules of MatMulGgmlQuantizedTransBWithPath
-    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K
+    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K and Q5_K
     if (!a || !w_data || !c || m <= 0 || w_rows <= 0 || w_cols <= 0 || k != w_cols || lda < k || ldc < w_rows ||
-        w_type_id != (int32_t)GGML_TYPE_Q4_K || w_cols % kSuperBlock != 0 ||
-        w_row_bytes != (size_t)(w_cols / kSuperBlock) * kQ4KBlockBytes) {
+        kquant_block_bytes(w_type_id) == 0 || w_cols % kSuperBlock != 0 ||
+        w_row_bytes != (size_t)(w_cols / kSuperBlock) * kquant_block_bytes(w_type_id)) {
         note(MQ_ERR_INVALID);
         return 0;
     }
-    const mq_weight* w = device_weight(w_data, w_cols, w_rows, 1, w_row_bytes, w_row_bytes * (size_t)w_rows);
+    const mq_weight* w = device_weight(w_data, w_type_id, w_cols, w_rows, 1, w_row_bytes, w_row_bytes * (size_t)w_rows);
     if (!w) return 0;
     return note(mq_mul_mat_q4k_host(w, a, m, lda, c, ldc)) == MQ_OK ? 1 : 0;
 }

@@ -265,15 +265,22 @@ int mq_gguf_get_string(const mq_gguf* g, const char* key, const char** out, size
     return MQ_OK;
 }
 
-int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out) {
+namespace {
+int load_kquant(const mq_gguf* g, const char* name, bool q4k_only, mq_weight** out) {
     if (!g || !name || !out) return fail("null argument");
     const int64_t idx = mq_gguf_find_tensor(g, name);
     if (idx < 0) return fail(std::string("no tensor ") + name);
     const mq_gguf_tensor& t = g->tensors[(size_t)idx];
-    if (t.ggml_type != 12) return fail(std::string("tensor ") + name + " is not GGML_TYPE_Q4_K");
+    if (t.ggml_type != 12 && (q4k_only || t.ggml_type != 13))
+        return fail(std::string("tensor ") + name + (q4k_only ? " is not GGML_TYPE_Q4_K" : " is neither GGML_TYPE_Q4_K nor GGML_TYPE_Q5_K"));
     if (t.n_dims > 3 || t.ne[3] != 1) return fail(std::string("tensor ") + name + " has more than three dimensions");
-    const size_t row_bytes = (size_t)(t.ne[0] / 256) * 144;
-    return mq_weight_upload(t.data, t.ne[1], t.ne[0], t.ne[2], row_bytes, row_bytes * (size_t)t.ne[1], out);
+    const size_t row_bytes = (size_t)(t.ne[0] / 256) * (t.ggml_type == 12 ? 144 : 176);
+    return mq_weight_upload_typed(t.ggml_type, t.data, t.ne[1], t.ne[0], t.ne[2], row_bytes, row_bytes * (size_t)t.ne[1], out);
 }
+}  // namespace
+
+int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out) { return load_kquant(g, name, true, out); }
+
+int mq_gguf_load_weight(const mq_gguf* g, const char* name, mq_weight** out) { return load_kquant(g, name, false, out); }
 
 }  // extern "C"

@@ -19,6 +19,7 @@ def _write(tmp_path, alignment=32, version=3):
     f32 = rng.normal(size=(3, 8)).astype(np.float32)
     q2 = synth.q4k_matrix(11, 48, 512)                                   # [K=512, N=48]
     q3 = np.stack([synth.q4k_matrix(20 + e, 32, 256) for e in range(4)])   # [K=256, N=32, E=4]
+    q5 = np.stack([synth.q5k_matrix(30 + e, 16, 512) for e in range(3)])   # [K=512, N=16, E=3], Q5_K
     path = str(tmp_path / f"model_a{alignment}_v{version}.gguf")
     gguf.write_gguf(path, {
         "general.architecture": ("str", "qwen35moe"),
@@ -34,13 +35,14 @@ def _write(tmp_path, alignment=32, version=3):
         ("token_embd.weight", gguf.GGML_F32, [8, 3], f32),
         ("blk.0.attn_q.weight", gguf.GGML_Q4_K, [512, 48], q2),
         ("blk.0.ffn_gate_exps.weight", gguf.GGML_Q4_K, [256, 32, 4], q3),
+        ("blk.0.ffn_down_exps.weight", gguf.GGML_Q5_K, [512, 16, 3], q5),
     ], alignment=alignment, version=version)
-    return path, f32, q2, q3
+    return path, f32, q2, q3, q5
 
 
 @pytest.mark.parametrize("alignment,version", [(32, 3), (64, 2), (4096, 3)])
 def test_metadata_and_tensor_table(tmp_path, alignment, version):
-    path, f32, q2, q3 = _write(tmp_path, alignment, version)
+    path, f32, q2, q3, q5 = _write(tmp_path, alignment, version)
     with gguf.GgufFile(path) as g:
         assert g.get_string("general.architecture") == "qwen35moe"
         assert g.get_int("qwen35moe.block_count") == 40 and g.get_int("qwen35moe.expert_used_count") == 8
@@ -50,14 +52,16 @@ def test_metadata_and_tensor_table(tmp_path, alignment, version):
         with pytest.raises(KeyError):
             g.get_string("missing.key")
         ts = g.tensors()
-        assert [t["name"] for t in ts] == ["token_embd.weight", "blk.0.attn_q.weight", "blk.0.ffn_gate_exps.weight"]
-        assert [t["ne"] for t in ts] == [[8, 3], [512, 48], [256, 32, 4]]
-        assert [t["nbytes"] for t in ts] == [96, 48 * 2 * 144, 4 * 32 * 144]
+        assert [t["name"] for t in ts] == ["token_embd.weight", "blk.0.attn_q.weight", "blk.0.ffn_gate_exps.weight",
+                                           "blk.0.ffn_down_exps.weight"]
+        assert [t["ne"] for t in ts] == [[8, 3], [512, 48], [256, 32, 4], [512, 16, 3]]
+        assert [t["type"] for t in ts] == [0, 12, 12, 13]
+        assert [t["nbytes"] for t in ts] == [96, 48 * 2 * 144, 4 * 32 * 144, 3 * 16 * 2 * 176]
         assert all(t["offset"] % alignment == 0 for t in ts)
         assert g.find("blk.0.attn_q.weight") == 1 and g.find("nope") == -1
         # the data pointers address the very bytes that were written
         import ctypes
-        for t, ref in zip(ts, (f32, q2, q3)):
+        for t, ref in zip(ts, (f32, q2, q3, q5)):
             assert ctypes.string_at(t["data"], t["nbytes"]) == ref.tobytes()
 
 
@@ -96,12 +100,25 @@ def test_q4k_tensors_upload_and_multiply(tmp_path):
     from densecore_amd import ops
     from oracle import binding as orc
     from tests._parity import assert_fp32_parity
-    path, _, q2, q3 = _write(tmp_path)
+    path, _, q2, q3, q5 = _write(tmp_path)
     with gguf.GgufFile(path) as g:
         w2 = g.load_q4k("blk.0.attn_q.weight")
-        w3 = g.load_q4k("blk.0.ffn_gate_exps.weight")
+        w3 = g.load_weight("blk.0.ffn_gate_exps.weight")
+        w5 = g.load_weight("blk.0.ffn_down_exps.weight")
         with pytest.raises(Exception):
             g.load_q4k("token_embd.weight")            # F32: not this path
+        with pytest.raises(Exception):
+            g.load_q4k("blk.0.ffn_down_exps.weight")   # Q5_K through the Q4_K-only entry
+    assert (w5.rows, w5.cols, w5.n_experts, w5.ggml_type) == (16, 512, 3, 13) and np.array_equal(w5.to_ggml(), q5)
+    xk = synth.normal_f32(6, (2, 3, 512))
+    ids = np.array([[0, 1, 2], [2, 2, 0]], np.int32)
+    yk = ops.mul_mat_id(w5, torch.from_numpy(xk).cuda(), torch.from_numpy(ids).cuda()).cpu().numpy()
+    for t in range(2):
+        for k in range(3):
+            q8 = orc.quantize_rows_q8k(xk[t, k][None])
+            assert_fp32_parity(yk[t, k][None], orc.mul_mat_q5k_q8k(q5[ids[t, k]], 512, q8),
+                               orc.q5k_dot_dequant_f64(q5[ids[t, k]], 512, q8, magnitude=True))
+    w5.free()
     assert (w2.rows, w2.cols, w2.n_experts) == (48, 512, 1) and (w3.rows, w3.cols, w3.n_experts) == (32, 256, 4)
     assert np.array_equal(w2.to_ggml(), q2) and np.array_equal(w3.to_ggml(), q3)
     x = synth.normal_f32(5, (3, 512))

@@ -106,6 +106,49 @@ def test_moe_nodes(ga, n):
     np.testing.assert_allclose(y, ref_y, rtol=2e-4, atol=2e-4 * np.abs(ref_y).max())
 
 
+def test_moe_down_node_with_q5k_experts_and_q5k_dense_node(ga):
+    """The down callback replaced is the reference's Q5_K one (cb_qwen35_native_moe_down_q5k_weighted_logits,
+    core/src/llm/moe/native.cpp:3051): Q5_K expert stacks and Q5_K dense weights go through the same nodes."""
+    n, hidden, inter, n_exp, top_k = 3, 512, 256, 6, 2
+    down = np.stack([synth.q5k_matrix(2130 + e, hidden, inter) for e in range(n_exp)])
+    hid = synth.normal_f32(2131, (n, top_k, inter))
+    logits = synth.normal_f32(2132, (n, n_exp))
+    ids, _ = orc.route_topk(logits, top_k, 1)
+    y = np.zeros((n, hidden), np.float32)
+    td = ga.tensor(down, ga.GGML_TYPE_Q5_K, [inter, hidden, n_exp])
+    th = ga.tensor(hid, ga.GGML_TYPE_F32, [inter, top_k, n])
+    ts = ga.tensor(ids, ga.GGML_TYPE_I32, [top_k, n])
+    tl = ga.tensor(logits, ga.GGML_TYPE_F32, [n_exp, n])
+    ty = ga.tensor(y, ga.GGML_TYPE_F32, [hidden, n])
+    ga.set_src(ty, td, th, ts, tl)
+    ga.lib().mq_cb_moe_down_weighted_logits(C.byref(ty), 0, 8, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    w_ref = orc.route_weights_from_ids(logits, ids)
+    want = np.zeros((n, hidden))
+    for t in range(n):
+        for k in range(top_k):
+            want[t] += np.float64(w_ref[t, k]) * orc.mul_mat_q5k_f32(down[ids[t, k]], inter, hid[t, k][None])[0]
+    np.testing.assert_allclose(y, want, rtol=2e-4, atol=2e-4 * np.abs(want).max())
+    # dense node
+    rows, cols, m = 96, 768, 2
+    w = synth.q5k_matrix(2140, rows, cols)
+    x = synth.normal_f32(2141, (m, cols))
+    out = np.zeros((m, rows), np.float32)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q5_K, [cols, rows])
+    tx = ga.tensor(x, ga.GGML_TYPE_F32, [cols, m])
+    to = ga.tensor(out, ga.GGML_TYPE_F32, [rows, m])
+    ga.set_src(to, tx, tw)
+    ga.lib().mq_cb_gemv_batched_custom(C.byref(to), 0, 1, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    q8 = orc.quantize_rows_q8k(x)
+    assert_fp32_parity(out, orc.mul_mat_q5k_q8k(w, cols, q8), orc.q5k_dot_dequant_f64(w, cols, q8, magnitude=True))
+    # library level
+    c = np.zeros((m, rows), np.float32)
+    assert ga.lib().mq_matmul_ggml_quantized_transb(x.ctypes.data, m, cols, cols, w.ctypes.data, ga.GGML_TYPE_Q5_K, rows,
+                                                    cols, 176 * (cols // 256), c.ctypes.data, rows) == 1
+    assert np.array_equal(c.view(np.uint32), out.view(np.uint32))
+
+
 def test_library_level_matmul(ga):
     m, rows, cols = 7, 384, 768
     w = synth.q4k_matrix(301, rows, cols)
@@ -115,6 +158,6 @@ def test_library_level_matmul(ga):
                                                   cols, 144 * (cols // 256), c.ctypes.data, rows)
     assert ok == 1
     assert_fp32_parity(c, _dense_ref(w, cols, a), orc.dot_magnitude_f64(w, cols, orc.quantize_rows_q8k(a)))
-    # a type other than Q4_K is rejected like an unsupported ggml type
+    # a type other than Q4_K and Q5_K is rejected like an unsupported ggml type
     assert ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, 2, rows, cols,
                                                     144 * (cols // 256), c.ctypes.data, rows) == 0
