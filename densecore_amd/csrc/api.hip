@@ -968,6 +968,188 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
                         x_dev, y_dev, s);
 }
 
+// ---------------------------------------------------------------------------------- fused decoder layers
+struct mq_decoder {
+    DecoderLayerDev* dev_layers = nullptr;
+    int n_layers = 0;
+    int64_t max_tokens = 0, qkv_rows = 0;
+    int hidden = 0, inter = 0, n_q = 0, n_experts = 0, top_k = 0, has_shared = 0, route_mode = 0;
+    float eps = 0.0f;
+    float* qkv = nullptr;
+    float* o = nullptr;
+    float* logits = nullptr;
+    float* mid = nullptr;
+    float* y = nullptr;
+    uint32_t* sync = nullptr;
+    int n_workgroups = 0;
+    long long spin_ticks = 0;
+};
+
+namespace {
+
+void decoder_release(mq_decoder* d) {
+    for (void* q : {(void*)d->dev_layers, (void*)d->qkv, (void*)d->o, (void*)d->logits, (void*)d->mid, (void*)d->y, (void*)d->sync})
+        if (q) (void)hipFree(q);
+    delete d;
+}
+
+// Workgroups of the persistent kernel: one per compute unit, all resident at once.
+int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
+    hipDeviceProp_t prop;
+    MQ_HIP(hipGetDeviceProperties(&prop, g.device));
+    if (lds_bytes > (size_t)prop.maxSharedMemoryPerMultiProcessor)
+        return fail(MQ_ERR_UNSUPPORTED, "fused decoder layers need %zu bytes of LDS per workgroup, the device has %zu", lds_bytes,
+                    (size_t)prop.maxSharedMemoryPerMultiProcessor);
+    MQ_HIP(prepare_decoder_layers(lds_bytes));
+    int rate_khz = 0;
+    if (hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, g.device) != hipSuccess || rate_khz <= 0) rate_khz = 100000;
+    *spin_ticks = (long long)rate_khz * 200;  // 200 ms: a phase takes microseconds
+    *n_workgroups = prop.multiProcessorCount;
+    return MQ_OK;
+}
+
+}  // namespace
+
+int mq_decoder_create(const mq_decoder_layer_desc* layers, int n_layers, int64_t max_tokens, float eps, mq_decoder** out) {
+    if (int rc = check_ready()) return rc;
+    if (!out) return fail(MQ_ERR_INVALID, "mq_decoder_create: null output handle");
+    *out = nullptr;
+    if (!layers || n_layers <= 0) return fail(MQ_ERR_INVALID, "mq_decoder_create: no layers");
+    if (max_tokens < 1 || max_tokens > 8) return fail(MQ_ERR_UNSUPPORTED, "mq_decoder_create: 1..8 tokens per step, asked for %lld", (long long)max_tokens);
+    std::vector<DecoderLayerDev> host((size_t)n_layers);
+    const mq_moe_layer_desc& m0 = layers[0].moe;
+    if (int rc = check_weight(m0.gate_exps, "mq_decoder_create(gate_exps)")) return rc;
+    if (int rc = check_weight(layers[0].wqkv, "mq_decoder_create(wqkv)")) return rc;
+    if (int rc = check_weight(layers[0].wo, "mq_decoder_create(wo)")) return rc;
+    const int64_t hidden = m0.gate_exps->cols, inter = m0.gate_exps->rows, E = m0.gate_exps->n_experts;
+    const int64_t qkv_rows = layers[0].wqkv->rows, n_q = layers[0].wo->cols;
+    const bool has_shared = m0.shared_gate != nullptr;
+    if (E > kDecoderMaxExperts) return fail(MQ_ERR_UNSUPPORTED, "mq_decoder_create: at most %d experts", kDecoderMaxExperts);
+    if (m0.top_k < 1 || m0.top_k > 8 || m0.top_k > E) return fail(MQ_ERR_INVALID, "mq_decoder_create: top_k %d", m0.top_k);
+    if (m0.route_mode < 0 || m0.route_mode > 2) return fail(MQ_ERR_INVALID, "mq_decoder_create: bad route_mode");
+    if (n_q > qkv_rows || (qkv_rows & 15) || (hidden & 15)) return fail(MQ_ERR_INVALID, "mq_decoder_create: n_q exceeds the qkv rows, or rows not a multiple of 16");
+    for (int i = 0; i < n_layers; ++i) {
+        const mq_decoder_layer_desc& L = layers[i];
+        const mq_moe_layer_desc& m = L.moe;
+        const mq_weight* all[8] = {L.wqkv, L.wo, m.gate_exps, m.up_exps, m.down_exps, m.shared_gate, m.shared_up, m.shared_down};
+        for (int j = 0; j < 8; ++j) {
+            if (j >= 5 && !has_shared) {
+                if (all[j]) return fail(MQ_ERR_INVALID, "mq_decoder_create: layer %d has a shared expert, layer 0 has none", i);
+                continue;
+            }
+            if (int rc = check_weight(all[j], "mq_decoder_create")) return rc;
+            if (all[j]->type != kTypeQ4K) return fail(MQ_ERR_UNSUPPORTED, "mq_decoder_create: layer %d holds a non-Q4_K weight; run such layers node by node", i);
+        }
+        if (int rc = check_experts(m.gate_exps, m.up_exps, m.down_exps, m.top_k, "mq_decoder_create")) return rc;
+        const bool same = L.wqkv->rows == qkv_rows && L.wqkv->cols == hidden && L.wqkv->n_experts == 1 && L.wo->rows == hidden &&
+                          L.wo->cols == n_q && L.wo->n_experts == 1 && m.gate_exps->cols == hidden && m.gate_exps->rows == inter &&
+                          m.gate_exps->n_experts == E && m.top_k == m0.top_k && m.route_mode == m0.route_mode && L.router_dev &&
+                          (!has_shared || (m.shared_gate->rows == inter && m.shared_gate->cols == hidden && m.shared_up->rows == inter &&
+                                           m.shared_up->cols == hidden && m.shared_down->rows == hidden && m.shared_down->cols == inter &&
+                                           m.shared_gate->n_experts == 1 && m.shared_up->n_experts == 1 && m.shared_down->n_experts == 1));
+        if (!same) return fail(MQ_ERR_INVALID, "mq_decoder_create: layer %d differs in shape from layer 0, or has no router", i);
+        DecoderLayerDev& h = host[(size_t)i];
+        h.wqkv = L.wqkv->data;
+        h.wo = L.wo->data;
+        h.qkv_rows = qkv_rows;
+        h.attn_norm = L.attn_norm_dev;
+        h.ffn_norm = L.ffn_norm_dev;
+        h.router = L.router_dev;
+        h.fixed_logits = L.fixed_logits_dev;
+        h.gate_exps = m.gate_exps->data;
+        h.up_exps = m.up_exps->data;
+        h.down_exps = m.down_exps->data;
+        h.gu_expert_bytes = m.gate_exps->expert_bytes;
+        h.down_expert_bytes = m.down_exps->expert_bytes;
+        if (m.up_exps->expert_bytes != m.gate_exps->expert_bytes) return fail(MQ_ERR_INVALID, "mq_decoder_create: gate/up expert strides differ");
+        if (has_shared) {
+            h.sh_gate = m.shared_gate->data;
+            h.sh_up = m.shared_up->data;
+            h.sh_down = m.shared_down->data;
+            h.sh_gate_inp = m.sh_gate_inp_dev;
+        }
+    }
+    std::lock_guard<std::mutex> lock(g.mu);
+    mq_decoder* d = new mq_decoder;
+    d->n_layers = n_layers;
+    d->max_tokens = max_tokens;
+    d->qkv_rows = qkv_rows;
+    d->hidden = (int)hidden, d->inter = (int)inter, d->n_q = (int)n_q, d->n_experts = (int)E, d->top_k = m0.top_k;
+    d->has_shared = has_shared ? 1 : 0;
+    d->route_mode = m0.route_mode;
+    d->eps = eps;
+    DecoderArgs probe;
+    probe.n = (int)max_tokens, probe.hidden = d->hidden, probe.n_q = d->n_q;
+    if (int rc = decoder_grid(decoder_layers_lds_bytes(probe), &d->n_workgroups, &d->spin_ticks)) {
+        decoder_release(d);
+        return rc;
+    }
+    const size_t slots = (size_t)d->top_k + (size_t)d->has_shared;
+    const size_t sync_bytes = decoder_sync_bytes(d->n_workgroups);
+    hipError_t e = hipMalloc(&d->dev_layers, host.size() * sizeof(DecoderLayerDev));
+    if (e == hipSuccess) e = hipMemcpy(d->dev_layers, host.data(), host.size() * sizeof(DecoderLayerDev), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc(&d->qkv, (size_t)max_tokens * qkv_rows * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&d->o, (size_t)max_tokens * hidden * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&d->logits, (size_t)max_tokens * E * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&d->mid, (size_t)max_tokens * slots * inter * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&d->y, (size_t)max_tokens * hidden * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&d->sync, sync_bytes);
+    if (e == hipSuccess) e = hipMemset(d->sync, 0, sync_bytes);
+    if (e != hipSuccess) {
+        decoder_release(d);
+        return fail(MQ_ERR_HIP, "mq_decoder_create: %s", hipGetErrorString(e));
+    }
+    *out = d;
+    return MQ_OK;
+}
+
+int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode, float* out_dev, int32_t* ids_out_dev,
+                    float* weights_out_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!d || !x_dev || !out_dev) return fail(MQ_ERR_INVALID, "mq_decoder_step: null argument");
+    if (n < 1 || n > d->max_tokens) return fail(MQ_ERR_INVALID, "mq_decoder_step: %lld tokens, the handle holds 1..%lld", (long long)n, (long long)d->max_tokens);
+    if (silu_mode < -1 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_decoder_step: bad silu_mode");
+    if ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 3u) return fail(MQ_ERR_INVALID, "mq_decoder_step: unaligned pointer");
+    std::lock_guard<std::mutex> lock(g.mu);
+    DecoderArgs a;
+    a.layers = d->dev_layers;
+    a.n_layers = d->n_layers;
+    a.n = (int)n;
+    a.hidden = d->hidden, a.inter = d->inter, a.n_q = d->n_q, a.n_experts = d->n_experts, a.top_k = d->top_k;
+    a.has_shared = d->has_shared;
+    // decode widths use the exact exponential, wider ones the polynomial (core/src/llm/moe/native.cpp:3614-3616)
+    a.silu_mode = silu_mode >= 0 ? silu_mode : (n <= 4 ? MQ_SILU_EXACT : MQ_SILU_FAST);
+    a.route_mode = d->route_mode;
+    a.eps = d->eps;
+    a.spin_ticks = d->spin_ticks;
+    a.x_in = x_dev, a.out = out_dev;
+    a.qkv = d->qkv, a.o = d->o, a.logits = d->logits, a.mid = d->mid, a.y = d->y;
+    a.ids_out = ids_out_dev, a.wts_out = weights_out_dev;
+    a.sync = d->sync;
+    MQ_HIP(launch_decoder_layers(a, d->n_workgroups, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_decoder_status(mq_decoder* d) {
+    if (int rc = check_ready()) return rc;
+    if (!d) return fail(MQ_ERR_INVALID, "mq_decoder_status: null handle");
+    std::lock_guard<std::mutex> lock(g.mu);
+    MQ_HIP(hipDeviceSynchronize());
+    uint32_t flag = 0;
+    MQ_HIP(hipMemcpy(&flag, d->sync + 128, sizeof flag, hipMemcpyDeviceToHost));
+    if (flag == 0) return MQ_OK;
+    // a barrier was abandoned: the outputs of that step are void; make the handle usable again
+    MQ_HIP(hipMemset(d->sync, 0, decoder_sync_bytes(d->n_workgroups)));
+    return fail(MQ_ERR_STATE, "mq_decoder_step: a device-wide barrier timed out (are all compute units free for this process?)");
+}
+
+void mq_decoder_free(mq_decoder* d) {
+    if (!d) return;
+    std::lock_guard<std::mutex> lock(g.mu);
+    (void)hipDeviceSynchronize();
+    decoder_release(d);
+}
+
 // ---------------------------------------------------------------------------------- census
 int mq_census_enable(int on) {
     std::lock_guard<std::mutex> lock(g.mu);

@@ -1,0 +1,511 @@
+// A run of MoE decoder layers at decode width (n <= 8 tokens) as ONE persistent launch on gfx950.
+//
+// The reference executes a decoder graph node by node on a pool of CPU threads that meet at a spin
+// barrier after every node (ggml_graph_compute as driven by core/src/llm/graph/decoder.cpp; the custom
+// nodes of core/src/llm/moe/native.cpp:4831-4911).  At n <= 8 every node of such a layer moves a few
+// megabytes, so on the GPU a launch per node is all latency: nine dependent launches per layer.  Here
+// one workgroup per compute unit stays resident for the whole run of layers and the workgroups meet at a
+// device-wide barrier between the phases of a layer, as the CPU threads do between nodes:
+//
+//   A  x += delta; rmsnorm; Q8_K                        (every workgroup, redundantly, into its own LDS)
+//      qkv = W_qkv . q8k(h)                             row tiles spread over the workgroups        | barrier
+//   B  o = W_o . q8k(qkv[:, :n_q])                      (input re-quantized by every workgroup)     | barrier
+//   C  x += o; rmsnorm; Q8_K; logits = W_router . h2    one wavefront per (expert, token)           | barrier
+//   D  top-k + softmax (one wavefront per token, keys in registers);
+//      hidden = silu(gate_e . h2) * (up_e . h2)         per (token, slot) pair, shared expert extra | barrier
+//   E  y = sum_k w_k * (down_e . q8k(hidden_k)) + sigmoid(g . h2) * shared                          | barrier
+//
+// The residual stream x lives in every workgroup's LDS (all replicas see the same numbers and apply the
+// same arithmetic); what crosses workgroups (qkv, o, logits, hidden, y: a few KB each) is written with
+// device-scope stores and read with device-scope loads, which is all the coherence the barrier needs --
+// no cache write-back or invalidate.  Per-tile arithmetic, wave split of K, reduction order, rmsnorm,
+// router dot, top-k, softmax and combine are those of the one-node kernels (matmul.hip, elementwise.hip,
+// router.hip), so a fused run returns the bits of the node-by-node run.
+//
+// Barrier: two-level arrival counters (16 workgroups per first-level counter, every counter on its own
+// 256-byte line) and a generation word that the waiters poll; counters return to zero by themselves.  A
+// waiter gives up after a bounded time and raises a failure flag that every other waiter sees, so the
+// launch always drains; the host reports the flag as an error.
+#include "common.h"
+#include "kernels.h"
+#include "decode_tile.h"
+#include "q8k_block.h"
+#include "route_block.h"
+
+namespace mq {
+
+namespace {
+
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
+constexpr int kSyncLine = 64;   // uint32 words between counters
+constexpr int kSyncGroup = 16;  // workgroups per first-level counter
+constexpr int kMaxSlots = 9;    // top_k <= 8 routed slots + the shared expert
+constexpr int kKeysPerLane = kDecoderMaxExperts / 64;
+
+__device__ __forceinline__ float ld_dev(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_dev(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t ld_dev(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct Shared {
+    uint8_t* aq;    // A-major Q8_K codes of the current projection input, one 8-row tile: [nb][4096]
+    float* ad;      // [nb][8]
+    float* xres;    // residual stream [n][hidden]
+    float* red;     // cross-wave partial sums [7][2][2][64]
+    float* part;    // down-projection results per slot [kMaxSlots][16]
+    float* scale;   // [8] rmsnorm scale per token
+    float* gate;    // [8] shared-expert gate per token
+    float* wsum;    // [4]
+    float* wts;     // [8][8] routing weights
+    int32_t* ids;   // [8][8] routed experts
+    int* ok;        // barrier verdict of this workgroup
+};
+
+// Device-wide barrier.  Every thread's device-scope stores are acknowledged (vmcnt) before its workgroup is
+// counted.  Returns false when the barrier was abandoned.
+__device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, int* ok, long long spin_ticks) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t* top = sync;
+        uint32_t* gen = sync + kSyncLine;
+        uint32_t* fail = sync + 2 * kSyncLine;
+        const uint32_t n_wg = gridDim.x;
+        const uint32_t grp = blockIdx.x / kSyncGroup;
+        const uint32_t n_grp = (n_wg + kSyncGroup - 1) / kSyncGroup;
+        const uint32_t grp_size = (grp + 1) * kSyncGroup <= n_wg ? kSyncGroup : n_wg - grp * kSyncGroup;
+        uint32_t* gc = sync + (4 + grp) * kSyncLine;
+        bool released = false, good = true;
+        if (__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == grp_size - 1) {
+            __hip_atomic_store(gc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (__hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
+                __hip_atomic_store(top, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // the two resets above are acknowledged before anybody is let go
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __hip_atomic_fetch_add(gen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                released = true;
+            }
+        }
+        if (!released) {
+            const long long t0 = wall_clock64();
+            while (ld_dev(gen) == my_gen) {
+                if (ld_dev(fail) != 0u || wall_clock64() - t0 > spin_ticks) {
+                    __hip_atomic_store(fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    good = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        *ok = good ? 1 : 0;
+    }
+    my_gen += 1;
+    __syncthreads();
+    return *ok != 0;
+}
+
+// xres[t][c] += delta[t][c] (delta: device-scope reads; may be null), then scale[t] = 1/sqrt(mean(x^2) + eps)
+// with the summation order of add_rmsnorm_kernel (256 threads, column-strided, butterfly, pairwise over waves).
+__device__ __forceinline__ void residual_norm(const Shared& s, const float* delta, int n, int hidden, float eps) {
+    const int tid = threadIdx.x;
+    if (delta) {
+        for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = __fadd_rn(s.xres[i], ld_dev(delta + i));
+        __syncthreads();
+    }
+    for (int t = 0; t < n; ++t) {
+        if (tid < 256) {
+            float ssq = 0.0f;
+            for (int c = tid; c < hidden; c += 256) {
+                const float v = s.xres[t * hidden + c];
+                ssq = __fmaf_rn(v, v, ssq);
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+            if ((tid & 63) == 0) s.wsum[tid >> 6] = ssq;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const float total = (s.wsum[0] + s.wsum[1]) + (s.wsum[2] + s.wsum[3]);
+            s.scale[t] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)hidden), eps)));
+        }
+        __syncthreads();
+    }
+}
+
+// normalised value of column c of token t, as add_rmsnorm_kernel forms it
+__device__ __forceinline__ float normed_at(const Shared& s, const float* __restrict__ weight, int t, int hidden, int c) {
+    const float sw = weight ? __fmul_rn(s.scale[t], weight[c]) : s.scale[t];
+    return __fmul_rn(s.xres[t * hidden + c], sw);
+}
+
+// Q8_K of n rows into the LDS A tile, one wavefront per (row, super-block).  get(t, c) returns element c of row t.
+template <typename Get>
+__device__ __forceinline__ void quantize_rows(const Shared& s, int n, int nb, Get get) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int u = wave; u < n * nb; u += kWaves) {
+        const int t = u / nb, b = u - t * nb;
+        const int c0 = b * kQK + lane * 4;
+        const float e[4] = {get(t, c0), get(t, c0 + 1), get(t, c0 + 2), get(t, c0 + 3)};
+        store_amajor(s.aq, s.ad, t, b, nb, lane, quantize_block_q8k(e, lane));
+    }
+}
+
+// This lane's A operand of super-block b from the LDS tile (rows past the live ones read the last live row;
+// their results are never stored).
+__device__ __forceinline__ void load_a_lds(ARegs<1>& a, const Shared& s, int b, int n, int lane) {
+    const int slot = lane & 15, kq = lane >> 4;
+    const int row = (slot >> 1) < n ? (slot >> 1) : n - 1;
+    const uint8_t* base = s.aq + (size_t)b * 4096 + row * 32 + kq * 256 + (slot & 1) * 16;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) a.q[0][c] = *reinterpret_cast<const v4u*>(base + c * 1024);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int r = 2 * kq + j < n ? 2 * kq + j : n - 1;
+        a.yd[0][j] = s.ad[b * 8 + r];
+    }
+}
+
+// One 16-row tile of NMAT matrices against the LDS activations: the waves split the super-blocks
+// (b = wave, wave + 8, ...), partial sums meet in wave order, wave 0 ends up with the totals.
+template <int NMAT>
+__device__ __forceinline__ void tile_rows(const Shared& s, const uint8_t* const (&w)[NMAT], int64_t rt, int nb, int n,
+                                          float (&acc)[NMAT][1][2]) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) acc[m][0][0] = acc[m][0][1] = 0.0f;
+    for (int b = wave; b < nb; b += kWaves) {
+        TileRegs t[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) load_tile(t[m], w[m] + tile_offset(rt, b, nb), lane);
+        ARegs<1> a;
+        load_a_lds(a, s, b, n, lane);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            int32_t dsum[1][2], msum[1][2];
+            compute_tile<1>(t[m], a, acc[m], dsum, msum);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) s.red[(((wave - 1) * NMAT + m) * 2 + j) * 64 + lane] = acc[m][0][j];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        for (int wv = 1; wv < kWaves; ++wv) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[m][0][j] = __fadd_rn(acc[m][0][j], s.red[(((wv - 1) * NMAT + m) * 2 + j) * 64 + lane]);
+        }
+    }
+}
+
+// Dense projection of the LDS activations: y[t][row] for every live token, row tiles spread over the grid.
+__device__ __forceinline__ void dense_phase(const Shared& s, const uint8_t* w, int64_t rows, int nb, int n, float* y,
+                                            int64_t ldy) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rowtiles = (rows + 15) >> 4;
+    for (int64_t rt = blockIdx.x; rt < rowtiles; rt += gridDim.x) {
+        const uint8_t* const ws[1] = {w};
+        float acc[1][1][2];
+        tile_rows<1>(s, ws, rt, nb, n, acc);
+        const int64_t row = rt * 16 + slot;
+        if (wave == 0 && row < rows) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (2 * kq + j < n) st_dev(y + (size_t)(2 * kq + j) * ldy + row, acc[0][0][j]);
+        }
+        __syncthreads();  // red[] is reused by the next row tile
+    }
+}
+
+// Top-k of one token by one wavefront: lane l owns the experts l, l + 64, ...; k rounds of a wave-wide maximum
+// over the 64-bit keys (route_block.h), the owner clears the winner.  Lane 0 then forms the weights.
+__device__ __forceinline__ void route_token_wave(const float* row, bool coherent, int n_experts, int top_k, int mode,
+                                                 int32_t* ids, float* wts, int lane) {
+    unsigned long long key[kKeysPerLane];
+#pragma unroll
+    for (int i = 0; i < kKeysPerLane; ++i) {
+        const int e = lane + 64 * i;
+        key[i] = 0ull;
+        if (e < n_experts) key[i] = route_key(coherent ? ld_dev(row + e) : row[e], e);
+    }
+    float sel[8];
+    for (int r = 0; r < top_k; ++r) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int i = 0; i < kKeysPerLane; ++i) best = key[i] > best ? key[i] : best;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const unsigned long long o = __shfl_xor(best, off, 64);
+            best = o > best ? o : best;
+        }
+        const int id = (int)~(uint32_t)best;
+#pragma unroll
+        for (int i = 0; i < kKeysPerLane; ++i)
+            if (lane + 64 * i == id) key[i] = 0ull;
+        if (lane == 0) ids[r] = id;
+        sel[r] = route_key_logit(best);
+    }
+    if (lane == 0) route_weights(sel, top_k, mode, wts);
+}
+
+// The A operand of one activation row quantized by this wavefront (row 0 of the tile; the other rows are dead):
+// codes move from the quantizer's lanes into the split-slot operand with eight cross-lane reads per super-block.
+__device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
+    const int slot = lane & 15, kq = lane >> 4;
+    const int src = 8 * (slot & 1) + 2 * kq;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t lo = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
+        const uint32_t hi = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
+        a.q[0][c] = slot == 0 ? v4u{lo, hi, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, lo, hi} : v4u{0u, 0u, 0u, 0u});
+    }
+    a.yd[0][0] = q.d;
+    a.yd[0][1] = 0.0f;
+}
+
+__global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slot = lane & 15, kq = lane >> 4;
+    const int n = p.n, hidden = p.hidden, inter = p.inter, top_k = p.top_k, n_experts = p.n_experts;
+    const int nb_h = hidden / kQK, nb_q = p.n_q / kQK, nb_i = inter / kQK;
+    const int nb_max = nb_h > nb_q ? nb_h : nb_q;
+    const int slots = top_k + (p.has_shared ? 1 : 0);
+
+    Shared s;
+    {
+        uint8_t* at = lds_raw;
+        s.aq = at;
+        at += (size_t)nb_max * 4096;
+        s.ad = reinterpret_cast<float*>(at);
+        at += (size_t)nb_max * 8 * sizeof(float);
+        s.xres = reinterpret_cast<float*>(at);
+        at += (size_t)n * hidden * sizeof(float);
+        s.red = reinterpret_cast<float*>(at);
+        at += (size_t)(kWaves - 1) * 2 * 2 * 64 * sizeof(float);
+        s.part = reinterpret_cast<float*>(at);
+        at += (size_t)kMaxSlots * 16 * sizeof(float);
+        s.scale = reinterpret_cast<float*>(at);
+        s.gate = s.scale + 8;
+        s.wsum = s.gate + 8;
+        s.wts = s.wsum + 8;
+        s.ids = reinterpret_cast<int32_t*>(s.wts + 64);
+        s.ok = reinterpret_cast<int*>(s.ids + 64);
+    }
+    if (ld_dev(p.sync + 2 * kSyncLine) != 0u) return;  // an earlier launch abandoned a barrier: the state is unusable
+    uint32_t my_gen = ld_dev(p.sync + kSyncLine);      // cannot move before this workgroup's own first arrival
+
+    for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = p.x_in[i];
+    __syncthreads();
+
+    const float* delta = nullptr;
+    for (int li = 0; li < p.n_layers; ++li) {
+        const DecoderLayerDev& L = p.layers[li];
+
+        if (!p.moe_only) {
+            // ---- A: residual add, rmsnorm, Q8_K, qkv projection -------------------------------------------
+            residual_norm(s, delta, n, hidden, p.eps);
+            {
+                const float* wn = L.attn_norm;
+                quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
+            }
+            __syncthreads();
+            dense_phase(s, L.wqkv, L.qkv_rows, nb_h, n, p.qkv, L.qkv_rows);
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+
+            // ---- B: output projection of the first n_q columns ---------------------------------------------
+            {
+                const float* src = p.qkv;
+                const int64_t ld = L.qkv_rows;
+                quantize_rows(s, n, nb_q, [&](int t, int c) { return ld_dev(src + (size_t)t * ld + c); });
+            }
+            __syncthreads();
+            dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden);
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+
+            // ---- C: residual add, rmsnorm, Q8_K, router projection -----------------------------------------
+            residual_norm(s, p.o, n, hidden, p.eps);
+            {
+                const float* wn = L.ffn_norm;
+                quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
+            }
+            __syncthreads();
+            // one wavefront per (token, expert), the dot of router_logits_kernel
+            for (int u = wave * gridDim.x + blockIdx.x; u < n * n_experts; u += kWaves * gridDim.x) {
+                const int t = u / n_experts, e = u - t * n_experts;
+                const float* wr = L.router + (size_t)e * hidden;
+                float acc = 0.0f;
+                for (int c = lane * 4; c + 3 < hidden; c += 256) {
+                    const float4 a = *reinterpret_cast<const float4*>(wr + c);
+                    acc = __fmaf_rn(a.x, normed_at(s, L.ffn_norm, t, hidden, c), acc);
+                    acc = __fmaf_rn(a.y, normed_at(s, L.ffn_norm, t, hidden, c + 1), acc);
+                    acc = __fmaf_rn(a.z, normed_at(s, L.ffn_norm, t, hidden, c + 2), acc);
+                    acc = __fmaf_rn(a.w, normed_at(s, L.ffn_norm, t, hidden, c + 3), acc);
+                }
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+                if (lane == 0) st_dev(p.logits + (size_t)t * n_experts + e, acc);
+            }
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+        } else {
+            // MoE block alone: x is its (already normalised) input
+            for (int t = tid; t < n; t += kThreads) s.scale[t] = 1.0f;
+            __syncthreads();
+            quantize_rows(s, n, nb_h, [&](int t, int c) { return s.xres[t * hidden + c]; });
+            __syncthreads();
+        }
+
+        // ---- D: routing, then gate/up + SwiGLU per (token, slot) and for the shared expert -------------------
+        if (wave < n) {
+            const bool fixed = L.fixed_logits != nullptr;
+            const float* row = (fixed ? L.fixed_logits : p.logits) + (size_t)wave * n_experts;
+            route_token_wave(row, !fixed, n_experts, top_k, p.route_mode, s.ids + wave * 8, s.wts + wave * 8, lane);
+        }
+        __syncthreads();
+        if (blockIdx.x == 0 && tid < n * top_k) {
+            const int t = tid / top_k, k = tid - t * top_k;
+            if (p.ids_out) p.ids_out[((size_t)li * n + t) * top_k + k] = s.ids[t * 8 + k];
+            if (p.wts_out) p.wts_out[((size_t)li * n + t) * top_k + k] = s.wts[t * 8 + k];
+        }
+        {
+            const int rt_i = inter / 16;
+            const int pairs = n * top_k;
+            const int units = (pairs + (p.has_shared ? 1 : 0)) * rt_i;
+            for (int u = blockIdx.x; u < units; u += gridDim.x) {
+                const int g = u / rt_i, rt = u - g * rt_i;
+                const bool shared = g >= pairs;
+                const int t = shared ? 0 : g / top_k, k = shared ? top_k : g - t * top_k;
+                const int e = shared ? 0 : s.ids[t * 8 + k];
+                if (!shared && (e < 0 || e >= n_experts)) continue;  // whole workgroup skips together
+                const uint8_t* const ws[2] = {shared ? L.sh_gate : L.gate_exps + (size_t)e * L.gu_expert_bytes,
+                                              shared ? L.sh_up : L.up_exps + (size_t)e * L.gu_expert_bytes};
+                float acc[2][1][2];
+                tile_rows<2>(s, ws, rt, nb_h, n, acc);
+                if (wave == 0) {
+                    const int mode = shared ? 2 : p.silu_mode;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int r = 2 * kq + j;  // activation row of this accumulator
+                        if (r < n && (shared || r == t))
+                            st_dev(p.mid + ((size_t)r * slots + k) * inter + rt * 16 + slot,
+                                   silu_mul(acc[0][0][j], acc[1][0][j], mode));
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+
+        // ---- E: down projection per slot, weighted combine in routing order -----------------------------------
+        if (p.has_shared) {
+            for (int t = 0; t < n; ++t) {  // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel
+                if (L.sh_gate_inp) {
+                    if (tid < 256) {
+                        float acc = 0.0f;
+                        for (int c = tid; c < hidden; c += 256)
+                            acc = fmaf(L.sh_gate_inp[c], p.moe_only ? s.xres[t * hidden + c] : normed_at(s, L.ffn_norm, t, hidden, c), acc);
+#pragma unroll
+                        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+                        if ((tid & 63) == 0) s.wsum[tid >> 6] = acc;
+                    }
+                    __syncthreads();
+                    if (tid == 0) s.gate[t] = stable_sigmoid((s.wsum[0] + s.wsum[1]) + (s.wsum[2] + s.wsum[3]));
+                    __syncthreads();
+                } else if (tid == 0) {
+                    s.gate[t] = 1.0f;
+                }
+            }
+            __syncthreads();
+        }
+        {
+            const int rt_h = hidden / 16;
+            for (int u = blockIdx.x; u < n * rt_h; u += gridDim.x) {
+                const int t = u / rt_h, rt = u - t * rt_h;
+                for (int sl = wave; sl < slots; sl += kWaves) {
+                    const bool shared = sl >= top_k;
+                    const int e = shared ? 0 : s.ids[t * 8 + sl];
+                    float acc[1][2] = {{0.0f, 0.0f}};
+                    if (shared || (e >= 0 && e < n_experts)) {  // wave-uniform
+                        const uint8_t* w = shared ? L.sh_down : L.down_exps + (size_t)e * L.down_expert_bytes;
+                        const float* hrow = p.mid + ((size_t)t * slots + sl) * inter;
+                        for (int b = 0; b < nb_i; ++b) {
+                            TileRegs tr;
+                            load_tile(tr, w + tile_offset(rt, b, nb_i), lane);
+                            float ev[4];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) ev[j] = ld_dev(hrow + b * kQK + lane * 4 + j);
+                            ARegs<1> a;
+                            a_from_lane_codes(a, quantize_block_q8k(ev, lane), lane);
+                            int32_t dsum[1][2], msum[1][2];
+                            compute_tile<1>(tr, a, acc, dsum, msum);
+                        }
+                    }
+                    if (kq == 0) s.part[sl * 16 + slot] = acc[0][0];
+                }
+                __syncthreads();
+                if (tid < 16) {
+                    float acc = 0.0f;
+                    for (int k = 0; k < top_k; ++k) {
+                        const int e = s.ids[t * 8 + k];
+                        const float w = s.wts[t * 8 + k];
+                        if (e < 0 || e >= n_experts || w == 0.0f) continue;
+                        acc = __fadd_rn(acc, __fmul_rn(s.part[k * 16 + tid], w));
+                    }
+                    if (p.has_shared) acc = __fadd_rn(acc, __fmul_rn(s.part[top_k * 16 + tid], s.gate[t]));
+                    st_dev(p.y + (size_t)t * hidden + rt * 16 + tid, acc);
+                }
+                __syncthreads();
+            }
+        }
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+        delta = p.y;
+    }
+
+    // ---- the last residual add (or, for the MoE block alone, its output as it is) ---------------------------
+    for (int i = blockIdx.x * kThreads + tid; i < n * hidden; i += gridDim.x * kThreads)
+        p.out[i] = p.moe_only ? ld_dev(p.y + i) : __fadd_rn(s.xres[i], ld_dev(p.y + i));
+}
+
+}  // namespace
+
+size_t decoder_layers_lds_bytes(const DecoderArgs& a) {
+    const int nb_h = a.hidden / kQK, nb_q = a.n_q / kQK;
+    const int nb_max = nb_h > nb_q ? nb_h : nb_q;
+    return (size_t)nb_max * 4096 + (size_t)nb_max * 8 * 4 + (size_t)a.n * a.hidden * 4 + (size_t)(kWaves - 1) * 2 * 2 * 64 * 4 +
+           (size_t)kMaxSlots * 16 * 4 + (8 + 8 + 8 + 64 + 64 + 4) * 4;
+}
+
+size_t decoder_sync_bytes(int n_workgroups) {
+    return (size_t)(4 + (n_workgroups + kSyncGroup - 1) / kSyncGroup) * kSyncLine * sizeof(uint32_t);
+}
+
+hipError_t prepare_decoder_layers(size_t lds_bytes) {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(decoder_layers_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+}
+
+hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream) {
+    if (a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
+        a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || n_workgroups < 1 ||
+        (!a.moe_only && (a.n_q <= 0 || (a.n_q % kQK))))
+        return hipErrorInvalidValue;
+    hipLaunchKernelGGL(decoder_layers_kernel, dim3((unsigned)n_workgroups), dim3(kThreads), decoder_layers_lds_bytes(a),
+                       stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace mq

@@ -123,4 +123,51 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
                               const float* x, float* y, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
 
+// ---- decoder_layers.hip ----------------------------------------------------------------------
+// A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,
+// device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.
+constexpr int kDecoderMaxExperts = 512;
+struct DecoderLayerDev {               // one per layer, in device memory
+    const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]
+    const uint8_t* wo = nullptr;       // [hidden x n_q]; its input is qkv[:, :n_q]
+    int64_t qkv_rows = 0;
+    const float* attn_norm = nullptr;  // [hidden] or null (ones)
+    const float* ffn_norm = nullptr;
+    const float* router = nullptr;     // fp32 [n_experts x hidden]
+    const float* fixed_logits = nullptr;  // fp32 [n x n_experts] or null: route on these instead of router . h2
+    const uint8_t* gate_exps = nullptr;
+    const uint8_t* up_exps = nullptr;
+    const uint8_t* down_exps = nullptr;
+    size_t gu_expert_bytes = 0, down_expert_bytes = 0;
+    const uint8_t* sh_gate = nullptr;  // shared expert (all three or none, as DecoderArgs::has_shared says)
+    const uint8_t* sh_up = nullptr;
+    const uint8_t* sh_down = nullptr;
+    const float* sh_gate_inp = nullptr;  // fp32 [hidden] or null (gate = 1)
+};
+struct DecoderArgs {
+    const DecoderLayerDev* layers = nullptr;
+    int n_layers = 0;
+    int n = 0;                         // tokens, 1..8
+    int hidden = 0, inter = 0, n_q = 0, n_experts = 0, top_k = 0;
+    int has_shared = 0;
+    int moe_only = 0;                  // 1: every "layer" is the MoE block alone on x (no projections, no residual)
+    int silu_mode = 0, route_mode = 0;
+    float eps = 0.0f;
+    long long spin_ticks = 0;          // barrier patience in wall_clock64 ticks
+    const float* x_in = nullptr;       // [n x hidden]
+    float* out = nullptr;              // [n x hidden]
+    float* qkv = nullptr;              // exchange buffers: [n x qkv_rows]
+    float* o = nullptr;                // [n x hidden]
+    float* logits = nullptr;           // [n x n_experts]
+    float* mid = nullptr;              // [n x (top_k + has_shared) x inter]
+    float* y = nullptr;                // [n x hidden]
+    int32_t* ids_out = nullptr;        // optional [n_layers x n x top_k]
+    float* wts_out = nullptr;
+    uint32_t* sync = nullptr;          // decoder_sync_bytes(), zero before the first launch
+};
+size_t decoder_layers_lds_bytes(const DecoderArgs& a);
+size_t decoder_sync_bytes(int n_workgroups);
+hipError_t prepare_decoder_layers(size_t lds_bytes);
+hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream);
+
 }  // namespace mq

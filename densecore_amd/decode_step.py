@@ -14,6 +14,9 @@ which is the operator sequence of a Qwen3.5-35B-A3B-class layer in the reference
 (core/src/llm/graph/decoder.cpp:2265, :2426-2600; core/src/llm/moe/native.cpp:4831-4911) with the
 attention core left out.  Weights are random-init Q4_K generated on the device from seeds.  The
 whole step can be captured in one HIP graph (torch.cuda.CUDAGraph) and replayed.
+
+FusedDecodeStep runs the same layers through mq_decoder_step: one persistent kernel for the whole run of
+layers (n <= 8), whose results are bit-identical to DecodeStep's.
 """
 import ctypes as C
 from dataclasses import dataclass
@@ -154,3 +157,60 @@ class DecodeStep:
             for ly in self.layers:
                 ly.free()
         self.layers = []
+
+
+class FusedDecodeStep:
+    """The layers of a DecodeStep through mq_decoder_step (one launch per step, n <= 8 tokens)."""
+
+    def __init__(self, cfg: StepConfig, n_tokens: int, layers, fixed_logits=None):
+        self.cfg, self.n, self.layers = cfg, n_tokens, layers
+        f = lambda *shape: torch.empty(shape, dtype=torch.float32, device="cuda")
+        self.x, self.out = f(n_tokens, cfg.hidden), f(n_tokens, cfg.hidden)
+        self.ids = torch.empty((len(layers), n_tokens, cfg.top_k), dtype=torch.int32, device="cuda")
+        self.wts = f(len(layers), n_tokens, cfg.top_k)
+        self.fixed_logits = fixed_logits          # [n_layers, n_tokens, n_experts] or None
+        table = (_lib.DecoderLayerDesc * len(layers))()
+        for i, ly in enumerate(layers):
+            table[i].wqkv, table[i].wo = ly.wqkv._h, ly.wo._h
+            table[i].attn_norm_dev = table[i].ffn_norm_dev = None
+            table[i].router_dev = ly.router.data_ptr()
+            table[i].fixed_logits_dev = fixed_logits[i].data_ptr() if fixed_logits is not None else None
+            table[i].moe = ly.desc
+        h = C.c_void_p()
+        _lib.check(_lib.lib().mq_decoder_create(table, len(layers), n_tokens, C.c_float(cfg.eps), C.byref(h)),
+                   "mq_decoder_create")
+        self._h = h
+        self._graph = None
+
+    def _launch(self) -> None:
+        p = lambda t: C.c_void_p(t.data_ptr())
+        st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(_lib.lib().mq_decoder_step(self._h, p(self.x), self.n, -1, p(self.out), p(self.ids), p(self.wts), st),
+                   "mq_decoder_step")
+
+    def run(self, x_in: torch.Tensor) -> torch.Tensor:
+        self.x.copy_(x_in)
+        self._launch()
+        return self.out
+
+    def status(self) -> None:
+        """Synchronise and raise if a step abandoned a device-wide barrier."""
+        _lib.check(_lib.lib().mq_decoder_status(self._h), "mq_decoder_status")
+
+    def capture(self) -> None:
+        self._launch()
+        self.status()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._launch()
+        self._graph = g
+
+    def replay(self) -> torch.Tensor:
+        self._graph.replay()
+        return self.out
+
+    def free(self) -> None:
+        self._graph = None
+        if self._h:
+            _lib.lib().mq_decoder_free(self._h)
+            self._h = None

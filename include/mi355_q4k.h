@@ -213,6 +213,42 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const f
                      float* y_dev, int32_t* ids_out_dev /* may be NULL */, float* weights_out_dev /* may be NULL */,
                      void* stream);
 
+/* ---- a run of decoder layers in one launch --------------------------------------------
+ * Per layer, for n <= 8 tokens (x is the residual stream, fp32 [n][hidden]):
+ *   h   = rmsnorm(x) * attn_norm          qkv = wqkv . q8k(h)          o = wo . q8k(qkv[:, :n_q])
+ *   x  += o          h2 = rmsnorm(x) * ffn_norm          logits = router . h2 (fp32)
+ *   x  += moe(h2, logits)                 (mq_moe_layer_q4k's arithmetic, shared expert included)
+ * i.e. the node sequence the reference's graph builder emits for a Qwen3.5-MoE-class layer
+ * (core/src/llm/graph/decoder.cpp:2265, :2426-2600; core/src/llm/moe/native.cpp:4831-4911) with the attention
+ * core left out (the first n_q columns of qkv stand in for its output).  The reference runs those nodes on CPU
+ * threads that meet at a barrier after each one; here one persistent kernel does, with device-wide barriers
+ * between the phases, and returns bit for bit what the node-by-node entry points above return
+ * (mq_add_rmsnorm_q8k, mq_mul_mat_q4k_acts, mq_mul_mat_q4k, mq_add_rmsnorm_f32, mq_router_logits_f32,
+ * mq_moe_layer_q4k).  All weights Q4_K; every layer has layer 0's shapes; n_experts <= 512; top_k <= 8.
+ * The kernel needs every compute unit of the device free for this process: a barrier that is not met within
+ * 200 ms is abandoned, the launch drains, and mq_decoder_status reports it. */
+typedef struct mq_decoder mq_decoder;
+typedef struct {
+    const mq_weight* wqkv;            /* [n_q + 2 n_kv][hidden], wq / wk / wv stacked row-wise */
+    const mq_weight* wo;              /* [hidden][n_q] */
+    const float* attn_norm_dev;       /* fp32 [hidden] or NULL (ones) */
+    const float* ffn_norm_dev;
+    const float* router_dev;          /* fp32 [n_experts][hidden] */
+    const float* fixed_logits_dev;    /* NULL, or fp32 [n][n_experts]: route on these, not on router . h2 */
+    mq_moe_layer_desc moe;            /* silu_mode is taken from mq_decoder_step, not from here */
+} mq_decoder_layer_desc;
+/* Copies the layer table to the device and allocates the exchange buffers; the weights stay the caller's. */
+int mq_decoder_create(const mq_decoder_layer_desc* layers, int n_layers, int64_t max_tokens, float eps, mq_decoder** out);
+/* out = x after the last layer, fp32 [n][hidden].  silu_mode: MQ_SILU_* for the routed experts, or -1 for the
+ * reference's rule (exact for n <= 4, polynomial above; core/src/llm/moe/native.cpp:3614-3616).
+ * ids_out_dev int32 / weights_out_dev fp32 [n_layers][n][top_k], or NULL.  Allocates nothing (capturable). */
+int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode, float* out_dev, int32_t* ids_out_dev,
+                    float* weights_out_dev, void* stream);
+/* Synchronises the device; MQ_OK, or MQ_ERR_STATE when a step since the last call abandoned a barrier (its
+ * outputs are void; the handle is usable again afterwards). */
+int mq_decoder_status(mq_decoder* d);
+void mq_decoder_free(mq_decoder* d);
+
 /* ---- the fp32 operators either side of the path --------------------------------------------
  * sum = x + delta (delta_dev may be NULL: sum = x), normed = sum * (weight / sqrt(mean(sum^2) + eps));
  * x/delta/sum/normed fp32 [n][cols] dense, weight_dev fp32 [cols] or NULL (ones), sum_out_dev may be NULL
