@@ -387,12 +387,29 @@ def side_measurements(ops, synth, torch, np, dev):
         for _ in range(reps):
             st.replay()
         torch.cuda.synchronize()
+        dt_nodes = (time.perf_counter() - t) / reps
+        # the same layers as one persistent launch (mq_decoder_step)
+        fz = decode_step.FusedDecodeStep(cfg, n, base.layers, st.fixed_logits)
+        fz.x.copy_(x)
+        fz.capture()
+        fz.replay()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(reps):
+            fz.replay()
+        torch.cuda.synchronize()
         dt = (time.perf_counter() - t) / reps
+        fz.status()
+        same = bool(torch.equal(fz.ids, st.ids))
+        fz.free()
         q4 = lambda r, c: r * c // 256 * 144
         per_expert = 2 * q4(cfg.inter, cfg.hidden) + q4(cfg.hidden, cfg.inter)
         fixed = per_expert + q4(cfg.n_q + 2 * cfg.n_kv, cfg.hidden) + q4(cfg.hidden, cfg.n_q) + cfg.n_experts * cfg.hidden * 4
         step_bytes = sum(d * per_expert + fixed + n * cfg.hidden * 8 for d in distinct)
-        steps[str(n)] = {"ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(n / dt, 1),
+        steps[str(n)] = {"launch": "one persistent kernel per step (mq_decoder_step)", "same_experts_as_node_by_node": same,
+                         "node_by_node_ms_per_step": round(dt_nodes * 1e3, 3),
+                         "node_by_node_tokens_per_s": round(n / dt_nodes, 1),
+                         "ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(n / dt, 1),
                          "us_per_layer": round(dt * 1e6 / cfg.n_layers, 2),
                          "distinct_experts_per_layer": round(sum(distinct) / len(distinct), 1),
                          "per_layer_GBps": round(step_bytes / cfg.n_layers / (dt / cfg.n_layers) / 1e9, 1),

@@ -118,6 +118,31 @@ __device__ __forceinline__ v4u load_stream16(const void* p) {
 }
 __device__ __forceinline__ v4u load16(const void* p) { return *reinterpret_cast<const v4u*>(p); }
 
+// Value of lane (i ^ 1), (i ^ 2), the mirrored lane of each 8, of each 16: data-parallel-primitive moves,
+// an order of magnitude cheaper than a cross-lane read through LDS.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, true);
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
+// Maximum of an unsigned value over the 64 lanes, returned in every lane (wave-uniform).
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+    uint32_t t;
+    t = dpp_u32<kDppXor1>(x);
+    x = t > x ? t : x;
+    t = dpp_u32<kDppXor2>(x);
+    x = t > x ? t : x;
+    t = dpp_u32<kDppHalfMirror>(x);
+    x = t > x ? t : x;
+    t = dpp_u32<kDppMirror>(x);
+    x = t > x ? t : x;
+    const uint32_t a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16);
+    const uint32_t c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
 // The reference's fast exp (core/src/backend/cpu_backend_internal.h:99-114): unfused Horner.
 __device__ __forceinline__ float fast_exp_plain(float x) {
     x = x < -50.0f ? -50.0f : x;

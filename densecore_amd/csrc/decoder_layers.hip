@@ -41,6 +41,7 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kSyncLine = 64;   // uint32 words between counters
 constexpr int kSyncGroup = 16;  // workgroups per first-level counter
 constexpr int kMaxSlots = 9;    // top_k <= 8 routed slots + the shared expert
+constexpr int kMaxInterBlocks = 8;  // inter <= 2048
 constexpr int kKeysPerLane = kDecoderMaxExperts / 64;
 
 __device__ __forceinline__ float ld_dev(const float* p) {
@@ -58,20 +59,22 @@ struct Shared {
     float* ad;      // [nb][8]
     float* xres;    // residual stream [n][hidden]
     float* red;     // cross-wave partial sums [7][2][2][64]
-    float* part;    // down-projection results per slot [kMaxSlots][16]
+    float* term;    // down-projection terms per (slot, super-block) [kMaxSlots][kMaxInterBlocks][16]
     float* scale;   // [8] rmsnorm scale per token
     float* gate;    // [8] shared-expert gate per token
-    float* wsum;    // [4]
     float* wts;     // [8][8] routing weights
     int32_t* ids;   // [8][8] routed experts
     int* ok;        // barrier verdict of this workgroup
 };
 
 // Device-wide barrier.  Every thread's device-scope stores are acknowledged (vmcnt) before its workgroup is
-// counted.  Returns false when the barrier was abandoned.
-__device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, int* ok, long long spin_ticks) {
+// counted.  `ahead()` runs in every thread once that is so and before the wait: the place to request weights
+// of the next phase, whose latency then overlaps the barrier's.  Returns false when the barrier was abandoned.
+template <typename Ahead>
+__device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, int* ok, long long spin_ticks, Ahead ahead) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    ahead();
     if (threadIdx.x == 0) {
         uint32_t* top = sync;
         uint32_t* gen = sync + kSyncLine;
@@ -110,32 +113,40 @@ __device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, i
     return *ok != 0;
 }
 
+// Sum over the columns of `term(c)` in the order of a 256-thread workgroup of the one-node kernels (thread j
+// takes columns j, j + 256, ... with fused multiply-adds, a butterfly inside each wavefront, then
+// (w0 + w1) + (w2 + w3)), evaluated by ONE wavefront: lane l plays threads l, l + 64, l + 128, l + 192.
+template <typename Term>
+__device__ __forceinline__ float sum_like_256_threads(int hidden, int lane, Term term) {
+    float part[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        float acc = 0.0f;
+        for (int c = v * 64 + lane; c < hidden; c += 256) acc = term(c, acc);
+        part[v] = acc;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part[v] += __shfl_xor(part[v], off, 64);
+    }
+    return (part[0] + part[1]) + (part[2] + part[3]);
+}
+
 // xres[t][c] += delta[t][c] (delta: device-scope reads; may be null), then scale[t] = 1/sqrt(mean(x^2) + eps)
-// with the summation order of add_rmsnorm_kernel (256 threads, column-strided, butterfly, pairwise over waves).
+// with the summation order of add_rmsnorm_kernel; one wavefront per token.
 __device__ __forceinline__ void residual_norm(const Shared& s, const float* delta, int n, int hidden, float eps) {
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (delta) {
         for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = __fadd_rn(s.xres[i], ld_dev(delta + i));
         __syncthreads();
     }
-    for (int t = 0; t < n; ++t) {
-        if (tid < 256) {
-            float ssq = 0.0f;
-            for (int c = tid; c < hidden; c += 256) {
-                const float v = s.xres[t * hidden + c];
-                ssq = __fmaf_rn(v, v, ssq);
-            }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
-            if ((tid & 63) == 0) s.wsum[tid >> 6] = ssq;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            const float total = (s.wsum[0] + s.wsum[1]) + (s.wsum[2] + s.wsum[3]);
-            s.scale[t] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)hidden), eps)));
-        }
-        __syncthreads();
+    if (wave < n) {
+        const float* row = s.xres + wave * hidden;
+        const float total = sum_like_256_threads(hidden, lane, [&](int c, float acc) { return __fmaf_rn(row[c], row[c], acc); });
+        if (lane == 0) s.scale[wave] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)hidden), eps)));
     }
+    __syncthreads();
 }
 
 // normalised value of column c of token t, as add_rmsnorm_kernel forms it
@@ -171,16 +182,37 @@ __device__ __forceinline__ void load_a_lds(ARegs<1>& a, const Shared& s, int b, 
     }
 }
 
-// One 16-row tile of NMAT matrices against the LDS activations: the waves split the super-blocks
-// (b = wave, wave + 8, ...), partial sums meet in wave order, wave 0 ends up with the totals.
+// The weight tiles of super-block `wave` of row tile rt, requested ahead of their use.
 template <int NMAT>
-__device__ __forceinline__ void tile_rows(const Shared& s, const uint8_t* const (&w)[NMAT], int64_t rt, int nb, int n,
-                                          float (&acc)[NMAT][1][2]) {
+__device__ __forceinline__ void fetch_tiles(TileRegs (&t)[NMAT], const uint8_t* const (&w)[NMAT], int64_t rt, int nb) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // a wavefront past the last super-block fetches block 0 and never uses it: the load count stays uniform
+    const int b = wave < nb ? wave : 0;
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) load_tile(t[m], w[m] + tile_offset(rt, b, nb), lane);
+}
+
+// One 16-row tile of NMAT matrices against the LDS activations: the waves split the super-blocks
+// (b = wave, wave + 8, ...), partial sums meet in wave order, wave 0 ends up with the totals.  `first` holds
+// the tiles of super-block `wave` (fetch_tiles).
+template <int NMAT>
+__device__ __forceinline__ void tile_rows(const Shared& s, const TileRegs (&first)[NMAT], const uint8_t* const (&w)[NMAT],
+                                          int64_t rt, int nb, int n, float (&acc)[NMAT][1][2]) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) acc[m][0][0] = acc[m][0][1] = 0.0f;
-    for (int b = wave; b < nb; b += kWaves) {
+    if (wave < nb) {
+        ARegs<1> a;
+        load_a_lds(a, s, wave, n, lane);
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            int32_t dsum[1][2], msum[1][2];
+            compute_tile<1>(first[m], a, acc[m], dsum, msum);
+        }
+    }
+    for (int b = wave + kWaves; b < nb; b += kWaves) {
         TileRegs t[NMAT];
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) load_tile(t[m], w[m] + tile_offset(rt, b, nb), lane);
@@ -211,15 +243,20 @@ __device__ __forceinline__ void tile_rows(const Shared& s, const uint8_t* const 
 }
 
 // Dense projection of the LDS activations: y[t][row] for every live token, row tiles spread over the grid.
+// `first` holds the tiles of this workgroup's first row tile (requested during the barrier that precedes the
+// phase); the next row tile's are requested before the current one is multiplied.
 __device__ __forceinline__ void dense_phase(const Shared& s, const uint8_t* w, int64_t rows, int nb, int n, float* y,
-                                            int64_t ldy) {
+                                            int64_t ldy, TileRegs (&first)[1]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rowtiles = (rows + 15) >> 4;
+    const uint8_t* const ws[1] = {w};
     for (int64_t rt = blockIdx.x; rt < rowtiles; rt += gridDim.x) {
-        const uint8_t* const ws[1] = {w};
+        TileRegs next[1];
+        const bool more = rt + gridDim.x < rowtiles;
+        if (more) fetch_tiles<1>(next, ws, rt + gridDim.x, nb);
         float acc[1][1][2];
-        tile_rows<1>(s, ws, rt, nb, n, acc);
+        tile_rows<1>(s, first, ws, rt, nb, n, acc);
         const int64_t row = rt * 16 + slot;
         if (wave == 0 && row < rows) {
 #pragma unroll
@@ -227,6 +264,7 @@ __device__ __forceinline__ void dense_phase(const Shared& s, const uint8_t* w, i
                 if (2 * kq + j < n) st_dev(y + (size_t)(2 * kq + j) * ldy + row, acc[0][0][j]);
         }
         __syncthreads();  // red[] is reused by the next row tile
+        if (more) first[0] = next[0];
     }
 }
 
@@ -246,11 +284,7 @@ __device__ __forceinline__ void route_token_wave(const float* row, bool coherent
         unsigned long long best = 0ull;
 #pragma unroll
         for (int i = 0; i < kKeysPerLane; ++i) best = key[i] > best ? key[i] : best;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const unsigned long long o = __shfl_xor(best, off, 64);
-            best = o > best ? o : best;
-        }
+        best = wave_max_key(best);
         const int id = (int)~(uint32_t)best;
 #pragma unroll
         for (int i = 0; i < kKeysPerLane; ++i)
@@ -276,6 +310,8 @@ __device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, 
     a.yd[0][1] = 0.0f;
 }
 
+constexpr int kItems = 3;  // (slot, super-block) items of the down projection a wavefront keeps in flight
+
 __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -297,17 +333,26 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         at += (size_t)n * hidden * sizeof(float);
         s.red = reinterpret_cast<float*>(at);
         at += (size_t)(kWaves - 1) * 2 * 2 * 64 * sizeof(float);
-        s.part = reinterpret_cast<float*>(at);
-        at += (size_t)kMaxSlots * 16 * sizeof(float);
+        s.term = reinterpret_cast<float*>(at);
+        at += (size_t)kMaxSlots * kMaxInterBlocks * 16 * sizeof(float);
         s.scale = reinterpret_cast<float*>(at);
         s.gate = s.scale + 8;
-        s.wsum = s.gate + 8;
-        s.wts = s.wsum + 8;
+        s.wts = s.gate + 8;
         s.ids = reinterpret_cast<int32_t*>(s.wts + 64);
         s.ok = reinterpret_cast<int*>(s.ids + 64);
     }
     if (ld_dev(p.sync + 2 * kSyncLine) != 0u) return;  // an earlier launch abandoned a barrier: the state is unusable
     uint32_t my_gen = ld_dev(p.sync + kSyncLine);      // cannot move before this workgroup's own first arrival
+    const auto nothing = [] {};
+
+    // Weights of this workgroup's first row tile of a dense projection, requested a phase ahead.  Workgroups
+    // without a row tile fetch tile 0 and never use it, so that the registers are defined on every path.
+    auto request_dense = [&](TileRegs (&dst)[1], const uint8_t* w, int64_t rows, int nb) {
+        const uint8_t* const ws[1] = {w};
+        fetch_tiles<1>(dst, ws, (int64_t)blockIdx.x < ((rows + 15) >> 4) ? blockIdx.x : 0, nb);
+    };
+    TileRegs ahead_qkv[1];
+    if (!p.moe_only) request_dense(ahead_qkv, p.layers[0].wqkv, p.layers[0].qkv_rows, nb_h);
 
     for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = p.x_in[i];
     __syncthreads();
@@ -324,8 +369,9 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
             }
             __syncthreads();
-            dense_phase(s, L.wqkv, L.qkv_rows, nb_h, n, p.qkv, L.qkv_rows);
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+            dense_phase(s, L.wqkv, L.qkv_rows, nb_h, n, p.qkv, L.qkv_rows, ahead_qkv);
+            TileRegs ahead_wo[1];
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] { request_dense(ahead_wo, L.wo, hidden, nb_q); })) return;
 
             // ---- B: output projection of the first n_q columns ---------------------------------------------
             {
@@ -334,8 +380,8 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 quantize_rows(s, n, nb_q, [&](int t, int c) { return ld_dev(src + (size_t)t * ld + c); });
             }
             __syncthreads();
-            dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden);
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+            dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden, ahead_wo);
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, nothing)) return;
 
             // ---- C: residual add, rmsnorm, Q8_K, router projection -----------------------------------------
             residual_norm(s, p.o, n, hidden, p.eps);
@@ -360,7 +406,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
                 if (lane == 0) st_dev(p.logits + (size_t)t * n_experts + e, acc);
             }
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, nothing)) return;
         } else {
             // MoE block alone: x is its (already normalised) input
             for (int t = tid; t < n; t += kThreads) s.scale[t] = 1.0f;
@@ -385,93 +431,164 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
             const int rt_i = inter / 16;
             const int pairs = n * top_k;
             const int units = (pairs + (p.has_shared ? 1 : 0)) * rt_i;
-            for (int u = blockIdx.x; u < units; u += gridDim.x) {
-                const int g = u / rt_i, rt = u - g * rt_i;
-                const bool shared = g >= pairs;
-                const int t = shared ? 0 : g / top_k, k = shared ? top_k : g - t * top_k;
+            // unit u -> (pair or shared pass, row tile); a dropped pair (id out of range) has no weights
+            auto unit_weights = [&](int u, const uint8_t* (&ws)[2], int& t, int& k, int& rt, bool& shared) -> bool {
+                const int g = u / rt_i;
+                rt = u - g * rt_i;
+                shared = g >= pairs;
+                t = shared ? 0 : g / top_k;
+                k = shared ? top_k : g - t * top_k;
                 const int e = shared ? 0 : s.ids[t * 8 + k];
-                if (!shared && (e < 0 || e >= n_experts)) continue;  // whole workgroup skips together
-                const uint8_t* const ws[2] = {shared ? L.sh_gate : L.gate_exps + (size_t)e * L.gu_expert_bytes,
-                                              shared ? L.sh_up : L.up_exps + (size_t)e * L.gu_expert_bytes};
-                float acc[2][1][2];
-                tile_rows<2>(s, ws, rt, nb_h, n, acc);
-                if (wave == 0) {
-                    const int mode = shared ? 2 : p.silu_mode;
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        const int r = 2 * kq + j;  // activation row of this accumulator
-                        if (r < n && (shared || r == t))
-                            st_dev(p.mid + ((size_t)r * slots + k) * inter + rt * 16 + slot,
-                                   silu_mul(acc[0][0][j], acc[1][0][j], mode));
+                if (!shared && (e < 0 || e >= n_experts)) return false;
+                ws[0] = shared ? L.sh_gate : L.gate_exps + (size_t)e * L.gu_expert_bytes;
+                ws[1] = shared ? L.sh_up : L.up_exps + (size_t)e * L.gu_expert_bytes;
+                return true;
+            };
+            TileRegs cur[2], nxt[2];
+            const uint8_t* ws[2];
+            const uint8_t* wn[2];
+            int t, k, rt, tn, kn, rtn;
+            bool shared, sharedn;
+            bool live = false;
+            if ((int)blockIdx.x < units) {
+                live = unit_weights(blockIdx.x, ws, t, k, rt, shared);
+                if (live) {
+                    const uint8_t* const wc[2] = {ws[0], ws[1]};
+                    fetch_tiles<2>(cur, wc, rt, nb_h);
+                }
+            }
+            for (int u = blockIdx.x; u < units; u += gridDim.x) {
+                bool live_n = false;
+                if (u + (int)gridDim.x < units) {
+                    live_n = unit_weights(u + gridDim.x, wn, tn, kn, rtn, sharedn);
+                    if (live_n) {
+                        const uint8_t* const wc[2] = {wn[0], wn[1]};
+                        fetch_tiles<2>(nxt, wc, rtn, nb_h);
                     }
                 }
-                __syncthreads();
+                if (live) {  // the whole workgroup takes the same branch
+                    const uint8_t* const wc[2] = {ws[0], ws[1]};
+                    float acc[2][1][2];
+                    tile_rows<2>(s, cur, wc, rt, nb_h, n, acc);
+                    if (wave == 0) {
+                        const int mode = shared ? 2 : p.silu_mode;
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            const int r = 2 * kq + j;  // activation row of this accumulator
+                            if (r < n && (shared || r == t))
+                                st_dev(p.mid + ((size_t)r * slots + k) * inter + rt * 16 + slot,
+                                       silu_mul(acc[0][0][j], acc[1][0][j], mode));
+                        }
+                    }
+                    __syncthreads();
+                }
+                live = live_n;
+                if (live_n) {
+                    cur[0] = nxt[0], cur[1] = nxt[1];
+                    ws[0] = wn[0], ws[1] = wn[1];
+                    t = tn, k = kn, rt = rtn, shared = sharedn;
+                }
             }
         }
-        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
 
         // ---- E: down projection per slot, weighted combine in routing order -----------------------------------
-        if (p.has_shared) {
-            for (int t = 0; t < n; ++t) {  // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel
-                if (L.sh_gate_inp) {
-                    if (tid < 256) {
-                        float acc = 0.0f;
-                        for (int c = tid; c < hidden; c += 256)
-                            acc = fmaf(L.sh_gate_inp[c], p.moe_only ? s.xres[t * hidden + c] : normed_at(s, L.ffn_norm, t, hidden, c), acc);
+        // A unit is one (token, 16-row tile); its slots x super-blocks are spread over the wavefronts.
+        const int rt_h = hidden / 16;
+        const int n_items = slots * nb_i;
+        TileRegs etile[kItems];
+        auto item_tile = [&](int t, int rt, int i) -> const uint8_t* {  // null for a dropped slot
+            const int sl = i / nb_i, b = i - sl * nb_i;
+            const bool shared = sl >= top_k;
+            const int e = shared ? 0 : s.ids[t * 8 + sl];
+            if (!shared && (e < 0 || e >= n_experts)) return nullptr;
+            return (shared ? L.sh_down : L.down_exps + (size_t)e * L.down_expert_bytes) + tile_offset(rt, b, nb_i);
+        };
+        auto fetch_items = [&](int t, int rt, int base) {
 #pragma unroll
-                        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-                        if ((tid & 63) == 0) s.wsum[tid >> 6] = acc;
-                    }
-                    __syncthreads();
-                    if (tid == 0) s.gate[t] = stable_sigmoid((s.wsum[0] + s.wsum[1]) + (s.wsum[2] + s.wsum[3]));
-                    __syncthreads();
-                } else if (tid == 0) {
-                    s.gate[t] = 1.0f;
+            for (int j = 0; j < kItems; ++j) {
+                const int i = base + wave + kWaves * j;
+                const uint8_t* w = i < n_items ? item_tile(t, rt, i) : nullptr;
+                load_tile(etile[j], w ? w : L.down_exps, lane);  // a dropped item reads a harmless tile
+            }
+        };
+        const bool e_unit = (int)blockIdx.x < n * rt_h;
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                if (e_unit) fetch_items(blockIdx.x / rt_h, blockIdx.x % rt_h, 0);
+            }))
+            return;
+
+        if (p.has_shared) {  // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel
+            if (wave < n) {
+                float g = 1.0f;
+                if (L.sh_gate_inp) {
+                    const float* gi = L.sh_gate_inp;
+                    const float* wn = L.ffn_norm;
+                    const bool raw = p.moe_only != 0;
+                    g = stable_sigmoid(sum_like_256_threads(hidden, lane, [&](int c, float acc) {
+                        return fmaf(gi[c], raw ? s.xres[wave * hidden + c] : normed_at(s, wn, wave, hidden, c), acc);
+                    }));
                 }
+                if (lane == 0) s.gate[wave] = g;
+            }
+            __syncthreads();
+        }
+        for (int u = blockIdx.x; u < n * rt_h; u += gridDim.x) {
+            const int t = u / rt_h, rt = u - t * rt_h;
+            for (int base = 0; base < n_items; base += kWaves * kItems) {
+                if (u != (int)blockIdx.x || base != 0) fetch_items(t, rt, base);
+                float ev[kItems][4];
+#pragma unroll
+                for (int j = 0; j < kItems; ++j) {
+                    const int i = base + wave + kWaves * j;
+                    const int ii = i < n_items ? i : 0;
+                    const int sl = ii / nb_i, b = ii - sl * nb_i;
+                    const float* hrow = p.mid + ((size_t)t * slots + sl) * inter + b * kQK + lane * 4;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) ev[j][q] = ld_dev(hrow + q);
+                }
+#pragma unroll
+                for (int j = 0; j < kItems; ++j) {
+                    const int i = base + wave + kWaves * j;
+                    if (i < n_items) {  // wave-uniform
+                        float acc[1][2] = {{0.0f, 0.0f}};
+                        if (item_tile(t, rt, i)) {
+                            ARegs<1> a;
+                            a_from_lane_codes(a, quantize_block_q8k(ev[j], lane), lane);
+                            int32_t dsum[1][2], msum[1][2];
+                            compute_tile<1>(etile[j], a, acc, dsum, msum);
+                        }
+                        if (kq == 0) s.term[i * 16 + slot] = acc[0][0];
+                    }
+                }
+            }
+            __syncthreads();
+            if (tid < 16) {
+                // per slot the super-block terms in order, then the slots in routing order (moe_combine_kernel)
+                float acc = 0.0f;
+                for (int k = 0; k < slots; ++k) {
+                    float part = s.term[(k * nb_i) * 16 + tid];
+                    for (int b = 1; b < nb_i; ++b) part = __fadd_rn(part, s.term[(k * nb_i + b) * 16 + tid]);
+                    if (k < top_k) {
+                        const int e = s.ids[t * 8 + k];
+                        const float w = s.wts[t * 8 + k];
+                        if (e < 0 || e >= n_experts || w == 0.0f) continue;
+                        acc = __fadd_rn(acc, __fmul_rn(part, w));
+                    } else {
+                        acc = __fadd_rn(acc, __fmul_rn(part, s.gate[t]));
+                    }
+                }
+                st_dev(p.y + (size_t)t * hidden + rt * 16 + tid, acc);
             }
             __syncthreads();
         }
         {
-            const int rt_h = hidden / 16;
-            for (int u = blockIdx.x; u < n * rt_h; u += gridDim.x) {
-                const int t = u / rt_h, rt = u - t * rt_h;
-                for (int sl = wave; sl < slots; sl += kWaves) {
-                    const bool shared = sl >= top_k;
-                    const int e = shared ? 0 : s.ids[t * 8 + sl];
-                    float acc[1][2] = {{0.0f, 0.0f}};
-                    if (shared || (e >= 0 && e < n_experts)) {  // wave-uniform
-                        const uint8_t* w = shared ? L.sh_down : L.down_exps + (size_t)e * L.down_expert_bytes;
-                        const float* hrow = p.mid + ((size_t)t * slots + sl) * inter;
-                        for (int b = 0; b < nb_i; ++b) {
-                            TileRegs tr;
-                            load_tile(tr, w + tile_offset(rt, b, nb_i), lane);
-                            float ev[4];
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) ev[j] = ld_dev(hrow + b * kQK + lane * 4 + j);
-                            ARegs<1> a;
-                            a_from_lane_codes(a, quantize_block_q8k(ev, lane), lane);
-                            int32_t dsum[1][2], msum[1][2];
-                            compute_tile<1>(tr, a, acc, dsum, msum);
-                        }
-                    }
-                    if (kq == 0) s.part[sl * 16 + slot] = acc[0][0];
-                }
-                __syncthreads();
-                if (tid < 16) {
-                    float acc = 0.0f;
-                    for (int k = 0; k < top_k; ++k) {
-                        const int e = s.ids[t * 8 + k];
-                        const float w = s.wts[t * 8 + k];
-                        if (e < 0 || e >= n_experts || w == 0.0f) continue;
-                        acc = __fadd_rn(acc, __fmul_rn(s.part[k * 16 + tid], w));
-                    }
-                    if (p.has_shared) acc = __fadd_rn(acc, __fmul_rn(s.part[top_k * 16 + tid], s.gate[t]));
-                    st_dev(p.y + (size_t)t * hidden + rt * 16 + tid, acc);
-                }
-                __syncthreads();
-            }
+            // the next layer's first projection (the last layer re-requests its own: unused, but defined)
+            const DecoderLayerDev& N = p.layers[li + 1 < p.n_layers ? li + 1 : li];
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                    if (!p.moe_only) request_dense(ahead_qkv, N.wqkv, N.qkv_rows, nb_h);
+                }))
+                return;
         }
-        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks)) return;
         delta = p.y;
     }
 
@@ -486,7 +603,7 @@ size_t decoder_layers_lds_bytes(const DecoderArgs& a) {
     const int nb_h = a.hidden / kQK, nb_q = a.n_q / kQK;
     const int nb_max = nb_h > nb_q ? nb_h : nb_q;
     return (size_t)nb_max * 4096 + (size_t)nb_max * 8 * 4 + (size_t)a.n * a.hidden * 4 + (size_t)(kWaves - 1) * 2 * 2 * 64 * 4 +
-           (size_t)kMaxSlots * 16 * 4 + (8 + 8 + 8 + 64 + 64 + 4) * 4;
+           (size_t)kMaxSlots * kMaxInterBlocks * 16 * 4 + (8 + 8 + 64 + 64 + 4) * 4;
 }
 
 size_t decoder_sync_bytes(int n_workgroups) {
@@ -500,7 +617,8 @@ hipError_t prepare_decoder_layers(size_t lds_bytes) {
 
 hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream) {
     if (a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
-        a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || n_workgroups < 1 ||
+        a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || a.inter > kMaxInterBlocks * kQK ||
+        n_workgroups < 1 ||
         (!a.moe_only && (a.n_q <= 0 || (a.n_q % kQK))))
         return hipErrorInvalidValue;
     hipLaunchKernelGGL(decoder_layers_kernel, dim3((unsigned)n_workgroups), dim3(kThreads), decoder_layers_lds_bytes(a),

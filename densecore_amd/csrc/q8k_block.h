@@ -28,27 +28,21 @@ struct Q8Lane {
 // Every lane of the wave passes elements 4*lane .. 4*lane+3 of the block.
 __device__ __forceinline__ Q8Lane quantize_block_q8k(const float (&e)[4], int lane) {
     float best_abs = 0.0f, best = 0.0f;
-    int best_idx = lane * 4;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4; ++j) {  // strict >: the first of equal magnitudes stays
         const float a = fabsf(e[j]);
         if (a > best_abs) {
             best_abs = a;
             best = e[j];
-            best_idx = lane * 4 + j;
         }
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float o_abs = __shfl_xor(best_abs, off, 64);
-        const float o_val = __shfl_xor(best, off, 64);
-        const int o_idx = __shfl_xor(best_idx, off, 64);
-        if (o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx)) {
-            best_abs = o_abs;
-            best = o_val;
-            best_idx = o_idx;
-        }
-    }
+    // Wave-wide: the largest magnitude (non-negative floats order like their bit patterns), then the first
+    // lane that holds it -- lanes own ascending element ranges, so that is the first such element.
+    const uint32_t top = wave_max_u32(__float_as_uint(best_abs));
+    const unsigned long long holders = __ballot(__float_as_uint(best_abs) == top);
+    const int first = __builtin_amdgcn_readfirstlane(__ffsll((long long)holders) - 1);
+    best = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(best), first));
+    best_abs = __uint_as_float(top);
     int q[4] = {0, 0, 0, 0};
     Q8Lane r;
     r.d = 0.0f;
@@ -64,8 +58,8 @@ __device__ __forceinline__ Q8Lane quantize_block_q8k(const float (&e)[4], int la
     r.packed = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) | ((uint32_t)(q[2] & 0xff) << 16) |
                ((uint32_t)(q[3] & 0xff) << 24);
     int s = q[0] + q[1] + q[2] + q[3];
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
+    s += (int)dpp_u32<kDppXor1>((uint32_t)s);
+    s += (int)dpp_u32<kDppXor2>((uint32_t)s);
     r.bsum = s;
     return r;
 }

@@ -30,6 +30,15 @@ __device__ __forceinline__ unsigned long long route_key(float v, int id) {
     return ((unsigned long long)hi << 32) | (unsigned long long)(uint32_t)(~(uint32_t)id);
 }
 
+// The largest 64-bit key held by any lane, in every lane: the high words first, then the low words of the
+// lanes that hold that high word (two 32-bit wave maxima instead of a 64-bit butterfly through LDS).
+__device__ __forceinline__ unsigned long long wave_max_key(unsigned long long key) {
+    const uint32_t hi = (uint32_t)(key >> 32), lo = (uint32_t)key;
+    const uint32_t top_hi = wave_max_u32(hi);
+    const uint32_t top_lo = wave_max_u32(hi == top_hi ? lo : 0u);
+    return ((unsigned long long)top_hi << 32) | top_lo;
+}
+
 // softmax over the selected logits, summed in routing order (three reference variants)
 __device__ __forceinline__ void route_weights(const float* l, int top_k, int mode, float* __restrict__ out) {
     float w[8];

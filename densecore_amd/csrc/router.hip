@@ -32,11 +32,7 @@ __device__ __forceinline__ void route_token_block(const float* __restrict__ row,
                 const unsigned long long k = keys[e];
                 best = k > best ? k : best;
             }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                const unsigned long long o = __shfl_xor(best, off, 64);
-                best = o > best ? o : best;
-            }
+            best = wave_max_key(best);
             const int id = (int)~(uint32_t)best;
             if (tid == (id & 63)) keys[id] = 0ull;  // the owning lane is the only one that reads this key again
             if (tid == 0) {
