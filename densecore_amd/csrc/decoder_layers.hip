@@ -62,6 +62,7 @@ struct Shared {
     float* term;    // down-projection terms per (slot, super-block) [kMaxSlots][kMaxInterBlocks][16]
     float* scale;   // [8] rmsnorm scale per token
     float* gate;    // [8] shared-expert gate per token
+    float* vsum;    // [32] partial sums per (token, wavefront of a 256-thread workgroup)
     float* wts;     // [8][8] routing weights
     int32_t* ids;   // [8][8] routed experts
     int* ok;        // barrier verdict of this workgroup
@@ -113,40 +114,42 @@ __device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, i
     return *ok != 0;
 }
 
-// Sum over the columns of `term(c)` in the order of a 256-thread workgroup of the one-node kernels (thread j
-// takes columns j, j + 256, ... with fused multiply-adds, a butterfly inside each wavefront, then
-// (w0 + w1) + (w2 + w3)), evaluated by ONE wavefront: lane l plays threads l, l + 64, l + 128, l + 192.
-template <typename Term>
-__device__ __forceinline__ float sum_like_256_threads(int hidden, int lane, Term term) {
-    float part[4];
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
+// Per-token sums over the columns in the order of a 256-thread workgroup of the one-node kernels: thread j
+// takes columns j, j + 256, ... with fused multiply-adds, a butterfly inside each of the four wavefronts,
+// then (w0 + w1) + (w2 + w3).  Here the (token, wavefront) pairs are spread over the eight wavefronts;
+// term(t, c, acc) returns the running sum with column c of token t added, finish(t, total) consumes a total.
+template <typename Term, typename Finish>
+__device__ __forceinline__ void token_sums(const Shared& s, int n, int hidden, Term term, Finish finish) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = wave; i < 4 * n; i += kWaves) {
+        const int t = i >> 2, v = i & 3;
         float acc = 0.0f;
-        for (int c = v * 64 + lane; c < hidden; c += 256) acc = term(c, acc);
-        part[v] = acc;
-    }
+#pragma unroll 4
+        for (int c = v * 64 + lane; c < hidden; c += 256) acc = term(t, c, acc);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) part[v] += __shfl_xor(part[v], off, 64);
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (lane == 0) s.vsum[i] = acc;
     }
-    return (part[0] + part[1]) + (part[2] + part[3]);
+    __syncthreads();
+    if (tid < n) finish(tid, (s.vsum[4 * tid] + s.vsum[4 * tid + 1]) + (s.vsum[4 * tid + 2] + s.vsum[4 * tid + 3]));
+    __syncthreads();
 }
 
 // xres[t][c] += delta[t][c] (delta: device-scope reads; may be null), then scale[t] = 1/sqrt(mean(x^2) + eps)
-// with the summation order of add_rmsnorm_kernel; one wavefront per token.
+// with the summation order of add_rmsnorm_kernel.
 __device__ __forceinline__ void residual_norm(const Shared& s, const float* delta, int n, int hidden, float eps) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x;
     if (delta) {
         for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = __fadd_rn(s.xres[i], ld_dev(delta + i));
         __syncthreads();
     }
-    if (wave < n) {
-        const float* row = s.xres + wave * hidden;
-        const float total = sum_like_256_threads(hidden, lane, [&](int c, float acc) { return __fmaf_rn(row[c], row[c], acc); });
-        if (lane == 0) s.scale[wave] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)hidden), eps)));
-    }
-    __syncthreads();
+    token_sums(
+        s, n, hidden,
+        [&](int t, int c, float acc) {
+            const float v = s.xres[t * hidden + c];
+            return __fmaf_rn(v, v, acc);
+        },
+        [&](int t, float total) { s.scale[t] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)hidden), eps))); });
 }
 
 // normalised value of column c of token t, as add_rmsnorm_kernel forms it
@@ -179,6 +182,16 @@ __device__ __forceinline__ void load_a_lds(ARegs<1>& a, const Shared& s, int b, 
     for (int j = 0; j < 2; ++j) {
         const int r = 2 * kq + j < n ? 2 * kq + j : n - 1;
         a.yd[0][j] = s.ad[b * 8 + r];
+    }
+}
+
+// Pulls `bytes` bytes at p (16-byte aligned, a multiple of 16) towards this compute unit's caches: the whole
+// workgroup reads them once and folds them into `sink`, which only exists so that the reads survive.
+__device__ __forceinline__ void warm(const void* p, size_t bytes, uint32_t& sink) {
+    const v4u* q = reinterpret_cast<const v4u*>(p);
+    for (size_t i = threadIdx.x; i < bytes / 16; i += kThreads) {
+        const v4u v = q[i];
+        sink ^= v.x ^ v.y ^ v.z ^ v.w;
     }
 }
 
@@ -268,33 +281,6 @@ __device__ __forceinline__ void dense_phase(const Shared& s, const uint8_t* w, i
     }
 }
 
-// Top-k of one token by one wavefront: lane l owns the experts l, l + 64, ...; k rounds of a wave-wide maximum
-// over the 64-bit keys (route_block.h), the owner clears the winner.  Lane 0 then forms the weights.
-__device__ __forceinline__ void route_token_wave(const float* row, bool coherent, int n_experts, int top_k, int mode,
-                                                 int32_t* ids, float* wts, int lane) {
-    unsigned long long key[kKeysPerLane];
-#pragma unroll
-    for (int i = 0; i < kKeysPerLane; ++i) {
-        const int e = lane + 64 * i;
-        key[i] = 0ull;
-        if (e < n_experts) key[i] = route_key(coherent ? ld_dev(row + e) : row[e], e);
-    }
-    float sel[8];
-    for (int r = 0; r < top_k; ++r) {
-        unsigned long long best = 0ull;
-#pragma unroll
-        for (int i = 0; i < kKeysPerLane; ++i) best = key[i] > best ? key[i] : best;
-        best = wave_max_key(best);
-        const int id = (int)~(uint32_t)best;
-#pragma unroll
-        for (int i = 0; i < kKeysPerLane; ++i)
-            if (lane + 64 * i == id) key[i] = 0ull;
-        if (lane == 0) ids[r] = id;
-        sel[r] = route_key_logit(best);
-    }
-    if (lane == 0) route_weights(sel, top_k, mode, wts);
-}
-
 // The A operand of one activation row quantized by this wavefront (row 0 of the tile; the other rows are dead):
 // codes move from the quantizer's lanes into the split-slot operand with eight cross-lane reads per super-block.
 __device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
@@ -337,13 +323,15 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         at += (size_t)kMaxSlots * kMaxInterBlocks * 16 * sizeof(float);
         s.scale = reinterpret_cast<float*>(at);
         s.gate = s.scale + 8;
-        s.wts = s.gate + 8;
+        s.vsum = s.gate + 8;
+        s.wts = s.vsum + 32;
         s.ids = reinterpret_cast<int32_t*>(s.wts + 64);
         s.ok = reinterpret_cast<int*>(s.ids + 64);
     }
     if (ld_dev(p.sync + 2 * kSyncLine) != 0u) return;  // an earlier launch abandoned a barrier: the state is unusable
     uint32_t my_gen = ld_dev(p.sync + kSyncLine);      // cannot move before this workgroup's own first arrival
     const auto nothing = [] {};
+    uint32_t sink = 0u;  // see warm()
 
     // Weights of this workgroup's first row tile of a dense projection, requested a phase ahead.  Workgroups
     // without a row tile fetch tile 0 and never use it, so that the registers are defined on every path.
@@ -356,6 +344,22 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
 
     for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = p.x_in[i];
     __syncthreads();
+
+    // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel; h2 = the MoE block's input
+    auto shared_gates = [&](const DecoderLayerDev& L, bool raw) {
+        if (!p.has_shared) return;
+        if (!L.sh_gate_inp) {
+            if (tid < n) s.gate[tid] = 1.0f;
+            __syncthreads();
+            return;
+        }
+        const float* gi = L.sh_gate_inp;
+        const float* wn = L.ffn_norm;
+        token_sums(
+            s, n, hidden,
+            [&](int t, int c, float acc) { return fmaf(gi[c], raw ? s.xres[t * hidden + c] : normed_at(s, wn, t, hidden, c), acc); },
+            [&](int t, float total) { s.gate[t] = stable_sigmoid(total); });
+    };
 
     const float* delta = nullptr;
     for (int li = 0; li < p.n_layers; ++li) {
@@ -381,7 +385,12 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
             }
             __syncthreads();
             dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden, ahead_wo);
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, nothing)) return;
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                    // what phase C reads that does not depend on o: this workgroup's first router row, the gate vector
+                    if ((int)blockIdx.x < n_experts) warm(L.router + (size_t)blockIdx.x * hidden, (size_t)hidden * 4, sink);
+                    if (p.has_shared && L.sh_gate_inp) warm(L.sh_gate_inp, (size_t)hidden * 4, sink);
+                }))
+                return;
 
             // ---- C: residual add, rmsnorm, Q8_K, router projection -----------------------------------------
             residual_norm(s, p.o, n, hidden, p.eps);
@@ -390,8 +399,9 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
             }
             __syncthreads();
-            // one wavefront per (token, expert), the dot of router_logits_kernel
-            for (int u = wave * gridDim.x + blockIdx.x; u < n * n_experts; u += kWaves * gridDim.x) {
+            // one wavefront per (token, expert), the dot of router_logits_kernel; the last wavefront takes the
+            // first unit so that the gates below, which start with the first wavefronts, run beside it
+            for (int u = (kWaves - 1 - wave) * gridDim.x + blockIdx.x; u < n * n_experts; u += kWaves * gridDim.x) {
                 const int t = u / n_experts, e = u - t * n_experts;
                 const float* wr = L.router + (size_t)e * hidden;
                 float acc = 0.0f;
@@ -406,36 +416,48 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
                 if (lane == 0) st_dev(p.logits + (size_t)t * n_experts + e, acc);
             }
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, nothing)) return;
+            shared_gates(L, false);
+            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                    // the shared expert's gate/up tiles of this workgroup's first unit do not wait for the routing
+                    if (p.has_shared && (int)blockIdx.x < inter / 16) {
+                        warm(L.sh_gate + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
+                        warm(L.sh_up + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
+                    }
+                }))
+                return;
         } else {
             // MoE block alone: x is its (already normalised) input
             for (int t = tid; t < n; t += kThreads) s.scale[t] = 1.0f;
             __syncthreads();
             quantize_rows(s, n, nb_h, [&](int t, int c) { return s.xres[t * hidden + c]; });
             __syncthreads();
+            shared_gates(L, true);
         }
 
         // ---- D: routing, then gate/up + SwiGLU per (token, slot) and for the shared expert -------------------
+        float routed_logit = 0.0f;  // lane k of wavefront t: logit of token t's k-th expert
         if (wave < n) {
             const bool fixed = L.fixed_logits != nullptr;
             const float* row = (fixed ? L.fixed_logits : p.logits) + (size_t)wave * n_experts;
-            route_token_wave(row, !fixed, n_experts, top_k, p.route_mode, s.ids + wave * 8, s.wts + wave * 8, lane);
+            auto load = [&](int e) { return fixed ? row[e] : ld_dev(row + e); };
+            int id;
+            if (n_experts <= 256) route_token_wave<4>(load, n_experts, top_k, lane, id, routed_logit);
+            else route_token_wave<kKeysPerLane>(load, n_experts, top_k, lane, id, routed_logit);
+            if (lane < top_k) s.ids[wave * 8 + lane] = id;
         }
         __syncthreads();
-        if (blockIdx.x == 0 && tid < n * top_k) {
-            const int t = tid / top_k, k = tid - t * top_k;
-            if (p.ids_out) p.ids_out[((size_t)li * n + t) * top_k + k] = s.ids[t * 8 + k];
-            if (p.wts_out) p.wts_out[((size_t)li * n + t) * top_k + k] = s.wts[t * 8 + k];
-        }
         {
             const int rt_i = inter / 16;
             const int pairs = n * top_k;
-            const int units = (pairs + (p.has_shared ? 1 : 0)) * rt_i;
-            // unit u -> (pair or shared pass, row tile); a dropped pair (id out of range) has no weights
+            const int sh_units = p.has_shared ? rt_i : 0;
+            const int units = sh_units + pairs * rt_i;
+            // unit u -> (shared pass or (token, slot) pair, row tile); a dropped pair (id out of range) has no
+            // weights.  The shared expert's units come first: their weights do not wait for the routing and
+            // were pulled into cache during the barrier.
             auto unit_weights = [&](int u, const uint8_t* (&ws)[2], int& t, int& k, int& rt, bool& shared) -> bool {
-                const int g = u / rt_i;
-                rt = u - g * rt_i;
-                shared = g >= pairs;
+                shared = u < sh_units;
+                const int g = shared ? 0 : (u - sh_units) / rt_i;
+                rt = shared ? u : (u - sh_units) - g * rt_i;
                 t = shared ? 0 : g / top_k;
                 k = shared ? top_k : g - t * top_k;
                 const int e = shared ? 0 : s.ids[t * 8 + k];
@@ -447,25 +469,28 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
             TileRegs cur[2], nxt[2];
             const uint8_t* ws[2];
             const uint8_t* wn[2];
-            int t, k, rt, tn, kn, rtn;
-            bool shared, sharedn;
-            bool live = false;
-            if ((int)blockIdx.x < units) {
-                live = unit_weights(blockIdx.x, ws, t, k, rt, shared);
-                if (live) {
-                    const uint8_t* const wc[2] = {ws[0], ws[1]};
-                    fetch_tiles<2>(cur, wc, rt, nb_h);
+            int t = 0, k = 0, rt = 0, tn = 0, kn = 0, rtn = 0;
+            bool shared = false, sharedn = false;
+            // Every fetch is issued whether or not the unit exists: the number of loads in flight is then the same
+            // on every path and the waits can count them.
+            // (a missing unit re-reads `again`, tiles that were fetched a moment ago and still sit in cache)
+            auto fetch_unit = [&](int u, TileRegs (&dst)[2], const uint8_t* (&w)[2], int& tt, int& kk, int& rr, bool& sh,
+                                  const uint8_t* const (&again)[2], int again_rt) -> bool {
+                bool live = false;
+                if (u < units) live = unit_weights(u, w, tt, kk, rr, sh);
+                if (!live) {
+                    w[0] = again[0], w[1] = again[1];
+                    rr = again_rt;
                 }
-            }
+                const uint8_t* const wc[2] = {w[0], w[1]};
+                fetch_tiles<2>(dst, wc, rr, nb_h);
+                return live;
+            };
+            const uint8_t* const cold[2] = {L.gate_exps, L.up_exps};
+            bool live = fetch_unit(blockIdx.x, cur, ws, t, k, rt, shared, cold, 0);
             for (int u = blockIdx.x; u < units; u += gridDim.x) {
-                bool live_n = false;
-                if (u + (int)gridDim.x < units) {
-                    live_n = unit_weights(u + gridDim.x, wn, tn, kn, rtn, sharedn);
-                    if (live_n) {
-                        const uint8_t* const wc[2] = {wn[0], wn[1]};
-                        fetch_tiles<2>(nxt, wc, rtn, nb_h);
-                    }
-                }
+                const uint8_t* const here[2] = {ws[0], ws[1]};
+                const bool live_n = fetch_unit(u + gridDim.x, nxt, wn, tn, kn, rtn, sharedn, here, rt);
                 if (live) {  // the whole workgroup takes the same branch
                     const uint8_t* const wc[2] = {ws[0], ws[1]};
                     float acc[2][1][2];
@@ -483,11 +508,9 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                     __syncthreads();
                 }
                 live = live_n;
-                if (live_n) {
-                    cur[0] = nxt[0], cur[1] = nxt[1];
-                    ws[0] = wn[0], ws[1] = wn[1];
-                    t = tn, k = kn, rt = rtn, shared = sharedn;
-                }
+                cur[0] = nxt[0], cur[1] = nxt[1];
+                ws[0] = wn[0], ws[1] = wn[1];
+                t = tn, k = kn, rt = rtn, shared = sharedn;
             }
         }
 
@@ -517,49 +540,58 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
             }))
             return;
 
-        if (p.has_shared) {  // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel
-            if (wave < n) {
-                float g = 1.0f;
-                if (L.sh_gate_inp) {
-                    const float* gi = L.sh_gate_inp;
-                    const float* wn = L.ffn_norm;
-                    const bool raw = p.moe_only != 0;
-                    g = stable_sigmoid(sum_like_256_threads(hidden, lane, [&](int c, float acc) {
-                        return fmaf(gi[c], raw ? s.xres[wave * hidden + c] : normed_at(s, wn, wave, hidden, c), acc);
-                    }));
-                }
-                if (lane == 0) s.gate[wave] = g;
+        // quantize this wavefront's hidden blocks, multiply them by the tiles in etile[], park the terms in LDS
+        auto load_hidden = [&](float (&ev)[kItems][4], int t, int base) {
+#pragma unroll
+            for (int j = 0; j < kItems; ++j) {
+                const int i = base + wave + kWaves * j;
+                const int ii = i < n_items ? i : 0;
+                const int sl = ii / nb_i, b = ii - sl * nb_i;
+                const float* hrow = p.mid + ((size_t)t * slots + sl) * inter + b * kQK + lane * 4;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) ev[j][q] = ld_dev(hrow + q);
             }
-            __syncthreads();
+        };
+        auto multiply_items = [&](const float (&ev)[kItems][4], int t, int rt, int base) {
+#pragma unroll
+            for (int j = 0; j < kItems; ++j) {
+                const int i = base + wave + kWaves * j;
+                if (i < n_items) {  // wave-uniform
+                    float acc[1][2] = {{0.0f, 0.0f}};
+                    if (item_tile(t, rt, i)) {
+                        ARegs<1> a;
+                        a_from_lane_codes(a, quantize_block_q8k(ev[j], lane), lane);
+                        int32_t dsum[1][2], msum[1][2];
+                        compute_tile<1>(etile[j], a, acc, dsum, msum);
+                    }
+                    if (kq == 0) s.term[i * 16 + slot] = acc[0][0];
+                }
+            }
+        };
+        float ev[kItems][4];
+        if (e_unit) load_hidden(ev, blockIdx.x / rt_h, 0);
+        // the routing weights are first needed by the combine below: formed while the hidden rows travel
+        if (wave < n) {
+            const float w = route_weight_lane(routed_logit, lane, top_k, p.route_mode);
+            if (lane < top_k) {
+                s.wts[wave * 8 + lane] = w;
+                if (blockIdx.x == 0) {
+                    if (p.ids_out) p.ids_out[((size_t)li * n + wave) * top_k + lane] = s.ids[wave * 8 + lane];
+                    if (p.wts_out) p.wts_out[((size_t)li * n + wave) * top_k + lane] = w;
+                }
+            }
         }
         for (int u = blockIdx.x; u < n * rt_h; u += gridDim.x) {
             const int t = u / rt_h, rt = u - t * rt_h;
-            for (int base = 0; base < n_items; base += kWaves * kItems) {
-                if (u != (int)blockIdx.x || base != 0) fetch_items(t, rt, base);
-                float ev[kItems][4];
-#pragma unroll
-                for (int j = 0; j < kItems; ++j) {
-                    const int i = base + wave + kWaves * j;
-                    const int ii = i < n_items ? i : 0;
-                    const int sl = ii / nb_i, b = ii - sl * nb_i;
-                    const float* hrow = p.mid + ((size_t)t * slots + sl) * inter + b * kQK + lane * 4;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) ev[j][q] = ld_dev(hrow + q);
-                }
-#pragma unroll
-                for (int j = 0; j < kItems; ++j) {
-                    const int i = base + wave + kWaves * j;
-                    if (i < n_items) {  // wave-uniform
-                        float acc[1][2] = {{0.0f, 0.0f}};
-                        if (item_tile(t, rt, i)) {
-                            ARegs<1> a;
-                            a_from_lane_codes(a, quantize_block_q8k(ev[j], lane), lane);
-                            int32_t dsum[1][2], msum[1][2];
-                            compute_tile<1>(etile[j], a, acc, dsum, msum);
-                        }
-                        if (kq == 0) s.term[i * 16 + slot] = acc[0][0];
-                    }
-                }
+            if (u != (int)blockIdx.x) {  // the first unit's tiles and hidden rows are already on their way
+                fetch_items(t, rt, 0);
+                load_hidden(ev, t, 0);
+            }
+            multiply_items(ev, t, rt, 0);
+            for (int base = kWaves * kItems; base < n_items; base += kWaves * kItems) {
+                fetch_items(t, rt, base);
+                load_hidden(ev, t, base);
+                multiply_items(ev, t, rt, base);
             }
             __syncthreads();
             if (tid < 16) {
@@ -595,6 +627,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
     // ---- the last residual add (or, for the MoE block alone, its output as it is) ---------------------------
     for (int i = blockIdx.x * kThreads + tid; i < n * hidden; i += gridDim.x * kThreads)
         p.out[i] = p.moe_only ? ld_dev(p.y + i) : __fadd_rn(s.xres[i], ld_dev(p.y + i));
+    if (sink == 0x9e3779b9u && p.n < 0) p.out[0] = 0.0f;  // never true: keeps the warm-up reads alive
 }
 
 }  // namespace
@@ -603,7 +636,7 @@ size_t decoder_layers_lds_bytes(const DecoderArgs& a) {
     const int nb_h = a.hidden / kQK, nb_q = a.n_q / kQK;
     const int nb_max = nb_h > nb_q ? nb_h : nb_q;
     return (size_t)nb_max * 4096 + (size_t)nb_max * 8 * 4 + (size_t)a.n * a.hidden * 4 + (size_t)(kWaves - 1) * 2 * 2 * 64 * 4 +
-           (size_t)kMaxSlots * kMaxInterBlocks * 16 * 4 + (8 + 8 + 64 + 64 + 4) * 4;
+           (size_t)kMaxSlots * kMaxInterBlocks * 16 * 4 + (8 + 8 + 32 + 64 + 64 + 4) * 4;
 }
 
 size_t decoder_sync_bytes(int n_workgroups) {

@@ -87,6 +87,90 @@ __device__ __forceinline__ void route_weights(const float* l, int top_k, int mod
     }
 }
 
+__device__ __forceinline__ float route_key_logit(unsigned long long key);
+
+// ---- routing of one token by one wavefront ---------------------------------------------------------
+// 32-bit order key of a logit: larger = earlier in the routing order, NaN = 1 (after every number), 0 = absent.
+__device__ __forceinline__ uint32_t route_key32(float v) { return (uint32_t)(route_key(v, 0) >> 32) + 1u; }
+__device__ __forceinline__ float route_key32_logit(uint32_t key) { return route_key_logit((unsigned long long)(key - 1u) << 32); }
+
+// float maximum over lanes 0..7 (fmaxf semantics: a NaN operand is ignored), valid in lanes 0..7
+__device__ __forceinline__ float max_first8(float x) {
+    x = fmaxf(x, __uint_as_float(dpp_u32<kDppXor1>(__float_as_uint(x))));
+    x = fmaxf(x, __uint_as_float(dpp_u32<kDppXor2>(__float_as_uint(x))));
+    x = fmaxf(x, __uint_as_float(dpp_u32<kDppHalfMirror>(__float_as_uint(x))));
+    return x;
+}
+
+// route_weights with lane k holding logit k (k < top_k <= 8): the same maxima, the same exponentials, the
+// denominator summed in routing order by reading the lanes one after the other.  Returns lane k's weight.
+__device__ __forceinline__ float route_weight_lane(float l, int lane, int top_k, int mode) {
+    const bool in = lane < top_k;
+    const bool fin = isfinite(l);
+    const float uni = __fdiv_rn(1.0f, (float)top_k);
+    float mx = max_first8(in && (mode == 1 || fin) ? l : -INFINITY);
+    mx = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(mx)));
+    if (mode == 1 && !isfinite(mx)) mx = 0.0f;
+    const bool all_finite = __ballot(in && !fin) == 0ull;
+    const float w = expf(__fsub_rn(l, mx));
+    // which slots enter the denominator
+    bool counted;
+    if (mode == 0) counted = in && all_finite && isfinite(mx);
+    else if (mode == 1) counted = in;
+    else counted = in && fin && isfinite(mx);
+    const unsigned long long counted_mask = __ballot(counted);
+    float den = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float wk = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w), k));
+        if ((counted_mask >> k) & 1ull) den = __fadd_rn(den, wk);
+    }
+    if (mode == 0) return (!(den > 0.0f) || !isfinite(den)) ? uni : __fdiv_rn(w, den);
+    if (mode == 1) return __fdiv_rn(w, fmaxf(den, 6.103515625e-5f));
+    const bool uniform = !(den > 0.0f) || !isfinite(den);
+    den = uniform ? 1.0f : fmaxf(den, 6.103515625e-5f);
+    return (uniform || !fin || !isfinite(mx)) ? uni : __fdiv_rn(w, den);
+}
+
+// Stable top-k of one token (ComputeQwenNativeMoEStableTopK, core/src/llm/moe/native.cpp:610-645) and its
+// weights.  Lane l owns the experts l, l + 64, ...: per round a wave-wide maximum of the 32-bit keys, the
+// lowest expert id among the holders of that key (ballots, scanned in expert order), and the owner retires it.
+// load(e) returns logit e.  Lanes k < top_k end up with expert k of the routing order and its logit
+// (route_weight_lane turns those logits into the weights).
+template <int KPL, typename Load>
+__device__ __forceinline__ void route_token_wave(Load load, int n_experts, int top_k, int lane, int& id_out,
+                                                 float& logit_out) {
+    uint32_t key[KPL];
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) {
+        const int e = lane + 64 * i;
+        key[i] = e < n_experts ? route_key32(load(e)) : 0u;
+    }
+    float my_logit = 0.0f;
+    int my_id = -1;
+    for (int r = 0; r < top_k; ++r) {
+        uint32_t best = key[0];
+#pragma unroll
+        for (int i = 1; i < KPL; ++i) best = key[i] > best ? key[i] : best;
+        const uint32_t top = wave_max_u32(best);
+        int id = -1;
+#pragma unroll
+        for (int i = 0; i < KPL; ++i) {
+            const unsigned long long holders = __ballot(key[i] == top);
+            if (id < 0 && holders != 0ull) id = 64 * i + __ffsll((long long)holders) - 1;
+        }
+#pragma unroll
+        for (int i = 0; i < KPL; ++i)
+            if (lane + 64 * i == id) key[i] = 0u;
+        if (lane == r) {
+            my_logit = route_key32_logit(top);
+            my_id = id;
+        }
+    }
+    id_out = my_id;
+    logit_out = my_logit;
+}
+
 // The logit behind a route_key (NaN comes back as a canonical NaN, -0 as +0: neither changes a weight).
 __device__ __forceinline__ float route_key_logit(unsigned long long key) {
     const uint32_t hi = (uint32_t)(key >> 32);
