@@ -363,7 +363,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
 
     const float* delta = nullptr;
     for (int li = 0; li < p.n_layers; ++li) {
-        const DecoderLayerDev& L = p.layers[li];
+        const DecoderLayerDev& L = p.layers ? p.layers[li] : p.single;
 
         if (!p.moe_only) {
             // ---- A: residual add, rmsnorm, Q8_K, qkv projection -------------------------------------------
@@ -615,7 +615,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         }
         {
             // the next layer's first projection (the last layer re-requests its own: unused, but defined)
-            const DecoderLayerDev& N = p.layers[li + 1 < p.n_layers ? li + 1 : li];
+            const DecoderLayerDev& N = p.layers ? p.layers[li + 1 < p.n_layers ? li + 1 : li] : p.single;
             if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
                     if (!p.moe_only) request_dense(ahead_qkv, N.wqkv, N.qkv_rows, nb_h);
                 }))
@@ -649,7 +649,7 @@ hipError_t prepare_decoder_layers(size_t lds_bytes) {
 }
 
 hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream) {
-    if (a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
+    if ((!a.layers && (!a.moe_only || a.n_layers != 1)) || a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
         a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || a.inter > kMaxInterBlocks * kQK ||
         n_workgroups < 1 ||
         (!a.moe_only && (a.n_q <= 0 || (a.n_q % kQK))))

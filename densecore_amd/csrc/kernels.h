@@ -127,6 +127,7 @@ hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,
 // device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.
 constexpr int kDecoderMaxExperts = 512;
+constexpr int kMoeFusedMaxTokens = 2;  // widest MoE block that mq_moe_layer_q4k runs as one launch
 struct DecoderLayerDev {               // one per layer, in device memory
     const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]
     const uint8_t* wo = nullptr;       // [hidden x n_q]; its input is qkv[:, :n_q]
@@ -145,7 +146,8 @@ struct DecoderLayerDev {               // one per layer, in device memory
     const float* sh_gate_inp = nullptr;  // fp32 [hidden] or null (gate = 1)
 };
 struct DecoderArgs {
-    const DecoderLayerDev* layers = nullptr;
+    const DecoderLayerDev* layers = nullptr;  // device table; null: one MoE block described by `single`
+    DecoderLayerDev single;
     int n_layers = 0;
     int n = 0;                         // tokens, 1..8
     int hidden = 0, inter = 0, n_q = 0, n_experts = 0, top_k = 0;
