@@ -162,7 +162,8 @@ int reserve_counters(size_t count) {
 int alloc_weight(int type, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
     if (!out) return fail(MQ_ERR_INVALID, "null output handle");
     *out = nullptr;
-    if (type != kTypeQ4K && type != kTypeQ5K) return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12) and Q5_K (13) weights are supported", type);
+    if (type != kTypeQ4K && type != kTypeQ5K && type != kTypeQ6K)
+        return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12), Q5_K (13) and Q6_K (14) weights are supported", type);
     if (rows <= 0 || cols <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "rows, cols and n_experts must be positive");
     if (cols % kQK) return fail(MQ_ERR_INVALID, "cols %lld is not a multiple of 256", (long long)cols);
     mq_weight* w = new mq_weight;
@@ -247,7 +248,8 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
 int mq_weight_upload_typed(int ggml_type, const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts,
                            size_t row_bytes, size_t expert_bytes, mq_weight** out) {
     if (int rc = check_ready()) return rc;
-    if (ggml_type != kTypeQ4K && ggml_type != kTypeQ5K) return fail(MQ_ERR_UNSUPPORTED, "mq_weight_upload: ggml type %d (only 12 = Q4_K and 13 = Q5_K)", ggml_type);
+    if (ggml_type != kTypeQ4K && ggml_type != kTypeQ5K && ggml_type != kTypeQ6K)
+        return fail(MQ_ERR_UNSUPPORTED, "mq_weight_upload: ggml type %d (only 12 = Q4_K, 13 = Q5_K and 14 = Q6_K)", ggml_type);
     if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_upload: null host pointer");
     if (cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_weight_upload: cols %lld is not a positive multiple of 256", (long long)cols);
     const size_t min_row = (size_t)(cols / kQK) * (size_t)block_bytes_of(ggml_type);

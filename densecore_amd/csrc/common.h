@@ -51,9 +51,44 @@ __host__ __device__ inline int tile_word_offset(int r, int word) {
 constexpr int kQ5Block = 176;
 constexpr int kTile5Bytes = kTileRows * kQ5Block;  // 2816
 constexpr int kTileHBytes = kTileBytes;            // offset of the qh part
-constexpr int kTypeQ4K = 12, kTypeQ5K = 13;        // ggml_type values
-__host__ __device__ inline int tile_bytes_of(int type) { return type == kTypeQ5K ? kTile5Bytes : kTileBytes; }
-__host__ __device__ inline int block_bytes_of(int type) { return type == kTypeQ5K ? kQ5Block : kQ4Block; }
+constexpr int kTypeQ4K = 12, kTypeQ5K = 13, kTypeQ6K = 14;  // ggml_type values
+
+// ---------------------------------------------------------------------------------------------
+// Q6_K (block_q6_K, 210 bytes: ql[128] low nibbles, qh[64] top two bits, scales[16] signed bytes -- one per
+// 16 weights --, fp16 d; core/src/llm/matmul/q6_small_batch.h:13-24,56-76).  Element 128 j + 32 z + l has
+// nibble ql[64 j + 32 (z & 1) + l] (low for z < 2, high otherwise) and top bits (qh[32 j + l] >> 2 z) & 3; the
+// weight is d * scale * (code - 32).  Tile of 16 rows x one super-block, 3392 bytes:
+//   bytes [j*1024 + (kq*16 + r)*16, +16), j = 0,1 = ql[64 j + 8 kq .. +7], ql[64 j + 32 + 8 kq .. +7] of row r:
+//        low nibbles are the 64-weight chunk 2 j of the MFMA loop, high nibbles chunk 2 j + 1
+//   bytes [2048 + (kq*16 + r)*16, +16)            = qh[8 kq .. +7], qh[32 + 8 kq .. +7], every byte XOR 0xAA:
+//        with bit 5 of each code flipped the six bits are the two's complement of (code - 32), so that
+//        (bits << 2) read as a signed byte is 4 * (code - 32) -- the B operand needs no subtraction
+//   bytes [3072 + r*16, +16)                      = scales[16] of row r
+//   bytes [3328 + r*4, +4)                        = fp16 d of row r, two zero bytes
+// Words of a block_q6_K as the re-tiling kernels move them: 0..15 ql, 16..23 qh, 24..25 scales (8 bytes each),
+// 26 = d (2 bytes).
+// ---------------------------------------------------------------------------------------------
+constexpr int kQ6Block = 210;
+constexpr int kTile6HOff = 2048, kTile6SOff = 3072, kTile6DOff = 3328;
+constexpr int kTile6Bytes = 3392;
+__host__ __device__ inline int tile_word_offset_q6(int r, int word) {
+    if (word < 16) {
+        const int x = word * 8, j = x >> 6, within = x & 63;
+        return j * 1024 + (((within & 31) >> 3) * 16 + r) * 16 + (within >> 5) * 8;
+    }
+    if (word < 24) {
+        const int x = (word - 16) * 8, j = x >> 5;
+        return kTile6HOff + (((x & 31) >> 3) * 16 + r) * 16 + j * 8;
+    }
+    if (word < 26) return kTile6SOff + r * 16 + (word - 24) * 8;
+    return kTile6DOff + r * 4;
+}
+__host__ __device__ inline int tile_bytes_of(int type) {
+    return type == kTypeQ6K ? kTile6Bytes : type == kTypeQ5K ? kTile5Bytes : kTileBytes;
+}
+__host__ __device__ inline int block_bytes_of(int type) {
+    return type == kTypeQ6K ? kQ6Block : type == kTypeQ5K ? kQ5Block : kQ4Block;
+}
 __host__ __device__ inline int tile_word_offset_q5(int r, int word) {
     if (word < 2) return kTileQBytes + r * 16 + word * 8;
     if (word < 6) return kTileHBytes + ((word - 2) * 16 + r) * 8;

@@ -110,6 +110,96 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
     }
 }
 
+// ---- Q6_K (tile layout in common.h) -------------------------------------------------------------------
+struct TileRegs6 {
+    v4u ql0, ql1;  // nibbles of the two 128-weight halves
+    v4u qh;        // top bits: .x .y half 0, .z .w half 1 (bit 5 of every code already flipped)
+    v4u sc;        // the row's 16 signed scales, byte g = scale of weights 16 g .. 16 g + 15
+    uint32_t d;    // fp16 d in the low half
+};
+
+__device__ __forceinline__ void load_tile6(TileRegs6& t, const uint8_t* tile, int lane) {
+    t.ql0 = load_stream16(tile + lane * 16);
+    t.ql1 = load_stream16(tile + 1024 + lane * 16);
+    t.qh = load_stream16(tile + kTile6HOff + lane * 16);
+    t.sc = load_stream16(tile + kTile6SOff + (lane & 15) * 16);
+    t.d = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(tile + kTile6DOff + (lane & 15) * 4));
+}
+
+// One Q6_K tile against up to 8 activation rows.  The B bytes are (six code bits) << 2, i.e. 4 * (code - 32) as a
+// signed byte; scales apply per 16 weights, so every 64-weight chunk takes two MFMAs, one with the activations of
+// k-groups 0..1 (weights 0..15 of each 32-wide half) and one with those of k-groups 2..3 (weights 16..31): the four
+// sums that come out are the chunk's four 16-weight groups.  dot_out = sum_g scale_g * sum (code - 32) * q8 exactly
+// (core/src/llm/matmul/q6_small_batch.h:56-83); fp32: acc = fma(d * yd, float(dot), acc) (:84-86).
+template <int TT>
+__device__ __forceinline__ void compute_tile6(const TileRegs6& t, const ARegs<TT>& a, float (&acc)[TT][2],
+                                              int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2], int lane) {
+    const uint32_t keep_lo = (lane & 32) ? 0u : 0xffffffffu;  // k-groups 0 and 1
+    const uint32_t keep_hi = ~keep_lo;
+    const uint32_t qlw[8] = {t.ql0.x, t.ql0.y, t.ql0.z, t.ql0.w, t.ql1.x, t.ql1.y, t.ql1.z, t.ql1.w};
+    const uint32_t qhw[4] = {t.qh.x, t.qh.y, t.qh.z, t.qh.w};
+    const uint32_t scw[4] = {t.sc.x, t.sc.y, t.sc.z, t.sc.w};
+    int32_t dot[TT][2];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) dot[tt][0] = dot[tt][1] = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {  // 64-weight chunk: half j = c / 2, nibble side hn = c % 2
+        const int j = c >> 1, hn = c & 1;
+        v4i b_q;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {  // dwords 0,1: first 32 weights of the chunk (z = 2 hn), dwords 2,3: z = 2 hn + 1
+            const int z = 2 * hn + (w >> 1);
+            const uint32_t nib = (hn ? qlw[4 * j + w] >> 2 : qlw[4 * j + w] << 2) & 0x3c3c3c3cu;
+            const uint32_t hi = qhw[2 * j + (w & 1)];
+            const uint32_t top = z == 3 ? hi : hi << (6 - 2 * z);
+            b_q[w] = (int)((top & 0xc0c0c0c0u) | nib);
+        }
+        const int s0 = (int)(int8_t)(scw[c] & 0xffu), s1 = (int)(int8_t)((scw[c] >> 8) & 0xffu);
+        const int s2 = (int)(int8_t)((scw[c] >> 16) & 0xffu), s3 = (int)(int8_t)(scw[c] >> 24);
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+            const v4u av = a.q[tt][c];
+            const v4i a_lo = {(int)(av.x & keep_lo), (int)(av.y & keep_lo), (int)(av.z & keep_lo), (int)(av.w & keep_lo)};
+            const v4i a_hi = {(int)(av.x & keep_hi), (int)(av.y & keep_hi), (int)(av.z & keep_hi), (int)(av.w & keep_hi)};
+            const v4i zero = {0, 0, 0, 0};
+            // p[0], p[2]: first 32-wide half of the chunk for rows 2kq and 2kq+1; p[1], p[3]: second half
+            const v4i pl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b_q, zero, 0, 0, 0);
+            const v4i ph = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b_q, zero, 0, 0, 0);
+            dot[tt][0] += __mul24(pl[0], s0) + __mul24(ph[0], s1) + __mul24(pl[1], s2) + __mul24(ph[1], s3);
+            dot[tt][1] += __mul24(pl[2], s0) + __mul24(ph[2], s1) + __mul24(pl[3], s2) + __mul24(ph[3], s3);
+        }
+    }
+    const float wd = half_bits_to_float(t.d & 0xffffu);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int32_t isum = dot[tt][j] >> 2;  // the B bytes carried a factor 4
+            acc[tt][j] = __fmaf_rn(__fmul_rn(a.yd[tt][j], wd), (float)isum, acc[tt][j]);
+            dot_out[tt][j] = isum;
+            min_out[tt][j] = 0;
+        }
+    }
+}
+
+// ---- one name per weight type ---------------------------------------------------------------------------
+constexpr int kWtQ4 = 0, kWtQ5 = 1, kWtQ6 = 2;
+template <int WT> struct TileOf { using Regs = TileRegs; };
+template <> struct TileOf<kWtQ6> { using Regs = TileRegs6; };
+template <int WT> constexpr int tile_stride() { return WT == kWtQ6 ? kTile6Bytes : WT == kWtQ5 ? kTile5Bytes : kTileBytes; }
+
+template <int WT>
+__device__ __forceinline__ void load_tile_wt(typename TileOf<WT>::Regs& t, const uint8_t* tile, int lane) {
+    if constexpr (WT == kWtQ6) load_tile6(t, tile, lane);
+    else load_tile<WT == kWtQ5>(t, tile, lane);
+}
+template <int TT, int WT>
+__device__ __forceinline__ void compute_tile_wt(const typename TileOf<WT>::Regs& t, const ARegs<TT>& a, float (&acc)[TT][2],
+                                                int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2], int lane) {
+    if constexpr (WT == kWtQ6) compute_tile6<TT>(t, a, acc, dot_out, min_out, lane);
+    else compute_tile<TT, WT == kWtQ5>(t, a, acc, dot_out, min_out);
+}
+
 #endif
 
 }  // namespace mq

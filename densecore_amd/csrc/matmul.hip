@@ -62,18 +62,18 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
 // arithmetic: HBM latency under load is 1.5-2.5 us, so a CU needs on the order of 100 KB of
 // outstanding tile loads.  A stage is one super-block's activations (A operand) plus the NMAT
 // weight tiles that share them; at 2 waves per SIMD the register file holds four such stages.
-template <int NMAT, int TT>
+template <int NMAT, int TT, int WT>
 struct Depth {
-    static constexpr int kStages = TT == 1 ? (NMAT == 2 ? 3 : 4) : 2;
+    static constexpr int kStages = WT == kWtQ6 ? (TT == 1 && NMAT == 1 ? 3 : 2) : TT == 1 ? (NMAT == 2 ? 3 : 4) : 2;
 };
 
 // One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
 // waves split the super-blocks of the row.  NMAT == 2: gate and up tiles of the same rows share
 // the activations in registers and meet in silu(gate)*up.
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, bool Q5>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
-    constexpr int kTileStride = Q5 ? kTile5Bytes : kTileBytes;
-    constexpr int S = Depth<NMAT, TT>::kStages;
+    constexpr int kTileStride = tile_stride<WT>();
+    constexpr int S = Depth<NMAT, TT, WT>::kStages;
     extern __shared__ float red[];  // [W-1][NMAT][TT][2][64]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps tile addresses scalar
@@ -190,7 +190,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
         if (wave < nb) {
             const int per_rt = (int)((nb - wave + n_waves - 1) / n_waves);  // super-blocks of this wave per row tile
             const int cnt = per_rt * rt_count;                              // stages of this wave
-            TileRegs ring_t[S][NMAT];
+            typename TileOf<WT>::Regs ring_t[S][NMAT];
             ARegs<TT> ring_a[S];
             // Requests past the wave's last super-block are pointed at the (cache-resident)
             // activation buffer instead of being skipped: the number of loads per stage stays
@@ -203,14 +203,14 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 const int b = rt_per_wg > 1 ? t % per_rt : t;
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    load_tile<Q5>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : p.aq, lane);
+                    load_tile_wt<WT>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : p.aq, lane);
                 load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             };
             auto consume = [&](int st, int i) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][2], msum[TT][2];
-                    compute_tile<TT, Q5>(ring_t[st][m], ring_a[st], acc[m], dsum, msum);
+                    compute_tile_wt<TT, WT>(ring_t[st][m], ring_a[st], acc[m], dsum, msum, lane);
                     if (DEBUG && p.dbg_dot) {  // debug launches own one row tile per workgroup
                         const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;
@@ -311,15 +311,15 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     }
 }
 
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, bool Q5>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT>
 hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
     if (start && stop) {
         // the events take the dispatch's own begin / end timestamps: no extra packets around the kernel
-        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, Q5>), grid, dim3(64 * waves), lds, stream, start, stop,
+        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT>), grid, dim3(64 * waves), lds, stream, start, stop,
                               0, a);
     } else {
-        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, Q5>), grid, dim3(64 * waves), lds, stream, a);
+        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT>), grid, dim3(64 * waves), lds, stream, a);
     }
     return hipGetLastError();
 }
@@ -346,8 +346,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int64_t rowtiles = (a.rows + 15) / 16;
     const int nmat = a.swiglu ? 2 : 1;
     const bool debug = a.dbg_dot != nullptr;
-    const bool q5 = a.wtype == kTypeQ5K;
-    if (a.wtype != kTypeQ4K && a.wtype != kTypeQ5K) return hipErrorInvalidValue;
+    if (a.wtype != kTypeQ4K && a.wtype != kTypeQ5K && a.wtype != kTypeQ6K) return hipErrorInvalidValue;
     // widest activation group this launch can see decides how many 8-row token tiles a pass holds
     const int64_t widest = a.grouped ? (a.n > a.sh_tokens ? a.n : a.sh_tokens) : a.n;
     // Expert groups rarely hold more than 8 rows at decode widths; the few that do (and the shared
@@ -366,16 +365,17 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     }
     const dim3 grid((unsigned)(rowtiles / b.rt_per_wg), (unsigned)groups);
 
-#define MQ_LAUNCH(NM, T)                                                              \
-    do {                                                                              \
-        if (q5) {                                                                                         \
-            if (a.grouped) return launch_one<NM, T, true, false, true>(b, waves, grid, stream, start, stop); \
-            if (debug) return launch_one<NM, T, false, true, true>(b, waves, grid, stream, start, stop);     \
-            return launch_one<NM, T, false, false, true>(b, waves, grid, stream, start, stop);               \
-        }                                                                                                 \
-        if (a.grouped) return launch_one<NM, T, true, false, false>(b, waves, grid, stream, start, stop);    \
-        if (debug) return launch_one<NM, T, false, true, false>(b, waves, grid, stream, start, stop);        \
-        return launch_one<NM, T, false, false, false>(b, waves, grid, stream, start, stop);                  \
+#define MQ_LAUNCH_WT(NM, T, W)                                                                            \
+    do {                                                                                                  \
+        if (a.grouped) return launch_one<NM, T, true, false, W>(b, waves, grid, stream, start, stop);     \
+        if (debug) return launch_one<NM, T, false, true, W>(b, waves, grid, stream, start, stop);         \
+        return launch_one<NM, T, false, false, W>(b, waves, grid, stream, start, stop);                   \
+    } while (0)
+#define MQ_LAUNCH(NM, T)                                 \
+    do {                                                 \
+        if (a.wtype == kTypeQ6K) MQ_LAUNCH_WT(NM, T, kWtQ6); \
+        if (a.wtype == kTypeQ5K) MQ_LAUNCH_WT(NM, T, kWtQ5); \
+        MQ_LAUNCH_WT(NM, T, kWtQ4);                      \
     } while (0)
 
     if (nmat == 1) {
@@ -386,6 +386,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
         MQ_LAUNCH(2, 2);
     }
 #undef MQ_LAUNCH
+#undef MQ_LAUNCH_WT
     return hipSuccess;
 }
 

@@ -1,6 +1,7 @@
-// Weight re-tiling (ggml block_q4_K / block_q5_K rows <-> the 16-row tile layouts of common.h) and the
-// on-device synthetic fill.  One thread moves one 8-byte word of a block; each such word lands in one
-// contiguous 8-byte slot of a tile (tile_word_offset, tile_word_offset_q5).
+// Weight re-tiling (ggml block_q4_K / block_q5_K / block_q6_K rows <-> the 16-row tile layouts of common.h)
+// and the on-device synthetic fill.  One thread moves one 8-byte word of a block; each such word lands in one
+// contiguous 8-byte slot of a tile (tile_word_offset, tile_word_offset_q5, tile_word_offset_q6).  The last
+// "word" of a block_q6_K is its two-byte d.
 #include "common.h"
 #include "kernels.h"
 
@@ -8,8 +9,12 @@ namespace mq {
 
 namespace {
 
-// 8-byte words per block: 18 (Q4_K) or 22 (Q5_K)
-__host__ __device__ inline int words_per_block(int type) { return block_bytes_of(type) / 8; }
+// 8-byte words per block: 18 (Q4_K), 22 (Q5_K), 26 + the two-byte d (Q6_K)
+__host__ __device__ inline int words_per_block(int type) { return type == kTypeQ6K ? 27 : block_bytes_of(type) / 8; }
+// Q6_K: the qh words are stored with bit 5 of every code flipped (common.h)
+__host__ __device__ inline uint64_t stored_form(uint64_t v, int type, int word) {
+    return (type == kTypeQ6K && word >= 16 && word < 24) ? v ^ 0xAAAAAAAAAAAAAAAAull : v;
+}
 
 __device__ __forceinline__ bool decode_word(int64_t idx, int64_t rows, int64_t nb, int type, int64_t& row, int64_t& b,
                                             int& word) {
@@ -25,8 +30,11 @@ __device__ __forceinline__ bool decode_word(int64_t idx, int64_t rows, int64_t n
 
 // where word `word` of row r's block lives inside its tile
 __device__ __forceinline__ size_t word_in_tiles(int64_t row, int64_t b, int64_t nb, int word, int type) {
+    const int r = (int)(row & 15);
     return tile_offset(row >> 4, b, nb, tile_bytes_of(type)) +
-           (size_t)(type == kTypeQ5K ? tile_word_offset_q5((int)(row & 15), word) : tile_word_offset((int)(row & 15), word));
+           (size_t)(type == kTypeQ6K   ? tile_word_offset_q6(r, word)
+                    : type == kTypeQ5K ? tile_word_offset_q5(r, word)
+                                       : tile_word_offset(r, word));
 }
 
 __global__ void __launch_bounds__(256) tile_weights_kernel(const uint8_t* __restrict__ raw, int64_t rows, int64_t nb,
@@ -41,8 +49,12 @@ __global__ void __launch_bounds__(256) tile_weights_kernel(const uint8_t* __rest
     uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
     // the blocks are only 2-byte aligned in general: go through 2-byte loads to stay correct for odd host strides
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(src);
+    if (type == kTypeQ6K && word == 26) {  // fp16 d, padded to four bytes
+        *reinterpret_cast<uint32_t*>(dst) = (uint32_t)s16[0];
+        return;
+    }
     const uint64_t v = (uint64_t)s16[0] | ((uint64_t)s16[1] << 16) | ((uint64_t)s16[2] << 32) | ((uint64_t)s16[3] << 48);
-    *reinterpret_cast<uint64_t*>(dst) = v;
+    *reinterpret_cast<uint64_t*>(dst) = stored_form(v, type, word);
 }
 
 __global__ void __launch_bounds__(256) untile_weights_kernel(const uint8_t* __restrict__ tiled, int64_t rows,
@@ -56,8 +68,12 @@ __global__ void __launch_bounds__(256) untile_weights_kernel(const uint8_t* __re
     const int64_t e = blockIdx.y;
     const uint8_t* src = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
     uint8_t* dst = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + word * 8;
-    const uint64_t v = *reinterpret_cast<const uint64_t*>(src);
     uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+    if (type == kTypeQ6K && word == 26) {
+        d16[0] = (uint16_t)*reinterpret_cast<const uint32_t*>(src);
+        return;
+    }
+    const uint64_t v = stored_form(*reinterpret_cast<const uint64_t*>(src), type, word);
     d16[0] = (uint16_t)v;
     d16[1] = (uint16_t)(v >> 16);
     d16[2] = (uint16_t)(v >> 32);
@@ -82,13 +98,18 @@ __global__ void __launch_bounds__(256) synth_weights_kernel(uint64_t seed, int64
     const uint64_t flat_block = ((uint64_t)e * (uint64_t)rows + (uint64_t)row) * (uint64_t)nb + (uint64_t)b;
     const uint64_t pos = flat_block * (uint64_t)words_per_block(type) + (uint64_t)word;
     uint64_t v = mix64(seed + (pos + 1) * kGamma);
-    if (word == 0) {
+    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
+    if (type == kTypeQ6K) {  // d is the block's last field
+        if (word == 26) {
+            *reinterpret_cast<uint32_t*>(dst) = unit_scale_f16(mix64((seed ^ kScaleStream) + (flat_block * 2 + 1) * kGamma));
+            return;
+        }
+    } else if (word == 0) {
         const uint64_t s0 = mix64((seed ^ kScaleStream) + (flat_block * 2 + 1) * kGamma);
         const uint64_t s1 = mix64((seed ^ kScaleStream) + (flat_block * 2 + 2) * kGamma);
         v = (v & 0xffffffff00000000ull) | (uint64_t)unit_scale_f16(s0) | ((uint64_t)unit_scale_f16(s1) << 16);
     }
-    uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
-    *reinterpret_cast<uint64_t*>(dst) = v;
+    *reinterpret_cast<uint64_t*>(dst) = stored_form(v, type, word);
 }
 
 inline dim3 word_grid(int64_t rows, int64_t nb, int64_t n_experts, int type) {

@@ -22,7 +22,7 @@ EXPORTS = [
     "mq_matmul_ggml_quantized_transb",
 ]
 
-GGML_TYPE_F32, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_I32 = 0, 12, 13, 26
+GGML_TYPE_F32, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K, GGML_TYPE_I32 = 0, 12, 13, 14, 26
 GGML_OP_CUSTOM_PLACEHOLDER = 0  # the adapters never read dst->op
 
 
@@ -69,8 +69,8 @@ def tensor(array: np.ndarray, ggml_type: int, ne, nb=None, name: bytes = b"") ->
     t.type = ggml_type
     ne = list(ne) + [1] * (4 - len(ne))
     if nb is None:
-        if ggml_type in (GGML_TYPE_Q4_K, GGML_TYPE_Q5_K):
-            bb = 144 if ggml_type == GGML_TYPE_Q4_K else 176
+        if ggml_type in (GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K):
+            bb = {GGML_TYPE_Q4_K: 144, GGML_TYPE_Q5_K: 176, GGML_TYPE_Q6_K: 210}[ggml_type]
             nb = [bb, bb * (ne[0] // 256)]
         else:
             nb = [4, 4 * ne[0]]

@@ -19,9 +19,13 @@ namespace {
 constexpr int64_t kSuperBlock = 256;
 constexpr size_t kQ4KBlockBytes = 144;
 constexpr size_t kQ5KBlockBytes = 176;
+constexpr size_t kQ6KBlockBytes = 210;
 // block bytes of a weight type this library multiplies, 0 for any other
 constexpr size_t kquant_block_bytes(int type) {
-    return type == (int)GGML_TYPE_Q4_K ? kQ4KBlockBytes : type == (int)GGML_TYPE_Q5_K ? kQ5KBlockBytes : 0;
+    return type == (int)GGML_TYPE_Q4_K   ? kQ4KBlockBytes
+           : type == (int)GGML_TYPE_Q5_K ? kQ5KBlockBytes
+           : type == (int)GGML_TYPE_Q6_K ? kQ6KBlockBytes
+                                         : 0;
 }
 
 thread_local int t_status = MQ_OK;
@@ -43,8 +47,8 @@ struct CachedWeight {
 std::mutex g_cache_mu;
 std::unordered_map<const void*, CachedWeight> g_cache;
 
-// Q4_K or Q5_K rows of whole super-blocks (the two weight types of the callbacks replaced:
-// core/src/llm/moe/native.cpp:2745-2752 accepts exactly these for the expert stacks)
+// Q4_K, Q5_K or Q6_K rows of whole super-blocks (the K-quant weight types of the callbacks replaced:
+// core/src/llm/moe/native.cpp:2745-2752, core/src/backend/cpu_backend_moe_raw_batched.inl:1552)
 bool is_kquant_matrix(const ggml_tensor* w) {
     if (!w || !w->data) return false;
     const size_t bb = kquant_block_bytes((int)w->type);
@@ -310,7 +314,7 @@ int mq_matmul_ggml_quantized_transb(const float* a, int64_t m, int64_t k, int64_
                                     int32_t w_type_id, int64_t w_rows, int64_t w_cols, size_t w_row_bytes, float* c,
                                     int64_t ldc) {
     // rejection rules of MatMulGgmlQuantizedTransBWithPath
-    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K and Q5_K
+    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K, Q5_K and Q6_K
     if (!a || !w_data || !c || m <= 0 || w_rows <= 0 || w_cols <= 0 || k != w_cols || lda < k || ldc < w_rows ||
         kquant_block_bytes(w_type_id) == 0 || w_cols % kSuperBlock != 0 ||
         w_row_bytes != (size_t)(w_cols / kSuperBlock) * kquant_block_bytes(w_type_id)) {

@@ -37,7 +37,7 @@ class Mi355Q4KBackend {
 public:
     struct GgmlQuantizedMatrixView {
         const void* data = nullptr;
-        int32_t type_id = -1;  // ggml_type; 12 (GGML_TYPE_Q4_K) and 13 (GGML_TYPE_Q5_K) are accepted
+        int32_t type_id = -1;  // ggml_type; 12 (GGML_TYPE_Q4_K), 13 (GGML_TYPE_Q5_K) and 14 (GGML_TYPE_Q6_K) are accepted
         int64_t rows = 0;      // N
         int64_t cols = 0;      // K
         size_t row_bytes = 0;

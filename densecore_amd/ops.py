@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .synth import BLOCK_BYTES, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
+from .synth import BLOCK_BYTES, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K, Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
 
 SILU_EXACT, SILU_FAST, SILU_FAST_FMA = 0, 1, 2
 ROUTE_FUSED, ROUTE_FLOOR, ROUTE_FLOOR_FINITE = 0, 1, 2
@@ -45,8 +45,8 @@ class Q4KWeight:
 
     @classmethod
     def from_ggml(cls, data: np.ndarray, cols: int, ggml_type: int = GGML_TYPE_Q4_K) -> "Q4KWeight":
-        """data: uint8 [rows, row_bytes] or [n_experts, rows, row_bytes] in ggml block_q4_K (type 12) or
-        block_q5_K (type 13) row layout."""
+        """data: uint8 [rows, row_bytes] or [n_experts, rows, row_bytes] in ggml block_q4_K (type 12),
+        block_q5_K (type 13) or block_q6_K (type 14) row layout."""
         a = np.ascontiguousarray(data, dtype=np.uint8)
         if a.ndim == 2:
             a = a[None]

@@ -22,10 +22,12 @@ import numpy as np
 QK_K = 256
 Q4K_BLOCK_BYTES = 144
 Q5K_BLOCK_BYTES = 176
+Q6K_BLOCK_BYTES = 210
 Q8K_BLOCK_BYTES = 292
 GGML_TYPE_Q4_K = 12
 GGML_TYPE_Q5_K = 13
-BLOCK_BYTES = {GGML_TYPE_Q4_K: Q4K_BLOCK_BYTES, GGML_TYPE_Q5_K: Q5K_BLOCK_BYTES}
+GGML_TYPE_Q6_K = 14
+BLOCK_BYTES = {GGML_TYPE_Q4_K: Q4K_BLOCK_BYTES, GGML_TYPE_Q5_K: Q5K_BLOCK_BYTES, GGML_TYPE_Q6_K: Q6K_BLOCK_BYTES}
 
 _GAMMA = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -94,6 +96,25 @@ def q5k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:
         raise ValueError("cols must be a multiple of 256")
     nb = cols // QK_K
     return q5k_blocks(seed, rows * nb).reshape(rows, nb * Q5K_BLOCK_BYTES)
+
+
+def q6k_blocks(seed: int, n_blocks: int, first_block: int = 0) -> np.ndarray:
+    """``[n_blocks, 210]`` uint8 array of seeded Q6_K super-blocks (ql[128], qh[64], scales[16] signed, fp16 d;
+    core/src/llm/matmul/q6_small_batch.h:13-24): 27 stream words a block, the first 210 bytes of them taken,
+    then ``d`` overwritten with ``fp16(U(0.001, 0.01))``."""
+    words = stream_u64(seed, first_block * 27, n_blocks * 27).reshape(n_blocks, 27)
+    raw = words.view(np.uint8).reshape(n_blocks, 216)[:, :Q6K_BLOCK_BYTES].copy()
+    sw = stream_u64(seed ^ 0x5CA1E5CA1E5CA1E5, first_block * 2, n_blocks * 2).reshape(n_blocks, 2)
+    raw[:, 208:210] = unit_scale_f16(sw[:, 0]).view(np.uint8).reshape(n_blocks, 2)
+    return raw
+
+
+def q6k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:
+    """Row-major Q6_K matrix ``[rows, cols/256 * 210]`` uint8 (ggml row layout)."""
+    if cols % QK_K:
+        raise ValueError("cols must be a multiple of 256")
+    nb = cols // QK_K
+    return q6k_blocks(seed, rows * nb).reshape(rows, nb * Q6K_BLOCK_BYTES)
 
 
 def q4k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:

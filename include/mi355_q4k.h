@@ -63,12 +63,16 @@ int mq_device_info(char* name_out, size_t name_cap, int* cu_count, size_t* hbm_b
  * (core/src/kernels/q4k_repacked_gemv.cpp:403). */
 int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts, size_t row_bytes,
                      size_t expert_bytes, mq_weight** out);
-/* The same for a tensor of another K-quant type.  ggml_type 12 = Q4_K (what mq_weight_upload takes) or
+/* The same for a tensor of another K-quant type.  ggml_type 12 = Q4_K (what mq_weight_upload takes),
  * 13 = Q5_K: block_q5_K is block_q4_K plus one high bit per weight (176 bytes: fp16 d, fp16 dmin, scales[12],
  * qh[32], qs[128]; core/src/kernels/hwy/hwy_moe_quant.cc:36-45), the type Q4_K_M files use for many down
  * projections (core/src/llm/moe/native.cpp:4611-4616) and DotKQ8KImpl<MoEQ5KBlock, true> multiplies
- * (core/src/kernels/hwy/hwy_moe_quant.cc:145-258).  Every product entry point accepts handles of either type
- * (gate and up of one call must share theirs); the matrix-core GEMM (mq_gemm_q4k) is Q4_K only, wide Q5_K
+ * (core/src/kernels/hwy/hwy_moe_quant.cc:145-258); or 14 = Q6_K: 210 bytes, ql[128], qh[64], 16 signed
+ * scales, fp16 d, weight = d * scale * (code - 32), multiplied as ComputeQ6KQ8KM4Native does
+ * (core/src/llm/matmul/q6_small_batch.h:13-92): one integer sum_g scale_g * sum (code - 32) * q8 per
+ * super-block (what mq_debug_block_sums returns as dot_scaled; min_dot is 0), one fused multiply-add per block.
+ * Every product entry point accepts handles of any of the three types (gate and up of one call must share
+ * theirs); the matrix-core GEMM (mq_gemm_q4k) and the one-launch decoder are Q4_K only, wide Q5_K / Q6_K
  * products run through the decode kernel in passes of 16 rows.  Other types: MQ_ERR_UNSUPPORTED. */
 int mq_weight_upload_typed(int ggml_type, const void* blocks_host, int64_t rows, int64_t cols, int64_t n_experts,
                            size_t row_bytes, size_t expert_bytes, mq_weight** out);

@@ -18,6 +18,7 @@ SILU_EXACT, SILU_FAST, SILU_FAST_FMA = 0, 1, 2
 
 Q4K = 144
 Q5K = 176
+Q6K = 210
 Q8K = 292
 
 
@@ -60,6 +61,9 @@ def lib() -> C.CDLL:
         L.orc_dot_magnitude_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
         L.orc_build_assignments.restype = C.c_int64
         L.orc_q5k_block_bytes.restype = C.c_size_t
+        L.orc_q6k_block_bytes.restype = C.c_size_t
+        L.orc_dot_dequant_q6k_f64.restype = C.c_double
+        L.orc_dot_dequant_q6k_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.orc_dot_q5k_q8k.restype = C.c_float
         L.orc_dot_q5k_q8k.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.orc_dot_dequant_q5k_f64.restype = C.c_double
@@ -250,6 +254,49 @@ def q5k_from_q4k(w4: np.ndarray, qh: np.ndarray | None = None) -> np.ndarray:
         b5[:, :, 16:48] = qh
     b5[:, :, 48:176] = b4[:, :, 16:144]
     return b5.reshape(rows, nb * Q5K)
+
+
+# ---------------------------------------------------------------- Q6_K weights
+def q6k_matrix_block_sums(w: np.ndarray, cols: int, q8: np.ndarray) -> np.ndarray:
+    """w uint8 [rows, nb*210], q8 uint8 [n, nb*292] -> int32 [rows, n, nb]: sum_g scale_g * sum (q - 32) * y."""
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    rows, n, nb = w.shape[0], q8.shape[0], cols // 256
+    out = np.zeros((rows, n, nb), np.int32)
+    rc = lib().orc_q6k_matrix_block_sums(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+                                         C.c_int64(n), C.c_size_t(q8.shape[1]), _p(out))
+    if rc:
+        raise ValueError(f"orc_q6k_matrix_block_sums rc={rc}")
+    return out
+
+
+def mul_mat_q6k_q8k(w: np.ndarray, cols: int, q8: np.ndarray, order: int = ORDER_DOTPROD) -> np.ndarray:
+    """-> fp32 [n, rows]; ORDER_HWY is the reference's eight-lane kernel, anything else the per-block form."""
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    rows, n = w.shape[0], q8.shape[0]
+    out = np.zeros((n, rows), np.float32)
+    rc = lib().orc_mul_mat_q6k_q8k(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+                                   C.c_int64(n), C.c_size_t(q8.shape[1]), _p(out), C.c_int64(rows), C.c_int(order))
+    if rc:
+        raise ValueError(f"orc_mul_mat_q6k_q8k rc={rc}")
+    return out
+
+
+def mul_mat_q6k_f32(w: np.ndarray, cols: int, x: np.ndarray, order: int = ORDER_DOTPROD) -> np.ndarray:
+    return mul_mat_q6k_q8k(w, cols, quantize_rows_q8k(x), order)
+
+
+def q6k_dot_dequant_f64(w: np.ndarray, cols: int, q8: np.ndarray, magnitude: bool = False) -> np.ndarray:
+    w = _c(w, np.uint8)
+    q8 = _c(q8, np.uint8)
+    L = lib()
+    out = np.zeros((q8.shape[0], w.shape[0]), np.float64)
+    for m in range(q8.shape[0]):
+        for r in range(w.shape[0]):
+            out[m, r] = L.orc_dot_dequant_q6k_f64(C.c_void_p(w[r].ctypes.data), C.c_void_p(q8[m].ctypes.data),
+                                                  C.c_int64(cols), C.c_int(int(magnitude)))
+    return out
 
 
 # ---------------------------------------------------------------- FFN / router / MoE

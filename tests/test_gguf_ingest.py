@@ -20,6 +20,7 @@ def _write(tmp_path, alignment=32, version=3):
     q2 = synth.q4k_matrix(11, 48, 512)                                   # [K=512, N=48]
     q3 = np.stack([synth.q4k_matrix(20 + e, 32, 256) for e in range(4)])   # [K=256, N=32, E=4]
     q5 = np.stack([synth.q5k_matrix(30 + e, 16, 512) for e in range(3)])   # [K=512, N=16, E=3], Q5_K
+    q6 = synth.q6k_matrix(40, 32, 768)                                      # [K=768, N=32], Q6_K
     path = str(tmp_path / f"model_a{alignment}_v{version}.gguf")
     gguf.write_gguf(path, {
         "general.architecture": ("str", "qwen35moe"),
@@ -36,13 +37,14 @@ def _write(tmp_path, alignment=32, version=3):
         ("blk.0.attn_q.weight", gguf.GGML_Q4_K, [512, 48], q2),
         ("blk.0.ffn_gate_exps.weight", gguf.GGML_Q4_K, [256, 32, 4], q3),
         ("blk.0.ffn_down_exps.weight", gguf.GGML_Q5_K, [512, 16, 3], q5),
+        ("output.weight", gguf.GGML_Q6_K, [768, 32], q6),
     ], alignment=alignment, version=version)
-    return path, f32, q2, q3, q5
+    return path, f32, q2, q3, q5, q6
 
 
 @pytest.mark.parametrize("alignment,version", [(32, 3), (64, 2), (4096, 3)])
 def test_metadata_and_tensor_table(tmp_path, alignment, version):
-    path, f32, q2, q3, q5 = _write(tmp_path, alignment, version)
+    path, f32, q2, q3, q5, q6 = _write(tmp_path, alignment, version)
     with gguf.GgufFile(path) as g:
         assert g.get_string("general.architecture") == "qwen35moe"
         assert g.get_int("qwen35moe.block_count") == 40 and g.get_int("qwen35moe.expert_used_count") == 8
@@ -53,15 +55,15 @@ def test_metadata_and_tensor_table(tmp_path, alignment, version):
             g.get_string("missing.key")
         ts = g.tensors()
         assert [t["name"] for t in ts] == ["token_embd.weight", "blk.0.attn_q.weight", "blk.0.ffn_gate_exps.weight",
-                                           "blk.0.ffn_down_exps.weight"]
-        assert [t["ne"] for t in ts] == [[8, 3], [512, 48], [256, 32, 4], [512, 16, 3]]
-        assert [t["type"] for t in ts] == [0, 12, 12, 13]
-        assert [t["nbytes"] for t in ts] == [96, 48 * 2 * 144, 4 * 32 * 144, 3 * 16 * 2 * 176]
+                                           "blk.0.ffn_down_exps.weight", "output.weight"]
+        assert [t["ne"] for t in ts] == [[8, 3], [512, 48], [256, 32, 4], [512, 16, 3], [768, 32]]
+        assert [t["type"] for t in ts] == [0, 12, 12, 13, 14]
+        assert [t["nbytes"] for t in ts] == [96, 48 * 2 * 144, 4 * 32 * 144, 3 * 16 * 2 * 176, 32 * 3 * 210]
         assert all(t["offset"] % alignment == 0 for t in ts)
         assert g.find("blk.0.attn_q.weight") == 1 and g.find("nope") == -1
         # the data pointers address the very bytes that were written
         import ctypes
-        for t, ref in zip(ts, (f32, q2, q3, q5)):
+        for t, ref in zip(ts, (f32, q2, q3, q5, q6)):
             assert ctypes.string_at(t["data"], t["nbytes"]) == ref.tobytes()
 
 
@@ -100,11 +102,12 @@ def test_q4k_tensors_upload_and_multiply(tmp_path):
     from densecore_amd import ops
     from oracle import binding as orc
     from tests._parity import assert_fp32_parity
-    path, _, q2, q3, q5 = _write(tmp_path)
+    path, _, q2, q3, q5, q6 = _write(tmp_path)
     with gguf.GgufFile(path) as g:
         w2 = g.load_q4k("blk.0.attn_q.weight")
         w3 = g.load_weight("blk.0.ffn_gate_exps.weight")
         w5 = g.load_weight("blk.0.ffn_down_exps.weight")
+        w6 = g.load_weight("output.weight")
         with pytest.raises(Exception):
             g.load_q4k("token_embd.weight")            # F32: not this path
         with pytest.raises(Exception):
@@ -119,6 +122,12 @@ def test_q4k_tensors_upload_and_multiply(tmp_path):
             assert_fp32_parity(yk[t, k][None], orc.mul_mat_q5k_q8k(q5[ids[t, k]], 512, q8),
                                orc.q5k_dot_dequant_f64(q5[ids[t, k]], 512, q8, magnitude=True))
     w5.free()
+    assert (w6.rows, w6.cols, w6.ggml_type) == (32, 768, 14) and np.array_equal(w6.to_ggml(), q6)
+    x6 = synth.normal_f32(7, (2, 768))
+    q8 = orc.quantize_rows_q8k(x6)
+    assert_fp32_parity(ops.mul_mat(w6, torch.from_numpy(x6).cuda()).cpu().numpy(), orc.mul_mat_q6k_q8k(q6, 768, q8),
+                       orc.q6k_dot_dequant_f64(q6, 768, q8, magnitude=True))
+    w6.free()
     assert (w2.rows, w2.cols, w2.n_experts) == (48, 512, 1) and (w3.rows, w3.cols, w3.n_experts) == (32, 256, 4)
     assert np.array_equal(w2.to_ggml(), q2) and np.array_equal(w3.to_ggml(), q3)
     x = synth.normal_f32(5, (3, 512))

@@ -149,6 +149,26 @@ def test_moe_down_node_with_q5k_experts_and_q5k_dense_node(ga):
     assert np.array_equal(c.view(np.uint32), out.view(np.uint32))
 
 
+def test_dense_node_and_library_matmul_with_q6k_weights(ga):
+    """Q6_K rows (210-byte blocks; the reference's kernel for the type is core/src/llm/matmul/q6_small_batch.h)."""
+    rows, cols, m = 80, 1024, 3
+    w = synth.q6k_matrix(2240, rows, cols)
+    x = synth.normal_f32(2241, (m, cols))
+    out = np.zeros((m, rows), np.float32)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q6_K, [cols, rows])
+    tx = ga.tensor(x, ga.GGML_TYPE_F32, [cols, m])
+    to = ga.tensor(out, ga.GGML_TYPE_F32, [rows, m])
+    ga.set_src(to, tx, tw)
+    ga.lib().mq_cb_gemv_batched_custom(C.byref(to), 0, 1, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    q8 = orc.quantize_rows_q8k(x)
+    assert_fp32_parity(out, orc.mul_mat_q6k_q8k(w, cols, q8), orc.q6k_dot_dequant_f64(w, cols, q8, magnitude=True))
+    c = np.zeros((m, rows), np.float32)
+    assert ga.lib().mq_matmul_ggml_quantized_transb(x.ctypes.data, m, cols, cols, w.ctypes.data, ga.GGML_TYPE_Q6_K, rows,
+                                                    cols, 210 * (cols // 256), c.ctypes.data, rows) == 1
+    assert np.array_equal(c.view(np.uint32), out.view(np.uint32))
+
+
 def test_library_level_matmul(ga):
     m, rows, cols = 7, 384, 768
     w = synth.q4k_matrix(301, rows, cols)
@@ -158,6 +178,6 @@ def test_library_level_matmul(ga):
                                                   cols, 144 * (cols // 256), c.ctypes.data, rows)
     assert ok == 1
     assert_fp32_parity(c, _dense_ref(w, cols, a), orc.dot_magnitude_f64(w, cols, orc.quantize_rows_q8k(a)))
-    # a type other than Q4_K and Q5_K is rejected like an unsupported ggml type
+    # a type other than Q4_K, Q5_K and Q6_K is rejected like an unsupported ggml type
     assert ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, 2, rows, cols,
                                                     144 * (cols // 256), c.ctypes.data, rows) == 0

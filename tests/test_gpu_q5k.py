@@ -202,6 +202,6 @@ def test_q5k_rejections(ops):
     with pytest.raises(MqError):
         ops.Q4KWeight.from_ggml(np.zeros((4, 144), np.uint8), 256, Q5)  # a Q5_K row needs 176 bytes
     with pytest.raises(MqError):
-        ops.Q4KWeight.from_ggml(np.zeros((4, 210), np.uint8), 256, 14)  # Q6_K is not handled
+        ops.Q4KWeight.from_ggml(np.zeros((4, 84), np.uint8), 256, 10)   # Q2_K is not handled
     w4.free()
     w5.free()

@@ -512,3 +512,90 @@ def test_q5k_sums_brute_force_and_fp32_against_double():
         assert np.max(np.abs(got - ref) / mag) < 2e-6
         ok = np.abs(ref) > 1e-3 * mag
         assert np.max(np.abs(got - ref)[ok] / np.abs(ref)[ok]) < 1e-4
+
+
+# ----------------------------------------------------------------- Q6_K weights
+def np_unpack_q6k(w):
+    """Independent decode of block_q6_K rows -> (d, scales[16], q[256] unsigned codes), from the published format."""
+    b = w.reshape(-1, 210)
+    ql = b[:, 0:128].astype(np.int64).reshape(-1, 2, 2, 32)      # [blk, j, half of the 64 bytes, l]
+    qh = b[:, 128:192].astype(np.int64).reshape(-1, 2, 32)       # [blk, j, l]
+    sc = b[:, 192:208].copy().view(np.int8).astype(np.int64)
+    d = b[:, 208:210].copy().view(np.float16).astype(np.float64)[:, 0]
+    q = np.zeros((b.shape[0], 2, 4, 32), np.int64)               # [blk, j, z, l]
+    for z in range(4):
+        nib = ql[:, :, z & 1, :] & 15 if z < 2 else ql[:, :, z & 1, :] >> 4
+        q[:, :, z, :] = nib | (((qh >> (2 * z)) & 3) << 4)
+    return d, sc, q.reshape(-1, 256)
+
+
+def test_q6k_layout_sums_brute_force_and_closed_forms():
+    assert orc.lib().orc_q6k_block_bytes() == 210
+    cols = 1024
+    w = synth.q6k_matrix(401, 10, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(402, (3, cols)))
+    d, sc, q = np_unpack_q6k(w)
+    assert q.min() == 0 and q.max() == 63 and sc.min() < -100 and sc.max() > 100
+    nb = cols // 256
+    _, yq, ybs = orc.split_q8k(q8)
+    yq = yq.astype(np.int64).reshape(3, nb, 16, 16)
+    sub = np.einsum("rbgi,mbgi->rmbg", (q - 32).reshape(10, nb, 16, 16), yq)
+    want = np.einsum("rmbg,rbg->rmb", sub, sc.reshape(10, nb, 16))
+    assert np.array_equal(orc.q6k_matrix_block_sums(w, cols, q8), want)
+    # every code 32 -> weights are all zero; every code 0 -> -32 * sum_g scale_g * bsums_g
+    blocks = w.reshape(10, nb, 210).copy()
+    blocks[:, :, 0:128] = 0
+    blocks[:, :, 128:192] = 0xAA          # each two-bit field = 2 -> code 32
+    assert not orc.q6k_matrix_block_sums(blocks.reshape(10, -1), cols, q8).any()
+    blocks[:, :, 128:192] = 0
+    got = orc.q6k_matrix_block_sums(blocks.reshape(10, -1), cols, q8)
+    closed = -32 * np.einsum("rbg,mbg->rmb", sc.reshape(10, nb, 16), ybs.astype(np.int64).reshape(3, nb, 16))
+    assert np.array_equal(got, closed)
+
+
+def test_q6k_single_element_placement():
+    rng = np.random.default_rng(6)
+    for _ in range(300):
+        e = int(rng.integers(0, 256))
+        blk = np.zeros((1, 210), np.uint8)
+        blk[0, 128:192] = 0xAA                               # every code 32: contributes nothing
+        scales = rng.integers(-128, 128, 16).astype(np.int8)
+        blk[0, 192:208] = scales.view(np.uint8)
+        code = int(rng.integers(0, 64))
+        j, z, l = e // 128, (e // 32) % 4, e % 32
+        byte = 64 * j + 32 * (z & 1) + l
+        blk[0, byte] = (code & 15) if z < 2 else (code & 15) << 4
+        hb = 128 + 32 * j + l
+        blk[0, hb] = (int(blk[0, hb]) & (0xFF ^ (3 << (2 * z)))) | ((code >> 4) << (2 * z))
+        # the nibble that shares the byte belongs to element e +- 64 and must read as code 32 there: its top bits stay 2
+        q8 = np.zeros((1, 292), np.uint8)
+        for probe in (e, (e + 64) % 256, (e + 32) % 256):
+            q8[:] = 0
+            q8[0, 4 + probe] = np.int8(-7).view(np.uint8)
+            got = orc.q6k_matrix_block_sums(blk, 256, q8)[0, 0, 0]
+            if probe == e:
+                assert got == int(scales[e // 16]) * (code - 32) * -7
+            elif probe == (e + 64) % 256 and (e // 128) == (probe // 128):
+                # same ql byte, other nibble: zero nibble with top bits 2 -> code 32 -> nothing
+                assert got == 0
+            else:
+                assert got == 0
+
+
+@pytest.mark.parametrize("cols", [256, 2048])
+def test_q6k_fp32_orders_against_double(cols):
+    w = synth.q6k_matrix(411 + cols, 24, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(412 + cols, (3, cols)))
+    d, sc, q = np_unpack_q6k(w)
+    wq = (d[:, None] * np.repeat(sc, 16, axis=1) * (q - 32)).reshape(24, cols)
+    yd, yq8, _ = orc.split_q8k(q8)
+    act = (yd[..., None].astype(np.float64) * yq8).reshape(3, cols)
+    want = act @ wq.T
+    ref = orc.q6k_dot_dequant_f64(w, cols, q8)
+    assert np.allclose(ref, want, rtol=1e-12, atol=1e-12)
+    mag = orc.q6k_dot_dequant_f64(w, cols, q8, magnitude=True)
+    for order in (orc.ORDER_HWY, orc.ORDER_DOTPROD):
+        got = orc.mul_mat_q6k_q8k(w, cols, q8, order).astype(np.float64)
+        assert np.max(np.abs(got - ref) / mag) < 2e-6
+        ok = np.abs(ref) > 1e-3 * mag
+        assert np.max(np.abs(got - ref)[ok] / np.abs(ref)[ok]) < 1e-4
