@@ -321,6 +321,27 @@ def side_measurements(ops, synth, torch, np, dev):
     for w in ring:
         w.free()
 
+    # the sibling K-quant types through the same decode kernel: the FFN down projection 14336 -> 4096 at n = 1 and 8
+    # on a ring of 12 matrices per type (Q4_K 396 MB, Q5_K 484 MB, Q6_K 578 MB)
+    sib = {}
+    for name, gtype, bb in (("Q4_K", synth.GGML_TYPE_Q4_K, 144), ("Q5_K", synth.GGML_TYPE_Q5_K, 176),
+                            ("Q6_K", synth.GGML_TYPE_Q6_K, 210)):
+        ring = [ops.Q4KWeight.synthetic(synth.tensor_seed("sib", name, r), 4096, 14336, 1, gtype) for r in range(12)]
+        per = {}
+        for n in (1, 8):
+            acts = ops.Q8KActs(n, 14336).quantize(torch.from_numpy(synth.normal_f32(synth.tensor_seed("sib-x", n), (n, 14336))).to(dev))
+            y = torch.empty((n, 4096), dtype=torch.float32, device=dev)
+            dt = time_graph(lambda: [acts.mul_mat(w, out=y) for w in ring], 20) / len(ring)
+            b = 4096 * 56 * bb + n * (14336 + 4096) * 4
+            per[str(n)] = {"us": round(dt * 1e6, 2), "GBps": round(b / dt / 1e9, 1),
+                           "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+            acts.free()
+        sib[name] = per
+        for w in ring:
+            w.free()
+    sib["note"] = "matmul from pre-quantized activations, 4096 x 14336 weights, bytes = ggml bytes of the type + fp32 in/out"
+    res["down_projection_by_weight_type"] = sib
+
     # cfg3: MoE layer, hidden 2048, 256 + 1 experts, inter 512, top-8; ring of 4 layers (1.8 GB)
     E, H, I, K = 256, 2048, 512, 8
     layers = []
