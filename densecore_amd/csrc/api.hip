@@ -1239,6 +1239,16 @@ int mq_decoder_status(mq_decoder* d) {
     return fail(MQ_ERR_STATE, "mq_decoder_step: a device-wide barrier timed out (are all compute units free for this process?)");
 }
 
+int mq_decoder_set_patience(mq_decoder* d, int64_t microseconds) {
+    if (int rc = check_ready()) return rc;
+    if (!d || microseconds < 0) return fail(MQ_ERR_INVALID, "mq_decoder_set_patience: null handle or negative time");
+    std::lock_guard<std::mutex> lock(g.mu);
+    int rate_khz = 0;
+    if (hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, g.device) != hipSuccess || rate_khz <= 0) rate_khz = 100000;
+    d->spin_ticks = (long long)rate_khz * microseconds / 1000;
+    return MQ_OK;
+}
+
 void mq_decoder_free(mq_decoder* d) {
     if (!d) return;
     std::lock_guard<std::mutex> lock(g.mu);

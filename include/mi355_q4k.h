@@ -255,6 +255,9 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
 /* Synchronises the device; MQ_OK, or MQ_ERR_STATE when a step since the last call abandoned a barrier (its
  * outputs are void; the handle is usable again afterwards). */
 int mq_decoder_status(mq_decoder* d);
+/* How long a workgroup waits at a device-wide barrier before it abandons the step (default 200 ms).  0 makes
+ * every waiter give up at once: the error path can be exercised without hanging anything. */
+int mq_decoder_set_patience(mq_decoder* d, int64_t microseconds);
 void mq_decoder_free(mq_decoder* d);
 
 /* ---- the fp32 operators either side of the path --------------------------------------------

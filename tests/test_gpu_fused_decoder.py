@@ -120,6 +120,27 @@ def test_graph_replays_and_repeated_steps(ds):
     step.free()
 
 
+def test_abandoned_barrier_is_reported_and_the_handle_recovers(ds):
+    """With no patience every workgroup that has to wait gives up at its first barrier: the launch drains by
+    itself, the status call reports it, and the next step is right again."""
+    import torch
+    from densecore_amd import _lib
+    cfg = ds.StepConfig(n_layers=2, hidden=512, n_experts=16, inter=256, top_k=4, n_q=512, n_kv=128, seed=13)
+    step, fused, x = _pair(ds, cfg, 2, 55)
+    want = step.run(x).clone()
+    assert torch.equal(fused.run(x), want)
+    fused.status()
+    _lib.check(_lib.lib().mq_decoder_set_patience(fused._h, 0), "mq_decoder_set_patience")
+    fused.run(x)
+    with pytest.raises(_lib.MqError):
+        fused.status()
+    _lib.check(_lib.lib().mq_decoder_set_patience(fused._h, 200000), "mq_decoder_set_patience")
+    assert torch.equal(fused.run(x), want)
+    fused.status()
+    fused.free()
+    step.free()
+
+
 def test_rejections(ds):
     import torch
     from densecore_amd import _lib, ops, synth
