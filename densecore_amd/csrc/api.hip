@@ -134,8 +134,9 @@ int check_weight(const mq_weight* w, const char* name) {
 }
 
 int check_x(const float* x, int64_t n, int64_t ldx, int64_t cols, const char* name) {
-    if (!x) return fail(MQ_ERR_INVALID, "%s: null activation pointer", name);
     if (n < 0) return fail(MQ_ERR_INVALID, "%s: negative row count", name);
+    if (n == 0) return MQ_OK;  // an empty matrix may come with null pointers; every caller returns before using them
+    if (!x) return fail(MQ_ERR_INVALID, "%s: null activation pointer", name);
     if (ldx < cols) return fail(MQ_ERR_INVALID, "%s: ldx %lld < cols %lld", name, (long long)ldx, (long long)cols);
     if (!aligned16(x) || (ldx & 3)) return fail(MQ_ERR_INVALID, "%s: activations must be 16-byte aligned with ldx %% 4 == 0", name);
     return MQ_OK;
@@ -338,6 +339,7 @@ int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void*
     if (int rc = check_ready()) return rc;
     if (k <= 0 || k % kQK) return fail(MQ_ERR_INVALID, "mq_quantize_q8k: k %lld is not a positive multiple of 256", (long long)k);
     if (int rc = check_x(x_dev, n, ldx, k, "mq_quantize_q8k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!q8_dev || (reinterpret_cast<uintptr_t>(q8_dev) & 3u)) return fail(MQ_ERR_INVALID, "mq_quantize_q8k: output must be non-null and 4-byte aligned");
     MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, k, q8_dev, (size_t)(k / kQK) * kQ8Block, nullptr, nullptr, (hipStream_t)stream));
     return MQ_OK;
@@ -382,6 +384,7 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: weight is an expert stack");
     if (w->type != kTypeQ4K) return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
     return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, (hipStream_t)stream);
@@ -393,6 +396,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     if (int rc = check_weight(w, "mq_mul_mat_q4k")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: weight is an expert stack; use mq_mul_mat_id_q4k");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_mul_mat_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
@@ -413,6 +417,7 @@ int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_mul_mat_q4k_q8k")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: weight is an expert stack");
+    if (n == 0) return MQ_OK;
     if (!q8_dev || !y_dev || n < 0 || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: bad arguments");
     if (q8_row_bytes < (size_t)w->nb * kQ8Block || (q8_row_bytes & 3) || (reinterpret_cast<uintptr_t>(q8_dev) & 3u))
         return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: q8 rows too short or not 4-byte aligned");
@@ -450,6 +455,7 @@ int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64
     if (int rc = check_weight(w, "mq_debug_block_sums")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: dense weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_debug_block_sums")) return rc;
+    if (n == 0) return MQ_OK;
     if (!dot_scaled_dev || !min_dot_dev || !y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: null output");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
@@ -472,6 +478,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (inter % kQK) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: inter %lld is not a multiple of 256", (long long)inter);
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: silu_mode %d", silu_mode);
     if (int rc = check_x(x_dev, n, hidden, hidden, "mq_ffn_swiglu_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!y_dev) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: null output");
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
@@ -547,6 +554,7 @@ int carve_route(int64_t n, int top_k, int64_t n_experts, RouteWs& r) {
 int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int top_k, int weights_mode,
                       int32_t* ids_dev, float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;
+    if (n == 0) return MQ_OK;
     if (!logits_dev || !ids_dev || !weights_dev) return fail(MQ_ERR_INVALID, "mq_moe_route_topk: null pointer");
     if (n < 0 || n_experts <= 0 || n_experts > 2048 || top_k <= 0 || top_k > n_experts || top_k > 8)
         return fail(MQ_ERR_INVALID, "mq_moe_route_topk: need 0 < top_k <= min(8, n_experts) and n_experts <= 2048");
@@ -559,6 +567,7 @@ int mq_moe_route_topk(const float* logits_dev, int64_t n_experts, int64_t n, int
 int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
                        float eps, float* sum_out_dev, float* normed_out_dev, void* stream) {
     if (int rc = check_ready()) return rc;
+    if (n == 0) return MQ_OK;
     if (!x_dev || !normed_out_dev || n < 0 || cols <= 0) return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_f32: bad arguments");
     MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, nullptr, nullptr,
                               (hipStream_t)stream));
@@ -591,6 +600,7 @@ int mq_router_logits_f32(const float* w_dev, int64_t n_experts, int64_t cols, co
 int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev, int top_k,
                                float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;
+    if (n == 0) return MQ_OK;
     if (!logits_dev || !ids_dev || !weights_dev) return fail(MQ_ERR_INVALID, "mq_moe_weights_from_logits: null pointer");
     if (n < 0 || n_experts <= 0 || top_k <= 0 || top_k > 8)
         return fail(MQ_ERR_INVALID, "mq_moe_weights_from_logits: need n_experts > 0 and 0 < top_k <= 8");
@@ -603,6 +613,7 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
                       int top_k, float* y_dev, void* stream) {
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_mul_mat_id_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!ids_dev || !y_dev || top_k <= 0) return fail(MQ_ERR_INVALID, "mq_mul_mat_id_q4k: null pointer or top_k <= 0");
     if (x_slots != 1 && x_slots != top_k) return fail(MQ_ERR_INVALID, "mq_mul_mat_id_q4k: x_slots must be 1 or top_k");
     if (int rc = check_x(x_dev, n * x_slots, w->cols, w->cols, "mq_mul_mat_id_q4k")) return rc;
@@ -786,6 +797,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
         return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: gate and up must be dense matrices of one shape and type");
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: silu_mode %d", silu_mode);
     if (int rc = check_x(x_dev, n, ldx, gate->cols, "mq_swiglu_mul_mat_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!h_dev || ldh < gate->rows) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: null output or ldh < rows");
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
@@ -891,6 +903,7 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
     if (int rc = check_experts(gate_exps, up_exps, nullptr, top_k, "mq_moe_gateup_swiglu_q4k")) return rc;
     if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_moe_gateup_swiglu_q4k: silu_mode %d", silu_mode);
     if (int rc = check_x(x_dev, n, gate_exps->cols, gate_exps->cols, "mq_moe_gateup_swiglu_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!ids_dev || !hidden_dev) return fail(MQ_ERR_INVALID, "mq_moe_gateup_swiglu_q4k: null ids or output");
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
@@ -910,6 +923,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
     if (int rc = check_weight(down_exps, "mq_moe_down_weighted_q4k(down_exps)")) return rc;
     if (int rc = check_experts(nullptr, nullptr, down_exps, top_k, "mq_moe_down_weighted_q4k")) return rc;
     if (int rc = check_x(hidden_dev, n * top_k, down_exps->cols, down_exps->cols, "mq_moe_down_weighted_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!ids_dev || !weights_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_down_weighted_q4k: null pointer");
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
@@ -1048,6 +1062,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         sh.down = L->shared_down;
     }
     if (int rc = check_x(x_dev, n, hidden, hidden, "mq_moe_layer_q4k")) return rc;
+    if (n == 0) return MQ_OK;
     if (!logits_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null logits or output");
     if (n == 0) return MQ_OK;
 
