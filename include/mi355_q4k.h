@@ -234,7 +234,8 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* layer, const float* x_dev, const f
  * (mq_add_rmsnorm_q8k, mq_mul_mat_q4k_acts, mq_mul_mat_q4k, mq_add_rmsnorm_f32, mq_router_logits_f32,
  * mq_moe_layer_q4k).  All weights Q4_K; every layer has layer 0's shapes; n_experts <= 512; top_k <= 8.
  * The kernel needs every compute unit of the device free for this process: a barrier that is not met within
- * 200 ms is abandoned, the launch drains, and mq_decoder_status reports it. */
+ * 200 ms is abandoned, the launch drains, and mq_decoder_status reports it.  Steps of one handle, and steps of
+ * different handles, must not overlap on the device (one stream, or streams ordered by events). */
 typedef struct mq_decoder mq_decoder;
 typedef struct {
     const mq_weight* wqkv;            /* [n_q + 2 n_kv][hidden], wq / wk / wv stacked row-wise */
