@@ -12,7 +12,8 @@ namespace {
 
 constexpr int kMaxExperts = 2048;
 
-// Routing of one token by one workgroup of 256 threads.  All threads turn the logits into sort keys in
+// Routing of one token by one workgroup of 256 threads.  Up to 512 experts: one wavefront, keys in registers.
+// More: all threads turn the logits into sort keys in
 // LDS; wavefront 0 then extracts the top_k largest keys one after the other (lane l owns the experts
 // e = l mod 64: a local maximum over its keys, a 6-step butterfly across the lanes, and the owner of
 // the winner clears it).  The keys are unique and totally ordered exactly like
@@ -23,6 +24,31 @@ __device__ __forceinline__ void route_token_block(const float* __restrict__ row,
                                                   int32_t* __restrict__ ids_out, float* __restrict__ w_out,
                                                   bool coherent_ids) {
     const int tid = threadIdx.x;
+    if (n_experts <= 512) {
+        // few enough experts for one wavefront's registers: eight 32-bit keys per lane, winners by ballot,
+        // softmax lane-parallel (route_block.h); the other wavefronts only pass the barriers
+        if (tid < 64) {
+            int id;
+            float logit;
+            auto load = [&](int e) { return row[e]; };
+            if (n_experts <= 256) route_token_wave<4>(load, n_experts, top_k, tid, id, logit);
+            else route_token_wave<8>(load, n_experts, top_k, tid, id, logit);
+            const float w = route_weight_lane(logit, tid, top_k, mode);
+            if (tid < top_k) {
+                sel_id[tid] = id;
+                w_out[tid] = w;
+            }
+        }
+        __syncthreads();
+        if (tid < top_k) {
+            if (coherent_ids) {
+                __hip_atomic_store(ids_out + tid, sel_id[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                ids_out[tid] = sel_id[tid];
+            }
+        }
+        return;
+    }
     for (int e = tid; e < n_experts; e += 256) keys[e] = route_key(row[e], e);
     __syncthreads();
     if (tid < 64) {
