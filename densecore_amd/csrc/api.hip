@@ -730,6 +730,22 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     if (!hidden_is_quantized) {
         if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
     }
+    if (n <= kTokenMajorDownMaxTokens && !census.on && (hidden_dim & 15) == 0 &&
+        (size_t)slots * (size_t)down->nb * 64 <= 48 * 1024) {
+        // few tokens: a workgroup per (token, 16 output rows) multiplies and combines in one launch
+        MoeDownTokenArgs a;
+        a.w = down->data;
+        a.expert_bytes = down->expert_bytes;
+        a.sh_w = sh.down ? sh.down->data : nullptr;
+        a.wtype = down->type;
+        a.rows = hidden_dim, a.nb = down->nb, a.n = n;
+        a.top_k = top_k, a.n_experts = (int)down->n_experts;
+        a.aq = (const uint8_t*)g.aq2.ptr, a.ad = (const float*)g.ad2.ptr;
+        a.ids = ids, a.weights = weights;
+        a.sh_gate_inp = sh_gate_inp, a.x = x, a.y = y;
+        MQ_HIP(launch_moe_down_token(a, s));
+        return MQ_OK;
+    }
     MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden_dim * sizeof(float)));
     MatmulArgs d;
     d.w0 = down->data;

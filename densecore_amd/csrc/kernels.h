@@ -123,10 +123,32 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
                               const float* x, float* y, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
 
+// ---- moe_down.hip ----------------------------------------------------------------------------
+// Down projection + weighted combine, one workgroup per (token, 16 output rows): for decode widths, where
+// grouping by expert shares nothing.  Hidden rows are Q8_K in the A-major layout, row = token * slots + slot.
+struct MoeDownTokenArgs {
+    const uint8_t* w = nullptr;        // tiled down experts [n_experts][rows x nb]
+    size_t expert_bytes = 0;
+    const uint8_t* sh_w = nullptr;     // shared expert's down matrix or null; its hidden row is slot top_k
+    int wtype = 12;
+    int64_t rows = 0, nb = 0;          // output rows (hidden), super-blocks per row (inter / 256)
+    int64_t n = 0;
+    int top_k = 0, n_experts = 0;
+    const uint8_t* aq = nullptr;       // A-major hidden rows
+    const float* ad = nullptr;
+    const int32_t* ids = nullptr;      // [n][top_k]
+    const float* weights = nullptr;    // [n][top_k]
+    const float* sh_gate_inp = nullptr;  // [rows] or null (gate = 1)
+    const float* x = nullptr;          // [n][rows]: the MoE block's input, for the gate
+    float* y = nullptr;                // [n][rows]
+};
+hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream);
+
 // ---- decoder_layers.hip ----------------------------------------------------------------------
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,
 // device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.
 constexpr int kDecoderMaxExperts = 512;
+constexpr int kTokenMajorDownMaxTokens = 4;  // widest MoE block whose down projection runs token-major (measured: 8 and 16 lose)
 constexpr int kMoeFusedMaxTokens = 2;  // widest MoE block that mq_moe_layer_q4k runs as one launch
 struct DecoderLayerDev {               // one per layer, in device memory
     const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]

@@ -1,0 +1,123 @@
+// MoE down projection with the weighted combine inside, token-major, for decode widths.
+//
+// The expert-grouped launch (matmul.hip) writes one partial row per (token, slot) and a second launch adds them
+// up in routing order.  With few tokens almost every (token, slot) pair has an expert of its own, so grouping by
+// expert shares nothing; here a workgroup owns one (token, 16-row tile) of the OUTPUT instead, streams the tiles
+// of that token's top_k experts (and of the shared expert), and adds the results in routing order itself:
+//   y[t][r] = sum_k w[t][k] * (down_e(t,k)[r] . q8k(hidden[t][k]))  (+ sigmoid(g . x[t]) * shared)
+// (cb_qwen35_native_moe_down_q5k_weighted_logits, core/src/llm/moe/native.cpp:3051-3295; zero weights and ids out
+// of range skipped as at :3237).  Per-tile arithmetic, the order of the super-block terms and of the slots, and
+// the gate are those of the grouped launch + moe_combine_kernel: same bits, one launch less, no partial rows.
+#include "common.h"
+#include "kernels.h"
+#include "decode_tile.h"
+#include "route_block.h"
+
+namespace mq {
+
+namespace {
+
+constexpr int kWaves = 8;
+constexpr int kItems = 3;  // (slot, super-block) items a wavefront keeps in flight
+
+template <int WT>
+__global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDownTokenArgs p) {
+    constexpr int kTileStride = tile_stride<WT>();
+    extern __shared__ float term[];  // [slots * nb][16], then 4 floats of gate scratch
+    __shared__ float wave_sum[4];
+    __shared__ float gate_sh;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rt = blockIdx.x, t = blockIdx.y;
+    const int nb = (int)p.nb, slots = p.top_k + (p.sh_w ? 1 : 0), n_items = slots * nb;
+
+    auto item_tile = [&](int i) -> const uint8_t* {  // null for a dropped slot
+        const int sl = i / nb, b = i - sl * nb;
+        const bool shared = sl >= p.top_k;
+        const int e = shared ? 0 : p.ids[t * p.top_k + sl];
+        if (!shared && (e < 0 || e >= p.n_experts)) return nullptr;
+        return (shared ? p.sh_w : p.w + (size_t)e * p.expert_bytes) + tile_offset(rt, b, nb, kTileStride);
+    };
+
+    for (int base = 0; base < n_items; base += kWaves * kItems) {
+        typename TileOf<WT>::Regs tiles[kItems];
+        ARegs<1> a[kItems];
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) {  // every load is issued; a missing item reads a harmless tile
+            const int i = base + wave + kWaves * j;
+            const int ii = i < n_items ? i : 0;
+            const uint8_t* w = i < n_items ? item_tile(i) : nullptr;
+            load_tile_wt<WT>(tiles[j], w ? w : p.w, lane);
+            const int sl = ii / nb, b = ii - sl * nb;
+            const int64_t row = t * slots + sl;  // hidden row; its 8-row tile comes along, only this row is kept
+            const int64_t row0 = row & ~(int64_t)7;
+            const size_t a_off[1] = {aq_row_offset(row0 + (slot >> 1), nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16};
+            const int d_idx[1][2] = {{(int)ad_index(row0 + 2 * kq, 0, nb), (int)ad_index(row0 + 2 * kq + 1, 0, nb)}};
+            load_a<1>(a[j], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+        }
+        if (base == 0 && p.sh_w) {  // the shared expert's gate while the tiles travel (moe_combine_kernel's order)
+            float gate = 1.0f;
+            if (p.sh_gate_inp) {
+                if (tid < 256) {
+                    float acc = 0.0f;
+                    for (int64_t c = tid; c < p.rows; c += 256) acc = fmaf(p.sh_gate_inp[c], p.x[t * p.rows + c], acc);
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+                    if ((tid & 63) == 0) wave_sum[tid >> 6] = acc;
+                }
+                __syncthreads();
+                gate = stable_sigmoid((wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]));
+            }
+            if (tid == 0) gate_sh = gate;
+        }
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) {
+            const int i = base + wave + kWaves * j;
+            if (i < n_items) {  // wave-uniform
+                float acc[1][2] = {{0.0f, 0.0f}};
+                if (item_tile(i)) {
+                    int32_t dsum[1][2], msum[1][2];
+                    compute_tile_wt<1, WT>(tiles[j], a[j], acc, dsum, msum, lane);
+                }
+                const int pos = (int)((t * slots + i / nb) & 7);  // the row's place in its 8-row tile
+                if (kq == (pos >> 1)) term[i * 16 + slot] = (pos & 1) ? acc[0][1] : acc[0][0];
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < 16) {
+        const int64_t row = rt * 16 + tid;
+        float acc = 0.0f;
+        for (int k = 0; k < slots; ++k) {
+            float part = __fadd_rn(0.0f, term[(k * nb) * 16 + tid]);
+            for (int b = 1; b < nb; ++b) part = __fadd_rn(part, term[(k * nb + b) * 16 + tid]);
+            if (k < p.top_k) {
+                const int e = p.ids[t * p.top_k + k];
+                const float w = p.weights[t * p.top_k + k];
+                if (e < 0 || e >= p.n_experts || w == 0.0f) continue;
+                acc = __fadd_rn(acc, __fmul_rn(part, w));
+            } else {
+                acc = __fadd_rn(acc, __fmul_rn(part, gate_sh));
+            }
+        }
+        if (row < p.rows) p.y[t * p.rows + row] = acc;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) {
+    if (a.n <= 0 || a.rows <= 0 || (a.rows & 15) || a.nb <= 0 || a.top_k <= 0 || a.top_k > 8) return hipErrorInvalidValue;
+    const int slots = a.top_k + (a.sh_w ? 1 : 0);
+    const size_t lds = (size_t)slots * (size_t)a.nb * 16 * sizeof(float);
+    if (lds > 48 * 1024) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)(a.rows / 16), (unsigned)a.n);
+    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ6>, grid, dim3(kWaves * 64), lds, stream, a);
+    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ5>, grid, dim3(kWaves * 64), lds, stream, a);
+    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ4>, grid, dim3(kWaves * 64), lds, stream, a);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+}  // namespace mq
