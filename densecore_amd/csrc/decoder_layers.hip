@@ -29,6 +29,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "decode_tile.h"
+#include "grid_sync.h"
 #include "q8k_block.h"
 #include "route_block.h"
 
@@ -38,21 +39,9 @@ namespace {
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kSyncLine = 64;   // uint32 words between counters
-constexpr int kSyncGroup = 16;  // workgroups per first-level counter
 constexpr int kMaxSlots = 9;    // top_k <= 8 routed slots + the shared expert
 constexpr int kMaxInterBlocks = 8;  // inter <= 2048
 constexpr int kKeysPerLane = kDecoderMaxExperts / 64;
-
-__device__ __forceinline__ float ld_dev(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_dev(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint32_t ld_dev(const uint32_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 struct Shared {
     uint8_t* aq;    // A-major Q8_K codes of the current projection input, one 8-row tile: [nb][4096]
@@ -67,52 +56,6 @@ struct Shared {
     int32_t* ids;   // [8][8] routed experts
     int* ok;        // barrier verdict of this workgroup
 };
-
-// Device-wide barrier.  Every thread's device-scope stores are acknowledged (vmcnt) before its workgroup is
-// counted.  `ahead()` runs in every thread once that is so and before the wait: the place to request weights
-// of the next phase, whose latency then overlaps the barrier's.  Returns false when the barrier was abandoned.
-template <typename Ahead>
-__device__ __forceinline__ bool grid_barrier(uint32_t* sync, uint32_t& my_gen, int* ok, long long spin_ticks, Ahead ahead) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    ahead();
-    if (threadIdx.x == 0) {
-        uint32_t* top = sync;
-        uint32_t* gen = sync + kSyncLine;
-        uint32_t* fail = sync + 2 * kSyncLine;
-        const uint32_t n_wg = gridDim.x;
-        const uint32_t grp = blockIdx.x / kSyncGroup;
-        const uint32_t n_grp = (n_wg + kSyncGroup - 1) / kSyncGroup;
-        const uint32_t grp_size = (grp + 1) * kSyncGroup <= n_wg ? kSyncGroup : n_wg - grp * kSyncGroup;
-        uint32_t* gc = sync + (4 + grp) * kSyncLine;
-        bool released = false, good = true;
-        if (__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == grp_size - 1) {
-            __hip_atomic_store(gc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (__hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
-                __hip_atomic_store(top, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                // the two resets above are acknowledged before anybody is let go
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __hip_atomic_fetch_add(gen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                released = true;
-            }
-        }
-        if (!released) {
-            const long long t0 = wall_clock64();
-            while (ld_dev(gen) == my_gen) {
-                if (ld_dev(fail) != 0u || wall_clock64() - t0 > spin_ticks) {
-                    __hip_atomic_store(fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    good = false;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-        }
-        *ok = good ? 1 : 0;
-    }
-    my_gen += 1;
-    __syncthreads();
-    return *ok != 0;
-}
 
 // Per-token sums over the columns in the order of a 256-thread workgroup of the one-node kernels: thread j
 // takes columns j, j + 256, ... with fused multiply-adds, a butterfly inside each of the four wavefronts,
@@ -330,7 +273,6 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
     }
     if (ld_dev(p.sync + 2 * kSyncLine) != 0u) return;  // an earlier launch abandoned a barrier: the state is unusable
     uint32_t my_gen = ld_dev(p.sync + kSyncLine);      // cannot move before this workgroup's own first arrival
-    const auto nothing = [] {};
     uint32_t sink = 0u;  // see warm()
 
     // Weights of this workgroup's first row tile of a dense projection, requested a phase ahead.  Workgroups

@@ -286,7 +286,12 @@ def moe_layer(gate_exps: Q4KWeight, up_exps: Q4KWeight, down_exps: Q4KWeight, x:
     return y, ids, wts
 
 
-KIND_DENSE, KIND_DENSE_SWIGLU, KIND_GROUPED, KIND_GROUPED_SWIGLU = 0, 1, 2, 3
+KIND_DENSE, KIND_DENSE_SWIGLU, KIND_GROUPED, KIND_GROUPED_SWIGLU, KIND_FFN_ONE_LAUNCH = 0, 1, 2, 3, 4
+
+
+def stream_synchronize() -> None:
+    """Waits for the current stream and raises if a persistent launch on it gave up at a device-wide barrier."""
+    _lib.check(_lib.lib().mq_stream_synchronize(_stream()), "mq_stream_synchronize")
 
 
 def census_enable(on: bool) -> None:
