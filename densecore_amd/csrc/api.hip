@@ -202,8 +202,6 @@ const char* mq_last_error(void) { return g_error.c_str(); }
 namespace {
 void release_moe_fused();
 int check_moe_fused();
-int run_ffn_fused(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev, int64_t n,
-                  float* y_dev, int silu_mode, hipStream_t s, bool* done);
 }  // namespace
 
 int mq_init(int device) {
@@ -485,11 +483,6 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    {
-        bool done = false;
-        if (int rc = run_ffn_fused(gate, up, down, x_dev, n, y_dev, silu_mode, s, &done)) return rc;
-        if (done) return MQ_OK;
-    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
     MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
     MatmulArgs a;
@@ -1002,70 +995,7 @@ int check_moe_fused() {
     MQ_HIP(hipMemcpy(&flag, moe_fused.sync + 128, sizeof flag, hipMemcpyDeviceToHost));
     if (flag == 0) return MQ_OK;
     MQ_HIP(hipMemset(moe_fused.sync, 0, decoder_sync_bytes(moe_fused.n_workgroups)));
-    return fail(MQ_ERR_STATE, "a one-launch MoE block or FFN: a device-wide barrier timed out (are all compute units free for this process?); the outputs of that call are void");
-}
-
-// The persistent launches share one set of barrier words: launches on one stream follow each other, and
-// launches that overlap are ruled out by the interface.
-int reserve_barrier_words() {
-    if (moe_fused.sync) return MQ_OK;
-    long long ticks = 0;
-    int wgs = 0;
-    if (int rc = decoder_grid(0, &wgs, &ticks)) return rc;
-    const size_t bytes = decoder_sync_bytes(wgs);
-    MQ_HIP(hipMalloc(&moe_fused.sync, bytes));
-    MQ_HIP(hipMemset(moe_fused.sync, 0, bytes));
-    moe_fused.n_workgroups = wgs;
-    moe_fused.spin_ticks = ticks;
-    return MQ_OK;
-}
-
-// Dense FFN of up to kFfnFusedMaxTokens rows as one persistent launch (ffn_fused.hip); *done = false when
-// the shape or the weight types are outside what that kernel takes.
-int run_ffn_fused(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev, int64_t n,
-                  float* y_dev, int silu_mode, hipStream_t s, bool* done) {
-    *done = false;
-    const int64_t hidden = gate->cols, inter = gate->rows;
-    if (n > kFfnFusedMaxTokens || gate->type != kTypeQ4K || up->type != kTypeQ4K || down->type != kTypeQ4K) return MQ_OK;
-    if ((hidden % kQK) || (inter % kQK) || hidden > (1 << 20) || inter > (1 << 20)) return MQ_OK;
-    const size_t lds = ffn_fused_lds_bytes((int)n, (int)hidden, (int)inter);
-    static size_t lds_ready = 0, lds_limit = 0;  // caller holds g.mu
-    if (!lds_limit) {
-        hipDeviceProp_t prop;
-        MQ_HIP(hipGetDeviceProperties(&prop, g.device));
-        lds_limit = prop.maxSharedMemoryPerMultiProcessor;
-    }
-    if (lds > lds_limit) return MQ_OK;
-    if (int rc = reserve_barrier_words()) return rc;
-    if (lds > lds_ready) {
-        MQ_HIP(prepare_ffn_fused(lds));
-        lds_ready = lds;
-    }
-    MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
-    FfnFusedArgs a;
-    a.gate = gate->data, a.up = up->data, a.down = down->data;
-    a.x = x_dev, a.h = (float*)g.mid.ptr, a.y = y_dev;
-    a.n = (int)n, a.hidden = (int)hidden, a.inter = (int)inter;
-    a.waves1 = pick_waves(gate->nb, (inter + 15) / 16);
-    a.waves2 = pick_waves(down->nb, (hidden + 15) / 16);
-    a.silu_mode = silu_mode;
-    a.spin_ticks = moe_fused.spin_ticks;
-    a.sync = moe_fused.sync;
-    if (census.on && census.used < Census::kMax) {
-        if (census.used == census.pool.size()) {
-            Census::Rec r;
-            MQ_HIP(hipEventCreate(&r.start));
-            MQ_HIP(hipEventCreate(&r.stop));
-            census.pool.push_back(r);
-        }
-        Census::Rec& r = census.pool[census.used++];
-        r.kind = 4;
-        MQ_HIP(launch_ffn_fused(a, moe_fused.n_workgroups, s, r.start, r.stop));
-    } else {
-        MQ_HIP(launch_ffn_fused(a, moe_fused.n_workgroups, s));
-    }
-    *done = true;
-    return MQ_OK;
+    return fail(MQ_ERR_STATE, "mq_moe_layer_q4k: a device-wide barrier timed out (are all compute units free for this process?); the outputs of that call are void");
 }
 
 int run_moe_fused(const mq_moe_layer_desc* L, const SharedExpert& sh, const float* x_dev, const float* logits_dev, int64_t n,
@@ -1088,7 +1018,11 @@ int run_moe_fused(const mq_moe_layer_desc* L, const SharedExpert& sh, const floa
     if (!moe_fused.sync || lds > moe_fused.lds_ready) {  // first use (or a larger shape): not capturable, like any workspace growth
         if (int rc = decoder_grid(lds, &moe_fused.n_workgroups, &moe_fused.spin_ticks)) return rc;
         moe_fused.lds_ready = lds;
-        if (int rc = reserve_barrier_words()) return rc;
+        if (!moe_fused.sync) {
+            const size_t bytes = decoder_sync_bytes(moe_fused.n_workgroups);
+            MQ_HIP(hipMalloc(&moe_fused.sync, bytes));
+            MQ_HIP(hipMemset(moe_fused.sync, 0, bytes));
+        }
     }
     const int slots = L->top_k + a.has_shared;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));

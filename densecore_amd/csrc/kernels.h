@@ -150,7 +150,6 @@ hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream);
 constexpr int kDecoderMaxExperts = 512;
 constexpr int kTokenMajorDownMaxTokens = 4;  // widest MoE block whose down projection runs token-major (measured: 8 and 16 lose)
 constexpr int kMoeFusedMaxTokens = 2;  // widest MoE block that mq_moe_layer_q4k runs as one launch
-constexpr int kFfnFusedMaxTokens = 8;  // widest dense FFN that mq_ffn_swiglu_q4k runs as one launch
 struct DecoderLayerDev {               // one per layer, in device memory
     const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]
     const uint8_t* wo = nullptr;       // [hidden x n_q]; its input is qkv[:, :n_q]
@@ -194,27 +193,5 @@ size_t decoder_layers_lds_bytes(const DecoderArgs& a);
 size_t decoder_sync_bytes(int n_workgroups);
 hipError_t prepare_decoder_layers(size_t lds_bytes);
 hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream);
-
-
-// ---- ffn_fused.hip ---------------------------------------------------------------------------
-// Dense SwiGLU FFN of up to 8 rows as one persistent launch (quantize, gate/up + SwiGLU, device-wide barrier,
-// re-quantize, down).  Q4_K weights in the tiled layout; bit-identical to the four one-node launches.
-struct FfnFusedArgs {
-    const uint8_t* gate = nullptr;     // [inter x hidden]
-    const uint8_t* up = nullptr;
-    const uint8_t* down = nullptr;     // [hidden x inter]
-    const float* x = nullptr;          // [n x hidden], 16-byte aligned
-    float* h = nullptr;                // exchange buffer [n x inter]
-    float* y = nullptr;                // [n x hidden]
-    int n = 0, hidden = 0, inter = 0;
-    int waves1 = 0, waves2 = 0;        // wavefronts per row tile in gate/up and in down: pick_waves() of the one-node launches
-    int silu_mode = 0;
-    long long spin_ticks = 0;          // barrier patience in wall_clock64 ticks
-    uint32_t* sync = nullptr;          // decoder_sync_bytes(), zero before the first launch
-};
-size_t ffn_fused_lds_bytes(int n, int hidden, int inter);
-hipError_t prepare_ffn_fused(size_t lds_bytes);
-hipError_t launch_ffn_fused(const FfnFusedArgs& a, int n_workgroups, hipStream_t stream, hipEvent_t start = nullptr,
-                            hipEvent_t stop = nullptr);
 
 }  // namespace mq

@@ -286,7 +286,7 @@ def moe_layer(gate_exps: Q4KWeight, up_exps: Q4KWeight, down_exps: Q4KWeight, x:
     return y, ids, wts
 
 
-KIND_DENSE, KIND_DENSE_SWIGLU, KIND_GROUPED, KIND_GROUPED_SWIGLU, KIND_FFN_ONE_LAUNCH = 0, 1, 2, 3, 4
+KIND_DENSE, KIND_DENSE_SWIGLU, KIND_GROUPED, KIND_GROUPED_SWIGLU = 0, 1, 2, 3
 
 
 def stream_synchronize() -> None:

@@ -149,11 +149,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
  * y = down( silu(gate x) * (up x) ), x_dev [n][hidden], y_dev [n][hidden].
  * gate/up: rows = inter, cols = hidden; down: rows = hidden, cols = inter.
  * The three smart_mul_mat calls plus cb_silu_mul_fused of a dense FFN block
- * (core/src/llm/graph/decoder.cpp:2662-2730, core/src/llm/graph/fused_ops.cpp:317-366).
- * Up to 8 rows of Q4_K weights run as ONE persistent launch (one workgroup per compute unit, a device-wide
- * barrier between the two projections); the result is bit-identical to mq_swiglu_mul_mat_q4k followed by
- * mq_mul_mat_q4k.  Such a launch must not overlap another persistent launch of this library on the same
- * device, and a barrier that times out is reported by mq_stream_synchronize (MQ_ERR_STATE). */
+ * (core/src/llm/graph/decoder.cpp:2662-2730, core/src/llm/graph/fused_ops.cpp:317-366). */
 int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev,
                       int64_t n, float* y_dev, int silu_mode, void* stream);
 
@@ -302,8 +298,7 @@ int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64
 #define MQ_KIND_DENSE_SWIGLU 1   /* gate + up fused, dense               */
 #define MQ_KIND_GROUPED 2        /* expert-routed                        */
 #define MQ_KIND_GROUPED_SWIGLU 3 /* expert-routed gate + up fused        */
-#define MQ_KIND_FFN_ONE_LAUNCH 4  /* whole dense FFN in one persistent launch */
-#define MQ_KIND_COUNT 5
+#define MQ_KIND_COUNT 4
 int mq_census_enable(int on);
 int mq_census_reset(void);
 int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int64_t* count);
