@@ -190,6 +190,18 @@ def main() -> int:
     step_bytes = sum(ffn_bytes(n) for n in WIDTHS)
     value = step_bytes * args.steps / elapsed / 1e9
 
+    # spread of single steps (outside the timed region): an event after every step, differences of neighbours
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(min(args.steps, 200) + 1)]
+    marks[0].record()
+    for i in range(len(marks) - 1):
+        step(i)
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    singles = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(len(marks) - 1))
+    pick = lambda q: round(singles[min(len(singles) - 1, int(q * len(singles)))], 4)
+    step_spread = {"p10_ms": pick(0.10), "p50_ms": pick(0.50), "p90_ms": pick(0.90), "steps": len(singles),
+                   "how": "HIP events between consecutive steps, after the timed region"}
+
     # ---------------------------------------------------------------- dominant kernel, live
     narrow = tuple(n for n in WIDTHS if n <= 8)      # one activation tile:  matmul_kernel<2,1,...>
     wide = tuple(n for n in WIDTHS if n > 8)         # two activation tiles: matmul_kernel<2,2,...>
@@ -282,6 +294,7 @@ def main() -> int:
                    "launch": "eager" if graphs is None else "hip-graph replay",
                    "bytes_per_step": step_bytes},
         "pct_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 1),
+        "step_spread": step_spread,
         "per_width": per_width,
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -318,6 +331,9 @@ def side_measurements(ops, synth, torch, np, dev):
     b = 4096 * 16 * 144 + 2 * 4096 * 4
     res["gemv_4096x4096_n1"] = {"us": round(dt * 1e6, 2), "GBps": round(b / dt / 1e9, 1),
                                 "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+    # the same launch on ONE matrix over and over (9.4 MB: it stays in the last-level cache) -- not the roofline claim
+    dt = time_graph(lambda: [ops.mul_mat(ring[0], x1) for _ in range(64)], 20) / 64
+    res["gemv_4096x4096_n1"]["cache_hot_single_matrix_us"] = round(dt * 1e6, 2)
     for w in ring:
         w.free()
 
@@ -462,6 +478,14 @@ def cpu_baseline(weight_set, xs, seconds, np):
             break
     dt = time.perf_counter() - t0
     total = done * sum(ffn_bytes(n) for n in WIDTHS)
+    # one thread, one n = 1 pass at a time, for about a sixth of the sample time: the per-core figure
+    one_done, t1 = 0, time.perf_counter()
+    while True:
+        orc.simd_ffn_swiglu(g, u, d, HIDDEN, INTER, x_host[1], 1)
+        one_done += 1
+        if time.perf_counter() - t1 >= seconds / 6:
+            break
+    one_dt = time.perf_counter() - t1
     model = "unknown"
     try:
         for line in open("/proc/cpuinfo"):
@@ -473,6 +497,7 @@ def cpu_baseline(weight_set, xs, seconds, np):
     return {"value": round(total / dt / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{done} passes over the five FFN widths (n=1,2,4,8,16) on weight set 0, {dt:.1f} s, "
                       f"AVX2 + {threads} pthreads, rows split as ith*ceil(N/nth)",
+            "one_core_GBps": round(one_done * ffn_bytes(1) / one_dt / 1e9, 2),
             "cpu": model}
 
 

@@ -199,11 +199,6 @@ extern "C" {
 
 const char* mq_last_error(void) { return g_error.c_str(); }
 
-namespace {
-void release_moe_fused();
-int check_moe_fused();
-}  // namespace
-
 int mq_init(int device) {
     std::lock_guard<std::mutex> lock(g.mu);
     int count = 0;
@@ -225,7 +220,6 @@ int mq_shutdown(void) {
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
     for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
-    release_moe_fused();
     g.ready = false;
     return MQ_OK;
 }
@@ -670,7 +664,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     MatmulArgs a;
     if (quantize_hidden) {  // hidden rows leave the kernel already in Q8_K (A-major), ready for the down projection
         const int64_t out_nb = gate->rows / kQK;
-        const int64_t groups = (pairs < gate->n_experts ? pairs : gate->n_experts) + (n + 7) / 8;  // + shared-expert passes
+        const int64_t groups = (r.direct_ids || pairs < gate->n_experts ? pairs : gate->n_experts) + (n + 7) / 8;  // + shared-expert passes
         MQ_HIP(g.aq2.reserve(aq_bytes(n * slots, out_nb)));
         MQ_HIP(g.ad2.reserve(ad_count(n * slots, out_nb) * sizeof(float)));
         if (int rc = reserve_counters((size_t)(groups * out_nb))) return rc;
@@ -701,7 +695,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     a.a_k_stride = 0;
     a.y_tok_stride = slots;
     a.y_k_stride = 1;
-    a.max_groups = (int)(pairs < gate->n_experts ? pairs : gate->n_experts);
+    a.max_groups = (int)(r.direct_ids || pairs < gate->n_experts ? pairs : gate->n_experts);
     a.direct_ids = r.direct_ids;
     a.direct_top_k = top_k;
     a.n_experts = (int)gate->n_experts;
@@ -768,7 +762,7 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     d.a_k_stride = 1;
     d.y_tok_stride = slots;
     d.y_k_stride = 1;
-    d.max_groups = (int)(pairs < down->n_experts ? pairs : down->n_experts);
+    d.max_groups = (int)(r.direct_ids || pairs < down->n_experts ? pairs : down->n_experts);
     d.direct_ids = r.direct_ids;
     d.direct_top_k = top_k;
     d.n_experts = (int)down->n_experts;
@@ -954,10 +948,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
 
 namespace {
 
-// One- and two-token MoE blocks run as a single persistent launch (decoder_layers.hip, MoE-only mode): route,
-// gate/up and down meet at device-wide barriers instead of launch boundaries.  Same arithmetic and orders as
-// the launches below.  Returns MQ_OK with *done = false when the shape is outside what that kernel takes.
-// Workgroups of the persistent kernel: one per compute unit, all resident at once.
+// Workgroups of the persistent decoder kernel (decoder_layers.hip): one per compute unit, all resident at once.
 int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
     hipDeviceProp_t prop;
     MQ_HIP(hipGetDeviceProperties(&prop, g.device));
@@ -973,78 +964,6 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
     if (hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, g.device) != hipSuccess || rate_khz <= 0) rate_khz = 100000;
     *spin_ticks = (long long)rate_khz * 200;  // 200 ms: a phase takes microseconds
     *n_workgroups = prop.multiProcessorCount;
-    return MQ_OK;
-}
-
-struct MoeFusedState {
-    uint32_t* sync = nullptr;
-    int n_workgroups = 0;
-    long long spin_ticks = 0;
-    size_t lds_ready = 0;
-} moe_fused;
-
-void release_moe_fused() {
-    if (moe_fused.sync) (void)hipFree(moe_fused.sync);
-    moe_fused = MoeFusedState{};
-}
-
-// After a synchronisation: did a one-launch MoE block abandon a barrier since the last check?
-int check_moe_fused() {
-    if (!moe_fused.sync) return MQ_OK;
-    uint32_t flag = 0;
-    MQ_HIP(hipMemcpy(&flag, moe_fused.sync + 128, sizeof flag, hipMemcpyDeviceToHost));
-    if (flag == 0) return MQ_OK;
-    MQ_HIP(hipMemset(moe_fused.sync, 0, decoder_sync_bytes(moe_fused.n_workgroups)));
-    return fail(MQ_ERR_STATE, "mq_moe_layer_q4k: a device-wide barrier timed out (are all compute units free for this process?); the outputs of that call are void");
-}
-
-int run_moe_fused(const mq_moe_layer_desc* L, const SharedExpert& sh, const float* x_dev, const float* logits_dev, int64_t n,
-                  float* y_dev, int32_t* ids_out_dev, float* weights_out_dev, hipStream_t s, bool* done) {
-    *done = false;
-    const mq_weight* ge = L->gate_exps;
-    const int64_t hidden = ge->cols, inter = ge->rows, E = ge->n_experts;
-    if (n > kMoeFusedMaxTokens || E > kDecoderMaxExperts || inter > 2048 || census.on) return MQ_OK;
-    if (ge->type != kTypeQ4K || L->down_exps->type != kTypeQ4K) return MQ_OK;
-    if (L->up_exps->expert_bytes != ge->expert_bytes) return MQ_OK;
-    DecoderArgs a;
-    a.n_layers = 1;
-    a.n = (int)n;
-    a.hidden = (int)hidden, a.inter = (int)inter, a.n_q = 0, a.n_experts = (int)E, a.top_k = L->top_k;
-    a.has_shared = sh.gate ? 1 : 0;
-    a.moe_only = 1;
-    a.silu_mode = L->silu_mode;
-    a.route_mode = L->route_mode;
-    const size_t lds = decoder_layers_lds_bytes(a);
-    if (!moe_fused.sync || lds > moe_fused.lds_ready) {  // first use (or a larger shape): not capturable, like any workspace growth
-        if (int rc = decoder_grid(lds, &moe_fused.n_workgroups, &moe_fused.spin_ticks)) return rc;
-        moe_fused.lds_ready = lds;
-        if (!moe_fused.sync) {
-            const size_t bytes = decoder_sync_bytes(moe_fused.n_workgroups);
-            MQ_HIP(hipMalloc(&moe_fused.sync, bytes));
-            MQ_HIP(hipMemset(moe_fused.sync, 0, bytes));
-        }
-    }
-    const int slots = L->top_k + a.has_shared;
-    MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
-    MQ_HIP(g.part.reserve((size_t)n * (size_t)hidden * sizeof(float)));
-    RouteWs r;
-    if (int rc = carve_route(n, L->top_k, E, r)) return rc;
-    DecoderLayerDev& d = a.single;
-    d.fixed_logits = logits_dev;
-    d.gate_exps = ge->data, d.up_exps = L->up_exps->data, d.down_exps = L->down_exps->data;
-    d.gu_expert_bytes = ge->expert_bytes, d.down_expert_bytes = L->down_exps->expert_bytes;
-    if (sh.gate) {
-        d.sh_gate = sh.gate->data, d.sh_up = sh.up->data, d.sh_down = sh.down->data;
-        d.sh_gate_inp = L->sh_gate_inp_dev;
-    }
-    a.spin_ticks = moe_fused.spin_ticks;
-    a.x_in = x_dev, a.out = y_dev;
-    a.mid = (float*)g.mid.ptr, a.y = (float*)g.part.ptr;
-    a.ids_out = ids_out_dev ? ids_out_dev : r.ids;
-    a.wts_out = weights_out_dev ? weights_out_dev : r.weights;
-    a.sync = moe_fused.sync;
-    MQ_HIP(launch_decoder_layers(a, moe_fused.n_workgroups, s));
-    *done = true;
     return MQ_OK;
 }
 
@@ -1084,11 +1003,6 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
 
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    {
-        bool done = false;
-        if (int rc = run_moe_fused(L, sh, x_dev, logits_dev, n, y_dev, ids_out_dev, weights_out_dev, s, &done)) return rc;
-        if (done) return MQ_OK;
-    }
     const int slots = K + (sh.gate ? 1 : 0);  // hidden / partial rows per token
     RouteWs r;
     if (int rc = carve_route(n, K, E, r)) return rc;
@@ -1101,9 +1015,10 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     MQ_HIP(g.aq.reserve(aq_bytes(n, hidden / kQK)));
     MQ_HIP(g.ad.reserve(ad_count(n, hidden / kQK) * sizeof(float)));
     MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
-                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, n > 1, x_dev, hidden,
-                                  hidden, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
-    if (n == 1) r.direct_ids = ids;  // the routing slots of the one token are the expert groups
+                                  r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k,
+                                  n > kDirectPairsMaxTokens, x_dev, hidden, hidden, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
+    // few tokens: nearly every (token, slot) pair has an expert of its own, so the pairs are the groups
+    if (n <= kDirectPairsMaxTokens) r.direct_ids = ids;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
     if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
     return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
@@ -1344,8 +1259,7 @@ int mq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes) {
 }
 int mq_stream_synchronize(void* stream) {
     MQ_HIP(hipStreamSynchronize((hipStream_t)stream));
-    std::lock_guard<std::mutex> lock(g.mu);
-    return check_moe_fused();
+    return MQ_OK;
 }
 
 }  // extern "C"

@@ -282,13 +282,13 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         fetch_tiles<1>(dst, ws, (int64_t)blockIdx.x < ((rows + 15) >> 4) ? blockIdx.x : 0, nb);
     };
     TileRegs ahead_qkv[1];
-    if (!p.moe_only) request_dense(ahead_qkv, p.layers[0].wqkv, p.layers[0].qkv_rows, nb_h);
+    request_dense(ahead_qkv, p.layers[0].wqkv, p.layers[0].qkv_rows, nb_h);
 
     for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = p.x_in[i];
     __syncthreads();
 
     // sigmoid(sh_gate_inp . h2[t]) with the summation order of moe_combine_kernel; h2 = the MoE block's input
-    auto shared_gates = [&](const DecoderLayerDev& L, bool raw) {
+    auto shared_gates = [&](const DecoderLayerDev& L) {
         if (!p.has_shared) return;
         if (!L.sh_gate_inp) {
             if (tid < n) s.gate[tid] = 1.0f;
@@ -299,82 +299,73 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         const float* wn = L.ffn_norm;
         token_sums(
             s, n, hidden,
-            [&](int t, int c, float acc) { return fmaf(gi[c], raw ? s.xres[t * hidden + c] : normed_at(s, wn, t, hidden, c), acc); },
+            [&](int t, int c, float acc) { return fmaf(gi[c], normed_at(s, wn, t, hidden, c), acc); },
             [&](int t, float total) { s.gate[t] = stable_sigmoid(total); });
     };
 
     const float* delta = nullptr;
     for (int li = 0; li < p.n_layers; ++li) {
-        const DecoderLayerDev& L = p.layers ? p.layers[li] : p.single;
+        const DecoderLayerDev& L = p.layers[li];
 
-        if (!p.moe_only) {
-            // ---- A: residual add, rmsnorm, Q8_K, qkv projection -------------------------------------------
-            residual_norm(s, delta, n, hidden, p.eps);
-            {
-                const float* wn = L.attn_norm;
-                quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
-            }
-            __syncthreads();
-            dense_phase(s, L.wqkv, L.qkv_rows, nb_h, n, p.qkv, L.qkv_rows, ahead_qkv);
-            TileRegs ahead_wo[1];
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] { request_dense(ahead_wo, L.wo, hidden, nb_q); })) return;
-
-            // ---- B: output projection of the first n_q columns ---------------------------------------------
-            {
-                const float* src = p.qkv;
-                const int64_t ld = L.qkv_rows;
-                quantize_rows(s, n, nb_q, [&](int t, int c) { return ld_dev(src + (size_t)t * ld + c); });
-            }
-            __syncthreads();
-            dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden, ahead_wo);
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
-                    // what phase C reads that does not depend on o: this workgroup's first router row, the gate vector
-                    if ((int)blockIdx.x < n_experts) warm(L.router + (size_t)blockIdx.x * hidden, (size_t)hidden * 4, sink);
-                    if (p.has_shared && L.sh_gate_inp) warm(L.sh_gate_inp, (size_t)hidden * 4, sink);
-                }))
-                return;
-
-            // ---- C: residual add, rmsnorm, Q8_K, router projection -----------------------------------------
-            residual_norm(s, p.o, n, hidden, p.eps);
-            {
-                const float* wn = L.ffn_norm;
-                quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
-            }
-            __syncthreads();
-            // one wavefront per (token, expert), the dot of router_logits_kernel; the last wavefront takes the
-            // first unit so that the gates below, which start with the first wavefronts, run beside it
-            for (int u = (kWaves - 1 - wave) * gridDim.x + blockIdx.x; u < n * n_experts; u += kWaves * gridDim.x) {
-                const int t = u / n_experts, e = u - t * n_experts;
-                const float* wr = L.router + (size_t)e * hidden;
-                float acc = 0.0f;
-                for (int c = lane * 4; c + 3 < hidden; c += 256) {
-                    const float4 a = *reinterpret_cast<const float4*>(wr + c);
-                    acc = __fmaf_rn(a.x, normed_at(s, L.ffn_norm, t, hidden, c), acc);
-                    acc = __fmaf_rn(a.y, normed_at(s, L.ffn_norm, t, hidden, c + 1), acc);
-                    acc = __fmaf_rn(a.z, normed_at(s, L.ffn_norm, t, hidden, c + 2), acc);
-                    acc = __fmaf_rn(a.w, normed_at(s, L.ffn_norm, t, hidden, c + 3), acc);
-                }
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-                if (lane == 0) st_dev(p.logits + (size_t)t * n_experts + e, acc);
-            }
-            shared_gates(L, false);
-            if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
-                    // the shared expert's gate/up tiles of this workgroup's first unit do not wait for the routing
-                    if (p.has_shared && (int)blockIdx.x < inter / 16) {
-                        warm(L.sh_gate + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
-                        warm(L.sh_up + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
-                    }
-                }))
-                return;
-        } else {
-            // MoE block alone: x is its (already normalised) input
-            for (int t = tid; t < n; t += kThreads) s.scale[t] = 1.0f;
-            __syncthreads();
-            quantize_rows(s, n, nb_h, [&](int t, int c) { return s.xres[t * hidden + c]; });
-            __syncthreads();
-            shared_gates(L, true);
+        // ---- A: residual add, rmsnorm, Q8_K, qkv projection -------------------------------------------
+        residual_norm(s, delta, n, hidden, p.eps);
+        {
+            const float* wn = L.attn_norm;
+            quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
         }
+        __syncthreads();
+        dense_phase(s, L.wqkv, L.qkv_rows, nb_h, n, p.qkv, L.qkv_rows, ahead_qkv);
+        TileRegs ahead_wo[1];
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] { request_dense(ahead_wo, L.wo, hidden, nb_q); })) return;
+
+        // ---- B: output projection of the first n_q columns ---------------------------------------------
+        {
+            const float* src = p.qkv;
+            const int64_t ld = L.qkv_rows;
+            quantize_rows(s, n, nb_q, [&](int t, int c) { return ld_dev(src + (size_t)t * ld + c); });
+        }
+        __syncthreads();
+        dense_phase(s, L.wo, hidden, nb_q, n, p.o, hidden, ahead_wo);
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                // what phase C reads that does not depend on o: this workgroup's first router row, the gate vector
+                if ((int)blockIdx.x < n_experts) warm(L.router + (size_t)blockIdx.x * hidden, (size_t)hidden * 4, sink);
+                if (p.has_shared && L.sh_gate_inp) warm(L.sh_gate_inp, (size_t)hidden * 4, sink);
+            }))
+            return;
+
+        // ---- C: residual add, rmsnorm, Q8_K, router projection -----------------------------------------
+        residual_norm(s, p.o, n, hidden, p.eps);
+        {
+            const float* wn = L.ffn_norm;
+            quantize_rows(s, n, nb_h, [&](int t, int c) { return normed_at(s, wn, t, hidden, c); });
+        }
+        __syncthreads();
+        // one wavefront per (token, expert), the dot of router_logits_kernel; the last wavefront takes the
+        // first unit so that the gates below, which start with the first wavefronts, run beside it
+        for (int u = (kWaves - 1 - wave) * gridDim.x + blockIdx.x; u < n * n_experts; u += kWaves * gridDim.x) {
+            const int t = u / n_experts, e = u - t * n_experts;
+            const float* wr = L.router + (size_t)e * hidden;
+            float acc = 0.0f;
+            for (int c = lane * 4; c + 3 < hidden; c += 256) {
+                const float4 a = *reinterpret_cast<const float4*>(wr + c);
+                acc = __fmaf_rn(a.x, normed_at(s, L.ffn_norm, t, hidden, c), acc);
+                acc = __fmaf_rn(a.y, normed_at(s, L.ffn_norm, t, hidden, c + 1), acc);
+                acc = __fmaf_rn(a.z, normed_at(s, L.ffn_norm, t, hidden, c + 2), acc);
+                acc = __fmaf_rn(a.w, normed_at(s, L.ffn_norm, t, hidden, c + 3), acc);
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+            if (lane == 0) st_dev(p.logits + (size_t)t * n_experts + e, acc);
+        }
+        shared_gates(L);
+        if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
+                // the shared expert's gate/up tiles of this workgroup's first unit do not wait for the routing
+                if (p.has_shared && (int)blockIdx.x < inter / 16) {
+                    warm(L.sh_gate + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
+                    warm(L.sh_up + tile_offset(blockIdx.x, 0, nb_h), (size_t)nb_h * kTileBytes, sink);
+                }
+            }))
+            return;
 
         // ---- D: routing, then gate/up + SwiGLU per (token, slot) and for the shared expert -------------------
         float routed_logit = 0.0f;  // lane k of wavefront t: logit of token t's k-th expert
@@ -557,18 +548,18 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         }
         {
             // the next layer's first projection (the last layer re-requests its own: unused, but defined)
-            const DecoderLayerDev& N = p.layers ? p.layers[li + 1 < p.n_layers ? li + 1 : li] : p.single;
+            const DecoderLayerDev& N = p.layers[li + 1 < p.n_layers ? li + 1 : li];
             if (!grid_barrier(p.sync, my_gen, s.ok, p.spin_ticks, [&] {
-                    if (!p.moe_only) request_dense(ahead_qkv, N.wqkv, N.qkv_rows, nb_h);
+                    request_dense(ahead_qkv, N.wqkv, N.qkv_rows, nb_h);
                 }))
                 return;
         }
         delta = p.y;
     }
 
-    // ---- the last residual add (or, for the MoE block alone, its output as it is) ---------------------------
+    // ---- the last residual add ---------------------------------------------------------------------------------
     for (int i = blockIdx.x * kThreads + tid; i < n * hidden; i += gridDim.x * kThreads)
-        p.out[i] = p.moe_only ? ld_dev(p.y + i) : __fadd_rn(s.xres[i], ld_dev(p.y + i));
+        p.out[i] = __fadd_rn(s.xres[i], ld_dev(p.y + i));
     if (sink == 0x9e3779b9u && p.n < 0) p.out[0] = 0.0f;  // never true: keeps the warm-up reads alive
 }
 
@@ -591,10 +582,9 @@ hipError_t prepare_decoder_layers(size_t lds_bytes) {
 }
 
 hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStream_t stream) {
-    if ((!a.layers && (!a.moe_only || a.n_layers != 1)) || a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
+    if (!a.layers || a.n_layers < 1 || a.n < 1 || a.n > 8 || a.top_k < 1 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > kDecoderMaxExperts ||
         a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || a.inter > kMaxInterBlocks * kQK ||
-        n_workgroups < 1 ||
-        (!a.moe_only && (a.n_q <= 0 || (a.n_q % kQK))))
+        n_workgroups < 1 || a.n_q <= 0 || (a.n_q % kQK))
         return hipErrorInvalidValue;
     hipLaunchKernelGGL(decoder_layers_kernel, dim3((unsigned)n_workgroups), dim3(kThreads), decoder_layers_lds_bytes(a),
                        stream, a);

@@ -61,7 +61,8 @@ struct MatmulArgs {
     int a_tok_stride = 1, a_k_stride = 0;   // activation row of an entry = token * a_tok_stride + k * a_k_stride
     int y_tok_stride = 1, y_k_stride = 0;   // output row of an entry
     int max_groups = 0;
-    // one-token shortcut: group g is routing slot g of token 0 with expert direct_ids[g]; no lists are read
+    // few tokens: group g is the pair (token g / direct_top_k, slot g % direct_top_k) with expert direct_ids[g];
+    // no lists are read (grouping by expert shares nothing when nearly every pair has an expert of its own)
     const int32_t* direct_ids = nullptr;
     int direct_top_k = 0;
     int n_experts = 0;             // for range-checking direct_ids
@@ -149,7 +150,7 @@ hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream);
 // device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.
 constexpr int kDecoderMaxExperts = 512;
 constexpr int kTokenMajorDownMaxTokens = 4;  // widest MoE block whose down projection runs token-major (measured: 8 and 16 lose)
-constexpr int kMoeFusedMaxTokens = 2;  // widest MoE block that mq_moe_layer_q4k runs as one launch
+constexpr int kDirectPairsMaxTokens = 4;  // widest MoE block whose (token, slot) pairs are not grouped by expert
 struct DecoderLayerDev {               // one per layer, in device memory
     const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]
     const uint8_t* wo = nullptr;       // [hidden x n_q]; its input is qkv[:, :n_q]
@@ -168,13 +169,11 @@ struct DecoderLayerDev {               // one per layer, in device memory
     const float* sh_gate_inp = nullptr;  // fp32 [hidden] or null (gate = 1)
 };
 struct DecoderArgs {
-    const DecoderLayerDev* layers = nullptr;  // device table; null: one MoE block described by `single`
-    DecoderLayerDev single;
+    const DecoderLayerDev* layers = nullptr;  // device table
     int n_layers = 0;
     int n = 0;                         // tokens, 1..8
     int hidden = 0, inter = 0, n_q = 0, n_experts = 0, top_k = 0;
     int has_shared = 0;
-    int moe_only = 0;                  // 1: every "layer" is the MoE block alone on x (no projections, no residual)
     int silu_mode = 0, route_mode = 0;
     float eps = 0.0f;
     long long spin_ticks = 0;          // barrier patience in wall_clock64 ticks

@@ -48,8 +48,11 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
         ar = (begin + e) * p.sh_arow_stride + p.sh_arow_offset;
         yr = (begin + e) * p.sh_yrow_stride + p.sh_yrow_offset;
     } else {
-        int tok = 0, kk = begin + e;  // one-token shortcut: entry = (token 0, slot begin)
-        if (!p.direct_ids) {
+        int tok, kk;
+        if (p.direct_ids) {  // few tokens: the group is the one pair `begin` = (token, slot); e is always 0
+            tok = begin / p.direct_top_k;  // wave-uniform
+            kk = begin - tok * p.direct_top_k;
+        } else {
             tok = p.entry_token[begin + e];
             kk = p.entry_k[begin + e];
         }
@@ -98,8 +101,8 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
         // possible group), so they cost one memory round trip, not three
         const int g = blockIdx.y;
         int ng, g_expert, g_begin, g_end;
-        if (p.direct_ids) {  // one token: its routing slots are the groups, nothing was sorted
-            ng = p.direct_top_k;
+        if (p.direct_ids) {  // few tokens: every (token, slot) pair is a group of its own, nothing was sorted
+            ng = p.direct_top_k * (int)p.n;
             g_expert = p.direct_ids[g < ng ? g : 0];
             g_begin = g;
             g_end = g + 1;

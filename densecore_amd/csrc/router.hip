@@ -254,6 +254,7 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
                           ids + (size_t)tok * top_k, weights + (size_t)tok * top_k, !solo);
         __syncthreads();  // keys / sel are reused by the next token and by the grouping below
     }
+    if (!build_groups) return;  // the consumer takes the ids as they are (few tokens)
     if (!solo) {
         // the ids were stored device-coherently; wait for their acknowledgement before being counted
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -266,7 +267,6 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
         __syncthreads();
         if (!is_last) return;
     }
-    if (!build_groups) return;  // the consumer takes the ids as they are (one token)
     int32_t* count = reinterpret_cast<int32_t*>(route_sh);
     int32_t* ids_s = count + n_experts;
     const int n_entries = n * top_k;

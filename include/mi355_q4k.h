@@ -201,10 +201,9 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  *   route top_k -> gate/up + SwiGLU per (token, k) -> Q8_K -> down ->
  *   y[t] = sum_k w[t][k] * down_k (k in routing order) + sigmoid(sh_gate_inp . x[t]) * shared_ffn(x[t]).
  * shared_* may all be NULL (no shared expert); sh_gate_inp_dev fp32 [hidden] or NULL (gate = 1).
- * With one or two tokens, Q4_K experts and n_experts <= 512 the whole block is one persistent launch whose
- * workgroups meet at device-wide barriers (same arithmetic, same bits); should such a barrier not be met within
- * 200 ms -- other work holding compute units -- the launch drains, the outputs are void and the next
- * mq_stream_synchronize returns MQ_ERR_STATE. */
+ * Three launches at decode widths: router (+ expert grouping above four tokens, + Q8_K of x), gate/up + SwiGLU
+ * leaving its rows in Q8_K, down with the weighted combine inside (up to four tokens; a combine launch of its
+ * own above). */
 typedef struct {
     const mq_weight* gate_exps; /* n_experts x [inter][hidden]  */
     const mq_weight* up_exps;
