@@ -713,6 +713,12 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     return MQ_OK;
 }
 
+// Does the down projection of this MoE block run token-major (moe_down.hip)?
+bool token_major_down(const mq_weight* down, int64_t n, int slots) {
+    return n <= kTokenMajorDownMaxTokens && !census.on && (down->rows & 15) == 0 &&
+           (size_t)slots * (size_t)down->nb * 64 <= 48 * 1024;
+}
+
 // Q8_K of the hidden rows, down projection per (token, k) into g.part, then the weighted combine.
 int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hidden, bool hidden_is_quantized, int64_t n,
                  int top_k, int slots, const RouteWs& r, const int32_t* ids, const float* weights,
@@ -721,12 +727,13 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     const int64_t mid_rows = n * slots;
     const int64_t inter = down->cols, hidden_dim = down->rows;
     // rows of dropped entries may hold anything; they are never read
-    if (!hidden_is_quantized) {
+    const bool token_major = token_major_down(down, n, slots);
+    if (!hidden_is_quantized && !token_major) {
         if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
     }
-    if (n <= kTokenMajorDownMaxTokens && !census.on && (hidden_dim & 15) == 0 &&
-        (size_t)slots * (size_t)down->nb * 64 <= 48 * 1024) {
-        // few tokens: a workgroup per (token, 16 output rows) multiplies and combines in one launch
+    if (token_major) {
+        // few tokens: a workgroup per (token, 16 output rows) multiplies and combines in one launch, and
+        // quantizes the hidden rows it reads when they come as fp32
         MoeDownTokenArgs a;
         a.w = down->data;
         a.expert_bytes = down->expert_bytes;
@@ -734,7 +741,8 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
         a.wtype = down->type;
         a.rows = hidden_dim, a.nb = down->nb, a.n = n;
         a.top_k = top_k, a.n_experts = (int)down->n_experts;
-        a.aq = (const uint8_t*)g.aq2.ptr, a.ad = (const float*)g.ad2.ptr;
+        if (hidden_is_quantized) a.aq = (const uint8_t*)g.aq2.ptr, a.ad = (const float*)g.ad2.ptr;
+        else a.hidden = hidden;
         a.ids = ids, a.weights = weights;
         a.sh_gate_inp = sh_gate_inp, a.x = x, a.y = y;
         MQ_HIP(launch_moe_down_token(a, s));
@@ -1020,8 +1028,11 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     // few tokens: nearly every (token, slot) pair has an expert of its own, so the pairs are the groups
     if (n <= kDirectPairsMaxTokens) r.direct_ids = ids;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
-    if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, true, s)) return rc;
-    return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, true, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
+    // the hidden rows leave gate/up in Q8_K, unless the token-major down launch quantizes what it reads itself
+    const bool quantize_in_gateup = !token_major_down(L->down_exps, n, slots);
+    if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, quantize_in_gateup, s))
+        return rc;
+    return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, quantize_in_gateup, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
                         x_dev, y_dev, s);
 }
 

@@ -224,21 +224,6 @@ __device__ __forceinline__ void dense_phase(const Shared& s, const uint8_t* w, i
     }
 }
 
-// The A operand of one activation row quantized by this wavefront (row 0 of the tile; the other rows are dead):
-// codes move from the quantizer's lanes into the split-slot operand with eight cross-lane reads per super-block.
-__device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
-    const int slot = lane & 15, kq = lane >> 4;
-    const int src = 8 * (slot & 1) + 2 * kq;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const uint32_t lo = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
-        const uint32_t hi = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
-        a.q[0][c] = slot == 0 ? v4u{lo, hi, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, lo, hi} : v4u{0u, 0u, 0u, 0u});
-    }
-    a.yd[0][0] = q.d;
-    a.yd[0][1] = 0.0f;
-}
-
 constexpr int kItems = 3;  // (slot, super-block) items of the down projection a wavefront keeps in flight
 
 __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderArgs p) {

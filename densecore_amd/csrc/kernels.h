@@ -126,7 +126,7 @@ hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
 
 // ---- moe_down.hip ----------------------------------------------------------------------------
 // Down projection + weighted combine, one workgroup per (token, 16 output rows): for decode widths, where
-// grouping by expert shares nothing.  Hidden rows are Q8_K in the A-major layout, row = token * slots + slot.
+// grouping by expert shares nothing.  Hidden rows (row = token * slots + slot) are Q8_K in the A-major layout or fp32.
 struct MoeDownTokenArgs {
     const uint8_t* w = nullptr;        // tiled down experts [n_experts][rows x nb]
     size_t expert_bytes = 0;
@@ -135,8 +135,9 @@ struct MoeDownTokenArgs {
     int64_t rows = 0, nb = 0;          // output rows (hidden), super-blocks per row (inter / 256)
     int64_t n = 0;
     int top_k = 0, n_experts = 0;
-    const uint8_t* aq = nullptr;       // A-major hidden rows
+    const uint8_t* aq = nullptr;       // A-major hidden rows, or
     const float* ad = nullptr;
+    const float* hidden = nullptr;     // fp32 hidden rows [n * slots][nb * 256] (quantized inside the kernel)
     const int32_t* ids = nullptr;      // [n][top_k]
     const float* weights = nullptr;    // [n][top_k]
     const float* sh_gate_inp = nullptr;  // [rows] or null (gate = 1)

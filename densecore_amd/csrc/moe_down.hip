@@ -8,9 +8,13 @@
 // (cb_qwen35_native_moe_down_q5k_weighted_logits, core/src/llm/moe/native.cpp:3051-3295; zero weights and ids out
 // of range skipped as at :3237).  Per-tile arithmetic, the order of the super-block terms and of the slots, and
 // the gate are those of the grouped launch + moe_combine_kernel: same bits, one launch less, no partial rows.
+// kFromF32: the hidden rows come as fp32 and every wavefront quantizes the super-blocks it multiplies (the block
+// quantizer of quantize_q8k_kernel: same codes and scale), which takes the re-quantization off the tail of the
+// gate/up launch; the work is repeated by every workgroup of a token, a few hundred instructions each.
 #include "common.h"
 #include "kernels.h"
 #include "decode_tile.h"
+#include "q8k_block.h"
 #include "route_block.h"
 
 namespace mq {
@@ -20,7 +24,7 @@ namespace {
 constexpr int kWaves = 8;
 constexpr int kItems = 3;  // (slot, super-block) items a wavefront keeps in flight
 
-template <int WT>
+template <int WT, bool kFromF32>
 __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDownTokenArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
     extern __shared__ float term[];  // [slots * nb][16], then 4 floats of gate scratch
@@ -43,6 +47,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
     for (int base = 0; base < n_items; base += kWaves * kItems) {
         typename TileOf<WT>::Regs tiles[kItems];
         ARegs<1> a[kItems];
+        float4 hv[kItems];
 #pragma unroll
         for (int j = 0; j < kItems; ++j) {  // every load is issued; a missing item reads a harmless tile
             const int i = base + wave + kWaves * j;
@@ -50,11 +55,15 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
             const uint8_t* w = i < n_items ? item_tile(i) : nullptr;
             load_tile_wt<WT>(tiles[j], w ? w : p.w, lane);
             const int sl = ii / nb, b = ii - sl * nb;
-            const int64_t row = t * slots + sl;  // hidden row; its 8-row tile comes along, only this row is kept
-            const int64_t row0 = row & ~(int64_t)7;
-            const size_t a_off[1] = {aq_row_offset(row0 + (slot >> 1), nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16};
-            const int d_idx[1][2] = {{(int)ad_index(row0 + 2 * kq, 0, nb), (int)ad_index(row0 + 2 * kq + 1, 0, nb)}};
-            load_a<1>(a[j], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+            const int64_t row = t * slots + sl;  // hidden row
+            if (kFromF32) {
+                hv[j] = *reinterpret_cast<const float4*>(p.hidden + (size_t)row * (size_t)(nb * kQK) + (size_t)b * kQK + lane * 4);
+            } else {  // its 8-row tile comes along, only this row is kept
+                const int64_t row0 = row & ~(int64_t)7;
+                const size_t a_off[1] = {aq_row_offset(row0 + (slot >> 1), nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16};
+                const int d_idx[1][2] = {{(int)ad_index(row0 + 2 * kq, 0, nb), (int)ad_index(row0 + 2 * kq + 1, 0, nb)}};
+                load_a<1>(a[j], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+            }
         }
         if (base == 0 && p.sh_w) {  // the shared expert's gate while the tiles travel (moe_combine_kernel's order)
             float gate = 1.0f;
@@ -77,10 +86,14 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
             if (i < n_items) {  // wave-uniform
                 float acc[1][2] = {{0.0f, 0.0f}};
                 if (item_tile(i)) {
+                    if (kFromF32) {  // the row becomes row 0 of the operand
+                        const float e[4] = {hv[j].x, hv[j].y, hv[j].z, hv[j].w};
+                        a_from_lane_codes(a[j], quantize_block_q8k(e, lane), lane);
+                    }
                     int32_t dsum[1][2], msum[1][2];
                     compute_tile_wt<1, WT>(tiles[j], a[j], acc, dsum, msum, lane);
                 }
-                const int pos = (int)((t * slots + i / nb) & 7);  // the row's place in its 8-row tile
+                const int pos = kFromF32 ? 0 : (int)((t * slots + i / nb) & 7);  // the row's place in its 8-row tile
                 if (kq == (pos >> 1)) term[i * 16 + slot] = (pos & 1) ? acc[0][1] : acc[0][0];
             }
         }
@@ -113,10 +126,17 @@ hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) 
     const size_t lds = (size_t)slots * (size_t)a.nb * 16 * sizeof(float);
     if (lds > 48 * 1024) return hipErrorInvalidValue;
     const dim3 grid((unsigned)(a.rows / 16), (unsigned)a.n);
-    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ6>, grid, dim3(kWaves * 64), lds, stream, a);
-    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ5>, grid, dim3(kWaves * 64), lds, stream, a);
-    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_down_token_kernel<kWtQ4>, grid, dim3(kWaves * 64), lds, stream, a);
+    if ((a.hidden == nullptr) == (a.aq == nullptr)) return hipErrorInvalidValue;  // one source of hidden rows
+#define MQ_DOWN_TOKEN(WT)                                                                                              \
+    do {                                                                                                               \
+        if (a.hidden) hipLaunchKernelGGL((moe_down_token_kernel<WT, true>), grid, dim3(kWaves * 64), lds, stream, a);  \
+        else hipLaunchKernelGGL((moe_down_token_kernel<WT, false>), grid, dim3(kWaves * 64), lds, stream, a);          \
+    } while (0)
+    if (a.wtype == kTypeQ6K) MQ_DOWN_TOKEN(kWtQ6);
+    else if (a.wtype == kTypeQ5K) MQ_DOWN_TOKEN(kWtQ5);
+    else if (a.wtype == kTypeQ4K) MQ_DOWN_TOKEN(kWtQ4);
     else return hipErrorInvalidValue;
+#undef MQ_DOWN_TOKEN
     return hipGetLastError();
 }
 

@@ -10,6 +10,7 @@
 #pragma once
 
 #include "common.h"
+#include "decode_tile.h"
 
 namespace mq {
 
@@ -75,6 +76,21 @@ __device__ __forceinline__ void store_amajor(uint8_t* aq, float* ad, int64_t m, 
     *reinterpret_cast<uint32_t*>(aq + off + h * 8) = r.packed;
     *reinterpret_cast<uint32_t*>(aq + off + (1 - h) * 8) = 0u;
     if (lane == 0) ad[ad_index(m, b, nb)] = r.d;
+}
+
+// The A operand of one activation row quantized by this wavefront (row 0 of the tile; the other rows are dead):
+// codes move from the quantizer's lanes into the split-slot operand with eight cross-lane reads per super-block.
+__device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
+    const int slot = lane & 15, kq = lane >> 4;
+    const int src = 8 * (slot & 1) + 2 * kq;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t lo = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
+        const uint32_t hi = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
+        a.q[0][c] = slot == 0 ? v4u{lo, hi, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, lo, hi} : v4u{0u, 0u, 0u, 0u});
+    }
+    a.yd[0][0] = q.d;
+    a.yd[0][1] = 0.0f;
 }
 #endif
 
