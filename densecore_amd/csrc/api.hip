@@ -1173,6 +1173,13 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
     // decode widths use the exact exponential, wider ones the polynomial (core/src/llm/moe/native.cpp:3614-3616)
     a.silu_mode = silu_mode >= 0 ? silu_mode : (n <= 4 ? MQ_SILU_EXACT : MQ_SILU_FAST);
     a.route_mode = d->route_mode;
+    {
+        // the expert gate/up launch of mq_moe_layer_q4k at this width: (token, slot) pairs up to four tokens, expert
+        // groups above, plus one pass of the shared expert; the kernel keeps that launch's summation order
+        const int64_t pairs = n * (int64_t)d->top_k;
+        const int64_t groups = (n <= kDirectPairsMaxTokens || pairs < d->n_experts ? pairs : d->n_experts) + (d->has_shared ? (n + 7) / 8 : 0);
+        a.gateup_order = pick_waves(d->hidden / kQK, (int64_t)(d->inter / 16) * groups);
+    }
     a.eps = d->eps;
     a.spin_ticks = d->spin_ticks;
     a.x_in = x_dev, a.out = out_dev;

@@ -152,9 +152,12 @@ __device__ __forceinline__ void fetch_tiles(TileRegs (&t)[NMAT], const uint8_t* 
 // One 16-row tile of NMAT matrices against the LDS activations: the waves split the super-blocks
 // (b = wave, wave + 8, ...), partial sums meet in wave order, wave 0 ends up with the totals.  `first` holds
 // the tiles of super-block `wave` (fetch_tiles).
+// `order`: the wavefronts per row tile of the one-node launch whose summation order is to be kept when every
+// wavefront here holds one super-block (nb <= 8): that launch adds the super-blocks w, w + order, ... in each of
+// its `order` wavefronts and then the wavefronts' sums in turn.  order == 8 is this kernel's own order.
 template <int NMAT>
 __device__ __forceinline__ void tile_rows(const Shared& s, const TileRegs (&first)[NMAT], const uint8_t* const (&w)[NMAT],
-                                          int64_t rt, int nb, int n, float (&acc)[NMAT][1][2]) {
+                                          int64_t rt, int nb, int n, float (&acc)[NMAT][1][2], int order = kWaves) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
@@ -188,12 +191,38 @@ __device__ __forceinline__ void tile_rows(const Shared& s, const TileRegs (&firs
     }
     __syncthreads();
     if (wave == 0) {
-        for (int wv = 1; wv < kWaves; ++wv) {
+        if (order >= kWaves || nb > kWaves) {
+            for (int wv = 1; wv < kWaves; ++wv) {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[m][0][j] = __fadd_rn(acc[m][0][j], s.red[(((wv - 1) * NMAT + m) * 2 + j) * 64 + lane]);
+            }
+        } else {
+            // wavefront wv of this kernel holds the term of super-block wv alone (zero past the last one)
+            float total[NMAT][2];
+            for (int ow = 0; ow < order; ++ow) {
+                float part[NMAT][2];
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) part[m][j] = ow == 0 ? acc[m][0][j] : s.red[(((ow - 1) * NMAT + m) * 2 + j) * 64 + lane];
+                for (int b = ow + order; b < nb; b += order) {
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) part[m][j] = __fadd_rn(part[m][j], s.red[(((b - 1) * NMAT + m) * 2 + j) * 64 + lane]);
+                }
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) total[m][j] = ow == 0 ? part[m][j] : __fadd_rn(total[m][j], part[m][j]);
+            }
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[m][0][j] = __fadd_rn(acc[m][0][j], s.red[(((wv - 1) * NMAT + m) * 2 + j) * 64 + lane]);
+                for (int j = 0; j < 2; ++j) acc[m][0][j] = total[m][j];
         }
     }
 }
@@ -412,7 +441,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
                 if (live) {  // the whole workgroup takes the same branch
                     const uint8_t* const wc[2] = {ws[0], ws[1]};
                     float acc[2][1][2];
-                    tile_rows<2>(s, cur, wc, rt, nb_h, n, acc);
+                    tile_rows<2>(s, cur, wc, rt, nb_h, n, acc, p.gateup_order);
                     if (wave == 0) {
                         const int mode = shared ? 2 : p.silu_mode;
 #pragma unroll

@@ -176,6 +176,7 @@ struct DecoderArgs {
     int hidden = 0, inter = 0, n_q = 0, n_experts = 0, top_k = 0;
     int has_shared = 0;
     int silu_mode = 0, route_mode = 0;
+    int gateup_order = 8;              // wavefronts per row tile of the one-node expert gate/up launch at this width (pick_waves)
     float eps = 0.0f;
     long long spin_ticks = 0;          // barrier patience in wall_clock64 ticks
     const float* x_in = nullptr;       // [n x hidden]

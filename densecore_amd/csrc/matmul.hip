@@ -330,10 +330,12 @@ hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t str
 }  // namespace
 
 // Waves per workgroup: the chip holds 2 waves per SIMD of this kernel (2048 in all); aim at filling
-// that once, with a count that divides the super-blocks of a row evenly and at most 8.
+// that once and never overfilling it -- a launch a few wavefronts over the limit waits for a second round of
+// workgroups that start when the first ones end -- with a count that divides the super-blocks of a row evenly
+// and at most 8.
 int pick_waves(int64_t nb, int64_t workgroups) {
     const int64_t target = 2048;
-    int64_t ideal = (target + workgroups - 1) / (workgroups > 0 ? workgroups : 1);
+    int64_t ideal = target / (workgroups > 0 ? workgroups : 1);
     if (ideal < 1) ideal = 1;
     if (ideal > 8) ideal = 8;
     if (ideal > nb) ideal = nb;

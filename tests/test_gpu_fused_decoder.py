@@ -76,8 +76,8 @@ def test_full_size_layers_bitwise_equal(ds, n, fixed):
     """hidden 2048, 256 experts + shared, inter 512, top-8, 16 query / 2 KV heads of 128: three layers."""
     cfg = ds.StepConfig(n_layers=3, seed=11)
     step, fused, x = _pair(ds, cfg, n, 5 + n, fixed)
-    # wider steps: the node-by-node gate/up launch splits K over two wavefronts, the fused kernel over eight
-    _assert_same(step, fused, x, exact=(n == 1))
+    # the fused kernel adds a row tile's super-blocks in the order of the node-by-node gate/up launch of this width
+    _assert_same(step, fused, x)
     fused.free()
     step.free()
 
