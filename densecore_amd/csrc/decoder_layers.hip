@@ -61,14 +61,23 @@ struct Shared {
 // takes columns j, j + 256, ... with fused multiply-adds, a butterfly inside each of the four wavefronts,
 // then (w0 + w1) + (w2 + w3).  Here the (token, wavefront) pairs are spread over the eight wavefronts;
 // term(t, c, acc) returns the running sum with column c of token t added, finish(t, total) consumes a total.
-template <typename Term, typename Finish>
+// kBlocks: the order of add_rmsnorm_blocks_kernel instead -- wavefront v takes the super-blocks v, v + 4, ... and
+// lane l their elements 4l .. 4l+3 in turn.
+template <bool kBlocks, typename Term, typename Finish>
 __device__ __forceinline__ void token_sums(const Shared& s, int n, int hidden, Term term, Finish finish) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     for (int i = wave; i < 4 * n; i += kWaves) {
         const int t = i >> 2, v = i & 3;
         float acc = 0.0f;
+        if (kBlocks) {
+            for (int c0 = v * kQK + lane * 4; c0 < hidden; c0 += 4 * kQK) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc = term(t, c0 + q, acc);
+            }
+        } else {
 #pragma unroll 4
-        for (int c = v * 64 + lane; c < hidden; c += 256) acc = term(t, c, acc);
+            for (int c = v * 64 + lane; c < hidden; c += 256) acc = term(t, c, acc);
+        }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
         if (lane == 0) s.vsum[i] = acc;
@@ -86,7 +95,7 @@ __device__ __forceinline__ void residual_norm(const Shared& s, const float* delt
         for (int i = tid; i < n * hidden; i += kThreads) s.xres[i] = __fadd_rn(s.xres[i], ld_dev(delta + i));
         __syncthreads();
     }
-    token_sums(
+    token_sums<true>(
         s, n, hidden,
         [&](int t, int c, float acc) {
             const float v = s.xres[t * hidden + c];
@@ -311,7 +320,7 @@ __global__ void __launch_bounds__(kThreads) decoder_layers_kernel(const DecoderA
         }
         const float* gi = L.sh_gate_inp;
         const float* wn = L.ffn_norm;
-        token_sums(
+        token_sums<false>(
             s, n, hidden,
             [&](int t, int c, float acc) { return fmaf(gi[c], normed_at(s, wn, t, hidden, c), acc); },
             [&](int t, float total) { s.gate[t] = stable_sigmoid(total); });

@@ -13,7 +13,8 @@ namespace {
 // sum[t] = x[t] + delta[t] (delta may be null); normed[t] = sum[t] * (rsqrt(mean(sum^2) + eps) * weight)
 // AddRMSNorm (core/src/kernels/hwy/hwy_normalization.cc:102-153; plain form in
 // core/tests/kernels/test_normalization.cpp:57-68).  One workgroup per token; the squares are
-// summed per thread in column order, then across lanes and waves in a fixed order.
+// summed per thread in column order, then across lanes and waves in a fixed order.  This general form takes
+// rows of any length and alignment; rows of whole super-blocks take add_rmsnorm_blocks_kernel below.
 // When q_aq is given (cols % 256 == 0) the normalised row also leaves as Q8_K in the layout the matmul
 // kernels read, quantized from the very floats that normed_out receives.
 __global__ void __launch_bounds__(256) add_rmsnorm_kernel(const float* x, const float* __restrict__ delta,
@@ -56,6 +57,76 @@ __global__ void __launch_bounds__(256) add_rmsnorm_kernel(const float* x, const 
     }
 }
 
+// The same operator for rows of whole super-blocks (cols % 256 == 0: every projection input), one pass: wavefront v of
+// the workgroup owns the super-blocks v, v + 4, ... of the row and lane l their elements 4l .. 4l+3 -- the mapping
+// the quantizer wants -- from the first load on, and keeps up to kKeep super-blocks in registers, so nothing is read
+// twice and nothing waits for a store.  The squares are summed per thread in that order (super-block by
+// super-block, element by element), then across the lanes of a wavefront by butterfly, then (w0 + w1) + (w2 + w3).
+// kKeep == 0: longer rows; the thread re-reads what it stored (or adds again).
+template <int kKeep>
+__global__ void __launch_bounds__(256) add_rmsnorm_blocks_kernel(const float* x, const float* __restrict__ delta,
+                                                                 const float* __restrict__ weight, int64_t cols, float eps,
+                                                                 float* sum_out, float* __restrict__ normed_out,
+                                                                 uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
+    __shared__ float wave_sum[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t base = (int64_t)blockIdx.x * cols;
+    const int64_t nb = cols / kQK;
+    auto fetch = [&](int64_t c0) {
+        float4 a = *reinterpret_cast<const float4*>(x + base + c0);
+        if (delta) {
+            const float4 d = *reinterpret_cast<const float4*>(delta + base + c0);
+            a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
+        }
+        return a;
+    };
+    float4 kept[kKeep > 0 ? kKeep : 1];
+    float ssq = 0.0f;
+    auto first_pass = [&](int64_t b, float4& slot) {
+        const int64_t c0 = b * kQK + lane * 4;
+        const float4 a = fetch(c0);
+        if (sum_out) *reinterpret_cast<float4*>(sum_out + base + c0) = a;
+        ssq = __fmaf_rn(a.x, a.x, ssq);
+        ssq = __fmaf_rn(a.y, a.y, ssq);
+        ssq = __fmaf_rn(a.z, a.z, ssq);
+        ssq = __fmaf_rn(a.w, a.w, ssq);
+        slot = a;
+    };
+    if (kKeep > 0) {
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i)
+            if (wave + 4 * i < nb) first_pass(wave + 4 * i, kept[i]);
+    } else {
+        for (int64_t b = wave; b < nb; b += 4) first_pass(b, kept[0]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+    if (lane == 0) wave_sum[wave] = ssq;
+    __syncthreads();
+    const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+    const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
+    auto second_pass = [&](int64_t b, const float4& a) {
+        const int64_t c0 = b * kQK + lane * 4;
+        float4 w = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+        if (weight) w = *reinterpret_cast<const float4*>(weight + c0);
+        const float e[4] = {__fmul_rn(a.x, weight ? __fmul_rn(scale, w.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, w.y) : scale),
+                            __fmul_rn(a.z, weight ? __fmul_rn(scale, w.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, w.w) : scale)};
+        if (normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = make_float4(e[0], e[1], e[2], e[3]);
+        if (q_aq) store_amajor(q_aq, q_ad, blockIdx.x, b, nb, lane, quantize_block_q8k(e, lane));
+    };
+    if (kKeep > 0) {
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i)
+            if (wave + 4 * i < nb) second_pass(wave + 4 * i, kept[i]);
+    } else {
+        for (int64_t b = wave; b < nb; b += 4) {
+            const int64_t c0 = b * kQK + lane * 4;
+            // sum_out may alias x: the thread re-reads what it stored itself rather than adding delta twice
+            second_pass(b, sum_out ? *reinterpret_cast<const float4*>(sum_out + base + c0) : fetch(c0));
+        }
+    }
+}
+
 // logits[t][e] = w[e] . x[t], fp32 (the ffn_gate_inp projection, core/src/llm/graph/decoder.cpp:2265).
 // One wavefront per (expert, token): lanes stride the columns, fixed-order butterfly at the end.
 __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restrict__ w, int64_t n_experts,
@@ -88,8 +159,19 @@ hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* w
                               hipStream_t stream) {
     if (n == 0) return hipSuccess;
     if (q_aq && (cols % kQK)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
-                       normed_out, q_aq, q_ad);
+    const bool vec = (cols % kQK) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(delta) |
+                                            reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(sum_out) |
+                                            reinterpret_cast<uintptr_t>(normed_out)) & 15u) == 0;
+    if (vec && cols <= 4 * 4 * kQK) {
+        hipLaunchKernelGGL(add_rmsnorm_blocks_kernel<4>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
+                           sum_out, normed_out, q_aq, q_ad);
+    } else if (vec) {
+        hipLaunchKernelGGL(add_rmsnorm_blocks_kernel<0>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
+                           sum_out, normed_out, q_aq, q_ad);
+    } else {
+        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
+                           normed_out, q_aq, q_ad);
+    }
     return hipGetLastError();
 }
 
