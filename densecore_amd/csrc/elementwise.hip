@@ -139,14 +139,26 @@ __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restr
     const float* wr = w + e * cols;
     const float* xr = x + t * ldx;
     float acc = 0.0f;
-    for (int64_t c = (int64_t)lane * 4; c + 3 < cols; c += 256) {
-        const float4 a = *reinterpret_cast<const float4*>(wr + c);
-        const float4 b = *reinterpret_cast<const float4*>(xr + c);
+    auto add4 = [&](const float4& a, const float4& b) {
         acc = __fmaf_rn(a.x, b.x, acc);
         acc = __fmaf_rn(a.y, b.y, acc);
         acc = __fmaf_rn(a.z, b.z, acc);
         acc = __fmaf_rn(a.w, b.w, acc);
+    };
+    // same order of additions as one column group after the other; the operands of eight groups are requested
+    // together so that their latencies overlap (a row of 2048 columns is one such batch)
+    int64_t c = (int64_t)lane * 4;
+    for (; c + 7 * 256 + 3 < cols; c += 8 * 256) {
+        float4 a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            a[u] = *reinterpret_cast<const float4*>(wr + c + u * 256);
+            b[u] = *reinterpret_cast<const float4*>(xr + c + u * 256);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) add4(a[u], b[u]);
     }
+    for (; c + 3 < cols; c += 256) add4(*reinterpret_cast<const float4*>(wr + c), *reinterpret_cast<const float4*>(xr + c));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
     if (lane == 0) logits[t * n_experts + e] = acc;

@@ -27,9 +27,11 @@ constexpr int kItems = 3;  // (slot, super-block) items a wavefront keeps in fli
 template <int WT, bool kFromF32>
 __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDownTokenArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
-    extern __shared__ float term[];  // [slots * nb][16], then 4 floats of gate scratch
+    extern __shared__ float term[];  // [slots * nb][16]
     __shared__ float wave_sum[4];
     __shared__ float gate_sh;
+    __shared__ int ids_sh[8];        // the token's experts and routing weights, fetched once
+    __shared__ float wts_sh[8];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int slot = lane & 15, kq = lane >> 4;
@@ -65,12 +67,27 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
                 load_a<1>(a[j], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             }
         }
-        if (base == 0 && p.sh_w) {  // the shared expert's gate while the tiles travel (moe_combine_kernel's order)
-            float gate = 1.0f;
+        if (base == 0 && tid < p.top_k) {  // the token's experts and routing weights for the combine, fetched once
+            ids_sh[tid] = p.ids[t * p.top_k + tid];
+            wts_sh[tid] = p.weights[t * p.top_k + tid];
+        }
+        if (base == 0 && p.sh_w) {  // the shared expert's gate while the tiles travel (moe_combine_kernel's order:
+            float gate = 1.0f;      // thread j takes columns j, j + 256, ... in turn)
             if (p.sh_gate_inp) {
                 if (tid < 256) {
+                    // the operands are requested eight columns at a time so that their latencies overlap
+                    const float* gi = p.sh_gate_inp;
+                    const float* xr = p.x + t * p.rows;
                     float acc = 0.0f;
-                    for (int64_t c = tid; c < p.rows; c += 256) acc = fmaf(p.sh_gate_inp[c], p.x[t * p.rows + c], acc);
+                    int64_t c = tid;
+                    for (; c + 7 * 256 < p.rows; c += 8 * 256) {
+                        float ga[8], xa[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) ga[u] = gi[c + u * 256], xa[u] = xr[c + u * 256];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) acc = fmaf(ga[u], xa[u], acc);
+                    }
+                    for (; c < p.rows; c += 256) acc = fmaf(gi[c], xr[c], acc);
 #pragma unroll
                     for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
                     if ((tid & 63) == 0) wave_sum[tid >> 6] = acc;
@@ -106,8 +123,8 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
             float part = __fadd_rn(0.0f, term[(k * nb) * 16 + tid]);
             for (int b = 1; b < nb; ++b) part = __fadd_rn(part, term[(k * nb + b) * 16 + tid]);
             if (k < p.top_k) {
-                const int e = p.ids[t * p.top_k + k];
-                const float w = p.weights[t * p.top_k + k];
+                const int e = ids_sh[k];
+                const float w = wts_sh[k];
                 if (e < 0 || e >= p.n_experts || w == 0.0f) continue;
                 acc = __fadd_rn(acc, __fmul_rn(part, w));
             } else {
