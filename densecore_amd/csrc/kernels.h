@@ -146,6 +146,29 @@ struct MoeDownTokenArgs {
 };
 hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream);
 
+// ---- moe_gateup.hip --------------------------------------------------------------------------
+// Gate/up + SwiGLU with the router and the Q8_K of the layer input inside, one workgroup per (token, slot,
+// 16 hidden rows): decode widths, where neither grouping by expert nor separate routing / quantizing launches pay.
+struct MoeGateupTokenArgs {
+    const uint8_t* gate = nullptr;     // tiled experts [n_experts][rows x nb]
+    const uint8_t* up = nullptr;
+    size_t expert_bytes = 0;
+    const uint8_t* sh_gate = nullptr;  // shared expert (both or neither); its hidden row is slot top_k
+    const uint8_t* sh_up = nullptr;
+    int wtype = 12;
+    int64_t rows = 0, nb = 0;          // hidden rows per expert (inter), super-blocks per row (hidden / 256)
+    int64_t n = 0;
+    int top_k = 0, n_experts = 0;      // n_experts <= 512
+    int route_mode = 0, silu_mode = 0, sh_silu_mode = 2;
+    int waves = 1;                     // wavefronts per workgroup: pick_waves(nb, row tiles x n x slots)
+    const float* x = nullptr;          // [n][nb * 256]
+    const float* logits = nullptr;     // [n][n_experts]
+    float* hidden = nullptr;           // [n * slots][rows]
+    int32_t* ids_out = nullptr;        // [n][top_k]
+    float* weights_out = nullptr;      // [n][top_k]
+};
+hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stream);
+
 // ---- decoder_layers.hip ----------------------------------------------------------------------
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,
 // device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.

@@ -1,0 +1,147 @@
+// MoE gate/up + SwiGLU for decode widths with the router and the input quantizer inside, token-major.
+//
+// With few tokens nearly every (token, slot) pair has an expert of its own, so nothing is gained by grouping the
+// pairs by expert -- and the two launches that only prepare the expert-grouped product (routing, Q8_K of the
+// layer input) cost as much as the product.  Here a workgroup owns one (token, slot, 16-row tile) of the hidden
+// rows and does everything it needs itself:
+//   * its first wavefront routes the token (stable top-k over the logits in one wavefront, route_block.h;
+//     ComputeQwenNativeMoEStableTopK, core/src/llm/moe/native.cpp:610-676) -- every workgroup of the token repeats
+//     that, a few hundred instructions -- and one workgroup per token also forms the routing weights and writes
+//     ids and weights out for the down projection (cb_moe_topk_weights_from_logits, :800-868);
+//   * every wavefront quantizes the super-blocks of x it multiplies (the block quantizer of quantize_q8k_kernel)
+//     while its weight tiles travel;
+//   * hidden[t][k][r] = silu(gate_e[r] . q8k(x_t)) * (up_e[r] . q8k(x_t)), e = ids[t][k]
+//     (RunQwen35NativeMoEGateUpRawQXKSwiGLU, core/src/llm/moe/native.cpp:3929-4345); the shared expert is slot
+//     top_k of every token.
+// Per-tile arithmetic, the wave split of K and the reduction order are those of matmul_kernel<2,1>: the same bits
+// as routing + quantize + the expert-grouped launch.
+#include "common.h"
+#include "kernels.h"
+#include "decode_tile.h"
+#include "q8k_block.h"
+#include "route_block.h"
+
+namespace mq {
+
+namespace {
+
+constexpr int kStages = 3;  // register stages of a wavefront: a stage is one super-block of x and its two weight tiles
+
+template <int WT>
+__global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTokenArgs p) {
+    constexpr int kTileStride = tile_stride<WT>();
+    extern __shared__ float red[];  // [W-1][2][64]
+    __shared__ int ids_sh[8];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rt = blockIdx.x;
+    const int slots = p.top_k + (p.sh_gate ? 1 : 0);
+    const int tok = blockIdx.y / slots, sl = blockIdx.y - tok * slots;
+    const bool shared = sl >= p.top_k;
+    const int nb = (int)p.nb;
+    const int cnt = wave < nb ? (nb - wave + n_waves - 1) / n_waves : 0;  // super-blocks wave, wave + W, ... of this wavefront
+    const float* xrow = p.x + (size_t)tok * (size_t)nb * kQK + lane * 4;
+
+    // Ring of kStages register stages; the activations are requested first, they do not wait for the routing.
+    typename TileOf<WT>::Regs ring_t[kStages][2];
+    float4 ring_x[kStages];
+    auto issue_x = [&](int st, int i) {
+        const int b = i < cnt ? wave + i * n_waves : 0;  // a stage past the end re-reads block 0: the load count stays fixed
+        ring_x[st] = *reinterpret_cast<const float4*>(xrow + (size_t)b * kQK);
+    };
+#pragma unroll
+    for (int st = 0; st < kStages - 1; ++st) issue_x(st, st);
+
+    // ---- routing (every workgroup of a routed slot; the shared expert needs none) ----
+    int expert = 0;
+    if (!shared) {
+        if (wave == 0) {
+            const float* row = p.logits + (size_t)tok * p.n_experts;
+            auto load = [&](int e) { return row[e]; };
+            int id;
+            float logit;
+            if (p.n_experts <= 256) route_token_wave<4>(load, p.n_experts, p.top_k, lane, id, logit);
+            else route_token_wave<8>(load, p.n_experts, p.top_k, lane, id, logit);
+            if (lane < p.top_k) ids_sh[lane] = id;
+            if (rt == 0 && sl == 0) {  // one workgroup per token hands ids and weights to the down projection
+                const float w = route_weight_lane(logit, lane, p.top_k, p.route_mode);
+                if (lane < p.top_k) {
+                    p.ids_out[(size_t)tok * p.top_k + lane] = id;
+                    p.weights_out[(size_t)tok * p.top_k + lane] = w;
+                }
+            }
+        }
+        __syncthreads();
+        expert = ids_sh[sl];
+        if (expert < 0 || expert >= p.n_experts) return;  // dropped slot: the whole workgroup leaves, its row is never read
+    }
+    const uint8_t* tiles[2] = {(shared ? p.sh_gate : p.gate + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride),
+                               (shared ? p.sh_up : p.up + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride)};
+    auto issue_t = [&](int st, int i) {
+        const int b = i < cnt ? wave + i * n_waves : 0;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)b * kTileStride, lane);
+    };
+#pragma unroll
+    for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
+
+    float acc[2][1][2] = {{{0.0f, 0.0f}}, {{0.0f, 0.0f}}};
+    for (int base = 0; base < cnt; base += kStages) {
+#pragma unroll
+        for (int st = 0; st < kStages; ++st) {
+            const int i = base + st;
+            issue_t((st + kStages - 1) % kStages, i + kStages - 1);
+            issue_x((st + kStages - 1) % kStages, i + kStages - 1);
+            if (i < cnt) {
+                const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
+                ARegs<1> a;
+                a_from_lane_codes(a, quantize_block_q8k(e, lane), lane);  // the token is row 0 of the operand
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    int32_t dsum[1][2], msum[1][2];
+                    compute_tile_wt<1, WT>(ring_t[st][m], a, acc[m], dsum, msum, lane);
+                }
+            }
+        }
+    }
+
+    // ---- partial sums meet in wave order (as in matmul_kernel), SwiGLU, one store per weight row ----
+    if (n_waves > 1) {
+        if (wave > 0) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m) red[((wave - 1) * 2 + m) * 64 + lane] = acc[m][0][0];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+        for (int wv = 1; wv < n_waves; ++wv) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m) acc[m][0][0] = __fadd_rn(acc[m][0][0], red[((wv - 1) * 2 + m) * 64 + lane]);
+        }
+        const int64_t row = rt * 16 + slot;
+        if (kq == 0 && row < p.rows)
+            p.hidden[((size_t)tok * slots + sl) * (size_t)p.rows + row] =
+                silu_mul(acc[0][0][0], acc[1][0][0], shared ? p.sh_silu_mode : p.silu_mode);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stream) {
+    if (a.n <= 0 || a.rows <= 0 || a.nb <= 0 || a.top_k <= 0 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > 512 ||
+        a.waves < 1 || a.waves > 8 || (a.nb % a.waves) || !a.gate || !a.up || !a.x || !a.logits || !a.hidden || !a.ids_out ||
+        !a.weights_out || (a.sh_gate == nullptr) != (a.sh_up == nullptr))
+        return hipErrorInvalidValue;
+    const int slots = a.top_k + (a.sh_gate ? 1 : 0);
+    const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)(a.n * slots));
+    const size_t lds = a.waves > 1 ? (size_t)(a.waves - 1) * 2 * 64 * sizeof(float) : 0;
+    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ6>, grid, dim3(64 * a.waves), lds, stream, a);
+    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ5>, grid, dim3(64 * a.waves), lds, stream, a);
+    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ4>, grid, dim3(64 * a.waves), lds, stream, a);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+}  // namespace mq
