@@ -591,6 +591,24 @@ int mq_router_logits_f32(const float* w_dev, int64_t n_experts, int64_t cols, co
     return MQ_OK;
 }
 
+int mq_add_rmsnorm_router_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                              float eps, float* sum_out_dev, float* normed_out_dev, const float* router_dev, int64_t n_experts,
+                              float* logits_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (n == 0) return MQ_OK;
+    if (!x_dev || !router_dev || !logits_dev || n < 0 || n > 65535 || n_experts <= 0 || cols <= 0)
+        return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_router_f32: bad arguments");
+    if ((cols & 255) || cols > 4096) return fail(MQ_ERR_UNSUPPORTED, "mq_add_rmsnorm_router_f32: cols %lld (a multiple of 256 up to 4096)", (long long)cols);
+    if (sum_out_dev && (sum_out_dev == x_dev || sum_out_dev == delta_dev))
+        return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_router_f32: the sum must not overwrite x or delta (every workgroup of a row reads them)");
+    if ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(delta_dev) | reinterpret_cast<uintptr_t>(weight_dev) |
+         reinterpret_cast<uintptr_t>(sum_out_dev) | reinterpret_cast<uintptr_t>(normed_out_dev) | reinterpret_cast<uintptr_t>(router_dev)) & 15u)
+        return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_router_f32: rows must be 16-byte aligned");
+    MQ_HIP(launch_add_rmsnorm_router(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, router_dev, n_experts,
+                                     logits_dev, (hipStream_t)stream));
+    return MQ_OK;
+}
+
 int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev, int top_k,
                                float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;

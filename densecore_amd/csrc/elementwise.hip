@@ -164,7 +164,99 @@ __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restr
     if (lane == 0) logits[t * n_experts + e] = acc;
 }
 
+// Residual add + RMSNorm + router projection in one launch: workgroup (g, t) normalises row t itself (the
+// arithmetic and the summation order of add_rmsnorm_blocks_kernel, repeated by every workgroup of the row: 8 KB
+// of loads), parks the normalised row in LDS and its four wavefronts form the logits of the experts 4g .. 4g+3
+// (router_logits_kernel's order); workgroup g = 0 also writes the sum and the normalised row out.  Same bits as
+// the two launches.  sum_out must not be x or delta: other workgroups still read them.
+__global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __restrict__ x, const float* __restrict__ delta,
+                                                                 const float* __restrict__ weight, int64_t cols, float eps,
+                                                                 float* __restrict__ sum_out, float* __restrict__ normed_out,
+                                                                 const float* __restrict__ w_router, int64_t n_experts,
+                                                                 float* __restrict__ logits) {
+    extern __shared__ __attribute__((aligned(16))) float row_sh[];  // [cols]
+    __shared__ float wave_sum[4];
+    constexpr int kKeep = 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t t = blockIdx.y, base = t * cols, nb = cols / kQK;
+    const bool writer = blockIdx.x == 0;
+    float4 kept[kKeep];
+    float ssq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+        const int64_t b = wave + 4 * i;
+        if (b < nb) {
+            const int64_t c0 = b * kQK + lane * 4;
+            float4 a = *reinterpret_cast<const float4*>(x + base + c0);
+            if (delta) {
+                const float4 d = *reinterpret_cast<const float4*>(delta + base + c0);
+                a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
+            }
+            if (writer && sum_out) *reinterpret_cast<float4*>(sum_out + base + c0) = a;
+            ssq = __fmaf_rn(a.x, a.x, ssq);
+            ssq = __fmaf_rn(a.y, a.y, ssq);
+            ssq = __fmaf_rn(a.z, a.z, ssq);
+            ssq = __fmaf_rn(a.w, a.w, ssq);
+            kept[i] = a;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+    if (lane == 0) wave_sum[wave] = ssq;
+    __syncthreads();
+    const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+    const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+        const int64_t b = wave + 4 * i;
+        if (b < nb) {
+            const int64_t c0 = b * kQK + lane * 4;
+            const float4 a = kept[i];
+            float4 w = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+            if (weight) w = *reinterpret_cast<const float4*>(weight + c0);
+            const float4 e = make_float4(__fmul_rn(a.x, weight ? __fmul_rn(scale, w.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, w.y) : scale),
+                                         __fmul_rn(a.z, weight ? __fmul_rn(scale, w.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, w.w) : scale));
+            *reinterpret_cast<float4*>(row_sh + c0) = e;
+            if (writer && normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = e;
+        }
+    }
+    __syncthreads();
+    const int64_t ex = (int64_t)blockIdx.x * 4 + wave;
+    if (ex >= n_experts) return;
+    const float* wr = w_router + ex * cols;
+    float acc = 0.0f;
+    auto add4 = [&](const float4& a, const float4& b) {
+        acc = __fmaf_rn(a.x, b.x, acc);
+        acc = __fmaf_rn(a.y, b.y, acc);
+        acc = __fmaf_rn(a.z, b.z, acc);
+        acc = __fmaf_rn(a.w, b.w, acc);
+    };
+    int64_t c = (int64_t)lane * 4;
+    for (; c + 7 * 256 + 3 < cols; c += 8 * 256) {
+        float4 a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = *reinterpret_cast<const float4*>(wr + c + u * 256);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) add4(a[u], *reinterpret_cast<const float4*>(row_sh + c + u * 256));
+    }
+    for (; c + 3 < cols; c += 256) add4(*reinterpret_cast<const float4*>(wr + c), *reinterpret_cast<const float4*>(row_sh + c));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) logits[t * n_experts + ex] = acc;
+}
+
 }  // namespace
+
+hipError_t launch_add_rmsnorm_router(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols, float eps,
+                                     float* sum_out, float* normed_out, const float* w_router, int64_t n_experts, float* logits,
+                                     hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    if ((cols % kQK) || cols > 4 * 4 * kQK || n > 65535 || n_experts <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(add_rmsnorm_router_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256),
+                       (size_t)cols * sizeof(float), stream, x, delta, weight, cols, eps, sum_out, normed_out, w_router, n_experts,
+                       logits);
+    return hipGetLastError();
+}
 
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
                               float eps, float* sum_out, float* normed_out, uint8_t* q_aq, float* q_ad,

@@ -100,6 +100,10 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,
                               float eps, float* sum_out, float* normed_out, uint8_t* q_aq, float* q_ad,
                               hipStream_t stream);
+// Residual add + RMSNorm + router projection in one launch (cols % 256 == 0, cols <= 4096; sum_out apart from x and delta).
+hipError_t launch_add_rmsnorm_router(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols, float eps,
+                                     float* sum_out, float* normed_out, const float* w_router, int64_t n_experts, float* logits,
+                                     hipStream_t stream);
 hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols, const float* x, int64_t n, int64_t ldx,
                                 float* logits, hipStream_t stream);
 

@@ -5,8 +5,8 @@
     qkv = W_qkv . h                                    mq_mul_mat_q4k_acts (wq, wk, wv stacked row-wise)
     o   = W_o . q8k(qkv[:, :n_q])                      mq_mul_mat_q4k     (the attention core itself is not on
                                                                            this path: q stands in for its output)
-    x   = x + o ; h2 = rmsnorm(x)                      mq_add_rmsnorm_f32
-    logits = W_router . h2                             mq_router_logits_f32
+    x   = x + o ; h2 = rmsnorm(x)                      mq_add_rmsnorm_router_f32 (one launch; mq_add_rmsnorm_f32 +
+    logits = W_router . h2                                                        mq_router_logits_f32 for hidden > 4096)
     y   = moe_layer(h2, logits) (+ shared expert)      mq_moe_layer_q4k
     x   = x + y                                        (fused into the next layer's first call)
 
@@ -90,6 +90,7 @@ class DecodeStep:
         f = lambda *shape: torch.empty(shape, dtype=torch.float32, device="cuda")
         H = cfg.hidden
         self.x, self.h, self.o, self.y = f(n_tokens, H), f(n_tokens, H), f(n_tokens, H), f(n_tokens, H)
+        self.x_alt = f(n_tokens, H)
         self.qkv = f(n_tokens, cfg.n_q + 2 * cfg.n_kv)
         self.logits = f(n_tokens, cfg.n_experts)
         self.ids = torch.empty((cfg.n_layers, n_tokens, cfg.top_k), dtype=torch.int32, device="cuda")
@@ -118,23 +119,32 @@ class DecodeStep:
         p = lambda t: C.c_void_p(t.data_ptr())
         chk = _lib.check
         delta = None
+        x, x_next = self.x, self.x_alt   # the residual stream alternates between two buffers (see below)
+        fused_router = cfg.hidden % 256 == 0 and cfg.hidden <= 4096
         for i, ly in enumerate(self.layers):
             ly.desc.silu_mode = self.silu_mode()
-            chk(L.mq_add_rmsnorm_q8k(p(self.x), p(delta) if delta is not None else None, None, n, cfg.hidden,
-                                     C.c_float(cfg.eps), p(self.x), None, C.c_void_p(self.h_q8._h), st),
+            chk(L.mq_add_rmsnorm_q8k(p(x), p(delta) if delta is not None else None, None, n, cfg.hidden,
+                                     C.c_float(cfg.eps), p(x), None, C.c_void_p(self.h_q8._h), st),
                 "mq_add_rmsnorm_q8k")
             chk(L.mq_mul_mat_q4k_acts(ly.wqkv._h, C.c_void_p(self.h_q8._h), p(self.qkv), self.qkv.shape[1], st), "qkv")
             chk(L.mq_mul_mat_q4k(ly.wo._h, p(self.qkv), n, self.qkv.shape[1], p(self.o), cfg.hidden, st), "wo")
-            chk(L.mq_add_rmsnorm_f32(p(self.x), p(self.o), None, n, cfg.hidden, C.c_float(cfg.eps), p(self.x),
-                                     p(self.h), st), "mq_add_rmsnorm_f32")
-            chk(L.mq_router_logits_f32(p(ly.router), cfg.n_experts, cfg.hidden, p(self.h), n, cfg.hidden,
-                                       p(self.logits), st), "mq_router_logits_f32")
+            if fused_router:
+                # residual add, norm and router projection in one launch; its sum goes to the other buffer because
+                # every workgroup of a row reads x while one of them writes the sum
+                chk(L.mq_add_rmsnorm_router_f32(p(x), p(self.o), None, n, cfg.hidden, C.c_float(cfg.eps), p(x_next), p(self.h),
+                                                p(ly.router), cfg.n_experts, p(self.logits), st), "mq_add_rmsnorm_router_f32")
+                x, x_next = x_next, x
+            else:
+                chk(L.mq_add_rmsnorm_f32(p(x), p(self.o), None, n, cfg.hidden, C.c_float(cfg.eps), p(x), p(self.h), st),
+                    "mq_add_rmsnorm_f32")
+                chk(L.mq_router_logits_f32(p(ly.router), cfg.n_experts, cfg.hidden, p(self.h), n, cfg.hidden,
+                                           p(self.logits), st), "mq_router_logits_f32")
             lg = self.fixed_logits[i] if self.fixed_logits is not None else self.logits
             chk(L.mq_moe_layer_q4k(C.byref(ly.desc), p(self.h), p(lg), n, p(self.y), p(self.ids[i]),
                                    p(self.wts[i]), st), "mq_moe_layer_q4k")
             delta = self.y
         # final residual add; the normalised copy lands in self.h and is not used
-        chk(L.mq_add_rmsnorm_f32(p(self.x), p(delta), None, n, cfg.hidden, C.c_float(cfg.eps), p(self.out), p(self.h),
+        chk(L.mq_add_rmsnorm_f32(p(x), p(delta), None, n, cfg.hidden, C.c_float(cfg.eps), p(self.out), p(self.h),
                                  st), "mq_add_rmsnorm_f32")
 
     def capture(self) -> None:

@@ -278,6 +278,12 @@ int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* 
  * [n_experts][cols], x_dev fp32 [n][ldx], logits_dev fp32 [n][n_experts]; cols % 256 == 0. */
 int mq_router_logits_f32(const float* w_dev, int64_t n_experts, int64_t cols, const float* x_dev, int64_t n,
                          int64_t ldx, float* logits_dev, void* stream);
+/* mq_add_rmsnorm_f32 followed by mq_router_logits_f32 on its normalised rows, in one launch and with the same
+ * bits: sum = x + delta, normed = rmsnorm(sum) * weight, logits[t][e] = router[e] . normed[t].  cols a multiple
+ * of 256 up to 4096; sum_out_dev (may be NULL, as normed_out_dev) must be neither x_dev nor delta_dev. */
+int mq_add_rmsnorm_router_f32(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
+                              float eps, float* sum_out_dev, float* normed_out_dev, const float* router_dev, int64_t n_experts,
+                              float* logits_dev, void* stream);
 
 /* ---- verification hook -------------------------------------------------------------
  * Runs the production matmul kernel with its per-super-block integer sums

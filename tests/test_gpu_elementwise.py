@@ -76,3 +76,33 @@ def test_add_rmsnorm_q8k_equals_norm_then_quantize(n, cols):
                                              C.c_void_p(acts._h), None), "q8k in place")
     assert torch.equal(x2, ref_sum) and torch.equal(acts.mul_mat(w), ops.mul_mat(w, ref_h))
     acts.free(), w.free()
+
+
+@pytest.mark.parametrize("n,cols,n_experts,with_delta,with_weight", [(1, 2048, 256, True, False), (4, 2048, 256, True, True),
+                                                                      (3, 512, 10, False, True), (8, 4096, 64, True, False)])
+def test_add_rmsnorm_router_equals_the_two_launches(n, cols, n_experts, with_delta, with_weight):
+    """mq_add_rmsnorm_router_f32: the bits of mq_add_rmsnorm_f32 followed by mq_router_logits_f32."""
+    import torch
+    from densecore_amd import _lib
+    g = torch.Generator(device="cuda").manual_seed(n * 1000 + cols)
+    x = torch.randn((n, cols), device="cuda", generator=g)
+    d = torch.randn((n, cols), device="cuda", generator=g) if with_delta else None
+    w = (torch.rand((cols,), device="cuda", generator=g) + 0.5) if with_weight else None
+    router = torch.randn((n_experts, cols), device="cuda", generator=g) * 0.05
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    L = _lib.lib()
+    ref_sum, ref_h = torch.empty_like(x), torch.empty_like(x)
+    ref_lg = torch.empty((n, n_experts), device="cuda")
+    _lib.check(L.mq_add_rmsnorm_f32(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(ref_sum), p(ref_h), None), "norm")
+    _lib.check(L.mq_router_logits_f32(p(router), n_experts, cols, p(ref_h), n, cols, p(ref_lg), None), "router")
+    got_sum, got_h = torch.empty_like(x), torch.empty_like(x)
+    got_lg = torch.empty((n, n_experts), device="cuda")
+    _lib.check(L.mq_add_rmsnorm_router_f32(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(got_sum), p(got_h), p(router),
+                                           n_experts, p(got_lg), None), "fused")
+    torch.cuda.synchronize()
+    assert torch.equal(got_sum, ref_sum) and torch.equal(got_h, ref_h)
+    assert torch.equal(got_lg, ref_lg), f"max |diff| {(got_lg - ref_lg).abs().max().item():.3e}"
+    # the sum may not overwrite an input: every workgroup of a row reads x and delta
+    with pytest.raises(_lib.MqError):
+        _lib.check(L.mq_add_rmsnorm_router_f32(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(x), p(got_h), p(router),
+                                               n_experts, p(got_lg), None), "fused in place")
