@@ -731,11 +731,6 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
     return MQ_OK;
 }
 
-// Wavefronts per workgroup of the token-major gate/up launch (moe_gateup.hip): one workgroup per (token, slot, row tile).
-int moe_gateup_token_waves(int64_t nb, int64_t inter, int64_t n, int slots) {
-    return pick_waves(nb, ((inter + 15) / 16) * n * slots);
-}
-
 // Does the down projection of this MoE block run token-major (moe_down.hip)?
 bool token_major_down(const mq_weight* down, int64_t n, int slots) {
     return n <= kTokenMajorDownMaxTokens && !census.on && (down->rows & 15) == 0 &&
@@ -1051,7 +1046,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         a.rows = inter, a.nb = L->gate_exps->nb, a.n = n;
         a.top_k = K, a.n_experts = (int)E;
         a.route_mode = L->route_mode, a.silu_mode = L->silu_mode, a.sh_silu_mode = MQ_SILU_FAST_FMA;
-        a.waves = moe_gateup_token_waves(L->gate_exps->nb, inter, n, slots);
+        a.waves = moe_gateup_token_waves(L->gate_exps->nb, inter, n, slots, L->gate_exps->type);
         a.x = x_dev, a.logits = logits_dev, a.hidden = (float*)g.mid.ptr, a.ids_out = ids, a.weights_out = wts;
         MQ_HIP(launch_moe_gateup_token(a, s));
         return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, false, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
@@ -1218,7 +1213,7 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
         // groups above, plus one pass of the shared expert; the kernel keeps that launch's summation order
         const int64_t pairs = n * (int64_t)d->top_k;
         const int64_t groups = (pairs < d->n_experts ? pairs : d->n_experts) + (d->has_shared ? (n + 7) / 8 : 0);
-        a.gateup_order = n <= kDirectPairsMaxTokens ? moe_gateup_token_waves(d->hidden / kQK, d->inter, n, d->top_k + d->has_shared)
+        a.gateup_order = n <= kDirectPairsMaxTokens ? moe_gateup_token_waves(d->hidden / kQK, d->inter, n, d->top_k + d->has_shared, kTypeQ4K)
                                                     : pick_waves(d->hidden / kQK, (int64_t)(d->inter / 16) * groups);
     }
     a.eps = d->eps;

@@ -164,7 +164,7 @@ struct MoeGateupTokenArgs {
     int64_t n = 0;
     int top_k = 0, n_experts = 0;      // n_experts <= 512
     int route_mode = 0, silu_mode = 0, sh_silu_mode = 2;
-    int waves = 1;                     // wavefronts per workgroup: pick_waves(nb, row tiles x n x slots)
+    int waves = 1;                     // wavefronts per workgroup: moe_gateup_token_waves()
     const float* x = nullptr;          // [n][nb * 256]
     const float* logits = nullptr;     // [n][n_experts]
     float* hidden = nullptr;           // [n * slots][rows]
@@ -172,6 +172,9 @@ struct MoeGateupTokenArgs {
     float* weights_out = nullptr;      // [n][top_k]
 };
 hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stream);
+// Wavefronts per workgroup for that launch (rows = hidden rows per expert), and the wavefronts the chip holds of it.
+int moe_gateup_token_waves(int64_t nb, int64_t rows, int64_t n, int slots, int wtype);
+int moe_gateup_token_capacity(int wtype);
 
 // ---- decoder_layers.hip ----------------------------------------------------------------------
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,

@@ -329,19 +329,14 @@ hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t str
 
 }  // namespace
 
-// Waves per workgroup: the chip holds 2 waves per SIMD of this kernel (2048 in all); aim at filling
-// that once and never overfilling it -- a launch a few wavefronts over the limit waits for a second round of
-// workgroups that start when the first ones end -- with a count that divides the super-blocks of a row evenly
-// and at most 8.
+// Waves per workgroup: a compute unit holds 8 wavefronts of this kernel (2 per SIMD) and whole workgroups only;
+// aim at having every workgroup of the launch resident at once -- a launch a few workgroups over that waits for
+// a second round that starts when the first ones end -- with a count that divides the super-blocks of a row
+// evenly and at most 8.
 int pick_waves(int64_t nb, int64_t workgroups) {
-    const int64_t target = 2048;
-    int64_t ideal = target / (workgroups > 0 ? workgroups : 1);
-    if (ideal < 1) ideal = 1;
-    if (ideal > 8) ideal = 8;
-    if (ideal > nb) ideal = nb;
-    for (int64_t w = ideal; w >= 1; --w) {
-        if (nb % w == 0) return (int)w;
-    }
+    const int64_t compute_units = 256;
+    for (int64_t w = nb < 8 ? nb : 8; w > 1; --w)
+        if (nb % w == 0 && workgroups <= compute_units * (8 / w)) return (int)w;
     return 1;
 }
 

@@ -129,6 +129,39 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
 
 }  // namespace
 
+// Wavefronts of this kernel that ONE compute unit holds at once: by the registers the compiled kernel takes (512 per
+// SIMD lane, handed out in blocks of 8), four SIMDs per compute unit.
+int moe_gateup_token_capacity(int wtype) {
+    static int cached[3] = {0, 0, 0};
+    const int k = wtype == kTypeQ6K ? 2 : wtype == kTypeQ5K ? 1 : 0;
+    if (!cached[k]) {
+        const void* fn = wtype == kTypeQ6K   ? reinterpret_cast<const void*>(moe_gateup_token_kernel<kWtQ6>)
+                         : wtype == kTypeQ5K ? reinterpret_cast<const void*>(moe_gateup_token_kernel<kWtQ5>)
+                                             : reinterpret_cast<const void*>(moe_gateup_token_kernel<kWtQ4>);
+        hipFuncAttributes attr;
+        int per_simd = 2;
+        if (hipFuncGetAttributes(&attr, fn) == hipSuccess && attr.numRegs > 0) {
+            per_simd = 512 / ((attr.numRegs + 7) / 8 * 8);
+            per_simd = per_simd < 1 ? 1 : per_simd > 8 ? 8 : per_simd;
+        }
+        cached[k] = per_simd * 4;
+    }
+    return cached[k];
+}
+
+// Wavefronts per workgroup: as many as divide the super-blocks of a row evenly (at most 8) while all workgroups of
+// the launch are resident at once -- a compute unit holds whole workgroups only.
+int moe_gateup_token_waves(int64_t nb, int64_t rows, int64_t n, int slots, int wtype) {
+    const int64_t workgroups = ((rows + 15) / 16) * n * slots;
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+        cus = 256;
+    const int per_cu = moe_gateup_token_capacity(wtype);
+    for (int64_t w = nb < 8 ? nb : 8; w > 1; --w)
+        if (nb % w == 0 && workgroups <= (int64_t)cus * (per_cu / w)) return (int)w;
+    return 1;
+}
+
 hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stream) {
     if (a.n <= 0 || a.rows <= 0 || a.nb <= 0 || a.top_k <= 0 || a.top_k > 8 || a.n_experts < a.top_k || a.n_experts > 512 ||
         a.waves < 1 || a.waves > 8 || (a.nb % a.waves) || !a.gate || !a.up || !a.x || !a.logits || !a.hidden || !a.ids_out ||
