@@ -1209,7 +1209,7 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
     a.silu_mode = silu_mode >= 0 ? silu_mode : (n <= 4 ? MQ_SILU_EXACT : MQ_SILU_FAST);
     a.route_mode = d->route_mode;
     {
-        // the expert gate/up launch of mq_moe_layer_q4k at this width: (token, slot) pairs up to four tokens, expert
+        // the expert gate/up launch of mq_moe_layer_q4k at this width: (token, slot) pairs up to eight tokens, expert
         // groups above, plus one pass of the shared expert; the kernel keeps that launch's summation order
         const int64_t pairs = n * (int64_t)d->top_k;
         const int64_t groups = (pairs < d->n_experts ? pairs : d->n_experts) + (d->has_shared ? (n + 7) / 8 : 0);

@@ -180,8 +180,8 @@ int moe_gateup_token_capacity(int wtype);
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,
 // device-wide barriers between the phases of a layer).  All weights are Q4_K in the tiled layout.
 constexpr int kDecoderMaxExperts = 512;
-constexpr int kTokenMajorDownMaxTokens = 4;  // widest MoE block whose down projection runs token-major (measured: 8 and 16 lose)
-constexpr int kDirectPairsMaxTokens = 4;  // widest MoE block whose (token, slot) pairs are not grouped by expert
+constexpr int kTokenMajorDownMaxTokens = 8;  // widest MoE block whose down projection runs token-major (measured: 16 loses)
+constexpr int kDirectPairsMaxTokens = 8;  // widest MoE block whose (token, slot) pairs are not grouped by expert (measured: 16 loses)
 struct DecoderLayerDev {               // one per layer, in device memory
     const uint8_t* wqkv = nullptr;     // [qkv_rows x hidden]
     const uint8_t* wo = nullptr;       // [hidden x n_q]; its input is qkv[:, :n_q]

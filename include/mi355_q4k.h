@@ -201,7 +201,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  *   route top_k -> gate/up + SwiGLU per (token, k) -> Q8_K -> down ->
  *   y[t] = sum_k w[t][k] * down_k (k in routing order) + sigmoid(sh_gate_inp . x[t]) * shared_ffn(x[t]).
  * shared_* may all be NULL (no shared expert); sh_gate_inp_dev fp32 [hidden] or NULL (gate = 1).
- * Up to four tokens (and 512 experts) two launches: gate/up + SwiGLU with the router and the Q8_K of x inside,
+ * Up to eight tokens (and 512 experts) two launches: gate/up + SwiGLU with the router and the Q8_K of x inside,
  * down with the Q8_K of the hidden rows and the weighted combine inside.  Above: router + expert grouping + Q8_K
  * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way. */
 typedef struct {
