@@ -406,6 +406,34 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }
 
+int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n,
+                           float eps, float* sum_out_dev, float* y_dev, int64_t ldy, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_rmsnorm_mul_mat_q4k")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: weight is an expert stack");
+    if (int rc = check_x(x_dev, n, w->cols, w->cols, "mq_rmsnorm_mul_mat_q4k")) return rc;
+    if (n == 0) return MQ_OK;
+    if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: null output or ldy < rows");
+    if (sum_out_dev && (sum_out_dev == x_dev || sum_out_dev == delta_dev))
+        return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: the sum must not overwrite x or delta (every workgroup reads them)");
+    if ((reinterpret_cast<uintptr_t>(delta_dev) | reinterpret_cast<uintptr_t>(weight_dev) | reinterpret_cast<uintptr_t>(sum_out_dev)) & 15u)
+        return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: rows must be 16-byte aligned");
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    if (n == 1 && !census.on && w->type == kTypeQ4K) {  // one row, short K per wave: norm and quantizer run inside the GEMV kernel
+        const int waves = pick_waves(w->nb, w->rowtiles);
+        if (gemv1_fused_applies(w->nb, waves)) {
+            MQ_HIP(launch_gemv1_norm_fused(w->data, w->rows, w->nb, x_dev, delta_dev, weight_dev, eps, sum_out_dev, y_dev, waves, s));
+            return MQ_OK;
+        }
+    }
+    const int64_t nb = w->cols / kQK;
+    MQ_HIP(g.aq.reserve(aq_bytes(n, nb)));
+    MQ_HIP(g.ad.reserve(ad_count(n, nb) * sizeof(float)));
+    MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, w->cols, eps, sum_out_dev, nullptr, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
+    return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
+}
+
 int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t q8_row_bytes, float* y_dev,
                        int64_t ldy, void* stream) {
     if (int rc = check_ready()) return rc;

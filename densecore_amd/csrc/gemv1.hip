@@ -73,7 +73,101 @@ __global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restr
     }
 }
 
+// The same GEMV with the residual add and the RMSNorm of its input inside as well (one row):
+//     s = x + delta;  h = s * (weight / sqrt(mean(s^2) + eps));  y[r] = W[r] . q8k(h)
+// The first four wavefronts of every workgroup sum the squares of the row exactly as add_rmsnorm_blocks_kernel does
+// (wavefront v takes the super-blocks v, v + 4, ..., lane l their elements 4l .. 4l+3; butterfly; (w0 + w1) +
+// (w2 + w3)) while the weight tiles travel -- 8 KB of loads repeated per workgroup -- then every wavefront
+// normalises and quantizes the super-blocks it multiplies.  Workgroup 0 also writes s out (sum_out must not be x or
+// delta: the other workgroups still read them).  Same bits as mq_add_rmsnorm_q8k followed by the product.
+__global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __restrict__ w, int64_t rows, int64_t nb,
+                                                               const float* __restrict__ x, const float* __restrict__ delta,
+                                                               const float* __restrict__ weight, float eps,
+                                                               float* __restrict__ sum_out, float* __restrict__ y) {
+    extern __shared__ float red[];  // [W-1][64]
+    __shared__ float wave_sum[4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rt = blockIdx.x;
+    const uint8_t* tiles = w + tile_offset(rt, 0, nb);
+    const int cnt = wave < nb ? (int)((nb - wave + n_waves - 1) / n_waves) : 0;  // <= kMaxStages (host-checked)
+    auto fetch = [&](int64_t c0) {
+        float4 a = *reinterpret_cast<const float4*>(x + c0);
+        if (delta) {
+            const float4 d = *reinterpret_cast<const float4*>(delta + c0);
+            a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
+        }
+        return a;
+    };
+
+    TileRegs t[kMaxStages];
+    float4 xv[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        const int b = i < cnt ? wave + i * n_waves : 0;
+        load_tile(t[i], tiles + (size_t)b * kTileBytes, lane);
+        xv[i] = fetch((int64_t)b * kQK + lane * 4);
+    }
+    // sum of squares in the order of the 256-thread norm kernel: virtual wavefront v = 0..3
+    for (int v = wave; v < 4; v += n_waves) {
+        float ssq = 0.0f;
+        for (int64_t b = v; b < nb; b += 4) {
+            const float4 a = fetch(b * kQK + lane * 4);
+            ssq = __fmaf_rn(a.x, a.x, ssq);
+            ssq = __fmaf_rn(a.y, a.y, ssq);
+            ssq = __fmaf_rn(a.z, a.z, ssq);
+            ssq = __fmaf_rn(a.w, a.w, ssq);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+        if (lane == 0) wave_sum[v] = ssq;
+    }
+    __syncthreads();
+    const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+    const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)(nb * kQK)), eps)));
+
+    float acc[1][2] = {{0.0f, 0.0f}};
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        if (i < cnt) {
+            const int64_t c0 = (int64_t)(wave + i * n_waves) * kQK + lane * 4;
+            const float4 a = xv[i];
+            if (rt == 0 && sum_out) *reinterpret_cast<float4*>(sum_out + c0) = a;
+            float4 wn = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+            if (weight) wn = *reinterpret_cast<const float4*>(weight + c0);
+            const float e[4] = {__fmul_rn(a.x, weight ? __fmul_rn(scale, wn.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, wn.y) : scale),
+                                __fmul_rn(a.z, weight ? __fmul_rn(scale, wn.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, wn.w) : scale)};
+            ARegs<1> ar;
+            a_from_lane_codes(ar, quantize_block_q8k(e, lane), lane);
+            int32_t dsum[1][2], msum[1][2];
+            compute_tile<1>(t[i], ar, acc, dsum, msum);
+        }
+    }
+    if (n_waves > 1) {
+        if (wave > 0) red[(wave - 1) * 64 + lane] = acc[0][0];
+        __syncthreads();
+    }
+    if (wave == 0) {
+        float v = acc[0][0];
+        for (int wv = 1; wv < n_waves; ++wv) v = __fadd_rn(v, red[(wv - 1) * 64 + lane]);
+        const int64_t row = rt * 16 + slot;
+        if (kq == 0 && row < rows) y[row] = v;
+    }
+}
+
 }  // namespace
+
+hipError_t launch_gemv1_norm_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, const float* delta,
+                                   const float* weight, float eps, float* sum_out, float* y, int waves, hipStream_t stream) {
+    if (!gemv1_fused_applies(nb, waves) || rows <= 0) return hipErrorInvalidValue;
+    const int64_t rowtiles = (rows + 15) / 16;
+    hipLaunchKernelGGL(gemv1_norm_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
+                       waves > 1 ? (size_t)(waves - 1) * 64 * sizeof(float) : 0, stream, w, rows, nb, x, delta, weight, eps, sum_out,
+                       y);
+    return hipGetLastError();
+}
 
 bool gemv1_fused_applies(int64_t nb, int waves) { return waves >= 1 && (nb + waves - 1) / waves <= kMaxStages; }
 

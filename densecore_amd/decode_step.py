@@ -1,8 +1,7 @@
 """A synthetic MoE decoder step built from the C-ABI operators: per layer
 
-    h   = q8k(rmsnorm(x))                              mq_add_rmsnorm_q8k (fused with the previous residual add and
-                                                                           with the projection's quantizer)
-    qkv = W_qkv . h                                    mq_mul_mat_q4k_acts (wq, wk, wv stacked row-wise)
+    h   = q8k(rmsnorm(x))                              mq_rmsnorm_mul_mat_q4k (with the previous residual add; one launch
+    qkv = W_qkv . h                                                            at one token; wq, wk, wv stacked row-wise)
     o   = W_o . q8k(qkv[:, :n_q])                      mq_mul_mat_q4k     (the attention core itself is not on
                                                                            this path: q stands in for its output)
     x   = x + o ; h2 = rmsnorm(x)                      mq_add_rmsnorm_router_f32 (one launch; mq_add_rmsnorm_f32 +
@@ -123,10 +122,10 @@ class DecodeStep:
         fused_router = cfg.hidden % 256 == 0 and cfg.hidden <= 4096
         for i, ly in enumerate(self.layers):
             ly.desc.silu_mode = self.silu_mode()
-            chk(L.mq_add_rmsnorm_q8k(p(x), p(delta) if delta is not None else None, None, n, cfg.hidden,
-                                     C.c_float(cfg.eps), p(x), None, C.c_void_p(self.h_q8._h), st),
-                "mq_add_rmsnorm_q8k")
-            chk(L.mq_mul_mat_q4k_acts(ly.wqkv._h, C.c_void_p(self.h_q8._h), p(self.qkv), self.qkv.shape[1], st), "qkv")
+            # residual add, norm, Q8_K and the qkv projection (one launch at one token); the sum goes to the other buffer
+            chk(L.mq_rmsnorm_mul_mat_q4k(ly.wqkv._h, p(x), p(delta) if delta is not None else None, None, n, C.c_float(cfg.eps),
+                                         p(x_next), p(self.qkv), self.qkv.shape[1], st), "mq_rmsnorm_mul_mat_q4k")
+            x, x_next = x_next, x
             chk(L.mq_mul_mat_q4k(ly.wo._h, p(self.qkv), n, self.qkv.shape[1], p(self.o), cfg.hidden, st), "wo")
             if fused_router:
                 # residual add, norm and router projection in one launch; its sum goes to the other buffer because

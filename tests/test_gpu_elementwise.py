@@ -106,3 +106,32 @@ def test_add_rmsnorm_router_equals_the_two_launches(n, cols, n_experts, with_del
     with pytest.raises(_lib.MqError):
         _lib.check(L.mq_add_rmsnorm_router_f32(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(x), p(got_h), p(router),
                                                n_experts, p(got_lg), None), "fused in place")
+
+
+@pytest.mark.parametrize("n,rows,cols,with_delta,with_weight", [(1, 2560, 2048, True, False), (1, 512, 4096, False, True),
+                                                                 (1, 64, 512, True, True), (3, 2560, 2048, True, False)])
+def test_rmsnorm_mul_mat_equals_norm_then_product(n, rows, cols, with_delta, with_weight):
+    """mq_rmsnorm_mul_mat_q4k: the bits of mq_add_rmsnorm_q8k followed by mq_mul_mat_q4k_acts (one launch at one row)."""
+    import torch
+    from densecore_amd import _lib, ops
+    g = torch.Generator(device="cuda").manual_seed(rows + cols + n)
+    x = torch.randn((n, cols), device="cuda", generator=g)
+    d = torch.randn((n, cols), device="cuda", generator=g) if with_delta else None
+    w = (torch.rand((cols,), device="cuda", generator=g) + 0.5) if with_weight else None
+    W = ops.Q4KWeight.synthetic(rows * 7 + cols, rows, cols)
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    L = _lib.lib()
+    acts = ops.Q8KActs(n, cols)
+    ref_sum = torch.empty_like(x)
+    _lib.check(L.mq_add_rmsnorm_q8k(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(ref_sum), None, C.c_void_p(acts._h), None), "norm")
+    ref_y = acts.mul_mat(W, out=torch.empty((n, rows), device="cuda"))
+    got_sum = torch.empty_like(x)
+    got_y = torch.empty((n, rows), device="cuda")
+    _lib.check(L.mq_rmsnorm_mul_mat_q4k(W._h, p(x), p(d), p(w), n, C.c_float(1e-6), p(got_sum), p(got_y), rows, None), "fused")
+    torch.cuda.synchronize()
+    assert torch.equal(got_sum, ref_sum)
+    assert torch.equal(got_y, ref_y), f"max |diff| {(got_y - ref_y).abs().max().item():.3e}"
+    with pytest.raises(_lib.MqError):
+        _lib.check(L.mq_rmsnorm_mul_mat_q4k(W._h, p(x), p(d), p(w), n, C.c_float(1e-6), p(x), p(got_y), rows, None), "in place")
+    acts.free()
+    W.free()
