@@ -361,6 +361,7 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
 
 // Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk.
 constexpr int64_t kPrefillMinRows = 48;
+constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer (and norm) run inside the GEMV kernel (measured: 8 loses)
 
 static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                        hipStream_t s) {
@@ -402,6 +403,13 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
             return MQ_OK;
         }
     }
+    if (n <= kGemvFusedMaxRows && !census.on && w->type == kTypeQ4K) {  // a few rows, short K per wave: the same with the rows' codes going through LDS
+        const int waves = pick_waves(w->nb, w->rowtiles);
+        if (gemv1_fused_applies(w->nb, waves)) {
+            MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, ldx, nullptr, nullptr, 0.0f, nullptr, y_dev, ldy, (int)n, false, waves, s));
+            return MQ_OK;
+        }
+    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }
@@ -424,6 +432,14 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemv1_norm_fused(w->data, w->rows, w->nb, x_dev, delta_dev, weight_dev, eps, sum_out_dev, y_dev, waves, s));
+            return MQ_OK;
+        }
+    }
+    if (n <= kGemvFusedMaxRows && !census.on && w->type == kTypeQ4K) {
+        const int waves = pick_waves(w->nb, w->rowtiles);
+        if (gemv1_fused_applies(w->nb, waves)) {
+            MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, w->cols, delta_dev, weight_dev, eps, sum_out_dev, y_dev, ldy, (int)n, true,
+                                      waves, s));
             return MQ_OK;
         }
     }

@@ -157,7 +157,158 @@ __global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __
     }
 }
 
+// Up to eight rows, the same two ideas: every wavefront quantizes the super-blocks it multiplies -- one block per
+// row, parked as compact codes in a corner of LDS that only this wavefront uses (block of row t at t * 256, its
+// 64-byte chunks permuted by t & 3 so that the rows an MFMA reads side by side fall on different banks) and read
+// back as the split-slot A operand (common.h) -- and with kNorm the residual add and the RMSNorm of the rows run
+// inside as in gemv1_norm_fused_kernel.  Wave split of K, accumulation order and epilogue are matmul_kernel<1,1>'s:
+// the bits of quantize (or mq_add_rmsnorm_q8k) + matmul.
+template <bool kNorm>
+__global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restrict__ w, int64_t rows, int64_t nb,
+                                                          const float* __restrict__ x, int64_t ldx, const float* __restrict__ delta,
+                                                          const float* __restrict__ weight, float eps, float* __restrict__ sum_out,
+                                                          float* __restrict__ y, int64_t ldy, int n) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];  // [W][8 * 256 + 32] codes and scales, then red [W-1][2][64]
+    __shared__ float wave_sum[8][4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rt = blockIdx.x;
+    const uint8_t* tiles = w + tile_offset(rt, 0, nb);
+    const int cnt = wave < nb ? (int)((nb - wave + n_waves - 1) / n_waves) : 0;  // <= kMaxStages (host-checked)
+    uint8_t* codes = lds_raw + (size_t)wave * (8 * 256 + 32);
+    float* scales = reinterpret_cast<float*>(codes + 8 * 256);
+    float* red = reinterpret_cast<float*>(lds_raw + (size_t)n_waves * (8 * 256 + 32));
+    const int64_t cols = nb * kQK;
+    auto fetch = [&](int t, int64_t c0) {
+        float4 a = *reinterpret_cast<const float4*>(x + (size_t)t * ldx + c0);
+        if (kNorm && delta) {
+            const float4 d = *reinterpret_cast<const float4*>(delta + (size_t)t * cols + c0);
+            a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
+        }
+        return a;
+    };
+
+    TileRegs t[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) load_tile(t[i], tiles + (size_t)(i < cnt ? wave + i * n_waves : 0) * kTileBytes, lane);
+
+    float scale[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) scale[r] = 1.0f;
+    if (kNorm) {
+        // sums of squares in the order of the 256-thread norm kernel: virtual wavefront v = 0..3, row by row
+        for (int v = wave; v < 4; v += n_waves) {
+            for (int r = 0; r < n; ++r) {
+                float ssq = 0.0f;
+                for (int64_t b = v; b < nb; b += 4) {
+                    const float4 a = fetch(r, b * kQK + lane * 4);
+                    ssq = __fmaf_rn(a.x, a.x, ssq);
+                    ssq = __fmaf_rn(a.y, a.y, ssq);
+                    ssq = __fmaf_rn(a.z, a.z, ssq);
+                    ssq = __fmaf_rn(a.w, a.w, ssq);
+                }
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+                if (lane == 0) wave_sum[r][v] = ssq;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            if (r < n) {
+                const float total = (wave_sum[r][0] + wave_sum[r][1]) + (wave_sum[r][2] + wave_sum[r][3]);
+                scale[r] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
+            }
+        }
+    }
+
+    // this lane's part of the A operand: row (slot / 2, the last live one for a dead slot), half slot % 2
+    const int arow = (slot >> 1) < n ? (slot >> 1) : n - 1;
+    const int a_off = arow * 256 + 32 * (slot & 1) + 8 * kq, a_swz = arow & 3;
+    const uint32_t keep_lo = (slot & 1) ? 0u : 0xffffffffu, keep_hi = ~keep_lo;
+    const int d0 = 2 * kq < n ? 2 * kq : n - 1, d1 = 2 * kq + 1 < n ? 2 * kq + 1 : n - 1;
+
+    float acc[1][2] = {{0.0f, 0.0f}};
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        if (i < cnt) {
+            const int64_t c0 = (int64_t)(wave + i * n_waves) * kQK + lane * 4;
+            float4 xv[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+                if (r < n) xv[r] = fetch(r, c0);
+            float4 wn = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+            if (kNorm && weight) wn = *reinterpret_cast<const float4*>(weight + c0);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                if (r < n) {  // wave-uniform
+                    const float4 a = xv[r];
+                    if (kNorm && rt == 0 && sum_out) *reinterpret_cast<float4*>(sum_out + (size_t)r * cols + c0) = a;
+                    float e[4] = {a.x, a.y, a.z, a.w};
+                    if (kNorm) {
+                        e[0] = __fmul_rn(a.x, weight ? __fmul_rn(scale[r], wn.x) : scale[r]);
+                        e[1] = __fmul_rn(a.y, weight ? __fmul_rn(scale[r], wn.y) : scale[r]);
+                        e[2] = __fmul_rn(a.z, weight ? __fmul_rn(scale[r], wn.z) : scale[r]);
+                        e[3] = __fmul_rn(a.w, weight ? __fmul_rn(scale[r], wn.w) : scale[r]);
+                    }
+                    const Q8Lane q = quantize_block_q8k(e, lane);
+                    *reinterpret_cast<uint32_t*>(codes + r * 256 + ((((lane >> 4) ^ (r & 3)) << 6) | ((lane & 15) << 2))) = q.packed;
+                    if (lane == 0) scales[r] = q.d;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();  // the codes above are read by other lanes of this wavefront below
+            ARegs<1> ar;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const v2u v = *reinterpret_cast<const v2u*>(codes + a_off + ((c ^ a_swz) << 6));
+                ar.q[0][c] = v4u{v.x & keep_lo, v.y & keep_lo, v.x & keep_hi, v.y & keep_hi};
+            }
+            ar.yd[0][0] = scales[d0];
+            ar.yd[0][1] = scales[d1];
+            __builtin_amdgcn_wave_barrier();  // the next stage overwrites the codes
+            int32_t dsum[1][2], msum[1][2];
+            compute_tile<1>(t[i], ar, acc, dsum, msum);
+        }
+    }
+    if (n_waves > 1) {
+        if (wave > 0) {
+            red[((wave - 1) * 2 + 0) * 64 + lane] = acc[0][0];
+            red[((wave - 1) * 2 + 1) * 64 + lane] = acc[0][1];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+        for (int wv = 1; wv < n_waves; ++wv) {
+            acc[0][0] = __fadd_rn(acc[0][0], red[((wv - 1) * 2 + 0) * 64 + lane]);
+            acc[0][1] = __fadd_rn(acc[0][1], red[((wv - 1) * 2 + 1) * 64 + lane]);
+        }
+        const int64_t row = rt * 16 + slot;
+        if (row < rows) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (2 * kq + j < n) y[(size_t)(2 * kq + j) * ldy + row] = acc[0][j];
+        }
+    }
+}
+
 }  // namespace
+
+hipError_t launch_gemvn_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, int64_t ldx, const float* delta,
+                              const float* weight, float eps, float* sum_out, float* y, int64_t ldy, int n, bool norm, int waves,
+                              hipStream_t stream) {
+    if (!gemv1_fused_applies(nb, waves) || rows <= 0 || n < 1 || n > 8) return hipErrorInvalidValue;
+    const int64_t rowtiles = (rows + 15) / 16;
+    const size_t lds = (size_t)waves * (8 * 256 + 32) + (waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0);
+    if (norm)
+        hipLaunchKernelGGL(gemvn_fused_kernel<true>, dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx, delta,
+                           weight, eps, sum_out, y, ldy, n);
+    else
+        hipLaunchKernelGGL(gemvn_fused_kernel<false>, dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx,
+                           delta, weight, eps, sum_out, y, ldy, n);
+    return hipGetLastError();
+}
 
 hipError_t launch_gemv1_norm_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, const float* delta,
                                    const float* weight, float eps, float* sum_out, float* y, int waves, hipStream_t stream) {

@@ -84,6 +84,11 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
 // ---- gemv1.hip -------------------------------------------------------------------------------
 // One activation row, quantizer inside the kernel; applies when a wave sees at most two super-blocks.
 bool gemv1_fused_applies(int64_t nb, int waves);
+// Up to eight rows with the quantizer inside, optionally with the residual add and the RMSNorm of the rows as well
+// (norm: delta, weight, eps, sum_out as in launch_add_rmsnorm; x rows then dense, ldx == cols).
+hipError_t launch_gemvn_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, int64_t ldx, const float* delta,
+                              const float* weight, float eps, float* sum_out, float* y, int64_t ldy, int n, bool norm, int waves,
+                              hipStream_t stream);
 // The same with the residual add and the RMSNorm of the row inside (sum_out apart from x and delta).
 hipError_t launch_gemv1_norm_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, const float* delta,
                                    const float* weight, float eps, float* sum_out, float* y, int waves, hipStream_t stream);
