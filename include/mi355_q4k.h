@@ -274,9 +274,9 @@ int mq_add_rmsnorm_f32(const float* x_dev, const float* delta_dev, const float* 
 int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n, int64_t cols,
                        float eps, float* sum_out_dev, float* normed_out_dev, mq_acts* acts, void* stream);
 /* mq_add_rmsnorm_q8k followed by mq_mul_mat_q4k_acts: sum = x + delta (delta_dev may be NULL), h = rmsnorm(sum) *
- * weight (weight_dev may be NULL), y[t] = W . q8k(h[t]); x/delta/sum fp32 [n][cols] dense, y fp32 [n][ldy].  One row
- * of Q4_K weights with short rows runs as ONE launch (norm and quantizer inside the GEMV), otherwise two; the same
- * bits either way.  sum_out_dev (may be NULL) must be neither x_dev nor delta_dev.  Meant for decode widths (wide
+ * weight (weight_dev may be NULL), y[t] = W . q8k(h[t]); x/delta/sum fp32 [n][cols] dense, y fp32 [n][ldy].  Up to
+ * four rows of input against Q4_K weights with short rows run as ONE launch (norm and quantizer inside the GEMV),
+ * otherwise two; the same bits either way.  sum_out_dev (may be NULL) must be neither x_dev nor delta_dev.  Meant for decode widths (wide
  * inputs take the decode kernel in passes, not the matrix-core GEMM). */
 int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n,
                            float eps, float* sum_out_dev, float* y_dev, int64_t ldy, void* stream);
