@@ -410,6 +410,19 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
             return MQ_OK;
         }
     }
+    if (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) {  // single row, long K per wave: the quantizer runs inside the decode kernel
+        MatmulArgs a;
+        a.w0 = w->data;
+        a.wtype = w->type;
+        a.rows = w->rows;
+        a.nb = w->nb;
+        a.xf = x_dev;
+        a.n = 1;
+        a.y = y_dev;
+        a.ldy = ldy;
+        MQ_HIP(census_launch(a, s));
+        return MQ_OK;
+    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }
@@ -521,7 +534,10 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+    // One row: both quantizers run inside the products (two launches instead of four, the same bits).
+    const bool inline_quant = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
+    if (!inline_quant)
+        if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
     MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
     MatmulArgs a;
     a.w0 = gate->data;
@@ -529,8 +545,12 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.w1 = up->data;
     a.rows = inter;
     a.nb = gate->nb;
-    a.aq = (const uint8_t*)g.aq.ptr;
-    a.ad = (const float*)g.ad.ptr;
+    if (inline_quant) {
+        a.xf = x_dev;
+    } else {
+        a.aq = (const uint8_t*)g.aq.ptr;
+        a.ad = (const float*)g.ad.ptr;
+    }
     a.n = n;
     a.y = (float*)g.mid.ptr;
     a.ldy = inter;
@@ -539,14 +559,19 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     MQ_HIP(census_launch(a, s));
     // The SwiGLU output is re-quantized by a launch of its own: the kernel's fused re-quantization (last
     // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
-    if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    if (!inline_quant)
+        if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
     d.wtype = down->type;
     d.rows = hidden;
     d.nb = down->nb;
-    d.aq = (const uint8_t*)g.aq2.ptr;
-    d.ad = (const float*)g.ad2.ptr;
+    if (inline_quant) {
+        d.xf = (const float*)g.mid.ptr;
+    } else {
+        d.aq = (const uint8_t*)g.aq2.ptr;
+        d.ad = (const float*)g.ad2.ptr;
+    }
     d.n = n;
     d.y = y_dev;
     d.ldy = hidden;
@@ -882,15 +907,21 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
+    const bool inline_quant = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);  // one row: the quantizer runs inside the product
+    if (!inline_quant)
+        if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
     MatmulArgs a;
     a.w0 = gate->data;
     a.wtype = gate->type;
     a.w1 = up->data;
     a.rows = gate->rows;
     a.nb = gate->nb;
-    a.aq = (const uint8_t*)g.aq.ptr;
-    a.ad = (const float*)g.ad.ptr;
+    if (inline_quant) {
+        a.xf = x_dev;
+    } else {
+        a.aq = (const uint8_t*)g.aq.ptr;
+        a.ad = (const float*)g.ad.ptr;
+    }
     a.n = n;
     a.y = h_dev;
     a.ldy = ldh;

@@ -48,7 +48,9 @@ __device__ __forceinline__ uint32_t fifth_bits(uint32_t h, int s) {
     return (s <= 4 ? h << (4 - s) : h >> (s - 4)) & 0x10101010u;
 }
 
-template <int TT, bool Q5 = false>
+// J = 1: only the first of a lane's two activation rows is formed (a single activation row sits in row 0 of the
+// operand: j = 1 would be work on a row that is never stored); the same bits for the row that is.
+template <int TT, bool Q5 = false, int J = 2>
 __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>& a, float (&acc)[TT][2],
                                              int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2]) {
     // 6-bit scale / min unpack, word-parallel (core/src/kernels/hwy/hwy_moe_quant.cc:90-101)
@@ -89,7 +91,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
             // p[0], p[2]: sub-block 2c of rows 2kq and 2kq+1;  p[1], p[3]: sub-block 2c+1
             const v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(a16, b_q, zero, 0, 0, 0);
             dot[tt][0] += __mul24(p[0], s_lo) + __mul24(p[1], s_hi);
-            dot[tt][1] += __mul24(p[2], s_lo) + __mul24(p[3], s_hi);
+            if (J > 1) dot[tt][1] += __mul24(p[2], s_lo) + __mul24(p[3], s_hi);
             mnd[tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a16, b_min, mnd[tt], 0, 0, 0);
         }
     }
@@ -98,7 +100,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs& t, const ARegs<TT>&
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < J; ++j) {
             const int32_t md = mnd[tt][2 * j] + mnd[tt][2 * j + 1];
             const float d = __fmul_rn(wd, a.yd[tt][j]);
             const float dm = __fmul_rn(wm, a.yd[tt][j]);
@@ -131,7 +133,7 @@ __device__ __forceinline__ void load_tile6(TileRegs6& t, const uint8_t* tile, in
 // k-groups 0..1 (weights 0..15 of each 32-wide half) and one with those of k-groups 2..3 (weights 16..31): the four
 // sums that come out are the chunk's four 16-weight groups.  dot_out = sum_g scale_g * sum (code - 32) * q8 exactly
 // (core/src/llm/matmul/q6_small_batch.h:56-83); fp32: acc = fma(d * yd, float(dot), acc) (:84-86).
-template <int TT>
+template <int TT, int J = 2>
 __device__ __forceinline__ void compute_tile6(const TileRegs6& t, const ARegs<TT>& a, float (&acc)[TT][2],
                                               int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2], int lane) {
     const uint32_t keep_lo = (lane & 32) ? 0u : 0xffffffffu;  // k-groups 0 and 1
@@ -166,14 +168,14 @@ __device__ __forceinline__ void compute_tile6(const TileRegs6& t, const ARegs<TT
             const v4i pl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_lo, b_q, zero, 0, 0, 0);
             const v4i ph = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_hi, b_q, zero, 0, 0, 0);
             dot[tt][0] += __mul24(pl[0], s0) + __mul24(ph[0], s1) + __mul24(pl[1], s2) + __mul24(ph[1], s3);
-            dot[tt][1] += __mul24(pl[2], s0) + __mul24(ph[2], s1) + __mul24(pl[3], s2) + __mul24(ph[3], s3);
+            if (J > 1) dot[tt][1] += __mul24(pl[2], s0) + __mul24(ph[2], s1) + __mul24(pl[3], s2) + __mul24(ph[3], s3);
         }
     }
     const float wd = half_bits_to_float(t.d & 0xffffu);
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < J; ++j) {
             const int32_t isum = dot[tt][j] >> 2;  // the B bytes carried a factor 4
             acc[tt][j] = __fmaf_rn(__fmul_rn(a.yd[tt][j], wd), (float)isum, acc[tt][j]);
             dot_out[tt][j] = isum;
@@ -193,11 +195,11 @@ __device__ __forceinline__ void load_tile_wt(typename TileOf<WT>::Regs& t, const
     if constexpr (WT == kWtQ6) load_tile6(t, tile, lane);
     else load_tile<WT == kWtQ5>(t, tile, lane);
 }
-template <int TT, int WT>
+template <int TT, int WT, int J = 2>
 __device__ __forceinline__ void compute_tile_wt(const typename TileOf<WT>::Regs& t, const ARegs<TT>& a, float (&acc)[TT][2],
                                                 int32_t (&dot_out)[TT][2], int32_t (&min_out)[TT][2], int lane) {
-    if constexpr (WT == kWtQ6) compute_tile6<TT>(t, a, acc, dot_out, min_out, lane);
-    else compute_tile<TT, WT == kWtQ5>(t, a, acc, dot_out, min_out);
+    if constexpr (WT == kWtQ6) compute_tile6<TT, J>(t, a, acc, dot_out, min_out, lane);
+    else compute_tile<TT, WT == kWtQ5, J>(t, a, acc, dot_out, min_out);
 }
 
 #endif

@@ -36,6 +36,9 @@ struct MatmulArgs {
     size_t expert_bytes = 0;       // tiled bytes per expert (grouped mode)
     const uint8_t* aq = nullptr;   // A-major activations
     const float* ad = nullptr;
+    // dense mode, n == 1: the activation row as fp32 instead; every wavefront quantizes the super-blocks it
+    // multiplies (same codes and scales as the stand-alone quantizer, so the same result)
+    const float* xf = nullptr;
     int64_t n = 0;                 // activation rows (dense mode)
     float* y = nullptr;            // dense: [n][ldy]; grouped: [entry][ldy]
     int64_t ldy = 0;

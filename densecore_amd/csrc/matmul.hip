@@ -73,7 +73,12 @@ struct Depth {
 // One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
 // waves split the super-blocks of the row.  NMAT == 2: gate and up tiles of the same rows share
 // the activations in registers and meet in silu(gate)*up.
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT>
+// J == 1: a single activation row (dense, n == 1): the second of a lane's two activation rows is not formed at all.
+// XQ (dense, n == 1): the activation row comes as fp32 (p.xf) and every wavefront quantizes the super-blocks it
+// multiplies while their weight tiles travel -- the block quantizer of quantize_q8k_kernel, so the same codes,
+// scales and result as the stand-alone quantizer followed by this kernel, one launch less.  (With two rows the
+// repeated quantization costs what the saved launch gains, with four it loses a third.)
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
     constexpr int S = Depth<NMAT, TT, WT>::kStages;
@@ -172,7 +177,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < J; ++j) {
                     if (yrow[tt][j] >= 0) {
                         float v = acc[0][tt][j];
                         if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][tt][j], silu_mode);
@@ -195,9 +200,10 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             const int cnt = per_rt * rt_count;                              // stages of this wave
             typename TileOf<WT>::Regs ring_t[S][NMAT];
             ARegs<TT> ring_a[S];
+            float4 ring_x[S];
             // Requests past the wave's last super-block are pointed at the (cache-resident)
-            // activation buffer instead of being skipped: the number of loads per stage stays
-            // fixed, so every wait below can count exactly.
+            // activation buffer (without one: at the wave's first tile again) instead of being
+            // skipped: the number of loads per stage stays fixed, so every wait below can count exactly.
             auto issue = [&](int st, int i) {
                 const bool valid = i < cnt;
                 // several row tiles (one wave, per_rt == nb): stage i is tile i of the contiguous run,
@@ -206,14 +212,24 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 const int b = rt_per_wg > 1 ? t % per_rt : t;
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    load_tile_wt<WT>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : p.aq, lane);
-                load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+                    load_tile_wt<WT>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : XQ ? tiles[m] + (size_t)wave * kTileStride : p.aq, lane);
+                if constexpr (XQ) {
+                    ring_x[st] = *reinterpret_cast<const float4*>(p.xf + (size_t)b * kQK + lane * 4);
+                } else {
+                    load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+                }
             };
             auto consume = [&](int st, int i) {
+                ARegs<TT> quantized;
+                if constexpr (XQ) {  // the row becomes row 0 of the operand
+                    const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
+                    a_from_lane_codes(quantized, quantize_block_q8k(e, lane), lane);
+                }
+                const ARegs<TT>& a_regs = XQ ? quantized : ring_a[st];
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][2], msum[TT][2];
-                    compute_tile_wt<TT, WT>(ring_t[st][m], ring_a[st], acc[m], dsum, msum, lane);
+                    compute_tile_wt<TT, WT, J>(ring_t[st][m], a_regs, acc[m], dsum, msum, lane);
                     if (DEBUG && p.dbg_dot) {  // debug launches own one row tile per workgroup
                         const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;
@@ -259,7 +275,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                        for (int j = 0; j < 2; ++j)
+                        for (int j = 0; j < J; ++j)
                             red[((((wave - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane] = acc[m][tt][j];
             }
             __syncthreads();
@@ -271,7 +287,7 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
-                        for (int j = 0; j < 2; ++j)
+                        for (int j = 0; j < J; ++j)
                             acc[m][tt][j] =
                                 __fadd_rn(acc[m][tt][j], red[((((wv - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane]);
             }
@@ -314,15 +330,15 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     }
 }
 
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false>
 hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
     if (start && stop) {
         // the events take the dispatch's own begin / end timestamps: no extra packets around the kernel
-        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT>), grid, dim3(64 * waves), lds, stream, start, stop,
+        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ>), grid, dim3(64 * waves), lds, stream, start, stop,
                               0, a);
     } else {
-        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT>), grid, dim3(64 * waves), lds, stream, a);
+        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ>), grid, dim3(64 * waves), lds, stream, a);
     }
     return hipGetLastError();
 }
@@ -343,6 +359,7 @@ int pick_waves(int64_t nb, int64_t workgroups) {
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     if (a.rows <= 0 || a.nb <= 0) return hipErrorInvalidValue;
     if (a.out_aq && (a.rows & 255)) return hipErrorInvalidValue;
+    if (a.xf && (a.grouped || a.dbg_dot || a.out_aq || a.n != 1 || (reinterpret_cast<uintptr_t>(a.xf) & 15u))) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
     const int nmat = a.swiglu ? 2 : 1;
     const bool debug = a.dbg_dot != nullptr;
@@ -369,6 +386,8 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     do {                                                                                                  \
         if (a.grouped) return launch_one<NM, T, true, false, W>(b, waves, grid, stream, start, stop);     \
         if (debug) return launch_one<NM, T, false, true, W>(b, waves, grid, stream, start, stop);         \
+        if (T == 1 && a.xf) return launch_one<NM, 1, false, false, W, 1, true>(b, waves, grid, stream, start, stop); \
+        if (T == 1 && a.n == 1) return launch_one<NM, 1, false, false, W, 1>(b, waves, grid, stream, start, stop); \
         return launch_one<NM, T, false, false, W>(b, waves, grid, stream, start, stop);                   \
     } while (0)
 #define MQ_LAUNCH(NM, T)                                 \

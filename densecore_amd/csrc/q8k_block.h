@@ -92,6 +92,7 @@ __device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, 
     a.yd[0][0] = q.d;
     a.yd[0][1] = 0.0f;
 }
+
 #endif
 
 }  // namespace mq

@@ -43,7 +43,7 @@ def down_mag(w, cols, x):
     return orc.dot_magnitude_f64(w, cols, q8)
 
 
-@pytest.mark.parametrize("n", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 8, 16])
 @pytest.mark.parametrize("silu", [0, 1, 2])
 def test_swiglu_and_ffn_stagewise(ops, n, silu):
     H, I = 1024, 1792
