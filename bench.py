@@ -358,6 +358,22 @@ def side_measurements(ops, synth, torch, np, dev):
     sib["note"] = "matmul from pre-quantized activations, 4096 x 14336 weights, bytes = ggml bytes of the type + fp32 in/out"
     res["down_projection_by_weight_type"] = sib
 
+    # Q8_0 weights against Q8_0 activations (the reference's vec_dot_type for the type): the same shape, quantizer
+    # launch included, ring of 10 matrices (624 MB)
+    ring = [ops.Q4KWeight.synthetic(synth.tensor_seed("sib", "Q8_0", r), 4096, 14336, 1, synth.GGML_TYPE_Q8_0) for r in range(10)]
+    per = {}
+    for n in (1, 8):
+        xq = torch.from_numpy(synth.normal_f32(synth.tensor_seed("sib-x", n), (n, 14336))).to(dev)
+        y = torch.empty((n, 4096), dtype=torch.float32, device=dev)
+        dt = time_graph(lambda: [ops.mul_mat(w, xq, out=y) for w in ring], 20) / len(ring)
+        b = 4096 * (14336 // 32) * 34 + n * (14336 + 4096) * 4
+        per[str(n)] = {"us": round(dt * 1e6, 2), "GBps": round(b / dt / 1e9, 1),
+                       "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+    per["note"] = "quantize (Q8_0) + matmul, two launches, 4096 x 14336 weights, bytes = ggml bytes + fp32 in/out"
+    res["q8_0_projection"] = per
+    for w in ring:
+        w.free()
+
     # cfg3: MoE layer, hidden 2048, 256 + 1 experts, inter 512, top-8; ring of 4 layers (1.8 GB)
     E, H, I, K = 256, 2048, 512, 8
     layers = []

@@ -128,8 +128,10 @@ int check_ready() {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int check_weight(const mq_weight* w, const char* name) {
+// Q8_0 matrices are dense projections only: mq_mul_mat_q4k (and the handle queries) take them, nothing else does.
+int check_weight(const mq_weight* w, const char* name, bool q80_ok = false) {
     if (!w || !w->data) return fail(MQ_ERR_INVALID, "%s: null weight handle", name);
+    if (w->type == kTypeQ80 && !q80_ok) return fail(MQ_ERR_UNSUPPORTED, "%s: Q8_0 weights are taken by mq_mul_mat_q4k only", name);
     return MQ_OK;
 }
 
@@ -163,8 +165,9 @@ int reserve_counters(size_t count) {
 int alloc_weight(int type, int64_t rows, int64_t cols, int64_t n_experts, mq_weight** out) {
     if (!out) return fail(MQ_ERR_INVALID, "null output handle");
     *out = nullptr;
-    if (type != kTypeQ4K && type != kTypeQ5K && type != kTypeQ6K)
-        return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12), Q5_K (13) and Q6_K (14) weights are supported", type);
+    if (type != kTypeQ4K && type != kTypeQ5K && type != kTypeQ6K && type != kTypeQ80)
+        return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12), Q5_K (13), Q6_K (14) and Q8_0 (8) weights are supported", type);
+    if (type == kTypeQ80 && n_experts != 1) return fail(MQ_ERR_UNSUPPORTED, "Q8_0 expert stacks are not supported");
     if (rows <= 0 || cols <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "rows, cols and n_experts must be positive");
     if (cols % kQK) return fail(MQ_ERR_INVALID, "cols %lld is not a multiple of 256", (long long)cols);
     mq_weight* w = new mq_weight;
@@ -243,8 +246,8 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
 int mq_weight_upload_typed(int ggml_type, const void* q4k_host, int64_t rows, int64_t cols, int64_t n_experts,
                            size_t row_bytes, size_t expert_bytes, mq_weight** out) {
     if (int rc = check_ready()) return rc;
-    if (ggml_type != kTypeQ4K && ggml_type != kTypeQ5K && ggml_type != kTypeQ6K)
-        return fail(MQ_ERR_UNSUPPORTED, "mq_weight_upload: ggml type %d (only 12 = Q4_K, 13 = Q5_K and 14 = Q6_K)", ggml_type);
+    if (ggml_type != kTypeQ4K && ggml_type != kTypeQ5K && ggml_type != kTypeQ6K && ggml_type != kTypeQ80)
+        return fail(MQ_ERR_UNSUPPORTED, "mq_weight_upload: ggml type %d (only 12 = Q4_K, 13 = Q5_K, 14 = Q6_K and 8 = Q8_0)", ggml_type);
     if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_upload: null host pointer");
     if (cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_weight_upload: cols %lld is not a positive multiple of 256", (long long)cols);
     const size_t min_row = (size_t)(cols / kQK) * (size_t)block_bytes_of(ggml_type);
@@ -291,7 +294,7 @@ int mq_weight_synthetic_typed(int ggml_type, uint64_t seed, int64_t rows, int64_
 
 int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, size_t expert_bytes) {
     if (int rc = check_ready()) return rc;
-    if (int rc = check_weight(w, "mq_weight_download")) return rc;
+    if (int rc = check_weight(w, "mq_weight_download", true)) return rc;
     if (!q4k_host) return fail(MQ_ERR_INVALID, "mq_weight_download: null host pointer");
     const size_t min_row = (size_t)w->nb * (size_t)block_bytes_of(w->type);
     if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_download: bad row_bytes");
@@ -311,7 +314,7 @@ int mq_weight_download(const mq_weight* w, void* q4k_host, size_t row_bytes, siz
 }
 
 int mq_weight_shape(const mq_weight* w, int64_t* rows, int64_t* cols, int64_t* n_experts, size_t* device_bytes) {
-    if (int rc = check_weight(w, "mq_weight_shape")) return rc;
+    if (int rc = check_weight(w, "mq_weight_shape", true)) return rc;
     if (rows) *rows = w->rows;
     if (cols) *cols = w->cols;
     if (n_experts) *n_experts = w->n_experts;
@@ -372,6 +375,29 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
     return MQ_OK;
 }
 
+// Q8_0 weights: the activations are quantized to Q8_0 as well (codes into g.aq in the A-major order, fp16 scales
+// into g.ad), then one launch.
+static int mul_mat_q80_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                              int32_t* dbg_sum, hipStream_t s) {
+    if ((ldx & 3) || (reinterpret_cast<uintptr_t>(x_dev) & 15u))
+        return fail(MQ_ERR_INVALID, "Q8_0 product: activation rows must be 16-byte aligned (ldx %% 4 == 0)");
+    MQ_HIP(g.aq.reserve(aq_bytes(n, w->nb)));
+    MQ_HIP(g.ad.reserve(q80_scale_bytes(n, w->nb)));
+    MQ_HIP(launch_quantize_q80(x_dev, n, ldx, w->cols, (uint8_t*)g.aq.ptr, (uint16_t*)g.ad.ptr, s));
+    Q80MatmulArgs a;
+    a.w = w->data;
+    a.rows = w->rows;
+    a.nb = w->nb;
+    a.aq = (const uint8_t*)g.aq.ptr;
+    a.ah = (const uint16_t*)g.ad.ptr;
+    a.n = n;
+    a.y = y_dev;
+    a.ldy = ldy;
+    a.dbg_sum = dbg_sum;
+    MQ_HIP(launch_q80_matmul(a, s));
+    return MQ_OK;
+}
+
 int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                 void* stream) {
     if (int rc = check_ready()) return rc;
@@ -388,13 +414,14 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
 int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                    void* stream) {
     if (int rc = check_ready()) return rc;
-    if (int rc = check_weight(w, "mq_mul_mat_q4k")) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k", true)) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: weight is an expert stack; use mq_mul_mat_id_q4k");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_mul_mat_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, nullptr, s);
     if (n >= kPrefillMinRows && w->type == kTypeQ4K) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
     if (n == 1 && !census.on && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
@@ -482,7 +509,7 @@ int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t
 
 int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int64_t ldx, float* y_host, int64_t ldy) {
     if (int rc = check_ready()) return rc;
-    if (int rc = check_weight(w, "mq_mul_mat_q4k_host")) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k_host", true)) return rc;
     if (!x_host || !y_host || n < 0 || ldx < w->cols || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_host: bad arguments");
     if (n == 0) return MQ_OK;
     float* xin = nullptr;
@@ -503,13 +530,15 @@ int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int6
 int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, int32_t* dot_scaled_dev,
                         int32_t* min_dot_dev, float* y_dev, int64_t ldy, void* stream) {
     if (int rc = check_ready()) return rc;
-    if (int rc = check_weight(w, "mq_debug_block_sums")) return rc;
+    if (int rc = check_weight(w, "mq_debug_block_sums", true)) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: dense weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_debug_block_sums")) return rc;
     if (n == 0) return MQ_OK;
-    if (!dot_scaled_dev || !min_dot_dev || !y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_debug_block_sums: null output");
+    if (!dot_scaled_dev || (!min_dot_dev && w->type != kTypeQ80) || !y_dev || ldy < w->rows)
+        return fail(MQ_ERR_INVALID, "mq_debug_block_sums: null output");
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, dot_scaled_dev, s);
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, dot_scaled_dev, min_dot_dev, s);
 }

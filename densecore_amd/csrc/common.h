@@ -83,11 +83,34 @@ __host__ __device__ inline int tile_word_offset_q6(int r, int word) {
     if (word < 26) return kTile6SOff + r * 16 + (word - 24) * 8;
     return kTile6DOff + r * 4;
 }
-__host__ __device__ inline int tile_bytes_of(int type) {
-    return type == kTypeQ6K ? kTile6Bytes : type == kTypeQ5K ? kTile5Bytes : kTileBytes;
+// ---------------------------------------------------------------------------------------------
+// Q8_0 (fp16 d, int8 qs[32]; 34 bytes per 32 weights, core/src/llm/matmul/q8_small_batch.h:9-14).  Eight
+// consecutive blocks of a row -- 256 weights, 272 bytes -- take the place of a super-block.  Tile of 16 rows x 256
+// weights, 4352 bytes:
+//   bytes [c*1024 + (kq*16 + r)*16, +16), c = 0..3 = qs[8 kq .. +7] of block 2c, then of block 2c + 1, of row r:
+//        the B operand of the MFMA over the 64-weight chunk c, the same element order as the Q4_K tile
+//   bytes [4096 + r*16, +16)                       = the eight fp16 d of row r
+// Words as the re-tiling kernels move them: 0..31 = eight code bytes each (word 4k + j = qs[8j .. 8j+7] of block
+// k), 32..39 = the two-byte d of block k = word - 32.
+// ---------------------------------------------------------------------------------------------
+constexpr int kTypeQ80 = 8;  // ggml_type value
+constexpr int kQ80Block = 34, kQ80Super = 8 * kQ80Block;
+constexpr int kTile80SOff = 4096, kTile80Bytes = 4352;
+__host__ __device__ inline int tile_word_offset_q80(int r, int word) {
+    if (word >= 32) return kTile80SOff + r * 16 + (word - 32) * 2;
+    const int k = word >> 2, j = word & 3;
+    return (k >> 1) * 1024 + (j * 16 + r) * 16 + (k & 1) * 8;
 }
+// byte offset of a word inside the 272 bytes of its eight blocks in a ggml row
+__host__ __device__ inline int row_word_offset_q80(int word) {
+    return word >= 32 ? (word - 32) * kQ80Block : (word >> 2) * kQ80Block + 2 + (word & 3) * 8;
+}
+__host__ __device__ inline int tile_bytes_of(int type) {
+    return type == kTypeQ80 ? kTile80Bytes : type == kTypeQ6K ? kTile6Bytes : type == kTypeQ5K ? kTile5Bytes : kTileBytes;
+}
+// bytes of one row's 256 weights in ggml's layout
 __host__ __device__ inline int block_bytes_of(int type) {
-    return type == kTypeQ6K ? kQ6Block : type == kTypeQ5K ? kQ5Block : kQ4Block;
+    return type == kTypeQ80 ? kQ80Super : type == kTypeQ6K ? kQ6Block : type == kTypeQ5K ? kQ5Block : kQ4Block;
 }
 __host__ __device__ inline int tile_word_offset_q5(int r, int word) {
     if (word < 2) return kTileQBytes + r * 16 + word * 8;

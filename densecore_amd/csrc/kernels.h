@@ -84,6 +84,24 @@ int pick_waves(int64_t nb, int64_t workgroups);
 // start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
+// ---- q8_0.hip --------------------------------------------------------------------------------
+// Q8_0 weights (16-row tiles of common.h) x Q8_0 activations, dense, any n (passes of eight rows).
+struct Q80MatmulArgs {
+    const uint8_t* w = nullptr;    // tiled weights
+    int64_t rows = 0;
+    int64_t nb = 0;                // 256-weight groups per row (cols / 256)
+    const uint8_t* aq = nullptr;   // A-major codes (the layout of the Q8_K codes)
+    const uint16_t* ah = nullptr;  // fp16 d: eight per (row, group), at ad_index(row, group, nb) * 8
+    int64_t n = 0;
+    float* y = nullptr;            // [n][ldy]
+    int64_t ldy = 0;
+    int32_t* dbg_sum = nullptr;    // optional [rows][n][cols / 32] integer block sums
+};
+size_t q80_scale_bytes(int64_t n, int64_t nb);
+// x rows 16-byte aligned (ldx % 4 == 0), cols % 256 == 0
+hipError_t launch_quantize_q80(const float* x, int64_t n, int64_t ldx, int64_t cols, uint8_t* aq, uint16_t* ah, hipStream_t stream);
+hipError_t launch_q80_matmul(const Q80MatmulArgs& a, hipStream_t stream);
+
 // ---- gemv1.hip -------------------------------------------------------------------------------
 // One activation row, quantizer inside the kernel; applies when a wave sees at most two super-blocks.
 bool gemv1_fused_applies(int64_t nb, int waves);

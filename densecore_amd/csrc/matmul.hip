@@ -229,7 +229,10 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m) {
                     int32_t dsum[TT][2], msum[TT][2];
-                    compute_tile_wt<TT, WT, J>(ring_t[st][m], a_regs, acc[m], dsum, msum, lane);
+                    if (GROUPED && TT == 1 && count == 1)  // most expert groups hold one row: its partner row is not formed
+                        compute_tile_wt<TT, WT, 1>(ring_t[st][m], a_regs, acc[m], dsum, msum, lane);
+                    else
+                        compute_tile_wt<TT, WT, J>(ring_t[st][m], a_regs, acc[m], dsum, msum, lane);
                     if (DEBUG && p.dbg_dot) {  // debug launches own one row tile per workgroup
                         const int b = wave + i * n_waves;
                         const int64_t row = rt * 16 + slot;

@@ -1,7 +1,8 @@
-// Weight re-tiling (ggml block_q4_K / block_q5_K / block_q6_K rows <-> the 16-row tile layouts of common.h)
+// Weight re-tiling (ggml block_q4_K / block_q5_K / block_q6_K / Q8_0 rows <-> the 16-row tile layouts of common.h)
 // and the on-device synthetic fill.  One thread moves one 8-byte word of a block; each such word lands in one
-// contiguous 8-byte slot of a tile (tile_word_offset, tile_word_offset_q5, tile_word_offset_q6).  The last
-// "word" of a block_q6_K is its two-byte d.
+// contiguous 8-byte slot of a tile (tile_word_offset, tile_word_offset_q5, tile_word_offset_q6,
+// tile_word_offset_q80).  The last "word" of a block_q6_K is its two-byte d, and so are the last eight "words" of
+// a row's eight Q8_0 blocks.
 #include "common.h"
 #include "kernels.h"
 
@@ -9,8 +10,16 @@ namespace mq {
 
 namespace {
 
-// 8-byte words per block: 18 (Q4_K), 22 (Q5_K), 26 + the two-byte d (Q6_K)
-__host__ __device__ inline int words_per_block(int type) { return type == kTypeQ6K ? 27 : block_bytes_of(type) / 8; }
+// 8-byte words per block: 18 (Q4_K), 22 (Q5_K), 26 + the two-byte d (Q6_K), 32 + eight two-byte d (eight Q8_0 blocks)
+__host__ __device__ inline int words_per_block(int type) {
+    return type == kTypeQ80 ? 40 : type == kTypeQ6K ? 27 : block_bytes_of(type) / 8;
+}
+// a word that is a lone fp16 scale (two bytes)
+__host__ __device__ inline bool scale_word(int type, int word) {
+    return (type == kTypeQ6K && word == 26) || (type == kTypeQ80 && word >= 32);
+}
+// where a word starts inside its block in a ggml row
+__host__ __device__ inline int row_word_offset(int type, int word) { return type == kTypeQ80 ? row_word_offset_q80(word) : word * 8; }
 // Q6_K: the qh words are stored with bit 5 of every code flipped (common.h)
 __host__ __device__ inline uint64_t stored_form(uint64_t v, int type, int word) {
     return (type == kTypeQ6K && word >= 16 && word < 24) ? v ^ 0xAAAAAAAAAAAAAAAAull : v;
@@ -32,7 +41,8 @@ __device__ __forceinline__ bool decode_word(int64_t idx, int64_t rows, int64_t n
 __device__ __forceinline__ size_t word_in_tiles(int64_t row, int64_t b, int64_t nb, int word, int type) {
     const int r = (int)(row & 15);
     return tile_offset(row >> 4, b, nb, tile_bytes_of(type)) +
-           (size_t)(type == kTypeQ6K   ? tile_word_offset_q6(r, word)
+           (size_t)(type == kTypeQ80   ? tile_word_offset_q80(r, word)
+                    : type == kTypeQ6K ? tile_word_offset_q6(r, word)
                     : type == kTypeQ5K ? tile_word_offset_q5(r, word)
                                        : tile_word_offset(r, word));
 }
@@ -45,12 +55,13 @@ __global__ void __launch_bounds__(256) tile_weights_kernel(const uint8_t* __rest
     int word;
     if (!decode_word(idx, rows, nb, type, row, b, word)) return;
     const int64_t e = blockIdx.y;
-    const uint8_t* src = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + word * 8;
+    const uint8_t* src = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + row_word_offset(type, word);
     uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
     // the blocks are only 2-byte aligned in general: go through 2-byte loads to stay correct for odd host strides
     const uint16_t* s16 = reinterpret_cast<const uint16_t*>(src);
-    if (type == kTypeQ6K && word == 26) {  // fp16 d, padded to four bytes
-        *reinterpret_cast<uint32_t*>(dst) = (uint32_t)s16[0];
+    if (scale_word(type, word)) {  // fp16 d (Q6_K: padded to four bytes)
+        if (type == kTypeQ6K) *reinterpret_cast<uint32_t*>(dst) = (uint32_t)s16[0];
+        else *reinterpret_cast<uint16_t*>(dst) = s16[0];
         return;
     }
     const uint64_t v = (uint64_t)s16[0] | ((uint64_t)s16[1] << 16) | ((uint64_t)s16[2] << 32) | ((uint64_t)s16[3] << 48);
@@ -67,10 +78,10 @@ __global__ void __launch_bounds__(256) untile_weights_kernel(const uint8_t* __re
     if (!decode_word(idx, rows, nb, type, row, b, word)) return;
     const int64_t e = blockIdx.y;
     const uint8_t* src = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
-    uint8_t* dst = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + word * 8;
+    uint8_t* dst = raw + (size_t)e * expert_bytes + (size_t)row * row_bytes + (size_t)b * block_bytes_of(type) + row_word_offset(type, word);
     uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
-    if (type == kTypeQ6K && word == 26) {
-        d16[0] = (uint16_t)*reinterpret_cast<const uint32_t*>(src);
+    if (scale_word(type, word)) {
+        d16[0] = *reinterpret_cast<const uint16_t*>(src);
         return;
     }
     const uint64_t v = stored_form(*reinterpret_cast<const uint64_t*>(src), type, word);
@@ -99,7 +110,19 @@ __global__ void __launch_bounds__(256) synth_weights_kernel(uint64_t seed, int64
     const uint64_t pos = flat_block * (uint64_t)words_per_block(type) + (uint64_t)word;
     uint64_t v = mix64(seed + (pos + 1) * kGamma);
     uint8_t* dst = tiled + (size_t)e * tiled_expert_bytes + word_in_tiles(row, b, nb, word, type);
-    if (type == kTypeQ6K) {  // d is the block's last field
+    if (type == kTypeQ80) {  // codes in [-127, 127] (ggml never writes -128), one d per 32 weights
+        if (word >= 32) {
+            *reinterpret_cast<uint16_t*>(dst) =
+                (uint16_t)unit_scale_f16(mix64((seed ^ kScaleStream) + (flat_block * 8 + (uint64_t)(word - 32) + 1) * kGamma));
+            return;
+        }
+        uint64_t fixed = 0;
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t byte = (v >> (8 * i)) & 0xffu;
+            fixed |= (byte == 0x80u ? 0x81ull : byte) << (8 * i);
+        }
+        v = fixed;
+    } else if (type == kTypeQ6K) {  // d is the block's last field
         if (word == 26) {
             *reinterpret_cast<uint32_t*>(dst) = unit_scale_f16(mix64((seed ^ kScaleStream) + (flat_block * 2 + 1) * kGamma));
             return;

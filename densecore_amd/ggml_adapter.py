@@ -23,6 +23,7 @@ EXPORTS = [
 ]
 
 GGML_TYPE_F32, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K, GGML_TYPE_I32 = 0, 12, 13, 14, 26
+GGML_TYPE_Q8_0 = 8
 GGML_OP_CUSTOM_PLACEHOLDER = 0  # the adapters never read dst->op
 
 
@@ -72,6 +73,8 @@ def tensor(array: np.ndarray, ggml_type: int, ne, nb=None, name: bytes = b"") ->
         if ggml_type in (GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K):
             bb = {GGML_TYPE_Q4_K: 144, GGML_TYPE_Q5_K: 176, GGML_TYPE_Q6_K: 210}[ggml_type]
             nb = [bb, bb * (ne[0] // 256)]
+        elif ggml_type == GGML_TYPE_Q8_0:
+            nb = [34, 34 * (ne[0] // 32)]
         else:
             nb = [4, 4 * ne[0]]
         while len(nb) < 4:

@@ -16,6 +16,7 @@ EXPORTS = [
 ]
 
 GGML_F32, GGML_F16, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_I32 = 0, 1, 12, 13, 14, 26
+GGML_Q8_0 = 8
 
 
 class TensorInfo(C.Structure):
@@ -97,7 +98,7 @@ class GgufFile:
         return self._load(name, "mq_gguf_load_q4k")
 
     def load_weight(self, name: str) -> "ops.Q4KWeight":
-        """Upload a GGML_TYPE_Q4_K, Q5_K or Q6_K tensor ([K, N] or [K, N, E]) to the GPU."""
+        """Upload a GGML_TYPE_Q4_K, Q5_K or Q6_K tensor ([K, N] or [K, N, E]) or a dense Q8_0 matrix to the GPU."""
         return self._load(name, "mq_gguf_load_weight")
 
     def _load(self, name: str, entry: str) -> "ops.Q4KWeight":

@@ -47,6 +47,14 @@ struct CachedWeight {
 std::mutex g_cache_mu;
 std::unordered_map<const void*, CachedWeight> g_cache;
 
+// A dense Q8_0 matrix (34-byte blocks of 32 weights, core/src/llm/matmul/q8_small_batch.h:9-14) whose rows hold
+// whole groups of 256 weights: the dense callback and the library entry take it, the MoE callbacks do not.
+constexpr size_t kQ80BlockBytes = 34;
+bool is_q80_matrix(const ggml_tensor* w) {
+    return w && w->data && (int)w->type == (int)GGML_TYPE_Q8_0 && w->ne[0] > 0 && w->ne[0] % kSuperBlock == 0 && w->ne[1] > 0 &&
+           w->ne[2] == 1 && w->ne[3] == 1 && w->nb[0] == kQ80BlockBytes && w->nb[1] >= (size_t)(w->ne[0] / 32) * kQ80BlockBytes;
+}
+
 // Q4_K, Q5_K or Q6_K rows of whole super-blocks (the K-quant weight types of the callbacks replaced:
 // core/src/llm/moe/native.cpp:2745-2752, core/src/backend/cpu_backend_moe_raw_batched.inl:1552)
 bool is_kquant_matrix(const ggml_tensor* w) {
@@ -164,7 +172,7 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
     const ggml_tensor* weight = dst->src[1];
     Options o = options_for(userdata, 1);
     if (!src || !weight || !src->data || !dst->data) return finish(o, MQ_ERR_INVALID);
-    if (!is_kquant_matrix(weight) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
+    if ((!is_kquant_matrix(weight) && !is_q80_matrix(weight)) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t k_in = weight->ne[0], n_out = weight->ne[1];
     const int64_t m = src->ne[1] * src->ne[2] * src->ne[3];
     // the reference leaves dst untouched on a shape mismatch (core/src/llm/matmul/gemv_exec.cpp:131-143)
@@ -314,10 +322,10 @@ int mq_matmul_ggml_quantized_transb(const float* a, int64_t m, int64_t k, int64_
                                     int32_t w_type_id, int64_t w_rows, int64_t w_cols, size_t w_row_bytes, float* c,
                                     int64_t ldc) {
     // rejection rules of MatMulGgmlQuantizedTransBWithPath
-    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K, Q5_K and Q6_K
+    // (core/src/backend/cpu_backend_quantized_matmul.cpp:150-163), narrowed to Q4_K, Q5_K, Q6_K and Q8_0
+    const size_t group_bytes = w_type_id == (int)GGML_TYPE_Q8_0 ? 8 * kQ80BlockBytes : kquant_block_bytes(w_type_id);
     if (!a || !w_data || !c || m <= 0 || w_rows <= 0 || w_cols <= 0 || k != w_cols || lda < k || ldc < w_rows ||
-        kquant_block_bytes(w_type_id) == 0 || w_cols % kSuperBlock != 0 ||
-        w_row_bytes != (size_t)(w_cols / kSuperBlock) * kquant_block_bytes(w_type_id)) {
+        group_bytes == 0 || w_cols % kSuperBlock != 0 || w_row_bytes != (size_t)(w_cols / kSuperBlock) * group_bytes) {
         note(MQ_ERR_INVALID);
         return 0;
     }

@@ -10,7 +10,7 @@
 #include <cstdint>
 
 extern "C" {
-enum ggml_type : int { GGML_TYPE_F32 = 0, GGML_TYPE_F16 = 1, GGML_TYPE_Q4_K = 12, GGML_TYPE_Q5_K = 13, GGML_TYPE_Q6_K = 14, GGML_TYPE_Q8_K = 15, GGML_TYPE_I32 = 26 };
+enum ggml_type : int { GGML_TYPE_F32 = 0, GGML_TYPE_F16 = 1, GGML_TYPE_Q8_0 = 8, GGML_TYPE_Q4_K = 12, GGML_TYPE_Q5_K = 13, GGML_TYPE_Q6_K = 14, GGML_TYPE_Q8_K = 15, GGML_TYPE_I32 = 26 };
 #define GGML_MAX_DIMS 4
 #define GGML_MAX_SRC 10
 #define GGML_MAX_OP_PARAMS 64

@@ -271,10 +271,11 @@ int load_kquant(const mq_gguf* g, const char* name, bool q4k_only, mq_weight** o
     const int64_t idx = mq_gguf_find_tensor(g, name);
     if (idx < 0) return fail(std::string("no tensor ") + name);
     const mq_gguf_tensor& t = g->tensors[(size_t)idx];
-    if (t.ggml_type != 12 && (q4k_only || (t.ggml_type != 13 && t.ggml_type != 14)))
-        return fail(std::string("tensor ") + name + (q4k_only ? " is not GGML_TYPE_Q4_K" : " is not of type Q4_K, Q5_K or Q6_K"));
+    if (t.ggml_type != 12 && (q4k_only || (t.ggml_type != 13 && t.ggml_type != 14 && t.ggml_type != 8)))
+        return fail(std::string("tensor ") + name + (q4k_only ? " is not GGML_TYPE_Q4_K" : " is not of type Q4_K, Q5_K, Q6_K or Q8_0"));
     if (t.n_dims > 3 || t.ne[3] != 1) return fail(std::string("tensor ") + name + " has more than three dimensions");
-    const size_t row_bytes = (size_t)(t.ne[0] / 256) * (t.ggml_type == 12 ? 144 : t.ggml_type == 13 ? 176 : 210);
+    // bytes of 256 weights of a row: one K-quant super-block, or eight Q8_0 blocks
+    const size_t row_bytes = (size_t)(t.ne[0] / 256) * (t.ggml_type == 12 ? 144 : t.ggml_type == 13 ? 176 : t.ggml_type == 14 ? 210 : 272);
     return mq_weight_upload_typed(t.ggml_type, t.data, t.ne[1], t.ne[0], t.ne[2], row_bytes, row_bytes * (size_t)t.ne[1], out);
 }
 }  // namespace

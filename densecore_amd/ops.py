@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .synth import BLOCK_BYTES, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K, Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
+from .synth import BLOCK_BYTES, GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K, GGML_TYPE_Q8_0, Q4K_BLOCK_BYTES, Q8K_BLOCK_BYTES, QK_K
 
 SILU_EXACT, SILU_FAST, SILU_FAST_FMA = 0, 1, 2
 ROUTE_FUSED, ROUTE_FLOOR, ROUTE_FLOOR_FINITE = 0, 1, 2
@@ -46,7 +46,7 @@ class Q4KWeight:
     @classmethod
     def from_ggml(cls, data: np.ndarray, cols: int, ggml_type: int = GGML_TYPE_Q4_K) -> "Q4KWeight":
         """data: uint8 [rows, row_bytes] or [n_experts, rows, row_bytes] in ggml block_q4_K (type 12),
-        block_q5_K (type 13) or block_q6_K (type 14) row layout."""
+        block_q5_K (type 13), block_q6_K (type 14) or -- dense matrices for mul_mat only -- Q8_0 (type 8) row layout."""
         a = np.ascontiguousarray(data, dtype=np.uint8)
         if a.ndim == 2:
             a = a[None]
@@ -100,14 +100,14 @@ def quantize_row_q8_k(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def mul_mat(w: Q4KWeight, x: torch.Tensor) -> torch.Tensor:
+def mul_mat(w: Q4KWeight, x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     """ggml_mul_mat(Q4_K w, F32 x): y[m, r] = w[r] . q8k(x[m]).  cb_gemv_custom / cb_gemv_batched_custom
     (core/src/llm/matmul/gemv_exec.cpp:99, batched_exec.cpp:55) and MatMulGgmlQuantizedTransB."""
     x = _f32(x)
     if x.dim() == 1:
         x = x[None]
     n = x.shape[0]
-    y = torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
+    y = out if out is not None else torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
     _lib.check(_lib.lib().mq_mul_mat_q4k(w._h, _ptr(x), n, x.stride(0), _ptr(y), w.rows, _stream()), "mq_mul_mat_q4k")
     return y
 
@@ -176,9 +176,10 @@ def mul_mat_host(w: Q4KWeight, x: np.ndarray) -> np.ndarray:
 
 def debug_block_sums(w: Q4KWeight, x: torch.Tensor):
     """Production matmul with its per-super-block integer sums written out:
-    (dot_scaled [rows, n, nb] int32, min_dot [rows, n, nb] int32, y [n, rows] fp32)."""
+    (dot_scaled [rows, n, nb] int32, min_dot [rows, n, nb] int32, y [n, rows] fp32).  Q8_0 weights: dot_scaled is
+    [rows, n, cols / 32], the integer sum of every 32-weight block, and min_dot stays zero."""
     x = _f32(x)
-    n, nb = x.shape[0], w.cols // QK_K
+    n, nb = x.shape[0], w.cols // (32 if w.ggml_type == GGML_TYPE_Q8_0 else QK_K)
     ds = torch.zeros((w.rows, n, nb), dtype=torch.int32, device=x.device)
     md = torch.zeros_like(ds)
     y = torch.empty((n, w.rows), dtype=torch.float32, device=x.device)

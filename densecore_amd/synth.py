@@ -27,7 +27,12 @@ Q8K_BLOCK_BYTES = 292
 GGML_TYPE_Q4_K = 12
 GGML_TYPE_Q5_K = 13
 GGML_TYPE_Q6_K = 14
-BLOCK_BYTES = {GGML_TYPE_Q4_K: Q4K_BLOCK_BYTES, GGML_TYPE_Q5_K: Q5K_BLOCK_BYTES, GGML_TYPE_Q6_K: Q6K_BLOCK_BYTES}
+GGML_TYPE_Q8_0 = 8
+Q80_BLOCK_BYTES = 34       # fp16 d + 32 int8 codes
+Q80_GROUP_BYTES = 8 * 34   # the eight blocks that cover 256 weights of a row
+# bytes of 256 weights of a row, per weight type
+BLOCK_BYTES = {GGML_TYPE_Q4_K: Q4K_BLOCK_BYTES, GGML_TYPE_Q5_K: Q5K_BLOCK_BYTES, GGML_TYPE_Q6_K: Q6K_BLOCK_BYTES,
+               GGML_TYPE_Q8_0: Q80_GROUP_BYTES}
 
 _GAMMA = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -115,6 +120,23 @@ def q6k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:
         raise ValueError("cols must be a multiple of 256")
     nb = cols // QK_K
     return q6k_blocks(seed, rows * nb).reshape(rows, nb * Q6K_BLOCK_BYTES)
+
+
+def q80_matrix(seed: int, rows: int, cols: int) -> np.ndarray:
+    """Row-major Q8_0 matrix ``[rows, cols/32 * 34]`` uint8 (ggml row layout).  Per 256 weights of a row: 40 stream
+    words, the first 32 of them the codes of the eight blocks in order (a byte 0x80 becomes 0x81: ggml's quantizer
+    never writes -128), and ``d = fp16(U(0.001, 0.01))`` per block from the scale stream."""
+    if cols % QK_K:
+        raise ValueError("cols must be a multiple of 256")
+    groups = rows * cols // QK_K
+    words = stream_u64(seed, 0, groups * 40).reshape(groups, 40)
+    codes = np.ascontiguousarray(words[:, :32]).view(np.uint8).reshape(groups, 8, 32).copy()
+    codes[codes == 0x80] = 0x81
+    raw = np.zeros((groups, 8, Q80_BLOCK_BYTES), np.uint8)
+    raw[:, :, 2:] = codes
+    sw = stream_u64(seed ^ 0x5CA1E5CA1E5CA1E5, 0, groups * 8).reshape(groups, 8)
+    raw[:, :, 0:2] = unit_scale_f16(sw).view(np.uint8).reshape(groups, 8, 2)
+    return raw.reshape(rows, cols // 32 * Q80_BLOCK_BYTES)
 
 
 def q4k_matrix(seed: int, rows: int, cols: int) -> np.ndarray:

@@ -73,12 +73,22 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
  * super-block (what mq_debug_block_sums returns as dot_scaled; min_dot is 0), one fused multiply-add per block.
  * Every product entry point accepts handles of any of the three types (gate and up of one call must share
  * theirs); the matrix-core GEMM (mq_gemm_q4k) and the one-launch decoder are Q4_K only, wide Q5_K / Q6_K
- * products run through the decode kernel in passes of 16 rows.  Other types: MQ_ERR_UNSUPPORTED. */
+ * products run through the decode kernel in passes of 16 rows.
+ * 8 = Q8_0 (fp16 d + 32 int8 codes, 34 bytes per 32 weights; core/src/llm/matmul/q8_small_batch.h:9-14): dense
+ * matrices only (n_experts == 1, cols % 256 == 0, row_bytes >= cols / 32 * 34), taken by mq_mul_mat_q4k (and
+ * mq_mul_mat_q4k_host, mq_debug_block_sums, the handle queries) and refused by every other entry point.  As in
+ * the reference the activations of such a product are quantized to Q8_0 too (vec_dot_type of the type,
+ * core/src/llm/matmul/batched_exec.cpp:630): d = amax / 127 per 32 values stored as fp16, codes =
+ * round-half-even(x * (127 / amax)) -- ggml's x86 quantizer, which is not part of the reference tree, so its
+ * parity is unpinned; y = sum over blocks of fp16(dx) * fp16(dy) * (integer dot), one fused multiply-add per block
+ * (Q8SmallBatchDot4, core/src/llm/matmul/q8_small_batch.h:29-77).  x rows must be 16-byte aligned.
+ * mq_debug_block_sums on such a handle writes dot_scaled as [rows][n][cols / 32], the integer dot of every block,
+ * and leaves min_dot (may be NULL) alone.  Other types: MQ_ERR_UNSUPPORTED. */
 int mq_weight_upload_typed(int ggml_type, const void* blocks_host, int64_t rows, int64_t cols, int64_t n_experts,
                            size_t row_bytes, size_t expert_bytes, mq_weight** out);
 int mq_weight_synthetic_typed(int ggml_type, uint64_t seed, int64_t rows, int64_t cols, int64_t n_experts,
                               mq_weight** out);
-int mq_weight_type(const mq_weight* w); /* 12, 13, or -1 for NULL */
+int mq_weight_type(const mq_weight* w); /* 12, 13, 14, 8, or -1 for NULL */
 /* Same tensor filled on the device from a 64-bit seed with the synthetic
  * recipe of densecore_amd/synth.py (byte-identical to uploading
  * synth.q4k_matrix(seed, rows*n_experts, cols)); for multi-GB benchmark sets. */

@@ -53,8 +53,9 @@ int mq_gguf_get_string(const mq_gguf* g, const char* key, const char** out, size
 /* Uploads tensor `name` (GGML_TYPE_Q4_K; 2-D [K, N] -> one matrix of N rows, 3-D [K, N, E] -> an expert
  * stack) with mq_weight_upload.  mq_init must have been called. */
 int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out);
-/* The same for a tensor of any type the product entry points multiply: GGML_TYPE_Q4_K, Q5_K or Q6_K
- * (mq_weight_upload_typed).  A Q4_K_M file stores part of its down projections as Q5_K or Q6_K. */
+/* The same for a tensor of any type the product entry points multiply: GGML_TYPE_Q4_K, Q5_K or Q6_K, or a
+ * dense (2-D) Q8_0 matrix (mq_weight_upload_typed).  A Q4_K_M file stores part of its down projections as Q5_K or
+ * Q6_K. */
 int mq_gguf_load_weight(const mq_gguf* g, const char* name, mq_weight** out);
 
 #ifdef __cplusplus

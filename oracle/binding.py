@@ -68,6 +68,9 @@ def lib() -> C.CDLL:
         L.orc_dot_q5k_q8k.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.orc_dot_dequant_q5k_f64.restype = C.c_double
         L.orc_dot_dequant_q5k_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+        L.orc_q80_block_bytes.restype = C.c_size_t
+        L.orc_dot_dequant_q80_f64.restype = C.c_double
+        L.orc_dot_dequant_q80_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         _lib = L
     return _lib
 
@@ -300,6 +303,60 @@ def q6k_dot_dequant_f64(w: np.ndarray, cols: int, q8: np.ndarray, magnitude: boo
 
 
 # ---------------------------------------------------------------- FFN / router / MoE
+# ---------------------------------------------------------------- Q8_0 weights (activations Q8_0 as well)
+Q80 = 34
+Q80_X86, Q80_SCALAR = 0, 1  # the two published forms of ggml's Q8_0 activation quantizer (parity unpinned)
+
+
+def quantize_rows_q80(x: np.ndarray, variant: int = Q80_X86) -> np.ndarray:
+    """fp32 [n, cols] -> uint8 [n, cols/32*34] Q8_0 rows."""
+    x = _c(x, np.float32)
+    n, cols = x.shape
+    out = np.zeros((n, cols // 32 * Q80), np.uint8)
+    rc = lib().orc_quantize_rows_q80(_p(x), C.c_int64(n), C.c_int64(cols), _p(out), C.c_int64(cols), C.c_int(variant))
+    if rc:
+        raise ValueError(f"orc_quantize_rows_q80 rc={rc}")
+    return out
+
+
+def q80_matrix_block_sums(w: np.ndarray, cols: int, q: np.ndarray) -> np.ndarray:
+    """w uint8 [rows, cols/32*34], q uint8 [n, cols/32*34] -> int32 [rows, n, cols/32]."""
+    w = _c(w, np.uint8)
+    q = _c(q, np.uint8)
+    rows, n = w.shape[0], q.shape[0]
+    out = np.zeros((rows, n, cols // 32), np.int32)
+    rc = lib().orc_q80_matrix_block_sums(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q),
+                                         C.c_int64(n), C.c_size_t(q.shape[1]), _p(out))
+    if rc:
+        raise ValueError(f"orc_q80_matrix_block_sums rc={rc}")
+    return out
+
+
+def mul_mat_q80_q80(w: np.ndarray, cols: int, q: np.ndarray, order: int = ORDER_DOTPROD) -> np.ndarray:
+    """-> fp32 [n, rows]; ORDER_HWY is the reference's eight-lane kernel, anything else the per-block form."""
+    w = _c(w, np.uint8)
+    q = _c(q, np.uint8)
+    rows, n = w.shape[0], q.shape[0]
+    out = np.zeros((n, rows), np.float32)
+    rc = lib().orc_mul_mat_q80_q80(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q),
+                                   C.c_int64(n), C.c_size_t(q.shape[1]), _p(out), C.c_int64(rows), C.c_int(order))
+    if rc:
+        raise ValueError(f"orc_mul_mat_q80_q80 rc={rc}")
+    return out
+
+
+def q80_dot_dequant_f64(w: np.ndarray, cols: int, q: np.ndarray, magnitude: bool = False) -> np.ndarray:
+    w = _c(w, np.uint8)
+    q = _c(q, np.uint8)
+    L = lib()
+    out = np.zeros((q.shape[0], w.shape[0]), np.float64)
+    for m in range(q.shape[0]):
+        for r in range(w.shape[0]):
+            out[m, r] = L.orc_dot_dequant_q80_f64(C.c_void_p(w[r].ctypes.data), C.c_void_p(q[m].ctypes.data),
+                                                  C.c_int64(cols), C.c_int(int(magnitude)))
+    return out
+
+
 def ffn_swiglu(gate, up, down, hidden: int, inter: int, x, order=ORDER_DOTPROD, silu=SILU_FAST_FMA,
                want_inter=False):
     gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)

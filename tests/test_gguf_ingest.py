@@ -135,3 +135,27 @@ def test_q4k_tensors_upload_and_multiply(tmp_path):
     got = ops.mul_mat(w2, torch.from_numpy(x).cuda()).cpu().numpy()
     assert_fp32_parity(got, orc.mul_mat_q4k_q8k(q2, 512, q8, orc.ORDER_AVX2), orc.dot_magnitude_f64(q2, 512, q8))
     w2.free(), w3.free()
+
+
+@pytest.mark.gpu
+def test_q80_tensor_uploads_and_multiplies(tmp_path):
+    """A dense Q8_0 matrix (e.g. the output head of a mixed-precision file) through the same loader."""
+    import torch
+    from densecore_amd import ops
+    from oracle import binding as orc
+    from tests._parity import assert_fp32_parity
+    q80 = synth.q80_matrix(50, 24, 512)                                     # [K=512, N=24], Q8_0
+    path = str(tmp_path / "q80.gguf")
+    gguf.write_gguf(path, {"general.architecture": ("str", "qwen35moe")},
+                    [("output.weight", gguf.GGML_Q8_0, [512, 24], q80)])
+    with gguf.GgufFile(path) as g:
+        assert g.tensors()[0]["type"] == 8 and g.tensors()[0]["nbytes"] == 24 * 16 * 34
+        w = g.load_weight("output.weight")
+        with pytest.raises(Exception):
+            g.load_q4k("output.weight")
+    assert (w.rows, w.cols, w.n_experts, w.ggml_type) == (24, 512, 1, 8) and np.array_equal(w.to_ggml(), q80)
+    x = synth.normal_f32(51, (3, 512))
+    q = orc.quantize_rows_q80(x)
+    assert_fp32_parity(ops.mul_mat(w, torch.from_numpy(x).cuda()).cpu().numpy(), orc.mul_mat_q80_q80(q80, 512, q),
+                       orc.q80_dot_dequant_f64(q80, 512, q, magnitude=True))
+    w.free()

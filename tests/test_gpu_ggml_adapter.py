@@ -169,6 +169,27 @@ def test_dense_node_and_library_matmul_with_q6k_weights(ga):
     assert np.array_equal(c.view(np.uint32), out.view(np.uint32))
 
 
+def test_dense_node_and_library_matmul_with_q80_weights(ga):
+    """Q8_0 rows (34-byte blocks of 32; the reference's kernel for the type is core/src/llm/matmul/q8_small_batch.h);
+    the activations are quantized to Q8_0 as the reference's vec_dot_type asks."""
+    rows, cols, m = 80, 1024, 3
+    w = synth.q80_matrix(2250, rows, cols)
+    x = synth.normal_f32(2251, (m, cols))
+    out = np.zeros((m, rows), np.float32)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q8_0, [cols, rows])
+    tx = ga.tensor(x, ga.GGML_TYPE_F32, [cols, m])
+    to = ga.tensor(out, ga.GGML_TYPE_F32, [rows, m])
+    ga.set_src(to, tx, tw)
+    ga.lib().mq_cb_gemv_batched_custom(C.byref(to), 0, 1, None)
+    assert ga.lib().mq_ggml_last_status() == 0
+    q = orc.quantize_rows_q80(x)
+    assert_fp32_parity(out, orc.mul_mat_q80_q80(w, cols, q), orc.q80_dot_dequant_f64(w, cols, q, magnitude=True))
+    c = np.zeros((m, rows), np.float32)
+    assert ga.lib().mq_matmul_ggml_quantized_transb(x.ctypes.data, m, cols, cols, w.ctypes.data, ga.GGML_TYPE_Q8_0, rows,
+                                                    cols, 34 * (cols // 32), c.ctypes.data, rows) == 1
+    assert np.array_equal(c.view(np.uint32), out.view(np.uint32))
+
+
 def test_library_level_matmul(ga):
     m, rows, cols = 7, 384, 768
     w = synth.q4k_matrix(301, rows, cols)
@@ -178,6 +199,6 @@ def test_library_level_matmul(ga):
                                                   cols, 144 * (cols // 256), c.ctypes.data, rows)
     assert ok == 1
     assert_fp32_parity(c, _dense_ref(w, cols, a), orc.dot_magnitude_f64(w, cols, orc.quantize_rows_q8k(a)))
-    # a type other than Q4_K, Q5_K and Q6_K is rejected like an unsupported ggml type
+    # a type other than Q4_K, Q5_K, Q6_K and Q8_0 is rejected like an unsupported ggml type
     assert ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, 2, rows, cols,
                                                     144 * (cols // 256), c.ctypes.data, rows) == 0

@@ -599,3 +599,87 @@ def test_q6k_fp32_orders_against_double(cols):
         assert np.max(np.abs(got - ref) / mag) < 2e-6
         ok = np.abs(ref) > 1e-3 * mag
         assert np.max(np.abs(got - ref)[ok] / np.abs(ref)[ok]) < 1e-4
+
+
+# ---------------------------------------------------------------- Q8_0 x Q8_0 (core/src/llm/matmul/q8_small_batch.h)
+def np_unpack_q80(rows_u8: np.ndarray):
+    """-> (d float64 [rows, blocks], codes int64 [rows, blocks, 32]) by an independent numpy decode."""
+    b = rows_u8.reshape(rows_u8.shape[0], -1, 34)
+    d = np.ascontiguousarray(b[:, :, 0:2]).view(np.float16)[..., 0].astype(np.float64)
+    return d, np.ascontiguousarray(b[:, :, 2:]).view(np.int8).astype(np.int64)
+
+
+def test_q80_layout_sums_brute_force_and_closed_forms():
+    assert orc.lib().orc_q80_block_bytes() == 34                      # q8_small_batch.h:13-14
+    cols = 1024
+    w = synth.q80_matrix(801, 10, cols)
+    q = orc.quantize_rows_q80(synth.normal_f32(802, (3, cols)))
+    _, wq = np_unpack_q80(w)
+    _, yq = np_unpack_q80(q)
+    assert wq.min() == -127 and wq.max() == 127
+    assert np.array_equal(orc.q80_matrix_block_sums(w, cols, q), np.einsum("rbi,mbi->rmb", wq, yq))
+    # all codes one -> the block sum is the sum of the activation codes; a single non-zero pair -> its product
+    ones = w.reshape(10, -1, 34).copy()
+    ones[:, :, 2:] = 1
+    assert np.array_equal(orc.q80_matrix_block_sums(ones.reshape(10, -1), cols, q),
+                          np.broadcast_to(yq.sum(-1)[None], (10, 3, cols // 32)))
+    rng = np.random.default_rng(8)
+    for _ in range(100):
+        e, a, b = int(rng.integers(0, 256)), int(rng.integers(-127, 128)), int(rng.integers(-127, 128))
+        wr, qr = np.zeros((1, 8 * 34), np.uint8), np.zeros((1, 8 * 34), np.uint8)
+        wr[0, (e // 32) * 34 + 2 + e % 32] = np.int8(a).view(np.uint8)
+        qr[0, (e // 32) * 34 + 2 + e % 32] = np.int8(b).view(np.uint8)
+        got = orc.q80_matrix_block_sums(wr, 256, qr)[0, 0]
+        assert got[e // 32] == a * b and got.sum() == a * b
+
+
+@pytest.mark.parametrize("cols", [256, 2048])
+def test_q80_fp32_orders_against_double(cols):
+    w = synth.q80_matrix(811 + cols, 24, cols)
+    q = orc.quantize_rows_q80(synth.normal_f32(812 + cols, (3, cols)))
+    wd, wq = np_unpack_q80(w)
+    yd, yq = np_unpack_q80(q)
+    want = (yd[..., None] * yq).reshape(3, cols) @ (wd[..., None] * wq).reshape(24, cols).T
+    ref = orc.q80_dot_dequant_f64(w, cols, q)
+    assert np.allclose(ref, want, rtol=1e-12, atol=1e-12)
+    mag = orc.q80_dot_dequant_f64(w, cols, q, magnitude=True)
+    for order in (orc.ORDER_HWY, orc.ORDER_DOTPROD):
+        got = orc.mul_mat_q80_q80(w, cols, q, order).astype(np.float64)
+        assert np.max(np.abs(got - ref) / mag) < 2e-6
+        ok = np.abs(ref) > 1e-3 * mag
+        assert np.max(np.abs(got[ok] - ref[ok]) / np.abs(ref[ok])) < 1e-4
+
+
+@pytest.mark.parametrize("variant", [orc.Q80_X86, orc.Q80_SCALAR])
+def test_q80_activation_quantizer_invariants(variant):
+    """ggml's Q8_0 quantizer is third-party code the reference tree does not carry (parity unpinned): what is
+    checked is what either published form must satisfy."""
+    x = synth.normal_f32(821, (5, 512))
+    x[1] = 0.0
+    x[2, 64:96] = 0.0
+    x[3] *= np.float32(300.0)
+    q = orc.quantize_rows_q80(x, variant)
+    d, codes = np_unpack_q80(q)
+    xb = x.reshape(5, 16, 32).astype(np.float64)
+    amax = np.abs(xb).max(-1)
+    assert np.abs(codes).max() <= 127
+    assert not q[1].any() and not codes[2, 2].any() and d[2, 2] == 0.0
+    live = amax > 0
+    first = np.abs(xb).argmax(-1)
+    extreme = np.take_along_axis(codes, first[..., None], -1)[..., 0]
+    assert np.all(np.abs(extreme[live]) == 127)                          # the extreme element maps to +-127
+    assert np.all(np.sign(extreme[live]) == np.sign(np.take_along_axis(xb, first[..., None], -1)[..., 0][live]))
+    d32 = (amax / 127.0).astype(np.float32)
+    assert np.array_equal(d.astype(np.float16), d32.astype(np.float16))  # stored scale = fp16(amax / 127)
+    # reconstruction with the unrounded scale within half a step (plus fp32 rounding of the product)
+    assert np.all(np.abs(codes * d32[..., None].astype(np.float64) - xb) <= 0.5 * d32[..., None] * (1 + 1e-5))
+    qn = orc.quantize_rows_q80(-x, variant)                                 # sign symmetry
+    dn, cn = np_unpack_q80(qn)
+    assert np.array_equal(cn, -codes) and np.array_equal(dn, d)
+
+
+def test_q80_quantizer_variants_differ_only_at_ties():
+    x = synth.normal_f32(831, (4, 1024))
+    a = np_unpack_q80(orc.quantize_rows_q80(x, orc.Q80_X86))[1]
+    b = np_unpack_q80(orc.quantize_rows_q80(x, orc.Q80_SCALAR))[1]
+    assert np.abs(a - b).max() <= 1 and np.mean(a != b) < 1e-3
