@@ -30,10 +30,10 @@ RING = 8
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0          # dense int8 MFMA, MI355X
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
-# `bench.py --kernel-only`: 32,507.8 KiB fetched and 210.0 KiB written per dispatch on average, each scaled by what
+# `bench.py --kernel-only`: 32,524.6 KiB fetched and 210.0 KiB written per dispatch on average, each scaled by what
 # the same counter reads for the 256 MiB copy of `bench.py --copy-calibration` (FETCH_SIZE 131,083.8 KiB -> x2.000,
-# WRITE_SIZE 262,144.0 KiB -> x1.000): 66,570,000 B read + 215,000 B written.
-TRAFFIC_BYTES_PER_LAUNCH = 66785000
+# WRITE_SIZE 262,144.0 KiB -> x1.000): 66,610,000 B read + 215,000 B written.
+TRAFFIC_BYTES_PER_LAUNCH = 66825000
 Q4K_MATRIX_BYTES = INTER * (HIDDEN // 256) * 144          # 33,030,144: the same for gate, up and down
 
 
