@@ -288,8 +288,19 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
     const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
     float gate = 1.0f;
     if (has_shared && sh_gate_inp) {
+        // thread j takes columns j, j + 256, ... in turn; the operands are requested eight columns at a time so that
+        // their latencies overlap instead of adding up
+        const float* xr = x + tok * rows;
         float acc = 0.0f;
-        for (int64_t c = threadIdx.x; c < rows; c += 256) acc = fmaf(sh_gate_inp[c], x[tok * rows + c], acc);
+        int64_t c = threadIdx.x;
+        for (; c + 7 * 256 < rows; c += 8 * 256) {
+            float ga[8], xa[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ga[u] = sh_gate_inp[c + u * 256], xa[u] = xr[c + u * 256];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = fmaf(ga[u], xa[u], acc);
+        }
+        for (; c < rows; c += 256) acc = fmaf(sh_gate_inp[c], xr[c], acc);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
         if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = acc;
@@ -297,14 +308,26 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
         gate = stable_sigmoid((wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]));
     }
     if (r >= rows) return;
-    float acc = 0.0f;
-    for (int k = 0; k < top_k; ++k) {
-        const int e = ids[tok * top_k + k];
-        const float w = weights[tok * top_k + k];
-        if (e < 0 || e >= n_experts || w == 0.0f) continue;
-        acc = __fadd_rn(acc, __fmul_rn(part[(tok * slots + k) * rows + r], w));
+    // every partial row is requested before the first is added (a dropped slot's row may hold anything: it is read
+    // and thrown away), then the sum runs in routing order as before
+    float pv[9], wk[8];
+    bool live[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        live[k] = false;
+        if (k < top_k) {
+            const int e = ids[tok * top_k + k];
+            wk[k] = weights[tok * top_k + k];
+            live[k] = e >= 0 && e < n_experts && wk[k] != 0.0f;
+            pv[k] = part[(tok * slots + k) * rows + r];
+        }
     }
-    if (has_shared) acc = __fadd_rn(acc, __fmul_rn(part[(tok * slots + top_k) * rows + r], gate));
+    if (has_shared) pv[8] = part[(tok * slots + top_k) * rows + r];
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        if (live[k]) acc = __fadd_rn(acc, __fmul_rn(pv[k], wk[k]));
+    if (has_shared) acc = __fadd_rn(acc, __fmul_rn(pv[8], gate));
     y[tok * rows + r] = acc;
 }
 
@@ -375,6 +398,7 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
 hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots, int64_t rows, const float* weights,
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,
                               const float* x, float* y, hipStream_t stream) {
+    if (top_k < 0 || top_k > 8) return hipErrorInvalidValue;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((rows + 255) / 256), (unsigned)n), dim3(256), 0, stream, part,
                        top_k, slots, rows, weights, ids, (int)n_experts, has_shared, sh_gate_inp, x, y);
     return hipGetLastError();
