@@ -313,8 +313,9 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
         if (threadIdx.x == 0) {
             uint32_t* c = p.out_counters + (size_t)blockIdx.y * out_nb + hb;
             const uint32_t prev = atomicAdd(c, 1u);
-            is_last = prev == 15u;
-            if (prev == 15u) atomicExch(c, 0u);  // leave the counters zero for the next launch
+            const uint32_t last = (uint32_t)(16 / rt_per_wg - 1);  // a 256-row block is 16 row tiles, rt_per_wg of them per workgroup
+            is_last = prev == last;
+            if (prev == last) atomicExch(c, 0u);  // leave the counters zero for the next launch
         }
         __syncthreads();
         if (is_last) {
@@ -376,12 +377,24 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int waves = pick_waves(a.nb, rowtiles * groups);
     // Short rows (few super-blocks) in one-wave workgroups: let a workgroup stream several row tiles, so that
     // its look-ups and activation addressing are paid once per ~16 tiles rather than once per row tile.
+    // Expert-grouped launches with up to twice the one-wave workgroups the chip holds at once (8 per compute unit):
+    // the ones left over would start when the first ones end and pay their look-ups a second time, so a workgroup
+    // takes twice the row tiles and one round holds them all (measured on the gate/up launch: 73 -> 68 us for the
+    // MoE block at 16 tokens, 2-3 us at 32 and 48; on the down launch, whose workgroups already take eight row
+    // tiles, it loses, and fewer, longer workgroups than that lose at every width).  With the fused output quantization a workgroup must stay inside one 256-row block (16 row tiles).
     MatmulArgs b = a;
     b.rt_per_wg = 1;
-    if (waves == 1 && !debug && !a.out_aq) {
+    if (waves == 1 && !debug) {
         int64_t want = 16 / (a.nb * nmat);
-        while (want > 1 && rowtiles % want) --want;  // an even split keeps the last workgroup full
-        b.rt_per_wg = (int)(want > 1 ? want : 1);
+        if (want < 1) want = 1;
+        const int64_t resident = 2048, workgroups = rowtiles * groups / want;
+        if (a.grouped && nmat == 2 && workgroups > resident && workgroups <= 2 * resident + resident / 8 && want < 16) want *= 2;
+        if (a.out_aq) {
+            while (want > 1 && ((want & (want - 1)) || want > 16)) --want;  // a power of two up to 16 (rows % 256 == 0)
+        } else {
+            while (want > 1 && rowtiles % want) --want;  // an even split keeps the last workgroup full
+        }
+        b.rt_per_wg = (int)want;
     }
     const dim3 grid((unsigned)(rowtiles / b.rt_per_wg), (unsigned)groups);
 
