@@ -28,6 +28,7 @@
 #include <cstdlib>
 
 #include <hip/hip_ext.h>
+#include <cmath>
 
 #include "common.h"
 #include "kernels.h"
@@ -377,18 +378,27 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int waves = pick_waves(a.nb, rowtiles * groups);
     // Short rows (few super-blocks) in one-wave workgroups: let a workgroup stream several row tiles, so that
     // its look-ups and activation addressing are paid once per ~16 tiles rather than once per row tile.
-    // Expert-grouped launches with up to twice the one-wave workgroups the chip holds at once (8 per compute unit):
-    // the ones left over would start when the first ones end and pay their look-ups a second time, so a workgroup
-    // takes twice the row tiles and one round holds them all (measured on the gate/up launch: 73 -> 68 us for the
-    // MoE block at 16 tokens, 2-3 us at 32 and 48; on the down launch, whose workgroups already take eight row
-    // tiles, it loses, and fewer, longer workgroups than that lose at every width).  With the fused output quantization a workgroup must stay inside one 256-row block (16 row tiles).
+    // Expert-grouped gate/up with more one-wave workgroups than the chip holds at once (8 per compute unit): the ones
+    // left over start when the first ones end and pay their group look-ups again, so a workgroup takes two row
+    // tiles, four when even that leaves more than three rounds (measured, MoE block of 256 experts, top-8: 73 -> 68 us
+    // at 16 tokens, 100 -> 97 at 32, 143 -> 137 at 64; more row tiles than that leave too few wavefronts, and the
+    // down launch, whose workgroups already take eight row tiles, loses with any more).  The number of groups is
+    // only known on the device; its expectation for uniform routing stands in.  With the fused output quantization
+    // a workgroup must stay inside one 256-row block (16 row tiles).
     MatmulArgs b = a;
     b.rt_per_wg = 1;
     if (waves == 1 && !debug) {
         int64_t want = 16 / (a.nb * nmat);
         if (want < 1) want = 1;
-        const int64_t resident = 2048, workgroups = rowtiles * groups / want;
-        if (a.grouped && nmat == 2 && workgroups > resident && workgroups <= 2 * resident + resident / 8 && want < 16) want *= 2;
+        if (a.grouped && nmat == 2 && want == 1) {
+            double expect = (double)a.max_groups;
+            if (!a.direct_ids && a.n_experts > 0 && a.direct_top_k > 0)
+                expect = (double)a.n_experts * (1.0 - std::pow(1.0 - 1.0 / (double)a.n_experts, (double)(a.n * a.direct_top_k)));
+            const double workgroups = (double)rowtiles * (expect + (double)(groups - a.max_groups));
+            const double resident = 2048.0;
+            if (workgroups > 3.5 * resident) want = 4;
+            else if (workgroups > resident) want = 2;
+        }
         if (a.out_aq) {
             while (want > 1 && ((want & (want - 1)) || want > 16)) --want;  // a power of two up to 16 (rows % 256 == 0)
         } else {
