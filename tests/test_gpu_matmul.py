@@ -57,6 +57,26 @@ def test_matmul_integer_sums_exact_and_fp32_within_tolerance(ops, rows, cols, n)
         assert_fp32_parity(y, ref, mag, f"order={name}")
 
 
+@pytest.mark.parametrize("gtype", [synth.GGML_TYPE_Q4_K, synth.GGML_TYPE_Q5_K, synth.GGML_TYPE_Q6_K])
+@pytest.mark.parametrize("rows,cols", [(17, 2304), (100, 5120), (1000, 14336), (4097, 4608), (48, 28672)])
+def test_single_row_with_quantizer_inside_equals_the_two_launches(ops, rows, cols, gtype):
+    """One activation row against long weight rows runs with the quantizer inside the decode kernel and without
+    the lane's second activation row: the bits of quantize followed by the product from Q8_K rows, and the debug
+    launch (the two-row arithmetic) too; ragged row counts take the several-row-tiles-per-workgroup path."""
+    import torch
+    make = {synth.GGML_TYPE_Q4_K: synth.q4k_matrix, synth.GGML_TYPE_Q5_K: synth.q5k_matrix, synth.GGML_TYPE_Q6_K: synth.q6k_matrix}[gtype]
+    w_np = make(synth.tensor_seed("xq-w", rows, cols, gtype), rows, cols)
+    x = synth.normal_f32(synth.tensor_seed("xq-x", rows, cols), (1, cols))
+    w = ops.Q4KWeight.from_ggml(w_np, cols, gtype)
+    xd = torch.from_numpy(x).cuda()
+    y = ops.mul_mat(w, xd).cpu().numpy()
+    y_two = ops.mul_mat_q8k(w, ops.quantize_row_q8_k(xd)).cpu().numpy()
+    _, _, y_dbg = ops.debug_block_sums(w, xd)
+    assert np.array_equal(y.view(np.uint32), y_two.view(np.uint32))
+    assert np.array_equal(y.view(np.uint32), y_dbg.cpu().numpy().view(np.uint32))
+    w.free()
+
+
 def test_matmul_zero_and_constant_activations(ops):
     rows, cols = 64, 1024
     w = synth.q4k_matrix(5, rows, cols)
