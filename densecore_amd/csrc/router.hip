@@ -124,16 +124,30 @@ __global__ void __launch_bounds__(64) weights_from_ids_kernel(const float* __res
 // (token, k) order inside an expert, which is the (expert, token, k) order of
 // core/src/llm/moe/native.cpp:1726-1730.  Experts nobody selected produce no group.
 // ids may live in LDS or in global memory; count[] is n_experts ints of LDS.
+// token_mask (LDS, n_experts * mask_words + 1 words, or null): one bit per (expert, token).  A pair's place inside
+// its group is the number of earlier pairs of the same expert; when no token names an expert twice (always so for
+// routed ids) that is the number of earlier tokens whose bit is set -- a population count instead of a scan over
+// all earlier pairs.  A repeated (expert, token) raises the word after the masks and the scan is used.
 __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries, int top_k, int n_experts,
                                               int32_t* count, int32_t* __restrict__ group_expert,
                                               int32_t* __restrict__ group_begin, int32_t* __restrict__ n_groups,
-                                              int32_t* __restrict__ entry_token, int32_t* __restrict__ entry_k) {
+                                              int32_t* __restrict__ entry_token, int32_t* __restrict__ entry_k,
+                                              uint32_t* token_mask = nullptr, int mask_words = 0) {
     const int tid = threadIdx.x, nt = blockDim.x;
     for (int e = tid; e < n_experts; e += nt) count[e] = 0;
+    if (token_mask)
+        for (int w = tid; w <= n_experts * mask_words; w += nt) token_mask[w] = 0u;
     __syncthreads();
     for (int i = tid; i < n_entries; i += nt) {
         const int e = ids[i];
-        if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+        if (e >= 0 && e < n_experts) {
+            atomicAdd(&count[e], 1);
+            if (token_mask) {
+                const int t = i / top_k;
+                const uint32_t bit = 1u << (t & 31);
+                if (atomicOr(&token_mask[e * mask_words + (t >> 5)], bit) & bit) token_mask[n_experts * mask_words] = 1u;
+            }
+        }
     }
     __syncthreads();
     if (tid < 64) {  // wave 0: exclusive scan over the experts, lane l covers a run of consecutive experts
@@ -179,11 +193,19 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
         }
     }
     __syncthreads();
+    const bool by_mask = token_mask && token_mask[n_experts * mask_words] == 0u;
     for (int i = tid; i < n_entries; i += nt) {
         const int e = ids[i];
         if (e < 0 || e >= n_experts) continue;
         int rank = 0;  // earlier pairs routed to the same expert
         int j = 0;
+        if (by_mask) {
+            const int t = i / top_k;
+            const uint32_t* m = token_mask + e * mask_words;
+            for (int w = 0; w < (t >> 5); ++w) rank += __popc(m[w]);
+            rank += __popc(m[t >> 5] & ((1u << (t & 31)) - 1u));
+            j = i;  // nothing left to scan
+        }
         for (; j + 16 <= i; j += 16) {
             int v16[16];
 #pragma unroll
@@ -199,13 +221,13 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
 }
 
 __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __restrict__ ids, int n_entries,
-                                                            int top_k, int n_experts, int use_lds,
+                                                            int top_k, int n_experts, int use_lds, int mask_words,
                                                             int32_t* __restrict__ group_expert,
                                                             int32_t* __restrict__ group_begin,
                                                             int32_t* __restrict__ n_groups,
                                                             int32_t* __restrict__ entry_token,
                                                             int32_t* __restrict__ entry_k) {
-    extern __shared__ int32_t sh[];  // [n_experts] counts -> offsets, then [n_entries] ids when they fit
+    extern __shared__ int32_t sh[];  // [n_experts] counts -> offsets, [n_entries] ids when they fit, then the token masks
     int32_t* count = sh;
     const int32_t* src = ids;
     if (use_lds) {
@@ -213,7 +235,8 @@ __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __res
         for (int i = threadIdx.x; i < n_entries; i += blockDim.x) ids_s[i] = ids[i];
         src = ids_s;  // the barrier inside group_entries orders these stores
     }
-    group_entries(src, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k);
+    group_entries(src, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
+                  mask_words ? reinterpret_cast<uint32_t*>(sh + n_experts + (use_lds ? n_entries : 0)) : nullptr, mask_words);
 }
 
 // Router and grouping in one launch (decode widths): a workgroup per token routes it; the last
@@ -229,7 +252,7 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
                                                               int32_t* __restrict__ n_groups,
                                                               int32_t* __restrict__ entry_token,
                                                               int32_t* __restrict__ entry_k, int build_groups,
-                                                              int route_blocks,
+                                                              int route_blocks, int mask_words,
                                                               const float* __restrict__ qx, int64_t q_ldx, int64_t q_nb,
                                                               uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
     if ((int)blockIdx.x >= route_blocks) {
@@ -272,7 +295,8 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
     const int n_entries = n * top_k;
     for (int i = threadIdx.x; i < n_entries; i += 256)
         ids_s[i] = solo ? ids[i] : __hip_atomic_load(ids + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    group_entries(ids_s, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k);
+    group_entries(ids_s, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
+                  mask_words ? reinterpret_cast<uint32_t*>(ids_s + n_entries) : nullptr, mask_words);
 }
 
 // grid = (ceil(rows/256), n).  Routed experts are added in routing order k = 0..top_k-1
@@ -363,9 +387,12 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     if (entries > (int64_t)1 << 30 || n_experts > 8192) return hipErrorInvalidValue;
     const int threads = entries >= 1024 ? 1024 : (entries > 256 ? 512 : 256);
     const int use_lds = entries <= 8192;
-    const size_t lds = (size_t)n_experts * 4 + (use_lds ? (size_t)entries * 4 : 0);
+    size_t lds = (size_t)n_experts * 4 + (use_lds ? (size_t)entries * 4 : 0);
+    int mask_words = n <= 256 ? (int)((n + 31) / 32) : 0;  // one bit per (expert, token) when that fits
+    if (lds + ((size_t)n_experts * mask_words + 1) * 4 > 60 * 1024) mask_words = 0;
+    if (mask_words) lds += ((size_t)n_experts * mask_words + 1) * 4;
     hipLaunchKernelGGL(build_groups_kernel, dim3(1), dim3(threads), lds, stream, ids, (int)entries, top_k,
-                       (int)n_experts, use_lds, group_expert, group_begin, n_groups, entry_token, entry_k);
+                       (int)n_experts, use_lds, mask_words, group_expert, group_begin, n_groups, entry_token, entry_k);
     return hipGetLastError();
 }
 
@@ -375,7 +402,11 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
                                   const float* qx, int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
     const size_t lds_route = (size_t)n_experts * 8 + 64;
-    const size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
+    // one bit per (expert, token) for the grouping, up to 256 tokens
+    int mask_words = n <= 256 ? (int)((n + 31) / 32) : 0;
+    size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
+    if (lds_group + ((size_t)n_experts * mask_words + 1) * 4 > 60 * 1024) mask_words = 0;  // no room: the grouping scans instead
+    if (mask_words) lds_group += ((size_t)n_experts * mask_words + 1) * 4;
     if (lds_group > 60 * 1024) {  // prefill widths: route, then group from global memory, quantize on its own
         hipError_t e = launch_route_topk(logits, n_experts, n, top_k, mode, ids, weights, stream);
         if (e != hipSuccess) return e;
@@ -390,7 +421,7 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
     hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(256),
                        lds_route > lds_group ? lds_route : lds_group, stream, logits, (int)n_experts, (int)n, top_k, mode,
                        ids, weights, arrivals, group_expert, group_begin, n_groups, entry_token, entry_k, build_groups ? 1 : 0,
-                       route_blocks, qx,
+                       route_blocks, mask_words, qx,
                        q_ldx, q_nb, q_aq, q_ad);
     return hipGetLastError();
 }

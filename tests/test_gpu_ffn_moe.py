@@ -152,6 +152,7 @@ def test_mul_mat_id_matches_per_pair_dense_results(ops, n):
     if n >= 4:
         ids[1, 2] = -1        # invalid ids produce zero rows
         ids[2, 0] = E + 3
+        ids[3, 1] = ids[3, 0]  # a token may name an expert twice (the grouping then counts instead of using its token masks)
     y = ops.mul_mat_id(GE, cu(x), cu(ids)).cpu().numpy()                      # x broadcast over k
     xk = synth.normal_f32(synth.tensor_seed("mmid-xk", n), (n, K, I))
     yk = ops.mul_mat_id(DE, cu(xk), cu(ids)).cpu().numpy()                    # one row per (token, k)
