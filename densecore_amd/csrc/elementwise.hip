@@ -180,6 +180,16 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t t = blockIdx.y, base = t * cols, nb = cols / kQK;
     const bool writer = blockIdx.x == 0;
+    // this wavefront's router row does not depend on the norm: its first eight chunks are requested before anything
+    // else, so that their trip from HBM overlaps the norm instead of following it
+    const int64_t ex = (int64_t)blockIdx.x * 4 + wave;
+    const float* wr = w_router + (ex < n_experts ? ex : 0) * cols;
+    const bool ahead = cols >= 8 * 256;  // wave-uniform
+    float4 first[8];
+    if (ahead) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) first[u] = *reinterpret_cast<const float4*>(wr + lane * 4 + u * 256);
+    }
     float4 kept[kKeep];
     float ssq = 0.0f;
 #pragma unroll
@@ -221,9 +231,7 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
         }
     }
     __syncthreads();
-    const int64_t ex = (int64_t)blockIdx.x * 4 + wave;
     if (ex >= n_experts) return;
-    const float* wr = w_router + ex * cols;
     float acc = 0.0f;
     auto add4 = [&](const float4& a, const float4& b) {
         acc = __fmaf_rn(a.x, b.x, acc);
@@ -232,6 +240,11 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
         acc = __fmaf_rn(a.w, b.w, acc);
     };
     int64_t c = (int64_t)lane * 4;
+    if (ahead) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) add4(first[u], *reinterpret_cast<const float4*>(row_sh + c + u * 256));
+        c += 8 * 256;
+    }
     for (; c + 7 * 256 + 3 < cols; c += 8 * 256) {
         float4 a[8];
 #pragma unroll
