@@ -16,7 +16,7 @@ EXPORTS = [
     "mq_weight_upload", "mq_weight_upload_typed", "mq_weight_synthetic", "mq_weight_synthetic_typed", "mq_weight_type", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
     "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_gemm_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
-    "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums",
+    "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums", "mq_debug_moe_groups", "mq_debug_moe_hidden", "mq_debug_decoder_buffers",
     "mq_acts_create", "mq_acts_free", "mq_acts_quantize", "mq_mul_mat_q4k_acts", "mq_swiglu_mul_mat_q4k_acts",
     "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
     "mq_decoder_create", "mq_decoder_step", "mq_decoder_status", "mq_decoder_set_patience", "mq_decoder_free",
@@ -84,6 +84,9 @@ def load() -> C.CDLL:
     L.mq_mul_mat_id_q4k.argtypes = [vp, vp, i64, ci, vp, ci, vp, vp]
     L.mq_moe_layer_q4k.argtypes = [C.POINTER(MoELayerDesc), vp, vp, i64, vp, vp, vp, vp]
     L.mq_debug_block_sums.argtypes = [vp, vp, i64, i64, vp, vp, vp, i64, vp]
+    L.mq_debug_moe_groups.argtypes = [vp, vp, i64, i64, ci, vp, vp, vp]
+    L.mq_debug_moe_hidden.argtypes = [vp, sz, vp]
+    L.mq_debug_decoder_buffers.argtypes = [vp] + [C.POINTER(vp)] * 5
     L.mq_add_rmsnorm_f32.argtypes = [vp, vp, vp, i64, i64, C.c_float, vp, vp, vp]
     L.mq_add_rmsnorm_q8k.argtypes = [vp, vp, vp, i64, i64, C.c_float, vp, vp, vp, vp]
     L.mq_router_logits_f32.argtypes = [vp, i64, i64, vp, i64, i64, vp, vp]

@@ -764,6 +764,30 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     return MQ_OK;
 }
 
+int mq_debug_moe_groups(const float* logits_dev, const int32_t* ids_dev, int64_t n_experts, int64_t n, int top_k,
+                        int32_t* triples_dev, int32_t* count_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if ((logits_dev == nullptr) == (ids_dev == nullptr)) return fail(MQ_ERR_INVALID, "mq_debug_moe_groups: pass logits or ids, not both");
+    if (!triples_dev || !count_dev) return fail(MQ_ERR_INVALID, "mq_debug_moe_groups: null output");
+    if (n <= 0 || top_k <= 0 || top_k > 8 || n_experts <= 0 || n_experts > 2048 || (logits_dev && top_k > n_experts))
+        return fail(MQ_ERR_INVALID, "mq_debug_moe_groups: need n > 0, 0 < top_k <= 8, 0 < n_experts <= 2048");
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    RouteWs r;
+    if (int rc = carve_route(n, top_k, n_experts, r)) return rc;
+    if (ids_dev) {
+        MQ_HIP(launch_build_groups(ids_dev, n, top_k, n_experts, r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, s));
+    } else {
+        if (int rc = reserve_counters(4096)) return rc;
+        MQ_HIP(launch_route_and_group(logits_dev, n_experts, n, top_k, MQ_ROUTE_FUSED, r.ids, r.weights, (uint32_t*)g.counters.ptr + 4095,
+                                      r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, true, nullptr, 0, 0,
+                                      nullptr, nullptr, s));
+    }
+    MQ_HIP(launch_flatten_groups(r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, (int)(n * top_k), triples_dev,
+                                 count_dev, s));
+    return MQ_OK;
+}
+
 namespace {
 
 struct SharedExpert {
@@ -1327,6 +1351,25 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
     a.ids_out = ids_out_dev, a.wts_out = weights_out_dev;
     a.sync = d->sync;
     MQ_HIP(launch_decoder_layers(a, d->n_workgroups, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_debug_decoder_buffers(mq_decoder* d, float** qkv_dev, float** o_dev, float** logits_dev, float** hidden_dev, float** y_dev) {
+    if (!d) return fail(MQ_ERR_INVALID, "mq_debug_decoder_buffers: null handle");
+    if (qkv_dev) *qkv_dev = d->qkv;
+    if (o_dev) *o_dev = d->o;
+    if (logits_dev) *logits_dev = d->logits;
+    if (hidden_dev) *hidden_dev = d->mid;
+    if (y_dev) *y_dev = d->y;
+    return MQ_OK;
+}
+
+int mq_debug_moe_hidden(float* hidden_out_dev, size_t count, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (!hidden_out_dev) return fail(MQ_ERR_INVALID, "mq_debug_moe_hidden: null output");
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (count * sizeof(float) > g.mid.cap) return fail(MQ_ERR_INVALID, "mq_debug_moe_hidden: the intermediate buffer holds %zu bytes", g.mid.cap);
+    MQ_HIP(hipMemcpyAsync(hidden_out_dev, g.mid.ptr, count * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream));
     return MQ_OK;
 }
 

@@ -156,6 +156,10 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,
                               const float* x, float* y, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
+// The work list written out as (expert, token, k) triples in list order, and the number of entries.
+hipError_t launch_flatten_groups(const int32_t* group_expert, const int32_t* group_begin, const int32_t* n_groups,
+                                 const int32_t* entry_token, const int32_t* entry_k, int max_entries, int32_t* triples,
+                                 int32_t* count, hipStream_t stream);
 
 // ---- moe_down.hip ----------------------------------------------------------------------------
 // Down projection + weighted combine, one workgroup per (token, 16 output rows): for decode widths, where

@@ -6,7 +6,8 @@
 //               workgroup as a whole streams one contiguous run of tiles.
 //   wavefront = per super-block: three coalesced 16-byte-per-lane loads bring one 2304-byte tile
 //               (16 rows x 256 weights) straight into MFMA operand order; the next tile is
-//               requested before the current one is consumed (two register stages, ping-pong).
+//               requested before the current one is consumed (two register stages, ping-pong; no request
+//               is made past the wave's last super-block).
 //   arithmetic, per tile and per group of 8 activation rows (independent of how many are live):
 //       4 x v_mfma_i32_16x16x64_i8   one per 64-weight chunk.  Each activation row owns two M-side
 //                                    slots with complementary zero halves (see common.h), so the
@@ -62,15 +63,6 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
     }
 }
 
-// Register stages a wave keeps in flight.  The kernel is bound by bytes in flight, not by
-// arithmetic: HBM latency under load is 1.5-2.5 us, so a CU needs on the order of 100 KB of
-// outstanding tile loads.  A stage is one super-block's activations (A operand) plus the NMAT
-// weight tiles that share them; at 2 waves per SIMD the register file holds four such stages.
-template <int NMAT, int TT, int WT>
-struct Depth {
-    static constexpr int kStages = WT == kWtQ6 ? (TT == 1 && NMAT == 1 ? 3 : 2) : TT == 1 ? (NMAT == 2 ? 3 : 4) : 2;
-};
-
 // One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
 // waves split the super-blocks of the row.  NMAT == 2: gate and up tiles of the same rows share
 // the activations in registers and meet in silu(gate)*up.
@@ -82,7 +74,6 @@ struct Depth {
 template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
-    constexpr int S = Depth<NMAT, TT, WT>::kStages;
     extern __shared__ float red[];  // [W-1][NMAT][TT][2][64]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps tile addresses scalar
@@ -192,35 +183,37 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 }
         };
 
-        // Ring of S register stages.  Stage i of this wave is super-block wave + i*W.  S-1 stages are
-        // requested before the first is consumed, and every consume is preceded by the request for
-        // the stage S-1 ahead, so S-1 stages are in flight while the MFMAs of one run.  All branches
-        // are wave-uniform and the loads themselves unconditional.
+        // Stage i of this wave is super-block wave + i*W (several row tiles in a one-wave workgroup: tile i of the
+        // contiguous run); two register stages, one in flight while the other is multiplied (ring2: no request is
+        // ever made past the last stage).  All branches are wave-uniform and the loads themselves unconditional.
         if (wave < nb) {
             const int per_rt = (int)((nb - wave + n_waves - 1) / n_waves);  // super-blocks of this wave per row tile
             const int cnt = per_rt * rt_count;                              // stages of this wave
-            typename TileOf<WT>::Regs ring_t[S][NMAT];
-            ARegs<TT> ring_a[S];
-            float4 ring_x[S];
-            // Requests past the wave's last super-block are pointed at the (cache-resident)
-            // activation buffer (without one: at the wave's first tile again) instead of being
-            // skipped: the number of loads per stage stays fixed, so every wait below can count exactly.
-            auto issue = [&](int st, int i) {
+            typename TileOf<WT>::Regs ring_t[2][NMAT];
+            ARegs<TT> ring_a[2];
+            float4 ring_x[2];
+            auto issue = [&](auto st_c, int i) {
+                constexpr int st = decltype(st_c)::value;
+                // i == cnt (once, when cnt is odd): the same loads from fixed addresses in all lanes, a cache line each
                 const bool valid = i < cnt;
                 // several row tiles (one wave, per_rt == nb): stage i is tile i of the contiguous run,
                 // super-block i % nb; one row tile: super-block wave + i*W
                 const int t = valid ? (rt_per_wg > 1 ? i : wave + i * n_waves) : wave;
                 const int b = rt_per_wg > 1 ? t % per_rt : t;
+                const int ln = valid ? lane : 0;
 #pragma unroll
-                for (int m = 0; m < NMAT; ++m)
-                    load_tile_wt<WT>(ring_t[st][m], valid ? tiles[m] + (size_t)t * kTileStride : XQ ? tiles[m] + (size_t)wave * kTileStride : p.aq, lane);
+                for (int m = 0; m < NMAT; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)t * kTileStride, ln);
                 if constexpr (XQ) {
-                    ring_x[st] = *reinterpret_cast<const float4*>(p.xf + (size_t)b * kQK + lane * 4);
+                    ring_x[st] = *reinterpret_cast<const float4*>(p.xf + (size_t)b * kQK + ln * 4);
                 } else {
-                    load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+                    size_t off[TT];
+#pragma unroll
+                    for (int tt = 0; tt < TT; ++tt) off[tt] = valid ? a_off[tt] : 0;
+                    load_a<TT>(ring_a[st], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, off, d_idx);
                 }
             };
-            auto consume = [&](int st, int i) {
+            auto consume = [&](auto st_c, int i) {
+                constexpr int st = decltype(st_c)::value;
                 ARegs<TT> quantized;
                 if constexpr (XQ) {  // the row becomes row 0 of the operand
                     const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
@@ -249,26 +242,15 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                             }
                     }
                 }
-            };
+                if (rt_per_wg > 1 && (i + 1) % per_rt == 0) {  // a row tile is complete: store it, start the next
+                    store_rows(rt + i / per_rt);
 #pragma unroll
-            for (int st = 0; st < S - 1; ++st) issue(st, st);
-            for (int base = 0; base < cnt; base += S) {
+                    for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-                for (int st = 0; st < S; ++st) {
-                    const int i = base + st;
-                    issue((st + S - 1) % S, i + S - 1);
-                    if (i < cnt) {
-                        consume(st, i);
-                        if (rt_per_wg > 1 && (i + 1) % per_rt == 0) {  // a row tile is complete: store it, start the next
-                            store_rows(rt + i / per_rt);
-#pragma unroll
-                            for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-                                for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = acc[m][tt][1] = 0.0f;
-                        }
-                    }
+                        for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = acc[m][tt][1] = 0.0f;
                 }
-            }
+            };
+            ring2(cnt, issue, consume);
         }
 
         // ---- cross-wave reduction in wave order, then the epilogue on wave 0 ----

@@ -355,6 +355,26 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
     y[tok * rows + r] = acc;
 }
 
+// The work list as (expert, token, k) triples in list order, for comparison with the reference's sorted assignments
+// (core/src/llm/moe/native.cpp:1664-1733); one workgroup.
+__global__ void __launch_bounds__(256) flatten_groups_kernel(const int32_t* __restrict__ group_expert,
+                                                             const int32_t* __restrict__ group_begin,
+                                                             const int32_t* __restrict__ n_groups,
+                                                             const int32_t* __restrict__ entry_token,
+                                                             const int32_t* __restrict__ entry_k, int max_entries,
+                                                             int32_t* __restrict__ triples, int32_t* __restrict__ count) {
+    const int groups = *n_groups;
+    for (int g = 0; g < groups; ++g) {
+        const int b = group_begin[g], e = group_begin[g + 1];
+        for (int i = b + (int)threadIdx.x; i < e && i < max_entries; i += 256) {
+            triples[3 * i] = group_expert[g];
+            triples[3 * i + 1] = entry_token[i];
+            triples[3 * i + 2] = entry_k[i];
+        }
+    }
+    if (threadIdx.x == 0) *count = group_begin[groups];
+}
+
 __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t count) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * 256;
@@ -432,6 +452,14 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
     if (top_k < 0 || top_k > 8) return hipErrorInvalidValue;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((rows + 255) / 256), (unsigned)n), dim3(256), 0, stream, part,
                        top_k, slots, rows, weights, ids, (int)n_experts, has_shared, sh_gate_inp, x, y);
+    return hipGetLastError();
+}
+
+hipError_t launch_flatten_groups(const int32_t* group_expert, const int32_t* group_begin, const int32_t* n_groups,
+                                 const int32_t* entry_token, const int32_t* entry_k, int max_entries, int32_t* triples,
+                                 int32_t* count, hipStream_t stream) {
+    hipLaunchKernelGGL(flatten_groups_kernel, dim3(1), dim3(256), 0, stream, group_expert, group_begin, n_groups, entry_token,
+                       entry_k, max_entries, triples, count);
     return hipGetLastError();
 }
 

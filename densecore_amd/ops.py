@@ -188,6 +188,27 @@ def debug_block_sums(w: Q4KWeight, x: torch.Tensor):
     return ds, md, y
 
 
+def debug_moe_groups(n_experts: int, top_k: int, ids: torch.Tensor = None, logits: torch.Tensor = None) -> np.ndarray:
+    """The expert-grouped work list the grouped kernels read, as int32 [entries, 3] = (expert, token, k) in list
+    order (Qwen35BuildMoEAssignments, core/src/llm/moe/native.cpp:1664-1733).  ids int32 [n, top_k]: the grouping
+    launch of the expert nodes; logits fp32 [n, n_experts]: the route-and-group launch of the MoE layer."""
+    src = ids if ids is not None else logits
+    n = src.shape[0]
+    triples = torch.full((n * top_k, 3), -7, dtype=torch.int32, device=src.device)
+    count = torch.zeros(1, dtype=torch.int32, device=src.device)
+    _lib.check(_lib.lib().mq_debug_moe_groups(_ptr(_f32(logits)) if logits is not None else None,
+                                              _ptr(ids.contiguous()) if ids is not None else None, n_experts, n, top_k,
+                                              _ptr(triples), _ptr(count), _stream()), "mq_debug_moe_groups")
+    return triples.cpu().numpy()[:int(count.item())]
+
+
+def debug_moe_hidden(shape) -> torch.Tensor:
+    """The fp32 intermediate of the last moe_layer / ffn_swiglu call (hidden rows [n, slots, inter] / [n, inter])."""
+    out = torch.empty(shape, dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().mq_debug_moe_hidden(_ptr(out), out.numel(), _stream()), "mq_debug_moe_hidden")
+    return out
+
+
 def swiglu_mul_mat(gate: Q4KWeight, up: Q4KWeight, x: torch.Tensor, silu: int = SILU_EXACT) -> torch.Tensor:
     """FusedSwiGLUQ4KQ8KRows_Hwy (core/src/kernels/hwy/hwy_moe_quant.cc:359-380): silu(gate x) * (up x)."""
     x = _f32(x)

@@ -21,6 +21,7 @@ def assert_fp32_parity(got: np.ndarray, ref: np.ndarray, mag: np.ndarray, what: 
     worst = np.max(err / np.maximum(scale, 1e-300))
     assert worst <= REL_TOL, f"{what}: max relative error {worst:.3e} > {REL_TOL}"
     ok = np.abs(ref) >= mag * CANCEL_FLOOR
+    ok &= ref != 0          # ref == mag == 0 (an all-zero row): nothing to divide by
     return float(np.max(err[ok] / np.abs(ref[ok]))) if ok.any() else 0.0
 
 

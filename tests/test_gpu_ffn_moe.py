@@ -84,6 +84,27 @@ def test_ffn_full_size_single_token(ops):
         w.free()
 
 
+@pytest.mark.parametrize("n", [2, 4, 8, 16])
+def test_ffn_full_size_batched(ops, n):
+    """The same shape at the other widths of the benchmark: two rows per lane (2..8) and two token tiles (16) are
+    other instantiations of the decode kernel, with other wave counts, than the single-token case."""
+    H, I = 4096, 14336
+    seeds = [synth.tensor_seed("cfg2", nm) for nm in "gud"]
+    G, U, D = (ops.Q4KWeight.synthetic(s, r, c) for s, (r, c) in zip(seeds, ((I, H), (I, H), (H, I))))
+    g, u, d = G.to_ggml(), U.to_ggml(), D.to_ggml()
+    x = synth.normal_f32(synth.tensor_seed("cfg2-x", n), (n, H))
+    h_gpu = ops.swiglu_mul_mat(G, U, cu(x), 2).cpu().numpy()
+    assert_close_prod(h_gpu, orc.swiglu_mul_mat(g, u, H, I, x, orc.ORDER_DOTPROD, 2), "swiglu")
+    y_gpu = ops.ffn_swiglu(G, U, D, cu(x), 2).cpu().numpy()
+    assert np.array_equal(ops.debug_moe_hidden((n, I)).cpu().numpy().view(np.uint32), h_gpu.view(np.uint32))
+    q8 = orc.quantize_rows_q8k(h_gpu)
+    mag = np.stack([orc.dot_magnitude_f64(d, I, q8[t:t + 1])[0] for t in range(n)])
+    assert_fp32_parity(y_gpu, orc.simd_mul_mat_q4k_q8k(d, I, q8, 8), mag, "down (AVX2 order)")
+    assert_fp32_parity(y_gpu[:2], orc.mul_mat_q4k_q8k(d, I, q8[:2], orc.ORDER_HWY), mag[:2], "down (Highway order)")
+    for w in (G, U, D):
+        w.free()
+
+
 def reference_patterned_floats(rows, cols, scale):
     """Input recipe of the reference's MoE tests (core/tests/moe/test_moe_ops.cpp:119-129)."""
     r = np.arange(rows)[:, None]

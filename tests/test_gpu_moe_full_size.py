@@ -1,0 +1,82 @@
+"""The MoE block at the benchmark's own shape -- hidden 2048, 256 experts + 1 shared, expert intermediate 512,
+top-8 -- above eight tokens, where the expert-grouped gate/up launch lets a one-wavefront workgroup take two or
+four row tiles and counts 16 / 2 or 16 / 4 arrivals per 256-row block for the fused Q8_K of its output
+(widths 12..64 take two row tiles, 72 -- and 64 with the shared expert's groups added -- four).
+
+Stage by stage against the CPU restatement with the GPU's own intermediate fed forward (a Q8_K re-quantization sits
+between the stages; see tests/test_gpu_ffn_moe.py), the one-call layer bit-equal to its stages, and end to end."""
+import numpy as np
+import pytest
+
+from densecore_amd import synth
+from oracle import binding as orc
+from tests._parity import assert_fp32_parity
+from tests.test_gpu_ffn_moe import END_TO_END_REL, assert_close_prod
+
+pytestmark = pytest.mark.gpu
+
+E, H, I, K = 256, 2048, 512, 8
+
+
+@pytest.fixture(scope="module")
+def layer():
+    import torch
+    from densecore_amd import ops
+    assert torch.cuda.is_available()
+    dev = [ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", nm), r, c, E) for nm, r, c in
+           (("g", I, H), ("u", I, H), ("d", H, I))]
+    sh = [ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3-sh", nm), r, c) for nm, r, c in
+          (("g", I, H), ("u", I, H), ("d", H, I))]
+    host = [w.to_ggml() for w in dev]
+    sh_host = [w.to_ggml() for w in sh]
+    gate_inp = synth.normal_f32(synth.tensor_seed("cfg3-gi"), (H,)) * np.float32(0.02)
+    yield ops, dev, sh, host, sh_host, gate_inp
+    for w in dev + sh:
+        w.free()
+
+
+def cu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("n,silu", [(12, 1), (16, 1), (32, 1), (64, 1), (72, 2), (9, 0)])
+def test_cfg3_layer_stagewise(layer, n, silu):
+    ops, (GE, UE, DE), (SG, SU, SD), (ge, ue, de), (sg, su, sd), gate_inp = layer
+    x = synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))
+    logits = synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))
+    ids_t, w_t = ops.moe_route_topk(cu(logits), K, 0)
+    ids, wts = ids_t.cpu().numpy(), w_t.cpu().numpy()
+    oi, ow = orc.route_topk(logits, K, 0)
+    assert np.array_equal(ids, oi) and np.allclose(wts, ow, rtol=3e-6)
+
+    # stage 1: expert-grouped gate/up + SwiGLU (several row tiles per workgroup at these widths)
+    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids_t, silu).cpu().numpy()
+    assert_close_prod(hid, orc.moe_gateup_swiglu(ge, ue, H, I, x, ids, orc.ORDER_DOTPROD, silu), "gate/up")
+
+    # stage 2: expert-grouped down + combine on the GPU's own hidden rows and weights
+    y_routed = ops.moe_down_weighted(DE, cu(hid), ids_t, w_t).cpu().numpy()
+    mag = np.zeros((n, H))
+    hq = orc.quantize_rows_q8k(hid.reshape(n * K, I)).reshape(n, K, -1)
+    for t in range(n):
+        for k in range(K):
+            mag[t] += abs(wts[t, k]) * orc.dot_magnitude_f64(de[ids[t, k]], I, hq[t, k][None])[0]
+    assert_fp32_parity(y_routed, orc.moe_down_weighted(de, H, I, hid, ids, wts, orc.ORDER_DOTPROD, 0), mag, "down")
+
+    # the one-call layer without the shared expert: the same bits as its stages (its gate/up leaves the hidden rows
+    # in Q8_K through the arrival counters, its hidden rows are the stage's)
+    y_nosh, ids2, w2 = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=silu)
+    assert np.array_equal(ids2.cpu().numpy(), ids) and np.array_equal(w2.cpu().numpy().view(np.uint32), wts.view(np.uint32))
+    assert np.array_equal(ops.debug_moe_hidden((n, K, I)).cpu().numpy().view(np.uint32), hid.view(np.uint32))
+    assert np.array_equal(y_nosh.cpu().numpy().view(np.uint32), y_routed.view(np.uint32))
+
+    # with the shared expert (more groups in both launches): hidden rows of the routed slots unchanged, the shared
+    # slot against the dense SwiGLU of the same matrices, the output end to end against the CPU layer
+    y, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=(SG, SU, SD, cu(gate_inp)), silu=silu)
+    hid_sh = ops.debug_moe_hidden((n, K + 1, I)).cpu().numpy()
+    assert np.array_equal(hid_sh[:, :K].view(np.uint32), hid.view(np.uint32))
+    assert_close_prod(hid_sh[:, K], orc.swiglu_mul_mat(sg, su, H, I, x, orc.ORDER_DOTPROD, 2), "shared gate/up")
+    ref = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=(sg, su, sd, gate_inp), silu=silu)
+    y = y.cpu().numpy()
+    rel = np.max(np.abs(y - ref["y"]), axis=1) / np.max(np.abs(ref["y"]), axis=1)
+    assert np.max(rel) <= END_TO_END_REL and np.median(rel) <= 2e-5, (np.max(rel), np.median(rel))

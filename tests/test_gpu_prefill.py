@@ -125,3 +125,22 @@ def test_gemm_full_size_rows_against_decode_kernel(ops, m):
     # Q8_K quantization is odd (codes and scale flip sign together), so the product is too, exactly
     assert torch.equal(ops.gemm(W, -x), -y)
     W.free()
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+def test_gemm_full_size_sampled_rows_against_the_oracle(ops, m):
+    """W 4096 -> 14336 at M = 512 / 2048 against the CPU restatement itself: every 61st activation row (and the last)
+    over all 14336 outputs, the AVX2-order build for speed plus the Highway order on two of them."""
+    import torch
+    rows, cols = 14336, 4096
+    W = ops.Q4KWeight.synthetic(4, rows, cols)
+    w = W.to_ggml()
+    x = synth.normal_f32(synth.tensor_seed("pf-full", m), (m, cols))
+    y = ops.gemm(W, cu(x)).cpu().numpy()
+    pick = sorted(set(range(0, m, 61)) | {m - 1})
+    q8 = orc.quantize_rows_q8k(x[pick])
+    ref = orc.simd_mul_mat_q4k_q8k(w, cols, q8, 8)
+    mag = np.stack([orc.dot_magnitude_f64(w, cols, q8[i:i + 1])[0] for i in range(len(pick))])
+    assert_fp32_parity(y[pick], ref, mag, "sampled rows (AVX2 order)")
+    assert_fp32_parity(y[pick[:2]], orc.mul_mat_q4k_q8k(w, cols, q8[:2], orc.ORDER_HWY), mag[:2], "Highway order")
+    W.free()

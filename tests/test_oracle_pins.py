@@ -282,6 +282,35 @@ def test_simd_ffn_baseline_matches_scalar_oracle():
 
 
 # ----------------------------------------------------------------- activation
+def test_fast_exp_known_answers_from_the_references_literals():
+    """The cubic's three coefficients and log2(e) as the reference spells them
+    (core/src/backend/cpu_backend_internal.h:103 kLog2E, :108 the three coefficients;
+    core/src/kernels/hwy/hwy_fastexp.h:31-33 c0, c1, c2): the restatement must return, bit for bit, what those
+    literals give when every step is rounded to fp32 in the written order -- a wrong digit in any of them shows."""
+    f32 = np.float32
+    log2e, c0, c1, c2 = f32(1.4426950408889634), f32(0.6960656421638072), f32(0.224494337302845), f32(0.07944023841053369)
+    xs = np.concatenate([np.linspace(-60, 60, 2401), [0.0, -0.0, 1e-8, 49.999, 50.0, 50.001, -50.001]]).astype(f32)
+    xc = np.clip(xs, f32(-50), f32(50))
+    y = xc * log2e
+    fl = np.floor(y)
+    f = y - fl
+    two_i = ((fl.astype(np.int32) + 127) << 23).view(f32)
+    plain = two_i * (f32(1) + f * (c0 + f * (c1 + f * c2)))                      # unfused Horner, fp32 at every step
+    got = np.array([orc.lib().orc_fast_exp(float(v)) for v in xs], f32)
+    assert np.array_equal(got.view(np.uint32), plain.view(np.uint32))
+    # the fused form: each multiply-add rounded once (a double holds the exact product and, here, the exact sum)
+    fma = lambda a, b, c: (a.astype(np.float64) * b.astype(np.float64) + np.float64(c)).astype(f32)
+    p = fma(f, np.full_like(f, c2), c1)
+    p = fma(f, p, c0)
+    p = fma(f, p, f32(1))
+    got = np.array([orc.lib().orc_fast_exp_fma(float(v)) for v in xs], f32)
+    assert np.array_equal(got.view(np.uint32), (two_i * p).view(np.uint32))
+    # closed form: at f = 1/2 the cubic is 1 + c0/2 + c1/4 + c2/8, a 2e-4-accurate sqrt(2)
+    half = orc.lib().orc_fast_exp(float(f32(0.5) / log2e))
+    assert abs(half - (1 + 0.6960656421638072 / 2 + 0.224494337302845 / 4 + 0.07944023841053369 / 8)) < 2e-6
+    assert abs(half - 2 ** 0.5) < 3e-4
+
+
 def test_fast_exp_error_class_and_silu_flavours():
     xs = np.linspace(-20, 20, 4001, dtype=np.float32)
     fe = np.array([orc.lib().orc_fast_exp(float(v)) for v in xs])
