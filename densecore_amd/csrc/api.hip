@@ -31,6 +31,16 @@ struct mq_acts {
     int64_t n = 0;        // rows quantized by the last mq_acts_quantize
 };
 
+// Scratch of mq_mul_mat_q4k_noalloc: the quantized activations (A-major codes, then the scales) of at most
+// kNoAllocMaxRows rows of kNoAllocMaxCols columns.  One copy per GPU, held until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the device address is looked up once per device in mq_init.
+// (File scope, not the unnamed namespace below: there the device-side symbol is local to the code object and the
+// runtime cannot find it.)
+constexpr int64_t kNoAllocMaxRows = 16, kNoAllocMaxCols = 16384;
+constexpr size_t kNoAllocAqBytes = (size_t)((kNoAllocMaxRows + 7) / 8) * (kNoAllocMaxCols / mq::kQK) * 4096;
+constexpr size_t kNoAllocAdBytes = (size_t)((kNoAllocMaxRows + 7) / 8) * (kNoAllocMaxCols / mq::kQK) * 8 * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kNoAllocAqBytes + kNoAllocAdBytes];
+
 namespace {
 
 thread_local std::string g_error;
@@ -93,6 +103,9 @@ struct State {
     Buffer route;         // ids / weights / groups / entries
     Buffer stage_in, stage_out;  // host-pointer entry points
 } g;
+
+constexpr int kMaxDevices = 64;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU that mq_init has seen
 
 // Launch census: a start/stop event pair bound to each matmul-kernel dispatch (see mq_census_* in the public header).
 struct Census {
@@ -213,6 +226,11 @@ int mq_init(int device) {
     MQ_HIP(hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(MQ_ERR_UNSUPPORTED, "built for gfx950, device is %s", prop.gcnArchName);
+    if (device < kMaxDevices && !g_scratch_ptr[device]) {  // this GPU's copy of the allocation-free entry point's scratch
+        void* ptr = nullptr;
+        MQ_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[device] = static_cast<unsigned char*>(ptr);
+    }
     g.device = device;
     g.ready = true;
     return MQ_OK;
@@ -452,6 +470,40 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
+}
+
+int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                           void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (int rc = check_weight(w, "mq_mul_mat_q4k_noalloc")) return rc;
+    if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_noalloc: weight is an expert stack");
+    if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_mul_mat_q4k_noalloc")) return rc;
+    if (n > kNoAllocMaxRows || w->cols > kNoAllocMaxCols)
+        return fail(MQ_ERR_UNSUPPORTED, "mq_mul_mat_q4k_noalloc: %lld rows of %lld columns exceed the fixed scratch (at most %lld rows of %lld columns)",
+                    (long long)n, (long long)w->cols, (long long)kNoAllocMaxRows, (long long)kNoAllocMaxCols);
+    if (n == 0) return MQ_OK;
+    if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_noalloc: null output or ldy < rows");
+    unsigned char* ws = g.device >= 0 && g.device < kMaxDevices ? g_scratch_ptr[g.device] : nullptr;
+    if (!ws) return fail(MQ_ERR_STATE, "mq_mul_mat_q4k_noalloc: no scratch address for device %d (mq_init looks it up)", g.device);
+    std::lock_guard<std::mutex> lock(g.mu);
+    hipStream_t s = (hipStream_t)stream;
+    uint8_t* aq = ws;
+    float* ad = reinterpret_cast<float*>(ws + kNoAllocAqBytes);
+    // Every byte of the scratch that the product reads is written by this call's quantizer (slots past row n read
+    // row n - 1), so nothing of an earlier call is seen and nothing needs clearing.
+    MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, w->cols, nullptr, 0, aq, ad, s));
+    MatmulArgs a;
+    a.w0 = w->data;
+    a.wtype = w->type;
+    a.rows = w->rows;
+    a.nb = w->nb;
+    a.aq = aq;
+    a.ad = ad;
+    a.n = n;
+    a.y = y_dev;
+    a.ldy = ldy;
+    MQ_HIP(launch_matmul(a, s));
+    return MQ_OK;
 }
 
 int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n,

@@ -115,6 +115,14 @@ int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void*
  * (core/include/densecore/backend/cpu_backend.h:293-300, any n). */
 int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                    void* stream);
+/* mq_mul_mat_q4k for callers that cannot allocate (code under HIP-graph capture, serving loops and harnesses that
+ * forbid hipMalloc): the same product, bit for bit, for n <= 16 rows of cols <= 16384 (MQ_ERR_UNSUPPORTED beyond
+ * that), Q4_K / Q5_K / Q6_K weights.  It calls no allocating routine: the quantized activations go to a fixed
+ * 528,384-byte device array inside the library (one per GPU, held until the process ends) whose address mq_init
+ * looks up.  It has no counterpart in the reference.  Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads' launches in flight together) race; order them on one stream. */
+int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
+                           void* stream);
 /* The same product computed by the matrix-core GEMM kernel whatever n is (mq_mul_mat_q4k switches to it
  * by itself from a few dozen rows up): weights are read once per 128 activation rows and the int8 MFMA
  * units do the arithmetic.  RunQ4KRawBatchedDenseGemm (core/src/backend/cpu_backend_q4k_dense.cpp:57-101),
