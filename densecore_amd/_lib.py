@@ -20,7 +20,7 @@ EXPORTS = [
     "mq_acts_create", "mq_acts_free", "mq_acts_quantize", "mq_mul_mat_q4k_acts", "mq_swiglu_mul_mat_q4k_acts",
     "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
     "mq_decoder_create", "mq_decoder_step", "mq_decoder_status", "mq_decoder_set_patience", "mq_decoder_free",
-    "mq_census_enable", "mq_census_reset", "mq_census_read",
+    "mq_debug_set_dense_lds", "mq_census_enable", "mq_census_reset", "mq_census_read",
     "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_stream_synchronize",
 ]
 

@@ -119,8 +119,46 @@ struct Census {
     static constexpr size_t kMax = 8192;
 } census;
 
+// Dense products of up to 16 rows go to the kernel that stages the activations in LDS where the shape fits it (the
+// same bits as matmul_kernel on the same operands); mq_debug_set_dense_lds(0) keeps them on matmul_kernel.
+int g_dense_lds = 1;
+// Widest product whose fp32 rows the LDS-staged kernel quantizes itself (no quantizer launch).
+int64_t g_dense_xf_rows = 2;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
+
+bool dense_lds_takes(const MatmulArgs& a) {
+    return g_dense_lds && !a.grouped && !a.dbg_dot && !a.out_aq && a.n >= 1 && a.n <= 16 &&
+           dense_lds_applies(a.nb, (a.rows + 15) / 16, a.n, a.swiglu != 0, a.wtype);
+}
+// fp32 rows straight into the product (n rows, ldx apart): true when the call may skip its quantizer launch
+bool dense_lds_quantizes(const mq_weight* w, const float* x, int64_t n, int64_t ldx, bool swiglu) {
+    return g_dense_lds && n >= 1 && n <= g_dense_xf_rows && n <= 4 && n * w->nb <= 64 && !(reinterpret_cast<uintptr_t>(x) & 15u) && !(ldx & 3) &&
+           dense_lds_applies(w->nb, w->rowtiles, n, swiglu, w->type);
+}
+
+hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
+    if (!dense_lds_takes(a)) {
+        if (a.xf && a.n != 1) return hipErrorInvalidValue;  // callers ask dense_lds_quantizes first
+        return launch_matmul(a, s, start, stop);
+    }
+    DenseLdsArgs d;
+    d.w0 = a.w0;
+    d.w1 = a.swiglu ? a.w1 : nullptr;
+    d.rows = a.rows;
+    d.nb = a.nb;
+    d.aq = a.aq;
+    d.ad = a.ad;
+    d.xf = a.xf;
+    d.ldx = a.xf ? (a.n == 1 ? a.nb * kQK : a.ldx) : 0;
+    d.n = a.n;
+    d.y = a.y;
+    d.ldy = a.ldy;
+    d.wtype = a.wtype;
+    d.silu_mode = a.silu_mode;
+    return launch_dense_lds(d, s, start, stop);
+}
+
 hipError_t census_launch(const MatmulArgs& a, hipStream_t s) {
-    if (!census.on || census.used >= Census::kMax) return launch_matmul(a, s);
+    if (!census.on || census.used >= Census::kMax) return dense_launch(a, s);
     if (census.used == census.pool.size()) {
         Census::Rec r;
         hipError_t e = hipEventCreate(&r.start);
@@ -131,7 +169,7 @@ hipError_t census_launch(const MatmulArgs& a, hipStream_t s) {
     }
     Census::Rec& r = census.pool[census.used++];
     r.kind = (a.grouped ? 2 : 0) + (a.swiglu ? 1 : 0);
-    return launch_matmul(a, s, r.start, r.stop);
+    return dense_launch(a, s, r.start, r.stop);
 }
 
 int check_ready() {
@@ -455,14 +493,16 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
             return MQ_OK;
         }
     }
-    if (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) {  // single row, long K per wave: the quantizer runs inside the decode kernel
+    // single row (long K per wave), or a few rows where the LDS-staged kernel applies: the quantizer runs inside the product
+    if ((n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(w, x_dev, n, ldx, false)) {
         MatmulArgs a;
         a.w0 = w->data;
         a.wtype = w->type;
         a.rows = w->rows;
         a.nb = w->nb;
         a.xf = x_dev;
-        a.n = 1;
+        a.ldx = ldx;
+        a.n = n;
         a.y = y_dev;
         a.ldy = ldy;
         MQ_HIP(census_launch(a, s));
@@ -502,7 +542,7 @@ int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, in
     a.n = n;
     a.y = y_dev;
     a.ldy = ldy;
-    MQ_HIP(launch_matmul(a, s));
+    MQ_HIP(dense_launch(a, s));
     return MQ_OK;
 }
 
@@ -616,7 +656,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
     // One row: both quantizers run inside the products (two launches instead of four, the same bits).
-    const bool inline_quant = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
+    const bool one_row = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
+    const bool inline_quant = one_row || dense_lds_quantizes(gate, x_dev, n, hidden, true);
     if (!inline_quant)
         if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
     MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
@@ -628,6 +669,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.nb = gate->nb;
     if (inline_quant) {
         a.xf = x_dev;
+        a.ldx = hidden;
     } else {
         a.aq = (const uint8_t*)g.aq.ptr;
         a.ad = (const float*)g.ad.ptr;
@@ -640,15 +682,17 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     MQ_HIP(census_launch(a, s));
     // The SwiGLU output is re-quantized by a launch of its own: the kernel's fused re-quantization (last
     // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
-    if (!inline_quant)
+    const bool inline_quant_down = one_row || dense_lds_quantizes(down, (const float*)g.mid.ptr, n, inter, false);
+    if (!inline_quant_down)
         if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
     d.wtype = down->type;
     d.rows = hidden;
     d.nb = down->nb;
-    if (inline_quant) {
+    if (inline_quant_down) {
         d.xf = (const float*)g.mid.ptr;
+        d.ldx = inter;
     } else {
         d.aq = (const uint8_t*)g.aq2.ptr;
         d.ad = (const float*)g.ad2.ptr;
@@ -1012,7 +1056,8 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (n == 0) return MQ_OK;
     std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
-    const bool inline_quant = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);  // one row: the quantizer runs inside the product
+    // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
+    const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
     if (!inline_quant)
         if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
     MatmulArgs a;
@@ -1023,6 +1068,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     a.nb = gate->nb;
     if (inline_quant) {
         a.xf = x_dev;
+        a.ldx = ldx;
     } else {
         a.aq = (const uint8_t*)g.aq.ptr;
         a.ad = (const float*)g.ad.ptr;
@@ -1456,6 +1502,14 @@ void mq_decoder_free(mq_decoder* d) {
 }
 
 // ---------------------------------------------------------------------------------- census
+int mq_debug_set_dense_lds(int on) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    const int before = g_dense_lds;
+    g_dense_lds = on & 1;
+    if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
+    return before;
+}
+
 int mq_census_enable(int on) {
     std::lock_guard<std::mutex> lock(g.mu);
     census.on = on != 0;

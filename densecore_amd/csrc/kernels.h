@@ -39,6 +39,7 @@ struct MatmulArgs {
     // dense mode, n == 1: the activation row as fp32 instead; every wavefront quantizes the super-blocks it
     // multiplies (same codes and scales as the stand-alone quantizer, so the same result)
     const float* xf = nullptr;
+    int64_t ldx = 0;               // xf with n > 1 (taken by the LDS-staged dense kernel only): floats between rows
     int64_t n = 0;                 // activation rows (dense mode)
     float* y = nullptr;            // dense: [n][ldy]; grouped: [entry][ldy]
     int64_t ldy = 0;
@@ -83,6 +84,28 @@ struct MatmulArgs {
 int pick_waves(int64_t nb, int64_t workgroups);
 // start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
+
+// ---- dense_lds.hip ---------------------------------------------------------------------------
+// Dense product for 1..16 rows with the quantized activations staged once per workgroup in LDS (same bits as
+// launch_matmul on the same operands).  Either (aq, ad) -- the A-major workspace -- or xf: fp32 rows (n <= 8,
+// 16-byte aligned, ldx % 4 == 0) that the kernel quantizes itself.
+struct DenseLdsArgs {
+    const uint8_t* w0 = nullptr;   // tiled weights; gate when w1 is set
+    const uint8_t* w1 = nullptr;   // up weights: y = silu(w0 x) * (w1 x)
+    int64_t rows = 0, nb = 0;
+    const uint8_t* aq = nullptr;
+    const float* ad = nullptr;
+    const float* xf = nullptr;
+    int64_t ldx = 0;
+    int64_t n = 0;
+    float* y = nullptr;
+    int64_t ldy = 0;
+    int wtype = 12;
+    int silu_mode = 0;
+};
+// true when the shape fits the kernel (LDS capacity, wavefront split)
+bool dense_lds_applies(int64_t nb, int64_t rowtiles, int64_t n, bool swiglu, int wtype);
+hipError_t launch_dense_lds(const DenseLdsArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 // ---- q8_0.hip --------------------------------------------------------------------------------
 // Q8_0 weights (16-row tiles of common.h) x Q8_0 activations, dense, any n (passes of eight rows).
