@@ -21,7 +21,7 @@ EXPORTS = [
     "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
     "mq_decoder_create", "mq_decoder_step", "mq_decoder_status", "mq_decoder_set_patience", "mq_decoder_free",
     "mq_debug_set_dense_lds", "mq_census_enable", "mq_census_reset", "mq_census_read",
-    "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_stream_synchronize",
+    "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_host_malloc", "mq_host_free", "mq_memcpy_h2d_async", "mq_memcpy_d2h_async", "mq_stream_synchronize",
 ]
 
 

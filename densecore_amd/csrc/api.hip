@@ -55,6 +55,12 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+// Set once any entry point has been called on a stream under HIP-graph capture: from then on a graph may hold the
+// address of a workspace buffer, so a buffer that has to grow is retired (kept allocated until mq_shutdown) instead
+// of freed -- the graph's replays keep working on the addresses they captured.
+bool g_graph_seen = false;
+std::vector<void*> g_retired;
+
 int hip_fail(hipError_t e, const char* what) {
     return fail(MQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
@@ -65,13 +71,21 @@ int hip_fail(hipError_t e, const char* what) {
         if (e_ != hipSuccess) return hip_fail(e_, #call); \
     } while (0)
 
-// A device buffer that only grows.  Growing frees the old allocation, which synchronises the
-// device, so kernels already queued on any stream have finished with it.
+// A device buffer that only grows.  Growing frees the old allocation, which synchronises the device, so kernels
+// already queued on any stream have finished with it -- unless a HIP-graph capture has been seen: a captured graph
+// would keep launching kernels on the freed address, so the old allocation is retired instead (and the new one is at
+// least twice as large, which bounds what retirement can hold to the size of the live buffer).
 struct Buffer {
     void* ptr = nullptr;
     size_t cap = 0;
     hipError_t reserve(size_t bytes) {
         if (bytes <= cap) return hipSuccess;
+        if (ptr && g_graph_seen) {
+            g_retired.push_back(ptr);
+            if (bytes < 2 * cap) bytes = 2 * cap;
+            ptr = nullptr;
+            cap = 0;
+        }
         if (ptr) {
             hipError_t e = hipFree(ptr);
             ptr = nullptr;
@@ -90,10 +104,34 @@ struct Buffer {
     }
 };
 
+// Page-locked host memory for the host-pointer entry points (allocated, never registered).
+struct PinnedBuffer {
+    void* ptr = nullptr;
+    size_t cap = 0;
+    hipError_t reserve(size_t bytes) {
+        if (bytes <= cap) return hipSuccess;
+        if (ptr) {
+            hipError_t e = hipHostFree(ptr);
+            ptr = nullptr;
+            cap = 0;
+            if (e != hipSuccess) return e;
+        }
+        const size_t want = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
+        hipError_t e = hipHostMalloc(&ptr, want, hipHostMallocDefault);
+        if (e == hipSuccess) cap = want;
+        return e;
+    }
+    void release() {
+        if (ptr) (void)hipHostFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+    }
+};
+
 struct State {
     bool ready = false;
     int device = -1;
-    std::mutex mu;
+    std::recursive_mutex mu;  // recursive: the host-pointer entry points call the device-pointer ones while holding it
     Buffer aq, ad;        // A-major activations of the op input
     Buffer ap;            // P-major activations of the prefill GEMM
     Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
@@ -102,6 +140,11 @@ struct State {
     Buffer counters;      // arrival counters of the fused output quantization (kept zero between launches)
     Buffer route;         // ids / weights / groups / entries
     Buffer stage_in, stage_out;  // host-pointer entry points
+    PinnedBuffer pin_in, pin_out;
+    // the stream of the last call that used the workspaces above, and an event to order the next stream behind it
+    bool have_last_stream = false;
+    hipStream_t last_stream = nullptr;
+    hipEvent_t order_event = nullptr;
 } g;
 
 constexpr int kMaxDevices = 64;
@@ -172,6 +215,42 @@ hipError_t census_launch(const MatmulArgs& a, hipStream_t s) {
     return dense_launch(a, s, r.start, r.stop);
 }
 
+// Every entry point that touches the shared workspaces goes through this: it serialises host-side callers and orders
+// the device work of callers on DIFFERENT streams -- the workspaces (quantized activations, routing lists, arrival
+// counters) are one set per process, so a call on stream B must not start on the device before the previous call on
+// stream A has finished with them.  A stream under graph capture is left alone (an event recorded outside the capture
+// cannot be waited on inside it): a graph's replays are ordered by whoever launches them.
+int order_stream(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        st = hipStreamCaptureStatusNone;
+    }
+    if (st != hipStreamCaptureStatusNone) {
+        g_graph_seen = true;
+        return MQ_OK;
+    }
+    if (g.have_last_stream && g.last_stream != s) {
+        hipError_t e = hipSuccess;
+        if (!g.order_event) e = hipEventCreateWithFlags(&g.order_event, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventRecord(g.order_event, g.last_stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(s, g.order_event, 0);
+        if (e != hipSuccess) {  // e.g. the previous stream no longer exists: wait for everything instead
+            (void)hipGetLastError();
+            e = hipDeviceSynchronize();
+            if (e != hipSuccess) return hip_fail(e, "ordering a new stream behind the previous one");
+        }
+    }
+    g.last_stream = s;
+    g.have_last_stream = true;
+    return MQ_OK;
+}
+struct Entry {
+    std::lock_guard<std::recursive_mutex> lock;
+    int rc;
+    explicit Entry(hipStream_t s) : lock(g.mu), rc(order_stream(s)) {}
+};
+
 int check_ready() {
     if (!g.ready) return fail(MQ_ERR_STATE, "mq_init has not been called (or no GPU is present)");
     return MQ_OK;
@@ -179,10 +258,11 @@ int check_ready() {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Q8_0 matrices are dense projections only: mq_mul_mat_q4k (and the handle queries) take them, nothing else does.
+// Q8_0 weights: dense projections through mq_mul_mat_q4k, expert stacks as the down experts of the MoE down node and
+// of the MoE layer (their activations are Q8_0 too); nothing else takes them.
 int check_weight(const mq_weight* w, const char* name, bool q80_ok = false) {
     if (!w || !w->data) return fail(MQ_ERR_INVALID, "%s: null weight handle", name);
-    if (w->type == kTypeQ80 && !q80_ok) return fail(MQ_ERR_UNSUPPORTED, "%s: Q8_0 weights are taken by mq_mul_mat_q4k only", name);
+    if (w->type == kTypeQ80 && !q80_ok) return fail(MQ_ERR_UNSUPPORTED, "%s: Q8_0 weights are taken by mq_mul_mat_q4k and as MoE down experts only", name);
     return MQ_OK;
 }
 
@@ -218,7 +298,6 @@ int alloc_weight(int type, int64_t rows, int64_t cols, int64_t n_experts, mq_wei
     *out = nullptr;
     if (type != kTypeQ4K && type != kTypeQ5K && type != kTypeQ6K && type != kTypeQ80)
         return fail(MQ_ERR_UNSUPPORTED, "ggml type %d: only Q4_K (12), Q5_K (13), Q6_K (14) and Q8_0 (8) weights are supported", type);
-    if (type == kTypeQ80 && n_experts != 1) return fail(MQ_ERR_UNSUPPORTED, "Q8_0 expert stacks are not supported");
     if (rows <= 0 || cols <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "rows, cols and n_experts must be positive");
     if (cols % kQK) return fail(MQ_ERR_INVALID, "cols %lld is not a multiple of 256", (long long)cols);
     mq_weight* w = new mq_weight;
@@ -228,8 +307,16 @@ int alloc_weight(int type, int64_t rows, int64_t cols, int64_t n_experts, mq_wei
     w->n_experts = n_experts;
     w->nb = cols / kQK;
     w->rowtiles = (rows + 15) / 16;
-    w->expert_bytes = (size_t)w->rowtiles * (size_t)w->nb * (size_t)tile_bytes_of(type);
-    w->total_bytes = w->expert_bytes * (size_t)n_experts;
+    // shapes may come from an untrusted file header: no product may wrap
+    size_t eb = 0, tb = 0;
+    if (__builtin_mul_overflow((size_t)w->rowtiles, (size_t)w->nb, &eb) || __builtin_mul_overflow(eb, (size_t)tile_bytes_of(type), &eb) ||
+        __builtin_mul_overflow(eb, (size_t)n_experts, &tb) || tb > (size_t(1) << 46)) {
+        delete w;
+        return fail(MQ_ERR_INVALID, "a weight tensor of %lld x %lld x %lld does not fit a device allocation", (long long)rows, (long long)cols,
+                    (long long)n_experts);
+    }
+    w->expert_bytes = eb;
+    w->total_bytes = tb;
     hipError_t e = hipMalloc((void**)&w->data, w->total_bytes);
     if (e != hipSuccess) {
         delete w;
@@ -254,7 +341,7 @@ extern "C" {
 const char* mq_last_error(void) { return g_error.c_str(); }
 
 int mq_init(int device) {
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess || count <= 0) return fail(MQ_ERR_STATE, "no HIP device available (%s)", hipGetErrorString(e));
@@ -269,16 +356,25 @@ int mq_init(int device) {
         MQ_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         g_scratch_ptr[device] = static_cast<unsigned char*>(ptr);
     }
+    set_compute_units(prop.multiProcessorCount);
     g.device = device;
     g.ready = true;
     return MQ_OK;
 }
 
 int mq_shutdown(void) {
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
     for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    g.pin_in.release();
+    g.pin_out.release();
+    if (g.order_event) (void)hipEventDestroy(g.order_event);
+    g.order_event = nullptr;
+    g.have_last_stream = false;
+    for (void* p : g_retired) (void)hipFree(p);
+    g_retired.clear();
+    g_graph_seen = false;
     g.ready = false;
     return MQ_OK;
 }
@@ -308,11 +404,20 @@ int mq_weight_upload_typed(int ggml_type, const void* q4k_host, int64_t rows, in
     if (cols <= 0 || cols % kQK) return fail(MQ_ERR_INVALID, "mq_weight_upload: cols %lld is not a positive multiple of 256", (long long)cols);
     const size_t min_row = (size_t)(cols / kQK) * (size_t)block_bytes_of(ggml_type);
     if (row_bytes < min_row || (row_bytes & 1)) return fail(MQ_ERR_INVALID, "mq_weight_upload: row_bytes %zu < %zu or odd", row_bytes, min_row);
-    if (n_experts > 1 && expert_bytes < row_bytes * (size_t)rows) return fail(MQ_ERR_INVALID, "mq_weight_upload: expert_bytes too small");
+    if (rows <= 0 || n_experts <= 0) return fail(MQ_ERR_INVALID, "mq_weight_upload: rows and n_experts must be positive");
+    // bytes read from the host: checked products (the shape may come from a file header)
+    size_t one = 0, raw_total = 0;
+    bool overflow = __builtin_mul_overflow(row_bytes, (size_t)rows, &one);
+    if (n_experts > 1) {
+        if (!overflow && expert_bytes < one) return fail(MQ_ERR_INVALID, "mq_weight_upload: expert_bytes too small");
+        overflow = overflow || __builtin_mul_overflow(expert_bytes, (size_t)(n_experts - 1), &raw_total) ||
+                   __builtin_add_overflow(raw_total, one, &raw_total);
+    } else {
+        raw_total = one - row_bytes + min_row;
+    }
+    if (overflow || raw_total > (size_t(1) << 46)) return fail(MQ_ERR_INVALID, "mq_weight_upload: tensor size overflows");
     mq_weight* w = nullptr;
     if (int rc = alloc_weight(ggml_type, rows, cols, n_experts, &w)) return rc;
-    const size_t raw_total = n_experts > 1 ? expert_bytes * (size_t)(n_experts - 1) + row_bytes * (size_t)rows
-                                           : row_bytes * (size_t)(rows - 1) + min_row;
     void* raw = nullptr;
     hipError_t e = hipMalloc(&raw, raw_total);
     if (e == hipSuccess) e = hipMemcpy(raw, q4k_host, raw_total, hipMemcpyHostToDevice);
@@ -463,7 +568,8 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");
-    std::lock_guard<std::mutex> lock(g.mu);
+    Entry entry((hipStream_t)stream);
+    if (entry.rc) return entry.rc;
     return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, (hipStream_t)stream);
 }
 
@@ -475,8 +581,9 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_mul_mat_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k: null output or ldy < rows");
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, nullptr, s);
     if (n >= kPrefillMinRows && w->type == kTypeQ4K) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
     if (n == 1 && !census.on && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
@@ -525,8 +632,9 @@ int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, in
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_noalloc: null output or ldy < rows");
     unsigned char* ws = g.device >= 0 && g.device < kMaxDevices ? g_scratch_ptr[g.device] : nullptr;
     if (!ws) return fail(MQ_ERR_STATE, "mq_mul_mat_q4k_noalloc: no scratch address for device %d (mq_init looks it up)", g.device);
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     uint8_t* aq = ws;
     float* ad = reinterpret_cast<float*>(ws + kNoAllocAqBytes);
     // Every byte of the scratch that the product reads is written by this call's quantizer (slots past row n read
@@ -558,8 +666,9 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
         return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: the sum must not overwrite x or delta (every workgroup reads them)");
     if ((reinterpret_cast<uintptr_t>(delta_dev) | reinterpret_cast<uintptr_t>(weight_dev) | reinterpret_cast<uintptr_t>(sum_out_dev)) & 15u)
         return fail(MQ_ERR_INVALID, "mq_rmsnorm_mul_mat_q4k: rows must be 16-byte aligned");
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     if (n == 1 && !census.on && w->type == kTypeQ4K) {  // one row, short K per wave: norm and quantizer run inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
@@ -591,8 +700,9 @@ int mq_mul_mat_q4k_q8k(const mq_weight* w, const void* q8_dev, int64_t n, size_t
     if (!q8_dev || !y_dev || n < 0 || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: bad arguments");
     if (q8_row_bytes < (size_t)w->nb * kQ8Block || (q8_row_bytes & 3) || (reinterpret_cast<uintptr_t>(q8_dev) & 3u))
         return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_q8k: q8 rows too short or not 4-byte aligned");
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     MQ_HIP(g.aq.reserve(aq_bytes(n, w->nb)));
     MQ_HIP(g.ad.reserve(ad_count(n, w->nb) * sizeof(float)));
     MQ_HIP(launch_q8k_to_amajor(q8_dev, n, q8_row_bytes, w->cols, (uint8_t*)g.aq.ptr, (float*)g.ad.ptr, s));
@@ -604,18 +714,24 @@ int mq_mul_mat_q4k_host(const mq_weight* w, const float* x_host, int64_t n, int6
     if (int rc = check_weight(w, "mq_mul_mat_q4k_host", true)) return rc;
     if (!x_host || !y_host || n < 0 || ldx < w->cols || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_host: bad arguments");
     if (n == 0) return MQ_OK;
-    float* xin = nullptr;
-    float* yout = nullptr;
-    {
-        std::lock_guard<std::mutex> lock(g.mu);
-        MQ_HIP(g.stage_in.reserve((size_t)n * (size_t)w->cols * sizeof(float)));
-        MQ_HIP(g.stage_out.reserve((size_t)n * (size_t)w->rows * sizeof(float)));
-        xin = (float*)g.stage_in.ptr;
-        yout = (float*)g.stage_out.ptr;
-    }
-    MQ_HIP(hipMemcpy2D(xin, (size_t)w->cols * 4, x_host, (size_t)ldx * 4, (size_t)w->cols * 4, (size_t)n, hipMemcpyHostToDevice));
+    // The lock is held from the first staging copy to the last: a second thread's copy must not land between this
+    // call's copy and its launch.  Host rows go through page-locked staging buffers, so that both copies are
+    // asynchronous on the stream and the call synchronises once, at its end.
+    Entry entry(nullptr);
+    if (entry.rc) return entry.rc;
+    const size_t in_bytes = (size_t)n * (size_t)w->cols * sizeof(float), out_bytes = (size_t)n * (size_t)w->rows * sizeof(float);
+    MQ_HIP(g.stage_in.reserve(in_bytes));
+    MQ_HIP(g.stage_out.reserve(out_bytes));
+    MQ_HIP(g.pin_in.reserve(in_bytes));
+    MQ_HIP(g.pin_out.reserve(out_bytes));
+    float* xin = (float*)g.stage_in.ptr;
+    float* yout = (float*)g.stage_out.ptr;
+    for (int64_t m = 0; m < n; ++m) memcpy((float*)g.pin_in.ptr + m * w->cols, x_host + m * ldx, (size_t)w->cols * sizeof(float));
+    MQ_HIP(hipMemcpyAsync(xin, g.pin_in.ptr, in_bytes, hipMemcpyHostToDevice, nullptr));
     if (int rc = mq_mul_mat_q4k(w, xin, n, w->cols, yout, w->rows, nullptr)) return rc;
-    MQ_HIP(hipMemcpy2D(y_host, (size_t)ldy * 4, yout, (size_t)w->rows * 4, (size_t)w->rows * 4, (size_t)n, hipMemcpyDeviceToHost));
+    MQ_HIP(hipMemcpyAsync(g.pin_out.ptr, yout, out_bytes, hipMemcpyDeviceToHost, nullptr));
+    MQ_HIP(hipStreamSynchronize(nullptr));
+    for (int64_t m = 0; m < n; ++m) memcpy(y_host + m * ldy, (const float*)g.pin_out.ptr + m * w->rows, (size_t)w->rows * sizeof(float));
     return MQ_OK;
 }
 
@@ -628,8 +744,9 @@ int mq_debug_block_sums(const mq_weight* w, const float* x_dev, int64_t n, int64
     if (n == 0) return MQ_OK;
     if (!dot_scaled_dev || (!min_dot_dev && w->type != kTypeQ80) || !y_dev || ldy < w->rows)
         return fail(MQ_ERR_INVALID, "mq_debug_block_sums: null output");
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, dot_scaled_dev, s);
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, dot_scaled_dev, min_dot_dev, s);
@@ -653,8 +770,9 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (n == 0) return MQ_OK;
     if (!y_dev) return fail(MQ_ERR_INVALID, "mq_ffn_swiglu_q4k: null output");
     if (n == 0) return MQ_OK;
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     // One row: both quantizers run inside the products (two launches instead of four, the same bits).
     const bool one_row = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
     const bool inline_quant = one_row || dense_lds_quantizes(gate, x_dev, n, hidden, true);
@@ -824,8 +942,9 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     if (x_slots != 1 && x_slots != top_k) return fail(MQ_ERR_INVALID, "mq_mul_mat_id_q4k: x_slots must be 1 or top_k");
     if (int rc = check_x(x_dev, n * x_slots, w->cols, w->cols, "mq_mul_mat_id_q4k")) return rc;
     if (n == 0) return MQ_OK;
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n * x_slots, w->cols, w->cols, s)) return rc;
     RouteWs r;
     if (int rc = carve_route(n, top_k, w->n_experts, r)) return rc;
@@ -867,8 +986,9 @@ int mq_debug_moe_groups(const float* logits_dev, const int32_t* ids_dev, int64_t
     if (!triples_dev || !count_dev) return fail(MQ_ERR_INVALID, "mq_debug_moe_groups: null output");
     if (n <= 0 || top_k <= 0 || top_k > 8 || n_experts <= 0 || n_experts > 2048 || (logits_dev && top_k > n_experts))
         return fail(MQ_ERR_INVALID, "mq_debug_moe_groups: need n > 0, 0 < top_k <= 8, 0 < n_experts <= 2048");
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     RouteWs r;
     if (int rc = carve_route(n, top_k, n_experts, r)) return rc;
     if (ids_dev) {
@@ -951,7 +1071,7 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
 
 // Does the down projection of this MoE block run token-major (moe_down.hip)?
 bool token_major_down(const mq_weight* down, int64_t n, int slots) {
-    return n <= kTokenMajorDownMaxTokens && !census.on && (down->rows & 15) == 0 &&
+    return down->type != kTypeQ80 && n <= kTokenMajorDownMaxTokens && !census.on && (down->rows & 15) == 0 &&
            (size_t)slots * (size_t)down->nb * 64 <= 48 * 1024;
 }
 
@@ -964,7 +1084,7 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
     const int64_t inter = down->cols, hidden_dim = down->rows;
     // rows of dropped entries may hold anything; they are never read
     const bool token_major = token_major_down(down, n, slots);
-    if (!hidden_is_quantized && !token_major) {
+    if (!hidden_is_quantized && !token_major && down->type != kTypeQ80) {
         if (int rc = quantize_into(g.aq2, g.ad2, hidden, mid_rows, inter, inter, s)) return rc;
     }
     if (token_major) {
@@ -985,6 +1105,33 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
         return MQ_OK;
     }
     MQ_HIP(g.part.reserve((size_t)mid_rows * (size_t)hidden_dim * sizeof(float)));
+    if (down->type == kTypeQ80) {
+        // Q8_0 experts take Q8_0 hidden rows (core/src/llm/moe/native.cpp:3239-3245: the row is quantized for the
+        // weight's type), one (token, slot) pair per workgroup column, then the same k-ordered combine
+        if (hidden_is_quantized) return fail(MQ_ERR_STATE, "Q8_0 down experts need their hidden rows as fp32");
+        MQ_HIP(g.aq2.reserve(aq_bytes(mid_rows, down->nb)));
+        MQ_HIP(g.ad2.reserve(q80_scale_bytes(mid_rows, down->nb)));
+        MQ_HIP(launch_quantize_q80(hidden, mid_rows, inter, inter, (uint8_t*)g.aq2.ptr, (uint16_t*)g.ad2.ptr, s));
+        Q80MatmulArgs q;
+        q.w = down->data;
+        q.rows = hidden_dim;
+        q.nb = down->nb;
+        q.aq = (const uint8_t*)g.aq2.ptr;
+        q.ah = (const uint16_t*)g.ad2.ptr;
+        q.n = mid_rows;
+        q.y = (float*)g.part.ptr;
+        q.ldy = hidden_dim;
+        q.pair_ids = ids;
+        q.top_k = top_k;
+        q.slots = slots;
+        q.n_experts = (int)down->n_experts;
+        q.expert_bytes = down->expert_bytes;
+        q.sh_w = sh.down ? sh.down->data : nullptr;
+        MQ_HIP(launch_q80_matmul(q, s));
+        MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, slots, hidden_dim, weights, ids, down->n_experts,
+                                  sh.down ? 1 : 0, sh_gate_inp, x, y, s));
+        return MQ_OK;
+    }
     MatmulArgs d;
     d.w0 = down->data;
     d.wtype = down->type;
@@ -1054,8 +1201,9 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (n == 0) return MQ_OK;
     if (!h_dev || ldh < gate->rows) return fail(MQ_ERR_INVALID, "mq_swiglu_mul_mat_q4k: null output or ldh < rows");
     if (n == 0) return MQ_OK;
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
     if (!inline_quant)
@@ -1142,7 +1290,8 @@ static int acts_matmul(const mq_weight* w0, const mq_weight* w1, const mq_acts* 
     m.ldy = ldy;
     m.swiglu = swiglu;
     m.silu_mode = silu_mode;
-    std::lock_guard<std::mutex> lock(g.mu);
+    Entry entry((hipStream_t)stream);  // the handle's rows are the caller's; the launch itself shares nothing, but stays ordered
+    if (entry.rc) return entry.rc;
     MQ_HIP(census_launch(m, (hipStream_t)stream));
     return MQ_OK;
 }
@@ -1168,8 +1317,9 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
     if (n == 0) return MQ_OK;
     if (!ids_dev || !hidden_dev) return fail(MQ_ERR_INVALID, "mq_moe_gateup_swiglu_q4k: null ids or output");
     if (n == 0) return MQ_OK;
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     RouteWs r;
     if (int rc = carve_route(n, top_k, gate_exps->n_experts, r)) return rc;
     MQ_HIP(launch_fill_zero(hidden_dev, (size_t)n * top_k * (size_t)gate_exps->rows, s));
@@ -1182,14 +1332,15 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
 int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev, int64_t n, const int32_t* ids_dev,
                              const float* weights_dev, int top_k, float* y_dev, void* stream) {
     if (int rc = check_ready()) return rc;
-    if (int rc = check_weight(down_exps, "mq_moe_down_weighted_q4k(down_exps)")) return rc;
+    if (int rc = check_weight(down_exps, "mq_moe_down_weighted_q4k(down_exps)", true)) return rc;
     if (int rc = check_experts(nullptr, nullptr, down_exps, top_k, "mq_moe_down_weighted_q4k")) return rc;
     if (int rc = check_x(hidden_dev, n * top_k, down_exps->cols, down_exps->cols, "mq_moe_down_weighted_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!ids_dev || !weights_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_down_weighted_q4k: null pointer");
     if (n == 0) return MQ_OK;
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     RouteWs r;
     if (int rc = carve_route(n, top_k, down_exps->n_experts, r)) return rc;
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, down_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
@@ -1227,7 +1378,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     if (!L) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null layer");
     if (int rc = check_weight(L->gate_exps, "mq_moe_layer_q4k(gate_exps)")) return rc;
     if (int rc = check_weight(L->up_exps, "mq_moe_layer_q4k(up_exps)")) return rc;
-    if (int rc = check_weight(L->down_exps, "mq_moe_layer_q4k(down_exps)")) return rc;
+    if (int rc = check_weight(L->down_exps, "mq_moe_layer_q4k(down_exps)", true)) return rc;
     if (int rc = check_experts(L->gate_exps, L->up_exps, L->down_exps, L->top_k, "mq_moe_layer_q4k")) return rc;
     const int64_t hidden = L->gate_exps->cols, inter = L->gate_exps->rows, E = L->gate_exps->n_experts;
     const int K = L->top_k;
@@ -1237,7 +1388,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     if (L->shared_gate || L->shared_up || L->shared_down) {
         if (int rc = check_weight(L->shared_gate, "mq_moe_layer_q4k(shared_gate)")) return rc;
         if (int rc = check_weight(L->shared_up, "mq_moe_layer_q4k(shared_up)")) return rc;
-        if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)")) return rc;
+        if (int rc = check_weight(L->shared_down, "mq_moe_layer_q4k(shared_down)", true)) return rc;
         if (L->shared_gate->cols != hidden || L->shared_gate->rows != inter || L->shared_up->cols != hidden ||
             L->shared_up->rows != inter || L->shared_down->cols != inter || L->shared_down->rows != hidden ||
             L->shared_gate->n_experts != 1 || L->shared_up->n_experts != 1 || L->shared_down->n_experts != 1 ||
@@ -1253,8 +1404,9 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     if (!logits_dev || !y_dev) return fail(MQ_ERR_INVALID, "mq_moe_layer_q4k: null logits or output");
     if (n == 0) return MQ_OK;
 
-    std::lock_guard<std::mutex> lock(g.mu);
     hipStream_t s = (hipStream_t)stream;
+    Entry entry(s);
+    if (entry.rc) return entry.rc;
     const int slots = K + (sh.gate ? 1 : 0);  // hidden / partial rows per token
     RouteWs r;
     if (int rc = carve_route(n, K, E, r)) return rc;
@@ -1290,7 +1442,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     if (n <= kDirectPairsMaxTokens) r.direct_ids = ids;
     MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
     // the hidden rows leave gate/up in Q8_K, unless the token-major down launch quantizes what it reads itself
-    const bool quantize_in_gateup = !token_major_down(L->down_exps, n, slots);
+    const bool quantize_in_gateup = !token_major_down(L->down_exps, n, slots) && L->down_exps->type != kTypeQ80;
     if (int rc = run_moe_gateup(L->gate_exps, L->up_exps, sh, n, K, slots, L->silu_mode, r, (float*)g.mid.ptr, quantize_in_gateup, s))
         return rc;
     return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, quantize_in_gateup, n, K, slots, r, ids, wts, L->sh_gate_inp_dev,
@@ -1383,7 +1535,7 @@ int mq_decoder_create(const mq_decoder_layer_desc* layers, int n_layers, int64_t
             h.sh_gate_inp = m.sh_gate_inp_dev;
         }
     }
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     mq_decoder* d = new mq_decoder;
     d->n_layers = n_layers;
     d->max_tokens = max_tokens;
@@ -1424,7 +1576,7 @@ int mq_decoder_step(mq_decoder* d, const float* x_dev, int64_t n, int silu_mode,
     if (n < 1 || n > d->max_tokens) return fail(MQ_ERR_INVALID, "mq_decoder_step: %lld tokens, the handle holds 1..%lld", (long long)n, (long long)d->max_tokens);
     if (silu_mode < -1 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_decoder_step: bad silu_mode");
     if ((reinterpret_cast<uintptr_t>(x_dev) | reinterpret_cast<uintptr_t>(out_dev)) & 3u) return fail(MQ_ERR_INVALID, "mq_decoder_step: unaligned pointer");
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     DecoderArgs a;
     a.layers = d->dev_layers;
     a.n_layers = d->n_layers;
@@ -1465,7 +1617,8 @@ int mq_debug_decoder_buffers(mq_decoder* d, float** qkv_dev, float** o_dev, floa
 int mq_debug_moe_hidden(float* hidden_out_dev, size_t count, void* stream) {
     if (int rc = check_ready()) return rc;
     if (!hidden_out_dev) return fail(MQ_ERR_INVALID, "mq_debug_moe_hidden: null output");
-    std::lock_guard<std::mutex> lock(g.mu);
+    Entry entry((hipStream_t)stream);
+    if (entry.rc) return entry.rc;
     if (count * sizeof(float) > g.mid.cap) return fail(MQ_ERR_INVALID, "mq_debug_moe_hidden: the intermediate buffer holds %zu bytes", g.mid.cap);
     MQ_HIP(hipMemcpyAsync(hidden_out_dev, g.mid.ptr, count * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream));
     return MQ_OK;
@@ -1474,7 +1627,7 @@ int mq_debug_moe_hidden(float* hidden_out_dev, size_t count, void* stream) {
 int mq_decoder_status(mq_decoder* d) {
     if (int rc = check_ready()) return rc;
     if (!d) return fail(MQ_ERR_INVALID, "mq_decoder_status: null handle");
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     MQ_HIP(hipDeviceSynchronize());
     uint32_t flag = 0;
     MQ_HIP(hipMemcpy(&flag, d->sync + 128, sizeof flag, hipMemcpyDeviceToHost));
@@ -1487,7 +1640,7 @@ int mq_decoder_status(mq_decoder* d) {
 int mq_decoder_set_patience(mq_decoder* d, int64_t microseconds) {
     if (int rc = check_ready()) return rc;
     if (!d || microseconds < 0) return fail(MQ_ERR_INVALID, "mq_decoder_set_patience: null handle or negative time");
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     int rate_khz = 0;
     if (hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, g.device) != hipSuccess || rate_khz <= 0) rate_khz = 100000;
     d->spin_ticks = (long long)rate_khz * microseconds / 1000;
@@ -1496,14 +1649,14 @@ int mq_decoder_set_patience(mq_decoder* d, int64_t microseconds) {
 
 void mq_decoder_free(mq_decoder* d) {
     if (!d) return;
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     (void)hipDeviceSynchronize();
     decoder_release(d);
 }
 
 // ---------------------------------------------------------------------------------- census
 int mq_debug_set_dense_lds(int on) {
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     const int before = g_dense_lds;
     g_dense_lds = on & 1;
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
@@ -1511,12 +1664,12 @@ int mq_debug_set_dense_lds(int on) {
 }
 
 int mq_census_enable(int on) {
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     census.on = on != 0;
     return MQ_OK;
 }
 int mq_census_reset(void) {
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     if (census.used) (void)hipDeviceSynchronize();
     census.used = 0;
     return MQ_OK;
@@ -1524,7 +1677,7 @@ int mq_census_reset(void) {
 int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int64_t* count) {
     if (int rc = check_ready()) return rc;
     if (kind < 0 || kind >= MQ_KIND_COUNT) return fail(MQ_ERR_INVALID, "mq_census_read: kind %d", kind);
-    std::lock_guard<std::mutex> lock(g.mu);
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
     MQ_HIP(hipDeviceSynchronize());
     double sum = 0.0, lo = 1e30, hi = 0.0;
     int64_t n = 0;
@@ -1562,6 +1715,24 @@ int mq_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes) {
 }
 int mq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes) {
     MQ_HIP(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+    return MQ_OK;
+}
+int mq_host_malloc(void** ptr, size_t bytes) {
+    if (int rc = check_ready()) return rc;
+    if (!ptr || bytes == 0) return fail(MQ_ERR_INVALID, "mq_host_malloc: null pointer or zero size");
+    MQ_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+    return MQ_OK;
+}
+int mq_host_free(void* ptr) {
+    if (ptr) MQ_HIP(hipHostFree(ptr));
+    return MQ_OK;
+}
+int mq_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t bytes, void* stream) {
+    MQ_HIP(hipMemcpyAsync(dst_dev, src_pinned, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    return MQ_OK;
+}
+int mq_memcpy_d2h_async(void* dst_pinned, const void* src_dev, size_t bytes, void* stream) {
+    MQ_HIP(hipMemcpyAsync(dst_pinned, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
     return MQ_OK;
 }
 int mq_stream_synchronize(void* stream) {

@@ -82,6 +82,9 @@ struct MatmulArgs {
 };
 // Waves per workgroup that launch_matmul gives `workgroups` workgroups of rows with nb super-blocks.
 int pick_waves(int64_t nb, int64_t workgroups);
+// Compute units the launch heuristics size their grids for (mq_init sets the device's count; a partitioned device has fewer).
+void set_compute_units(int count);
+int compute_units();
 // start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
@@ -119,6 +122,13 @@ struct Q80MatmulArgs {
     float* y = nullptr;            // [n][ldy]
     int64_t ldy = 0;
     int32_t* dbg_sum = nullptr;    // optional [rows][n][cols / 32] integer block sums
+    // expert-routed mode (the MoE down node with Q8_0 experts): activation / output row g = token * slots + slot is
+    // multiplied by expert pair_ids[token * top_k + slot] (slot < top_k) or by the shared expert sh_w (slot >= top_k);
+    // n = tokens * slots rows; pairs with an id outside [0, n_experts) are skipped
+    const int32_t* pair_ids = nullptr;
+    int top_k = 0, slots = 0, n_experts = 0;
+    size_t expert_bytes = 0;
+    const uint8_t* sh_w = nullptr;
 };
 size_t q80_scale_bytes(int64_t n, int64_t nb);
 // x rows 16-byte aligned (ldx % 4 == 0), cols % 256 == 0

@@ -336,8 +336,14 @@ hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t str
 // aim at having every workgroup of the launch resident at once -- a launch a few workgroups over that waits for
 // a second round that starts when the first ones end -- with a count that divides the super-blocks of a row
 // evenly and at most 8.
+static int g_compute_units = 256;  // what an unpartitioned MI355X has; mq_init replaces it with the device's own count
+void set_compute_units(int count) {
+    if (count > 0) g_compute_units = count;
+}
+int compute_units() { return g_compute_units; }
+
 int pick_waves(int64_t nb, int64_t workgroups) {
-    const int64_t compute_units = 256;
+    const int64_t compute_units = g_compute_units;
     for (int64_t w = nb < 8 ? nb : 8; w > 1; --w)
         if (nb % w == 0 && workgroups <= compute_units * (8 / w)) return (int)w;
     return 1;
@@ -377,7 +383,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
             if (!a.direct_ids && a.n_experts > 0 && a.direct_top_k > 0)
                 expect = (double)a.n_experts * (1.0 - std::pow(1.0 - 1.0 / (double)a.n_experts, (double)(a.n * a.direct_top_k)));
             const double workgroups = (double)rowtiles * (expect + (double)(groups - a.max_groups));
-            const double resident = 2048.0;
+            const double resident = 8.0 * g_compute_units;  // one-wave workgroups the chip holds at once
             if (workgroups > 3.5 * resident) want = 4;
             else if (workgroups > resident) want = 2;
         }

@@ -84,11 +84,27 @@ __global__ void __launch_bounds__(512) q80_matmul_kernel(const Q80MatmulArgs p) 
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const int nb = (int)p.nb;
-    const uint8_t* tiles = p.w + tile_offset(rt, 0, nb, kTile80Bytes);
+    const uint8_t* w = p.w;
+    int first = 0, last = (int)p.n;  // activation rows this workgroup multiplies
+    if (p.pair_ids) {
+        // expert-routed: workgroup column g is hidden row g = token * slots + slot alone, against the expert that the
+        // token's slot names (slots past top_k: the shared expert); rows of dropped pairs are left as they are
+        const int g = blockIdx.y, tok = g / p.slots, k = g - tok * p.slots;
+        if (k < p.top_k) {
+            const int e = p.pair_ids[tok * p.top_k + k];
+            if (e < 0 || e >= p.n_experts) return;  // the whole workgroup, before any barrier
+            w += (size_t)e * p.expert_bytes;
+        } else {
+            w = p.sh_w;
+        }
+        first = g;
+        last = g + 1;
+    }
+    const uint8_t* tiles = w + tile_offset(rt, 0, nb, kTile80Bytes);
     const int cnt = wave < nb ? (nb - wave + n_waves - 1) / n_waves : 0;  // 256-weight groups wave, wave + W, ...
 
-    for (int chunk = 0; chunk < (int)p.n; chunk += kTokTile) {
-        const int count = (int)p.n - chunk < kTokTile ? (int)p.n - chunk : kTokTile;
+    for (int chunk = first; chunk < last; chunk += kTokTile) {
+        const int count = last - chunk < kTokTile ? last - chunk : kTokTile;
         // a dead slot reads a live row of the pass and stores nothing
         const int arow = chunk + ((slot >> 1) < count ? (slot >> 1) : count - 1);
         const size_t a_off = aq_row_offset(arow, nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
@@ -170,7 +186,7 @@ __global__ void __launch_bounds__(512) q80_matmul_kernel(const Q80MatmulArgs p) 
                     if (yrow[j] >= 0) p.y[(size_t)yrow[j] * (size_t)p.ldy + (size_t)row] = acc[j];
             }
         }
-        if (n_waves > 1 && chunk + kTokTile < (int)p.n) __syncthreads();  // red[] is reused by the next pass
+        if (n_waves > 1 && chunk + kTokTile < last) __syncthreads();  // red[] is reused by the next pass
     }
 }
 
@@ -188,9 +204,12 @@ hipError_t launch_quantize_q80(const float* x, int64_t n, int64_t ldx, int64_t c
 
 hipError_t launch_q80_matmul(const Q80MatmulArgs& a, hipStream_t stream) {
     if (a.rows <= 0 || a.nb <= 0 || a.n <= 0 || !a.w || !a.aq || !a.ah || !a.y || a.ldy < a.rows) return hipErrorInvalidValue;
+    if (a.pair_ids && (a.top_k <= 0 || a.slots < a.top_k || a.n % a.slots || a.dbg_sum || (a.slots > a.top_k && !a.sh_w)))
+        return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
-    const int waves = pick_waves(a.nb, rowtiles);
-    hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
+    const int64_t columns = a.pair_ids ? a.n : 1;
+    const int waves = pick_waves(a.nb, rowtiles * columns);
+    hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)rowtiles, (unsigned)columns), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0, stream, a);
     return hipGetLastError();
 }

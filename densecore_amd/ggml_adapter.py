@@ -16,9 +16,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi355q4k_ggml.so")
 
 # every symbol include/mi355_q4k_ggml.h declares
-EXPORTS = [
+CALLBACKS = [
     "mq_cb_gemv_custom", "mq_cb_gemv_batched_custom", "mq_cb_moe_gateup_swiglu", "mq_cb_moe_down_weighted_logits",
-    "mq_ggml_last_status", "mq_ggml_weight_cache_clear", "mq_ggml_weight_cache_size",
+    "mq_cb_moe_fused_router", "mq_cb_moe_topk_weights_from_logits", "mq_cb_mul_mat_id",
+]
+EXPORTS = CALLBACKS + [
+    "mq_ggml_last_status", "mq_ggml_weight_cache_clear", "mq_ggml_weight_cache_size", "mq_ggml_weight_fingerprint",
     "mq_matmul_ggml_quantized_transb",
 ]
 
@@ -40,7 +43,14 @@ GgmlTensor._fields_ = [
 
 
 class UserData(C.Structure):
-    _fields_ = [("silu_mode", C.c_int), ("route_mode", C.c_int), ("use_defaults", C.c_int), ("last_status", C.c_int)]
+    _fields_ = [("silu_mode", C.c_int), ("reserved", C.c_int), ("use_defaults", C.c_int), ("last_status", C.c_int),
+                ("keep_hidden_on_device", C.c_int)]
+
+
+class RouterState(C.Structure):
+    """QwenNativeMoEFusedRouterState (core/src/llm/moe/native.cpp:602-608) as the fused router node's userdata."""
+    _fields_ = [("n_experts", C.c_int64), ("n_tokens", C.c_int64), ("top_k", C.c_int64),
+                ("normalized_weights", C.c_void_p), ("work_ctx", C.c_void_p)]
 
 
 _handle = None
@@ -54,10 +64,12 @@ def lib():
             raise _lib.MqError(f"{LIB_PATH} is missing: run `make -C densecore_amd/host`")
         L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
         cb = [C.POINTER(GgmlTensor), C.c_int, C.c_int, C.c_void_p]
-        for name in EXPORTS[:4]:
+        for name in CALLBACKS:
             getattr(L, name).argtypes = cb
             getattr(L, name).restype = None
         L.mq_ggml_weight_cache_size.restype = C.c_int64
+        L.mq_ggml_weight_fingerprint.argtypes = [C.c_void_p, C.c_size_t]
+        L.mq_ggml_weight_fingerprint.restype = C.c_uint64
         L.mq_matmul_ggml_quantized_transb.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32,
                                                       C.c_int64, C.c_int64, C.c_size_t, C.c_void_p, C.c_int64]
         _handle = L

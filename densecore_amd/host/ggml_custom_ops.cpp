@@ -36,13 +36,15 @@ int note(int rc) {
 }
 
 // ---- device weight cache ---------------------------------------------------------------------
-// Keyed by the host data pointer; shape and strides are compared on every hit so that a graph
-// arena which reuses an address for another tensor is re-uploaded rather than mis-read.
+// Keyed by the host data pointer; type, shape, strides AND a fingerprint of the bytes are compared on every hit, so
+// that an address which now holds other weights (a reloaded model, an mmap reused for another file, a graph arena
+// that recycled the slot) is re-uploaded rather than answered from stale HBM tiles.
 struct CachedWeight {
     mq_weight* handle = nullptr;
     int type = -1;
     int64_t ne[3] = {0, 0, 0};
     size_t nb[3] = {0, 0, 0};
+    uint64_t fingerprint = 0;
 };
 std::mutex g_cache_mu;
 std::unordered_map<const void*, CachedWeight> g_cache;
@@ -64,12 +66,70 @@ bool is_kquant_matrix(const ggml_tensor* w) {
            w->nb[0] == bb && w->nb[1] >= (size_t)(w->ne[0] / kSuperBlock) * bb;
 }
 
+// Content key of a tensor: the byte count, the first and the last 4 KiB and 64 sixteen-byte samples spread evenly
+// between them, mixed eight bytes at a time through four independent multiply-xor streams (a byte-serial hash of
+// these 9 KB would cost more than the node's kernel) -- cheap enough for every node, and any reload that changes the
+// header blocks, the tail or one of the samples changes the key.  The reference keys its prepared weights the same
+// way, by content (FingerprintQ4KRepackedGemvWeight, core/src/kernels/q4k_repacked_gemv.cpp:353-393: length + first
+// and last window; core/tests/runtime/test_q4k_fingerprint.cpp).  0 only for an empty input.
+uint64_t fingerprint_bytes(const void* data, size_t bytes) {
+    if (!data || bytes == 0) return 0;
+    const auto* p = static_cast<const uint8_t*>(data);
+    constexpr uint64_t kMul[4] = {0x9E3779B97F4A7C15ull, 0xC2B2AE3D27D4EB4Full, 0x165667B19E3779F9ull, 0xD6E8FEB86659FD93ull};
+    uint64_t lane[4] = {bytes, ~(uint64_t)bytes, bytes * kMul[0], bytes ^ kMul[1]};
+    uint64_t position = 0;  // words mixed so far: equal words at different places give different keys
+    auto mix = [&](const uint8_t* q, size_t n) {
+        size_t i = 0;
+        for (; i + 8 <= n; i += 8, ++position) {
+            uint64_t w;
+            std::memcpy(&w, q + i, 8);  // any alignment
+            uint64_t& l = lane[position & 3];
+            l = (l ^ w ^ position) * kMul[position & 3];
+            l ^= l >> 29;
+        }
+        if (i < n) {
+            uint64_t w = 0;
+            std::memcpy(&w, q + i, n - i);
+            w |= (uint64_t)(n - i) << 56;
+            uint64_t& l = lane[position & 3];
+            l = (l ^ w ^ position) * kMul[position & 3];
+            l ^= l >> 29;
+            ++position;
+        }
+    };
+    constexpr size_t kWindow = 4096, kSamples = 64, kSampleBytes = 16;
+    if (bytes <= 2 * kWindow) {
+        mix(p, bytes);
+    } else {
+        mix(p, kWindow);
+        const size_t inner = bytes - 2 * kWindow;
+        if (inner >= kSamples * kSampleBytes) {
+            const size_t step = inner / kSamples;
+            for (size_t i = 0; i < kSamples; ++i) mix(p + kWindow + i * step, kSampleBytes);
+        } else {
+            mix(p + kWindow, inner);
+        }
+        mix(p + bytes - kWindow, kWindow);
+    }
+    uint64_t h = 0;
+    for (int i = 0; i < 4; ++i) {
+        h = (h ^ lane[i]) * kMul[(i + 1) & 3];
+        h ^= h >> 32;
+    }
+    return h ? h : 1;
+}
+
 const mq_weight* device_weight(const void* data, int type, int64_t cols, int64_t rows, int64_t n_experts,
                                size_t row_bytes, size_t expert_bytes) {
+    // bytes the tensor spans in host memory (strided rows and experts included)
+    const size_t span = (size_t)(n_experts - 1) * expert_bytes + (size_t)(rows - 1) * row_bytes +
+                        (size_t)(cols / (type == (int)GGML_TYPE_Q8_0 ? 32 : kSuperBlock)) *
+                            (type == (int)GGML_TYPE_Q8_0 ? 34 : kquant_block_bytes(type));
+    const uint64_t fp = fingerprint_bytes(data, span);
     std::lock_guard<std::mutex> lock(g_cache_mu);
     CachedWeight& slot = g_cache[data];
     const bool same = slot.handle && slot.type == type && slot.ne[0] == cols && slot.ne[1] == rows && slot.ne[2] == n_experts &&
-                      slot.nb[1] == row_bytes && slot.nb[2] == expert_bytes;
+                      slot.nb[1] == row_bytes && slot.nb[2] == expert_bytes && slot.fingerprint == fp;
     if (same) return slot.handle;
     if (slot.handle) mq_weight_free(slot.handle);
     slot = CachedWeight{};
@@ -82,6 +142,7 @@ const mq_weight* device_weight(const void* data, int type, int64_t cols, int64_t
     slot.type = type;
     slot.ne[0] = cols, slot.ne[1] = rows, slot.ne[2] = n_experts;
     slot.nb[1] = row_bytes, slot.nb[2] = expert_bytes;
+    slot.fingerprint = fp;
     return h;
 }
 
@@ -90,57 +151,81 @@ const mq_weight* device_weight(const ggml_tensor* w) {
                          w->ne[2] > 1 ? w->nb[2] : w->nb[1] * w->ne[1]);
 }
 
-// ---- per-thread staging in HBM -------------------------------------------------------------------
-// Grow-only device buffers for the host<->device hops of one node; a thread's buffers are reused
-// by its next call (callbacks of one graph run one node at a time per ggml thread 0).
+// ---- per-thread staging ---------------------------------------------------------------------------
+// Grow-only device buffers for the operands of one node, each with a page-locked host twin: graph tensors live in
+// pageable memory, so a row is first copied into the pinned twin (a strided tensor is gathered on the way), then
+// all copies and kernels of the node are queued asynchronously on the null stream and the node synchronises ONCE,
+// before it scatters its result into dst.  A thread's buffers are reused by its next call (callbacks of one graph
+// run one node at a time on ggml thread 0).
 struct Staging {
-    void* ptr = nullptr;
+    void* dev = nullptr;
+    void* pin = nullptr;
     size_t cap = 0;
-    void* get(size_t bytes) {
-        if (bytes <= cap) return ptr;
-        if (ptr) mq_device_free(ptr);
-        ptr = nullptr, cap = 0;
+    bool get(size_t bytes) {
+        if (bytes <= cap) return true;
+        release();
         const size_t want = bytes + bytes / 2 + 4096;
-        if (note(mq_device_malloc(&ptr, want)) != MQ_OK) return nullptr;
+        if (note(mq_device_malloc(&dev, want)) != MQ_OK) return false;
+        if (note(mq_host_malloc(&pin, want)) != MQ_OK) {
+            mq_device_free(dev);
+            dev = nullptr;
+            return false;
+        }
         cap = want;
-        return ptr;
+        return true;
     }
-    ~Staging() {
-        if (ptr) mq_device_free(ptr);
+    void release() {
+        if (dev) mq_device_free(dev);
+        if (pin) mq_host_free(pin);
+        dev = pin = nullptr;
+        cap = 0;
     }
+    ~Staging() { release(); }
 };
 struct ThreadStage {
-    Staging in, aux, ids, wts, out;
+    Staging in, aux, ids, wts, out, keep;
+    // the down node's own buffers for what it uploads: with the hand-over the gate/up node returns while the copies
+    // out of its pinned twins (in, ids) are still queued, so the node after it must not write those twins
+    Staging in2, ids2;
 };
 thread_local ThreadStage t_stage;
 
-// Copies a strided host matrix [rows][cols] of 4-byte elements (row stride in bytes) into a dense
-// device matrix.  Dense sources go in one copy.
-int upload_rows(void* dst_dev, const void* src_host, int64_t rows, int64_t cols, size_t row_stride_bytes) {
+// The gate/up node's result left on the device for the down node of the same graph (mq_ggml_userdata::
+// keep_hidden_on_device): which host tensor it stands for, and its shape.
+struct Resident {
+    const void* host = nullptr;
+    int64_t n_ff = 0, top_k = 0, n = 0;
+};
+thread_local Resident t_resident;
+
+// Gathers a strided host matrix [rows][cols] of 4-byte elements (row stride in bytes) into the pinned twin and queues
+// its copy to the device buffer.
+int upload_rows(Staging& st, size_t offset_bytes, const void* src_host, int64_t rows, int64_t cols, size_t row_stride_bytes) {
     const size_t row_bytes = (size_t)cols * 4;
-    if (row_stride_bytes == row_bytes || rows == 1) return mq_memcpy_h2d(dst_dev, src_host, row_bytes * (size_t)rows);
-    for (int64_t r = 0; r < rows; ++r) {
-        const int rc = mq_memcpy_h2d((char*)dst_dev + (size_t)r * row_bytes,
-                                     (const char*)src_host + (size_t)r * row_stride_bytes, row_bytes);
-        if (rc != MQ_OK) return rc;
+    char* pin = (char*)st.pin + offset_bytes;
+    if (row_stride_bytes == row_bytes || rows == 1) {
+        std::memcpy(pin, src_host, row_bytes * (size_t)rows);
+    } else {
+        for (int64_t r = 0; r < rows; ++r) std::memcpy(pin + (size_t)r * row_bytes, (const char*)src_host + (size_t)r * row_stride_bytes, row_bytes);
     }
-    return MQ_OK;
+    return mq_memcpy_h2d_async((char*)st.dev + offset_bytes, pin, row_bytes * (size_t)rows, nullptr);
 }
 
-int download_rows(void* dst_host, const void* src_dev, int64_t rows, int64_t cols, size_t row_stride_bytes) {
+// Queues the copy of a dense device matrix into its pinned twin; scatter_rows() moves it on after the synchronisation.
+int download_rows(Staging& st, size_t bytes) { return mq_memcpy_d2h_async(st.pin, st.dev, bytes, nullptr); }
+void scatter_rows(void* dst_host, const Staging& st, size_t offset_bytes, int64_t rows, int64_t cols, size_t row_stride_bytes) {
     const size_t row_bytes = (size_t)cols * 4;
-    if (row_stride_bytes == row_bytes || rows == 1) return mq_memcpy_d2h(dst_host, src_dev, row_bytes * (size_t)rows);
-    for (int64_t r = 0; r < rows; ++r) {
-        const int rc = mq_memcpy_d2h((char*)dst_host + (size_t)r * row_stride_bytes,
-                                     (const char*)src_dev + (size_t)r * row_bytes, row_bytes);
-        if (rc != MQ_OK) return rc;
+    const char* pin = (const char*)st.pin + offset_bytes;
+    if (row_stride_bytes == row_bytes || rows == 1) {
+        std::memcpy(dst_host, pin, row_bytes * (size_t)rows);
+    } else {
+        for (int64_t r = 0; r < rows; ++r) std::memcpy((char*)dst_host + (size_t)r * row_stride_bytes, pin + (size_t)r * row_bytes, row_bytes);
     }
-    return MQ_OK;
 }
 
 struct Options {
     int silu_mode;
-    int route_mode;
+    bool keep_hidden;
     mq_ggml_userdata* ud;
 };
 
@@ -150,12 +235,9 @@ Options options_for(void* userdata, int64_t n_tokens) {
     // decode widths use the exact exponential, wider batches the polynomial one
     // (core/src/llm/moe/native.cpp:3614-3616, core/src/backend/cpu_backend_moe_raw_batched.inl:1673)
     o.silu_mode = n_tokens <= 4 ? MQ_SILU_EXACT : MQ_SILU_FAST;
-    o.route_mode = MQ_ROUTE_FLOOR;
+    o.keep_hidden = ud && ud->keep_hidden_on_device != 0;
     o.ud = ud;
-    if (ud && !ud->use_defaults) {
-        o.silu_mode = ud->silu_mode;
-        o.route_mode = ud->route_mode;
-    }
+    if (ud && !ud->use_defaults) o.silu_mode = ud->silu_mode;
     return o;
 }
 
@@ -184,26 +266,47 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
         return finish(o, MQ_ERR_UNSUPPORTED);
     const mq_weight* w = device_weight(weight);
     if (!w) return finish(o, t_status);
-    float* x_dev = (float*)t_stage.in.get((size_t)m * k_in * 4);
-    float* y_dev = (float*)t_stage.out.get((size_t)m * n_out * 4);
-    if (!x_dev || !y_dev) return finish(o, t_status);
-    int rc = upload_rows(x_dev, src->data, m, k_in, src->nb[1]);
-    if (rc == MQ_OK) rc = mq_mul_mat_q4k(w, x_dev, m, k_in, y_dev, n_out, nullptr);
-    if (rc == MQ_OK) rc = download_rows(dst->data, y_dev, m, n_out, dst->nb[1]);  // blocking copy = synchronisation
+    Staging &in = t_stage.in, &out = t_stage.out;
+    if (!in.get((size_t)m * k_in * 4) || !out.get((size_t)m * n_out * 4)) return finish(o, t_status);
+    int rc = upload_rows(in, 0, src->data, m, k_in, src->nb[1]);
+    if (rc == MQ_OK) rc = mq_mul_mat_q4k(w, (const float*)in.dev, m, k_in, (float*)out.dev, n_out, nullptr);
+    if (rc == MQ_OK) rc = download_rows(out, (size_t)m * n_out * 4);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);  // the node's one synchronisation
+    if (rc == MQ_OK) scatter_rows(dst->data, out, 0, m, n_out, dst->nb[1]);
     finish(o, rc);
 }
 
-// selected_experts I32 ne=[top_k, n_tokens] -> dense device [n_tokens][top_k]
-int upload_ids(const ggml_tensor* sel, int32_t** ids_dev) {
+// selected_experts I32 ne=[top_k, n_tokens] -> dense device [n_tokens][top_k] (queued, not synchronised)
+int upload_ids(const ggml_tensor* sel, Staging& st) {
     const int64_t top_k = sel->ne[0], n = sel->ne[1];
-    *ids_dev = (int32_t*)t_stage.ids.get((size_t)n * top_k * 4);
-    if (!*ids_dev) return t_status;
-    if (sel->nb[0] == 4) return upload_rows(*ids_dev, sel->data, n, top_k, sel->nb[1]);
-    std::vector<int32_t> dense((size_t)n * top_k);  // element stride other than 4 bytes: gather on the host
+    if (!st.get((size_t)n * top_k * 4)) return t_status;
+    if (sel->nb[0] == 4) return upload_rows(st, 0, sel->data, n, top_k, sel->nb[1]);
+    auto* dense = (int32_t*)st.pin;  // element stride other than 4 bytes: gather element by element
     for (int64_t t = 0; t < n; ++t)
         for (int64_t k = 0; k < top_k; ++k)
             std::memcpy(&dense[(size_t)(t * top_k + k)], (const char*)sel->data + t * sel->nb[1] + k * sel->nb[0], 4);
-    return mq_memcpy_h2d(*ids_dev, dense.data(), dense.size() * 4);
+    return mq_memcpy_h2d_async(st.dev, st.pin, (size_t)n * top_k * 4, nullptr);
+}
+
+// rows (token, k) of an F32 tensor ne=[cols, top_k, n] whose token stride may differ from top_k * nb[1]
+int upload_pairs(Staging& st, const ggml_tensor* t, int64_t cols, int64_t top_k, int64_t n) {
+    if (t->nb[2] == t->nb[1] * (size_t)top_k) return upload_rows(st, 0, t->data, n * top_k, cols, t->nb[1]);
+    int rc = MQ_OK;
+    for (int64_t tok = 0; tok < n && rc == MQ_OK; ++tok)
+        rc = upload_rows(st, (size_t)tok * top_k * cols * 4, (const char*)t->data + tok * t->nb[2], top_k, cols, t->nb[1]);
+    return rc;
+}
+void scatter_pairs(const ggml_tensor* t, const Staging& st, int64_t cols, int64_t top_k, int64_t n) {
+    if (t->nb[2] == t->nb[1] * (size_t)top_k) return scatter_rows(t->data, st, 0, n * top_k, cols, t->nb[1]);
+    for (int64_t tok = 0; tok < n; ++tok)
+        scatter_rows((char*)t->data + tok * t->nb[2], st, (size_t)tok * top_k * cols * 4, top_k, cols, t->nb[1]);
+}
+
+// A Q8_0 expert stack (34-byte blocks, rows of whole 256-weight groups): the MoE down node takes it
+// (core/src/llm/moe/native.cpp:4611-4616), no other expert node does.
+bool is_q80_stack(const ggml_tensor* w) {
+    return w && w->data && (int)w->type == (int)GGML_TYPE_Q8_0 && w->ne[0] > 0 && w->ne[0] % kSuperBlock == 0 && w->ne[1] > 0 &&
+           w->ne[2] > 0 && w->ne[3] == 1 && w->nb[0] == kQ80BlockBytes && w->nb[1] >= (size_t)(w->ne[0] / 32) * kQ80BlockBytes;
 }
 
 }  // namespace
@@ -223,6 +326,7 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
     const ggml_tensor* input = dst->src[2];
     const ggml_tensor* sel = dst->src[3];
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
+    t_resident = Resident{};
     if (!gate || !up || !input || !sel || !input->data || !sel->data || !dst->data) return finish(o, MQ_ERR_INVALID);
     if (!is_kquant_matrix(gate) || !is_kquant_matrix(up) || gate->type != up->type) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t n_embd = gate->ne[0], n_ff = gate->ne[1], n_expert = gate->ne[2];
@@ -236,24 +340,29 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
     const mq_weight* wg = device_weight(gate);
     const mq_weight* wu = wg ? device_weight(up) : nullptr;
     if (!wg || !wu) return finish(o, t_status);
-    float* x_dev = (float*)t_stage.in.get((size_t)n * n_embd * 4);
-    float* h_dev = (float*)t_stage.out.get((size_t)n * top_k * n_ff * 4);
-    int32_t* ids_dev = nullptr;
-    if (!x_dev || !h_dev) return finish(o, t_status);
+    // with keep_hidden_on_device the result stays in a buffer of its own (the down node's output uses `out`)
+    Staging &in = t_stage.in, &out = o.keep_hidden ? t_stage.keep : t_stage.out;
+    const size_t out_bytes = (size_t)n * top_k * n_ff * 4;
+    if (!in.get((size_t)n * n_embd * 4) || !out.get(out_bytes)) return finish(o, t_status);
     const size_t x_stride = input->ne[1] == n ? input->nb[1] : input->nb[2];
-    int rc = upload_rows(x_dev, input->data, n, n_embd, x_stride);
-    if (rc == MQ_OK) rc = upload_ids(sel, &ids_dev);
-    if (rc == MQ_OK) rc = mq_moe_gateup_swiglu_q4k(wg, wu, x_dev, n, ids_dev, (int)top_k, o.silu_mode, h_dev, nullptr);
-    if (rc == MQ_OK) {
-        // dst may be a strided view (core/src/llm/moe/native.cpp:4201-4209): rows are (token, k) pairs
-        if (dst->nb[2] == dst->nb[1] * (size_t)top_k) {
-            rc = download_rows(dst->data, h_dev, n * top_k, n_ff, dst->nb[1]);
-        } else {
-            for (int64_t t = 0; t < n && rc == MQ_OK; ++t)
-                rc = download_rows((char*)dst->data + t * dst->nb[2], h_dev + (size_t)t * top_k * n_ff, top_k, n_ff,
-                                   dst->nb[1]);
-        }
+    int rc = upload_rows(in, 0, input->data, n, n_embd, x_stride);
+    if (rc == MQ_OK) rc = upload_ids(sel, t_stage.ids);
+    if (rc == MQ_OK)
+        rc = mq_moe_gateup_swiglu_q4k(wg, wu, (const float*)in.dev, n, (const int32_t*)t_stage.ids.dev, (int)top_k, o.silu_mode,
+                                      (float*)out.dev, nullptr);
+    if (rc == MQ_OK && o.keep_hidden) {
+        // The rows stay in HBM for the down node of this graph; dst->data is NOT written and nothing is waited for
+        // (the null stream keeps the order).  The pinned twins of `in` and `ids` are still being read by the queued
+        // copies; the down node uploads through buffers of its own (in2, ids2), and this node writes them again only
+        // after that node's synchronisation.
+        t_resident.host = dst->data;
+        t_resident.n_ff = n_ff, t_resident.top_k = top_k, t_resident.n = n;
+        return finish(o, rc);
     }
+    if (rc == MQ_OK) rc = download_rows(out, out_bytes);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    // dst may be a strided view (core/src/llm/moe/native.cpp:4201-4209): rows are (token, k) pairs
+    if (rc == MQ_OK) scatter_pairs(dst, out, n_ff, top_k, n);
     finish(o, rc);
 }
 
@@ -264,9 +373,11 @@ void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int /*nth*
     const ggml_tensor* sel = dst->src[2];
     const ggml_tensor* logits = dst->src[3];
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
+    const Resident resident = t_resident;  // valid for the node that follows the gate/up node only
+    t_resident = Resident{};
     if (!down || !hidden || !sel || !logits || !hidden->data || !sel->data || !logits->data || !dst->data)
         return finish(o, MQ_ERR_INVALID);
-    if (!is_kquant_matrix(down)) return finish(o, MQ_ERR_UNSUPPORTED);
+    if (!is_kquant_matrix(down) && !is_q80_stack(down)) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t n_ff = down->ne[0], n_embd = down->ne[1], n_expert = down->ne[2];
     const int64_t top_k = sel->ne[0], n = sel->ne[1];
     // operand checks of core/src/llm/moe/native.cpp:3060-3120 and :2309-2317
@@ -277,29 +388,117 @@ void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int /*nth*
         return finish(o, MQ_ERR_INVALID);
     const mq_weight* wd = device_weight(down);
     if (!wd) return finish(o, t_status);
-    float* h_dev = (float*)t_stage.in.get((size_t)n * top_k * n_ff * 4);
-    float* l_dev = (float*)t_stage.aux.get((size_t)n * n_expert * 4);
-    float* w_dev = (float*)t_stage.wts.get((size_t)n * top_k * 4);
-    float* y_dev = (float*)t_stage.out.get((size_t)n * n_embd * 4);
-    int32_t* ids_dev = nullptr;
-    if (!h_dev || !l_dev || !w_dev || !y_dev) return finish(o, t_status);
+    const bool on_device = resident.host == hidden->data && resident.n_ff == n_ff && resident.top_k == top_k && resident.n == n;
+    Staging &hin = t_stage.aux, &lg = t_stage.in2, &wts = t_stage.wts, &out = t_stage.out;
+    if ((!on_device && !hin.get((size_t)n * top_k * n_ff * 4)) || !lg.get((size_t)n * n_expert * 4) || !wts.get((size_t)n * top_k * 4) ||
+        !out.get((size_t)n * n_embd * 4))
+        return finish(o, t_status);
     int rc = MQ_OK;
-    if (hidden->nb[2] == hidden->nb[1] * (size_t)top_k) {
-        rc = upload_rows(h_dev, hidden->data, n * top_k, n_ff, hidden->nb[1]);
-    } else {
-        for (int64_t t = 0; t < n && rc == MQ_OK; ++t)
-            rc = upload_rows(h_dev + (size_t)t * top_k * n_ff, (const char*)hidden->data + t * hidden->nb[2], top_k,
-                             n_ff, hidden->nb[1]);
+    if (!on_device) rc = upload_pairs(hin, hidden, n_ff, top_k, n);
+    const float* h_dev = (const float*)(on_device ? t_stage.keep.dev : hin.dev);
+    if (rc == MQ_OK) rc = upload_rows(lg, 0, logits->data, n, n_expert, logits->nb[1]);
+    if (rc == MQ_OK) rc = upload_ids(sel, t_stage.ids2);
+    const int32_t* ids_dev = (const int32_t*)t_stage.ids2.dev;
+    if (rc == MQ_OK) rc = mq_moe_weights_from_logits((const float*)lg.dev, n_expert, n, ids_dev, (int)top_k, (float*)wts.dev, nullptr);
+    if (rc == MQ_OK) rc = mq_moe_down_weighted_q4k(wd, h_dev, n, ids_dev, (const float*)wts.dev, (int)top_k, (float*)out.dev, nullptr);
+    if (rc == MQ_OK) rc = download_rows(out, (size_t)n * n_embd * 4);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) scatter_rows(dst->data, out, 0, n, n_embd, dst->nb[1]);
+    finish(o, rc);
+}
+
+void mq_cb_moe_fused_router(struct ggml_tensor* dst, int ith, int /*nth*/, void* userdata) {
+    auto* state = static_cast<mq_ggml_router_state*>(userdata);
+    const ggml_tensor* logits = dst ? dst->src[0] : nullptr;
+    if (ith != 0) return;
+    // the checks of cb_qwen_native_moe_fused_router (core/src/llm/moe/native.cpp:710-718): a node that fails them is left alone
+    if (!dst || !state || !logits || !dst->data || !logits->data || dst->type != GGML_TYPE_I32 || logits->type != GGML_TYPE_F32 ||
+        logits->ne[0] != state->n_experts || logits->ne[1] != state->n_tokens || dst->ne[0] != state->top_k ||
+        dst->ne[1] != state->n_tokens || !state->normalized_weights || logits->nb[0] != 4 || dst->nb[0] != 4 ||
+        state->top_k <= 0 || state->top_k > 8 || state->top_k > state->n_experts || state->n_experts > 2048 || state->n_tokens <= 0) {
+        note(MQ_ERR_INVALID);
+        return;
     }
-    if (rc == MQ_OK) rc = upload_rows(l_dev, logits->data, n, n_expert, logits->nb[1]);
-    if (rc == MQ_OK) rc = upload_ids(sel, &ids_dev);
-    if (rc == MQ_OK) rc = mq_moe_weights_from_logits(l_dev, n_expert, n, ids_dev, (int)top_k, w_dev, nullptr);
-    if (rc == MQ_OK) rc = mq_moe_down_weighted_q4k(wd, h_dev, n, ids_dev, w_dev, (int)top_k, y_dev, nullptr);
-    if (rc == MQ_OK) rc = download_rows(dst->data, y_dev, n, n_embd, dst->nb[1]);
+    const int64_t E = state->n_experts, n = state->n_tokens, K = state->top_k;
+    Staging &lg = t_stage.in, &ids = t_stage.ids, &wts = t_stage.wts;
+    if (!lg.get((size_t)n * E * 4) || !ids.get((size_t)n * K * 4) || !wts.get((size_t)n * K * 4)) return;
+    int rc = upload_rows(lg, 0, logits->data, n, E, logits->nb[1]);
+    if (rc == MQ_OK) rc = mq_moe_route_topk((const float*)lg.dev, E, n, (int)K, MQ_ROUTE_FUSED, (int32_t*)ids.dev, (float*)wts.dev, nullptr);
+    if (rc == MQ_OK) rc = download_rows(ids, (size_t)n * K * 4);
+    if (rc == MQ_OK) rc = download_rows(wts, (size_t)n * K * 4);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) {
+        scatter_rows(dst->data, ids, 0, n, K, dst->nb[1]);
+        std::memcpy(state->normalized_weights, wts.pin, (size_t)n * K * 4);  // dense [n_tokens][top_k], as the reference keeps them
+    }
+    note(rc);
+    if (rc != MQ_OK) std::fprintf(stderr, "mi355_q4k adapter: %s\n", mq_last_error());
+}
+
+void mq_cb_moe_topk_weights_from_logits(struct ggml_tensor* dst, int ith, int /*nth*/, void* /*userdata*/) {
+    if (ith != 0) return;
+    // the checks of cb_moe_topk_weights_from_logits (core/src/llm/moe/native.cpp:800-813)
+    if (!dst || !dst->src[0] || !dst->src[1] || !dst->data || !dst->src[0]->data || !dst->src[1]->data) return;
+    const ggml_tensor* logits = dst->src[0];
+    const ggml_tensor* sel = dst->src[1];
+    if (dst->type != GGML_TYPE_F32 || logits->type != GGML_TYPE_F32 || sel->type != GGML_TYPE_I32 || logits->ne[0] <= 0 ||
+        logits->ne[1] <= 0 || sel->ne[0] <= 0 || sel->ne[1] != logits->ne[1] || dst->ne[0] != 1 || dst->ne[1] != sel->ne[0] ||
+        dst->ne[2] != logits->ne[1] || logits->nb[0] != 4 || sel->ne[0] > 8) {
+        note(MQ_ERR_INVALID);
+        return;
+    }
+    const int64_t E = logits->ne[0], n = logits->ne[1], K = sel->ne[0];
+    Staging &lg = t_stage.in, &wts = t_stage.wts;
+    if (!lg.get((size_t)n * E * 4) || !wts.get((size_t)n * K * 4)) return;
+    int rc = upload_rows(lg, 0, logits->data, n, E, logits->nb[1]);
+    if (rc == MQ_OK) rc = upload_ids(sel, t_stage.ids);
+    if (rc == MQ_OK) rc = mq_moe_weights_from_logits((const float*)lg.dev, E, n, (const int32_t*)t_stage.ids.dev, (int)K, (float*)wts.dev, nullptr);
+    if (rc == MQ_OK) rc = download_rows(wts, (size_t)n * K * 4);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) {  // dst ne = [1, top_k, n_tokens]: element (k, token) at k * nb[1] + token * nb[2]
+        const float* w = (const float*)wts.pin;
+        for (int64_t t = 0; t < n; ++t)
+            for (int64_t k = 0; k < K; ++k) std::memcpy((char*)dst->data + k * dst->nb[1] + t * dst->nb[2], &w[t * K + k], 4);
+    }
+    note(rc);
+    if (rc != MQ_OK) std::fprintf(stderr, "mi355_q4k adapter: %s\n", mq_last_error());
+}
+
+void mq_cb_mul_mat_id(struct ggml_tensor* dst, int ith, int /*nth*/, void* userdata) {
+    if (ith != 0 || !dst) return;
+    const ggml_tensor* as = dst->src[0];
+    const ggml_tensor* b = dst->src[1];
+    const ggml_tensor* sel = dst->src[2];
+    Options o = options_for(userdata, sel ? sel->ne[1] : 1);
+    if (!as || !b || !sel || !b->data || !sel->data || !dst->data) return finish(o, MQ_ERR_INVALID);
+    if (!is_kquant_matrix(as)) return finish(o, MQ_ERR_UNSUPPORTED);
+    // ggml_mul_mat_id: as [K, N, n_expert], b F32 [K, n_used or 1, n_tokens], ids I32 [n_used, n_tokens],
+    // dst F32 [N, n_used, n_tokens]
+    const int64_t k_in = as->ne[0], n_out = as->ne[1];
+    const int64_t top_k = sel->ne[0], n = sel->ne[1];
+    const int64_t x_slots = b->ne[1];
+    if (b->type != GGML_TYPE_F32 || sel->type != GGML_TYPE_I32 || dst->type != GGML_TYPE_F32 || b->ne[0] != k_in || b->ne[2] != n ||
+        (x_slots != 1 && x_slots != top_k) || dst->ne[0] != n_out || dst->ne[1] != top_k || dst->ne[2] != n || top_k <= 0 || top_k > 8 ||
+        top_k > as->ne[2] || n <= 0 || b->nb[0] != 4 || dst->nb[0] != 4)
+        return finish(o, MQ_ERR_INVALID);
+    const mq_weight* w = device_weight(as);
+    if (!w) return finish(o, t_status);
+    Staging &in = t_stage.in, &out = t_stage.out;
+    const size_t out_bytes = (size_t)n * top_k * n_out * 4;
+    if (!in.get((size_t)n * x_slots * k_in * 4) || !out.get(out_bytes)) return finish(o, t_status);
+    int rc = upload_pairs(in, b, k_in, x_slots, n);
+    if (rc == MQ_OK) rc = upload_ids(sel, t_stage.ids);
+    if (rc == MQ_OK)
+        rc = mq_mul_mat_id_q4k(w, (const float*)in.dev, n, (int)x_slots, (const int32_t*)t_stage.ids.dev, (int)top_k, (float*)out.dev, nullptr);
+    if (rc == MQ_OK) rc = download_rows(out, out_bytes);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) scatter_pairs(dst, out, n_out, top_k, n);
     finish(o, rc);
 }
 
 int mq_ggml_last_status(void) { return t_status; }
+
+uint64_t mq_ggml_weight_fingerprint(const void* data, size_t bytes) { return fingerprint_bytes(data, bytes); }
 
 int mq_ggml_weight_cache_clear(void) {
     std::lock_guard<std::mutex> lock(g_cache_mu);

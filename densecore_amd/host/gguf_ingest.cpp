@@ -203,9 +203,17 @@ int mq_gguf_open(const char* path, mq_gguf** out) {
         size_t bb = 0;
         int64_t be = 1;
         t.nbytes = 0;
+        for (int d = 0; d < 4; ++d)
+            if (t.ne[d] <= 0) return bail("tensor " + g->names.back() + ": dimension " + std::to_string(d) + " is not positive");
         if (type_layout(t.ggml_type, &bb, &be)) {
-            if (t.ne[0] <= 0 || t.ne[0] % be) return bail("tensor " + g->names.back() + ": row length is not a whole number of blocks");
-            t.nbytes = (uint64_t)(t.ne[0] / be) * bb * (uint64_t)t.ne[1] * (uint64_t)t.ne[2] * (uint64_t)t.ne[3];
+            if (t.ne[0] % be) return bail("tensor " + g->names.back() + ": row length is not a whole number of blocks");
+            // the product of untrusted 64-bit fields: every step checked, so that a crafted table cannot wrap the size
+            // to a small number and slip through the bounds test below
+            uint64_t bytes = (uint64_t)(t.ne[0] / be);
+            bool overflow = __builtin_mul_overflow(bytes, (uint64_t)bb, &bytes);
+            for (int d = 1; d < 4; ++d) overflow = overflow || __builtin_mul_overflow(bytes, (uint64_t)t.ne[d], &bytes);
+            if (overflow) return bail("tensor " + g->names.back() + ": size overflows 64 bits");
+            t.nbytes = bytes;
         }
     }
     const uint64_t header = (uint64_t)(c.p - g->map);
@@ -216,7 +224,9 @@ int mq_gguf_open(const char* path, mq_gguf** out) {
         mq_gguf_tensor& t = g->tensors[i];
         t.name = g->names[i].c_str();
         if (t.offset % g->alignment) return bail("tensor " + g->names[i] + ": misaligned offset");
-        if (base + t.offset > g->size || t.nbytes > g->size - base - t.offset) return bail("tensor " + g->names[i] + ": data runs past the end of the file");
+        // compare before adding: base + offset may wrap
+        const uint64_t room = g->size - base;
+        if (t.offset > room || t.nbytes > room - t.offset) return bail("tensor " + g->names[i] + ": data runs past the end of the file");
         t.data = g->data + t.offset;
         g->by_name.emplace(g->names[i], (int64_t)i);
     }
@@ -274,6 +284,7 @@ int load_kquant(const mq_gguf* g, const char* name, bool q4k_only, mq_weight** o
     if (t.ggml_type != 12 && (q4k_only || (t.ggml_type != 13 && t.ggml_type != 14 && t.ggml_type != 8)))
         return fail(std::string("tensor ") + name + (q4k_only ? " is not GGML_TYPE_Q4_K" : " is not of type Q4_K, Q5_K, Q6_K or Q8_0"));
     if (t.n_dims > 3 || t.ne[3] != 1) return fail(std::string("tensor ") + name + " has more than three dimensions");
+    if (t.ne[0] % 256) return fail(std::string("tensor ") + name + ": row length is not a multiple of 256");
     // bytes of 256 weights of a row: one K-quant super-block, or eight Q8_0 blocks
     const size_t row_bytes = (size_t)(t.ne[0] / 256) * (t.ggml_type == 12 ? 144 : t.ggml_type == 13 ? 176 : t.ggml_type == 14 ? 210 : 272);
     return mq_weight_upload_typed(t.ggml_type, t.data, t.ne[1], t.ne[0], t.ne[2], row_bytes, row_bytes * (size_t)t.ne[1], out);

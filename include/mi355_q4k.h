@@ -362,6 +362,13 @@ int mq_device_malloc(void** ptr, size_t bytes);
 int mq_device_free(void* ptr);
 int mq_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes);
 int mq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes);
+/* Page-locked host memory (allocated, not registered) and copies that are asynchronous on a stream when the host
+ * side is such memory: what the ggml adapters stage graph tensors through, so that a node costs one
+ * synchronisation instead of one per copy. */
+int mq_host_malloc(void** ptr, size_t bytes);
+int mq_host_free(void* ptr);
+int mq_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t bytes, void* stream);
+int mq_memcpy_d2h_async(void* dst_pinned, const void* src_dev, size_t bytes, void* stream);
 int mq_stream_synchronize(void* stream);
 
 #ifdef __cplusplus

@@ -17,7 +17,7 @@
  *
  * All tensor memory is host memory borrowed from the graph.  Weight tensors
  * are uploaded to HBM the first time their data pointer is seen and kept in a
- * process-wide cache keyed by (data, ne, nb) -- the counterpart of
+ * process-wide cache keyed by (data, type, ne, nb, content fingerprint) -- the counterpart of
  * GetOrCreateQ4KRepackedGemvWeight's cache
  * (core/src/kernels/q4k_repacked_gemv.cpp:403-470) -- until
  * mq_ggml_weight_cache_clear().
@@ -38,15 +38,23 @@ extern "C" {
 
 struct ggml_tensor;
 
-/* Optional userdata of every adapter (NULL = defaults).  The graph owns it, as it owns
+/* Optional userdata of the matmul and expert adapters (NULL = defaults).  The graph owns it, as it owns
  * GemvUserData / Qwen35SharedQ8RowsUserData (core/src/llm/runtime/work_context.h:10-11,
  * core/src/llm/moe/native.cpp:1027-1038). */
 typedef struct {
     int silu_mode;    /* MQ_SILU_*  (gate/up node); default MQ_SILU_EXACT for n <= 4, MQ_SILU_FAST above,
                          as core/src/llm/moe/native.cpp:3614-3616 and cpu_backend_moe_raw_batched.inl:1673 choose */
-    int route_mode;   /* MQ_ROUTE_* (down node: weights from logits); default MQ_ROUTE_FLOOR_FINITE */
-    int use_defaults; /* non-zero: ignore the two fields above */
+    int reserved;     /* not read (the down node always resolves its weights as
+                         Qwen35NativeMoEComputeTopKWeightsFromLogits does, core/src/llm/moe/native.cpp:2305-2357) */
+    int use_defaults; /* non-zero: ignore silu_mode */
     int last_status;  /* written by the adapter: MQ_OK or MQ_ERR_* */
+    /* Opt-in hand-over between the two expert nodes of one graph (core/src/llm/moe/native.cpp:4871-4909): non-zero on
+     * the gate/up node's userdata makes that node leave its result in HBM -- dst->data is NOT written and the node
+     * does not synchronise -- and the down node that runs next on the same thread with that tensor as its `hidden`
+     * operand reads it there (no download, no upload, one synchronisation for the pair).  Only for graphs in which
+     * nothing but the down node reads the gate/up node's output (true of the native MoE graph); any other consumer
+     * would read stale host memory. */
+    int keep_hidden_on_device;
 } mq_ggml_userdata;
 
 /* dst F32 ne=[N_out, M]; src[0] = input F32 ne=[K_in, M] (column stride nb[1]); src[1] = weight
@@ -58,17 +66,46 @@ void mq_cb_gemv_batched_custom(struct ggml_tensor* dst, int ith, int nth, void* 
  * input F32 ne=[n_embd, n_tokens], selected_experts I32 ne=[top_k, n_tokens]}.
  * cb_qwen35_native_moe_gateup_raw_qxk_swiglu (core/src/llm/moe/native.cpp:3929-4345, :4871-4874). */
 void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int nth, void* userdata);
-/* dst F32 ne=[n_embd, n_tokens]; src = {down_exps Q4_K ne=[n_ff, n_embd, n_expert], hidden F32
+/* dst F32 ne=[n_embd, n_tokens]; src = {down_exps Q4_K / Q5_K / Q6_K / Q8_0 ne=[n_ff, n_embd, n_expert], hidden F32
  * ne=[n_ff, top_k, n_tokens], selected_experts I32 ne=[top_k, n_tokens], gate_logits F32
  * ne=[n_expert, n_tokens]}.  cb_qwen35_native_moe_down_q5k_weighted_logits
  * (core/src/llm/moe/native.cpp:3051-3295, :4906-4909). */
 void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+
+/* The state block of the fused top-8 router node, laid out as the reference's QwenNativeMoEFusedRouterState
+ * (core/src/llm/moe/native.cpp:602-608): the node's userdata. */
+typedef struct {
+    int64_t n_experts;
+    int64_t n_tokens;
+    int64_t top_k;
+    float* normalized_weights; /* host, [n_tokens][top_k]: written by the node, read by the weights node */
+    void* work_ctx;            /* the reference's InferenceWorkContext*; not touched here */
+} mq_ggml_router_state;
+/* dst I32 ne=[top_k, n_tokens] = the selected experts; src[0] = gate logits F32 ne=[n_experts, n_tokens]; userdata =
+ * mq_ggml_router_state*, whose normalized_weights receive the softmax over the selection (uniform when a selected
+ * logit is not finite).  cb_qwen_native_moe_fused_router (core/src/llm/moe/native.cpp:710-735, emitted at :4831-4834
+ * for one token; ComputeQwenNativeMoEStableTopK :621-676).  A node that fails the reference's checks is left alone. */
+void mq_cb_moe_fused_router(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+/* dst F32 ne=[1, top_k, n_tokens]; src = {logits F32 ne=[n_experts, n_tokens], selected I32 ne=[top_k, n_tokens]}:
+ * softmax of the selected logits over the valid selection, denominator floored at 2^-14, uniform over the valid
+ * entries when nothing finite is left, 0 for ids outside [0, n_experts).  cb_moe_topk_weights_from_logits
+ * (core/src/llm/moe/native.cpp:800-868).  top_k <= 8. */
+void mq_cb_moe_topk_weights_from_logits(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+/* A ggml_mul_mat_id node: dst F32 ne=[N, n_used, n_tokens]; src = {as Q4_K/Q5_K/Q6_K ne=[K, N, n_expert], b F32
+ * ne=[K, n_used or 1, n_tokens], ids I32 ne=[n_used, n_tokens]}; dst[:, k, t] = as[ids[k, t]] . q8k(b[:, k or 0, t]).
+ * The nodes emitted at core/src/llm/moe/native_gemma.cpp:1509-1559 (gate, up, gate_up and down of the routed
+ * experts); rows whose id is outside [0, n_expert) come back as zeros. */
+void mq_cb_mul_mat_id(struct ggml_tensor* dst, int ith, int nth, void* userdata);
 
 /* Status of the calling thread's last adapter call (MQ_OK / MQ_ERR_*). */
 int mq_ggml_last_status(void);
 /* Frees every cached device weight (call when the model is unloaded). */
 int mq_ggml_weight_cache_clear(void);
 int64_t mq_ggml_weight_cache_size(void);
+/* The content key of the weight cache: a multiply-xor hash over the byte count, the first and last 4 KiB and 64
+ * sixteen-byte samples in between (0 for an empty input).  A cached tensor is re-uploaded when its pointer, type, shape, strides or this
+ * value changed -- FingerprintQ4KRepackedGemvWeight's role (core/src/kernels/q4k_repacked_gemv.cpp:353-393). */
+uint64_t mq_ggml_weight_fingerprint(const void* data, size_t bytes);
 
 /* Library-level boundary without a graph: C[M][N] = A[M][K] . W[N][K]^T with W raw ggml Q4_K rows.
  * CpuBackend::MatMulGgmlQuantizedTransB(const Tensor& A, const GgmlQuantizedMatrixView& W, Tensor* C, int)
