@@ -94,6 +94,54 @@ def test_q80_is_refused_where_it_is_not_supported(ops):
     x = cu(synth.normal_f32(84, (1, 256)))
     with pytest.raises(_lib.MqError):
         ops.swiglu_mul_mat(w, w, x, 0)
+    # an expert stack uploads (the MoE down node takes Q8_0 experts, core/src/llm/moe/native.cpp:4611-4616) and comes
+    # back bit for bit, but the K-quant expert products refuse it
+    stack_np = synth.q80_matrix(85, 32, 256).reshape(2, 16, -1)
+    stack = ops.Q4KWeight.from_ggml(stack_np, 256, Q80)
+    assert stack.n_experts == 2 and np.array_equal(stack.to_ggml(), stack_np)
+    ids = cu(np.zeros((1, 1), np.int32))
     with pytest.raises(_lib.MqError):
-        ops.Q4KWeight.from_ggml(synth.q80_matrix(85, 32, 256).reshape(2, 16, -1), 256, Q80)  # expert stack
+        ops.mul_mat_id(stack, x[:, None, :], ids)
+    stack.free()
     w.free()
+
+
+@pytest.mark.parametrize("n", [1, 3, 9, 24])
+def test_moe_layer_with_q80_down_experts_and_shared_expert(ops, n):
+    """Q4_K gate/up experts with Q8_0 down experts (an accepted pairing, core/src/llm/moe/native.cpp:4611-4616) through
+    the whole MoE layer, shared expert included: the layer must equal its own gate/up node followed by the Q8_0 down
+    arithmetic of the reference (hidden row -> Q8_0 -> dot -> += value * weight in k order, :3239-3286) and the
+    sigmoid-gated shared expert."""
+    import torch
+    hidden, inter, E, K = 512, 256, 10, 4
+    ge, ue = (np.stack([synth.q4k_matrix(synth.tensor_seed("q80moe", t, e), inter, hidden) for e in range(E)]) for t in "gu")
+    de = np.stack([synth.q80_matrix(synth.tensor_seed("q80moe", "d", e), hidden, inter) for e in range(E)])
+    sg, su = (synth.q4k_matrix(synth.tensor_seed("q80moe-sh", t), inter, hidden) for t in "gu")
+    sd = synth.q80_matrix(synth.tensor_seed("q80moe-sh", "d"), hidden, inter)
+    gate_inp = synth.normal_f32(8601, (hidden,)) * 0.05
+    x = synth.normal_f32(8600 + n, (n, hidden))
+    lg = synth.normal_f32(8700 + n, (n, E))
+    GE, UE = ops.Q4KWeight.from_ggml(ge, hidden), ops.Q4KWeight.from_ggml(ue, hidden)
+    DE = ops.Q4KWeight.from_ggml(de, inter, Q80)
+    SG, SU = ops.Q4KWeight.from_ggml(sg, hidden), ops.Q4KWeight.from_ggml(su, hidden)
+    SD = ops.Q4KWeight.from_ggml(sd, inter, Q80)
+    xd, lgd = cu(x), cu(lg)
+    y, ids, wts = ops.moe_layer(GE, UE, DE, xd, lgd, K, shared=(SG, SU, SD, cu(gate_inp)), silu=0)
+    ids_ref, w_ref = orc.route_topk(lg, K, 0)
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    # the layer's hidden rows, re-made by the gate/up node and the dense gate/up product on the same inputs
+    hid = ops.moe_gateup_swiglu(GE, UE, xd, ids, 0).cpu().numpy()
+    hid_sh = ops.swiglu_mul_mat(SG, SU, xd, 2).cpu().numpy()
+    w = wts.cpu().numpy()
+    want = np.zeros((n, hidden), np.float32)
+    for t in range(n):
+        for k in range(K):
+            q = orc.quantize_rows_q80(hid[t, k][None])
+            want[t] += np.float32(w[t, k]) * orc.mul_mat_q80_q80(de[ids_ref[t, k]], inter, q)[0].astype(np.float32)
+        q = orc.quantize_rows_q80(hid_sh[t][None])
+        gate = np.float32(1.0) / (np.float32(1.0) + np.exp(-np.float32(np.dot(gate_inp.astype(np.float64), x[t].astype(np.float64)))))
+        want[t] += np.float32(gate) * orc.mul_mat_q80_q80(sd, inter, q)[0].astype(np.float32)
+    got = y.cpu().numpy()
+    assert np.max(np.abs(got - want)) <= 2e-4 * np.max(np.abs(want))
+    for h in (GE, UE, DE, SG, SU, SD):
+        h.free()
