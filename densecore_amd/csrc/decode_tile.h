@@ -196,22 +196,25 @@ __device__ __forceinline__ void compute_tile6(const TileRegs6& t, const ARegs<TT
 // product (eight stages per wavefront): the old three- and four-deep rings padded their tails with two or three real
 // tile requests per wavefront (a quarter more load instructions: 15.7 -> 13.3 us without them), and deeper rings
 // make the wavefronts of a compute unit receive their first tiles one after the other instead of side by side.
+// issue()'s third argument tells whether the request is one of the first two (std::true_type) or a refill inside
+// the loop (std::false_type): a kernel whose stages alternate between two activation blocks keeps each block's
+// operand in its slot and only asks for it the first time.
 template <class Issue, class Consume>
 __device__ __forceinline__ void ring2(int cnt, Issue issue, Consume consume) {
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     if (cnt <= 0) return;
-    issue(S0{}, 0);
+    issue(S0{}, 0, std::true_type{});
     asm volatile("" ::: "memory");  // requests stay in stage order (the scheduler would group them by base register)
-    issue(S1{}, 1);
+    issue(S1{}, 1, std::true_type{});
     asm volatile("" ::: "memory");
     int i = 0;
     for (; i + 2 < cnt; i += 2) {
         consume(S0{}, i);
-        issue(S0{}, i + 2);
+        issue(S0{}, i + 2, std::false_type{});
         asm volatile("" ::: "memory");
         consume(S1{}, i + 1);
-        issue(S1{}, i + 3);
+        issue(S1{}, i + 3, std::false_type{});
         asm volatile("" ::: "memory");
     }
     consume(S0{}, i);

@@ -27,6 +27,7 @@
 // lane's four accumulators belong to ONE weight row (lane%16) and to two activation rows
 // (2*(lane/16) and 2*(lane/16)+1): it needs only that row's scales and writes two outputs.
 #include <cstdlib>
+#include <utility>
 
 #include <hip/hip_ext.h>
 #include <cmath>
@@ -39,6 +40,16 @@
 namespace mq {
 
 namespace {
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // Activation row and output row of entry e of the current group.
 template <bool GROUPED>
@@ -71,7 +82,15 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
 // multiplies while their weight tiles travel -- the block quantizer of quantize_q8k_kernel, so the same codes,
 // scales and result as the stand-alone quantizer followed by this kernel, one launch less.  (With two rows the
 // repeated quantization costs what the saved launch gains, with four it loses a third.)
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false>
+// REUSE_A (one-wave workgroups over several row tiles of rows that are two super-blocks long, the expert down
+// projections): stage i multiplies super-block i % 2, which is also its register slot, so every slot keeps the
+// activation operand it received with its first stage and later stages ask for weight tiles only -- a third of the
+// load instructions instead of all of them (a stage is three tile loads and six operand loads).
+// BM > 0 (one-wave workgroups over BM row tiles, an even number of super-blocks per row): the stages run block-major
+// -- super-block b of all BM row tiles, then super-block b + 1 -- so that the activation operand of a super-block is
+// requested once per workgroup instead of once per row tile (six of a stage's twelve load instructions are operand
+// loads); each row tile keeps its own accumulators and all of them are stored at the end.
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false, bool REUSE_A = false, int BM = 0>
 __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
     extern __shared__ float red[];  // [W-1][NMAT][TT][2][64]
@@ -183,6 +202,62 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 }
         };
 
+        if constexpr (BM > 0) {
+            // ---- block-major over BM row tiles: stage k of a pair of super-blocks (bb, bb + 1) is row tile k % BM of
+            // super-block bb + k / BM; register slot k % 2 for the tiles, operand set (k / BM) % 2 for the activations.
+            float accr[BM][NMAT][TT][2];
+#pragma unroll
+            for (int r = 0; r < BM; ++r)
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int tt = 0; tt < TT; ++tt) accr[r][m][tt][0] = accr[r][m][tt][1] = 0.0f;
+            typename TileOf<WT>::Regs ring_t[2][NMAT];
+            ARegs<TT> a_set[2];
+            auto issue_k = [&](auto k_c, int bb) {
+                constexpr int k = decltype(k_c)::value;
+                constexpr int st = k & 1, par = (k / BM) & 1, r = k % BM;
+                const int b = bb + k / BM;
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + ((size_t)r * nb + b) * kTileStride, lane);
+                if constexpr (r == 0) load_a<TT>(a_set[par], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
+                asm volatile("" ::: "memory");  // requests stay in stage order
+            };
+            auto consume_k = [&](auto k_c) {
+                constexpr int k = decltype(k_c)::value;
+                constexpr int st = k & 1, par = (k / BM) & 1, r = k % BM;
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m) {
+                    int32_t dsum[TT][2], msum[TT][2];
+                    if (GROUPED && TT == 1 && count == 1)  // most expert groups hold one row: its partner row is not formed
+                        compute_tile_wt<TT, WT, 1>(ring_t[st][m], a_set[par], accr[r][m], dsum, msum, lane);
+                    else
+                        compute_tile_wt<TT, WT, J>(ring_t[st][m], a_set[par], accr[r][m], dsum, msum, lane);
+                }
+            };
+            auto pair_of_blocks = [&](int bb, auto refill_c) {  // refill: the pair after this one exists
+                constexpr bool refill = decltype(refill_c)::value;
+                static_for<2 * BM>([&](auto k_c) {
+                    constexpr int k = decltype(k_c)::value;
+                    consume_k(k_c);
+                    if constexpr (k + 2 < 2 * BM) issue_k(std::integral_constant<int, k + 2>{}, bb);
+                    else if constexpr (refill) issue_k(std::integral_constant<int, k + 2 - 2 * BM>{}, bb + 2);
+                });
+            };
+            issue_k(std::integral_constant<int, 0>{}, 0);
+            issue_k(std::integral_constant<int, 1>{}, 0);
+            int bb = 0;
+            for (; bb + 2 < (int)nb; bb += 2) pair_of_blocks(bb, std::true_type{});
+            pair_of_blocks(bb, std::false_type{});
+#pragma unroll
+            for (int r = 0; r < BM; ++r) {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int tt = 0; tt < TT; ++tt) acc[m][tt][0] = accr[r][m][tt][0], acc[m][tt][1] = accr[r][m][tt][1];
+                store_rows(rt + r);
+            }
+        } else
         // Stage i of this wave is super-block wave + i*W (several row tiles in a one-wave workgroup: tile i of the
         // contiguous run); two register stages, one in flight while the other is multiplied (ring2: no request is
         // ever made past the last stage).  All branches are wave-uniform and the loads themselves unconditional.
@@ -192,8 +267,9 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             typename TileOf<WT>::Regs ring_t[2][NMAT];
             ARegs<TT> ring_a[2];
             float4 ring_x[2];
-            auto issue = [&](auto st_c, int i) {
+            auto issue = [&](auto st_c, int i, auto first_c) {
                 constexpr int st = decltype(st_c)::value;
+                constexpr bool first = decltype(first_c)::value;
                 // i == cnt (once, when cnt is odd): the same loads from fixed addresses in all lanes, a cache line each
                 const bool valid = i < cnt;
                 // several row tiles (one wave, per_rt == nb): stage i is tile i of the contiguous run,
@@ -205,6 +281,8 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
                 for (int m = 0; m < NMAT; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)t * kTileStride, ln);
                 if constexpr (XQ) {
                     ring_x[st] = *reinterpret_cast<const float4*>(p.xf + (size_t)b * kQK + ln * 4);
+                } else if constexpr (REUSE_A && !first) {
+                    // slot st still holds super-block st's operand
                 } else {
                     size_t off[TT];
 #pragma unroll
@@ -317,15 +395,15 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
     }
 }
 
-template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false>
+template <int NMAT, int TT, bool GROUPED, bool DEBUG, int WT, int J = 2, bool XQ = false, bool REUSE_A = false, int BM = 0>
 hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const size_t lds = waves > 1 ? (size_t)(waves - 1) * NMAT * TT * 2 * 64 * sizeof(float) : 0;
     if (start && stop) {
         // the events take the dispatch's own begin / end timestamps: no extra packets around the kernel
-        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ>), grid, dim3(64 * waves), lds, stream, start, stop,
+        hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ, REUSE_A, BM>), grid, dim3(64 * waves), lds, stream, start, stop,
                               0, a);
     } else {
-        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ>), grid, dim3(64 * waves), lds, stream, a);
+        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ, REUSE_A, BM>), grid, dim3(64 * waves), lds, stream, a);
     }
     return hipGetLastError();
 }
@@ -366,27 +444,18 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     const int waves = pick_waves(a.nb, rowtiles * groups);
     // Short rows (few super-blocks) in one-wave workgroups: let a workgroup stream several row tiles, so that
     // its look-ups and activation addressing are paid once per ~16 tiles rather than once per row tile.
-    // Expert-grouped gate/up with more one-wave workgroups than the chip holds at once (8 per compute unit): the ones
-    // left over start when the first ones end and pay their group look-ups again, so a workgroup takes two row
-    // tiles, four when even that leaves more than three rounds (measured, MoE block of 256 experts, top-8: 73 -> 68 us
-    // at 16 tokens, 100 -> 97 at 32, 143 -> 137 at 64; more row tiles than that leave too few wavefronts, and the
-    // down launch, whose workgroups already take eight row tiles, loses with any more).  The number of groups is
-    // only known on the device; its expectation for uniform routing stands in.  With the fused output quantization
-    // a workgroup must stay inside one 256-row block (16 row tiles).
+    // Expert-grouped gate/up in one-wave workgroups: a workgroup takes two row tiles and runs them block-major, so
+    // that the activation operand of a super-block is requested once for both and the group look-ups are paid half as
+    // often (measured, MoE block of 256 experts, top-8, row tiles per workgroup 1 / 2 / 4: 55.5 / 52.9 / 55.7 us at 12
+    // tokens, 61.2 / 55.9 / 57.2 at 16, 80.0 / 74.6 / 79.8 at 32, 106.2 / 100.5 / 99.3 at 64, 148.1 / 137.8 / 149.2 at
+    // 128; the down launch, whose workgroups already take eight row tiles, loses with any more).  With the fused output
+    // quantization a workgroup must stay inside one 256-row block (16 row tiles).
     MatmulArgs b = a;
     b.rt_per_wg = 1;
     if (waves == 1 && !debug) {
         int64_t want = 16 / (a.nb * nmat);
         if (want < 1) want = 1;
-        if (a.grouped && nmat == 2 && want == 1) {
-            double expect = (double)a.max_groups;
-            if (!a.direct_ids && a.n_experts > 0 && a.direct_top_k > 0)
-                expect = (double)a.n_experts * (1.0 - std::pow(1.0 - 1.0 / (double)a.n_experts, (double)(a.n * a.direct_top_k)));
-            const double workgroups = (double)rowtiles * (expect + (double)(groups - a.max_groups));
-            const double resident = 8.0 * g_compute_units;  // one-wave workgroups the chip holds at once
-            if (workgroups > 3.5 * resident) want = 4;
-            else if (workgroups > resident) want = 2;
-        }
+        if (a.grouped && nmat == 2 && want == 1) want = 2;
         if (a.out_aq) {
             while (want > 1 && ((want & (want - 1)) || want > 16)) --want;  // a power of two up to 16 (rows % 256 == 0)
         } else {
@@ -398,6 +467,11 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
 
 #define MQ_LAUNCH_WT(NM, T, W)                                                                            \
     do {                                                                                                  \
+        if (a.grouped && NM == 1 && T == 1 && waves == 1 && b.rt_per_wg > 1 && a.nb == 2)                  \
+            return launch_one<1, 1, true, false, W, 2, false, true>(b, waves, grid, stream, start, stop);  \
+        /* block-major order where its registers fit: Q4_K and Q5_K */                                        \
+        if (a.grouped && NM == 2 && T == 1 && waves == 1 && b.rt_per_wg == 2 && a.nb % 2 == 0 && W != kWtQ6) \
+            return launch_one<2, 1, true, false, W == kWtQ6 ? kWtQ4 : W, 2, false, false, 2>(b, waves, grid, stream, start, stop); \
         if (a.grouped) return launch_one<NM, T, true, false, W>(b, waves, grid, stream, start, stop);     \
         if (debug) return launch_one<NM, T, false, true, W>(b, waves, grid, stream, start, stop);         \
         if (T == 1 && a.xf) return launch_one<NM, 1, false, false, W, 1, true>(b, waves, grid, stream, start, stop); \
