@@ -30,10 +30,10 @@ RING = 8
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0          # dense int8 MFMA, MI355X
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
-# `bench.py --kernel-only`: 32,524.6 KiB fetched and 210.0 KiB written per dispatch on average, each scaled by what
+# `bench.py --kernel-only`: 32,585.1 KiB fetched and 210.0 KiB written per dispatch on average, each scaled by what
 # the same counter reads for the 256 MiB copy of `bench.py --copy-calibration` (FETCH_SIZE 131,083.8 KiB -> x2.000,
-# WRITE_SIZE 262,144.0 KiB -> x1.000): 66,610,000 B read + 215,000 B written.
-TRAFFIC_BYTES_PER_LAUNCH = 66825000
+# WRITE_SIZE 262,144.0 KiB -> x1.000): 66,728,000 B read + 215,000 B written.
+TRAFFIC_BYTES_PER_LAUNCH = 66943000
 Q4K_MATRIX_BYTES = INTER * (HIDDEN // 256) * 144          # 33,030,144: the same for gate, up and down
 
 
@@ -69,6 +69,8 @@ def main() -> int:
                     help="only run the back-to-back launches of the dominant kernel (for counter passes) and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run the 14336x4096 prefill GEMM at M = 2048 ten times (for counter passes) and exit")
+    ap.add_argument("--decode-step-only", type=int, default=0, metavar="N",
+                    help="only replay the 40-layer decoder step at N tokens ten times, one launch per graph node (for kernel traces), and exit")
     ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -103,6 +105,22 @@ def main() -> int:
             ops.gemm(W, x, out=y)
         torch.cuda.synchronize()
         print(json.dumps({"prefill_only": "prefill_gemm_kernel", "M": 2048, "launches": 10}))
+        return 0
+
+    if args.decode_step_only:
+        from densecore_amd import decode_step
+        n = args.decode_step_only
+        cfg = decode_step.StepConfig(synthetic_logits=True)
+        st = decode_step.DecodeStep(cfg, n)
+        x = torch.randn((n, cfg.hidden), device=dev, generator=torch.Generator(device=dev).manual_seed(100 + n))
+        st.run(x)
+        torch.cuda.synchronize()
+        st.x.copy_(x)
+        st.capture()
+        for _ in range(10):
+            st.replay()
+        torch.cuda.synchronize()
+        print(json.dumps({"decode_step_only": n, "layers": cfg.n_layers, "replays": 10}))
         return 0
 
     # ---------------------------------------------------------------- resident data
