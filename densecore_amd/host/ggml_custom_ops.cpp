@@ -58,7 +58,7 @@ bool is_q80_matrix(const ggml_tensor* w) {
 }
 
 // Q4_K, Q5_K or Q6_K rows of whole super-blocks (the K-quant weight types of the callbacks replaced:
-// core/src/llm/moe/native.cpp:2745-2752, core/src/backend/cpu_backend_moe_raw_batched.inl:1552)
+// core/src/llm/moe/native.cpp:4611-4620, core/src/backend/cpu_backend_moe_raw_batched.inl:1552)
 bool is_kquant_matrix(const ggml_tensor* w) {
     if (!w || !w->data) return false;
     const size_t bb = kquant_block_bytes((int)w->type);
@@ -197,6 +197,17 @@ struct Resident {
     int64_t n_ff = 0, top_k = 0, n = 0;
 };
 thread_local Resident t_resident;
+// True between a gate/up node that handed its rows over (and returned without waiting) and the next synchronisation
+// of this thread: the pinned twins of `in` and `ids` may still be read by queued copies.
+thread_local bool t_unsettled = false;
+
+// Every node but the down node of a hand-over starts here: if the previous node left copies queued, wait for them
+// before this node writes the same pinned twins (a graph whose gate/up node is not followed by its down node).
+void settle() {
+    if (!t_unsettled) return;
+    (void)mq_stream_synchronize(nullptr);
+    t_unsettled = false;
+}
 
 // Gathers a strided host matrix [rows][cols] of 4-byte elements (row stride in bytes) into the pinned twin and queues
 // its copy to the device buffer.
@@ -253,6 +264,8 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
     const ggml_tensor* src = dst->src[0];
     const ggml_tensor* weight = dst->src[1];
     Options o = options_for(userdata, 1);
+    settle();
+    t_resident = Resident{};
     if (!src || !weight || !src->data || !dst->data) return finish(o, MQ_ERR_INVALID);
     if ((!is_kquant_matrix(weight) && !is_q80_matrix(weight)) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t k_in = weight->ne[0], n_out = weight->ne[1];
@@ -262,7 +275,9 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
         dst->ne[1] * dst->ne[2] * dst->ne[3] != m || src->nb[0] != 4 || dst->nb[0] != 4 || m <= 0)
         return finish(o, MQ_ERR_INVALID);
     if ((src->ne[2] > 1 && src->nb[2] != src->nb[1] * (size_t)src->ne[1]) ||
-        (dst->ne[2] > 1 && dst->nb[2] != dst->nb[1] * (size_t)dst->ne[1]))
+        (dst->ne[2] > 1 && dst->nb[2] != dst->nb[1] * (size_t)dst->ne[1]) ||
+        (src->ne[3] > 1 && src->nb[3] != src->nb[2] * (size_t)src->ne[2]) ||
+        (dst->ne[3] > 1 && dst->nb[3] != dst->nb[2] * (size_t)dst->ne[2]))
         return finish(o, MQ_ERR_UNSUPPORTED);
     const mq_weight* w = device_weight(weight);
     if (!w) return finish(o, t_status);
@@ -326,6 +341,7 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
     const ggml_tensor* input = dst->src[2];
     const ggml_tensor* sel = dst->src[3];
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
+    settle();
     t_resident = Resident{};
     if (!gate || !up || !input || !sel || !input->data || !sel->data || !dst->data) return finish(o, MQ_ERR_INVALID);
     if (!is_kquant_matrix(gate) || !is_kquant_matrix(up) || gate->type != up->type) return finish(o, MQ_ERR_UNSUPPORTED);
@@ -333,7 +349,8 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
     const int64_t top_k = sel->ne[0], n = sel->ne[1];
     // operand checks of core/src/llm/moe/native.cpp:3935-3990
     if (up->ne[0] != n_embd || up->ne[1] != n_ff || up->ne[2] != n_expert || input->type != GGML_TYPE_F32 ||
-        input->ne[0] != n_embd || input->ne[1] * input->ne[2] != n || sel->type != GGML_TYPE_I32 ||
+        input->ne[0] != n_embd || input->ne[1] * input->ne[2] != n || (input->ne[1] != n && input->ne[1] != 1) ||
+        sel->type != GGML_TYPE_I32 ||
         dst->type != GGML_TYPE_F32 || dst->ne[0] != n_ff || dst->ne[1] != top_k || dst->ne[2] != n || top_k <= 0 ||
         top_k > 8 || n <= 0 || input->nb[0] != 4 || dst->nb[0] != 4)
         return finish(o, MQ_ERR_INVALID);
@@ -357,6 +374,7 @@ void mq_cb_moe_gateup_swiglu(struct ggml_tensor* dst, int ith, int /*nth*/, void
         // after that node's synchronisation.
         t_resident.host = dst->data;
         t_resident.n_ff = n_ff, t_resident.top_k = top_k, t_resident.n = n;
+        t_unsettled = true;
         return finish(o, rc);
     }
     if (rc == MQ_OK) rc = download_rows(out, out_bytes);
@@ -389,6 +407,7 @@ void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int /*nth*
     const mq_weight* wd = device_weight(down);
     if (!wd) return finish(o, t_status);
     const bool on_device = resident.host == hidden->data && resident.n_ff == n_ff && resident.top_k == top_k && resident.n == n;
+    if (!on_device) settle();
     Staging &hin = t_stage.aux, &lg = t_stage.in2, &wts = t_stage.wts, &out = t_stage.out;
     if ((!on_device && !hin.get((size_t)n * top_k * n_ff * 4)) || !lg.get((size_t)n * n_expert * 4) || !wts.get((size_t)n * top_k * 4) ||
         !out.get((size_t)n * n_embd * 4))
@@ -403,6 +422,7 @@ void mq_cb_moe_down_weighted_logits(struct ggml_tensor* dst, int ith, int /*nth*
     if (rc == MQ_OK) rc = mq_moe_down_weighted_q4k(wd, h_dev, n, ids_dev, (const float*)wts.dev, (int)top_k, (float*)out.dev, nullptr);
     if (rc == MQ_OK) rc = download_rows(out, (size_t)n * n_embd * 4);
     if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) t_unsettled = false;
     if (rc == MQ_OK) scatter_rows(dst->data, out, 0, n, n_embd, dst->nb[1]);
     finish(o, rc);
 }
@@ -411,6 +431,8 @@ void mq_cb_moe_fused_router(struct ggml_tensor* dst, int ith, int /*nth*/, void*
     auto* state = static_cast<mq_ggml_router_state*>(userdata);
     const ggml_tensor* logits = dst ? dst->src[0] : nullptr;
     if (ith != 0) return;
+    settle();
+    t_resident = Resident{};
     // the checks of cb_qwen_native_moe_fused_router (core/src/llm/moe/native.cpp:710-718): a node that fails them is left alone
     if (!dst || !state || !logits || !dst->data || !logits->data || dst->type != GGML_TYPE_I32 || logits->type != GGML_TYPE_F32 ||
         logits->ne[0] != state->n_experts || logits->ne[1] != state->n_tokens || dst->ne[0] != state->top_k ||
@@ -437,6 +459,8 @@ void mq_cb_moe_fused_router(struct ggml_tensor* dst, int ith, int /*nth*/, void*
 
 void mq_cb_moe_topk_weights_from_logits(struct ggml_tensor* dst, int ith, int /*nth*/, void* /*userdata*/) {
     if (ith != 0) return;
+    settle();
+    t_resident = Resident{};
     // the checks of cb_moe_topk_weights_from_logits (core/src/llm/moe/native.cpp:800-813)
     if (!dst || !dst->src[0] || !dst->src[1] || !dst->data || !dst->src[0]->data || !dst->src[1]->data) return;
     const ggml_tensor* logits = dst->src[0];
@@ -470,6 +494,8 @@ void mq_cb_mul_mat_id(struct ggml_tensor* dst, int ith, int /*nth*/, void* userd
     const ggml_tensor* b = dst->src[1];
     const ggml_tensor* sel = dst->src[2];
     Options o = options_for(userdata, sel ? sel->ne[1] : 1);
+    settle();
+    t_resident = Resident{};
     if (!as || !b || !sel || !b->data || !sel->data || !dst->data) return finish(o, MQ_ERR_INVALID);
     if (!is_kquant_matrix(as)) return finish(o, MQ_ERR_UNSUPPORTED);
     // ggml_mul_mat_id: as [K, N, n_expert], b F32 [K, n_used or 1, n_tokens], ids I32 [n_used, n_tokens],

@@ -205,6 +205,50 @@ def test_hidden_rows_handed_over_on_the_device(ga, n):
     assert np.array_equal(y2.view(np.uint32), y_host.view(np.uint32))
 
 
+def test_hand_over_followed_by_another_node(ga):
+    """A gate/up node that handed its rows over returns while its uploads are still queued.  If the node after it is
+    NOT its down node -- here a second gate/up node with other input, then a dense node -- that node first waits for
+    the queued copies before it reuses the staging buffers: both results equal the runs without any hand-over."""
+    hidden, inter, n_exp, top_k, n = 512, 256, 8, 2, 4
+    gate = np.stack([synth.q4k_matrix(5610 + e, inter, hidden) for e in range(n_exp)])
+    up = np.stack([synth.q4k_matrix(5620 + e, inter, hidden) for e in range(n_exp)])
+    tg = ga.tensor(gate, ga.GGML_TYPE_Q4_K, [hidden, inter, n_exp])
+    tu = ga.tensor(up, ga.GGML_TYPE_Q4_K, [hidden, inter, n_exp])
+    xs = [synth.normal_f32(5630 + i, (n, hidden)) for i in range(2)]
+    ids = [orc.route_topk(synth.normal_f32(5640 + i, (n, n_exp)), top_k, 1)[0] for i in range(2)]
+    dense = synth.q4k_matrix(5650, 128, hidden)
+    tw = ga.tensor(dense, ga.GGML_TYPE_Q4_K, [hidden, 128])
+
+    def gateup(i, keep):
+        hid = np.zeros((n, top_k, inter), np.float32)
+        th = ga.tensor(hid, ga.GGML_TYPE_F32, [inter, top_k, n])
+        tx = ga.tensor(xs[i], ga.GGML_TYPE_F32, [hidden, n])
+        ts = ga.tensor(ids[i], ga.GGML_TYPE_I32, [top_k, n])
+        ud = ga.UserData(0, 0, 1, 0, 1 if keep else 0)
+        ga.set_src(th, tg, tu, tx, ts)
+        ga.lib().mq_cb_moe_gateup_swiglu(C.byref(th), 0, 8, C.byref(ud))
+        assert ud.last_status == 0
+        return hid
+
+    def dense_node(i):
+        y = np.zeros((n, 128), np.float32)
+        ty = ga.tensor(y, ga.GGML_TYPE_F32, [128, n])
+        tx = ga.tensor(xs[i], ga.GGML_TYPE_F32, [hidden, n])
+        ga.set_src(ty, tx, tw)
+        ga.lib().mq_cb_gemv_batched_custom(C.byref(ty), 0, 1, None)
+        assert ga.lib().mq_ggml_last_status() == 0
+        return y
+
+    want_hid, want_y = gateup(1, False), dense_node(0)
+    for _ in range(3):
+        gateup(0, True)                      # rows kept on the device, uploads still queued
+        got_hid = gateup(1, False)           # another node reuses the same staging buffers
+        assert np.array_equal(got_hid.view(np.uint32), want_hid.view(np.uint32))
+        gateup(1, True)
+        got_y = dense_node(0)
+        assert np.array_equal(got_y.view(np.uint32), want_y.view(np.uint32))
+
+
 def test_weight_cache_notices_new_contents_at_the_same_address(ga):
     """A model reloaded into the same buffer (same pointer, shape and strides, other bytes) must not be answered from
     the tiles of the old one: the cache key holds a fingerprint of the contents."""
