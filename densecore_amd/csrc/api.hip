@@ -1659,6 +1659,7 @@ int mq_debug_set_dense_lds(int on) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     const int before = g_dense_lds;
     g_dense_lds = on & 1;
+    set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;
 }

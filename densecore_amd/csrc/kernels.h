@@ -88,6 +88,14 @@ int compute_units();
 // start/stop (both or neither): events that receive the kernel dispatch's own begin and end timestamps.
 hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
+// ---- grouped_lds.hip -------------------------------------------------------------------------
+// Expert-grouped launches with many groups: a group's activation rows gathered into LDS once per workgroup of eight
+// wavefronts (the same bits as matmul_kernel's one-wave workgroups).
+bool grouped_lds_applies(const MatmulArgs& a);
+hipError_t launch_grouped_lds(const MatmulArgs& a, int rt_per_wave, int groups, hipStream_t stream, hipEvent_t start = nullptr,
+                              hipEvent_t stop = nullptr);
+void set_grouped_lds(bool on);  // debug switch: off keeps these launches on matmul_kernel
+
 // ---- dense_lds.hip ---------------------------------------------------------------------------
 // Dense product for 1..16 rows with the quantized activations staged once per workgroup in LDS (same bits as
 // launch_matmul on the same operands).  Either (aq, ad) -- the A-major workspace -- or xf: fp32 rows (n <= 8,

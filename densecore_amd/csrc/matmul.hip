@@ -36,6 +36,7 @@
 #include "kernels.h"
 #include "decode_tile.h"
 #include "q8k_block.h"
+#include "group_entry.h"
 
 namespace mq {
 
@@ -49,29 +50,6 @@ __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int
 template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-// Activation row and output row of entry e of the current group.
-template <bool GROUPED>
-__device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_group, int begin, int e, int& ar, int& yr) {
-    if (!GROUPED) {
-        ar = e;
-        yr = e;
-    } else if (shared_group) {
-        ar = (begin + e) * p.sh_arow_stride + p.sh_arow_offset;
-        yr = (begin + e) * p.sh_yrow_stride + p.sh_yrow_offset;
-    } else {
-        int tok, kk;
-        if (p.direct_ids) {  // few tokens: the group is the one pair `begin` = (token, slot); e is always 0
-            tok = begin / p.direct_top_k;  // wave-uniform
-            kk = begin - tok * p.direct_top_k;
-        } else {
-            tok = p.entry_token[begin + e];
-            kk = p.entry_k[begin + e];
-        }
-        ar = tok * p.a_tok_stride + kk * p.a_k_stride;
-        yr = tok * p.y_tok_stride + kk * p.y_k_stride;
-    }
 }
 
 // One workgroup: row tile blockIdx.x of group blockIdx.y (dense mode has a single group); its
@@ -450,6 +428,19 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     // tokens, 61.2 / 55.9 / 57.2 at 16, 80.0 / 74.6 / 79.8 at 32, 106.2 / 100.5 / 99.3 at 64, 148.1 / 137.8 / 149.2 at
     // 128; the down launch, whose workgroups already take eight row tiles, loses with any more).  With the fused output
     // quantization a workgroup must stay inside one 256-row block (16 row tiles).
+    // Many groups (one-wave workgroups) of rows at least four super-blocks long: the kernel that gathers a group's rows
+    // into LDS once per eight wavefronts, a row tile per wavefront (two while a wavefront would have fewer than eight
+    // stages).  Measured on the MoE block of 256 experts, 2048 x 512, top-8: gate/up + SwiGLU 54.3 -> 52.1 us per
+    // block at 16 tokens, 80.3 -> 73.4 at 32, 99.4 -> 93.6 at 64, 131.7 -> 123.8 at 128; mul_mat_id over the same
+    // gate experts alone 24.8 -> 22.6 / 32.3 -> 28.9 / 46.0 -> 34.9 us at 16 / 32 / 64 tokens.  The down experts' rows
+    // (two super-blocks) gain nothing there (the launch below keeps their operand in registers) and stay.
+    if (a.grouped && waves == 1 && tt == 1 && a.nb >= 4 && grouped_lds_applies(a)) {
+        int per_wave = 1;
+        if (!a.out_aq) {
+            while (per_wave < 8 && per_wave * a.nb * nmat < 8 && rowtiles >= 16 * per_wave) per_wave *= 2;
+        }
+        return launch_grouped_lds(a, per_wave, groups, stream, start, stop);
+    }
     MatmulArgs b = a;
     b.rt_per_wg = 1;
     if (waves == 1 && !debug) {

@@ -352,9 +352,11 @@ int mq_census_reset(void);
 int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int64_t* count);
 
 /* Debug switch: dense products of up to 16 rows normally run on the kernel that stages the quantized activations
- * in LDS once per workgroup (and, for up to four fp32 rows, quantizes them itself); on = 0 keeps them on the
- * kernel that reads its operand from global memory at every stage.  Both return the same bits
- * (tests/test_gpu_dense_lds.py); returns the previous setting.  No counterpart in the reference. */
+ * in LDS once per workgroup (and, for up to four fp32 rows, quantizes them itself), and expert-grouped launches
+ * with many groups on the kernel that gathers a group's rows into LDS once per eight wavefronts; on = 0 keeps
+ * both on the kernel that reads its operand from global memory at every stage, on = 5 only the expert-grouped
+ * ones.  All return the same bits (tests/test_gpu_dense_lds.py, tests/test_gpu_grouped_lds.py); returns the
+ * previous setting of bit 0.  No counterpart in the reference. */
 int mq_debug_set_dense_lds(int on);
 
 /* ---- device memory helpers (so a C host needs no HIP headers) -------------------- */
