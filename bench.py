@@ -71,6 +71,9 @@ def main() -> int:
                     help="only run the 14336x4096 prefill GEMM at M = 2048 ten times (for counter passes) and exit")
     ap.add_argument("--decode-step-only", type=int, default=0, metavar="N",
                     help="only replay the 40-layer decoder step at N tokens ten times, one launch per graph node (for kernel traces), and exit")
+    ap.add_argument("--moe-layer-only", type=int, default=0, metavar="N",
+                    help="only run the cfg3 MoE layer (256 + 1 experts, 2048 x 512, top-8) at N tokens forty times over a ring "
+                         "of 4 layers (for kernel traces), and exit")
     ap.add_argument("--ring", type=int, default=RING, help="distinct weight sets visited round-robin (1 = cache-hot)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -121,6 +124,25 @@ def main() -> int:
             st.replay()
         torch.cuda.synchronize()
         print(json.dumps({"decode_step_only": n, "layers": cfg.n_layers, "replays": 10}))
+        return 0
+
+    if args.moe_layer_only:
+        n = args.moe_layer_only
+        E, H, I, K = 256, 2048, 512, 8
+        layers = []
+        for r in range(4):
+            ws = [ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, t), rows, cols, e)
+                  for t, rows, cols, e in (("gate", I, H, E), ("up", I, H, E), ("down", H, I, E), ("sg", I, H, 1), ("su", I, H, 1), ("sd", H, I, 1))]
+            gi = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3", r, "gi"), (H,)) * np.float32(0.02)).to(dev)
+            layers.append((ws[0], ws[1], ws[2], (ws[3], ws[4], ws[5], gi)))
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))).to(dev)
+        lg = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))).to(dev)
+        silu = ops.SILU_EXACT if n <= 4 else ops.SILU_FAST
+        for _ in range(10):
+            for ge, ue, de, sh in layers:
+                ops.moe_layer(ge, ue, de, x, lg, K, shared=sh, silu=silu)
+        torch.cuda.synchronize()
+        print(json.dumps({"moe_layer_only": n, "layers": 4, "passes": 10}))
         return 0
 
     # ---------------------------------------------------------------- resident data
