@@ -525,7 +525,11 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
 
 // Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk.
 constexpr int64_t kPrefillMinRows = 48;
-constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer (and norm) run inside the GEMV kernel (measured: 8 loses)
+constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
+// Widest product that also runs the residual add and the RMSNorm inside the GEMV kernel: every workgroup repeats the
+// rows' norm, about 1.25 us per row.  Decoder layer (2048 hidden, 64 experts) with the norm inside / as a launch of
+// its own that emits Q8_K for the LDS-staged product: 36.0 / 36.2 us at two rows, 43.9 / 42.4 at three, 48.6 / 45.7 at four.
+constexpr int64_t kNormFusedMaxRows = 2;
 
 static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                        hipStream_t s) {
@@ -676,7 +680,7 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
             return MQ_OK;
         }
     }
-    if (n <= kGemvFusedMaxRows && !census.on && w->type == kTypeQ4K) {
+    if (n <= kNormFusedMaxRows && !census.on && w->type == kTypeQ4K) {
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, w->cols, delta_dev, weight_dev, eps, sum_out_dev, y_dev, ldy, (int)n, true,
