@@ -165,12 +165,11 @@ struct Census {
 // Dense products of up to 16 rows go to the kernel that stages the activations in LDS where the shape fits it (the
 // same bits as matmul_kernel on the same operands); mq_debug_set_dense_lds(0) keeps them on matmul_kernel.
 int g_dense_lds = 1;
-bool g_fused_out_quant = true;  // the dense FFN's gate/up launch quantizes its own output (mq_debug_set_dense_lds bit 1 clears it)
 // Widest product whose fp32 rows the LDS-staged kernel quantizes itself (no quantizer launch).
 int64_t g_dense_xf_rows = 2;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
 
 bool dense_lds_takes(const MatmulArgs& a) {
-    return g_dense_lds && !a.grouped && !a.dbg_dot && a.n >= 1 && a.n <= 16 &&
+    return g_dense_lds && !a.grouped && !a.dbg_dot && !a.out_aq && a.n >= 1 && a.n <= 16 &&
            dense_lds_applies(a.nb, (a.rows + 15) / 16, a.n, a.swiglu != 0, a.wtype);
 }
 // fp32 rows straight into the product (n rows, ldx apart): true when the call may skip its quantizer launch
@@ -198,7 +197,6 @@ hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = n
     d.ldy = a.ldy;
     d.wtype = a.wtype;
     d.silu_mode = a.silu_mode;
-    d.out_aq = a.out_aq, d.out_ad = a.out_ad, d.out_counters = a.out_counters;
     return launch_dense_lds(d, s, start, stop);
 }
 
@@ -803,21 +801,11 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     a.ldy = inter;
     a.swiglu = 1;
     a.silu_mode = silu_mode;
-    // From three rows on the LDS-staged gate/up kernel also quantizes its output: the last of the four workgroups of a
-    // 256-row block to finish quantizes that block of every row, a row per wavefront -- one launch less.  (In
-    // matmul_kernel, whose workgroups have two wavefronts, the same scheme serialises the rows at the kernel's tail and
-    // is slower than the quantizer launch.)
-    const bool inline_quant_down = one_row || dense_lds_quantizes(down, (const float*)g.mid.ptr, n, inter, false);
-    const bool quant_in_gateup = !inline_quant_down && g_fused_out_quant && dense_lds_takes(a) && (inter & 255) == 0 && !census.on;
-    if (quant_in_gateup) {
-        if (int rc = reserve_counters(4096)) return rc;
-        if (inter / 256 > 4095) return fail(MQ_ERR_UNSUPPORTED, "mq_ffn_swiglu_q4k: inter too large");
-        MQ_HIP(g.aq2.reserve(aq_bytes(n, inter / kQK)));
-        MQ_HIP(g.ad2.reserve(ad_count(n, inter / kQK) * sizeof(float)));
-        a.out_aq = (uint8_t*)g.aq2.ptr, a.out_ad = (float*)g.ad2.ptr, a.out_counters = (uint32_t*)g.counters.ptr;
-    }
     MQ_HIP(census_launch(a, s));
-    if (!inline_quant_down && !quant_in_gateup)
+    // The SwiGLU output is re-quantized by a launch of its own: the kernel's fused re-quantization (last
+    // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
+    const bool inline_quant_down = one_row || dense_lds_quantizes(down, (const float*)g.mid.ptr, n, inter, false);
+    if (!inline_quant_down)
         if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     MatmulArgs d;
     d.w0 = down->data;
@@ -1675,7 +1663,6 @@ int mq_debug_set_dense_lds(int on) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     const int before = g_dense_lds;
     g_dense_lds = on & 1;
-    g_fused_out_quant = !(on & 2);
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;

@@ -237,40 +237,9 @@ __global__ void __launch_bounds__(512) dense_lds_kernel(const DenseLdsArgs p) {
                     if (tok < p.n) {
                         float v = acc[0][tt][j];
                         if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][tt][j], p.silu_mode);
-                        float* dst = p.y + (size_t)tok * (size_t)p.ldy + (size_t)row;
-                        if (p.out_aq) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // another workgroup re-reads it
-                        else *dst = v;
+                        p.y[(size_t)tok * (size_t)p.ldy + (size_t)row] = v;
                     }
                 }
-        }
-    }
-
-    // ---- optional: the last workgroup to finish a 256-row block of y quantizes it to Q8_K (matmul_kernel's scheme;
-    // here a row per wavefront, so eight rows are quantized side by side) ----
-    if (p.out_aq) {
-        int* is_last = reinterpret_cast<int*>(lds);  // the staged activations are no longer read (the kernel's LDS is all dynamic)
-        const int out_nb = (int)(p.rows >> 8);
-        const int hb = (int)(((int64_t)blockIdx.x * RPW) >> 4);
-        // the y stores are device-scope write-through stores: wait for their acknowledgement, then count the workgroup
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            uint32_t* c = p.out_counters + hb;
-            const uint32_t prev = atomicAdd(c, 1u);
-            const uint32_t last = (uint32_t)(16 / RPW - 1);  // a 256-row block is 16 row tiles, RPW of them per workgroup
-            *is_last = prev == last;
-            if (prev == last) atomicExch(c, 0u);  // leave the counters zero for the next launch
-        }
-        __syncthreads();
-        if (*is_last) {
-            for (int m = wave; m < (int)p.n; m += 8) {
-                const float* src = p.y + (size_t)m * (size_t)p.ldy + (size_t)hb * 256 + lane * 4;
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = __hip_atomic_load(src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const Q8Lane r = quantize_block_q8k(v, lane);
-                store_amajor(p.out_aq, p.out_ad, m, hb, out_nb, lane, r);
-            }
         }
     }
 }
@@ -350,7 +319,6 @@ bool dense_lds_applies(int64_t nb, int64_t rowtiles, int64_t n, bool swiglu, int
 
 hipError_t launch_dense_lds(const DenseLdsArgs& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 16 || !a.y || !a.w0) return hipErrorInvalidValue;
-    if (a.out_aq && ((a.rows & 255) || !a.out_ad || !a.out_counters)) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
     if (!dense_lds_applies(a.nb, rowtiles, a.n, a.w1 != nullptr, a.wtype)) return hipErrorInvalidValue;
     if (a.xf ? ((reinterpret_cast<uintptr_t>(a.xf) & 15u) || (a.ldx & 3) || a.n > 4 || a.n * a.nb > 64) : (!a.aq || !a.ad)) return hipErrorInvalidValue;

@@ -113,11 +113,6 @@ struct DenseLdsArgs {
     int64_t ldy = 0;
     int wtype = 12;
     int silu_mode = 0;
-    // optional fused Q8_K of the output (rows % 256 == 0): the last workgroup to finish a 256-row block of y quantizes
-    // that block of every activation row into the A-major layout, one row per wavefront
-    uint8_t* out_aq = nullptr;
-    float* out_ad = nullptr;
-    uint32_t* out_counters = nullptr;  // [rows / 256], zero before the launch, zero again after it
 };
 // true when the shape fits the kernel (LDS capacity, wavefront split)
 bool dense_lds_applies(int64_t nb, int64_t rowtiles, int64_t n, bool swiglu, int wtype);

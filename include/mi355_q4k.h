@@ -355,9 +355,8 @@ int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int
  * in LDS once per workgroup (and, for up to four fp32 rows, quantizes them itself), and expert-grouped launches
  * with many groups on the kernel that gathers a group's rows into LDS once per eight wavefronts; on = 0 keeps
  * both on the kernel that reads its operand from global memory at every stage, on = 5 only the expert-grouped
- * ones; on = 3 keeps the quantizer launch between the two products of mq_ffn_swiglu_q4k (normally the gate/up
- * launch quantizes its own output from three rows on).  All return the same bits (tests/test_gpu_dense_lds.py,
- * tests/test_gpu_grouped_lds.py); returns the previous setting of bit 0.  No counterpart in the reference. */
+ * ones.  All return the same bits (tests/test_gpu_dense_lds.py, tests/test_gpu_grouped_lds.py); returns the
+ * previous setting of bit 0.  No counterpart in the reference. */
 int mq_debug_set_dense_lds(int on);
 
 /* ---- device memory helpers (so a C host needs no HIP headers) -------------------- */
