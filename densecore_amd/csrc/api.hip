@@ -232,7 +232,8 @@ int order_stream(hipStream_t s) {
     }
     if (g.have_last_stream && g.last_stream != s) {
         hipError_t e = hipSuccess;
-        if (!g.order_event) e = hipEventCreateWithFlags(&g.order_event, hipEventDisableTiming);
+        // the event exists since mq_init: no entry point creates anything here (one of them must not allocate)
+        if (!g.order_event) e = hipErrorNotReady;
         if (e == hipSuccess) e = hipEventRecord(g.order_event, g.last_stream);
         if (e == hipSuccess) e = hipStreamWaitEvent(s, g.order_event, 0);
         if (e != hipSuccess) {  // e.g. the previous stream no longer exists: wait for everything instead
@@ -357,6 +358,7 @@ int mq_init(int device) {
         g_scratch_ptr[device] = static_cast<unsigned char*>(ptr);
     }
     set_compute_units(prop.multiProcessorCount);
+    if (!g.order_event) MQ_HIP(hipEventCreateWithFlags(&g.order_event, hipEventDisableTiming));  // orders calls on different streams
     g.device = device;
     g.ready = true;
     return MQ_OK;
