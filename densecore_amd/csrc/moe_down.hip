@@ -11,6 +11,10 @@
 // kFromF32: the hidden rows come as fp32 and every wavefront quantizes the super-blocks it multiplies (the block
 // quantizer of quantize_q8k_kernel: same codes and scale), which takes the re-quantization off the tail of the
 // gate/up launch; the work is repeated by every workgroup of a token, a few hundred instructions each.
+// Order of the requests: the token's experts (one vector load), the hidden rows and the gate operands go out first,
+// the tile requests follow as soon as the experts are known, and the quantization, the gate and the routing weights
+// are worked on while the tiles travel; requests are answered in order, so nothing that is needed early may be
+// asked for after a tile.
 #include "common.h"
 #include "kernels.h"
 #include "decode_tile.h"
@@ -27,35 +31,35 @@ constexpr int kItems = 3;  // (slot, super-block) items a wavefront keeps in fli
 template <int WT, bool kFromF32>
 __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDownTokenArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
-    extern __shared__ float term[];  // [slots * nb][16]
+    constexpr int J = kFromF32 ? 1 : 2;  // a row quantized here is row 0 of the operand: the second row is never formed
+    extern __shared__ float term[];  // [slots * nb][16] terms, then [slots][16] weighted slot sums
     __shared__ float wave_sum[4];
     __shared__ float gate_sh;
-    __shared__ int ids_sh[8];        // the token's experts and routing weights, fetched once
+    __shared__ int ids_sh[8];        // the token's experts and routing weights
     __shared__ float wts_sh[8];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x, t = blockIdx.y;
     const int nb = (int)p.nb, slots = p.top_k + (p.sh_w ? 1 : 0), n_items = slots * nb;
+    float* prod = term + n_items * 16;
 
-    auto item_tile = [&](int i) -> const uint8_t* {  // null for a dropped slot
-        const int sl = i / nb, b = i - sl * nb;
-        const bool shared = sl >= p.top_k;
-        const int e = shared ? 0 : p.ids[t * p.top_k + sl];
-        if (!shared && (e < 0 || e >= p.n_experts)) return nullptr;
-        return (shared ? p.sh_w : p.w + (size_t)e * p.expert_bytes) + tile_offset(rt, b, nb, kTileStride);
-    };
+    // The token's experts and weights in lanes 0 .. top_k-1 of every wavefront: ONE request, made before anything
+    // else, because the tile addresses wait for it (a scalar read per item would be a round trip per item).
+    const int k_lane = lane < p.top_k ? lane : 0;
+    const int id_lane = p.ids[t * p.top_k + k_lane];
+    const float w_lane = p.weights[t * p.top_k + k_lane];
 
     for (int base = 0; base < n_items; base += kWaves * kItems) {
         typename TileOf<WT>::Regs tiles[kItems];
         ARegs<1> a[kItems];
         float4 hv[kItems];
+        bool live[kItems];
+        // the hidden rows first: they do not depend on the routing, and requests are answered in order
 #pragma unroll
-        for (int j = 0; j < kItems; ++j) {  // every load is issued; a missing item reads a harmless tile
+        for (int j = 0; j < kItems; ++j) {
             const int i = base + wave + kWaves * j;
             const int ii = i < n_items ? i : 0;
-            const uint8_t* w = i < n_items ? item_tile(i) : nullptr;
-            load_tile_wt<WT>(tiles[j], w ? w : p.w, lane);
             const int sl = ii / nb, b = ii - sl * nb;
             const int64_t row = t * slots + sl;  // hidden row
             if (kFromF32) {
@@ -67,31 +71,56 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
                 load_a<1>(a[j], p.aq + (size_t)b * 4096, p.ad + (size_t)b * 8, a_off, d_idx);
             }
         }
-        if (base == 0 && tid < p.top_k) {  // the token's experts and routing weights for the combine, fetched once
-            ids_sh[tid] = p.ids[t * p.top_k + tid];
-            wts_sh[tid] = p.weights[t * p.top_k + tid];
+        // the shared expert's gate, also ahead of the tile requests (moe_combine_kernel's order: thread j takes
+        // columns j, j + 256, ... in turn; the operands are requested eight columns at a time)
+        float gate_part = 0.0f;
+        const bool with_gate = base == 0 && p.sh_w && p.sh_gate_inp;
+        if (with_gate && tid < 256) {
+            const float* gi = p.sh_gate_inp;
+            const float* xr = p.x + t * p.rows;
+            int64_t c = tid;
+            for (; c + 7 * 256 < p.rows; c += 8 * 256) {
+                float ga[8], xa[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) ga[u] = gi[c + u * 256], xa[u] = xr[c + u * 256];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) gate_part = fmaf(ga[u], xa[u], gate_part);
+            }
+            for (; c < p.rows; c += 256) gate_part = fmaf(gi[c], xr[c], gate_part);
         }
-        if (base == 0 && p.sh_w) {  // the shared expert's gate while the tiles travel (moe_combine_kernel's order:
-            float gate = 1.0f;      // thread j takes columns j, j + 256, ... in turn)
+        // the weight tiles: every load is issued; a missing or dropped item reads a harmless tile.  The experts
+        // of all items are read out of the lanes first (branch-free), so that no tile request waits for a tile.
+        const uint8_t* tile_ptr[kItems];
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) {
+            const int i = base + wave + kWaves * j;
+            const int ii = i < n_items ? i : 0;
+            const int sl = ii / nb, b = ii - sl * nb;
+            const bool shared = sl >= p.top_k;
+            const int e = __builtin_amdgcn_readlane(id_lane, sl & 7);
+            live[j] = i < n_items && (shared || (e >= 0 && e < p.n_experts));
+            const uint8_t* m = shared ? p.sh_w : p.w + (size_t)(live[j] ? e : 0) * p.expert_bytes;
+            tile_ptr[j] = m + (live[j] ? tile_offset(rt, b, nb, kTileStride) : 0);
+        }
+#pragma unroll
+        for (int j = 0; j < kItems; ++j) load_tile_wt<WT>(tiles[j], tile_ptr[j], lane);
+        // while the tiles travel: the routing for the combine, the gate, the quantization of the hidden rows
+        if (base == 0 && tid < p.top_k) ids_sh[tid] = id_lane, wts_sh[tid] = w_lane;
+        if (with_gate && tid < 256) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) gate_part += __shfl_xor(gate_part, off, 64);
+            if ((tid & 63) == 0) wave_sum[tid >> 6] = gate_part;
+        }
+        if (kFromF32) {
+#pragma unroll
+            for (int j = 0; j < kItems; ++j) {  // the row becomes row 0 of the operand
+                const float e[4] = {hv[j].x, hv[j].y, hv[j].z, hv[j].w};
+                a_from_lane_codes(a[j], quantize_block_q8k(e, lane), lane);
+            }
+        }
+        if (base == 0 && p.sh_w) {
+            float gate = 1.0f;
             if (p.sh_gate_inp) {
-                if (tid < 256) {
-                    // the operands are requested eight columns at a time so that their latencies overlap
-                    const float* gi = p.sh_gate_inp;
-                    const float* xr = p.x + t * p.rows;
-                    float acc = 0.0f;
-                    int64_t c = tid;
-                    for (; c + 7 * 256 < p.rows; c += 8 * 256) {
-                        float ga[8], xa[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) ga[u] = gi[c + u * 256], xa[u] = xr[c + u * 256];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) acc = fmaf(ga[u], xa[u], acc);
-                    }
-                    for (; c < p.rows; c += 256) acc = fmaf(gi[c], xr[c], acc);
-#pragma unroll
-                    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-                    if ((tid & 63) == 0) wave_sum[tid >> 6] = acc;
-                }
                 __syncthreads();
                 gate = stable_sigmoid((wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]));
             }
@@ -102,13 +131,9 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
             const int i = base + wave + kWaves * j;
             if (i < n_items) {  // wave-uniform
                 float acc[1][2] = {{0.0f, 0.0f}};
-                if (item_tile(i)) {
-                    if (kFromF32) {  // the row becomes row 0 of the operand
-                        const float e[4] = {hv[j].x, hv[j].y, hv[j].z, hv[j].w};
-                        a_from_lane_codes(a[j], quantize_block_q8k(e, lane), lane);
-                    }
+                if (live[j]) {
                     int32_t dsum[1][2], msum[1][2];
-                    compute_tile_wt<1, WT>(tiles[j], a[j], acc, dsum, msum, lane);
+                    compute_tile_wt<1, WT, J>(tiles[j], a[j], acc, dsum, msum, lane);
                 }
                 const int pos = kFromF32 ? 0 : (int)((t * slots + i / nb) & 7);  // the row's place in its 8-row tile
                 if (kq == (pos >> 1)) term[i * 16 + slot] = (pos & 1) ? acc[0][1] : acc[0][0];
@@ -116,21 +141,32 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
         }
     }
     __syncthreads();
+    // The combine in the order of the two-launch form: a slot's super-block terms added in turn and the sum times
+    // its weight -- every (slot, row) on a thread of its own -- then the slots in routing order, a row per thread.
+    // A slot that the two-launch form skips (id out of range, zero weight) and the slots past the last one enter as
+    // +0: the running sum starts at +0 and can never be -0, so adding +0 leaves its bits alone.
+    if (tid < 9 * 16) {
+        const int k = tid >> 4, r = tid & 15;
+        float v = 0.0f;
+        if (k < slots) {
+            float part = __fadd_rn(0.0f, term[(k * nb) * 16 + r]);
+            for (int b = 1; b < nb; ++b) part = __fadd_rn(part, term[(k * nb + b) * 16 + r]);
+            const int e = ids_sh[k & 7];
+            const float w = k < p.top_k ? wts_sh[k & 7] : gate_sh;
+            const bool skip = k < p.top_k && (e < 0 || e >= p.n_experts || w == 0.0f);
+            v = skip ? 0.0f : __fmul_rn(part, w);
+        }
+        prod[tid] = v;
+    }
+    __syncthreads();
     if (tid < 16) {
         const int64_t row = rt * 16 + tid;
+        float v[9];
+#pragma unroll
+        for (int k = 0; k < 9; ++k) v[k] = prod[k * 16 + tid];
         float acc = 0.0f;
-        for (int k = 0; k < slots; ++k) {
-            float part = __fadd_rn(0.0f, term[(k * nb) * 16 + tid]);
-            for (int b = 1; b < nb; ++b) part = __fadd_rn(part, term[(k * nb + b) * 16 + tid]);
-            if (k < p.top_k) {
-                const int e = ids_sh[k];
-                const float w = wts_sh[k];
-                if (e < 0 || e >= p.n_experts || w == 0.0f) continue;
-                acc = __fadd_rn(acc, __fmul_rn(part, w));
-            } else {
-                acc = __fadd_rn(acc, __fmul_rn(part, gate_sh));
-            }
-        }
+#pragma unroll
+        for (int k = 0; k < 9; ++k) acc = __fadd_rn(acc, v[k]);
         if (row < p.rows) p.y[t * p.rows + row] = acc;
     }
 }
@@ -140,7 +176,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
 hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) {
     if (a.n <= 0 || a.rows <= 0 || (a.rows & 15) || a.nb <= 0 || a.top_k <= 0 || a.top_k > 8) return hipErrorInvalidValue;
     const int slots = a.top_k + (a.sh_w ? 1 : 0);
-    const size_t lds = (size_t)slots * (size_t)a.nb * 16 * sizeof(float);
+    const size_t lds = ((size_t)slots * (size_t)a.nb + 9) * 16 * sizeof(float);
     if (lds > 48 * 1024) return hipErrorInvalidValue;
     const dim3 grid((unsigned)(a.rows / 16), (unsigned)a.n);
     if ((a.hidden == nullptr) == (a.aq == nullptr)) return hipErrorInvalidValue;  // one source of hidden rows

@@ -32,6 +32,7 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
     constexpr int kTileStride = tile_stride<WT>();
     extern __shared__ float red[];  // [W-1][2][64]
     __shared__ int ids_sh[8];
+    __shared__ unsigned long long route_sh[kRouteScratch];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
@@ -62,8 +63,8 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
             auto load = [&](int e) { return row[e]; };
             int id;
             float logit;
-            if (p.n_experts <= 256) route_token_wave<4>(load, p.n_experts, p.top_k, lane, id, logit);
-            else route_token_wave<8>(load, p.n_experts, p.top_k, lane, id, logit);
+            if (p.n_experts <= 256) route_token_wave_lds<4>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
+            else route_token_wave_lds<8>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
             if (lane < p.top_k) ids_sh[lane] = id;
             if (rt == 0 && sl == 0) {  // one workgroup per token hands ids and weights to the down projection
                 const float w = route_weight_lane(logit, lane, p.top_k, p.route_mode);
@@ -87,21 +88,32 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
 #pragma unroll
     for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
 
+    // while the first tiles travel their super-blocks of x are quantized (the token is row 0 of the operand)
+    ACodes a_first[kStages - 1];
+#pragma unroll
+    for (int st = 0; st < kStages - 1; ++st) {
+        const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
+        a_codes_from_lane_codes(a_first[st], quantize_block_q8k(e, lane), lane);
+    }
     float acc[2][1][2] = {{{0.0f, 0.0f}}, {{0.0f, 0.0f}}};
     for (int base = 0; base < cnt; base += kStages) {
 #pragma unroll
         for (int st = 0; st < kStages; ++st) {
             const int i = base + st;
-            issue_t((st + kStages - 1) % kStages, i + kStages - 1);
             issue_x((st + kStages - 1) % kStages, i + kStages - 1);
+            issue_t((st + kStages - 1) % kStages, i + kStages - 1);
             if (i < cnt) {
-                const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
                 ARegs<1> a;
-                a_from_lane_codes(a, quantize_block_q8k(e, lane), lane);  // the token is row 0 of the operand
+                if (st < kStages - 1 && base == 0) {
+                    a_from_codes(a, a_first[st < kStages - 1 ? st : 0], lane);
+                } else {
+                    const float e[4] = {ring_x[st].x, ring_x[st].y, ring_x[st].z, ring_x[st].w};
+                    a_from_lane_codes(a, quantize_block_q8k(e, lane), lane);
+                }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
+                for (int m = 0; m < 2; ++m) {  // only row 0 of the operand is formed (J = 1)
                     int32_t dsum[1][2], msum[1][2];
-                    compute_tile_wt<1, WT>(ring_t[st][m], a, acc[m], dsum, msum, lane);
+                    compute_tile_wt<1, WT, 1>(ring_t[st][m], a, acc[m], dsum, msum, lane);
                 }
             }
         }

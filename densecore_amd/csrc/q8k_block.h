@@ -80,17 +80,37 @@ __device__ __forceinline__ void store_amajor(uint8_t* aq, float* ad, int64_t m, 
 
 // The A operand of one activation row quantized by this wavefront (row 0 of the tile; the other rows are dead):
 // codes move from the quantizer's lanes into the split-slot operand with eight cross-lane reads per super-block.
-__device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
+// ACodes is the operand before the zeros of the dead rows are filled in: nine registers instead of eighteen for
+// a kernel that quantizes ahead of the tiles it multiplies.
+struct ACodes {
+    uint32_t lo[4], hi[4];
+    float d;
+};
+
+__device__ __forceinline__ void a_codes_from_lane_codes(ACodes& a, const Q8Lane& q, int lane) {
     const int slot = lane & 15, kq = lane >> 4;
     const int src = 8 * (slot & 1) + 2 * kq;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const uint32_t lo = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
-        const uint32_t hi = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
-        a.q[0][c] = slot == 0 ? v4u{lo, hi, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, lo, hi} : v4u{0u, 0u, 0u, 0u});
+        a.lo[c] = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
+        a.hi[c] = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
     }
-    a.yd[0][0] = q.d;
+    a.d = q.d;
+}
+
+__device__ __forceinline__ void a_from_codes(ARegs<1>& a, const ACodes& s, int lane) {
+    const int slot = lane & 15;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        a.q[0][c] = slot == 0 ? v4u{s.lo[c], s.hi[c], 0u, 0u} : (slot == 1 ? v4u{0u, 0u, s.lo[c], s.hi[c]} : v4u{0u, 0u, 0u, 0u});
+    a.yd[0][0] = s.d;
     a.yd[0][1] = 0.0f;
+}
+
+__device__ __forceinline__ void a_from_lane_codes(ARegs<1>& a, const Q8Lane& q, int lane) {
+    ACodes s;
+    a_codes_from_lane_codes(s, q, lane);
+    a_from_codes(a, s, lane);
 }
 
 #endif

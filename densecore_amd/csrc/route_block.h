@@ -141,11 +141,14 @@ template <int KPL, typename Load>
 __device__ __forceinline__ void route_token_wave(Load load, int n_experts, int top_k, int lane, int& id_out,
                                                  float& logit_out) {
     uint32_t key[KPL];
+    float logit[KPL];
 #pragma unroll
-    for (int i = 0; i < KPL; ++i) {
-        const int e = lane + 64 * i;
-        key[i] = e < n_experts ? route_key32(load(e)) : 0u;
+    for (int i = 0; i < KPL; ++i) {  // every lane reads KPL logits (a lane past the end re-reads the last one):
+        const int e = lane + 64 * i;  // unconditional loads are requested together, not one round trip each
+        logit[i] = load(e < n_experts ? e : n_experts - 1);
     }
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) key[i] = lane + 64 * i < n_experts ? route_key32(logit[i]) : 0u;
     float my_logit = 0.0f;
     int my_id = -1;
     for (int r = 0; r < top_k; ++r) {
@@ -169,6 +172,80 @@ __device__ __forceinline__ void route_token_wave(Load load, int n_experts, int t
     }
     id_out = my_id;
     logit_out = my_logit;
+}
+
+// The same routing in one pass for the common case, for a wavefront that has LDS of its own (kRouteScratch 64-bit
+// words, used by no other wavefront).  The smallest of the eight 8-lane group maxima is a key that at least eight
+// keys reach, so the top_k <= 8 first experts of the routing order are among the keys >= it (typically one or two
+// dozen of 256).  Those are packed into LDS as (key << 32 | ~id) -- larger = earlier in the routing order, never
+// equal -- and every candidate counts the candidates ahead of it: its place in the routing order.  More than 64
+// candidates (rows of equal logits) go the round-by-round way; ids and logits are the same either way.
+constexpr int kRouteScratch = 72;
+template <int KPL, typename Load>
+__device__ __forceinline__ void route_token_wave_lds(Load load, int n_experts, int top_k, int lane, int& id_out,
+                                                     float& logit_out, unsigned long long* scratch) {
+    uint32_t key[KPL];
+    float logit[KPL];
+    uint32_t best = 0u;
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) {  // unconditional loads (a lane past the end re-reads the last logit): one round trip
+        const int e = lane + 64 * i;
+        logit[i] = load(e < n_experts ? e : n_experts - 1);
+    }
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) {
+        key[i] = lane + 64 * i < n_experts ? route_key32(logit[i]) : 0u;
+        best = key[i] > best ? key[i] : best;
+    }
+    uint32_t t;
+    t = dpp_u32<kDppXor1>(best), best = t > best ? t : best;
+    t = dpp_u32<kDppXor2>(best), best = t > best ? t : best;
+    t = dpp_u32<kDppHalfMirror>(best), best = t > best ? t : best;  // the maximum of the lane's group of eight
+    t = dpp_u32<kDppMirror>(best), best = t < best ? t : best;      // the smaller of two groups
+    const uint32_t p0 = __builtin_amdgcn_readlane(best, 0), p1 = __builtin_amdgcn_readlane(best, 16);
+    const uint32_t p2 = __builtin_amdgcn_readlane(best, 32), p3 = __builtin_amdgcn_readlane(best, 48);
+    const uint32_t p01 = p0 < p1 ? p0 : p1, p23 = p2 < p3 ? p2 : p3;
+    const uint32_t pivot = p01 < p23 ? p01 : p23;
+    int total = 0;
+    unsigned long long mask[KPL];
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) {
+        mask[i] = __ballot(key[i] >= pivot && key[i] != 0u);
+        total += __popcll(mask[i]);
+    }
+    if (total > 64) {
+        route_token_wave<KPL>(load, n_experts, top_k, lane, id_out, logit_out);
+        return;
+    }
+    scratch[lane] = 0ull;  // an empty place is ahead of nobody
+    int base = 0;
+#pragma unroll
+    for (int i = 0; i < KPL; ++i) {
+        const int below = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask[i] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask[i], 0u));
+        if ((mask[i] >> lane) & 1ull)
+            scratch[base + below] = ((unsigned long long)key[i] << 32) | (unsigned long long)(uint32_t)(~(uint32_t)(lane + 64 * i));
+        base += __popcll(mask[i]);
+    }
+    // one wavefront: its LDS accesses are carried out in program order, the fence keeps the compiler to that order
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    const unsigned long long mine = scratch[lane < total ? lane : 0];
+    int rank = 0;
+    for (int c = 0; c < total; c += 8) {  // eight candidates per round trip to LDS (all lanes read the same words)
+        unsigned long long other[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) other[u] = scratch[c + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) rank += other[u] > mine ? 1 : 0;
+    }
+    if (lane < total && rank < top_k) scratch[64 + rank] = mine;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    id_out = -1;
+    logit_out = 0.0f;
+    if (lane < top_k) {
+        const unsigned long long sel = scratch[64 + lane];
+        id_out = (int)(~(uint32_t)sel);
+        logit_out = route_key32_logit((uint32_t)(sel >> 32));
+    }
 }
 
 // The logit behind a route_key (NaN comes back as a canonical NaN, -0 as +0: neither changes a weight).
