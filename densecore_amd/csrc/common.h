@@ -185,6 +185,15 @@ __device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {
 constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
 
 // Maximum of an unsigned value over the 64 lanes, returned in every lane (wave-uniform).
+// unit = row * nb + block, split again.  The launchers keep the unit count below 2^31, so the division is a
+// 32-bit one: a 64-bit division is some 150 dependent scalar instructions at the head of a kernel that otherwise
+// runs for a few microseconds.
+__device__ __forceinline__ void split_unit(int64_t unit, int64_t nb, int64_t& row, int64_t& block) {
+    const uint32_t q = (uint32_t)unit / (uint32_t)nb;
+    row = (int64_t)q;
+    block = (int64_t)((uint32_t)unit - q * (uint32_t)nb);
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
     uint32_t t;
     t = dpp_u32<kDppXor1>(x);

@@ -190,19 +190,28 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
 #pragma unroll
         for (int u = 0; u < 8; ++u) first[u] = *reinterpret_cast<const float4*>(wr + lane * 4 + u * 256);
     }
-    float4 kept[kKeep];
-    float ssq = 0.0f;
+    // The operands of the norm are requested together and unconditionally (a block past the end re-reads block 0,
+    // a missing residual or weight re-reads x): conditional loads would go out one round trip after the other.
+    const float* dp = delta ? delta : x;
+    const float* wp = weight ? weight : x;
+    float4 kept[kKeep], dl[kKeep], wn[kKeep];
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) {
         const int64_t b = wave + 4 * i;
-        if (b < nb) {
-            const int64_t c0 = b * kQK + lane * 4;
-            float4 a = *reinterpret_cast<const float4*>(x + base + c0);
+        const int64_t c0 = (b < nb ? b : 0) * kQK + lane * 4;
+        kept[i] = *reinterpret_cast<const float4*>(x + base + c0);
+        dl[i] = *reinterpret_cast<const float4*>(dp + base + c0);
+        wn[i] = *reinterpret_cast<const float4*>(wp + c0);
+    }
+    float ssq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+        if (wave + 4 * i < nb) {
+            float4 a = kept[i];
             if (delta) {
-                const float4 d = *reinterpret_cast<const float4*>(delta + base + c0);
+                const float4 d = dl[i];
                 a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
             }
-            if (writer && sum_out) *reinterpret_cast<float4*>(sum_out + base + c0) = a;
             ssq = __fmaf_rn(a.x, a.x, ssq);
             ssq = __fmaf_rn(a.y, a.y, ssq);
             ssq = __fmaf_rn(a.z, a.z, ssq);
@@ -218,20 +227,16 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
     const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) {
-        const int64_t b = wave + 4 * i;
-        if (b < nb) {
-            const int64_t c0 = b * kQK + lane * 4;
-            const float4 a = kept[i];
-            float4 w = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
-            if (weight) w = *reinterpret_cast<const float4*>(weight + c0);
+        if (wave + 4 * i < nb) {
+            const int64_t c0 = (int64_t)(wave + 4 * i) * kQK + lane * 4;
+            const float4 a = kept[i], w = wn[i];
             const float4 e = make_float4(__fmul_rn(a.x, weight ? __fmul_rn(scale, w.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, w.y) : scale),
                                          __fmul_rn(a.z, weight ? __fmul_rn(scale, w.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, w.w) : scale));
             *reinterpret_cast<float4*>(row_sh + c0) = e;
-            if (writer && normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = e;
         }
     }
     __syncthreads();
-    if (ex >= n_experts) return;
+    // a wavefront without an expert of its own forms expert 0's logit again and drops it (it may still have stores to make)
     float acc = 0.0f;
     auto add4 = [&](const float4& a, const float4& b) {
         acc = __fmaf_rn(a.x, b.x, acc);
@@ -255,7 +260,17 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
     for (; c + 3 < cols; c += 256) add4(*reinterpret_cast<const float4*>(wr + c), *reinterpret_cast<const float4*>(row_sh + c));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (lane == 0) logits[t * n_experts + ex] = acc;
+    if (lane == 0 && ex < n_experts) logits[t * n_experts + ex] = acc;
+    if (writer) {  // last: a store ahead of a barrier would make the barrier wait for it
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            if (wave + 4 * i < nb) {
+                const int64_t c0 = (int64_t)(wave + 4 * i) * kQK + lane * 4;
+                if (sum_out) *reinterpret_cast<float4*>(sum_out + base + c0) = kept[i];
+                if (normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = *reinterpret_cast<const float4*>(row_sh + c0);
+            }
+        }
+    }
 }
 
 }  // namespace

@@ -28,36 +28,32 @@ __global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restr
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const uint8_t* tiles = w + tile_offset(rt, 0, nb);
-    const int cnt = wave < nb ? (int)((nb - wave + n_waves - 1) / n_waves) : 0;  // <= kMaxStages (host-checked)
+    const int cnt = (wave < nb ? 1 : 0) + (wave + n_waves < nb ? 1 : 0);  // super-blocks wave, wave + W (at most kMaxStages, host-checked; no division)
 
+    // The activations are requested before the tiles (requests are answered in order) and quantized while the
+    // tiles travel; only row 0 of the operand is formed (J = 1).
     TileRegs t[kMaxStages];
     float4 xv[kMaxStages];
 #pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) xv[i] = *reinterpret_cast<const float4*>(x + (size_t)(i < cnt ? wave + i * n_waves : 0) * kQK + lane * 4);
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) load_tile(t[i], tiles + (size_t)(i < cnt ? wave + i * n_waves : 0) * kTileBytes, lane);
+    // code 4L + j sits in byte j of lane L.  Slot s (0: even sub-block, 1: odd) of k-group kq needs the eight codes
+    // 64c + 32s + 8kq + (0..7) of chunk c: lanes 16c + 8s + 2kq and the next one (a_codes_from_lane_codes).
+    ACodes codes[kMaxStages];
+#pragma unroll
     for (int i = 0; i < kMaxStages; ++i) {
-        const int b = i < cnt ? wave + i * n_waves : 0;
-        load_tile(t[i], tiles + (size_t)b * kTileBytes, lane);
-        xv[i] = *reinterpret_cast<const float4*>(x + (size_t)b * kQK + lane * 4);
+        const float e[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+        a_codes_from_lane_codes(codes[i], quantize_block_q8k(e, lane), lane);
     }
     float acc[1][2] = {{0.0f, 0.0f}};
 #pragma unroll
     for (int i = 0; i < kMaxStages; ++i) {
         if (i < cnt) {
-            const float e[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
-            const Q8Lane q = quantize_block_q8k(e, lane);
-            // code 4L + j sits in byte j of lane L.  Slot s (0: even sub-block, 1: odd) of k-group kq needs the
-            // eight codes 64c + 32s + 8kq + (0..7) of chunk c: lanes 16c + 8s + 2kq and the next one.
-            ARegs<1> a;
-            const int src = 8 * (slot & 1) + 2 * kq;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t lo = (uint32_t)__shfl((int)q.packed, 16 * c + src, 64);
-                const uint32_t hi = (uint32_t)__shfl((int)q.packed, 16 * c + src + 1, 64);
-                a.q[0][c] = slot == 0 ? v4u{lo, hi, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, lo, hi} : v4u{0u, 0u, 0u, 0u});
-            }
-            a.yd[0][0] = q.d;   // row 0 (meaningful in k-group 0 only, the others are never stored)
-            a.yd[0][1] = 0.0f;
+            ARegs<1> a;  // row 0 (meaningful in k-group 0 only, the others are never stored)
+            a_from_codes(a, codes[i], lane);
             int32_t dsum[1][2], msum[1][2];
-            compute_tile<1>(t[i], a, acc, dsum, msum);
+            compute_tile<1, false, 1>(t[i], a, acc, dsum, msum);
         }
     }
     // cross-wave reduction in wave order, epilogue on wave 0 (as matmul_kernel)
@@ -92,57 +88,94 @@ __global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const uint8_t* tiles = w + tile_offset(rt, 0, nb);
-    const int cnt = wave < nb ? (int)((nb - wave + n_waves - 1) / n_waves) : 0;  // <= kMaxStages (host-checked)
-    auto fetch = [&](int64_t c0) {
-        float4 a = *reinterpret_cast<const float4*>(x + c0);
-        if (delta) {
-            const float4 d = *reinterpret_cast<const float4*>(delta + c0);
-            a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
-        }
+    const int cnt = (wave < nb ? 1 : 0) + (wave + n_waves < nb ? 1 : 0);  // super-blocks wave, wave + W (at most kMaxStages, host-checked; no division)
+    // Every request is unconditional (without a residual or without norm weights x is simply read again) and made
+    // before the tile requests: requests are answered in order, and the norm must not wait for the tiles.
+    const float* dp = delta ? delta : x;
+    const float* wp = weight ? weight : x;
+    auto add = [&](float4 a, const float4& d) {
+        if (delta) a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
         return a;
     };
-
+    // sum of squares in the order of the 256-thread norm kernel: virtual wavefront v = 0..3 takes the super-blocks
+    // v, v + 4, ... (at most four of them here); with four or more wavefronts wavefront v is virtual wavefront v
+    const bool four = n_waves >= 4;
+    const int v4 = wave & 3;
+    float4 sx[4], sd[4];
+    if (four) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t c0 = (int64_t)(v4 + 4 * k < nb ? v4 + 4 * k : 0) * kQK + lane * 4;
+            sx[k] = *reinterpret_cast<const float4*>(x + c0);
+            sd[k] = *reinterpret_cast<const float4*>(dp + c0);
+        }
+    }
     TileRegs t[kMaxStages];
-    float4 xv[kMaxStages];
+    float4 xv[kMaxStages], dv[kMaxStages], wn[kMaxStages];
 #pragma unroll
     for (int i = 0; i < kMaxStages; ++i) {
-        const int b = i < cnt ? wave + i * n_waves : 0;
-        load_tile(t[i], tiles + (size_t)b * kTileBytes, lane);
-        xv[i] = fetch((int64_t)b * kQK + lane * 4);
+        const int64_t c0 = (int64_t)(i < cnt ? wave + i * n_waves : 0) * kQK + lane * 4;
+        xv[i] = *reinterpret_cast<const float4*>(x + c0);
+        dv[i] = *reinterpret_cast<const float4*>(dp + c0);
+        wn[i] = *reinterpret_cast<const float4*>(wp + c0);
     }
-    // sum of squares in the order of the 256-thread norm kernel: virtual wavefront v = 0..3
-    for (int v = wave; v < 4; v += n_waves) {
-        float ssq = 0.0f;
-        for (int64_t b = v; b < nb; b += 4) {
-            const float4 a = fetch(b * kQK + lane * 4);
-            ssq = __fmaf_rn(a.x, a.x, ssq);
-            ssq = __fmaf_rn(a.y, a.y, ssq);
-            ssq = __fmaf_rn(a.z, a.z, ssq);
-            ssq = __fmaf_rn(a.w, a.w, ssq);
-        }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
-        if (lane == 0) wave_sum[v] = ssq;
+    for (int i = 0; i < kMaxStages; ++i) load_tile(t[i], tiles + (size_t)(i < cnt ? wave + i * n_waves : 0) * kTileBytes, lane);
+    if (four) {
+        if (wave < 4) {
+            float ssq = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (v4 + 4 * k < nb) {
+                    const float4 a = add(sx[k], sd[k]);
+                    ssq = __fmaf_rn(a.x, a.x, ssq);
+                    ssq = __fmaf_rn(a.y, a.y, ssq);
+                    ssq = __fmaf_rn(a.z, a.z, ssq);
+                    ssq = __fmaf_rn(a.w, a.w, ssq);
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+            if (lane == 0) wave_sum[wave] = ssq;
+        }
+    } else {
+        for (int v = wave; v < 4; v += n_waves) {
+            float ssq = 0.0f;
+            for (int64_t b = v; b < nb; b += 4) {
+                const int64_t c0 = b * kQK + lane * 4;
+                const float4 a = add(*reinterpret_cast<const float4*>(x + c0), *reinterpret_cast<const float4*>(dp + c0));
+                ssq = __fmaf_rn(a.x, a.x, ssq);
+                ssq = __fmaf_rn(a.y, a.y, ssq);
+                ssq = __fmaf_rn(a.z, a.z, ssq);
+                ssq = __fmaf_rn(a.w, a.w, ssq);
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+            if (lane == 0) wave_sum[v] = ssq;
+        }
     }
     __syncthreads();
     const float total = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
     const float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)(nb * kQK)), eps)));
 
+    // normalise and quantize while the tiles travel, then multiply (only row 0 of the operand is formed)
+    ACodes codes[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        xv[i] = add(xv[i], dv[i]);
+        const float4 a = xv[i], w = wn[i];
+        const float e[4] = {__fmul_rn(a.x, weight ? __fmul_rn(scale, w.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, w.y) : scale),
+                            __fmul_rn(a.z, weight ? __fmul_rn(scale, w.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, w.w) : scale)};
+        a_codes_from_lane_codes(codes[i], quantize_block_q8k(e, lane), lane);
+    }
     float acc[1][2] = {{0.0f, 0.0f}};
 #pragma unroll
     for (int i = 0; i < kMaxStages; ++i) {
         if (i < cnt) {
-            const int64_t c0 = (int64_t)(wave + i * n_waves) * kQK + lane * 4;
-            const float4 a = xv[i];
-            if (rt == 0 && sum_out) *reinterpret_cast<float4*>(sum_out + c0) = a;
-            float4 wn = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
-            if (weight) wn = *reinterpret_cast<const float4*>(weight + c0);
-            const float e[4] = {__fmul_rn(a.x, weight ? __fmul_rn(scale, wn.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, wn.y) : scale),
-                                __fmul_rn(a.z, weight ? __fmul_rn(scale, wn.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, wn.w) : scale)};
             ARegs<1> ar;
-            a_from_lane_codes(ar, quantize_block_q8k(e, lane), lane);
+            a_from_codes(ar, codes[i], lane);
             int32_t dsum[1][2], msum[1][2];
-            compute_tile<1>(t[i], ar, acc, dsum, msum);
+            compute_tile<1, false, 1>(t[i], ar, acc, dsum, msum);
         }
     }
     if (n_waves > 1) {
@@ -154,6 +187,11 @@ __global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __
         for (int wv = 1; wv < n_waves; ++wv) v = __fadd_rn(v, red[(wv - 1) * 64 + lane]);
         const int64_t row = rt * 16 + slot;
         if (kq == 0 && row < rows) y[row] = v;
+    }
+    if (rt == 0 && sum_out) {  // last: a store ahead of a barrier would make the barrier wait for it
+#pragma unroll
+        for (int i = 0; i < kMaxStages; ++i)
+            if (i < cnt) *reinterpret_cast<float4*>(sum_out + (int64_t)(wave + i * n_waves) * kQK + lane * 4) = xv[i];
     }
 }
 
@@ -176,7 +214,7 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const uint8_t* tiles = w + tile_offset(rt, 0, nb);
-    const int cnt = wave < nb ? (int)((nb - wave + n_waves - 1) / n_waves) : 0;  // <= kMaxStages (host-checked)
+    const int cnt = (wave < nb ? 1 : 0) + (wave + n_waves < nb ? 1 : 0);  // super-blocks wave, wave + W (at most kMaxStages, host-checked; no division)
     uint8_t* codes = lds_raw + (size_t)wave * (8 * 256 + 32);
     float* scales = reinterpret_cast<float*>(codes + 8 * 256);
     float* red = reinterpret_cast<float*>(lds_raw + (size_t)n_waves * (8 * 256 + 32));

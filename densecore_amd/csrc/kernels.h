@@ -213,6 +213,7 @@ struct MoeDownTokenArgs {
     int64_t rows = 0, nb = 0;          // output rows (hidden), super-blocks per row (inter / 256)
     int64_t n = 0;
     int top_k = 0, n_experts = 0;
+    uint32_t inv_nb = 0;               // ceil(2^32 / nb) for nb > 1, filled in by the launcher: i / nb == umulhi(i, inv_nb) for i, nb < 2^16
     const uint8_t* aq = nullptr;       // A-major hidden rows, or
     const float* ad = nullptr;
     const float* hidden = nullptr;     // fp32 hidden rows [n * slots][nb * 256] (quantized inside the kernel)
@@ -238,7 +239,8 @@ struct MoeGateupTokenArgs {
     int64_t n = 0;
     int top_k = 0, n_experts = 0;      // n_experts <= 512
     int route_mode = 0, silu_mode = 0, sh_silu_mode = 2;
-    int waves = 1;                     // wavefronts per workgroup: moe_gateup_token_waves()
+    int waves = 1;                     // wavefronts per workgroup: moe_gateup_token_waves(); nb % waves == 0
+    int stages = 0;                    // nb / waves, filled in by the launcher (the kernel makes no division)
     const float* x = nullptr;          // [n][nb * 256]
     const float* logits = nullptr;     // [n][n_experts]
     float* hidden = nullptr;           // [n * slots][rows]

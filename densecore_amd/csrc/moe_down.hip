@@ -43,6 +43,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
     const int64_t rt = blockIdx.x, t = blockIdx.y;
     const int nb = (int)p.nb, slots = p.top_k + (p.sh_w ? 1 : 0), n_items = slots * nb;
     float* prod = term + n_items * 16;
+    auto item_slot = [&](int i) { return nb == 1 ? i : (int)__umulhi((uint32_t)i, p.inv_nb); };  // i / nb without a division
 
     // The token's experts and weights in lanes 0 .. top_k-1 of every wavefront: ONE request, made before anything
     // else, because the tile addresses wait for it (a scalar read per item would be a round trip per item).
@@ -60,7 +61,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
         for (int j = 0; j < kItems; ++j) {
             const int i = base + wave + kWaves * j;
             const int ii = i < n_items ? i : 0;
-            const int sl = ii / nb, b = ii - sl * nb;
+            const int sl = item_slot(ii), b = ii - sl * nb;
             const int64_t row = t * slots + sl;  // hidden row
             if (kFromF32) {
                 hv[j] = *reinterpret_cast<const float4*>(p.hidden + (size_t)row * (size_t)(nb * kQK) + (size_t)b * kQK + lane * 4);
@@ -95,7 +96,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
         for (int j = 0; j < kItems; ++j) {
             const int i = base + wave + kWaves * j;
             const int ii = i < n_items ? i : 0;
-            const int sl = ii / nb, b = ii - sl * nb;
+            const int sl = item_slot(ii), b = ii - sl * nb;
             const bool shared = sl >= p.top_k;
             const int e = __builtin_amdgcn_readlane(id_lane, sl & 7);
             live[j] = i < n_items && (shared || (e >= 0 && e < p.n_experts));
@@ -135,7 +136,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
                     int32_t dsum[1][2], msum[1][2];
                     compute_tile_wt<1, WT, J>(tiles[j], a[j], acc, dsum, msum, lane);
                 }
-                const int pos = kFromF32 ? 0 : (int)((t * slots + i / nb) & 7);  // the row's place in its 8-row tile
+                const int pos = kFromF32 ? 0 : (int)((t * slots + item_slot(i)) & 7);  // the row's place in its 8-row tile
                 if (kq == (pos >> 1)) term[i * 16 + slot] = (pos & 1) ? acc[0][1] : acc[0][0];
             }
         }
@@ -180,10 +181,12 @@ hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) 
     if (lds > 48 * 1024) return hipErrorInvalidValue;
     const dim3 grid((unsigned)(a.rows / 16), (unsigned)a.n);
     if ((a.hidden == nullptr) == (a.aq == nullptr)) return hipErrorInvalidValue;  // one source of hidden rows
+    MoeDownTokenArgs b = a;
+    b.inv_nb = a.nb > 1 ? (uint32_t)(((uint64_t)1 << 32) / (uint64_t)a.nb) + 1u : 0u;  // nb < 2^16 by the LDS limit above
 #define MQ_DOWN_TOKEN(WT)                                                                                              \
     do {                                                                                                               \
-        if (a.hidden) hipLaunchKernelGGL((moe_down_token_kernel<WT, true>), grid, dim3(kWaves * 64), lds, stream, a);  \
-        else hipLaunchKernelGGL((moe_down_token_kernel<WT, false>), grid, dim3(kWaves * 64), lds, stream, a);          \
+        if (a.hidden) hipLaunchKernelGGL((moe_down_token_kernel<WT, true>), grid, dim3(kWaves * 64), lds, stream, b);  \
+        else hipLaunchKernelGGL((moe_down_token_kernel<WT, false>), grid, dim3(kWaves * 64), lds, stream, b);          \
     } while (0)
     if (a.wtype == kTypeQ6K) MQ_DOWN_TOKEN(kWtQ6);
     else if (a.wtype == kTypeQ5K) MQ_DOWN_TOKEN(kWtQ5);

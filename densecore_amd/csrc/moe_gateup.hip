@@ -39,10 +39,10 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
     const int slots = p.top_k + (p.sh_gate ? 1 : 0);
-    const int tok = blockIdx.y / slots, sl = blockIdx.y - tok * slots;
+    const int tok = blockIdx.z, sl = blockIdx.y;
     const bool shared = sl >= p.top_k;
     const int nb = (int)p.nb;
-    const int cnt = wave < nb ? (nb - wave + n_waves - 1) / n_waves : 0;  // super-blocks wave, wave + W, ... of this wavefront
+    const int cnt = p.stages;  // super-blocks wave, wave + W, ... of this wavefront: W divides nb
     const float* xrow = p.x + (size_t)tok * (size_t)nb * kQK + lane * 4;
 
     // Ring of kStages register stages; the activations are requested first, they do not wait for the routing.
@@ -180,11 +180,13 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
         !a.weights_out || (a.sh_gate == nullptr) != (a.sh_up == nullptr))
         return hipErrorInvalidValue;
     const int slots = a.top_k + (a.sh_gate ? 1 : 0);
-    const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)(a.n * slots));
+    const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)slots, (unsigned)a.n);
+    MoeGateupTokenArgs b = a;
+    b.stages = (int)(a.nb / a.waves);
     const size_t lds = a.waves > 1 ? (size_t)(a.waves - 1) * 2 * 64 * sizeof(float) : 0;
-    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ6>, grid, dim3(64 * a.waves), lds, stream, a);
-    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ5>, grid, dim3(64 * a.waves), lds, stream, a);
-    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ4>, grid, dim3(64 * a.waves), lds, stream, a);
+    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ6>, grid, dim3(64 * a.waves), lds, stream, b);
+    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ5>, grid, dim3(64 * a.waves), lds, stream, b);
+    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ4>, grid, dim3(64 * a.waves), lds, stream, b);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -248,8 +248,8 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= m_tiles * 16 * nb) return;
-    const int64_t m = unit / nb;
-    const int64_t b = unit - m * nb;
+    int64_t m, b;
+    split_unit(unit, nb, m, b);
     float e[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (m < n) {
         const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
@@ -280,6 +280,7 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
     const int64_t units = m_tiles * 16 * nb;
     if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     hipLaunchKernelGGL(quantize_q8k_pmajor_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx,
                        nb, m_tiles, ap);
     return hipGetLastError();

@@ -31,7 +31,8 @@ __global__ void __launch_bounds__(256) quantize_q80_kernel(const float* __restri
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= n * nb) return;
-    const int64_t m = unit / nb, b = unit - m * nb;
+    int64_t m, b;
+    split_unit(unit, nb, m, b);
     const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
     const float e[4] = {v.x, v.y, v.z, v.w};
     float local = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
@@ -197,6 +198,7 @@ size_t q80_scale_bytes(int64_t n, int64_t nb) { return ad_count(n, nb) * 8 * siz
 hipError_t launch_quantize_q80(const float* x, int64_t n, int64_t ldx, int64_t cols, uint8_t* aq, uint16_t* ah, hipStream_t stream) {
     const int64_t nb = cols / kQK, units = n * nb;
     if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     if ((cols % kQK) || ldx < cols || (ldx & 3) || (reinterpret_cast<uintptr_t>(x) & 15u)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(quantize_q80_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx, nb, aq, ah);
     return hipGetLastError();

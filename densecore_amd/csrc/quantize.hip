@@ -15,8 +15,8 @@ __global__ void __launch_bounds__(256) quantize_q8k_kernel(const float* __restri
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (row, block) pair
     if (unit >= n * nb) return;
-    const int64_t m = unit / nb;
-    const int64_t b = unit - m * nb;
+    int64_t m, b;
+    split_unit(unit, nb, m, b);
 
     const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
     const float e[4] = {v.x, v.y, v.z, v.w};
@@ -37,8 +37,8 @@ __global__ void __launch_bounds__(256) q8k_to_amajor_kernel(const uint8_t* __res
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= n * nb) return;
-    const int64_t m = unit / nb;
-    const int64_t b = unit - m * nb;
+    int64_t m, b;
+    split_unit(unit, nb, m, b);
     const uint8_t* blk = q8_std + (size_t)m * q8_row_bytes + (size_t)b * kQ8Block;
     Q8Lane r;
     r.packed = *reinterpret_cast<const uint32_t*>(blk + 4 + lane * 4);
@@ -54,6 +54,7 @@ hipError_t launch_quantize_q8k(const float* x, int64_t n, int64_t ldx, int64_t k
     const int64_t nb = k / kQK;
     const int64_t units = n * nb;
     if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     const unsigned grid = (unsigned)((units + 3) / 4);
     hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(256), 0, stream, x, n, ldx, nb, (uint8_t*)q8_std,
                        q8_row_bytes, aq, ad);
@@ -65,6 +66,7 @@ hipError_t launch_q8k_to_amajor(const void* q8_std, int64_t n, size_t q8_row_byt
     const int64_t nb = k / kQK;
     const int64_t units = n * nb;
     if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     const unsigned grid = (unsigned)((units + 3) / 4);
     hipLaunchKernelGGL(q8k_to_amajor_kernel, dim3(grid), dim3(256), 0, stream, (const uint8_t*)q8_std, n, q8_row_bytes,
                        nb, aq, ad);

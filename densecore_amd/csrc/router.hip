@@ -259,7 +259,8 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
         const int lane = threadIdx.x & 63;
         const int64_t unit = (int64_t)(blockIdx.x - route_blocks) * 4 + (threadIdx.x >> 6);
         if (unit >= (int64_t)n * q_nb) return;
-        const int64_t m = unit / q_nb, b = unit - m * q_nb;
+        int64_t m, b;
+        split_unit(unit, q_nb, m, b);
         const float4 v = *reinterpret_cast<const float4*>(qx + m * q_ldx + b * kQK + lane * 4);
         const float e[4] = {v.x, v.y, v.z, v.w};
         store_amajor(q_aq, q_ad, m, b, q_nb, lane, quantize_block_q8k(e, lane));
