@@ -18,7 +18,7 @@ constexpr int kMaxExperts = 2048;
 // e = l mod 64: a local maximum over its keys, a 6-step butterfly across the lanes, and the owner of
 // the winner clears it).  The keys are unique and totally ordered exactly like
 // ComputeQwenNativeMoEStableTopK (core/src/llm/moe/native.cpp:610-645), so the k-th extraction is the
-// k-th expert of the routing order.  keys: n_experts 64-bit words of LDS; sel: 8 floats + 8 ints of LDS.
+// k-th expert of the routing order.  keys: max(n_experts, kRouteScratch) 64-bit words of LDS; sel: 8 floats + 8 ints of LDS.
 __device__ __forceinline__ void route_token_block(const float* __restrict__ row, int n_experts, int top_k, int mode,
                                                   unsigned long long* keys, float* sel_logit, int32_t* sel_id,
                                                   int32_t* __restrict__ ids_out, float* __restrict__ w_out,
@@ -31,8 +31,8 @@ __device__ __forceinline__ void route_token_block(const float* __restrict__ row,
             int id;
             float logit;
             auto load = [&](int e) { return row[e]; };
-            if (n_experts <= 256) route_token_wave<4>(load, n_experts, top_k, tid, id, logit);
-            else route_token_wave<8>(load, n_experts, top_k, tid, id, logit);
+            if (n_experts <= 256) route_token_wave_lds<4>(load, n_experts, top_k, tid, id, logit, keys);
+            else route_token_wave_lds<8>(load, n_experts, top_k, tid, id, logit, keys);
             const float w = route_weight_lane(logit, tid, top_k, mode);
             if (tid < top_k) {
                 sel_id[tid] = id;
@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
                                                          int mode, int32_t* __restrict__ ids,
                                                          float* __restrict__ weights) {
     extern __shared__ unsigned long long route_sh[];  // [n_experts] keys, then 8 floats, 8 ints
-    float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
+    float* sel_logit = reinterpret_cast<float*>(route_sh + (n_experts > kRouteScratch ? n_experts : kRouteScratch));
     int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
     const int64_t tok = blockIdx.x;
     route_token_block(logits + tok * n_experts, n_experts, top_k, mode, route_sh, sel_logit, sel_id, ids + tok * top_k,
@@ -244,7 +244,7 @@ __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __res
 // uint32 in device memory that the kernel leaves zero again.  Workgroups past `route_blocks` do an
 // unrelated job that needs nothing from the router and would otherwise cost a launch of its own: they
 // quantize the layer input to Q8_K (four (row, super-block) units each, as quantize_q8k_kernel does).
-__global__ void __launch_bounds__(256) route_and_group_kernel(const float* __restrict__ logits, int n_experts, int n,
+__global__ void __launch_bounds__(1024) route_and_group_kernel(const float* __restrict__ logits, int n_experts, int n,
                                                               int top_k, int mode, int32_t* __restrict__ ids,
                                                               float* __restrict__ weights, uint32_t* arrivals,
                                                               int32_t* __restrict__ group_expert,
@@ -252,12 +252,12 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
                                                               int32_t* __restrict__ n_groups,
                                                               int32_t* __restrict__ entry_token,
                                                               int32_t* __restrict__ entry_k, int build_groups,
-                                                              int route_blocks, int mask_words,
+                                                              int route_blocks, int mask_words, int wave_parallel,
                                                               const float* __restrict__ qx, int64_t q_ldx, int64_t q_nb,
                                                               uint8_t* __restrict__ q_aq, float* __restrict__ q_ad) {
     if ((int)blockIdx.x >= route_blocks) {
         const int lane = threadIdx.x & 63;
-        const int64_t unit = (int64_t)(blockIdx.x - route_blocks) * 4 + (threadIdx.x >> 6);
+        const int64_t unit = (int64_t)(blockIdx.x - route_blocks) * (blockDim.x >> 6) + (threadIdx.x >> 6);
         if (unit >= (int64_t)n * q_nb) return;
         int64_t m, b;
         split_unit(unit, q_nb, m, b);
@@ -268,8 +268,35 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
     }
     extern __shared__ unsigned long long route_sh[];  // keys | sel | then reused: counts, ids
     __shared__ int is_last;
-    float* sel_logit = reinterpret_cast<float*>(route_sh + n_experts);
+    float* sel_logit = reinterpret_cast<float*>(route_sh + (n_experts > kRouteScratch ? n_experts : kRouteScratch));
     int32_t* sel_id = reinterpret_cast<int32_t*>(sel_logit + 8);
+    if (wave_parallel) {
+        // One workgroup for all tokens, a token per wavefront (and round): the ids go to LDS as they are found and the
+        // grouping follows behind one barrier -- no device-coherent stores, arrival count and re-read between them.
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n_waves = blockDim.x >> 6;
+        unsigned long long* scratch = route_sh + wave * kRouteScratch;
+        int32_t* count = reinterpret_cast<int32_t*>(route_sh + n_waves * kRouteScratch);
+        int32_t* ids_s = count + n_experts;
+        for (int tok = wave; tok < n; tok += n_waves) {
+            const float* row = logits + (size_t)tok * n_experts;
+            auto load = [&](int e) { return row[e]; };
+            int id;
+            float logit;
+            if (n_experts <= 256) route_token_wave_lds<4>(load, n_experts, top_k, lane, id, logit, scratch);
+            else route_token_wave_lds<8>(load, n_experts, top_k, lane, id, logit, scratch);
+            const float w = route_weight_lane(logit, lane, top_k, mode);
+            if (lane < top_k) {
+                ids[(size_t)tok * top_k + lane] = id;
+                weights[(size_t)tok * top_k + lane] = w;
+                ids_s[tok * top_k + lane] = id;
+            }
+        }
+        if (!build_groups) return;
+        // group_entries zeroes its counters and passes a barrier before it reads the ids
+        group_entries(ids_s, n * top_k, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
+                      mask_words ? reinterpret_cast<uint32_t*>(ids_s + n * top_k) : nullptr, mask_words);
+        return;
+    }
     const bool solo = route_blocks == 1;  // one or two tokens: one workgroup does everything, no handshake
     const int per_block = solo ? n : 1;
     for (int t = 0; t < per_block; ++t) {
@@ -294,7 +321,7 @@ __global__ void __launch_bounds__(256) route_and_group_kernel(const float* __res
     int32_t* count = reinterpret_cast<int32_t*>(route_sh);
     int32_t* ids_s = count + n_experts;
     const int n_entries = n * top_k;
-    for (int i = threadIdx.x; i < n_entries; i += 256)
+    for (int i = threadIdx.x; i < n_entries; i += blockDim.x)
         ids_s[i] = solo ? ids[i] : __hip_atomic_load(ids + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     group_entries(ids_s, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
                   mask_words ? reinterpret_cast<uint32_t*>(ids_s + n_entries) : nullptr, mask_words);
@@ -387,7 +414,7 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, s
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                              float* weights, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
-    const size_t lds = (size_t)n_experts * 8 + 64;
+    const size_t lds = (size_t)(n_experts > kRouteScratch ? n_experts : kRouteScratch) * 8 + 64;
     hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)n), dim3(256), lds, stream, logits, (int)n_experts, top_k, mode,
                        ids, weights);
     return hipGetLastError();
@@ -422,7 +449,7 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
                                   int32_t* n_groups, int32_t* entry_token, int32_t* entry_k, bool build_groups,
                                   const float* qx, int64_t q_ldx, int64_t q_cols, uint8_t* q_aq, float* q_ad, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
-    const size_t lds_route = (size_t)n_experts * 8 + 64;
+    const size_t lds_route = (size_t)(n_experts > kRouteScratch ? n_experts : kRouteScratch) * 8 + 64;
     // one bit per (expert, token) for the grouping, up to 256 tokens
     int mask_words = n <= 256 ? (int)((n + 31) / 32) : 0;
     size_t lds_group = (size_t)n_experts * 4 + (size_t)n * top_k * 4;
@@ -436,14 +463,21 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
         if (e != hipSuccess || !qx) return e;
         return launch_quantize_q8k(qx, n, q_ldx, q_cols, nullptr, 0, q_aq, q_ad, stream);
     }
-    const int route_blocks = n <= 2 ? 1 : (int)n;
+    // Up to 64 tokens and 512 experts: one workgroup routes a token per wavefront and groups right away (measured
+    // against one workgroup per token + the last one to arrive grouping: the handshake costs more than the rounds).
+    const int threads = n <= 4 ? 256 : n <= 8 ? 512 : 1024;
+    const size_t lds_wave = (size_t)(threads / 64) * kRouteScratch * 8 + lds_group;
+    const bool wave_parallel = n <= 64 && n_experts <= 512 && lds_wave <= 60 * 1024;
+    const int route_blocks = wave_parallel || n <= 2 ? 1 : (int)n;
+    const int block = wave_parallel ? threads : 256;
     const int64_t q_nb = q_cols / kQK;
-    const int64_t quant_blocks = qx ? (n * q_nb + 3) / 4 : 0;
-    hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(256),
-                       lds_route > lds_group ? lds_route : lds_group, stream, logits, (int)n_experts, (int)n, top_k, mode,
-                       ids, weights, arrivals, group_expert, group_begin, n_groups, entry_token, entry_k, build_groups ? 1 : 0,
-                       route_blocks, mask_words, qx,
-                       q_ldx, q_nb, q_aq, q_ad);
+    const int64_t per_block = block / 64;
+    const int64_t quant_blocks = qx ? (n * q_nb + per_block - 1) / per_block : 0;
+    const size_t lds = wave_parallel ? lds_wave : (lds_route > lds_group ? lds_route : lds_group);
+    hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(block), lds, stream, logits,
+                       (int)n_experts, (int)n, top_k, mode, ids, weights, arrivals, group_expert, group_begin, n_groups,
+                       entry_token, entry_k, build_groups ? 1 : 0, route_blocks, mask_words, wave_parallel ? 1 : 0, qx, q_ldx,
+                       q_nb, q_aq, q_ad);
     return hipGetLastError();
 }
 

@@ -1,4 +1,5 @@
-"""The router inside the token-major MoE gate/up launch (up to eight tokens): the ids and weights that
+"""The routers inside the MoE launches -- in the token-major gate/up launch up to eight tokens, a token per
+wavefront of the routing + grouping launch up to 64, a workgroup per token beyond: the ids and weights that
 mq_moe_layer_q4k hands back against the oracle's stable top-k (core/src/llm/moe/native.cpp:610-676, :800-868) on rows
 made to hit every branch of the one-pass selection: plain rows, a few candidates, ties at the top (lower id first),
 ties that run across the cut, long runs of equal logits (more than 64 candidates: the round-by-round way), rows
@@ -47,7 +48,7 @@ def rows_for(e, n, seed):
 
 
 @pytest.mark.parametrize("e", [8, 40, 64, 100, 160, 256, 384, 512])
-@pytest.mark.parametrize("n", [1, 3, 8])
+@pytest.mark.parametrize("n", [1, 3, 8, 16, 40, 64, 70])
 def test_ids_and_weights_from_the_token_major_launch(ops, e, n):
     import torch
     hidden, inter, top_k = 256, 256, 8
