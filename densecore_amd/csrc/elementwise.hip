@@ -92,10 +92,36 @@ __global__ void __launch_bounds__(256) add_rmsnorm_blocks_kernel(const float* x,
         ssq = __fmaf_rn(a.w, a.w, ssq);
         slot = a;
     };
+    // kKeep > 0: every operand of the row -- x, residual, norm weights -- is requested first and unconditionally (a
+    // block past the end re-reads block 0, a missing residual or weight re-reads x), and nothing is stored before
+    // the barrier: conditional loads go out one round trip after the other, and a barrier waits for earlier stores.
+    float4 wn[kKeep > 0 ? kKeep : 1];
     if (kKeep > 0) {
+        const float* dp = delta ? delta : x;
+        const float* wp = weight ? weight : x;
+        float4 dl[kKeep > 0 ? kKeep : 1];
 #pragma unroll
-        for (int i = 0; i < kKeep; ++i)
-            if (wave + 4 * i < nb) first_pass(wave + 4 * i, kept[i]);
+        for (int i = 0; i < kKeep; ++i) {
+            const int64_t c0 = (wave + 4 * i < nb ? wave + 4 * i : 0) * kQK + lane * 4;
+            kept[i] = *reinterpret_cast<const float4*>(x + base + c0);
+            dl[i] = *reinterpret_cast<const float4*>(dp + base + c0);
+            wn[i] = *reinterpret_cast<const float4*>(wp + c0);
+        }
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i) {
+            if (wave + 4 * i < nb) {
+                float4 a = kept[i];
+                if (delta) {
+                    const float4 d = dl[i];
+                    a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
+                }
+                ssq = __fmaf_rn(a.x, a.x, ssq);
+                ssq = __fmaf_rn(a.y, a.y, ssq);
+                ssq = __fmaf_rn(a.z, a.z, ssq);
+                ssq = __fmaf_rn(a.w, a.w, ssq);
+                kept[i] = a;
+            }
+        }
     } else {
         for (int64_t b = wave; b < nb; b += 4) first_pass(b, kept[0]);
     }
@@ -116,8 +142,18 @@ __global__ void __launch_bounds__(256) add_rmsnorm_blocks_kernel(const float* x,
     };
     if (kKeep > 0) {
 #pragma unroll
-        for (int i = 0; i < kKeep; ++i)
-            if (wave + 4 * i < nb) second_pass(wave + 4 * i, kept[i]);
+        for (int i = 0; i < kKeep; ++i) {
+            if (wave + 4 * i < nb) {
+                const int64_t b = wave + 4 * i, c0 = b * kQK + lane * 4;
+                const float4 a = kept[i], w = wn[i];
+                // sum_out may alias x: every thread has read its own elements long before it stores them
+                if (sum_out) *reinterpret_cast<float4*>(sum_out + base + c0) = a;
+                const float e[4] = {__fmul_rn(a.x, weight ? __fmul_rn(scale, w.x) : scale), __fmul_rn(a.y, weight ? __fmul_rn(scale, w.y) : scale),
+                                    __fmul_rn(a.z, weight ? __fmul_rn(scale, w.z) : scale), __fmul_rn(a.w, weight ? __fmul_rn(scale, w.w) : scale)};
+                if (normed_out) *reinterpret_cast<float4*>(normed_out + base + c0) = make_float4(e[0], e[1], e[2], e[3]);
+                if (q_aq) store_amajor(q_aq, q_ad, blockIdx.x, b, nb, lane, quantize_block_q8k(e, lane));
+            }
+        }
     } else {
         for (int64_t b = wave; b < nb; b += 4) {
             const int64_t c0 = b * kQK + lane * 4;

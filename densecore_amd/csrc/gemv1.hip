@@ -201,7 +201,8 @@ __global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __
 // back as the split-slot A operand (common.h) -- and with kNorm the residual add and the RMSNorm of the rows run
 // inside as in gemv1_norm_fused_kernel.  Wave split of K, accumulation order and epilogue are matmul_kernel<1,1>'s:
 // the bits of quantize (or mq_add_rmsnorm_q8k) + matmul.
-template <bool kNorm>
+// RMAX (2, 4 or 8 >= n) bounds the registers of the stage operands, which are requested before the tiles.
+template <bool kNorm, int RMAX>
 __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restrict__ w, int64_t rows, int64_t nb,
                                                           const float* __restrict__ x, int64_t ldx, const float* __restrict__ delta,
                                                           const float* __restrict__ weight, float eps, float* __restrict__ sum_out,
@@ -219,29 +220,42 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
     float* scales = reinterpret_cast<float*>(codes + 8 * 256);
     float* red = reinterpret_cast<float*>(lds_raw + (size_t)n_waves * (8 * 256 + 32));
     const int64_t cols = nb * kQK;
-    auto fetch = [&](int t, int64_t c0) {
-        float4 a = *reinterpret_cast<const float4*>(x + (size_t)t * ldx + c0);
-        if (kNorm && delta) {
-            const float4 d = *reinterpret_cast<const float4*>(delta + (size_t)t * cols + c0);
-            a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
-        }
+    // Requests are unconditional (a row past n re-reads the last row, a stage past the end block 0, a missing
+    // residual or weight x) and those of the stages go out before the tiles: requests are answered in order.
+    const float* dp = kNorm && delta ? delta : x;
+    const int64_t ldd = kNorm && delta ? cols : ldx;
+    const float* wp = kNorm && weight ? weight : x;
+    auto add = [&](float4 a, const float4& d) {
+        if (kNorm && delta) a.x = __fadd_rn(a.x, d.x), a.y = __fadd_rn(a.y, d.y), a.z = __fadd_rn(a.z, d.z), a.w = __fadd_rn(a.w, d.w);
         return a;
     };
-
+    float4 xv[kMaxStages][RMAX], dv[kMaxStages][kNorm ? RMAX : 1], wn[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        const int64_t c0 = (int64_t)(i < cnt ? wave + i * n_waves : 0) * kQK + lane * 4;
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+            const int rr = r < n ? r : n - 1;
+            xv[i][r] = *reinterpret_cast<const float4*>(x + (size_t)rr * ldx + c0);
+            if (kNorm) dv[i][r] = *reinterpret_cast<const float4*>(dp + (size_t)rr * ldd + c0);
+        }
+        if (kNorm) wn[i] = *reinterpret_cast<const float4*>(wp + c0);
+    }
     TileRegs t[kMaxStages];
 #pragma unroll
     for (int i = 0; i < kMaxStages; ++i) load_tile(t[i], tiles + (size_t)(i < cnt ? wave + i * n_waves : 0) * kTileBytes, lane);
 
-    float scale[8];
+    float scale[RMAX];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) scale[r] = 1.0f;
+    for (int r = 0; r < RMAX; ++r) scale[r] = 1.0f;
     if (kNorm) {
         // sums of squares in the order of the 256-thread norm kernel: virtual wavefront v = 0..3, row by row
         for (int v = wave; v < 4; v += n_waves) {
             for (int r = 0; r < n; ++r) {
                 float ssq = 0.0f;
                 for (int64_t b = v; b < nb; b += 4) {
-                    const float4 a = fetch(r, b * kQK + lane * 4);
+                    const int64_t c0 = b * kQK + lane * 4;
+                    const float4 a = add(*reinterpret_cast<const float4*>(x + (size_t)r * ldx + c0), *reinterpret_cast<const float4*>(dp + (size_t)r * ldd + c0));
                     ssq = __fmaf_rn(a.x, a.x, ssq);
                     ssq = __fmaf_rn(a.y, a.y, ssq);
                     ssq = __fmaf_rn(a.z, a.z, ssq);
@@ -254,7 +268,7 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
         }
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
+        for (int r = 0; r < RMAX; ++r) {
             if (r < n) {
                 const float total = (wave_sum[r][0] + wave_sum[r][1]) + (wave_sum[r][2] + wave_sum[r][3]);
                 scale[r] = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)cols), eps)));
@@ -272,24 +286,18 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
 #pragma unroll
     for (int i = 0; i < kMaxStages; ++i) {
         if (i < cnt) {
-            const int64_t c0 = (int64_t)(wave + i * n_waves) * kQK + lane * 4;
-            float4 xv[8];
+            const float4 wv = wn[i];
 #pragma unroll
-            for (int r = 0; r < 8; ++r)
-                if (r < n) xv[r] = fetch(r, c0);
-            float4 wn = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
-            if (kNorm && weight) wn = *reinterpret_cast<const float4*>(weight + c0);
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
+            for (int r = 0; r < RMAX; ++r) {
                 if (r < n) {  // wave-uniform
-                    const float4 a = xv[r];
-                    if (kNorm && rt == 0 && sum_out) *reinterpret_cast<float4*>(sum_out + (size_t)r * cols + c0) = a;
+                    const float4 a = kNorm ? add(xv[i][r], dv[i][r]) : xv[i][r];
+                    xv[i][r] = a;
                     float e[4] = {a.x, a.y, a.z, a.w};
                     if (kNorm) {
-                        e[0] = __fmul_rn(a.x, weight ? __fmul_rn(scale[r], wn.x) : scale[r]);
-                        e[1] = __fmul_rn(a.y, weight ? __fmul_rn(scale[r], wn.y) : scale[r]);
-                        e[2] = __fmul_rn(a.z, weight ? __fmul_rn(scale[r], wn.z) : scale[r]);
-                        e[3] = __fmul_rn(a.w, weight ? __fmul_rn(scale[r], wn.w) : scale[r]);
+                        e[0] = __fmul_rn(a.x, weight ? __fmul_rn(scale[r], wv.x) : scale[r]);
+                        e[1] = __fmul_rn(a.y, weight ? __fmul_rn(scale[r], wv.y) : scale[r]);
+                        e[2] = __fmul_rn(a.z, weight ? __fmul_rn(scale[r], wv.z) : scale[r]);
+                        e[3] = __fmul_rn(a.w, weight ? __fmul_rn(scale[r], wv.w) : scale[r]);
                     }
                     const Q8Lane q = quantize_block_q8k(e, lane);
                     *reinterpret_cast<uint32_t*>(codes + r * 256 + ((((lane >> 4) ^ (r & 3)) << 6) | ((lane & 15) << 2))) = q.packed;
@@ -329,6 +337,17 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
                 if (2 * kq + j < n) y[(size_t)(2 * kq + j) * ldy + row] = acc[0][j];
         }
     }
+    if (kNorm && rt == 0 && sum_out) {  // last: a store ahead of a barrier would make the barrier wait for it
+#pragma unroll
+        for (int i = 0; i < kMaxStages; ++i) {
+            if (i < cnt) {
+                const int64_t c0 = (int64_t)(wave + i * n_waves) * kQK + lane * 4;
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r)
+                    if (r < n) *reinterpret_cast<float4*>(sum_out + (size_t)r * cols + c0) = xv[i][r];
+            }
+        }
+    }
 }
 
 }  // namespace
@@ -339,12 +358,19 @@ hipError_t launch_gemvn_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
     if (!gemv1_fused_applies(nb, waves) || rows <= 0 || n < 1 || n > 8) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16;
     const size_t lds = (size_t)waves * (8 * 256 + 32) + (waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0);
-    if (norm)
-        hipLaunchKernelGGL(gemvn_fused_kernel<true>, dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx, delta,
-                           weight, eps, sum_out, y, ldy, n);
-    else
-        hipLaunchKernelGGL(gemvn_fused_kernel<false>, dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx,
-                           delta, weight, eps, sum_out, y, ldy, n);
+#define MQ_GEMVN(NORM, RMAX)                                                                                                 \
+    hipLaunchKernelGGL((gemvn_fused_kernel<NORM, RMAX>), dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx, \
+                       delta, weight, eps, sum_out, y, ldy, n)
+    if (norm) {
+        if (n <= 2) MQ_GEMVN(true, 2);
+        else if (n <= 4) MQ_GEMVN(true, 4);
+        else MQ_GEMVN(true, 8);
+    } else {
+        if (n <= 2) MQ_GEMVN(false, 2);
+        else if (n <= 4) MQ_GEMVN(false, 4);
+        else MQ_GEMVN(false, 8);
+    }
+#undef MQ_GEMVN
     return hipGetLastError();
 }
 

@@ -338,6 +338,20 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
     __shared__ float wave_sum[4];
     const int64_t tok = blockIdx.y;
     const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    // Every partial row, id and weight is requested before anything else and unconditionally (a slot past top_k or
+    // a row past the end re-reads slot 0 / row 0; a dropped slot's row may hold anything: it is read and thrown
+    // away), so that all of them and the gate operands below travel together.
+    const int64_t rr = r < rows ? r : 0;
+    float pv[9], wk[8];
+    int ek[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int kk = k < top_k ? k : 0;
+        ek[k] = ids[tok * top_k + kk];
+        wk[k] = weights[tok * top_k + kk];
+        pv[k] = part[(tok * slots + kk) * rows + rr];
+    }
+    pv[8] = part[(tok * slots + (has_shared ? top_k : 0)) * rows + rr];
     float gate = 1.0f;
     if (has_shared && sh_gate_inp) {
         // thread j takes columns j, j + 256, ... in turn; the operands are requested eight columns at a time so that
@@ -360,25 +374,13 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
         gate = stable_sigmoid((wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]));
     }
     if (r >= rows) return;
-    // every partial row is requested before the first is added (a dropped slot's row may hold anything: it is read
-    // and thrown away), then the sum runs in routing order as before
-    float pv[9], wk[8];
-    bool live[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        live[k] = false;
-        if (k < top_k) {
-            const int e = ids[tok * top_k + k];
-            wk[k] = weights[tok * top_k + k];
-            live[k] = e >= 0 && e < n_experts && wk[k] != 0.0f;
-            pv[k] = part[(tok * slots + k) * rows + r];
-        }
-    }
-    if (has_shared) pv[8] = part[(tok * slots + top_k) * rows + r];
+    // the sum runs in routing order
     float acc = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-        if (live[k]) acc = __fadd_rn(acc, __fmul_rn(pv[k], wk[k]));
+    for (int k = 0; k < 8; ++k) {
+        const bool live = k < top_k && ek[k] >= 0 && ek[k] < n_experts && wk[k] != 0.0f;
+        if (live) acc = __fadd_rn(acc, __fmul_rn(pv[k], wk[k]));
+    }
     if (has_shared) acc = __fadd_rn(acc, __fmul_rn(pv[8], gate));
     y[tok * rows + r] = acc;
 }
