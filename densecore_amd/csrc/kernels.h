@@ -214,6 +214,8 @@ struct MoeDownTokenArgs {
     int64_t n = 0;
     int top_k = 0, n_experts = 0;
     uint32_t inv_nb = 0;               // ceil(2^32 / nb) for nb > 1, filled in by the launcher: i / nb == umulhi(i, inv_nb) for i, nb < 2^16
+    uint32_t inv_items = 0;            // the same for slots * nb (> 1)
+    int rt_per_wg = 1;                 // row tiles of one token per workgroup (launcher)
     const uint8_t* aq = nullptr;       // A-major hidden rows, or
     const float* ad = nullptr;
     const float* hidden = nullptr;     // fp32 hidden rows [n * slots][nb * 256] (quantized inside the kernel)

@@ -139,6 +139,103 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
     }
 }
 
+// The same product when a row takes one wavefront (many tokens: every (token, slot, row tile) would be a one-wave
+// workgroup that routes its token and quantizes all of x by itself, 288 times per token).  Here a workgroup owns a
+// (token, row tile) and has a wavefront per slot: wavefront 0 routes the token while the others quantize x into
+// LDS, one super-block each -- once per workgroup instead of once per slot -- and after one barrier every
+// wavefront streams its own expert's tiles against the shared codes.  A wavefront adds the super-blocks 0, 1, ...
+// in turn: the order of the one-wave workgroups, the same bits.
+template <int WT>
+__global__ void __launch_bounds__(576) moe_gateup_slots_kernel(const MoeGateupTokenArgs p) {
+    constexpr int kTileStride = tile_stride<WT>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t xq[];  // [nb][64] packed codes (lane l: elements 4l .. 4l+3), then [nb] scales
+    __shared__ int ids_sh[8];
+    __shared__ unsigned long long route_sh[kRouteScratch];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int slots = blockDim.x >> 6;  // top_k + shared expert
+    const int slot = lane & 15, kq = lane >> 4;
+    const int64_t rt = blockIdx.x;
+    const int tok = blockIdx.y, sl = wave;
+    const bool shared = sl >= p.top_k;
+    const int nb = (int)p.nb;
+    uint32_t* codes = reinterpret_cast<uint32_t*>(xq);
+    float* scales = reinterpret_cast<float*>(xq + (size_t)nb * 256);
+
+    if (wave == 0) {
+        const float* row = p.logits + (size_t)tok * p.n_experts;
+        auto load = [&](int e) { return row[e]; };
+        int id;
+        float logit;
+        if (p.n_experts <= 256) route_token_wave_lds<4>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
+        else route_token_wave_lds<8>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
+        if (lane < p.top_k) ids_sh[lane] = id;
+        if (rt == 0) {  // one workgroup per token hands ids and weights to the down projection
+            const float w = route_weight_lane(logit, lane, p.top_k, p.route_mode);
+            if (lane < p.top_k) {
+                p.ids_out[(size_t)tok * p.top_k + lane] = id;
+                p.weights_out[(size_t)tok * p.top_k + lane] = w;
+            }
+        }
+    }
+    if (wave > 0 || slots == 1) {  // the quantizing wavefronts share the super-blocks of x
+        const int first = slots > 1 ? wave - 1 : 0, step = slots > 1 ? slots - 1 : 1;
+        const float* xrow = p.x + (size_t)tok * (size_t)nb * kQK + lane * 4;
+        for (int b = first; b < nb; b += step) {
+            const float4 v = *reinterpret_cast<const float4*>(xrow + (size_t)b * kQK);
+            const float e[4] = {v.x, v.y, v.z, v.w};
+            const Q8Lane q = quantize_block_q8k(e, lane);
+            codes[b * 64 + lane] = q.packed;
+            if (lane == 0) scales[b] = q.d;
+        }
+    }
+    __syncthreads();
+    int expert = 0;
+    if (!shared) {
+        expert = ids_sh[sl];
+        if (expert < 0 || expert >= p.n_experts) return;  // dropped slot: its row is never read (no barrier follows)
+    }
+    const uint8_t* tiles[2] = {(shared ? p.sh_gate : p.gate + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride),
+                               (shared ? p.sh_up : p.up + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride)};
+    typename TileOf<WT>::Regs ring_t[kStages][2];
+    auto issue_t = [&](int st, int i) {
+        const int b = i < nb ? i : 0;  // a stage past the end re-reads block 0: the load count stays fixed
+#pragma unroll
+        for (int m = 0; m < 2; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)b * kTileStride, lane);
+    };
+#pragma unroll
+    for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
+    // this lane's words of a block's operand (a_codes_from_lane_codes): codes 64c + 32(slot & 1) + 8kq .. +7 of chunk c
+    const int src = 8 * (slot & 1) + 2 * kq;
+    float acc[2][1][2] = {{{0.0f, 0.0f}}, {{0.0f, 0.0f}}};
+    for (int base = 0; base < nb; base += kStages) {
+#pragma unroll
+        for (int st = 0; st < kStages; ++st) {
+            const int i = base + st;
+            issue_t((st + kStages - 1) % kStages, i + kStages - 1);
+            if (i < nb) {
+                ARegs<1> a;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const v2u v = *reinterpret_cast<const v2u*>(codes + i * 64 + 16 * c + src);
+                    a.q[0][c] = slot == 0 ? v4u{v.x, v.y, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, v.x, v.y} : v4u{0u, 0u, 0u, 0u});
+                }
+                a.yd[0][0] = scales[i];
+                a.yd[0][1] = 0.0f;
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {  // only row 0 of the operand is formed (J = 1)
+                    int32_t dsum[1][2], msum[1][2];
+                    compute_tile_wt<1, WT, 1>(ring_t[st][m], a, acc[m], dsum, msum, lane);
+                }
+            }
+        }
+    }
+    const int64_t row = rt * 16 + slot;
+    if (kq == 0 && row < p.rows)
+        p.hidden[((size_t)tok * slots + sl) * (size_t)p.rows + row] =
+            silu_mul(acc[0][0][0], acc[1][0][0], shared ? p.sh_silu_mode : p.silu_mode);
+}
+
 }  // namespace
 
 // Wavefronts of this kernel that ONE compute unit holds at once: by the registers the compiled kernel takes (512 per
@@ -180,6 +277,16 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
         !a.weights_out || (a.sh_gate == nullptr) != (a.sh_up == nullptr))
         return hipErrorInvalidValue;
     const int slots = a.top_k + (a.sh_gate ? 1 : 0);
+    if (a.waves == 1 && a.n <= 65535) {  // a row per wavefront: a workgroup per (token, row tile), a wavefront per slot
+        const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)a.n);
+        const size_t lds = (size_t)a.nb * 260;
+        if (lds > 48 * 1024) return hipErrorInvalidValue;
+        if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ6>, grid, dim3(64 * slots), lds, stream, a);
+        else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ5>, grid, dim3(64 * slots), lds, stream, a);
+        else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ4>, grid, dim3(64 * slots), lds, stream, a);
+        else return hipErrorInvalidValue;
+        return hipGetLastError();
+    }
     const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)slots, (unsigned)a.n);
     MoeGateupTokenArgs b = a;
     b.stages = (int)(a.nb / a.waves);
