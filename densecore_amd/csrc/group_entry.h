@@ -29,6 +29,26 @@ __device__ __forceinline__ void entry_rows(const MatmulArgs& p, bool shared_grou
     }
 }
 
+// The same for N entries at once: the list reads of all of them are requested together (one entry at a time they
+// are conditional loads, which go out one round trip after the other).
+template <bool GROUPED, int N>
+__device__ __forceinline__ void entry_rows_n(const MatmulArgs& p, bool shared_group, int begin, const int (&e)[N],
+                                             int (&ar)[N], int (&yr)[N]) {
+    if (!GROUPED || shared_group || p.direct_ids) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) entry_rows<GROUPED>(p, shared_group, begin, e[i], ar[i], yr[i]);
+    } else {
+        int tok[N], kk[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) tok[i] = p.entry_token[begin + e[i]], kk[i] = p.entry_k[begin + e[i]];
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            ar[i] = tok[i] * p.a_tok_stride + kk[i] * p.a_k_stride;
+            yr[i] = tok[i] * p.y_tok_stride + kk[i] * p.y_k_stride;
+        }
+    }
+}
+
 #endif
 
 }  // namespace mq

@@ -104,19 +104,17 @@ __global__ void __launch_bounds__(512, 4) grouped_lds_kernel(const MatmulArgs p)
 
     for (int chunk = 0; chunk < count; chunk += kTokTile) {
         // ---- rows behind this lane: its operand slot (gather source), its two outputs ----
-        auto map = [&](int pos, int& ar, int& yr) {
-            const int e_raw = chunk + pos;
-            const bool live = e_raw < count;
-            entry_rows<true>(p, shared_group, begin, live ? e_raw : count - 1, ar, yr);  // dead slot: a live row, never stored
-            if (!live) yr = -1;
-        };
-        int ar, yr, yrow[2];
-        map(slot >> 1, ar, yr);
-        const size_t a_off = aq_row_offset(ar, nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
-        map(2 * kq, ar, yrow[0]);
-        map(2 * kq + 1, ar, yrow[1]);
-        map(lane & 7, ar, yr);  // the scale this lane gathers: row lane % 8 of super-block lane / 8 (+ 8 per round)
-        const size_t d_row = (size_t)(ar >> 3) * (size_t)nb * 8 + (size_t)(ar & 7);
+        // the four entries this lane needs, looked up together: its operand row, the two rows it accumulates, and the
+        // row whose scale it gathers (row lane % 8 of super-block lane / 8, + 8 per round); a dead slot reads a live
+        // row and stores nothing
+        const int pos[4] = {slot >> 1, 2 * kq, 2 * kq + 1, lane & 7};
+        int ent[4], ars[4], yrs[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ent[i] = chunk + pos[i] < count ? chunk + pos[i] : count - 1;
+        entry_rows_n<true, 4>(p, shared_group, begin, ent, ars, yrs);
+        const size_t a_off = aq_row_offset(ars[0], nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
+        const int yrow[2] = {chunk + pos[1] < count ? yrs[1] : -1, chunk + pos[2] < count ? yrs[2] : -1};
+        const size_t d_row = (size_t)(ars[3] >> 3) * (size_t)nb * 8 + (size_t)(ars[3] & 7);
 
         if (chunk > 0) __syncthreads();  // everyone has finished reading the previous rows
         // ---- gather: operand chunk (b, c) = 1 KB in lane order; then the scales, eight super-blocks per copy ----

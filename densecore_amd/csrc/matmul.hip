@@ -136,20 +136,21 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
         int d_idx[TT][2], yrow[TT][2];
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
-            auto map = [&](int pos, int& ar, int& yr) {
-                const int e_raw = chunk + kTokTile * tt + pos;
-                const bool live = e_raw < count;
-                // dead slot: read a live row, store nothing
-                entry_rows<GROUPED>(p, shared_group, begin, live ? e_raw : count - 1, ar, yr);
-                if (!live) yr = -1;
-            };
-            int ar, yr;
-            map(slot >> 1, ar, yr);
-            a_off[tt] = aq_row_offset(ar, nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
+            // the three entries this lane needs, looked up together: its operand row and the two rows it
+            // accumulates; a dead slot reads a live row and stores nothing
+            const int pos[3] = {slot >> 1, 2 * kq, 2 * kq + 1};
+            int ent[3], ars[3], yrs[3];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                const int e_raw = chunk + kTokTile * tt + pos[i];
+                ent[i] = e_raw < count ? e_raw : count - 1;
+            }
+            entry_rows_n<GROUPED, 3>(p, shared_group, begin, ent, ars, yrs);
+            a_off[tt] = aq_row_offset(ars[0], nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                map(2 * kq + j, ar, yrow[tt][j]);
-                d_idx[tt][j] = (int)((size_t)(ar >> 3) * (size_t)nb * 8 + (size_t)(ar & 7));
+                yrow[tt][j] = chunk + kTokTile * tt + pos[1 + j] < count ? yrs[1 + j] : -1;
+                d_idx[tt][j] = (int)((size_t)(ars[1 + j] >> 3) * (size_t)nb * 8 + (size_t)(ars[1 + j] & 7));
             }
         }
 
