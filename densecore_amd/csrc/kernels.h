@@ -243,6 +243,7 @@ struct MoeGateupTokenArgs {
     int route_mode = 0, silu_mode = 0, sh_silu_mode = 2;
     int waves = 1;                     // wavefronts per workgroup: moe_gateup_token_waves(); nb % waves == 0
     int stages = 0;                    // nb / waves, filled in by the launcher (the kernel makes no division)
+    int slots_per_wg = 0;              // moe_gateup_slots_kernel: slots (wavefronts) of one workgroup, filled in by the launcher
     const float* x = nullptr;          // [n][nb * 256]
     const float* logits = nullptr;     // [n][n_experts]
     float* hidden = nullptr;           // [n * slots][rows]
@@ -253,6 +254,7 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
 // Wavefronts per workgroup for that launch (rows = hidden rows per expert), and the wavefronts the chip holds of it.
 int moe_gateup_token_waves(int64_t nb, int64_t rows, int64_t n, int slots, int wtype);
 int moe_gateup_token_capacity(int wtype);
+int moe_gateup_slots_capacity(int wtype);
 
 // ---- decoder_layers.hip ----------------------------------------------------------------------
 // A run of MoE decoder layers at decode width as one persistent launch (one workgroup per compute unit,

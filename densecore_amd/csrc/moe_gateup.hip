@@ -139,28 +139,33 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
     }
 }
 
-// The same product when a row takes one wavefront (many tokens: every (token, slot, row tile) would be a one-wave
-// workgroup that routes its token and quantizes all of x by itself, 288 times per token).  Here a workgroup owns a
-// (token, row tile) and has a wavefront per slot: wavefront 0 routes the token while the others quantize x into
-// LDS, one super-block each -- once per workgroup instead of once per slot -- and after one barrier every
-// wavefront streams its own expert's tiles against the shared codes.  A wavefront adds the super-blocks 0, 1, ...
-// in turn: the order of the one-wave workgroups, the same bits.
+// The same product for more (token, row tile) pairs (a workgroup per (token, slot, row tile) routes its token and
+// quantizes x by itself: 288 times per token).  Here a workgroup owns a (token, row tile) and a run of slots, W
+// wavefronts per slot (the wave split of moe_gateup_token_waves: the same partial sums, added in the same order)
+// -- all slots when there are enough (token, row tile) pairs for the chip, half or a third of them otherwise:
+// wavefront 0 routes the token while the others quantize x into LDS -- once per workgroup instead of once per
+// slot -- and after one barrier every wavefront streams its share of its expert's tiles against the shared codes.
 template <int WT>
-__global__ void __launch_bounds__(576) moe_gateup_slots_kernel(const MoeGateupTokenArgs p) {
+__global__ void __launch_bounds__(WT == kWtQ4 ? 1024 : 512) moe_gateup_slots_kernel(const MoeGateupTokenArgs p) {
     constexpr int kTileStride = tile_stride<WT>();
-    extern __shared__ __attribute__((aligned(16))) uint8_t xq[];  // [nb][64] packed codes (lane l: elements 4l .. 4l+3), then [nb] scales
+    extern __shared__ __attribute__((aligned(16))) uint8_t xq[];  // [nb][64] packed codes (lane l: elements 4l .. 4l+3), [nb] scales, then red [slots of the run][W-1][2][64]
     __shared__ int ids_sh[8];
     __shared__ unsigned long long route_sh[kRouteScratch];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int slots = blockDim.x >> 6;  // top_k + shared expert
+    const int slots = p.top_k + (p.sh_gate ? 1 : 0);
+    const int n_waves = blockDim.x >> 6, W = p.waves, per_wg = p.slots_per_wg;  // n_waves == per_wg * W
     const int slot = lane & 15, kq = lane >> 4;
     const int64_t rt = blockIdx.x;
-    const int tok = blockIdx.y, sl = wave;
+    // wave = local slot * W + part (W is 1, 2, 4 or 8: nb % W == 0 and W <= 8 -- W == 3, 5, 6, 7 go the other way)
+    const int wshift = W == 1 ? 0 : W == 2 ? 1 : W == 4 ? 2 : 3;
+    const int local = wave >> wshift, part = wave & (W - 1);
+    const int tok = blockIdx.z, sl = blockIdx.y * per_wg + local;
     const bool shared = sl >= p.top_k;
-    const int nb = (int)p.nb;
+    const int nb = (int)p.nb, cnt = p.stages;  // super-blocks part, part + W, ... of this wavefront
     uint32_t* codes = reinterpret_cast<uint32_t*>(xq);
     float* scales = reinterpret_cast<float*>(xq + (size_t)nb * 256);
+    float* red = scales + ((nb + 63) & ~63);
 
     if (wave == 0) {
         const float* row = p.logits + (size_t)tok * p.n_experts;
@@ -170,7 +175,7 @@ __global__ void __launch_bounds__(576) moe_gateup_slots_kernel(const MoeGateupTo
         if (p.n_experts <= 256) route_token_wave_lds<4>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
         else route_token_wave_lds<8>(load, p.n_experts, p.top_k, lane, id, logit, route_sh);
         if (lane < p.top_k) ids_sh[lane] = id;
-        if (rt == 0) {  // one workgroup per token hands ids and weights to the down projection
+        if (rt == 0 && blockIdx.y == 0) {  // one workgroup per token hands ids and weights to the down projection
             const float w = route_weight_lane(logit, lane, p.top_k, p.route_mode);
             if (lane < p.top_k) {
                 p.ids_out[(size_t)tok * p.top_k + lane] = id;
@@ -178,8 +183,8 @@ __global__ void __launch_bounds__(576) moe_gateup_slots_kernel(const MoeGateupTo
             }
         }
     }
-    if (wave > 0 || slots == 1) {  // the quantizing wavefronts share the super-blocks of x
-        const int first = slots > 1 ? wave - 1 : 0, step = slots > 1 ? slots - 1 : 1;
+    if (wave > 0 || n_waves == 1) {  // the quantizing wavefronts share the super-blocks of x
+        const int first = n_waves > 1 ? wave - 1 : 0, step = n_waves > 1 ? n_waves - 1 : 1;
         const float* xrow = p.x + (size_t)tok * (size_t)nb * kQK + lane * 4;
         for (int b = first; b < nb; b += step) {
             const float4 v = *reinterpret_cast<const float4*>(xrow + (size_t)b * kQK);
@@ -191,43 +196,61 @@ __global__ void __launch_bounds__(576) moe_gateup_slots_kernel(const MoeGateupTo
     }
     __syncthreads();
     int expert = 0;
-    if (!shared) {
+    bool live = sl < slots;  // the last run of slots may be shorter
+    if (live && !shared) {
         expert = ids_sh[sl];
-        if (expert < 0 || expert >= p.n_experts) return;  // dropped slot: its row is never read (no barrier follows)
+        live = expert >= 0 && expert < p.n_experts;  // dropped slot: its row is never read
     }
-    const uint8_t* tiles[2] = {(shared ? p.sh_gate : p.gate + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride),
-                               (shared ? p.sh_up : p.up + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride)};
-    typename TileOf<WT>::Regs ring_t[kStages][2];
-    auto issue_t = [&](int st, int i) {
-        const int b = i < nb ? i : 0;  // a stage past the end re-reads block 0: the load count stays fixed
-#pragma unroll
-        for (int m = 0; m < 2; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)b * kTileStride, lane);
-    };
-#pragma unroll
-    for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
-    // this lane's words of a block's operand (a_codes_from_lane_codes): codes 64c + 32(slot & 1) + 8kq .. +7 of chunk c
-    const int src = 8 * (slot & 1) + 2 * kq;
+    if (!live && W == 1) return;  // no barrier follows
     float acc[2][1][2] = {{{0.0f, 0.0f}}, {{0.0f, 0.0f}}};
-    for (int base = 0; base < nb; base += kStages) {
+    if (live) {
+        const uint8_t* tiles[2] = {(shared ? p.sh_gate : p.gate + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride),
+                                   (shared ? p.sh_up : p.up + (size_t)expert * p.expert_bytes) + tile_offset(rt, 0, nb, kTileStride)};
+        typename TileOf<WT>::Regs ring_t[kStages][2];
+        auto issue_t = [&](int st, int i) {
+            const int b = i < cnt ? part + i * W : 0;  // a stage past the end re-reads block 0: the load count stays fixed
 #pragma unroll
-        for (int st = 0; st < kStages; ++st) {
-            const int i = base + st;
-            issue_t((st + kStages - 1) % kStages, i + kStages - 1);
-            if (i < nb) {
-                ARegs<1> a;
+            for (int m = 0; m < 2; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)b * kTileStride, lane);
+        };
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const v2u v = *reinterpret_cast<const v2u*>(codes + i * 64 + 16 * c + src);
-                    a.q[0][c] = slot == 0 ? v4u{v.x, v.y, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, v.x, v.y} : v4u{0u, 0u, 0u, 0u});
-                }
-                a.yd[0][0] = scales[i];
-                a.yd[0][1] = 0.0f;
+        for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
+        // this lane's words of a block's operand (a_codes_from_lane_codes): codes 64c + 32(slot & 1) + 8kq .. +7 of chunk c
+        const int src = 8 * (slot & 1) + 2 * kq;
+        for (int base = 0; base < cnt; base += kStages) {
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {  // only row 0 of the operand is formed (J = 1)
-                    int32_t dsum[1][2], msum[1][2];
-                    compute_tile_wt<1, WT, 1>(ring_t[st][m], a, acc[m], dsum, msum, lane);
+            for (int st = 0; st < kStages; ++st) {
+                const int i = base + st;
+                issue_t((st + kStages - 1) % kStages, i + kStages - 1);
+                if (i < cnt) {
+                    const int b = part + i * W;
+                    ARegs<1> a;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const v2u v = *reinterpret_cast<const v2u*>(codes + b * 64 + 16 * c + src);
+                        a.q[0][c] = slot == 0 ? v4u{v.x, v.y, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, v.x, v.y} : v4u{0u, 0u, 0u, 0u});
+                    }
+                    a.yd[0][0] = scales[b];
+                    a.yd[0][1] = 0.0f;
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) {  // only row 0 of the operand is formed (J = 1)
+                        int32_t dsum[1][2], msum[1][2];
+                        compute_tile_wt<1, WT, 1>(ring_t[st][m], a, acc[m], dsum, msum, lane);
+                    }
                 }
             }
+        }
+    }
+    // partial sums of a slot meet in wave order (as in moe_gateup_token_kernel), SwiGLU, one store per weight row
+    if (W > 1) {
+        if (part > 0) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m) red[((local * (W - 1) + part - 1) * 2 + m) * 64 + lane] = acc[m][0][0];
+        }
+        __syncthreads();
+        if (!live || part > 0) return;
+        for (int wv = 1; wv < W; ++wv) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m) acc[m][0][0] = __fadd_rn(acc[m][0][0], red[((local * (W - 1) + wv - 1) * 2 + m) * 64 + lane]);
         }
     }
     const int64_t row = rt * 16 + slot;
@@ -258,6 +281,24 @@ int moe_gateup_token_capacity(int wtype) {
     return cached[k];
 }
 
+int moe_gateup_slots_capacity(int wtype) {
+    static int cached[3] = {0, 0, 0};
+    const int k = wtype == kTypeQ6K ? 2 : wtype == kTypeQ5K ? 1 : 0;
+    if (!cached[k]) {
+        const void* fn = wtype == kTypeQ6K   ? reinterpret_cast<const void*>(moe_gateup_slots_kernel<kWtQ6>)
+                         : wtype == kTypeQ5K ? reinterpret_cast<const void*>(moe_gateup_slots_kernel<kWtQ5>)
+                                             : reinterpret_cast<const void*>(moe_gateup_slots_kernel<kWtQ4>);
+        hipFuncAttributes attr;
+        int per_simd = 2;
+        if (hipFuncGetAttributes(&attr, fn) == hipSuccess && attr.numRegs > 0) {
+            per_simd = 512 / ((attr.numRegs + 7) / 8 * 8);
+            per_simd = per_simd < 1 ? 1 : per_simd > 8 ? 8 : per_simd;
+        }
+        cached[k] = per_simd * 4;
+    }
+    return cached[k];
+}
+
 // Wavefronts per workgroup: as many as divide the super-blocks of a row evenly (at most 8) while all workgroups of
 // the launch are resident at once -- a compute unit holds whole workgroups only.
 int moe_gateup_token_waves(int64_t nb, int64_t rows, int64_t n, int slots, int wtype) {
@@ -277,15 +318,39 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
         !a.weights_out || (a.sh_gate == nullptr) != (a.sh_up == nullptr))
         return hipErrorInvalidValue;
     const int slots = a.top_k + (a.sh_gate ? 1 : 0);
-    if (a.waves == 1 && a.n <= 65535) {  // a row per wavefront: a workgroup per (token, row tile), a wavefront per slot
-        const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)a.n);
-        const size_t lds = (size_t)a.nb * 260;
-        if (lds > 48 * 1024) return hipErrorInvalidValue;
-        if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ6>, grid, dim3(64 * slots), lds, stream, a);
-        else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ5>, grid, dim3(64 * slots), lds, stream, a);
-        else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ4>, grid, dim3(64 * slots), lds, stream, a);
-        else return hipErrorInvalidValue;
-        return hipGetLastError();
+    // A workgroup per (token, row tile, run of slots) with W wavefronts per slot (moe_gateup_slots_kernel) where that
+    // makes ONE round of one workgroup per compute unit with at least nine tenths of the units busy, and a slot takes
+    // one or two wavefronts (four and eight tokens at 256 compute units and 32 row tiles).  MoE block of 256 + 1
+    // experts, this form against the other at 1 .. 8 tokens with the nine-tenths rule off: 13.7 / 17.25 / 21.65 / 23.0 /
+    // (18 wavefronts: not possible) / 30.25 / 31.9 / 33.35 us against 13.55 / 17.15 / 21.3 / 24.4 / 29.6 / 30.75 /
+    // 31.5 / 35.0 -- with fewer units busy, or with four wavefronts per slot, nothing is gained.
+    const int64_t pairs = ((a.rows + 15) / 16) * a.n;
+    if ((a.waves == 1 || a.waves == 2) && a.n <= 65535 && (size_t)a.nb * 260 <= 32 * 1024) {
+        const int cus = compute_units();
+        const int cap = moe_gateup_slots_capacity(a.wtype);  // wavefronts of the kernel per compute unit
+        int per_wg = 0, runs = 0;
+        {
+            int r = (int)(cus / (pairs > 0 ? pairs : 1));
+            r = r < 1 ? 1 : r > slots ? slots : r;
+            const int pw = (slots + r - 1) / r, waves = pw * a.waves;
+            const int rr = (slots + pw - 1) / pw;
+            // Q5_K / Q6_K tiles take more registers: workgroups of eight wavefronts at most
+            if (waves <= (a.wtype == kTypeQ4K ? 16 : 8) && waves <= cap && pairs * rr <= cus && pairs * rr * 10 >= (int64_t)cus * 9)
+                per_wg = pw, runs = rr;
+        }
+        if (per_wg > 0) {
+            MoeGateupTokenArgs b = a;
+            b.stages = (int)(a.nb / a.waves);
+            b.slots_per_wg = per_wg;
+            const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)runs, (unsigned)a.n);
+            const size_t lds = (size_t)a.nb * 256 + (size_t)((a.nb + 63) & ~(int64_t)63) * 4 + (size_t)per_wg * (a.waves - 1) * 2 * 64 * 4;
+            const dim3 block(64 * per_wg * a.waves);
+            if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ6>, grid, block, lds, stream, b);
+            else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ5>, grid, block, lds, stream, b);
+            else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ4>, grid, block, lds, stream, b);
+            else return hipErrorInvalidValue;
+            return hipGetLastError();
+        }
     }
     const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)slots, (unsigned)a.n);
     MoeGateupTokenArgs b = a;
