@@ -185,6 +185,20 @@ __device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {
 constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
 
 // Maximum of an unsigned value over the 64 lanes, returned in every lane (wave-uniform).
+// acc + the partial sums of the wavefronts 1 .. n_waves-1 (n_waves <= 8) in wave order, part(wv) reading wavefront wv's
+// value from LDS: all seven reads are requested first (a wavefront past the end re-reads wavefront 1: its value is
+// read and dropped) -- inside a loop over a run-time wave count every read is a round trip to LDS of its own.
+template <class Part>
+__device__ __forceinline__ float add_wave_partials(float acc, int n_waves, Part part) {
+    float v[7];
+#pragma unroll
+    for (int wv = 1; wv < 8; ++wv) v[wv - 1] = part(wv < n_waves ? wv : 1);
+#pragma unroll
+    for (int wv = 1; wv < 8; ++wv)
+        if (wv < n_waves) acc = __fadd_rn(acc, v[wv - 1]);
+    return acc;
+}
+
 // unit = row * nb + block, split again.  The launchers keep the unit count below 2^31, so the division is a
 // 32-bit one: a 64-bit division is some 150 dependent scalar instructions at the head of a kernel that otherwise
 // runs for a few microseconds.

@@ -63,7 +63,7 @@ __global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restr
     }
     if (wave == 0) {
         float v = acc[0][0];
-        for (int wv = 1; wv < n_waves; ++wv) v = __fadd_rn(v, red[(wv - 1) * 64 + lane]);
+        if (n_waves > 1) v = add_wave_partials(v, n_waves, [&](int wv) { return red[(wv - 1) * 64 + lane]; });
         const int64_t row = rt * 16 + slot;
         if (kq == 0 && row < rows) y[row] = v;
     }
@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(512) gemv1_norm_fused_kernel(const uint8_t* __
     }
     if (wave == 0) {
         float v = acc[0][0];
-        for (int wv = 1; wv < n_waves; ++wv) v = __fadd_rn(v, red[(wv - 1) * 64 + lane]);
+        if (n_waves > 1) v = add_wave_partials(v, n_waves, [&](int wv) { return red[(wv - 1) * 64 + lane]; });
         const int64_t row = rt * 16 + slot;
         if (kq == 0 && row < rows) y[row] = v;
     }
@@ -326,9 +326,10 @@ __global__ void __launch_bounds__(512) gemvn_fused_kernel(const uint8_t* __restr
         __syncthreads();
     }
     if (wave == 0) {
-        for (int wv = 1; wv < n_waves; ++wv) {
-            acc[0][0] = __fadd_rn(acc[0][0], red[((wv - 1) * 2 + 0) * 64 + lane]);
-            acc[0][1] = __fadd_rn(acc[0][1], red[((wv - 1) * 2 + 1) * 64 + lane]);
+        if (n_waves > 1) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[0][j] = add_wave_partials(acc[0][j], n_waves, [&](int wv) { return red[((wv - 1) * 2 + j) * 64 + lane]; });
         }
         const int64_t row = rt * 16 + slot;
         if (row < rows) {

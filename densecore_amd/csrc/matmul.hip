@@ -324,15 +324,16 @@ __global__ void __launch_bounds__(512) matmul_kernel(const MatmulArgs p) {
             __syncthreads();
         }
         if (wave == 0 && rt_per_wg == 1) {
-            for (int wv = 1; wv < n_waves; ++wv) {
+            if (n_waves > 1) {
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
 #pragma unroll
                     for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
                         for (int j = 0; j < J; ++j)
-                            acc[m][tt][j] =
-                                __fadd_rn(acc[m][tt][j], red[((((wv - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane]);
+                            acc[m][tt][j] = add_wave_partials(acc[m][tt][j], n_waves, [&](int wv) {
+                                return red[((((wv - 1) * NMAT + m) * TT + tt) * 2 + j) * 64 + lane];
+                            });
             }
             store_rows(rt);
         }

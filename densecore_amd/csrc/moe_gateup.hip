@@ -128,9 +128,10 @@ __global__ void __launch_bounds__(512) moe_gateup_token_kernel(const MoeGateupTo
         __syncthreads();
     }
     if (wave == 0) {
-        for (int wv = 1; wv < n_waves; ++wv) {
+        if (n_waves > 1) {
 #pragma unroll
-            for (int m = 0; m < 2; ++m) acc[m][0][0] = __fadd_rn(acc[m][0][0], red[((wv - 1) * 2 + m) * 64 + lane]);
+            for (int m = 0; m < 2; ++m)
+                acc[m][0][0] = add_wave_partials(acc[m][0][0], n_waves, [&](int wv) { return red[((wv - 1) * 2 + m) * 64 + lane]; });
         }
         const int64_t row = rt * 16 + slot;
         if (kq == 0 && row < p.rows)
