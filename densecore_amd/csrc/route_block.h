@@ -137,16 +137,21 @@ __device__ __forceinline__ float route_weight_lane(float l, int lane, int top_k,
 // lowest expert id among the holders of that key (ballots, scanned in expert order), and the owner retires it.
 // load(e) returns logit e.  Lanes k < top_k end up with expert k of the routing order and its logit
 // (route_weight_lane turns those logits into the weights).
+// The logits of one token, KPL per lane (lane l: experts l, l + 64, ...).  Every lane reads KPL of them (a lane past
+// the end re-reads the last one): unconditional loads are requested together, not one round trip each.
 template <int KPL, typename Load>
-__device__ __forceinline__ void route_token_wave(Load load, int n_experts, int top_k, int lane, int& id_out,
-                                                 float& logit_out) {
-    uint32_t key[KPL];
-    float logit[KPL];
+__device__ __forceinline__ void route_load_logits(Load load, int n_experts, int lane, float (&logit)[KPL]) {
 #pragma unroll
-    for (int i = 0; i < KPL; ++i) {  // every lane reads KPL logits (a lane past the end re-reads the last one):
-        const int e = lane + 64 * i;  // unconditional loads are requested together, not one round trip each
+    for (int i = 0; i < KPL; ++i) {
+        const int e = lane + 64 * i;
         logit[i] = load(e < n_experts ? e : n_experts - 1);
     }
+}
+
+template <int KPL>
+__device__ __forceinline__ void route_logits_wave(const float (&logit)[KPL], int n_experts, int top_k, int lane, int& id_out,
+                                                  float& logit_out) {
+    uint32_t key[KPL];
 #pragma unroll
     for (int i = 0; i < KPL; ++i) key[i] = lane + 64 * i < n_experts ? route_key32(logit[i]) : 0u;
     float my_logit = 0.0f;
@@ -174,6 +179,14 @@ __device__ __forceinline__ void route_token_wave(Load load, int n_experts, int t
     logit_out = my_logit;
 }
 
+template <int KPL, typename Load>
+__device__ __forceinline__ void route_token_wave(Load load, int n_experts, int top_k, int lane, int& id_out,
+                                                 float& logit_out) {
+    float logit[KPL];
+    route_load_logits<KPL>(load, n_experts, lane, logit);
+    route_logits_wave<KPL>(logit, n_experts, top_k, lane, id_out, logit_out);
+}
+
 // The same routing in one pass for the common case, for a wavefront that has LDS of its own (kRouteScratch 64-bit
 // words, used by no other wavefront).  The smallest of the eight 8-lane group maxima is a key that at least eight
 // keys reach, so the top_k <= 8 first experts of the routing order are among the keys >= it (typically one or two
@@ -181,17 +194,11 @@ __device__ __forceinline__ void route_token_wave(Load load, int n_experts, int t
 // equal -- and every candidate counts the candidates ahead of it: its place in the routing order.  More than 64
 // candidates (rows of equal logits) go the round-by-round way; ids and logits are the same either way.
 constexpr int kRouteScratch = 72;
-template <int KPL, typename Load>
-__device__ __forceinline__ void route_token_wave_lds(Load load, int n_experts, int top_k, int lane, int& id_out,
-                                                     float& logit_out, unsigned long long* scratch) {
+template <int KPL>
+__device__ __forceinline__ void route_logits_wave_lds(const float (&logit)[KPL], int n_experts, int top_k, int lane, int& id_out,
+                                                      float& logit_out, unsigned long long* scratch) {
     uint32_t key[KPL];
-    float logit[KPL];
     uint32_t best = 0u;
-#pragma unroll
-    for (int i = 0; i < KPL; ++i) {  // unconditional loads (a lane past the end re-reads the last logit): one round trip
-        const int e = lane + 64 * i;
-        logit[i] = load(e < n_experts ? e : n_experts - 1);
-    }
 #pragma unroll
     for (int i = 0; i < KPL; ++i) {
         key[i] = lane + 64 * i < n_experts ? route_key32(logit[i]) : 0u;
@@ -214,7 +221,7 @@ __device__ __forceinline__ void route_token_wave_lds(Load load, int n_experts, i
         total += __popcll(mask[i]);
     }
     if (total > 64) {
-        route_token_wave<KPL>(load, n_experts, top_k, lane, id_out, logit_out);
+        route_logits_wave<KPL>(logit, n_experts, top_k, lane, id_out, logit_out);
         return;
     }
     scratch[lane] = 0ull;  // an empty place is ahead of nobody
@@ -246,6 +253,14 @@ __device__ __forceinline__ void route_token_wave_lds(Load load, int n_experts, i
         id_out = (int)(~(uint32_t)sel);
         logit_out = route_key32_logit((uint32_t)(sel >> 32));
     }
+}
+
+template <int KPL, typename Load>
+__device__ __forceinline__ void route_token_wave_lds(Load load, int n_experts, int top_k, int lane, int& id_out,
+                                                     float& logit_out, unsigned long long* scratch) {
+    float logit[KPL];
+    route_load_logits<KPL>(load, n_experts, lane, logit);
+    route_logits_wave_lds<KPL>(logit, n_experts, top_k, lane, id_out, logit_out, scratch);
 }
 
 // The logit behind a route_key (NaN comes back as a canonical NaN, -0 as +0: neither changes a weight).

@@ -1,6 +1,8 @@
 // MoE routing on the device: stable top-k + softmax over the selected logits, the expert-grouped
 // work list ("gather tokens by expert"), and the routing-order weighted combine.  Nothing here
 // returns to the host; the matmul kernels read the lists these kernels write.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 #include "q8k_block.h"
@@ -277,24 +279,45 @@ __global__ void __launch_bounds__(1024) route_and_group_kernel(const float* __re
         unsigned long long* scratch = route_sh + wave * kRouteScratch;
         int32_t* count = reinterpret_cast<int32_t*>(route_sh + n_waves * kRouteScratch);
         int32_t* ids_s = count + n_experts;
-        for (int tok = wave; tok < n; tok += n_waves) {
-            const float* row = logits + (size_t)tok * n_experts;
-            auto load = [&](int e) { return row[e]; };
-            int id;
-            float logit;
-            if (n_experts <= 256) route_token_wave_lds<4>(load, n_experts, top_k, lane, id, logit, scratch);
-            else route_token_wave_lds<8>(load, n_experts, top_k, lane, id, logit, scratch);
-            const float w = route_weight_lane(logit, lane, top_k, mode);
-            if (lane < top_k) {
-                ids[(size_t)tok * top_k + lane] = id;
-                weights[(size_t)tok * top_k + lane] = w;
-                ids_s[tok * top_k + lane] = id;
+        // the logits of all tokens of this wavefront (at most two: 32 tokens, 16 wavefronts) are requested first;
+        // ids and weights leave for global memory after the grouping (a store ahead of a barrier makes it wait)
+        int id_keep[2];
+        float w_keep[2];
+        auto route_all = [&](auto kpl_c) {
+            constexpr int KPL = decltype(kpl_c)::value;
+            float lg[2][KPL];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int tok = wave + r * n_waves < n ? wave + r * n_waves : n - 1;
+                const float* row = logits + (size_t)tok * n_experts;
+                route_load_logits<KPL>([&](int e) { return row[e]; }, n_experts, lane, lg[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int tok = wave + r * n_waves;
+                id_keep[r] = -1, w_keep[r] = 0.0f;
+                if (tok < n) {  // wave-uniform
+                    float logit;
+                    route_logits_wave_lds<KPL>(lg[r], n_experts, top_k, lane, id_keep[r], logit, scratch);
+                    w_keep[r] = route_weight_lane(logit, lane, top_k, mode);
+                    if (lane < top_k) ids_s[tok * top_k + lane] = id_keep[r];
+                }
+            }
+        };
+        if (n_experts <= 256) route_all(std::integral_constant<int, 4>{});
+        else route_all(std::integral_constant<int, 8>{});
+        // group_entries zeroes its counters and passes a barrier before it reads the ids
+        if (build_groups)
+            group_entries(ids_s, n * top_k, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
+                          mask_words ? reinterpret_cast<uint32_t*>(ids_s + n * top_k) : nullptr, mask_words);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int tok = wave + r * n_waves;
+            if (tok < n && lane < top_k) {
+                ids[(size_t)tok * top_k + lane] = id_keep[r];
+                weights[(size_t)tok * top_k + lane] = w_keep[r];
             }
         }
-        if (!build_groups) return;
-        // group_entries zeroes its counters and passes a barrier before it reads the ids
-        group_entries(ids_s, n * top_k, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
-                      mask_words ? reinterpret_cast<uint32_t*>(ids_s + n * top_k) : nullptr, mask_words);
         return;
     }
     const bool solo = route_blocks == 1;  // one or two tokens: one workgroup does everything, no handshake
@@ -465,11 +488,13 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
         if (e != hipSuccess || !qx) return e;
         return launch_quantize_q8k(qx, n, q_ldx, q_cols, nullptr, 0, q_aq, q_ad, stream);
     }
-    // Up to 64 tokens and 512 experts: one workgroup routes a token per wavefront and groups right away (measured
-    // against one workgroup per token + the last one to arrive grouping: the handshake costs more than the rounds).
+    // Up to 32 tokens and 512 experts: one workgroup routes a token or two per wavefront and groups right away.  Against
+    // one workgroup per token + the last one to arrive grouping (device-coherent id stores, an arrival count, a re-read):
+    // 6.0 against 8 us at 16 tokens, but 13.5 against 9 at 64 -- sixteen wavefronts on one compute unit route a token
+    // in 1.5-1.9 us each (they share its four SIMDs), and the handshake costs about 3 us.
     const int threads = n <= 4 ? 256 : n <= 8 ? 512 : 1024;
     const size_t lds_wave = (size_t)(threads / 64) * kRouteScratch * 8 + lds_group;
-    const bool wave_parallel = n <= 64 && n_experts <= 512 && lds_wave <= 60 * 1024;
+    const bool wave_parallel = n <= 32 && n_experts <= 512 && lds_wave <= 60 * 1024;
     const int route_blocks = wave_parallel || n <= 2 ? 1 : (int)n;
     const int block = wave_parallel ? threads : 256;
     const int64_t q_nb = q_cols / kQK;
