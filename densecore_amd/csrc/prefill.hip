@@ -8,29 +8,35 @@
 //     scale = 8*s1 + s0  (two 3-bit digits)   ->   (s1*q4) and (s0*q4) both fit a signed byte (<= 105)
 //     dot_scaled = 8 * sum_k (s1*q4)_k q8_k  +  sum_k (s0*q4)_k q8_k                  (exact, int32)
 // and the min term runs on the matrix cores as well, from the sub-block sums of the codes
-// bs_g = bsums[2g] + bsums[2g+1] = 128*h_g + l_g (h in [-32, 31], l in [0, 127], both bytes):
-//     min_dot = 128 * sum_g min_g h_g  +  sum_g min_g l_g                               (exact, int32)
+// bs_g = bsums[2g] + bsums[2g+1] = 128*h_g + l_g (h in [-32, 31], l in [0, 127]):
+//     min_dot = sum_g min_g (128 h_g)  +  sum_g min_g l_g
 // which is the reference's sum_j bsums[j] * min[j/2] (core/src/llm/matmul/kquant_batched_kernels.h:285-297).
-// Ten MFMAs per 16x16 output tile and super-block, no per-sub-block vector work; the fp32 update
+// One v_mfma_f32_16x16x32_f16 forms it: the sixteen operands l_g, 128 h_g and the mins are integers of at most
+// thirteen bits, exact as fp16; every product and every partial sum is an integer below 2^24, so the fp32 result
+// is the integer min_dot itself -- the value (float)min_dot that the update needs, with nothing to combine or
+// convert on the vector unit.
+// Nine MFMAs per 16x16 output tile and super-block, no per-sub-block vector work; the fp32 update
 //     acc += yd * (d * dot_scaled - dmin * min_dot)
-// is done once per super-block, as every reference kernel does (three fp32 operations per output; the reference's
+// is done once per super-block, as every reference kernel does (three fp32 operations per output, five vector
+// instructions with the digits' shift-add and one conversion; the reference's
 // grouping (d*yd) * dot_scaled - (dmin*yd) * min_dot takes four, and the update is what the kernel's vector unit is
 // busy with: 308 against 325 us at M = 2048; the two groupings differ in the last bits only).
 //
 //   grid      = (ceil(rowtiles / 8), ceil(m_tiles / 8)); workgroup = 4 wavefronts
-//   workgroup = 128 weight rows x 128 activation rows; per super-block the 128 activation rows (35 KB
+//   workgroup = 128 weight rows x 128 activation rows; per super-block the 128 activation rows (37 KB
 //               in the P-major layout below) are staged in LDS, double-buffered and requested one
 //               super-block ahead with LDS-direct loads
 //   wavefront = 2 weight tiles (32 rows) x the 8 activation tiles; it reads its weight tiles
 //               straight from HBM in MFMA lane order and expands them in registers
 //
-// P-major activations (written by quantize_q8k_pmajor_kernel): [b][mt][4416 B], mt = m / 16:
+// P-major activations (written by quantize_q8k_pmajor_kernel): [b][mt][4688 B], mt = m / 16:
 //   [j 0..3][kq 0..3][tok 0..15][16 B]   codes: bytes 0..7 = sub-block ga(j), elements 8kq..8kq+7,
 //                                        bytes 8..15 = sub-block gb(j), same elements, with
 //                                        (ga, gb) = (0,2) (1,3) (4,6) (5,7) for j = 0..3 -- the pairs
 //                                        that one 16-byte word of a weight tile holds per nibble half
-//   [tok][16 B] at 4096                  l_0..l_7, h_0..h_7
-//   [tok] fp32 at 4352                   block scale d
+//   [tok][32 B] at 4096                  fp16: l_0..l_7, then 128 h_0..128 h_7
+//   [tok] fp32 at 4608                   block scale d
+//   16 zero bytes at 4672                what the lanes of k-groups 2 and 3 feed the min MFMA
 #include "common.h"
 #include "kernels.h"
 #include "q8k_block.h"
@@ -39,28 +45,36 @@ namespace mq {
 
 namespace {
 
-constexpr int kPTileBytes = 4416;
-constexpr int kPTileWords = kPTileBytes / 16;  // 276
+constexpr int kPTileBytes = 4688;
+constexpr int kPTileWords = kPTileBytes / 16;  // 293
+constexpr int kPDigitOff = 4096, kPScaleOff = 4608, kPZeroOff = 4672;
 constexpr int kMTilesPerGroup = 8;             // activation tiles (of 16 rows) per workgroup
 constexpr int kWTilesPerWave = 2;
 
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
-// four bytes (each <= 15) times a 3-bit digit, bytewise; the digit comes replicated in both halves
-__device__ __forceinline__ uint32_t scale_bytes(uint32_t nibbles, uint32_t digit_pk) {
+// four bytes (each <= 15) times a 3-bit digit, bytewise: two 16-bit products whose bytes do not carry into each
+// other (15 * 7 < 256).  The digit is half H of `digits`, taken for both products (the operand-select bits of the
+// packed multiply: no instruction of its own).
+template <int H>
+__device__ __forceinline__ uint32_t scale_bytes(uint32_t nibbles, uint32_t digits) {
     const v2us a = __builtin_bit_cast(v2us, nibbles);
-    const v2us d = __builtin_bit_cast(v2us, digit_pk);
-    return __builtin_bit_cast(uint32_t, (v2us)(a * d));
+    const v2us d = __builtin_bit_cast(v2us, digits);
+    const v2us dd = H ? v2us{d.y, d.y} : v2us{d.x, d.x};
+    return __builtin_bit_cast(uint32_t, (v2us)(a * dd));
 }
 
-// byte `i` of `word` replicated into bits 0..7 and 16..23 (one v_perm_b32: selector 0x0c yields a zero byte)
+// bytes i and i + 1 of `word` as two 16-bit numbers (one v_perm_b32: selector 0x0c yields a zero byte)
 __device__ __forceinline__ uint32_t digit_pair(uint32_t word, int i) {
-    return __builtin_amdgcn_perm(0u, word, 0x0c000c00u | (uint32_t)i | ((uint32_t)i << 16));
+    return __builtin_amdgcn_perm(0u, word, 0x0c000c00u | (uint32_t)i | ((uint32_t)(i + 1) << 16));
 }
 
 struct WTile {
     v4i hi[4], lo[4];  // B operands of the four chunk pairs, scaled by the high / low scale digit
-    v4i mins;          // B operand of the min MFMAs (k-group 0 only)
+    v8h mins;          // B operand of the min MFMA: the eight mins as fp16, in every k-group
     float d, dmin;
 };
 
@@ -80,20 +94,25 @@ __device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, cons
         const uint32_t l2 = seg[i].z & 0x0f0f0f0fu, l3 = seg[i].w & 0x0f0f0f0fu;  // sub-block 4i+2
         const uint32_t h0 = (seg[i].x >> 4) & 0x0f0f0f0fu, h1 = (seg[i].y >> 4) & 0x0f0f0f0fu;  // 4i+1
         const uint32_t h2 = (seg[i].z >> 4) & 0x0f0f0f0fu, h3 = (seg[i].w >> 4) & 0x0f0f0f0fu;  // 4i+3
-        const uint32_t a1 = digit_pair(s1w, 0), a0 = digit_pair(s0w, 0);
-        const uint32_t b1 = digit_pair(s1w, 1), b0 = digit_pair(s0w, 1);
-        const uint32_t c1 = digit_pair(s1w, 2), c0 = digit_pair(s0w, 2);
-        const uint32_t e1 = digit_pair(s1w, 3), e0 = digit_pair(s0w, 3);
-        t.hi[2 * i] = v4i{(int)scale_bytes(l0, a1), (int)scale_bytes(l1, a1), (int)scale_bytes(l2, c1),
-                          (int)scale_bytes(l3, c1)};
-        t.lo[2 * i] = v4i{(int)scale_bytes(l0, a0), (int)scale_bytes(l1, a0), (int)scale_bytes(l2, c0),
-                          (int)scale_bytes(l3, c0)};
-        t.hi[2 * i + 1] = v4i{(int)scale_bytes(h0, b1), (int)scale_bytes(h1, b1), (int)scale_bytes(h2, e1),
-                              (int)scale_bytes(h3, e1)};
-        t.lo[2 * i + 1] = v4i{(int)scale_bytes(h0, b0), (int)scale_bytes(h1, b0), (int)scale_bytes(h2, e0),
-                              (int)scale_bytes(h3, e0)};
+        // digits of sub-blocks (4i, 4i+1) and (4i+2, 4i+3), two to a word
+        const uint32_t ab1 = digit_pair(s1w, 0), ab0 = digit_pair(s0w, 0);
+        const uint32_t ce1 = digit_pair(s1w, 2), ce0 = digit_pair(s0w, 2);
+        t.hi[2 * i] = v4i{(int)scale_bytes<0>(l0, ab1), (int)scale_bytes<0>(l1, ab1), (int)scale_bytes<0>(l2, ce1),
+                          (int)scale_bytes<0>(l3, ce1)};
+        t.lo[2 * i] = v4i{(int)scale_bytes<0>(l0, ab0), (int)scale_bytes<0>(l1, ab0), (int)scale_bytes<0>(l2, ce0),
+                          (int)scale_bytes<0>(l3, ce0)};
+        t.hi[2 * i + 1] = v4i{(int)scale_bytes<1>(h0, ab1), (int)scale_bytes<1>(h1, ab1), (int)scale_bytes<1>(h2, ce1),
+                              (int)scale_bytes<1>(h3, ce1)};
+        t.lo[2 * i + 1] = v4i{(int)scale_bytes<1>(h0, ab0), (int)scale_bytes<1>(h1, ab0), (int)scale_bytes<1>(h2, ce0),
+                              (int)scale_bytes<1>(h3, ce0)};
     }
-    t.mins = kq == 0 ? v4i{(int)mn03, (int)mn47, 0, 0} : v4i{0, 0, 0, 0};
+    // byte -> fp16: 0x6400 | n is 1024 + n; two at a time
+    const v2h bias = {(_Float16)1024.0f, (_Float16)1024.0f};
+    const v2h m01 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64006400u, mn03, 0x05010500u)) - bias;
+    const v2h m23 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64006400u, mn03, 0x05030502u)) - bias;
+    const v2h m45 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64006400u, mn47, 0x05010500u)) - bias;
+    const v2h m67 = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64006400u, mn47, 0x05030502u)) - bias;
+    t.mins = v8h{m01.x, m01.y, m23.x, m23.y, m45.x, m45.y, m67.x, m67.y};
     t.d = half_bits_to_float(hdr.x & 0xffffu);
     t.dmin = half_bits_to_float(hdr.x >> 16);
 }
@@ -112,8 +131,9 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
     // for them itself, with vmcnt(0) and a barrier, before the buffer is read.  M0 (the LDS base of the request)
     // is used by nothing else in this kernel.
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)buf;
+    static_assert(10 * 4 * 64 >= kMTilesPerGroup * kPTileWords, "ten rounds of requests cover the tiles of a group");
 #pragma unroll
-    for (int j = 0; j < 9; ++j) {  // 4 waves x 9 requests x 64 words >= 8 tiles x 276 words
+    for (int j = 0; j < 10; ++j) {  // 4 waves x 10 requests x 64 words >= 8 tiles x 293 words
         const int first = (j * 4 + wave) * 64;
         if (first + lane < copy_words) {
             const uint8_t* g = src + (size_t)(first + lane) * 16;
@@ -126,7 +146,7 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy) {
-    extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * 4416 bytes
+    extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -149,6 +169,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
             for (int i = 0; i < 4; ++i) acc[t][m][i] = 0.0f;
 
     const int copy_words = mt_count * kPTileWords;
+    // this lane's operand of the min MFMA: k-group 0 reads the l digits of token r, k-group 1 its 128 h digits, the others zeros
+    const int digit_off = kq < 2 ? kPDigitOff + r * 32 + kq * 16 : kPZeroOff;
     const uint8_t* a_src = ap + (size_t)mt0 * kPTileBytes;           // + b * a_stride
     const size_t a_stride = (size_t)m_tiles * kPTileBytes;
 
@@ -190,18 +212,17 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                 v4i a[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
-                const v4i dg = *reinterpret_cast<const v4i*>(at + 4096 + r * 16);
-                const float4 yd = *reinterpret_cast<const float4*>(at + 4352 + kq * 16);
-                const v4i a_l = kq == 0 ? v4i{dg.x, dg.y, 0, 0} : v4i{0, 0, 0, 0};
-                const v4i a_h = kq == 0 ? v4i{dg.z, dg.w, 0, 0} : v4i{0, 0, 0, 0};
+                const v8h dg = *reinterpret_cast<const v8h*>(at + digit_off);
+                const float4 yd = *reinterpret_cast<const float4*>(at + kPScaleOff + kq * 16);
                 const v4i zero = {0, 0, 0, 0};
-                v4i hi[kWTilesPerWave], lo[kWTilesPerWave], mh[kWTilesPerWave], ml[kWTilesPerWave];
+                const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
+                v4i hi[kWTilesPerWave], lo[kWTilesPerWave];
+                v4f mn[kWTilesPerWave];
 #pragma unroll
                 for (int t = 0; t < kWTilesPerWave; ++t) {
                     hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].hi[0], zero, 0, 0, 0);
                     lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].lo[0], zero, 0, 0, 0);
-                    mh[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_h, wt[t].mins, zero, 0, 0, 0);
-                    ml[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_l, wt[t].mins, zero, 0, 0, 0);
+                    mn[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt[t].mins, zero_f, 0, 0, 0);
                 }
 #pragma unroll
                 for (int j = 1; j < 4; ++j)
@@ -216,27 +237,30 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int dot = hi[t][i] * 8 + lo[t][i];
-                        const int mnd = mh[t][i] * 128 + ml[t][i];
                         // yd * (d * dot - dmin * min_dot): three fp32 operations per output and super-block
-                        const float v = __fmaf_rn(-wt[t].dmin, (float)mnd, __fmul_rn(wt[t].d, (float)dot));
+                        const float v = __fmaf_rn(-wt[t].dmin, mn[t][i], __fmul_rn(wt[t].d, (float)dot));
                         acc[t][m][i] = __fmaf_rn(ydv[i], v, acc[t][m][i]);
                     }
             }
         }
     }
 
+    // Stores: lane (r, kq) holds weight row r of its tiles for the tokens 16 m + 4 kq + i.  One pointer per lane walks
+    // down the token rows (an addition per store, no product).
+    const int tok_left = (int)(n_tokens - mt0 * 16) - kq * 4;  // tokens from this lane's first one to the end
 #pragma unroll
     for (int t = 0; t < kWTilesPerWave; ++t) {
         const int64_t row = (rt0 + t) * kTileRows + r;
         if (rt0 + t >= rowtiles || row >= rows) continue;
+        float* yp = y + (mt0 * 16 + kq * 4) * ldy + row;
 #pragma unroll
         for (int m = 0; m < kMTilesPerGroup; ++m) {
-            if (m >= mt_count) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int64_t tok = (mt0 + m) * 16 + kq * 4 + i;
-                if (tok < n_tokens) y[tok * ldy + row] = acc[t][m][i];
+                if (m < mt_count && m * 16 + i < tok_left) *yp = acc[t][m][i];
+                yp += ldy;
             }
+            yp += 12 * ldy;
         }
     }
 }
@@ -264,11 +288,13 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     const int kq = (lane & 7) >> 1;
     *reinterpret_cast<uint32_t*>(tile + j * 1024 + (kq * 16 + tok) * 16 + half * 8 + (lane & 1) * 4) = q.packed;
     const int bs = q.bsum + __shfl_xor(q.bsum, 4, 64);  // codes 32g .. 32g+31
-    if ((lane & 7) == 0) {
-        tile[4096 + tok * 16 + g] = (uint8_t)(bs & 127);
-        tile[4096 + tok * 16 + 8 + g] = (uint8_t)(bs >> 7);
+    if ((lane & 7) == 0) {  // bs = 128 h + l, both parts exact in fp16
+        _Float16* digits = reinterpret_cast<_Float16*>(tile + kPDigitOff + tok * 32);
+        digits[g] = (_Float16)(float)(bs & 127);
+        digits[8 + g] = (_Float16)(float)((bs >> 7) * 128);
     }
-    if (lane == 0) *reinterpret_cast<float*>(tile + 4352 + tok * 4) = q.d;
+    if (lane == 0) *reinterpret_cast<float*>(tile + kPScaleOff + tok * 4) = q.d;
+    if (tok == 0 && lane < 4) *reinterpret_cast<uint32_t*>(tile + kPZeroOff + lane * 4) = 0u;
 }
 
 }  // namespace
