@@ -525,8 +525,16 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
     return MQ_OK;
 }
 
-// Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk.
+// Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk: 48 in general,
+// 17 for matrices of 24 MB and more (14336 x 4096 and 4096 x 14336: 19 against 24 us at 17 rows, 21 against 35-38 us
+// at 47; 4096 x 4096: 17.4 against 14.1 us at 17 rows, 17.9 against 14.6 at 47).
 constexpr int64_t kPrefillMinRows = 48;
+constexpr int64_t kPrefillMinRowsLarge = 17;
+constexpr int64_t kPrefillLargeBytes = 24ll << 20;
+static bool prefill_applies(const mq_weight* w, int64_t n) {
+    if (w->type != kTypeQ4K) return false;
+    return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
+}
 constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
 // Widest product that also runs the residual add and the RMSNorm inside the GEMV kernel: every workgroup repeats the
 // rows' norm, about 1.25 us per row.  Decoder layer (2048 hidden, 64 experts) with the norm inside / as a launch of
@@ -538,7 +546,10 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
     if (n == 0) return MQ_OK;
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, w->nb)));
     MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, w->cols, (uint8_t*)g.ap.ptr, s));
-    MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy, s));
+    const size_t part_bytes = prefill_part_bytes(w->rows, w->nb, n);
+    if (part_bytes) MQ_HIP(g.part.reserve(part_bytes));
+    MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy,
+                               part_bytes ? (float*)g.part.ptr : nullptr, s));
     return MQ_OK;
 }
 
@@ -591,7 +602,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     Entry entry(s);
     if (entry.rc) return entry.rc;
     if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, nullptr, s);
-    if (n >= kPrefillMinRows && w->type == kTypeQ4K) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
+    if (prefill_applies(w, n)) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
     if (n == 1 && !census.on && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {

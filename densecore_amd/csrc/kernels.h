@@ -162,9 +162,12 @@ hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
 size_t pmajor_bytes(int64_t n, int64_t nb);
 hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
                                       hipStream_t stream);
-// y[n][ldy] = P-major activations . tiled weights^T on the int8 matrix cores.
+// y[n][ldy] = P-major activations . tiled weights^T on the int8 matrix cores.  A launch that would leave workgroup
+// slots empty splits K into runs of super-blocks whose sums go to planes of `part` (prefill_part_bytes() bytes, 0 when
+// nothing is split) and are added in order by a second launch.
+size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n);
 hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
-                               int64_t ldy, hipStream_t stream);
+                               int64_t ldy, float* part, hipStream_t stream);
 
 // ---- elementwise.hip -------------------------------------------------------------------------
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,

@@ -49,7 +49,6 @@ constexpr int kPTileBytes = 4688;
 constexpr int kPTileWords = kPTileBytes / 16;  // 293
 constexpr int kPDigitOff = 4096, kPScaleOff = 4608, kPZeroOff = 4672;
 constexpr int kMTilesPerGroup = 8;             // activation tiles (of 16 rows) per workgroup
-constexpr int kWTilesPerWave = 2;
 
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -143,9 +142,13 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
     }
 }
 
+// kWTilesPerWave = 2: the 128 x 128 workgroup tile above.  1: 64 weight rows per workgroup, for launches whose
+// 128-row workgroups would leave compute units without their two workgroups (M up to a few hundred).
+template <int kWTilesPerWave>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
-                                                           int64_t n_tokens, float* __restrict__ y, int64_t ldy) {
+                                                           int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
+                                                           int64_t split_stride) {
     extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     const int tid = threadIdx.x;
@@ -187,10 +190,15 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
             hdr[t] = load16(tile + kTileQBytes + r * 16);
         }
     };
-    request_a_tiles(a_src, a_lds, copy_words, wave, lane);
-    request_w(0);
+    // K split over grid.z: this workgroup multiplies the super-blocks [b_begin, b_end) and writes its sums to
+    // partial plane blockIdx.z (split_stride floats apart; the caller adds the planes in order)
+    const int64_t b_begin = (int64_t)blockIdx.z * sb_split;
+    const int64_t b_end = b_begin + sb_split < nb ? b_begin + sb_split : nb;
+    y += (size_t)blockIdx.z * (size_t)split_stride;
+    request_a_tiles(a_src + (size_t)b_begin * a_stride, a_lds + (b_begin & 1) * kBufBytes, copy_words, wave, lane);
+    request_w(b_begin);
 
-    for (int64_t b = 0; b < nb; ++b) {
+    for (int64_t b = b_begin; b < b_end; ++b) {
         // everything this thread requested for super-block b has landed ...
         __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4) | (0xF << 8));  // vmcnt(0)
         // ... and after the barrier so has everybody else's share of the activation tiles; every wave
@@ -199,7 +207,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         WTile wt[kWTilesPerWave];
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) expand_tile(seg0[t], seg1[t], hdr[t], kq, wt[t]);
-        if (b + 1 < nb) {
+        if (b + 1 < b_end) {
             request_a_tiles(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
             request_w(b + 1);
         }
@@ -297,7 +305,57 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     if (tok == 0 && lane < 4) *reinterpret_cast<uint32_t*>(tile + kPZeroOff + lane * 4) = 0u;
 }
 
+// y[tok][row] = plane 0 + plane 1 + ... in that order; four rows per thread (rows % 4 == 0)
+__global__ void __launch_bounds__(256) prefill_sum_planes_kernel(const float* __restrict__ part, int splits, int64_t n, int64_t rows,
+                                                                 float* __restrict__ y, int64_t ldy) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (token, group of four rows)
+    const int64_t per_row = rows >> 2;
+    if (i >= n * per_row) return;
+    const int64_t tok = i / per_row, q = i - tok * per_row;
+    const float4* src = reinterpret_cast<const float4*>(part + (size_t)tok * rows) + q;
+    float4 acc = src[0];
+    for (int z = 1; z < splits; ++z) {
+        const float4 v = src[(size_t)z * (size_t)(n * per_row)];
+        acc.x = __fadd_rn(acc.x, v.x), acc.y = __fadd_rn(acc.y, v.y), acc.z = __fadd_rn(acc.z, v.z), acc.w = __fadd_rn(acc.w, v.w);
+    }
+    float* dst = y + tok * ldy + q * 4;
+    dst[0] = acc.x, dst[1] = acc.y, dst[2] = acc.z, dst[3] = acc.w;
+}
+
+// Workgroup shape and K split of a launch: 64-row workgroups while the 128-row ones would not give every compute
+// unit one; K in `splits` runs of super-blocks while the launch would still leave workgroup slots empty (a
+// workgroup walks its super-blocks one after the other, 2.2 us each: 4096 rows x 14336 columns at M = 128 are 64
+// workgroups of 56 super-blocks, 115 us; in eight runs 37 us with the launch that adds the planes; at M = 256
+// 119 -> 56 us in four runs, at M = 512 128 -> 100 us in two; 14336 x 4096 at M = 128: 40 -> 35 us in two).
+struct PrefillShape {
+    bool narrow;
+    int splits, sb_split;
+    unsigned row_wgs, groups;
+};
+PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n) {
+    const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
+    PrefillShape ps;
+    ps.groups = (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup);
+    // two workgroups fit a compute unit: while the 128-row workgroups would not even give every unit one, 64-row
+    // ones fill the chip better (14336 rows on 256 units: up to M = 256; 52 -> 40 us at M = 128, 55 -> 51 at 256,
+    // and 76 -> 79, 78 -> 91 at M = 384, 512, where the wide ones stay)
+    ps.narrow = ((rowtiles + 7) / 8) * (int64_t)ps.groups <= (int64_t)compute_units();
+    ps.row_wgs = (unsigned)(ps.narrow ? (rowtiles + 3) / 4 : (rowtiles + 7) / 8);
+    const int64_t wgs = (int64_t)ps.row_wgs * ps.groups;
+    int splits = (int)(2 * (int64_t)compute_units() / (wgs > 0 ? wgs : 1));
+    if (splits > nb / 4) splits = (int)(nb / 4);  // at least four super-blocks per run
+    if (splits < 1 || (rows & 3)) splits = 1;
+    ps.sb_split = (int)((nb + splits - 1) / splits);
+    ps.splits = (int)((nb + ps.sb_split - 1) / ps.sb_split);  // every run holds a super-block
+    return ps;
+}
+
 }  // namespace
+
+size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n) {
+    const PrefillShape ps = prefill_shape(rows, nb, n);
+    return ps.splits > 1 ? (size_t)ps.splits * (size_t)n * (size_t)rows * sizeof(float) : 0;
+}
 
 size_t pmajor_bytes(int64_t n, int64_t nb) { return (size_t)((n + 15) / 16) * (size_t)nb * kPTileBytes; }
 
@@ -313,21 +371,38 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
 }
 
 hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
-                               int64_t ldy, hipStream_t stream) {
+                               int64_t ldy, float* part, hipStream_t stream) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
     if (rowtiles == 0 || m_tiles == 0) return hipSuccess;
-    const dim3 grid((unsigned)((rowtiles + 4 * kWTilesPerWave - 1) / (4 * kWTilesPerWave)),
-                    (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup));
-    if (grid.y > 65535u) return hipErrorInvalidValue;
+    const PrefillShape ps = prefill_shape(rows, nb, n);
+    if (ps.groups > 65535u) return hipErrorInvalidValue;
+    if (ps.splits > 1 && !part) return hipErrorInvalidValue;
     static bool raised = false;  // two activation buffers: more than the default 64 KB of dynamic LDS
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
-        if (e != hipSuccess) return e;
+        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>)}) {
+            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
+            if (e != hipSuccess) return e;
+        }
         raised = true;
     }
-    hipLaunchKernelGGL(prefill_gemm_kernel, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows,
-                       nb, ap, m_tiles, n, y, ldy);
+    const bool split = ps.splits > 1;
+    float* out = split ? part : y;
+    const int64_t ld = split ? rows : ldy;
+    const int64_t stride = split ? n * rows : 0;
+    const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
+    if (ps.narrow) {
+        hipLaunchKernelGGL(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride);
+    } else {
+        hipLaunchKernelGGL(prefill_gemm_kernel<2>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride);
+    }
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    if (split) {
+        const int64_t units = n * (rows >> 2);
+        hipLaunchKernelGGL(prefill_sum_planes_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, part, ps.splits, n,
+                           rows, y, ldy);
+    }
     return hipGetLastError();
 }
 

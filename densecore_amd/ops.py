@@ -118,7 +118,7 @@ def gemm(w: Q4KWeight, x: torch.Tensor, out: torch.Tensor = None) -> torch.Tenso
     x = _f32(x)
     n = x.shape[0]
     y = out if out is not None else torch.empty((n, w.rows), dtype=torch.float32, device=x.device)
-    _lib.check(_lib.lib().mq_gemm_q4k(w._h, _ptr(x), n, x.stride(0), _ptr(y), w.rows, _stream()), "mq_gemm_q4k")
+    _lib.check(_lib.lib().mq_gemm_q4k(w._h, _ptr(x), n, x.stride(0), _ptr(y), y.stride(0), _stream()), "mq_gemm_q4k")
     return y
 
 

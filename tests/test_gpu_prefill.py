@@ -108,6 +108,71 @@ def test_gemm_agrees_with_decode_kernel_and_dispatch(ops):
     W.free()
 
 
+@pytest.mark.parametrize("rows,cols,n", [(64, 4096, 50), (48, 14336, 130), (272, 2048, 33), (4096, 14336, 48)])
+def test_gemm_with_k_in_runs_matches_oracle_and_decode_kernel(ops, rows, cols, n):
+    """Few weight rows and a long K: the launch splits K into runs of super-blocks whose sums are added in order by
+    a second launch (64 x 4096: four runs; 48 x 14336: fourteen; 272 x 2048: two; 4096 x 14336 at 48 rows: eight).
+    Against the oracle on a sample of weight rows, and against the decode kernel on all of them."""
+    import torch
+    w = synth.q4k_matrix(synth.tensor_seed("pf-split", rows, cols), rows, cols)
+    x = synth.normal_f32(synth.tensor_seed("pf-split-x", n, cols), (n, cols))
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    got = ops.gemm(W, cu(x))
+    small = torch.cat([ops.mul_mat(W, cu(x[i:i + 16])) for i in range(0, n, 16)])
+    scale = small.abs().max().item()
+    assert (got - small).abs().max().item() <= 1e-5 * scale
+    pick = np.unique(np.concatenate([np.arange(0, rows, max(1, rows // 40)), [rows - 1]]))
+    q8 = orc.quantize_rows_q8k(x)
+    ref = orc.mul_mat_q4k_q8k(w[pick], cols, q8, orc.ORDER_SCALAR)
+    assert_fp32_parity(got.cpu().numpy()[:, pick], ref, orc.dot_magnitude_f64(w[pick], cols, q8), "K in runs")
+    # a padded output keeps its padding
+    yp = torch.full((n, rows + 8), 7.0, device="cuda")
+    ops.gemm(W, cu(x), out=yp[:, :rows])
+    assert torch.equal(yp[:, :rows], got) and bool((yp[:, rows:] == 7.0).all())
+    W.free()
+
+
+def test_gemm_integer_sums_are_exact_with_k_in_runs(ops):
+    """The exactness construction of test_gemm_integer_sums_are_exact on a shape whose K is split (32 rows x 4096
+    columns: four runs of four super-blocks): every partial sum is an integer below 2^24, so the planes add exactly."""
+    rows, cols, n = 32, 4096, 20
+    nb = cols // 256
+    w = synth.q4k_matrix(synth.tensor_seed("pf-int-split", rows), rows, cols).reshape(rows, nb, 144).copy()
+    w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[:, :, 2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[:, :, 4:16] &= 0x1F   # scales and mins below 32: the sixteen super-block sums stay below 2^24 in all
+    w = w.reshape(rows, nb * 144)
+    rng = np.random.default_rng(5)
+    x = rng.integers(-127, 128, size=(n, cols)).astype(np.float32)
+    x.reshape(n, nb, 256)[:, :, 7] = rng.choice([-127.0, 127.0], size=(n, nb))
+    q8 = orc.quantize_rows_q8k(x)
+    d, qs, _ = orc.split_q8k(q8)
+    assert np.all(np.abs(d) == 1.0)
+    ds, md = orc.matrix_block_sums(w, cols, q8)
+    want = ((ds.astype(np.int64) - md.astype(np.int64)) * d.astype(np.int64)[None]).sum(axis=2).T
+    assert np.abs(want).max() < 2 ** 24
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    assert np.array_equal(got, want.astype(np.float32))
+    W.free()
+
+
+def test_large_matrices_take_the_gemm_from_seventeen_rows(ops):
+    """24 MB of weights and more: mul_mat hands 17 rows and up to the matrix-core GEMM (smaller matrices from 48)."""
+    import torch
+    W = ops.Q4KWeight.synthetic(4, 14336, 4096)
+    x = torch.randn((20, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(20))
+    big = ops.gemm(W, x)
+    assert torch.equal(ops.mul_mat(W, x), big)
+    small = torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:])])
+    assert (big - small).abs().max().item() <= 1e-5 * small.abs().max().item()
+    W.free()
+    W = ops.Q4KWeight.synthetic(5, 4096, 4096)
+    x = torch.randn((20, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(21))
+    assert torch.equal(ops.mul_mat(W, x), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:])]))
+    W.free()
+
+
 @pytest.mark.parametrize("m", [512, 2048])
 def test_gemm_full_size_rows_against_decode_kernel(ops, m):
     """W 4096 -> 14336 at M = 512 / 2048: every 37th activation row is recomputed by the decode kernel,
