@@ -133,7 +133,8 @@ struct State {
     int device = -1;
     std::recursive_mutex mu;  // recursive: the host-pointer entry points call the device-pointer ones while holding it
     Buffer aq, ad;        // A-major activations of the op input
-    Buffer ap;            // P-major activations of the prefill GEMM
+    Buffer ap, ap2;       // P-major activations of the prefill GEMM (input; FFN intermediate)
+    Buffer mid2;          // gate and up products of a wide FFN, fp32
     Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
     Buffer aq2, ad2;      // A-major activations of the intermediate
     Buffer part;          // MoE per-(token,k) down results
@@ -368,7 +369,7 @@ int mq_shutdown(void) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
-    for (Buffer* b : {&g.aq, &g.ad, &g.mid, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    for (Buffer* b : {&g.aq, &g.ad, &g.ap, &g.ap2, &g.mid, &g.mid2, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
     g.pin_in.release();
     g.pin_out.release();
     if (g.order_event) (void)hipEventDestroy(g.order_event);
@@ -550,6 +551,35 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
     if (part_bytes) MQ_HIP(g.part.reserve(part_bytes));
     MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy,
                                part_bytes ? (float*)g.part.ptr : nullptr, s));
+    return MQ_OK;
+}
+
+// Wide FFN on the matrix-core GEMM: gate and up products into the two halves of g.mid2, their SwiGLU formed by the
+// quantizer of the down product (and written to h_dev / g.mid as fp32 as well), then the down product if asked for.
+static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev, int64_t n,
+                           int64_t ldx, int silu_mode, float* h_dev, int64_t ldh, float* y_dev, hipStream_t s) {
+    const int64_t inter = gate->rows;
+    MQ_HIP(g.mid2.reserve(2 * (size_t)n * (size_t)inter * sizeof(float)));
+    float* gbuf = (float*)g.mid2.ptr;
+    float* ubuf = gbuf + (size_t)n * (size_t)inter;
+    MQ_HIP(g.ap.reserve(pmajor_bytes(n, gate->nb)));
+    MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, gate->cols, (uint8_t*)g.ap.ptr, s));
+    const size_t part_bytes = prefill_part_bytes(inter, gate->nb, n);
+    if (part_bytes) MQ_HIP(g.part.reserve(part_bytes));
+    float* part = part_bytes ? (float*)g.part.ptr : nullptr;
+    MQ_HIP(launch_prefill_gemm(gate->data, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, gbuf, inter, part, s));
+    MQ_HIP(launch_prefill_gemm(up->data, inter, up->nb, (const uint8_t*)g.ap.ptr, n, ubuf, inter, part, s));
+    if (!down) {  // SwiGLU rows only: the quantizer's fp32 side output is the result
+        MQ_HIP(g.ap2.reserve(pmajor_bytes(n, inter / kQK)));
+        MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
+        return MQ_OK;
+    }
+    MQ_HIP(g.ap2.reserve(pmajor_bytes(n, down->nb)));
+    MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
+    const size_t part2 = prefill_part_bytes(down->rows, down->nb, n);
+    if (part2) MQ_HIP(g.part.reserve(part2));
+    MQ_HIP(launch_prefill_gemm(down->data, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, down->rows,
+                               part2 ? (float*)g.part.ptr : nullptr, s));
     return MQ_OK;
 }
 
@@ -790,6 +820,10 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
+    if (prefill_applies(gate, n) && prefill_applies(down, n) && !census.on) {  // wide: the matrix-core GEMM, three times
+        MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
+        return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, s);
+    }
     // One row: both quantizers run inside the products (two launches instead of four, the same bits).
     const bool one_row = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
     const bool inline_quant = one_row || dense_lds_quantizes(gate, x_dev, n, hidden, true);
@@ -1221,6 +1255,8 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
+    if (prefill_applies(gate, n) && !census.on && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
+        return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, s);
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
     if (!inline_quant)

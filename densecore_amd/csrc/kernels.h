@@ -162,6 +162,9 @@ hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
 size_t pmajor_bytes(int64_t n, int64_t nb);
 hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
                                       hipStream_t stream);
+// The same for the rows silu(gate) * up (both [n][ldx]); h_out (may be null) receives them as fp32 [n][ldh] as well.
+hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up, int64_t n, int64_t ldx, int64_t k,
+                                             int silu_mode, float* h_out, int64_t ldh, uint8_t* ap, hipStream_t stream);
 // y[n][ldy] = P-major activations . tiled weights^T on the int8 matrix cores.  A launch that would leave workgroup
 // slots empty splits K into runs of super-blocks whose sums go to planes of `part` (prefill_part_bytes() bytes, 0 when
 // nothing is split) and are added in order by a second launch.

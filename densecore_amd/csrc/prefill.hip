@@ -274,8 +274,12 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 }
 
 // One wavefront per (activation row, super-block); rows in [n, 16*m_tiles) are written as zeros.
-__global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* __restrict__ x, int64_t n, int64_t ldx,
-                                                                  int64_t nb, int64_t m_tiles,
+// kSwiglu: the row is silu(x) * x2 of two inputs (the gate and up products of an FFN), formed here instead of in a
+// pass of its own; h_out, if given, receives it as fp32 as well.
+template <bool kSwiglu>
+__global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* __restrict__ x, const float* __restrict__ x2,
+                                                                  int silu_mode, float* __restrict__ h_out, int64_t ldh,
+                                                                  int64_t n, int64_t ldx, int64_t nb, int64_t m_tiles,
                                                                   uint8_t* __restrict__ ap) {
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -286,6 +290,12 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     if (m < n) {
         const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
         e[0] = v.x, e[1] = v.y, e[2] = v.z, e[3] = v.w;
+        if (kSwiglu) {
+            const float4 u = *reinterpret_cast<const float4*>(x2 + m * ldx + b * kQK + lane * 4);
+            e[0] = silu_mul(e[0], u.x, silu_mode), e[1] = silu_mul(e[1], u.y, silu_mode);
+            e[2] = silu_mul(e[2], u.z, silu_mode), e[3] = silu_mul(e[3], u.w, silu_mode);
+            if (h_out) *reinterpret_cast<float4*>(h_out + m * ldh + b * kQK + lane * 4) = float4{e[0], e[1], e[2], e[3]};
+        }
     }
     const Q8Lane q = quantize_block_q8k(e, lane);
     uint8_t* tile = ap + ((size_t)b * (size_t)m_tiles + (size_t)(m >> 4)) * kPTileBytes;
@@ -365,8 +375,19 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     const int64_t units = m_tiles * 16 * nb;
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
-    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx,
-                       nb, m_tiles, ap);
+    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x,
+                       (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap);
+    return hipGetLastError();
+}
+
+hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up, int64_t n, int64_t ldx, int64_t k,
+                                             int silu_mode, float* h_out, int64_t ldh, uint8_t* ap, hipStream_t stream) {
+    const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
+    const int64_t units = m_tiles * 16 * nb;
+    if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, gate, up,
+                       silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap);
     return hipGetLastError();
 }
 

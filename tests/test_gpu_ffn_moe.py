@@ -69,6 +69,29 @@ def test_swiglu_and_ffn_stagewise(ops, n, silu):
         w.free()
 
 
+@pytest.mark.parametrize("n", [48, 100])
+def test_wide_ffn_runs_on_the_gemm_and_matches_its_stages(ops, n):
+    """48 rows and more: gate, up and down products on the matrix-core GEMM, SwiGLU formed by the down product's
+    quantizer.  The SwiGLU rows against the oracle; the FFN output bit for bit the GEMM of the GPU's own SwiGLU rows,
+    against the oracle's down product of those rows, and end to end."""
+    H, I, silu = 1024, 1792, 2
+    g, u, d = (synth.q4k_matrix(synth.tensor_seed("ffn", nm), r, c) for nm, r, c in
+               (("g", I, H), ("u", I, H), ("d", H, I)))
+    x = synth.normal_f32(synth.tensor_seed("ffn-x", n), (n, H))
+    G, U, D = ops.Q4KWeight.from_ggml(g, H), ops.Q4KWeight.from_ggml(u, H), ops.Q4KWeight.from_ggml(d, I)
+    h_gpu = ops.swiglu_mul_mat(G, U, cu(x), silu).cpu().numpy()
+    assert_close_prod(h_gpu, orc.swiglu_mul_mat(g, u, H, I, x, orc.ORDER_DOTPROD, silu), "wide swiglu")
+    y = ops.ffn_swiglu(G, U, D, cu(x), silu)
+    assert np.array_equal(ops.debug_moe_hidden((n, I)).cpu().numpy().view(np.uint32), h_gpu.view(np.uint32))
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), ops.gemm(D, cu(h_gpu)).cpu().numpy().view(np.uint32))
+    y_gpu = y.cpu().numpy()
+    assert_fp32_parity(y_gpu, orc.mul_mat_q4k_f32(d, I, h_gpu, orc.ORDER_DOTPROD), down_mag(d, I, h_gpu), "wide ffn-down")
+    y_ref = orc.ffn_swiglu(g, u, d, H, I, x, orc.ORDER_DOTPROD, silu)
+    assert np.max(np.abs(y_gpu - y_ref)) <= END_TO_END_REL * np.max(np.abs(y_ref))
+    for w in (G, U, D):
+        w.free()
+
+
 def test_ffn_full_size_single_token(ops):
     """The dense FFN shape of the benchmark (4096 -> 14336 -> 4096) at one token."""
     H, I = 4096, 14336
