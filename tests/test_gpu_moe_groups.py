@@ -25,17 +25,20 @@ def cu(a):
 
 
 @pytest.mark.parametrize("n,e,k", [(1, 256, 8), (2, 256, 8), (4, 256, 8), (9, 256, 8), (16, 256, 8), (64, 256, 8),
-                                   (257, 256, 8), (300, 64, 4), (7, 60, 4), (40, 12, 4), (3, 8, 8), (1100, 128, 8)])
+                                   (257, 256, 8), (300, 64, 4), (7, 60, 4), (40, 12, 4), (3, 8, 8), (1100, 128, 8),
+                                   (512, 256, 8), (1024, 256, 8), (2048, 256, 8), (4096, 256, 8), (4100, 64, 8),
+                                   (3000, 512, 8)])
 def test_group_lists_from_ids_equal_sorted_assignments(ops, n, e, k):
-    """launch_build_groups: the grouping of mq_mul_mat_id_q4k and of the two expert nodes (token masks up to 256
-    tokens, the scan above; ids in LDS up to 8192 pairs, in global memory above)."""
+    """launch_build_groups: the grouping of mq_mul_mat_id_q4k and of the two expert nodes (token masks while they fit
+    the LDS of a compute unit -- 4096 tokens at 256 experts --, the scan of earlier pairs beyond; ids in LDS up to 8192
+    pairs, in global memory above)."""
     ids, _ = orc.route_topk(synth.normal_f32(synth.tensor_seed("grp", n, e, k), (n, e)), k, 0)
     got = ops.debug_moe_groups(e, k, ids=cu(ids))
     assert np.array_equal(got, orc.build_assignments(ids, e))
     assert len(got) == n * k
 
 
-@pytest.mark.parametrize("n,e,k", [(5, 16, 4), (33, 256, 8), (70, 12, 6), (300, 40, 8)])
+@pytest.mark.parametrize("n,e,k", [(5, 16, 4), (33, 256, 8), (70, 12, 6), (300, 40, 8), (1500, 256, 8)])
 def test_group_lists_with_invalid_and_repeated_ids(ops, n, e, k):
     rng = np.random.default_rng(n * 1000 + e)
     ids = rng.integers(0, e, size=(n, k)).astype(np.int32)       # repeats inside a token are likely
@@ -51,7 +54,7 @@ def test_group_lists_with_invalid_and_repeated_ids(ops, n, e, k):
 
 
 @pytest.mark.parametrize("n,e,k", [(1, 256, 8), (2, 256, 8), (3, 256, 8), (12, 256, 8), (16, 256, 8), (64, 256, 8),
-                                   (200, 256, 8), (17, 60, 4), (31, 1000, 6)])
+                                   (200, 256, 8), (17, 60, 4), (31, 1000, 6), (512, 256, 8), (1024, 256, 8), (2048, 256, 8)])
 def test_route_and_group_in_one_launch(ops, n, e, k):
     """launch_route_and_group: the first launch of mq_moe_layer_q4k above eight tokens (one workgroup up to two
     tokens, a last-arriver handshake above); ties in the logits keep the lower expert first."""
