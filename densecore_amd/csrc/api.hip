@@ -135,6 +135,8 @@ struct State {
     Buffer aq, ad;        // A-major activations of the op input
     Buffer ap, ap2;       // P-major activations of the prefill GEMM (input; FFN intermediate)
     Buffer mid2;          // gate and up products of a wide FFN, fp32
+    Buffer kpart;         // planes of partial sums of a prefill GEMM whose K is split
+    Buffer plan;          // tile plan of the expert-grouped GEMM
     Buffer mid;           // fp32 intermediate (FFN hidden, MoE per-(token,k) hidden)
     Buffer aq2, ad2;      // A-major activations of the intermediate
     Buffer part;          // MoE per-(token,k) down results
@@ -369,7 +371,7 @@ int mq_shutdown(void) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
-    for (Buffer* b : {&g.aq, &g.ad, &g.ap, &g.ap2, &g.mid, &g.mid2, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    for (Buffer* b : {&g.aq, &g.ad, &g.ap, &g.ap2, &g.mid, &g.mid2, &g.kpart, &g.plan, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
     g.pin_in.release();
     g.pin_out.release();
     if (g.order_event) (void)hipEventDestroy(g.order_event);
@@ -548,16 +550,16 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, w->nb)));
     MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, w->cols, (uint8_t*)g.ap.ptr, s));
     const size_t part_bytes = prefill_part_bytes(w->rows, w->nb, n);
-    if (part_bytes) MQ_HIP(g.part.reserve(part_bytes));
+    if (part_bytes) MQ_HIP(g.kpart.reserve(part_bytes));
     MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy,
-                               part_bytes ? (float*)g.part.ptr : nullptr, s));
+                               part_bytes ? (float*)g.kpart.ptr : nullptr, s));
     return MQ_OK;
 }
 
 // Wide FFN on the matrix-core GEMM: gate and up products into the two halves of g.mid2, their SwiGLU formed by the
 // quantizer of the down product (and written to h_dev / g.mid as fp32 as well), then the down product if asked for.
 static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev, int64_t n,
-                           int64_t ldx, int silu_mode, float* h_dev, int64_t ldh, float* y_dev, hipStream_t s) {
+                           int64_t ldx, int silu_mode, float* h_dev, int64_t ldh, float* y_dev, int64_t ldy, hipStream_t s) {
     const int64_t inter = gate->rows;
     MQ_HIP(g.mid2.reserve(2 * (size_t)n * (size_t)inter * sizeof(float)));
     float* gbuf = (float*)g.mid2.ptr;
@@ -565,8 +567,8 @@ static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, gate->nb)));
     MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, gate->cols, (uint8_t*)g.ap.ptr, s));
     const size_t part_bytes = prefill_part_bytes(inter, gate->nb, n);
-    if (part_bytes) MQ_HIP(g.part.reserve(part_bytes));
-    float* part = part_bytes ? (float*)g.part.ptr : nullptr;
+    if (part_bytes) MQ_HIP(g.kpart.reserve(part_bytes));
+    float* part = part_bytes ? (float*)g.kpart.ptr : nullptr;
     MQ_HIP(launch_prefill_gemm(gate->data, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, gbuf, inter, part, s));
     MQ_HIP(launch_prefill_gemm(up->data, inter, up->nb, (const uint8_t*)g.ap.ptr, n, ubuf, inter, part, s));
     if (!down) {  // SwiGLU rows only: the quantizer's fp32 side output is the result
@@ -577,9 +579,9 @@ static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_
     MQ_HIP(g.ap2.reserve(pmajor_bytes(n, down->nb)));
     MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
     const size_t part2 = prefill_part_bytes(down->rows, down->nb, n);
-    if (part2) MQ_HIP(g.part.reserve(part2));
-    MQ_HIP(launch_prefill_gemm(down->data, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, down->rows,
-                               part2 ? (float*)g.part.ptr : nullptr, s));
+    if (part2) MQ_HIP(g.kpart.reserve(part2));
+    MQ_HIP(launch_prefill_gemm(down->data, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, ldy,
+                               part2 ? (float*)g.kpart.ptr : nullptr, s));
     return MQ_OK;
 }
 
@@ -822,7 +824,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (entry.rc) return entry.rc;
     if (prefill_applies(gate, n) && prefill_applies(down, n) && !census.on) {  // wide: the matrix-core GEMM, three times
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
-        return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, s);
+        return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, hidden, s);
     }
     // One row: both quantizers run inside the products (two launches instead of four, the same bits).
     const bool one_row = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
@@ -1256,7 +1258,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     Entry entry(s);
     if (entry.rc) return entry.rc;
     if (prefill_applies(gate, n) && !census.on && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
-        return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, s);
+        return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, 0, s);
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
     if (!inline_quant)
@@ -1425,6 +1427,17 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
 
 }  // namespace
 
+// The expert-grouped GEMM pays from a dozen routed rows per expert on average (its workgroups multiply 16-row tiles, up to
+// eight of an expert at a time): 256 experts, top-8, 2048 x 512: 242 against 250 us per block at 384 tokens, 262 against
+// 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.  Q4_K stacks.
+static bool moe_gemm_applies(const mq_moe_layer_desc* L, const SharedExpert& sh, int64_t n) {
+    const mq_weight* ge = L->gate_exps;
+    if (ge->type != kTypeQ4K || L->up_exps->type != kTypeQ4K || L->down_exps->type != kTypeQ4K) return false;
+    if (sh.gate && (sh.gate->type != kTypeQ4K || sh.down->type != kTypeQ4K)) return false;
+    if (ge->n_experts > 4096 || (ge->rows & 3) || (ge->cols & 3)) return false;
+    return n >= 256 && n * L->top_k >= 12 * ge->n_experts;
+}
+
 int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float* logits_dev, int64_t n, float* y_dev,
                      int32_t* ids_out_dev, float* weights_out_dev, void* stream) {
     if (int rc = check_ready()) return rc;
@@ -1485,6 +1498,40 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     }
     // one arrival counter, kept apart from the quantization counters (last slot of that buffer)
     if (int rc = reserve_counters(4096)) return rc;
+    if (moe_gemm_applies(L, sh, n) && !census.on) {
+        // Prefill widths: the three expert products on the matrix-core GEMM in its expert-grouped form, the shared
+        // expert as a dense FFN on it; per-(token, slot) rows and the combine as at the other widths.
+        const int64_t entries = n * K;
+        MQ_HIP(g.part.reserve((size_t)n * slots * (size_t)hidden * sizeof(float)));
+        float* part = (float*)g.part.ptr;
+        if (sh.gate)  // first: it uses the same staging buffers
+            if (int rc = ffn_wide_locked(sh.gate, sh.up, sh.down, x_dev, n, hidden, MQ_SILU_FAST_FMA, nullptr, 0, part + (size_t)K * hidden,
+                                         (int64_t)slots * hidden, s))
+                return rc;
+        MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
+                                      r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, true, nullptr, 0, 0,
+                                      nullptr, nullptr, s));
+        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int32_t* plan = (const int32_t*)g.plan.ptr;
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, entries, E,
+                                    (int32_t*)g.plan.ptr, s));
+        const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
+        MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, s));
+        MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
+        float* gbuf = (float*)g.mid2.ptr;
+        float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
+        MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->expert_bytes, inter, L->gate_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s));
+        MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->expert_bytes, inter, L->up_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
+        MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr, s));
+        MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->expert_bytes, hidden, L->down_exps->nb,
+                                           (const uint8_t*)g.ap2.ptr, entries, E, plan, true, part, hidden, s));
+        MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
+        return MQ_OK;
+    }
     // the same launch quantizes x: extra workgroups next to the routing ones
     MQ_HIP(g.aq.reserve(aq_bytes(n, hidden / kQK)));
     MQ_HIP(g.ad.reserve(ad_count(n, hidden / kQK) * sizeof(float)));

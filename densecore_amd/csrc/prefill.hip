@@ -148,15 +148,25 @@ template <int kWTilesPerWave>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
-                                                           int64_t split_stride) {
+                                                           int64_t split_stride, const int32_t* __restrict__ plan,
+                                                           int64_t expert_bytes, const int32_t* __restrict__ out_rows) {
     extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kq = lane >> 4;
-    const int64_t mt0 = (int64_t)blockIdx.y * kMTilesPerGroup;
-    const int mt_count = (int)(m_tiles - mt0 < kMTilesPerGroup ? m_tiles - mt0 : kMTilesPerGroup);
+    // Dense: workgroup column blockIdx.y takes the activation tiles 8 y .. 8 y + 7.  Expert-grouped (plan != null): it
+    // takes item blockIdx.y of the plan -- an expert's weights and a run of up to eight tiles of that expert's rows.
+    int64_t mt0 = (int64_t)blockIdx.y * kMTilesPerGroup;
+    int mt_count = (int)(m_tiles - mt0 < kMTilesPerGroup ? m_tiles - mt0 : kMTilesPerGroup);
+    if (plan) {
+        const int item = blockIdx.y;
+        if (item >= plan[0]) return;  // the whole workgroup, before any barrier
+        w += (size_t)plan[4 + 3 * item] * (size_t)expert_bytes;
+        mt0 = plan[5 + 3 * item];
+        mt_count = plan[6 + 3 * item];
+    }
     const int64_t rt0 = ((int64_t)blockIdx.x * 4 + wave) * kWTilesPerWave;
     // weight tiles past the end are replaced by the last valid one and simply not stored
     int64_t rt[kWTilesPerWave];
@@ -253,6 +263,23 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         }
     }
 
+    if (out_rows) {  // grouped down product: row 16 (mt0 + m) + 4 kq + i of the plan goes to row out_rows[..] of y (-1: padding)
+#pragma unroll
+        for (int t = 0; t < kWTilesPerWave; ++t) {
+            const int64_t row = (rt0 + t) * kTileRows + r;
+            if (rt0 + t >= rowtiles || row >= rows) continue;
+#pragma unroll
+            for (int m = 0; m < kMTilesPerGroup; ++m) {
+                if (m >= mt_count) continue;
+                const int4 dst = *reinterpret_cast<const int4*>(out_rows + (mt0 + m) * 16 + kq * 4);
+                const int dsts[4] = {dst.x, dst.y, dst.z, dst.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (dsts[i] >= 0) y[(size_t)dsts[i] * (size_t)ldy + row] = acc[t][m][i];
+            }
+        }
+        return;
+    }
     // Stores: lane (r, kq) holds weight row r of its tiles for the tokens 16 m + 4 kq + i.  One pointer per lane walks
     // down the token rows (an addition per store, no product).
     const int tok_left = (int)(n_tokens - mt0 * 16) - kq * 4;  // tokens from this lane's first one to the end
@@ -280,21 +307,25 @@ template <bool kSwiglu>
 __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* __restrict__ x, const float* __restrict__ x2,
                                                                   int silu_mode, float* __restrict__ h_out, int64_t ldh,
                                                                   int64_t n, int64_t ldx, int64_t nb, int64_t m_tiles,
-                                                                  uint8_t* __restrict__ ap) {
+                                                                  uint8_t* __restrict__ ap, const int32_t* __restrict__ plan,
+                                                                  const int32_t* __restrict__ row_src) {
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= m_tiles * 16 * nb) return;
     int64_t m, b;
     split_unit(unit, nb, m, b);
+    if (plan && m >= (int64_t)plan[1] * 16) return;  // expert-grouped rows: past the tiles the plan holds
+    // row_src (expert-grouped gather): row m of the tiles is row row_src[m] of x, or padding (-1: zeros)
+    const int64_t src = row_src ? row_src[m] : (m < n ? m : -1);
     float e[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (m < n) {
-        const float4 v = *reinterpret_cast<const float4*>(x + m * ldx + b * kQK + lane * 4);
+    if (src >= 0) {
+        const float4 v = *reinterpret_cast<const float4*>(x + src * ldx + b * kQK + lane * 4);
         e[0] = v.x, e[1] = v.y, e[2] = v.z, e[3] = v.w;
         if (kSwiglu) {
-            const float4 u = *reinterpret_cast<const float4*>(x2 + m * ldx + b * kQK + lane * 4);
+            const float4 u = *reinterpret_cast<const float4*>(x2 + src * ldx + b * kQK + lane * 4);
             e[0] = silu_mul(e[0], u.x, silu_mode), e[1] = silu_mul(e[1], u.y, silu_mode);
             e[2] = silu_mul(e[2], u.z, silu_mode), e[3] = silu_mul(e[3], u.w, silu_mode);
-            if (h_out) *reinterpret_cast<float4*>(h_out + m * ldh + b * kQK + lane * 4) = float4{e[0], e[1], e[2], e[3]};
+            if (h_out) *reinterpret_cast<float4*>(h_out + src * ldh + b * kQK + lane * 4) = float4{e[0], e[1], e[2], e[3]};
         }
     }
     const Q8Lane q = quantize_block_q8k(e, lane);
@@ -360,7 +391,133 @@ PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n) {
     return ps;
 }
 
+// ---- expert-grouped GEMM: the plan ------------------------------------------------------------------------
+// One workgroup.  From the expert groups of the routing (entries sorted by expert: group g holds the entries
+// group_begin[g] .. group_begin[g + 1] - 1 of expert group_expert[g]) it lays the entries out in tiles of 16 rows, every
+// group starting a new tile, and cuts every group's tiles into items of up to eight tiles, the unit a GEMM workgroup
+// column multiplies.  plan: [0] items, [1] tiles, [4 + 3 i ..] = (expert, first tile, tiles) of item i; row_src[r] /
+// out_row[r] for row r of the tiles: the token whose activations it holds and the row of the per-(token, slot) output
+// it produces (token * slots + k), -1 for padding.
+__global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __restrict__ n_groups, const int32_t* __restrict__ group_expert,
+                                                             const int32_t* __restrict__ group_begin,
+                                                             const int32_t* __restrict__ entry_token,
+                                                             const int32_t* __restrict__ entry_k, int slots, int groups_max,
+                                                             int32_t* __restrict__ plan, int32_t* __restrict__ row_src,
+                                                             int32_t* __restrict__ out_row) {
+    extern __shared__ int32_t plan_sh[];  // begin[g] (groups_max + 1), tile0[g] (groups_max + 1), item0[g] (groups_max + 1)
+    int32_t* begin = plan_sh;
+    int32_t* tile0 = begin + groups_max + 1;
+    int32_t* item0 = tile0 + groups_max + 1;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int ng = *n_groups < groups_max ? *n_groups : groups_max;
+    for (int g = tid; g <= ng; g += nt) begin[g] = group_begin[g];
+    __syncthreads();
+    if (tid == 0) {
+        int tiles = 0, items = 0;
+        for (int g = 0; g < ng; ++g) {
+            const int t = (begin[g + 1] - begin[g] + 15) >> 4;
+            tile0[g] = tiles, item0[g] = items;
+            tiles += t, items += (t + kMTilesPerGroup - 1) / kMTilesPerGroup;
+        }
+        tile0[ng] = tiles, item0[ng] = items;
+        plan[0] = items, plan[1] = tiles, plan[2] = 0, plan[3] = 0;
+    }
+    __syncthreads();
+    // the group of position q in a non-decreasing prefix array: the last g with first[g] <= q (empty groups cannot occur)
+    auto group_of = [&](const int32_t* first, int q) {
+        int lo = 0, hi = ng - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (first[mid] <= q) lo = mid;
+            else hi = mid - 1;
+        }
+        return lo;
+    };
+    const int tiles = tile0[ng], items = item0[ng];
+    for (int i = tid; i < items; i += nt) {
+        const int g = group_of(item0, i);
+        const int t_g = tile0[g + 1] - tile0[g], first = (i - item0[g]) * kMTilesPerGroup;
+        plan[4 + 3 * i] = group_expert[g];
+        plan[5 + 3 * i] = tile0[g] + first;
+        plan[6 + 3 * i] = t_g - first < kMTilesPerGroup ? t_g - first : kMTilesPerGroup;
+    }
+    for (int rr = tid; rr < tiles * 16; rr += nt) {
+        const int g = group_of(tile0, rr >> 4);
+        const int pos = rr - tile0[g] * 16;
+        int src = -1, dst = -1;
+        if (pos < begin[g + 1] - begin[g]) {
+            const int e = begin[g] + pos;
+            src = entry_token[e];
+            dst = src * slots + entry_k[e];
+        }
+        row_src[rr] = src, out_row[rr] = dst;
+    }
+}
+
 }  // namespace
+
+int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max) { return (entries + 15) / 16 + groups_max; }
+int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max) {  // a multiple of four: the row arrays behind the items stay 16-byte aligned
+    return ((entries + 16 * kMTilesPerGroup - 1) / (16 * kMTilesPerGroup) + groups_max + 3) & ~(int64_t)3;
+}
+size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max) {
+    return 4 + 3 * (size_t)moe_gemm_items_max(entries, groups_max) + 2 * 16 * (size_t)moe_gemm_tiles_max(entries, groups_max);
+}
+
+hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
+                                const int32_t* entry_token, const int32_t* entry_k, int slots, int64_t entries, int64_t groups_max,
+                                int32_t* plan, hipStream_t stream) {
+    if (groups_max > 4096) return hipErrorInvalidValue;
+    int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
+    int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
+    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(1), dim3(1024), 3 * (size_t)(groups_max + 1) * sizeof(int32_t), stream, n_groups,
+                       group_expert, group_begin, entry_token, entry_k, slots, (int)groups_max, plan, row_src, out_row);
+    return hipGetLastError();
+}
+
+// Rows of the plan's tiles in the P-major layout: gathered from x by token (swiglu == false), or silu(gate) * up of two
+// planes that already are in the plan's row order (swiglu == true).
+hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
+                                              int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap,
+                                              hipStream_t stream) {
+    const int64_t nb = k / kQK, m_tiles = moe_gemm_tiles_max(entries, groups_max);
+    const int64_t units = m_tiles * 16 * nb;
+    if (units == 0) return hipSuccess;
+    if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;
+    const int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
+    if (swiglu) {
+        hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, x2, silu_mode,
+                           (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr);
+    } else {
+        hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x,
+                           (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, row_src);
+    }
+    return hipGetLastError();
+}
+
+// y = the plan's tiles . W_expert^T per item.  scatter == false: y [tiles * 16][ldy] in the plan's row order;
+// true: row out_row[r] of y (the per-(token, slot) rows of the down product).
+hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, int64_t rows, int64_t nb, const uint8_t* ap,
+                                       int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter, float* y, int64_t ldy,
+                                       hipStream_t stream) {
+    const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
+    const int64_t items = moe_gemm_items_max(entries, groups_max);
+    if (rowtiles == 0 || items == 0) return hipSuccess;
+    if (items > 65535) return hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised) {
+        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>)}) {
+            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
+            if (e != hipSuccess) return e;
+        }
+        raised = true;
+    }
+    const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
+    hipLaunchKernelGGL(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
+                       2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
+                       (int64_t)0, plan, expert_bytes, out_row);
+    return hipGetLastError();
+}
 
 size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n) {
     const PrefillShape ps = prefill_shape(rows, nb, n);
@@ -376,7 +533,8 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x,
-                       (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap);
+                       (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr,
+                       (const int32_t*)nullptr);
     return hipGetLastError();
 }
 
@@ -387,7 +545,7 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;
     hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, gate, up,
-                       silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap);
+                       silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr, (const int32_t*)nullptr);
     return hipGetLastError();
 }
 
@@ -413,10 +571,10 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
     const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
     if (ps.narrow) {
         hipLaunchKernelGGL(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
-                           ap, m_tiles, n, out, ld, ps.sb_split, stride);
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr);
     } else {
         hipLaunchKernelGGL(prefill_gemm_kernel<2>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
-                           ap, m_tiles, n, out, ld, ps.sb_split, stride);
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr);
     }
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (split) {

@@ -225,7 +225,11 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  * shared_* may all be NULL (no shared expert); sh_gate_inp_dev fp32 [hidden] or NULL (gate = 1).
  * Up to eight tokens (and 512 experts) two launches: gate/up + SwiGLU with the router and the Q8_K of x inside,
  * down with the Q8_K of the hidden rows and the weighted combine inside.  Above: router + expert grouping + Q8_K
- * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way. */
+ * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way.
+ * Prefill widths (Q4_K stacks, 256 tokens and more with a dozen routed rows per expert on average): the expert
+ * products run on the int8 matrix-core GEMM in an expert-grouped form (entries in 16-row tiles per expert), the
+ * shared expert as a dense FFN on it; same routing, results within the fp32 tolerance of the other form (the
+ * summation order differs), and mq_debug_moe_hidden does not apply. */
 typedef struct {
     const mq_weight* gate_exps; /* n_experts x [inter][hidden]  */
     const mq_weight* up_exps;

@@ -274,6 +274,39 @@ def test_moe_layer_stagewise(ops, n, silu):
         w.free()
 
 
+@pytest.mark.parametrize("n,E,K,shared", [(300, 16, 4, True), (256, 8, 2, False), (1000, 12, 6, True)])
+def test_moe_layer_at_prefill_widths_runs_on_the_grouped_gemm(ops, n, E, K, shared):
+    """256 tokens and more with two dozen routed rows per expert: the expert products run on the matrix-core GEMM in its
+    expert-grouped form (entries laid out in 16-row tiles per expert, up to eight tiles per workgroup column: groups
+    of 75, 64 and 500 rows here -- padding rows, full tiles and several columns per expert).  End to end against the
+    oracle's layer, routing bit for bit, and against the stage-wise entries of the decode kernels on the same ids."""
+    H, I, silu = 512, 256, 1
+    ge, ue, de = make_experts("moe-pf", E, H, I)
+    sg, su, sd = (synth.q4k_matrix(synth.tensor_seed("moe-pf-sh", nm), r, c) for nm, r, c in
+                  (("g", I, H), ("u", I, H), ("d", H, I)))
+    gate_inp = synth.normal_f32(synth.tensor_seed("moe-pf-gi"), (H,)) * np.float32(0.02)
+    x = synth.normal_f32(synth.tensor_seed("moe-pf-x", n), (n, H))
+    logits = synth.normal_f32(synth.tensor_seed("moe-pf-l", n, E), (n, E))
+    logits[:, 0] += np.float32(1.5)          # a crowded expert: several workgroup columns
+    GE, UE, DE = ops.Q4KWeight.from_ggml(ge, H), ops.Q4KWeight.from_ggml(ue, H), ops.Q4KWeight.from_ggml(de, I)
+    SG, SU, SD = ops.Q4KWeight.from_ggml(sg, H), ops.Q4KWeight.from_ggml(su, H), ops.Q4KWeight.from_ggml(sd, I)
+    sh_gpu = (SG, SU, SD, cu(gate_inp)) if shared else None
+    sh_cpu = (sg, su, sd, gate_inp) if shared else None
+    y, ids, w = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=sh_gpu, silu=silu)
+    oi, ow = orc.route_topk(logits, K, 0)
+    assert np.array_equal(ids.cpu().numpy(), oi) and np.allclose(w.cpu().numpy(), ow, rtol=3e-6)
+    ref = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=sh_cpu, silu=silu)
+    y = y.cpu().numpy()
+    assert np.max(np.abs(y - ref["y"])) <= END_TO_END_REL * np.max(np.abs(ref["y"]))
+    # the routed part against the decode kernels' stages (same ids and weights; other summation order)
+    y_nosh, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=silu)
+    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids, silu)
+    y_stage = ops.moe_down_weighted(DE, hid, ids, w).cpu().numpy()
+    assert np.max(np.abs(y_nosh.cpu().numpy() - y_stage)) <= END_TO_END_REL * np.max(np.abs(y_stage))
+    for t in (GE, UE, DE, SG, SU, SD):
+        t.free()
+
+
 def test_moe_layer_zero_weight_and_duplicate_free_paths(ops):
     """One token whose logits make a single expert take all the weight: the others' weights underflow
     to exactly zero in fp32 and are skipped (core/src/llm/moe/native.cpp:3237)."""

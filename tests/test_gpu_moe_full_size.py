@@ -80,3 +80,30 @@ def test_cfg3_layer_stagewise(layer, n, silu):
     y = y.cpu().numpy()
     rel = np.max(np.abs(y - ref["y"]), axis=1) / np.max(np.abs(ref["y"]), axis=1)
     assert np.max(rel) <= END_TO_END_REL and np.median(rel) <= 2e-5, (np.max(rel), np.median(rel))
+
+
+@pytest.mark.parametrize("n", [400, 1024])
+def test_cfg3_layer_at_prefill_widths_on_the_grouped_gemm(layer, n):
+    """The full-size block (256 + 1 experts, 2048 x 512, top-8) at widths where the expert products run on the
+    matrix-core GEMM in its expert-grouped form: routing bit for bit; the routed part against the decode kernels' own
+    stages on the same ids (other summation order, see below); a sample of tokens end to end against
+    the CPU layer, which depends on those tokens' own rows only."""
+    import torch
+    ops, (GE, UE, DE), (SG, SU, SD), (ge, ue, de), (sg, su, sd), gate_inp = layer
+    x = synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))
+    logits = synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))
+    oi, ow = orc.route_topk(logits, K, 0)
+    y_nosh, ids, w = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=1)
+    assert np.array_equal(ids.cpu().numpy(), oi) and np.allclose(w.cpu().numpy(), ow, rtol=3e-6)
+    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids, 1)
+    y_stage = ops.moe_down_weighted(DE, hid, ids, w)
+    # the hidden rows are re-quantized to Q8_K for the down product: a last-bit difference between the two paths'
+    # SwiGLU rows can move a code by one step, so single tokens differ at the end-to-end tolerance, most by far less
+    rel = ((y_nosh - y_stage).abs() / y_stage.abs().max(dim=1, keepdim=True).values).max(dim=1).values
+    assert rel.max().item() <= END_TO_END_REL and rel.median().item() <= 2e-5, (rel.max().item(), rel.median().item())
+    y, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=(SG, SU, SD, cu(gate_inp)), silu=1)
+    pick = np.unique(np.concatenate([np.arange(0, n, max(1, n // 6)), [n - 1]]))
+    ref = orc.moe_layer(ge, ue, de, H, I, K, x[pick], logits[pick], shared=(sg, su, sd, gate_inp), silu=1)
+    got = y.cpu().numpy()[pick]
+    rel = np.max(np.abs(got - ref["y"]), axis=1) / np.max(np.abs(ref["y"]), axis=1)
+    assert np.max(rel) <= END_TO_END_REL, np.max(rel)
