@@ -986,6 +986,12 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
     return MQ_OK;
 }
 
+// Widths at which an expert product runs on the matrix-core GEMM in its expert-grouped form (see moe_gemm_applies).
+static bool moe_gemm_width(const mq_weight* w, int64_t n, int top_k) {
+    return w->type == kTypeQ4K && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
+           !(w->cols & 3) && !census.on;
+}
+
 int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
                       int top_k, float* y_dev, void* stream) {
     if (int rc = check_ready()) return rc;
@@ -998,13 +1004,28 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (int rc = quantize_into(g.aq, g.ad, x_dev, n * x_slots, w->cols, w->cols, s)) return rc;
+    // prefill widths: the matrix-core GEMM in its expert-grouped form (see mq_moe_layer_q4k)
+    const bool use_gemm = moe_gemm_width(w, n, top_k);
+    if (!use_gemm)
+        if (int rc = quantize_into(g.aq, g.ad, x_dev, n * x_slots, w->cols, w->cols, s)) return rc;
     RouteWs r;
     if (int rc = carve_route(n, top_k, w->n_experts, r)) return rc;
     // entries with ids outside [0, n_experts) are dropped by the grouping, so clear y first
     MQ_HIP(launch_fill_zero(y_dev, (size_t)n * top_k * (size_t)w->rows, s));
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, w->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
+    if (use_gemm) {
+        const int64_t entries = n * top_k, E = w->n_experts;
+        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, x_slots != 1, entries, E,
+                                    (int32_t*)g.plan.ptr, s));
+        MQ_HIP(g.ap.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, w->nb)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, w->cols, w->cols, entries, E, (const int32_t*)g.plan.ptr,
+                                                  (uint8_t*)g.ap.ptr, nullptr, 0, s));
+        MQ_HIP(launch_prefill_gemm_grouped(w->data, w->expert_bytes, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
+                                           (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s));
+        return MQ_OK;
+    }
     MatmulArgs a;
     a.w0 = w->data;
     a.wtype = w->type;
@@ -1380,6 +1401,28 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
     MQ_HIP(launch_fill_zero(hidden_dev, (size_t)n * top_k * (size_t)gate_exps->rows, s));
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, gate_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
+    if (moe_gemm_width(gate_exps, n, top_k) && up_exps->type == kTypeQ4K) {
+        // prefill widths: both products on the expert-grouped GEMM, SwiGLU rows scattered to their (token, slot) places
+        const int64_t entries = n * top_k, E = gate_exps->n_experts, inter = gate_exps->rows, hidden = gate_exps->cols;
+        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int32_t* plan = (const int32_t*)g.plan.ptr;
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, false, entries, E,
+                                    (int32_t*)g.plan.ptr, s));
+        const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
+        MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
+        MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
+        float* gbuf = (float*)g.mid2.ptr;
+        float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
+        MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->expert_bytes, inter, gate_exps->nb, (const uint8_t*)g.ap.ptr,
+                                           entries, E, plan, false, gbuf, inter, s));
+        MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->expert_bytes, inter, up_exps->nb, (const uint8_t*)g.ap.ptr,
+                                           entries, E, plan, false, ubuf, inter, s));
+        MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
+                                                  hidden_dev, inter, s));
+        return MQ_OK;
+    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, gate_exps->cols, gate_exps->cols, s)) return rc;
     return run_moe_gateup(gate_exps, up_exps, SharedExpert{}, n, top_k, top_k, silu_mode, r, hidden_dev, false, s);
 }
@@ -1400,6 +1443,22 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
     if (int rc = carve_route(n, top_k, down_exps->n_experts, r)) return rc;
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, down_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
+    if (moe_gemm_width(down_exps, n, top_k)) {
+        // prefill widths: the product on the expert-grouped GEMM into the per-(token, slot) rows, then the combine
+        const int64_t entries = n * top_k, E = down_exps->n_experts, hidden = down_exps->rows, inter = down_exps->cols;
+        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int32_t* plan = (const int32_t*)g.plan.ptr;
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, true, entries, E,
+                                    (int32_t*)g.plan.ptr, s));
+        MQ_HIP(g.ap2.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, inter / kQK)));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(hidden_dev, nullptr, false, 0, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
+                                                  nullptr, 0, s));
+        MQ_HIP(g.part.reserve((size_t)n * top_k * (size_t)hidden * sizeof(float)));
+        MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->expert_bytes, hidden, down_exps->nb, (const uint8_t*)g.ap2.ptr,
+                                           entries, E, plan, true, (float*)g.part.ptr, hidden, s));
+        MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, top_k, hidden, weights_dev, ids_dev, E, 0, nullptr, nullptr, y_dev, s));
+        return MQ_OK;
+    }
     return run_moe_down(down_exps, SharedExpert{}, hidden_dev, false, n, top_k, top_k, r, ids_dev, weights_dev, nullptr,
                         nullptr, y_dev, s);
 }
@@ -1513,11 +1572,11 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
                                       nullptr, nullptr, s));
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
         const int32_t* plan = (const int32_t*)g.plan.ptr;
-        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, entries, E,
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, false, entries, E,
                                     (int32_t*)g.plan.ptr, s));
         const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, s));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
@@ -1526,7 +1585,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->expert_bytes, inter, L->up_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr, s));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
         MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->expert_bytes, hidden, L->down_exps->nb,
                                            (const uint8_t*)g.ap2.ptr, entries, E, plan, true, part, hidden, s));
         MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));

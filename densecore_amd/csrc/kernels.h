@@ -179,11 +179,11 @@ int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max);
 int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max);
 size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max);
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
-                                const int32_t* entry_token, const int32_t* entry_k, int slots, int64_t entries, int64_t groups_max,
-                                int32_t* plan, hipStream_t stream);
+                                const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
+                                int64_t groups_max, int32_t* plan, hipStream_t stream);
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
-                                              int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap,
-                                              hipStream_t stream);
+                                              int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
+                                              int64_t ldh, hipStream_t stream);
 hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, int64_t rows, int64_t nb, const uint8_t* ap,
                                        int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter, float* y, int64_t ldy,
                                        hipStream_t stream);

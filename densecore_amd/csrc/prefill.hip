@@ -308,7 +308,8 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
                                                                   int silu_mode, float* __restrict__ h_out, int64_t ldh,
                                                                   int64_t n, int64_t ldx, int64_t nb, int64_t m_tiles,
                                                                   uint8_t* __restrict__ ap, const int32_t* __restrict__ plan,
-                                                                  const int32_t* __restrict__ row_src) {
+                                                                  const int32_t* __restrict__ row_src,
+                                                                  const int32_t* __restrict__ h_rows) {
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= m_tiles * 16 * nb) return;
@@ -325,7 +326,9 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
             const float4 u = *reinterpret_cast<const float4*>(x2 + src * ldx + b * kQK + lane * 4);
             e[0] = silu_mul(e[0], u.x, silu_mode), e[1] = silu_mul(e[1], u.y, silu_mode);
             e[2] = silu_mul(e[2], u.z, silu_mode), e[3] = silu_mul(e[3], u.w, silu_mode);
-            if (h_out) *reinterpret_cast<float4*>(h_out + src * ldh + b * kQK + lane * 4) = float4{e[0], e[1], e[2], e[3]};
+            // h_rows (expert-grouped): row m of the tiles is row h_rows[m] of h_out (-1: padding, not written)
+            const int64_t hr = h_rows ? h_rows[m] : src;
+            if (h_out && hr >= 0) *reinterpret_cast<float4*>(h_out + hr * ldh + b * kQK + lane * 4) = float4{e[0], e[1], e[2], e[3]};
         }
     }
     const Q8Lane q = quantize_block_q8k(e, lane);
@@ -397,13 +400,13 @@ PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n) {
 // group starting a new tile, and cuts every group's tiles into items of up to eight tiles, the unit a GEMM workgroup
 // column multiplies.  plan: [0] items, [1] tiles, [4 + 3 i ..] = (expert, first tile, tiles) of item i; row_src[r] /
 // out_row[r] for row r of the tiles: the token whose activations it holds and the row of the per-(token, slot) output
-// it produces (token * slots + k), -1 for padding.
+// it produces (token * slots + k), -1 for padding (src_per_slot: the activations are per (token, slot) rows too).
 __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __restrict__ n_groups, const int32_t* __restrict__ group_expert,
                                                              const int32_t* __restrict__ group_begin,
                                                              const int32_t* __restrict__ entry_token,
-                                                             const int32_t* __restrict__ entry_k, int slots, int groups_max,
-                                                             int32_t* __restrict__ plan, int32_t* __restrict__ row_src,
-                                                             int32_t* __restrict__ out_row) {
+                                                             const int32_t* __restrict__ entry_k, int slots, int src_per_slot,
+                                                             int groups_max, int32_t* __restrict__ plan,
+                                                             int32_t* __restrict__ row_src, int32_t* __restrict__ out_row) {
     extern __shared__ int32_t plan_sh[];  // begin[g] (groups_max + 1), tile0[g] (groups_max + 1), item0[g] (groups_max + 1)
     int32_t* begin = plan_sh;
     int32_t* tile0 = begin + groups_max + 1;
@@ -449,6 +452,7 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
             const int e = begin[g] + pos;
             src = entry_token[e];
             dst = src * slots + entry_k[e];
+            if (src_per_slot) src = dst;  // the activations come per (token, slot) as well
         }
         row_src[rr] = src, out_row[rr] = dst;
     }
@@ -465,21 +469,23 @@ size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max) {
 }
 
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
-                                const int32_t* entry_token, const int32_t* entry_k, int slots, int64_t entries, int64_t groups_max,
-                                int32_t* plan, hipStream_t stream) {
+                                const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
+                                int64_t groups_max, int32_t* plan, hipStream_t stream) {
     if (groups_max > 4096) return hipErrorInvalidValue;
     int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
     hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(1), dim3(1024), 3 * (size_t)(groups_max + 1) * sizeof(int32_t), stream, n_groups,
-                       group_expert, group_begin, entry_token, entry_k, slots, (int)groups_max, plan, row_src, out_row);
+                       group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, plan, row_src,
+                       out_row);
     return hipGetLastError();
 }
 
-// Rows of the plan's tiles in the P-major layout: gathered from x by token (swiglu == false), or silu(gate) * up of two
-// planes that already are in the plan's row order (swiglu == true).
+// Rows of the plan's tiles in the P-major layout: gathered from x by the plan's row list (swiglu == false), or
+// silu(gate) * up of two planes that already are in the plan's row order (swiglu == true; h_out, if given, receives
+// those rows as fp32 at their per-(token, slot) places).
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
-                                              int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap,
-                                              hipStream_t stream) {
+                                              int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
+                                              int64_t ldh, hipStream_t stream) {
     const int64_t nb = k / kQK, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t units = m_tiles * 16 * nb;
     if (units == 0) return hipSuccess;
@@ -487,10 +493,12 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
     const int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     if (swiglu) {
         hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, x2, silu_mode,
-                           (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr);
+                           h_out, ldh, m_tiles * 16, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr,
+                           row_src + 16 * m_tiles);
     } else {
         hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x,
-                           (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, row_src);
+                           (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, row_src,
+                           (const int32_t*)nullptr);
     }
     return hipGetLastError();
 }
@@ -534,7 +542,7 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x,
                        (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr,
-                       (const int32_t*)nullptr);
+                       (const int32_t*)nullptr, (const int32_t*)nullptr);
     return hipGetLastError();
 }
 
@@ -545,7 +553,8 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;
     hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, gate, up,
-                       silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr, (const int32_t*)nullptr);
+                       silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr, (const int32_t*)nullptr,
+                       (const int32_t*)nullptr);
     return hipGetLastError();
 }
 

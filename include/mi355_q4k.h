@@ -197,7 +197,10 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
  * [n][top_k]; entries outside [0, n_experts) produce zeros.  Tokens are grouped
  * by expert on the device; nothing returns to the host.  y_dev fp32
  * [n][top_k][rows].  (ggml_mul_mat_id as emitted at
- * core/src/llm/moe/native_gemma.cpp:1509-1559.) */
+ * core/src/llm/moe/native_gemma.cpp:1509-1559.)  Prefill widths (Q4_K, 256 tokens
+ * and more with a dozen rows per expert on average) run on the int8 matrix-core
+ * GEMM in its expert-grouped form, as do mq_moe_gateup_swiglu_q4k and
+ * mq_moe_down_weighted_q4k below. */
 int mq_mul_mat_id_q4k(const mq_weight* w_exps, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
                       int top_k, float* y_dev, void* stream);
 

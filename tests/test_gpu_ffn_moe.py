@@ -186,8 +186,9 @@ def make_experts(tag, E, H, I):
     return ge, ue, de
 
 
-@pytest.mark.parametrize("n", [1, 4, 16, 40])
+@pytest.mark.parametrize("n", [1, 4, 16, 40, 300])
 def test_mul_mat_id_matches_per_pair_dense_results(ops, n):
+    """300 tokens: a hundred rows per expert, the matrix-core GEMM in its expert-grouped form (both input forms)."""
     E, H, I, K = 12, 512, 256, 4
     ge, _, de = make_experts("mmid", E, H, I)
     GE, DE = ops.Q4KWeight.from_ggml(ge, H), ops.Q4KWeight.from_ggml(de, I)
@@ -279,7 +280,7 @@ def test_moe_layer_at_prefill_widths_runs_on_the_grouped_gemm(ops, n, E, K, shar
     """256 tokens and more with two dozen routed rows per expert: the expert products run on the matrix-core GEMM in its
     expert-grouped form (entries laid out in 16-row tiles per expert, up to eight tiles per workgroup column: groups
     of 75, 64 and 500 rows here -- padding rows, full tiles and several columns per expert).  End to end against the
-    oracle's layer, routing bit for bit, and against the stage-wise entries of the decode kernels on the same ids."""
+    oracle's layer, routing bit for bit; the two expert nodes at the same width against the oracle's stages."""
     H, I, silu = 512, 256, 1
     ge, ue, de = make_experts("moe-pf", E, H, I)
     sg, su, sd = (synth.q4k_matrix(synth.tensor_seed("moe-pf-sh", nm), r, c) for nm, r, c in
@@ -298,11 +299,20 @@ def test_moe_layer_at_prefill_widths_runs_on_the_grouped_gemm(ops, n, E, K, shar
     ref = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=sh_cpu, silu=silu)
     y = y.cpu().numpy()
     assert np.max(np.abs(y - ref["y"])) <= END_TO_END_REL * np.max(np.abs(ref["y"]))
-    # the routed part against the decode kernels' stages (same ids and weights; other summation order)
+    # the two expert nodes at the same width (the grouped GEMM as well): each against the oracle's stage, and the
+    # layer without its shared expert bit for bit their composition
+    wts = w.cpu().numpy()
+    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids, silu).cpu().numpy()
+    assert_close_prod(hid, orc.moe_gateup_swiglu(ge, ue, H, I, x, oi, orc.ORDER_DOTPROD, silu), "gate/up node")
+    y_stage = ops.moe_down_weighted(DE, cu(hid), ids, w).cpu().numpy()
+    mag = np.zeros((n, H))
+    hq = orc.quantize_rows_q8k(hid.reshape(n * K, I)).reshape(n, K, -1)
+    for t in range(n):
+        for k in range(K):
+            mag[t] += abs(wts[t, k]) * orc.dot_magnitude_f64(de[oi[t, k]], I, hq[t, k][None])[0]
+    assert_fp32_parity(y_stage, orc.moe_down_weighted(de, H, I, hid, oi, wts, orc.ORDER_DOTPROD, 0), mag, "down node")
     y_nosh, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=silu)
-    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids, silu)
-    y_stage = ops.moe_down_weighted(DE, hid, ids, w).cpu().numpy()
-    assert np.max(np.abs(y_nosh.cpu().numpy() - y_stage)) <= END_TO_END_REL * np.max(np.abs(y_stage))
+    assert np.array_equal(y_nosh.cpu().numpy().view(np.uint32), y_stage.view(np.uint32))
     for t in (GE, UE, DE, SG, SU, SD):
         t.free()
 

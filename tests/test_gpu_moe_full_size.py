@@ -95,12 +95,20 @@ def test_cfg3_layer_at_prefill_widths_on_the_grouped_gemm(layer, n):
     oi, ow = orc.route_topk(logits, K, 0)
     y_nosh, ids, w = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=None, silu=1)
     assert np.array_equal(ids.cpu().numpy(), oi) and np.allclose(w.cpu().numpy(), ow, rtol=3e-6)
-    hid = ops.moe_gateup_swiglu(GE, UE, cu(x), ids, 1)
-    y_stage = ops.moe_down_weighted(DE, hid, ids, w)
-    # the hidden rows are re-quantized to Q8_K for the down product: a last-bit difference between the two paths'
-    # SwiGLU rows can move a code by one step, so single tokens differ at the end-to-end tolerance, most by far less
+    # the decode kernels' stages on the same ids, in chunks of 128 tokens (below the width where the nodes switch to
+    # the GEMM themselves).  The hidden rows are re-quantized to Q8_K for the down product: a last-bit difference
+    # between the two paths' SwiGLU rows can move a code by one step, so single tokens differ at the end-to-end
+    # tolerance, most by far less
+    xs, parts = cu(x), []
+    for i in range(0, n, 128):
+        hid = ops.moe_gateup_swiglu(GE, UE, xs[i:i + 128], ids[i:i + 128], 1)
+        parts.append(ops.moe_down_weighted(DE, hid, ids[i:i + 128], w[i:i + 128]))
+    y_stage = torch.cat(parts)
     rel = ((y_nosh - y_stage).abs() / y_stage.abs().max(dim=1, keepdim=True).values).max(dim=1).values
     assert rel.max().item() <= END_TO_END_REL and rel.median().item() <= 2e-5, (rel.max().item(), rel.median().item())
+    # and the nodes at the full width (the GEMM): bit for bit the layer
+    hid = ops.moe_gateup_swiglu(GE, UE, xs, ids, 1)
+    assert torch.equal(ops.moe_down_weighted(DE, hid, ids, w), y_nosh)
     y, _, _ = ops.moe_layer(GE, UE, DE, cu(x), cu(logits), K, shared=(SG, SU, SD, cu(gate_inp)), silu=1)
     pick = np.unique(np.concatenate([np.arange(0, n, max(1, n // 6)), [n - 1]]))
     ref = orc.moe_layer(ge, ue, de, H, I, K, x[pick], logits[pick], shared=(sg, su, sd, gate_inp), silu=1)
