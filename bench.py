@@ -444,6 +444,18 @@ def side_measurements(ops, synth, torch, np, dev):
         moe[str(n)] = {"us": round(dt * 1e6, 2), "distinct_experts": distinct, "GBps": round(b / dt / 1e9, 1),
                        "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1), "tokens_per_s": round(n / dt, 1)}
     res["moe_layer_mul_mat_id"] = moe
+    # the same block at prefill widths: its expert products on the int8 matrix cores (expert-grouped GEMM)
+    moe_pf = {}
+    for n in (512, 2048):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))).to(dev)
+        lg = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))).to(dev)
+        dt = time_graph(lambda: [ops.moe_layer(ge, ue, de, x, lg, K, shared=sh, silu=ops.SILU_FAST)
+                                 for ge, ue, de, sh in layers], 5) / len(layers)
+        tops = 2.0 * n * (K + 1) * 3 * H * I / dt / 1e12
+        moe_pf[str(n)] = {"us": round(dt * 1e6, 1), "TOPs": round(tops, 1), "pct_int8_mfma_peak": round(tops / INT8_PEAK_TOPS * 100, 2),
+                          "tokens_per_s": round(n / dt, 1)}
+    moe_pf["note"] = "useful ops 2 * tokens * (top_k + shared) * 3 matrices * 2048 * 512 over the whole block (routing, gather, combine included)"
+    res["moe_layer_prefill"] = moe_pf
     for ge, ue, de, sh in layers:
         for w in (ge, ue, de) + sh[:3]:
             w.free()
