@@ -395,7 +395,9 @@ PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n) {
 }
 
 // ---- expert-grouped GEMM: the plan ------------------------------------------------------------------------
-// One workgroup.  From the expert groups of the routing (entries sorted by expert: group g holds the entries
+// Every workgroup repeats the (short) prefix sums over the groups and then takes its share of the items and rows:
+// each row costs two dependent reads of the entry lists, so one workgroup alone needs 29 us for 2048 tokens.
+// From the expert groups of the routing (entries sorted by expert: group g holds the entries
 // group_begin[g] .. group_begin[g + 1] - 1 of expert group_expert[g]) it lays the entries out in tiles of 16 rows, every
 // group starting a new tile, and cuts every group's tiles into items of up to eight tiles, the unit a GEMM workgroup
 // column multiplies.  plan: [0] items, [1] tiles, [4 + 3 i ..] = (expert, first tile, tiles) of item i; row_src[r] /
@@ -415,15 +417,30 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
     const int ng = *n_groups < groups_max ? *n_groups : groups_max;
     for (int g = tid; g <= ng; g += nt) begin[g] = group_begin[g];
     __syncthreads();
-    if (tid == 0) {
+    if (tid < 64) {  // wavefront 0: exclusive prefix sums of tiles and items, lane l over a run of consecutive groups
+        const int per = (ng + 63) / 64, g0 = tid * per;
         int tiles = 0, items = 0;
-        for (int g = 0; g < ng; ++g) {
+        for (int g = g0; g < g0 + per && g < ng; ++g) {
             const int t = (begin[g + 1] - begin[g] + 15) >> 4;
-            tile0[g] = tiles, item0[g] = items;
             tiles += t, items += (t + kMTilesPerGroup - 1) / kMTilesPerGroup;
         }
-        tile0[ng] = tiles, item0[ng] = items;
-        plan[0] = items, plan[1] = tiles, plan[2] = 0, plan[3] = 0;
+        int ts = tiles, is = items;  // inclusive scans across the lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int a = __shfl_up(ts, d, 64), b = __shfl_up(is, d, 64);
+            if (tid >= d) ts += a, is += b;
+        }
+        const int all_tiles = __shfl(ts, 63, 64), all_items = __shfl(is, 63, 64);
+        ts -= tiles, is -= items;
+        for (int g = g0; g < g0 + per && g < ng; ++g) {
+            const int t = (begin[g + 1] - begin[g] + 15) >> 4;
+            tile0[g] = ts, item0[g] = is;
+            ts += t, is += (t + kMTilesPerGroup - 1) / kMTilesPerGroup;
+        }
+        if (tid == 0) {
+            tile0[ng] = all_tiles, item0[ng] = all_items;
+            if (blockIdx.x == 0) plan[0] = all_items, plan[1] = all_tiles, plan[2] = 0, plan[3] = 0;
+        }
     }
     __syncthreads();
     // the group of position q in a non-decreasing prefix array: the last g with first[g] <= q (empty groups cannot occur)
@@ -437,14 +454,15 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
         return lo;
     };
     const int tiles = tile0[ng], items = item0[ng];
-    for (int i = tid; i < items; i += nt) {
+    const int first = blockIdx.x * nt + tid, step = gridDim.x * nt;
+    for (int i = first; i < items; i += step) {
         const int g = group_of(item0, i);
-        const int t_g = tile0[g + 1] - tile0[g], first = (i - item0[g]) * kMTilesPerGroup;
+        const int t_g = tile0[g + 1] - tile0[g], at = (i - item0[g]) * kMTilesPerGroup;
         plan[4 + 3 * i] = group_expert[g];
-        plan[5 + 3 * i] = tile0[g] + first;
-        plan[6 + 3 * i] = t_g - first < kMTilesPerGroup ? t_g - first : kMTilesPerGroup;
+        plan[5 + 3 * i] = tile0[g] + at;
+        plan[6 + 3 * i] = t_g - at < kMTilesPerGroup ? t_g - at : kMTilesPerGroup;
     }
-    for (int rr = tid; rr < tiles * 16; rr += nt) {
+    for (int rr = first; rr < tiles * 16; rr += step) {
         const int g = group_of(tile0, rr >> 4);
         const int pos = rr - tile0[g] * 16;
         int src = -1, dst = -1;
@@ -474,7 +492,9 @@ hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_ex
     if (groups_max > 4096) return hipErrorInvalidValue;
     int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
-    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(1), dim3(1024), 3 * (size_t)(groups_max + 1) * sizeof(int32_t), stream, n_groups,
+    const int64_t rows_max = 16 * moe_gemm_tiles_max(entries, groups_max);
+    const unsigned wgs = (unsigned)(rows_max / 1024 < 1 ? 1 : (rows_max / 1024 > 64 ? 64 : rows_max / 1024));
+    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 1) * sizeof(int32_t), stream, n_groups,
                        group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, plan, row_src,
                        out_row);
     return hipGetLastError();
