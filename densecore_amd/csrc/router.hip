@@ -463,13 +463,15 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     const int64_t entries = n * top_k;
     if (entries > (int64_t)1 << 30 || n_experts > 8192) return hipErrorInvalidValue;
     const int threads = entries >= 1024 ? 1024 : (entries > 256 ? 512 : 256);
-    const int use_lds = entries <= 8192;
-    size_t lds = (size_t)n_experts * 4 + (use_lds ? (size_t)entries * 4 : 0);
     // one bit per (expert, token) when that fits the 160 KB of a compute unit (256 experts: up to 4096 tokens); without
-    // it a pair's place in its group is found by scanning all earlier pairs -- 394 us at 512 tokens against 17 at 256
+    // it a pair's place in its group is found by scanning all earlier pairs -- 394 us at 512 tokens against 17 at 256.
+    // The ids join them in LDS while there is room (16384 pairs at 2048 tokens and 256 experts).
+    size_t lds = (size_t)n_experts * 4;
     int mask_words = n <= 4096 ? (int)((n + 31) / 32) : 0;
     if (lds + ((size_t)n_experts * (mask_words | 1) + 1) * 4 > 150 * 1024) mask_words = 0;
     if (mask_words) lds += ((size_t)n_experts * (mask_words | 1) + 1) * 4;
+    const int use_lds = lds + (size_t)entries * 4 <= 150 * 1024;
+    if (use_lds) lds += (size_t)entries * 4;
     if (lds > 64 * 1024) {
         static bool raised = false;
         if (!raised) {
