@@ -1018,11 +1018,11 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
         const int64_t entries = n * top_k, E = w->n_experts;
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, x_slots != 1, entries, E,
-                                    (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s));
         MQ_HIP(g.ap.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, w->nb)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, w->cols, w->cols, entries, E, (const int32_t*)g.plan.ptr,
                                                   (uint8_t*)g.ap.ptr, nullptr, 0, s));
-        MQ_HIP(launch_prefill_gemm_grouped(w->data, w->expert_bytes, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
+        MQ_HIP(launch_prefill_gemm_grouped(w->data, w->expert_bytes, nullptr, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
                                            (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s));
         return MQ_OK;
     }
@@ -1407,17 +1407,17 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
         const int32_t* plan = (const int32_t*)g.plan.ptr;
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, false, entries, E,
-                                    (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s));
         const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
-        MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->expert_bytes, inter, gate_exps->nb, (const uint8_t*)g.ap.ptr,
-                                           entries, E, plan, false, gbuf, inter, s));
-        MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->expert_bytes, inter, up_exps->nb, (const uint8_t*)g.ap.ptr,
-                                           entries, E, plan, false, ubuf, inter, s));
+        MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->expert_bytes, nullptr, inter, gate_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s));
+        MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->expert_bytes, nullptr, inter, up_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
                                                   hidden_dev, inter, s));
@@ -1449,13 +1449,13 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
         const int32_t* plan = (const int32_t*)g.plan.ptr;
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, true, entries, E,
-                                    (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(hidden_dev, nullptr, false, 0, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
                                                   nullptr, 0, s));
         MQ_HIP(g.part.reserve((size_t)n * top_k * (size_t)hidden * sizeof(float)));
-        MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->expert_bytes, hidden, down_exps->nb, (const uint8_t*)g.ap2.ptr,
-                                           entries, E, plan, true, (float*)g.part.ptr, hidden, s));
+        MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->expert_bytes, nullptr, hidden, down_exps->nb,
+                                           (const uint8_t*)g.ap2.ptr, entries, E, plan, true, (float*)g.part.ptr, hidden, s));
         MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, top_k, hidden, weights_dev, ids_dev, E, 0, nullptr, nullptr, y_dev, s));
         return MQ_OK;
     }
@@ -1560,34 +1560,34 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     if (moe_gemm_applies(L, sh, n) && !census.on) {
         // Prefill widths: the three expert products on the matrix-core GEMM in its expert-grouped form, the shared
         // expert as a dense FFN on it; per-(token, slot) rows and the combine as at the other widths.
-        const int64_t entries = n * K;
+        // The shared expert rides along as one more group of all tokens (its own weights, its own SiLU form, output slot K).
+        const int64_t entries = n * K + (sh.gate ? n : 0), G = E + (sh.gate ? 1 : 0);
         MQ_HIP(g.part.reserve((size_t)n * slots * (size_t)hidden * sizeof(float)));
         float* part = (float*)g.part.ptr;
-        if (sh.gate)  // first: it uses the same staging buffers
-            if (int rc = ffn_wide_locked(sh.gate, sh.up, sh.down, x_dev, n, hidden, MQ_SILU_FAST_FMA, nullptr, 0, part + (size_t)K * hidden,
-                                         (int64_t)slots * hidden, s))
-                return rc;
         MQ_HIP(launch_route_and_group(logits_dev, E, n, K, L->route_mode, ids, wts, (uint32_t*)g.counters.ptr + 4095,
                                       r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, true, nullptr, 0, 0,
                                       nullptr, nullptr, s));
-        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, G) * sizeof(int32_t)));
         const int32_t* plan = (const int32_t*)g.plan.ptr;
-        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, false, entries, E,
-                                    (int32_t*)g.plan.ptr, s));
-        const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
+        MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, false, entries, G,
+                                    sh.gate ? n : 0, MQ_SILU_FAST_FMA, (int32_t*)g.plan.ptr, s));
+        const int64_t rows_max = moe_gemm_tiles_max(entries, G) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, G, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
-        MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->expert_bytes, inter, L->gate_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s));
-        MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->expert_bytes, inter, L->up_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
+        const uint8_t* shg = sh.gate ? sh.gate->data : nullptr;
+        const uint8_t* shu = sh.gate ? sh.up->data : nullptr;
+        const uint8_t* shd = sh.gate ? sh.down->data : nullptr;
+        MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->expert_bytes, shg, inter, L->gate_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, gbuf, inter, s));
+        MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
+                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
-        MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->expert_bytes, hidden, L->down_exps->nb,
-                                           (const uint8_t*)g.ap2.ptr, entries, E, plan, true, part, hidden, s));
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, G, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
+        MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
+                                           (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
         MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
         return MQ_OK;
     }

@@ -175,18 +175,20 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
 // Expert-grouped form of the GEMM (a MoE block at prefill widths): a plan lays the routed entries out in 16-row tiles
 // per expert (moe_gemm_plan_ints() int32 of workspace; sizes from the upper bounds entries = n * top_k and groups_max),
 // the quantizer gathers or forms the rows of those tiles, the GEMM multiplies every item by its expert's weights.
+// sh_tokens > 0 appends the shared expert as one more group of all tokens (weights w_shared, output slot slots - 1);
+// `entries` and `groups_max` then count its rows and its group as well.
 int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max);
 int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max);
 size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max);
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
                                 const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
-                                int64_t groups_max, int32_t* plan, hipStream_t stream);
+                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream);
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
                                               int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
                                               int64_t ldh, hipStream_t stream);
-hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, int64_t rows, int64_t nb, const uint8_t* ap,
-                                       int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter, float* y, int64_t ldy,
-                                       hipStream_t stream);
+hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows, int64_t nb,
+                                       const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
+                                       float* y, int64_t ldy, hipStream_t stream);
 
 // ---- elementwise.hip -------------------------------------------------------------------------
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,

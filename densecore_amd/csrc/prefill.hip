@@ -149,7 +149,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
                                                            int64_t split_stride, const int32_t* __restrict__ plan,
-                                                           int64_t expert_bytes, const int32_t* __restrict__ out_rows) {
+                                                           int64_t expert_bytes, const int32_t* __restrict__ out_rows,
+                                                           const uint8_t* __restrict__ w_shared) {
     extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     const int tid = threadIdx.x;
@@ -163,7 +164,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     if (plan) {
         const int item = blockIdx.y;
         if (item >= plan[0]) return;  // the whole workgroup, before any barrier
-        w += (size_t)plan[4 + 3 * item] * (size_t)expert_bytes;
+        const int expert = plan[4 + 3 * item];  // -1: the shared expert's rows
+        w = expert < 0 ? w_shared : w + (size_t)expert * (size_t)expert_bytes;
         mt0 = plan[5 + 3 * item];
         mt_count = plan[6 + 3 * item];
     }
@@ -319,6 +321,7 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t tile = blockIdx.x, b = blockIdx.y;
     if (plan && tile >= (int64_t)plan[1]) return;  // the whole workgroup, before the barrier
+    if (plan && kSwiglu && tile >= (int64_t)plan[2]) silu_mode = plan[3];  // the shared expert's tiles: its own SiLU form
     int64_t src[4], hr[4];
     float4 v[4], u[4];
 #pragma unroll
@@ -424,15 +427,21 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
                                                              const int32_t* __restrict__ group_begin,
                                                              const int32_t* __restrict__ entry_token,
                                                              const int32_t* __restrict__ entry_k, int slots, int src_per_slot,
-                                                             int groups_max, int32_t* __restrict__ plan,
-                                                             int32_t* __restrict__ row_src, int32_t* __restrict__ out_row) {
-    extern __shared__ int32_t plan_sh[];  // begin[g] (groups_max + 1), tile0[g] (groups_max + 1), item0[g] (groups_max + 1)
+                                                             int groups_max, int sh_tokens, int sh_slot, int sh_silu_mode,
+                                                             int32_t* __restrict__ plan, int32_t* __restrict__ row_src,
+                                                             int32_t* __restrict__ out_row) {
+    extern __shared__ int32_t plan_sh[];  // begin[g], tile0[g], item0[g]: groups_max + 2 each
     int32_t* begin = plan_sh;
-    int32_t* tile0 = begin + groups_max + 1;
-    int32_t* item0 = tile0 + groups_max + 1;
+    int32_t* tile0 = begin + groups_max + 2;
+    int32_t* item0 = tile0 + groups_max + 2;
     const int tid = threadIdx.x, nt = blockDim.x;
-    const int ng = *n_groups < groups_max ? *n_groups : groups_max;
-    for (int g = tid; g <= ng; g += nt) begin[g] = group_begin[g];
+    // sh_tokens > 0: one more group behind the routed ones, the shared expert with every token in order (expert -1,
+    // output slot sh_slot); plan[2] = its first tile, plan[3] = its SiLU form
+    const int ng_routed = *n_groups < groups_max ? *n_groups : groups_max;
+    const int ng = ng_routed + (sh_tokens > 0 ? 1 : 0);
+    for (int g = tid; g <= ng_routed; g += nt) begin[g] = group_begin[g];
+    __syncthreads();
+    if (tid == 0 && sh_tokens > 0) begin[ng] = begin[ng_routed] + sh_tokens;
     __syncthreads();
     if (tid < 64) {  // wavefront 0: exclusive prefix sums of tiles and items, lane l over a run of consecutive groups
         const int per = (ng + 63) / 64, g0 = tid * per;
@@ -456,10 +465,11 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
         }
         if (tid == 0) {
             tile0[ng] = all_tiles, item0[ng] = all_items;
-            if (blockIdx.x == 0) plan[0] = all_items, plan[1] = all_tiles, plan[2] = 0, plan[3] = 0;
         }
     }
     __syncthreads();
+    if (tid == 0 && blockIdx.x == 0)
+        plan[0] = item0[ng], plan[1] = tile0[ng], plan[2] = sh_tokens > 0 ? tile0[ng_routed] : tile0[ng], plan[3] = sh_silu_mode;
     // the group of position q in a non-decreasing prefix array: the last g with first[g] <= q (empty groups cannot occur)
     auto group_of = [&](const int32_t* first, int q) {
         int lo = 0, hi = ng - 1;
@@ -475,7 +485,7 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
     for (int i = first; i < items; i += step) {
         const int g = group_of(item0, i);
         const int t_g = tile0[g + 1] - tile0[g], at = (i - item0[g]) * kMTilesPerGroup;
-        plan[4 + 3 * i] = group_expert[g];
+        plan[4 + 3 * i] = g < ng_routed ? group_expert[g] : -1;
         plan[5 + 3 * i] = tile0[g] + at;
         plan[6 + 3 * i] = t_g - at < kMTilesPerGroup ? t_g - at : kMTilesPerGroup;
     }
@@ -484,10 +494,15 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
         const int pos = rr - tile0[g] * 16;
         int src = -1, dst = -1;
         if (pos < begin[g + 1] - begin[g]) {
-            const int e = begin[g] + pos;
-            src = entry_token[e];
-            dst = src * slots + entry_k[e];
-            if (src_per_slot) src = dst;  // the activations come per (token, slot) as well
+            if (g < ng_routed) {
+                const int e = begin[g] + pos;
+                src = entry_token[e];
+                dst = src * slots + entry_k[e];
+                if (src_per_slot) src = dst;  // the activations come per (token, slot) as well
+            } else {
+                src = pos;
+                dst = pos * slots + sh_slot;
+            }
         }
         row_src[rr] = src, out_row[rr] = dst;
     }
@@ -495,6 +510,8 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
 
 }  // namespace
 
+// upper bounds: `entries` counts every row of the plan (the routed pairs and, with a shared expert, every token once
+// more), groups_max every group (the experts, + 1 with a shared expert)
 int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max) { return (entries + 15) / 16 + groups_max; }
 int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max) {  // a multiple of four: the row arrays behind the items stay 16-byte aligned
     return ((entries + 16 * kMTilesPerGroup - 1) / (16 * kMTilesPerGroup) + groups_max + 3) & ~(int64_t)3;
@@ -505,15 +522,15 @@ size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max) {
 
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
                                 const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
-                                int64_t groups_max, int32_t* plan, hipStream_t stream) {
-    if (groups_max > 4096) return hipErrorInvalidValue;
+                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream) {
+    if (groups_max > 4097) return hipErrorInvalidValue;
     int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
     const int64_t rows_max = 16 * moe_gemm_tiles_max(entries, groups_max);
     const unsigned wgs = (unsigned)(rows_max / 1024 < 1 ? 1 : (rows_max / 1024 > 64 ? 64 : rows_max / 1024));
-    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 1) * sizeof(int32_t), stream, n_groups,
-                       group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, plan, row_src,
-                       out_row);
+    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 2) * sizeof(int32_t), stream, n_groups,
+                       group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, (int)sh_tokens,
+                       slots - 1, sh_silu_mode, plan, row_src, out_row);
     return hipGetLastError();
 }
 
@@ -541,9 +558,9 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
 
 // y = the plan's tiles . W_expert^T per item.  scatter == false: y [tiles * 16][ldy] in the plan's row order;
 // true: row out_row[r] of y (the per-(token, slot) rows of the down product).
-hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, int64_t rows, int64_t nb, const uint8_t* ap,
-                                       int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter, float* y, int64_t ldy,
-                                       hipStream_t stream) {
+hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows, int64_t nb,
+                                       const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
+                                       float* y, int64_t ldy, hipStream_t stream) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t items = moe_gemm_items_max(entries, groups_max);
     if (rowtiles == 0 || items == 0) return hipSuccess;
@@ -559,7 +576,7 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, i
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
     hipLaunchKernelGGL(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
                        2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
-                       (int64_t)0, plan, expert_bytes, out_row);
+                       (int64_t)0, plan, expert_bytes, out_row, w_shared);
     return hipGetLastError();
 }
 
@@ -614,10 +631,12 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
     const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
     if (ps.narrow) {
         hipLaunchKernelGGL(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
-                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr);
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
+                           (const uint8_t*)nullptr);
     } else {
         hipLaunchKernelGGL(prefill_gemm_kernel<2>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
-                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr);
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
+                           (const uint8_t*)nullptr);
     }
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (split) {

@@ -231,7 +231,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way.
  * Prefill widths (Q4_K stacks, 256 tokens and more with a dozen routed rows per expert on average): the expert
  * products run on the int8 matrix-core GEMM in an expert-grouped form (entries in 16-row tiles per expert), the
- * shared expert as a dense FFN on it; same routing, results within the fp32 tolerance of the other form (the
+ * shared expert as one more group of all tokens; same routing, results within the fp32 tolerance of the other form (the
  * summation order differs), and mq_debug_moe_hidden does not apply. */
 typedef struct {
     const mq_weight* gate_exps; /* n_experts x [inter][hidden]  */
