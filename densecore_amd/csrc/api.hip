@@ -733,6 +733,12 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
             return MQ_OK;
         }
     }
+    if (prefill_applies(w, n) && !census.on) {
+        // prefill widths: the normalised rows as fp32, then the matrix-core GEMM (its quantizer reads them)
+        MQ_HIP(g.mid.reserve((size_t)n * (size_t)w->cols * sizeof(float)));
+        MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, w->cols, eps, sum_out_dev, (float*)g.mid.ptr, nullptr, nullptr, s));
+        return gemm_locked(w, (const float*)g.mid.ptr, n, w->cols, y_dev, ldy, s);
+    }
     const int64_t nb = w->cols / kQK;
     MQ_HIP(g.aq.reserve(aq_bytes(n, nb)));
     MQ_HIP(g.ad.reserve(ad_count(n, nb) * sizeof(float)));

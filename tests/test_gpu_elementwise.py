@@ -135,3 +135,27 @@ def test_rmsnorm_mul_mat_equals_norm_then_product(n, rows, cols, with_delta, wit
         _lib.check(L.mq_rmsnorm_mul_mat_q4k(W._h, p(x), p(d), p(w), n, C.c_float(1e-6), p(x), p(got_y), rows, None), "in place")
     acts.free()
     W.free()
+
+
+@pytest.mark.parametrize("n,rows,cols", [(64, 2560, 2048), (20, 14336, 4096)])
+def test_rmsnorm_mul_mat_at_prefill_widths_is_norm_then_gemm(n, rows, cols):
+    """Where mq_mul_mat_q4k takes the matrix-core GEMM (48 rows; 17 for 24 MB and more) the fused entry does too: the
+    bits of mq_add_rmsnorm_f32 followed by mq_gemm_q4k on the normalised rows."""
+    import torch
+    from densecore_amd import _lib, ops
+    g = torch.Generator(device="cuda").manual_seed(rows + cols + n)
+    x = torch.randn((n, cols), device="cuda", generator=g)
+    d = torch.randn((n, cols), device="cuda", generator=g)
+    w = torch.rand((cols,), device="cuda", generator=g) + 0.5
+    W = ops.Q4KWeight.synthetic(rows * 3 + cols, rows, cols)
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    L = _lib.lib()
+    ref_sum, ref_h = torch.empty_like(x), torch.empty_like(x)
+    _lib.check(L.mq_add_rmsnorm_f32(p(x), p(d), p(w), n, cols, C.c_float(1e-6), p(ref_sum), p(ref_h), None), "norm")
+    ref_y = ops.gemm(W, ref_h)
+    got_sum = torch.empty_like(x)
+    got_y = torch.empty((n, rows), device="cuda")
+    _lib.check(L.mq_rmsnorm_mul_mat_q4k(W._h, p(x), p(d), p(w), n, C.c_float(1e-6), p(got_sum), p(got_y), rows, None), "fused")
+    torch.cuda.synchronize()
+    assert torch.equal(got_sum, ref_sum) and torch.equal(got_y, ref_y)
+    W.free()
