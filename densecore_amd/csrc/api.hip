@@ -535,8 +535,8 @@ constexpr int64_t kPrefillMinRows = 48;
 constexpr int64_t kPrefillMinRowsLarge = 17;
 constexpr int64_t kPrefillLargeBytes = 24ll << 20;
 static bool prefill_applies(const mq_weight* w, int64_t n) {
-    if (w->type != kTypeQ4K) return false;
-    return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
+    if (w->type != kTypeQ4K && w->type != kTypeQ5K) return false;
+    return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->type == kTypeQ4K && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
 }
 constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
 // Widest product that also runs the residual add and the RMSNorm inside the GEMV kernel: every workgroup repeats the
@@ -549,9 +549,9 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
     if (n == 0) return MQ_OK;
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, w->nb)));
     MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, w->cols, (uint8_t*)g.ap.ptr, s));
-    const size_t part_bytes = prefill_part_bytes(w->rows, w->nb, n);
+    const size_t part_bytes = prefill_part_bytes(w->rows, w->nb, n, w->type);
     if (part_bytes) MQ_HIP(g.kpart.reserve(part_bytes));
-    MQ_HIP(launch_prefill_gemm(w->data, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy,
+    MQ_HIP(launch_prefill_gemm(w->data, w->type, w->rows, w->nb, (const uint8_t*)g.ap.ptr, n, y_dev, ldy,
                                part_bytes ? (float*)g.kpart.ptr : nullptr, s));
     return MQ_OK;
 }
@@ -566,11 +566,11 @@ static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_
     float* ubuf = gbuf + (size_t)n * (size_t)inter;
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, gate->nb)));
     MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, gate->cols, (uint8_t*)g.ap.ptr, s));
-    const size_t part_bytes = prefill_part_bytes(inter, gate->nb, n);
+    const size_t part_bytes = prefill_part_bytes(inter, gate->nb, n, gate->type);
     if (part_bytes) MQ_HIP(g.kpart.reserve(part_bytes));
     float* part = part_bytes ? (float*)g.kpart.ptr : nullptr;
-    MQ_HIP(launch_prefill_gemm(gate->data, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, gbuf, inter, part, s));
-    MQ_HIP(launch_prefill_gemm(up->data, inter, up->nb, (const uint8_t*)g.ap.ptr, n, ubuf, inter, part, s));
+    MQ_HIP(launch_prefill_gemm(gate->data, gate->type, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, gbuf, inter, part, s));
+    MQ_HIP(launch_prefill_gemm(up->data, up->type, inter, up->nb, (const uint8_t*)g.ap.ptr, n, ubuf, inter, part, s));
     if (!down) {  // SwiGLU rows only: the quantizer's fp32 side output is the result
         MQ_HIP(g.ap2.reserve(pmajor_bytes(n, inter / kQK)));
         MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
@@ -578,9 +578,9 @@ static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_
     }
     MQ_HIP(g.ap2.reserve(pmajor_bytes(n, down->nb)));
     MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
-    const size_t part2 = prefill_part_bytes(down->rows, down->nb, n);
+    const size_t part2 = prefill_part_bytes(down->rows, down->nb, n, down->type);
     if (part2) MQ_HIP(g.kpart.reserve(part2));
-    MQ_HIP(launch_prefill_gemm(down->data, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, ldy,
+    MQ_HIP(launch_prefill_gemm(down->data, down->type, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, ldy,
                                part2 ? (float*)g.kpart.ptr : nullptr, s));
     return MQ_OK;
 }
@@ -613,7 +613,8 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_gemm_q4k")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: weight is an expert stack");
-    if (w->type != kTypeQ4K) return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K weights only");
+    if (w->type != kTypeQ4K && w->type != kTypeQ5K)
+        return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K and Q5_K weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");

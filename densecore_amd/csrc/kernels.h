@@ -168,8 +168,9 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
 // y[n][ldy] = P-major activations . tiled weights^T on the int8 matrix cores.  A launch that would leave workgroup
 // slots empty splits K into runs of super-blocks whose sums go to planes of `part` (prefill_part_bytes() bytes, 0 when
 // nothing is split) and are added in order by a second launch.
-size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n);
-hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
+// wtype: kTypeQ4K, or kTypeQ5K (a third MFMA chain for the fifth code bits; 64-row workgroups).
+size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype);
+hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
                                int64_t ldy, float* part, hipStream_t stream);
 
 // Expert-grouped form of the GEMM (a MoE block at prefill widths): a plan lays the routed entries out in 16-row tiles

@@ -72,12 +72,16 @@ __device__ __forceinline__ uint32_t digit_pair(uint32_t word, int i) {
 }
 
 struct WTile {
+    v4i b5[4];         // Q5_K only: the fifth code bits times the whole 6-bit scale (16 * scale * bit is their share)
     v4i hi[4], lo[4];  // B operands of the four chunk pairs, scaled by the high / low scale digit
     v8h mins;          // B operand of the min MFMA: the eight mins as fp16, in every k-group
     float d, dmin;
 };
 
-__device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, const v4u hdr, int kq, WTile& t) {
+// Q5: the codes are nibble + 16 * bit (bit s of the bytes of qh = fifth bit in sub-block s, core/src/kernels/hwy/hwy_moe_quant.cc:177-200);
+// scale * code = scale * nibble + 16 * (scale * bit), and scale * bit <= 63 is a byte: a third MFMA chain.
+template <bool Q5>
+__device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, const v4u hdr, const v2u qh, int kq, WTile& t) {
     // 6-bit scales and mins (core/src/kernels/hwy/hwy_moe_quant.cc:90-101), four to a word
     const uint32_t sc03 = hdr.y & 0x3f3f3f3fu, mn03 = hdr.z & 0x3f3f3f3fu;
     const uint32_t sc47 = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
@@ -104,6 +108,15 @@ __device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, cons
                               (int)scale_bytes<1>(h3, ce1)};
         t.lo[2 * i + 1] = v4i{(int)scale_bytes<1>(h0, ab0), (int)scale_bytes<1>(h1, ab0), (int)scale_bytes<1>(h2, ce0),
                               (int)scale_bytes<1>(h3, ce0)};
+        if constexpr (Q5) {
+            const uint32_t scw = i ? sc47 : sc03;
+            const uint32_t abs_ = digit_pair(scw, 0), ces = digit_pair(scw, 2);  // whole scales of sub-blocks (4i, 4i+1), (4i+2, 4i+3)
+            auto bits = [&](uint32_t word, int sb) { return (word >> sb) & 0x01010101u; };
+            t.b5[2 * i] = v4i{(int)scale_bytes<0>(bits(qh.x, 4 * i), abs_), (int)scale_bytes<0>(bits(qh.y, 4 * i), abs_),
+                              (int)scale_bytes<0>(bits(qh.x, 4 * i + 2), ces), (int)scale_bytes<0>(bits(qh.y, 4 * i + 2), ces)};
+            t.b5[2 * i + 1] = v4i{(int)scale_bytes<1>(bits(qh.x, 4 * i + 1), abs_), (int)scale_bytes<1>(bits(qh.y, 4 * i + 1), abs_),
+                                  (int)scale_bytes<1>(bits(qh.x, 4 * i + 3), ces), (int)scale_bytes<1>(bits(qh.y, 4 * i + 3), ces)};
+        }
     }
     // byte -> fp16: 0x6400 | n is 1024 + n; two at a time
     const v2h bias = {(_Float16)1024.0f, (_Float16)1024.0f};
@@ -144,7 +157,7 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
 
 // kWTilesPerWave = 2: the 128 x 128 workgroup tile above.  1: 64 weight rows per workgroup, for launches whose
 // 128-row workgroups would leave compute units without their two workgroups (M up to a few hundred).
-template <int kWTilesPerWave>
+template <int kWTilesPerWave, bool Q5 = false>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
@@ -193,13 +206,16 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     // of b+1 travel HBM/L2 -> LDS (other buffer) and this wave's weight tiles of b+1 travel into
     // registers.  One workgroup barrier per super-block.
     v4u seg0[kWTilesPerWave], seg1[kWTilesPerWave], hdr[kWTilesPerWave];
+    v2u qh[kWTilesPerWave];
     auto request_w = [&](int64_t b) {
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
-            const uint8_t* tile = w + tile_offset(rt[t], b, nb);
+            const uint8_t* tile = w + tile_offset(rt[t], b, nb, Q5 ? kTile5Bytes : kTileBytes);
             seg0[t] = load16(tile + lane * 16);
             seg1[t] = load16(tile + 1024 + lane * 16);
             hdr[t] = load16(tile + kTileQBytes + r * 16);
+            if (Q5) qh[t] = *reinterpret_cast<const v2u*>(tile + kTileHBytes + lane * 8);
+            else qh[t] = v2u{0u, 0u};
         }
     };
     // K split over grid.z: this workgroup multiplies the super-blocks [b_begin, b_end) and writes its sums to
@@ -218,7 +234,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         __syncthreads();
         WTile wt[kWTilesPerWave];
 #pragma unroll
-        for (int t = 0; t < kWTilesPerWave; ++t) expand_tile(seg0[t], seg1[t], hdr[t], kq, wt[t]);
+        for (int t = 0; t < kWTilesPerWave; ++t) expand_tile<Q5>(seg0[t], seg1[t], hdr[t], qh[t], kq, wt[t]);
         if (b + 1 < b_end) {
             request_a_tiles(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
             request_w(b + 1);
@@ -236,12 +252,13 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                 const float4 yd = *reinterpret_cast<const float4*>(at + kPScaleOff + kq * 16);
                 const v4i zero = {0, 0, 0, 0};
                 const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
-                v4i hi[kWTilesPerWave], lo[kWTilesPerWave];
+                v4i hi[kWTilesPerWave], lo[kWTilesPerWave], fb[kWTilesPerWave];
                 v4f mn[kWTilesPerWave];
 #pragma unroll
                 for (int t = 0; t < kWTilesPerWave; ++t) {
                     hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].hi[0], zero, 0, 0, 0);
                     lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].lo[0], zero, 0, 0, 0);
+                    if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].b5[0], zero, 0, 0, 0);
                     mn[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt[t].mins, zero_f, 0, 0, 0);
                 }
 #pragma unroll
@@ -250,13 +267,15 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                     for (int t = 0; t < kWTilesPerWave; ++t) {
                         hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].hi[j], hi[t], 0, 0, 0);
                         lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].lo[j], lo[t], 0, 0, 0);
+                        if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].b5[j], fb[t], 0, 0, 0);
                     }
                 const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
 #pragma unroll
                 for (int t = 0; t < kWTilesPerWave; ++t)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int dot = hi[t][i] * 8 + lo[t][i];
+                        int dot = hi[t][i] * 8 + lo[t][i];
+                        if (Q5) dot += fb[t][i] * 16;
                         // yd * (d * dot - dmin * min_dot): three fp32 operations per output and super-block
                         const float v = __fmaf_rn(-wt[t].dmin, mn[t][i], __fmul_rn(wt[t].d, (float)dot));
                         acc[t][m][i] = __fmaf_rn(ydv[i], v, acc[t][m][i]);
@@ -396,14 +415,14 @@ struct PrefillShape {
     int splits, sb_split;
     unsigned row_wgs, groups;
 };
-PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n) {
+PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n, bool q5 = false) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
     PrefillShape ps;
     ps.groups = (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup);
     // two workgroups fit a compute unit: while the 128-row workgroups would not even give every unit one, 64-row
     // ones fill the chip better (14336 rows on 256 units: up to M = 256; 52 -> 40 us at M = 128, 55 -> 51 at 256,
     // and 76 -> 79, 78 -> 91 at M = 384, 512, where the wide ones stay)
-    ps.narrow = ((rowtiles + 7) / 8) * (int64_t)ps.groups <= (int64_t)compute_units();
+    ps.narrow = q5 || ((rowtiles + 7) / 8) * (int64_t)ps.groups <= (int64_t)compute_units();  // Q5_K: its third operand set only fits the registers of 64-row workgroups
     ps.row_wgs = (unsigned)(ps.narrow ? (rowtiles + 3) / 4 : (rowtiles + 7) / 8);
     const int64_t wgs = (int64_t)ps.row_wgs * ps.groups;
     int splits = (int)(2 * (int64_t)compute_units() / (wgs > 0 ? wgs : 1));
@@ -567,7 +586,8 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, c
     if (items > 65535) return hipErrorInvalidValue;
     static bool raised = false;
     if (!raised) {
-        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>)}) {
+        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>),
+                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, true>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
             if (e != hipSuccess) return e;
         }
@@ -580,8 +600,8 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, c
     return hipGetLastError();
 }
 
-size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n) {
-    const PrefillShape ps = prefill_shape(rows, nb, n);
+size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype) {
+    const PrefillShape ps = prefill_shape(rows, nb, n, wtype == kTypeQ5K);
     return ps.splits > 1 ? (size_t)ps.splits * (size_t)n * (size_t)rows * sizeof(float) : 0;
 }
 
@@ -609,16 +629,18 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
     return hipGetLastError();
 }
 
-hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
+hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
                                int64_t ldy, float* part, hipStream_t stream) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
     if (rowtiles == 0 || m_tiles == 0) return hipSuccess;
-    const PrefillShape ps = prefill_shape(rows, nb, n);
+    if (wtype != kTypeQ4K && wtype != kTypeQ5K) return hipErrorInvalidValue;
+    const PrefillShape ps = prefill_shape(rows, nb, n, wtype == kTypeQ5K);
     if (ps.groups > 65535u) return hipErrorInvalidValue;
     if (ps.splits > 1 && !part) return hipErrorInvalidValue;
     static bool raised = false;  // two activation buffers: more than the default 64 KB of dynamic LDS
     if (!raised) {
-        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>)}) {
+        for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>),
+                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, true>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
             if (e != hipSuccess) return e;
         }
@@ -629,7 +651,11 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int64_t rows, int64_t nb, const
     const int64_t ld = split ? rows : ldy;
     const int64_t stride = split ? n * rows : 0;
     const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
-    if (ps.narrow) {
+    if (wtype == kTypeQ5K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, true>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
+                           (const uint8_t*)nullptr);
+    } else if (ps.narrow) {
         hipLaunchKernelGGL(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);

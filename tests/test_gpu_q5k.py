@@ -69,7 +69,10 @@ def test_q5k_matmul_integer_sums_exact_and_fp32_within_tolerance(ops, rows, cols
     assert np.array_equal(ds.cpu().numpy(), ods), "dot_scaled differs"
     assert np.array_equal(md.cpu().numpy(), omd), "min_dot differs"
     y = y.cpu().numpy()
-    assert np.array_equal(y_dbg.cpu().numpy().view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    if n < 48:
+        assert np.array_equal(y_dbg.cpu().numpy().view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    else:  # from 48 rows the product runs on the matrix-core GEMM: the same integers, another summation order
+        assert np.max(np.abs(y_dbg.cpu().numpy() - y)) <= 1e-5 * np.max(np.abs(y))
     mag = orc.q5k_dot_dequant_f64(w_np, cols, q8, magnitude=True)
     for name, order in Q5_ORDERS.items():
         assert_fp32_parity(y, orc.mul_mat_q5k_q8k(w_np, cols, q8, order), mag, f"order={name}")
@@ -195,8 +198,10 @@ def test_q5k_rejections(ops):
     w5 = ops.Q4KWeight.from_ggml(synth.q5k_matrix(1, 64, 512), 512, Q5)
     w4 = ops.Q4KWeight.from_ggml(synth.q4k_matrix(1, 64, 512), 512)
     x = torch.zeros((64, 512), device="cuda")
+    w6 = ops.Q4KWeight.from_ggml(synth.q6k_matrix(1, 64, 512), 512, 14)
     with pytest.raises(MqError):
-        ops.gemm(w5, x)                                                 # matrix-core GEMM is Q4_K only
+        ops.gemm(w6, x)                                                 # the matrix-core GEMM takes Q4_K and Q5_K only
+    w6.free()
     with pytest.raises(MqError):
         ops.swiglu_mul_mat(w4, w5, x[:2], 0)                            # gate and up of different types
     with pytest.raises(MqError):
@@ -205,3 +210,64 @@ def test_q5k_rejections(ops):
         ops.Q4KWeight.from_ggml(np.zeros((4, 84), np.uint8), 256, 10)   # Q2_K is not handled
     w4.free()
     w5.free()
+
+
+# ----------------------------------------------------------------------------- matrix-core GEMM (prefill widths)
+@pytest.mark.parametrize("rows,cols,n", [(96, 768, 64), (80, 4096, 50), (272, 2048, 130)])
+def test_q5k_gemm_matches_oracle_and_decode_kernel(ops, rows, cols, n):
+    """48 rows and more of Q5_K: the int8 matrix-core GEMM with a third MFMA chain for the fifth code bits (the second
+    shape splits K into runs).  Against the oracle, against 16-row passes of the decode kernel, and through mq_mul_mat_q4k."""
+    import torch
+    w_np = synth.q5k_matrix(synth.tensor_seed("pf5-w", rows, cols), rows, cols)
+    x = synth.normal_f32(synth.tensor_seed("pf5-x", rows, cols, n), (n, cols))
+    W = ops.Q4KWeight.from_ggml(w_np, cols, Q5)
+    got = ops.gemm(W, cu(x))
+    assert torch.equal(ops.mul_mat(W, cu(x)), got)
+    small = torch.cat([ops.mul_mat(W, cu(x[i:i + 16])) for i in range(0, n, 16)])
+    assert (got - small).abs().max().item() <= 1e-5 * small.abs().max().item()
+    q8 = orc.quantize_rows_q8k(x)
+    mag = orc.q5k_dot_dequant_f64(w_np, cols, q8, magnitude=True)
+    assert_fp32_parity(got.cpu().numpy(), orc.mul_mat_q5k_q8k(w_np, cols, q8, orc.ORDER_DOTPROD), mag, "Q5_K GEMM")
+    W.free()
+
+
+def test_q5k_gemm_integer_sums_are_exact(ops):
+    """d = dmin = 1 and integer activations with a +-127 in every block: the output equals the oracle's integers."""
+    rows, cols, n = 48, 768, 70
+    nb = cols // 256
+    w = synth.q5k_matrix(synth.tensor_seed("pf5-int", rows), rows, cols).reshape(rows, nb, 176).copy()
+    w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[:, :, 2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w = w.reshape(rows, nb * 176)
+    rng = np.random.default_rng(11)
+    x = rng.integers(-127, 128, size=(n, cols)).astype(np.float32)
+    x.reshape(n, nb, 256)[:, :, 7] = rng.choice([-127.0, 127.0], size=(n, nb))
+    q8 = orc.quantize_rows_q8k(x)
+    d, _, _ = orc.split_q8k(q8)
+    assert np.all(np.abs(d) == 1.0)
+    ds, md = orc.q5k_matrix_block_sums(w, cols, q8)
+    want = ((ds.astype(np.int64) - md.astype(np.int64)) * d.astype(np.int64)[None]).sum(axis=2).T
+    assert np.abs(want).max() < 2 ** 24
+    W = ops.Q4KWeight.from_ggml(w, cols, Q5)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    assert np.array_equal(got, want.astype(np.float32))
+    W.free()
+
+
+def test_q5k_gemm_extreme_blocks(ops):
+    """All codes 31, scales and mins 63, activations at +-full scale: the largest bytes of all three operand sets."""
+    rows, cols, n = 32, 512, 48
+    w_np = np.zeros((rows, cols // 256 * 176), np.uint8)
+    blocks = w_np.reshape(rows, -1, 176)
+    blocks[:, :, 0:2] = np.array([0.01], np.float16).view(np.uint8)
+    blocks[:, :, 2:4] = np.array([0.005], np.float16).view(np.uint8)
+    blocks[:, :, 4:] = 0xFF
+    x = np.ones((n, cols), np.float32)
+    x[1::2] *= -1.0
+    x[2, ::2] *= -1.0
+    W = ops.Q4KWeight.from_ggml(w_np, cols, Q5)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    assert_fp32_parity(got, orc.mul_mat_q5k_q8k(w_np, cols, q8, orc.ORDER_DOTPROD),
+                       orc.q5k_dot_dequant_f64(w_np, cols, q8, magnitude=True), "Q5_K extremes")
+    W.free()

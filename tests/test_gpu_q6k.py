@@ -160,7 +160,7 @@ def test_q6k_rejections(ops):
     w6 = ops.Q4KWeight.from_ggml(synth.q6k_matrix(1, 64, 512), 512, Q6)
     x = torch.zeros((64, 512), device="cuda")
     with pytest.raises(MqError):
-        ops.gemm(w6, x)                                                 # matrix-core GEMM is Q4_K only
+        ops.gemm(w6, x)                                                 # the matrix-core GEMM takes Q4_K and Q5_K only
     with pytest.raises(MqError):
         ops.Q4KWeight.from_ggml(np.zeros((4, 176), np.uint8), 256, Q6)  # a Q6_K row needs 210 bytes
     w6.free()
