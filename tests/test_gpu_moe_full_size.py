@@ -115,3 +115,32 @@ def test_cfg3_layer_at_prefill_widths_on_the_grouped_gemm(layer, n):
     got = y.cpu().numpy()[pick]
     rel = np.max(np.abs(got - ref["y"]), axis=1) / np.max(np.abs(ref["y"]), axis=1)
     assert np.max(rel) <= END_TO_END_REL, np.max(rel)
+
+
+def test_prefill_width_paths_replay_from_a_graph(layer):
+    """The MoE block on the expert-grouped GEMM and the wide dense FFN, captured once and replayed several times with
+    eager work of the same entries in between: every replay returns the eager bits."""
+    import torch
+    ops, (GE, UE, DE), (SG, SU, SD), _, _, gate_inp = layer
+    n = 512
+    x = cu(synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H)))
+    logits = cu(synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E)))
+    sh = (SG, SU, SD, cu(gate_inp))
+    y_eager, ids_eager, _ = ops.moe_layer(GE, UE, DE, x, logits, K, shared=sh, silu=1)
+    f_eager = ops.ffn_swiglu(SG, SU, SD, x, 2)
+    y_eager, f_eager, ids_eager = y_eager.clone(), f_eager.clone(), ids_eager.clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        y_g, ids_g, _ = ops.moe_layer(GE, UE, DE, x, logits, K, shared=sh, silu=1)
+        f_g = ops.ffn_swiglu(SG, SU, SD, x, 2)
+    for rep in range(4):
+        y_g.zero_(), f_g.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_eager) and torch.equal(f_g, f_eager) and torch.equal(ids_g, ids_eager), f"replay {rep}"
+        # eager work of other widths through the same workspaces between the replays
+        ops.moe_layer(GE, UE, DE, x[:64], logits[:64], K, shared=sh, silu=1)
+        ops.ffn_swiglu(SG, SU, SD, x[:100], 2)
+        torch.cuda.synchronize()
