@@ -995,7 +995,7 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
 
 // Widths at which an expert product runs on the matrix-core GEMM in its expert-grouped form (see moe_gemm_applies).
 static bool moe_gemm_width(const mq_weight* w, int64_t n, int top_k) {
-    return w->type == kTypeQ4K && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
+    return (w->type == kTypeQ4K || w->type == kTypeQ5K) && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
            !(w->cols & 3) && !census.on;
 }
 
@@ -1029,7 +1029,7 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
         MQ_HIP(g.ap.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, w->nb)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, w->cols, w->cols, entries, E, (const int32_t*)g.plan.ptr,
                                                   (uint8_t*)g.ap.ptr, nullptr, 0, s));
-        MQ_HIP(launch_prefill_gemm_grouped(w->data, w->expert_bytes, nullptr, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
+        MQ_HIP(launch_prefill_gemm_grouped(w->data, w->type, w->expert_bytes, nullptr, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
                                            (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s));
         return MQ_OK;
     }
@@ -1408,7 +1408,7 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
     MQ_HIP(launch_fill_zero(hidden_dev, (size_t)n * top_k * (size_t)gate_exps->rows, s));
     MQ_HIP(launch_build_groups(ids_dev, n, top_k, gate_exps->n_experts, r.group_expert, r.group_begin, r.n_groups,
                                r.entry_token, r.entry_k, s));
-    if (moe_gemm_width(gate_exps, n, top_k) && up_exps->type == kTypeQ4K) {
+    if (moe_gemm_width(gate_exps, n, top_k)) {  // gate and up share their type
         // prefill widths: both products on the expert-grouped GEMM, SwiGLU rows scattered to their (token, slot) places
         const int64_t entries = n * top_k, E = gate_exps->n_experts, inter = gate_exps->rows, hidden = gate_exps->cols;
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
@@ -1421,9 +1421,9 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
-        MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->expert_bytes, nullptr, inter, gate_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->type, gate_exps->expert_bytes, nullptr, inter, gate_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s));
-        MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->expert_bytes, nullptr, inter, up_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->type, up_exps->expert_bytes, nullptr, inter, up_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
@@ -1461,7 +1461,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(hidden_dev, nullptr, false, 0, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
                                                   nullptr, 0, s));
         MQ_HIP(g.part.reserve((size_t)n * top_k * (size_t)hidden * sizeof(float)));
-        MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->expert_bytes, nullptr, hidden, down_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->type, down_exps->expert_bytes, nullptr, hidden, down_exps->nb,
                                            (const uint8_t*)g.ap2.ptr, entries, E, plan, true, (float*)g.part.ptr, hidden, s));
         MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, top_k, hidden, weights_dev, ids_dev, E, 0, nullptr, nullptr, y_dev, s));
         return MQ_OK;
@@ -1498,8 +1498,8 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
 // 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.  Q4_K stacks.
 static bool moe_gemm_applies(const mq_moe_layer_desc* L, const SharedExpert& sh, int64_t n) {
     const mq_weight* ge = L->gate_exps;
-    if (ge->type != kTypeQ4K || L->up_exps->type != kTypeQ4K || L->down_exps->type != kTypeQ4K) return false;
-    if (sh.gate && (sh.gate->type != kTypeQ4K || sh.down->type != kTypeQ4K)) return false;
+    auto takes = [](const mq_weight* w) { return w->type == kTypeQ4K || w->type == kTypeQ5K; };
+    if (!takes(ge) || !takes(L->up_exps) || !takes(L->down_exps)) return false;  // the shared expert has the stacks' types
     if (ge->n_experts > 4096 || (ge->rows & 3) || (ge->cols & 3)) return false;
     return n >= 256 && n * L->top_k >= 12 * ge->n_experts;
 }
@@ -1587,13 +1587,13 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         const uint8_t* shg = sh.gate ? sh.gate->data : nullptr;
         const uint8_t* shu = sh.gate ? sh.up->data : nullptr;
         const uint8_t* shd = sh.gate ? sh.down->data : nullptr;
-        MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->expert_bytes, shg, inter, L->gate_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->type, L->gate_exps->expert_bytes, shg, inter, L->gate_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, G, plan, false, gbuf, inter, s));
-        MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->type, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, G, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, G, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
-        MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
+        MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->type, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
                                            (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
         MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
         return MQ_OK;

@@ -577,9 +577,10 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
 
 // y = the plan's tiles . W_expert^T per item.  scatter == false: y [tiles * 16][ldy] in the plan's row order;
 // true: row out_row[r] of y (the per-(token, slot) rows of the down product).
-hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows, int64_t nb,
-                                       const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
-                                       float* y, int64_t ldy, hipStream_t stream) {
+hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows,
+                                       int64_t nb, const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan,
+                                       bool scatter, float* y, int64_t ldy, hipStream_t stream) {
+    if (wtype != kTypeQ4K && wtype != kTypeQ5K) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t items = moe_gemm_items_max(entries, groups_max);
     if (rowtiles == 0 || items == 0) return hipSuccess;
@@ -594,9 +595,15 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int64_t expert_bytes, c
         raised = true;
     }
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
-    hipLaunchKernelGGL(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
-                       2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
-                       (int64_t)0, plan, expert_bytes, out_row, w_shared);
+    if (wtype == kTypeQ5K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, true>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
+                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+    } else {
+        hipLaunchKernelGGL(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
+                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
+                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+    }
     return hipGetLastError();
 }
 

@@ -72,8 +72,8 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
  * (core/src/llm/matmul/q6_small_batch.h:13-92): one integer sum_g scale_g * sum (code - 32) * q8 per
  * super-block (what mq_debug_block_sums returns as dot_scaled; min_dot is 0), one fused multiply-add per block.
  * Every product entry point accepts handles of any of the three types (gate and up of one call must share
- * theirs); the matrix-core GEMM (mq_gemm_q4k) takes Q4_K and Q5_K dense matrices (its expert-grouped form and the
- * one-launch decoder Q4_K only), wide Q6_K products run through the decode kernel in passes of 16 rows.
+ * theirs); the matrix-core GEMM (mq_gemm_q4k) and its expert-grouped form take Q4_K and Q5_K (the one-launch decoder
+ * Q4_K only), wide Q6_K products run through the decode kernel in passes of 16 rows.
  * 8 = Q8_0 (fp16 d + 32 int8 codes, 34 bytes per 32 weights; core/src/llm/matmul/q8_small_batch.h:9-14): dense
  * matrices only (n_experts == 1, cols % 256 == 0, row_bytes >= cols / 32 * 34), taken by mq_mul_mat_q4k (and
  * mq_mul_mat_q4k_host, mq_debug_block_sums, the handle queries) and refused by every other entry point.  As in

@@ -148,9 +148,10 @@ def test_ffn_all_q5k(ops):
         w.free()
 
 
-@pytest.mark.parametrize("n", [1, 4, 16, 40])
+@pytest.mark.parametrize("n", [1, 4, 16, 40, 300])
 def test_moe_with_q5k_down_experts(ops, n):
-    """Routed layer with Q4_K gate/up and Q5_K down experts plus a shared expert of the same types."""
+    """Routed layer with Q4_K gate/up and Q5_K down experts plus a shared expert of the same types (300 tokens: a
+    hundred rows per expert, every product on the expert-grouped matrix-core GEMM, the Q5_K ones with its third chain)."""
     E, H, I, K = 12, 1024, 512, 4
     ge = np.stack([synth.q4k_matrix(synth.tensor_seed("moe5-g", e), I, H) for e in range(E)])
     ue = np.stack([synth.q4k_matrix(synth.tensor_seed("moe5-u", e), I, H) for e in range(E)])
@@ -187,7 +188,7 @@ def test_moe_with_q5k_down_experts(ops, n):
     gate = 1.0 / (1.0 + np.exp(-(x.astype(np.float64) @ gate_inp.astype(np.float64))))
     full = y_routed.astype(np.float64) + sh_gpu.astype(np.float64) * gate[:, None]
     rel = np.max(np.abs(y.cpu().numpy() - full), axis=1) / np.max(np.abs(full), axis=1)
-    assert np.max(rel) <= 2e-3 and np.median(rel) <= 2e-6
+    assert np.max(rel) <= 2e-3 and np.median(rel) <= (2e-6 if n < 256 else 2e-5)   # wide: the shared expert's sums in another order
     for w in (GE, UE, DE, SG, SU, SD):
         w.free()
 
