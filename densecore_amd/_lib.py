@@ -16,12 +16,16 @@ EXPORTS = [
     "mq_weight_upload", "mq_weight_upload_typed", "mq_weight_synthetic", "mq_weight_synthetic_typed", "mq_weight_type", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
     "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_mul_mat_q4k_noalloc", "mq_gemm_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
-    "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k", "mq_debug_block_sums", "mq_debug_moe_groups", "mq_debug_moe_hidden", "mq_debug_decoder_buffers",
+    "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k",
     "mq_acts_create", "mq_acts_free", "mq_acts_quantize", "mq_mul_mat_q4k_acts", "mq_swiglu_mul_mat_q4k_acts",
     "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
     "mq_decoder_create", "mq_decoder_step", "mq_decoder_status", "mq_decoder_set_patience", "mq_decoder_free",
-    "mq_debug_set_dense_lds", "mq_census_enable", "mq_census_reset", "mq_census_read",
     "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_host_malloc", "mq_host_free", "mq_memcpy_h2d_async", "mq_memcpy_d2h_async", "mq_stream_synchronize",
+]
+# every symbol include/mi355_q4k_debug.h declares (verification hooks and measurement instruments)
+DEBUG_EXPORTS = [
+    "mq_debug_block_sums", "mq_debug_moe_groups", "mq_debug_moe_hidden", "mq_debug_decoder_buffers",
+    "mq_census_enable", "mq_census_reset", "mq_census_read", "mq_debug_set_dense_lds",
 ]
 
 
@@ -111,7 +115,7 @@ def load() -> C.CDLL:
     L.mq_memcpy_h2d.argtypes = [vp, vp, sz]
     L.mq_memcpy_d2h.argtypes = [vp, vp, sz]
     L.mq_stream_synchronize.argtypes = [vp]
-    for name in EXPORTS:
+    for name in EXPORTS + DEBUG_EXPORTS:
         if name != "mq_last_error":
             getattr(L, name).restype = ci
     _lib = L

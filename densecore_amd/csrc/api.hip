@@ -1,6 +1,7 @@
 // C ABI of libmi355q4k.so (declared in include/mi355_q4k.h): argument checks, weight handles,
 // a grow-only device workspace and the sequencing of kernel launches.  No arithmetic lives here.
 #include "../../include/mi355_q4k.h"
+#include "../../include/mi355_q4k_debug.h"
 
 #include <cstdarg>
 #include <cstdio>
@@ -153,7 +154,9 @@ struct State {
 constexpr int kMaxDevices = 64;
 unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU that mq_init has seen
 
-// Launch census: a start/stop event pair bound to each matmul-kernel dispatch (see mq_census_* in the public header).
+// Launch census: a start/stop event pair bound to each dispatch of the decode matmul kernels (see mq_census_* in
+// include/mi355_q4k_debug.h).  Purely an observer: no entry point chooses its kernels by whether it is on; launches of
+// other kernels are simply not recorded.
 struct Census {
     bool on = false;
     struct Rec {
@@ -636,14 +639,14 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     if (entry.rc) return entry.rc;
     if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, nullptr, s);
     if (prefill_applies(w, n)) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
-    if (n == 1 && !census.on && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
+    if (n == 1 && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemv1_fused(w->data, w->rows, w->nb, x_dev, y_dev, waves, s));
             return MQ_OK;
         }
     }
-    if (n <= kGemvFusedMaxRows && !census.on && w->type == kTypeQ4K) {  // a few rows, short K per wave: the same with the rows' codes going through LDS
+    if (n <= kGemvFusedMaxRows && w->type == kTypeQ4K) {  // a few rows, short K per wave: the same with the rows' codes going through LDS
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, ldx, nullptr, nullptr, 0.0f, nullptr, y_dev, ldy, (int)n, false, waves, s));
@@ -719,14 +722,14 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (n == 1 && !census.on && w->type == kTypeQ4K) {  // one row, short K per wave: norm and quantizer run inside the GEMV kernel
+    if (n == 1 && w->type == kTypeQ4K) {  // one row, short K per wave: norm and quantizer run inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemv1_norm_fused(w->data, w->rows, w->nb, x_dev, delta_dev, weight_dev, eps, sum_out_dev, y_dev, waves, s));
             return MQ_OK;
         }
     }
-    if (n <= kNormFusedMaxRows && !census.on && w->type == kTypeQ4K) {
+    if (n <= kNormFusedMaxRows && w->type == kTypeQ4K) {
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, w->cols, delta_dev, weight_dev, eps, sum_out_dev, y_dev, ldy, (int)n, true,
@@ -734,7 +737,7 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
             return MQ_OK;
         }
     }
-    if (prefill_applies(w, n) && !census.on) {
+    if (prefill_applies(w, n)) {
         // prefill widths: the normalised rows as fp32, then the matrix-core GEMM (its quantizer reads them)
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)w->cols * sizeof(float)));
         MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, w->cols, eps, sum_out_dev, (float*)g.mid.ptr, nullptr, nullptr, s));
@@ -829,7 +832,7 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (prefill_applies(gate, n) && prefill_applies(down, n) && !census.on) {  // wide: the matrix-core GEMM, three times
+    if (prefill_applies(gate, n) && prefill_applies(down, n)) {  // wide: the matrix-core GEMM, three times
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
         return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, hidden, s);
     }
@@ -996,7 +999,7 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
 // Widths at which an expert product runs on the matrix-core GEMM in its expert-grouped form (see moe_gemm_applies).
 static bool moe_gemm_width(const mq_weight* w, int64_t n, int top_k) {
     return (w->type == kTypeQ4K || w->type == kTypeQ5K) && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
-           !(w->cols & 3) && !census.on;
+           !(w->cols & 3);
 }
 
 int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
@@ -1152,8 +1155,8 @@ int run_moe_gateup(const mq_weight* gate, const mq_weight* up, const SharedExper
 
 // Does the down projection of this MoE block run token-major (moe_down.hip)?
 bool token_major_down(const mq_weight* down, int64_t n, int slots) {
-    return down->type != kTypeQ80 && n <= kTokenMajorDownMaxTokens && !census.on && (down->rows & 15) == 0 &&
-           (size_t)slots * (size_t)down->nb * 64 <= 48 * 1024;
+    return down->type != kTypeQ80 && n <= kTokenMajorDownMaxTokens && (down->rows & 15) == 0 &&
+           moe_down_token_lds_bytes(slots, down->nb) <= kMoeDownTokenMaxLds;
 }
 
 // Q8_K of the hidden rows, down projection per (token, k) into g.part, then the weighted combine.
@@ -1285,7 +1288,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (prefill_applies(gate, n) && !census.on && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
+    if (prefill_applies(gate, n) && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
         return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, 0, s);
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
@@ -1545,7 +1548,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     // ids and weights go straight to the caller's buffers when it wants them
     int32_t* ids = ids_out_dev ? ids_out_dev : r.ids;
     float* wts = weights_out_dev ? weights_out_dev : r.weights;
-    if (n <= kDirectPairsMaxTokens && E <= kDecoderMaxExperts && !census.on && token_major_down(L->down_exps, n, slots)) {
+    if (n <= kDirectPairsMaxTokens && E <= kDecoderMaxExperts && token_major_down(L->down_exps, n, slots)) {
         // few tokens: two launches -- gate/up with the router and the input quantizer inside (moe_gateup.hip), down
         // with the hidden-row quantizer and the combine inside (moe_down.hip)
         MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
@@ -1564,7 +1567,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     }
     // one arrival counter, kept apart from the quantization counters (last slot of that buffer)
     if (int rc = reserve_counters(4096)) return rc;
-    if (moe_gemm_applies(L, sh, n) && !census.on) {
+    if (moe_gemm_applies(L, sh, n)) {
         // Prefill widths: the three expert products on the matrix-core GEMM in its expert-grouped form, the shared
         // expert as a dense FFN on it; per-(token, slot) rows and the combine as at the other widths.
         // The shared expert rides along as one more group of all tokens (its own weights, its own SiLU form, output slot K).

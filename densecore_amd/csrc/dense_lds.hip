@@ -81,14 +81,14 @@ __global__ void __launch_bounds__(512) dense_lds_kernel(const DenseLdsArgs p) {
         for (int c = wave; c < chunks; c += 8) {
             const uint8_t* g = p.aq + (size_t)c * 1024 + lane * 16;
             const uint32_t dst = base + (uint32_t)c * 1024u;
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
         }
         const uint32_t dbase = (uint32_t)(uintptr_t)(lds_ptr_t)d_lds;
         const int dchunks = d_floats / 64, d_live = TT * nb * 8;
         for (int c = wave; c < dchunks; c += 8) {
             const float* g = p.ad + (c * 64 + lane < d_live ? c * 64 + lane : 0);  // nothing is read past the workspace
             const uint32_t dst = dbase + (uint32_t)c * 256u;
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(dst) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
         }
     }
 

@@ -121,13 +121,13 @@ __global__ void __launch_bounds__(512, 4) grouped_lds_kernel(const MatmulArgs p)
         for (int ch = wave; ch < nb * 4; ch += 8) {
             const uint8_t* g = p.aq + a_off + (size_t)(ch >> 2) * 4096 + (size_t)(ch & 3) * 1024;
             const uint32_t dst = a_base + (uint32_t)ch * 1024u;
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
         }
         for (int c0 = wave; c0 < d_floats / 64; c0 += 8) {
             const int b = c0 * 8 + (lane >> 3);
             const float* g = p.ad + (size_t)(b < nb ? b : nb - 1) * 8 + d_row;  // the padding repeats the last super-block
             const uint32_t dst = d_base + (uint32_t)c0 * 256u;
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(dst) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
         }
 
         // A stage is ONE weight tile: with gate and up fused the stages alternate gate(b), up(b), gate(b + 1), ... so

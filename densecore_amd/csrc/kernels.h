@@ -251,6 +251,10 @@ struct MoeDownTokenArgs {
     float* y = nullptr;                // [n][rows]
 };
 hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream);
+// LDS that launch takes for `slots` hidden rows per token of nb super-blocks, and the most it may take: the one
+// predicate of the launcher and of the callers that choose between it and the expert-grouped launches.
+size_t moe_down_token_lds_bytes(int slots, int64_t nb);
+constexpr size_t kMoeDownTokenMaxLds = 48 * 1024;
 
 // ---- moe_gateup.hip --------------------------------------------------------------------------
 // Gate/up + SwiGLU with the router and the Q8_K of the layer input inside, one workgroup per (token, slot,

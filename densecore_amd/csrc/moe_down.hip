@@ -319,11 +319,13 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_rows_kernel(const MoeDow
 
 }  // namespace
 
+size_t moe_down_token_lds_bytes(int slots, int64_t nb) { return ((size_t)slots * (size_t)nb + 9) * 16 * sizeof(float); }
+
 hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) {
     if (a.n <= 0 || a.rows <= 0 || (a.rows & 15) || a.nb <= 0 || a.top_k <= 0 || a.top_k > 8) return hipErrorInvalidValue;
     const int slots = a.top_k + (a.sh_w ? 1 : 0);
-    const size_t lds = ((size_t)slots * (size_t)a.nb + 9) * 16 * sizeof(float);
-    if (lds > 48 * 1024) return hipErrorInvalidValue;
+    const size_t lds = moe_down_token_lds_bytes(slots, a.nb);
+    if (lds > kMoeDownTokenMaxLds) return hipErrorInvalidValue;
     const dim3 grid((unsigned)(a.rows / 16), (unsigned)a.n);
     if ((a.hidden == nullptr) == (a.aq == nullptr)) return hipErrorInvalidValue;  // one source of hidden rows
     MoeDownTokenArgs b = a;

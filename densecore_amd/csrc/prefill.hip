@@ -150,7 +150,7 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
         if (first + lane < copy_words) {
             const uint8_t* g = src + (size_t)(first + lane) * 16;
             const uint32_t dst = lds_base + (uint32_t)first * 16u;  // wave-uniform; lane l lands at dst + 16*l
-            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
         }
     }
 }

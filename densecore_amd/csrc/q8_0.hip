@@ -83,14 +83,18 @@ __global__ void __launch_bounds__(512) q80_matmul_kernel(const Q80MatmulArgs p) 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
     const int slot = lane & 15, kq = lane >> 4;
-    const int64_t rt = blockIdx.x;
+    int64_t rt = blockIdx.x;
     const int nb = (int)p.nb;
     const uint8_t* w = p.w;
     int first = 0, last = (int)p.n;  // activation rows this workgroup multiplies
     if (p.pair_ids) {
-        // expert-routed: workgroup column g is hidden row g = token * slots + slot alone, against the expert that the
-        // token's slot names (slots past top_k: the shared expert); rows of dropped pairs are left as they are
-        const int g = blockIdx.y, tok = g / p.slots, k = g - tok * p.slots;
+        // expert-routed: the grid is flat, workgroup = column g * rowtiles + row tile (a grid's second dimension ends
+        // at 65535, a prefill-width block has more pairs); column g is hidden row g = token * slots + slot alone,
+        // against the expert that the token's slot names (slots past top_k: the shared expert); rows of dropped
+        // pairs are left as they are
+        const uint32_t rowtiles = (uint32_t)((p.rows + 15) >> 4);
+        const int g = (int)(blockIdx.x / rowtiles), tok = g / p.slots, k = g - tok * p.slots;
+        rt = (int64_t)(blockIdx.x - (uint32_t)g * rowtiles);
         if (k < p.top_k) {
             const int e = p.pair_ids[tok * p.top_k + k];
             if (e < 0 || e >= p.n_experts) return;  // the whole workgroup, before any barrier
@@ -210,8 +214,9 @@ hipError_t launch_q80_matmul(const Q80MatmulArgs& a, hipStream_t stream) {
         return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
     const int64_t columns = a.pair_ids ? a.n : 1;
+    if (rowtiles * columns >= (int64_t)1 << 31) return hipErrorInvalidValue;
     const int waves = pick_waves(a.nb, rowtiles * columns);
-    hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)rowtiles, (unsigned)columns), dim3(64 * waves),
+    hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)(rowtiles * columns)), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0, stream, a);
     return hipGetLastError();
 }

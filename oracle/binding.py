@@ -69,6 +69,8 @@ def lib() -> C.CDLL:
         L.orc_dot_dequant_q5k_f64.restype = C.c_double
         L.orc_dot_dequant_q5k_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.orc_q80_block_bytes.restype = C.c_size_t
+        L.orc_dot_typed_q8k.restype = C.c_float
+        L.orc_dot_typed_q8k.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.orc_dot_dequant_q80_f64.restype = C.c_double
         L.orc_dot_dequant_q80_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         _lib = L
@@ -371,6 +373,20 @@ def ffn_swiglu(gate, up, down, hidden: int, inter: int, x, order=ORDER_DOTPROD, 
     return (y, mid) if want_inter else y
 
 
+def ffn_swiglu_typed(gu_type, down_type, gate, up, down, hidden: int, inter: int, x, order=ORDER_DOTPROD,
+                     silu=SILU_FAST_FMA, want_inter=False):
+    gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+    x = _c(x, np.float32)
+    n = x.shape[0]
+    y = np.zeros((n, hidden), np.float32)
+    mid = np.zeros((n, inter), np.float32)
+    rc = lib().orc_ffn_swiglu_typed(C.c_int(gu_type), C.c_int(down_type), _p(gate), _p(up), _p(down), C.c_int64(hidden),
+                                    C.c_int64(inter), _p(x), C.c_int64(n), _p(y), C.c_int(order), C.c_int(silu), _p(mid))
+    if rc:
+        raise ValueError(f"orc_ffn_swiglu_typed rc={rc}")
+    return (y, mid) if want_inter else y
+
+
 def swiglu_mul_mat(gate, up, hidden: int, inter: int, x, order=ORDER_DOTPROD, silu=SILU_EXACT):
     gate, up = _c(gate, np.uint8), _c(up, np.uint8)
     x = _c(x, np.float32)
@@ -417,12 +433,13 @@ class _MoEWeights(C.Structure):
     _fields_ = [("hidden", C.c_int64), ("inter", C.c_int64), ("n_experts", C.c_int64), ("top_k", C.c_int),
                 ("gate_exps", C.c_void_p), ("up_exps", C.c_void_p), ("down_exps", C.c_void_p),
                 ("sh_gate", C.c_void_p), ("sh_up", C.c_void_p), ("sh_down", C.c_void_p),
-                ("sh_gate_inp", C.c_void_p)]
+                ("sh_gate_inp", C.c_void_p),
+                ("gu_type", C.c_int), ("down_type", C.c_int), ("sh_gu_type", C.c_int), ("sh_down_type", C.c_int)]
 
 
-def _moe_w(gate_exps, up_exps, down_exps, hidden, inter, top_k, keep):
+def _moe_w(gate_exps, up_exps, down_exps, hidden, inter, top_k, keep, gu_type=12, down_type=12):
     n_exp = (gate_exps if gate_exps is not None else down_exps).shape[0]
-    W = _MoEWeights(hidden, inter, n_exp, top_k, None, None, None, None, None, None, None)
+    W = _MoEWeights(hidden, inter, n_exp, top_k, None, None, None, None, None, None, None, gu_type, down_type, 12, 12)
     for name, arr in (("gate_exps", gate_exps), ("up_exps", up_exps), ("down_exps", down_exps)):
         if arr is not None:
             a = _c(arr, np.uint8)
@@ -431,11 +448,12 @@ def _moe_w(gate_exps, up_exps, down_exps, hidden, inter, top_k, keep):
     return W
 
 
-def moe_gateup_swiglu(gate_exps, up_exps, hidden, inter, x, ids, order=ORDER_DOTPROD, silu=SILU_EXACT):
+def moe_gateup_swiglu(gate_exps, up_exps, hidden, inter, x, ids, order=ORDER_DOTPROD, silu=SILU_EXACT, gu_type=12):
+    """gu_type: ggml_type of both stacks (12 Q4_K, 13 Q5_K, 14 Q6_K); rows of the matching block size."""
     keep = []
     ids = _c(ids, np.int32)
     x = _c(x, np.float32)
-    W = _moe_w(gate_exps, up_exps, None, hidden, inter, ids.shape[1], keep)
+    W = _moe_w(gate_exps, up_exps, None, hidden, inter, ids.shape[1], keep, gu_type=gu_type)
     out = np.zeros((x.shape[0], ids.shape[1], inter), np.float32)
     rc = lib().orc_moe_gateup_swiglu(C.byref(W), _p(x), _p(ids), C.c_int64(x.shape[0]), C.c_int(order), C.c_int(silu),
                                      _p(out))
@@ -444,12 +462,12 @@ def moe_gateup_swiglu(gate_exps, up_exps, hidden, inter, x, ids, order=ORDER_DOT
     return out
 
 
-def moe_down_weighted(down_exps, hidden, inter, hid, ids, weights, order=ORDER_DOTPROD, accumulate_mode=0):
+def moe_down_weighted(down_exps, hidden, inter, hid, ids, weights, order=ORDER_DOTPROD, accumulate_mode=0, down_type=12):
     keep = []
     ids = _c(ids, np.int32)
     hid = _c(hid, np.float32)
     weights = _c(weights, np.float32)
-    W = _moe_w(None, None, down_exps, hidden, inter, ids.shape[1], keep)
+    W = _moe_w(None, None, down_exps, hidden, inter, ids.shape[1], keep, down_type=down_type)
     y = np.zeros((ids.shape[0], hidden), np.float32)
     rc = lib().orc_moe_down_weighted(C.byref(W), _p(hid), _p(ids), _p(weights), C.c_int64(ids.shape[0]),
                                      C.c_int(order), C.c_int(accumulate_mode), _p(y))
@@ -459,9 +477,10 @@ def moe_down_weighted(down_exps, hidden, inter, hid, ids, weights, order=ORDER_D
 
 
 def moe_layer(gate_exps, up_exps, down_exps, hidden, inter, top_k, x, logits, shared=None, order=ORDER_DOTPROD,
-              silu=SILU_EXACT, weights_mode=0, accumulate_mode=0):
+              silu=SILU_EXACT, weights_mode=0, accumulate_mode=0, types=(12, 12, 12, 12)):
     """gate_exps/up_exps: uint8 [E, inter, hidden/256*144]; down_exps: uint8 [E, hidden, inter/256*144].
     shared: None or (gate, up, down, gate_inp[hidden] or None).
+    types: ggml_type of (gate/up stacks, down stack, shared gate/up, shared down); rows of the matching block size.
     Returns dict(y, ids, weights, hidden)."""
     ge, ue, de = _c(gate_exps, np.uint8), _c(up_exps, np.uint8), _c(down_exps, np.uint8)
     x = _c(x, np.float32)
@@ -469,7 +488,7 @@ def moe_layer(gate_exps, up_exps, down_exps, hidden, inter, top_k, x, logits, sh
     n = x.shape[0]
     keep = [ge, ue, de, x, logits]
     W = _MoEWeights(hidden, inter, ge.shape[0], top_k, ge.ctypes.data, ue.ctypes.data, de.ctypes.data, None, None,
-                    None, None)
+                    None, None, *types)
     if shared is not None:
         sg, su, sd = (_c(a, np.uint8) for a in shared[:3])
         keep += [sg, su, sd]

@@ -24,8 +24,9 @@ def router_logits(w_router, h):
     return (h.astype(np.float64) @ w_router.astype(np.float64).T).astype(np.float32)
 
 
-def layer_forward(lw: dict, x, delta, cfg, silu, order=orc.ORDER_DOTPROD):
-    """One layer on host weights `lw` (ggml-layout uint8 arrays + fp32 router).  Returns the stage outputs."""
+def layer_forward(lw: dict, x, delta, cfg, silu, order=orc.ORDER_DOTPROD, fixed_logits=None):
+    """One layer on host weights `lw` (ggml-layout uint8 arrays + fp32 router).  Returns the stage outputs.
+    fixed_logits: route on these [n, n_experts] instead of on the router projection (which is still returned)."""
     H, I = cfg.hidden, cfg.inter
     x1, h = add_rmsnorm(x, delta, cfg.eps)
     qkv = orc.mul_mat_q4k_f32(lw["wqkv"], H, h, order)
@@ -33,7 +34,7 @@ def layer_forward(lw: dict, x, delta, cfg, silu, order=orc.ORDER_DOTPROD):
     x2, h2 = add_rmsnorm(x1, o, cfg.eps)
     logits = router_logits(lw["router"], h2)
     shared = (lw["sh_gate"], lw["sh_up"], lw["sh_down"], lw["sh_gate_inp"]) if "sh_gate" in lw else None
-    moe = orc.moe_layer(lw["gate_exps"], lw["up_exps"], lw["down_exps"], H, I, cfg.top_k, h2, logits, shared, order,
-                        silu, 1, 0)
+    moe = orc.moe_layer(lw["gate_exps"], lw["up_exps"], lw["down_exps"], H, I, cfg.top_k, h2,
+                        logits if fixed_logits is None else fixed_logits, shared, order, silu, 1, 0)
     return {"h": h, "qkv": qkv, "o": o, "x": x2, "h2": h2, "logits": logits, "y": moe["y"], "ids": moe["ids"],
             "weights": moe["weights"]}

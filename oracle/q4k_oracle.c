@@ -636,6 +636,46 @@ static float stable_sigmoid(float x) { /* fused_ops.cpp:451-458 */
     return z / (1.0f + z);
 }
 
+/* One row product for any of the K-quant types a stack may have. */
+float orc_dot_q5k_q8k(const void* w_row, const void* q8_row, int64_t cols, int order);
+float orc_dot_q6k_q8k(const void* w_row, const void* q8_row, int64_t cols, int order);
+float orc_dot_typed_q8k(int ggml_type, const void* w_row, const void* q8_row, int64_t cols, int order) {
+    if (ggml_type == 13) return orc_dot_q5k_q8k(w_row, q8_row, cols, order);
+    if (ggml_type == 14) return orc_dot_q6k_q8k(w_row, q8_row, cols, order);
+    return orc_dot_q4k_q8k(w_row, q8_row, cols, order);
+}
+size_t orc_row_bytes_typed(int ggml_type, int64_t cols) {
+    const size_t blocks = (size_t)(cols / ORC_QK_K);
+    return blocks * (ggml_type == 13 ? 176u : ggml_type == 14 ? 210u : sizeof(orc_block_q4k));
+}
+
+int orc_ffn_swiglu_typed(int gu_type, int down_type, const void* gate, const void* up, const void* down, int64_t hidden,
+                         int64_t inter, const float* x, int64_t n, float* y, int order, int silu_mode, float* inter_out) {
+    if (!gate || !up || !down || !x || !y || hidden <= 0 || inter <= 0 || hidden % ORC_QK_K || inter % ORC_QK_K)
+        return -1;
+    const size_t wrow_in = orc_row_bytes_typed(gu_type, hidden), wrow_mid = orc_row_bytes_typed(down_type, inter);
+    const size_t q8_in = (size_t)(hidden / ORC_QK_K) * sizeof(orc_block_q8k);
+    const size_t q8_mid = (size_t)(inter / ORC_QK_K) * sizeof(orc_block_q8k);
+    uint8_t* xq = (uint8_t*)malloc(q8_in > q8_mid ? q8_in : q8_mid);
+    float* h = (float*)malloc(sizeof(float) * (size_t)inter);
+    int rc = (xq && h) ? 0 : -2;
+    for (int64_t m = 0; rc == 0 && m < n; ++m) {
+        rc = orc_quantize_row_q8k(x + (size_t)m * hidden, xq, hidden);
+        for (int64_t r = 0; rc == 0 && r < inter; ++r) {
+            const float g = orc_dot_typed_q8k(gu_type, (const uint8_t*)gate + (size_t)r * wrow_in, xq, hidden, order);
+            const float u = orc_dot_typed_q8k(gu_type, (const uint8_t*)up + (size_t)r * wrow_in, xq, hidden, order);
+            h[r] = orc_silu_mul(g, u, silu_mode);
+        }
+        if (rc == 0 && inter_out) memcpy(inter_out + (size_t)m * inter, h, sizeof(float) * (size_t)inter);
+        if (rc == 0) rc = orc_quantize_row_q8k(h, xq, inter);
+        for (int64_t r = 0; rc == 0 && r < hidden; ++r)
+            y[(size_t)m * hidden + r] = orc_dot_typed_q8k(down_type, (const uint8_t*)down + (size_t)r * wrow_mid, xq, inter, order);
+    }
+    free(xq);
+    free(h);
+    return rc;
+}
+
 /* hidden[t][k][r] = silu(gate_e[r] . q8(x[t])) * (up_e[r] . q8(x[t])), e = ids[t][k]
  * (native.cpp:4306-4342 / hwy_moe_quant.cc:359-380; raw_batched.inl:1629-1698 for n > 4).
  * Entries whose id is outside [0, n_experts) are left untouched. */
@@ -644,7 +684,7 @@ int orc_moe_gateup_swiglu(const orc_moe_weights* w, const float* x, const int32_
     if (!w || !x || !ids || !hidden || w->hidden % ORC_QK_K) return -1;
     const int64_t H = w->hidden, I = w->inter;
     const int K = w->top_k;
-    const size_t row_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t row_in = orc_row_bytes_typed(w->gu_type, H);
     const size_t exp_in = row_in * (size_t)I;
     const size_t q8_in = (size_t)(H / ORC_QK_K) * sizeof(orc_block_q8k);
     uint8_t* xq = (uint8_t*)malloc(q8_in * (size_t)n_tokens);
@@ -658,8 +698,8 @@ int orc_moe_gateup_swiglu(const orc_moe_weights* w, const float* x, const int32_
             const uint8_t* ue = (const uint8_t*)w->up_exps + (size_t)e * exp_in;
             float* h = hidden + ((size_t)t * K + k) * (size_t)I;
             for (int64_t r = 0; r < I; ++r) {
-                const float g = orc_dot_q4k_q8k(ge + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
-                const float u = orc_dot_q4k_q8k(ue + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
+                const float g = orc_dot_typed_q8k(w->gu_type, ge + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
+                const float u = orc_dot_typed_q8k(w->gu_type, ue + (size_t)r * row_in, xq + (size_t)t * q8_in, H, order);
                 h[r] = orc_silu_mul(g, u, silu_mode);
             }
         }
@@ -676,7 +716,7 @@ int orc_moe_down_weighted(const orc_moe_weights* w, const float* hidden, const i
     if (!w || !hidden || !ids || !weights || !y || w->inter % ORC_QK_K) return -1;
     const int64_t H = w->hidden, I = w->inter, E = w->n_experts;
     const int K = w->top_k;
-    const size_t row_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q4k);
+    const size_t row_mid = orc_row_bytes_typed(w->down_type, I);
     const size_t exp_mid = row_mid * (size_t)H;
     const size_t q8_mid = (size_t)(I / ORC_QK_K) * sizeof(orc_block_q8k);
     uint8_t* hq = (uint8_t*)malloc(q8_mid * (size_t)n_tokens * K);
@@ -707,7 +747,7 @@ int orc_moe_down_weighted(const orc_moe_weights* w, const float* hidden, const i
         const uint8_t* de = (const uint8_t*)w->down_exps + (size_t)asg[a].expert * exp_mid;
         const uint8_t* q = hq + ((size_t)asg[a].token * K + asg[a].k) * q8_mid;
         for (int64_t r = 0; r < H; ++r) {
-            const float v = orc_dot_q4k_q8k(de + (size_t)r * row_mid, q, I, order);
+            const float v = orc_dot_typed_q8k(w->down_type, de + (size_t)r * row_mid, q, I, order);
             y[(size_t)asg[a].token * H + r] += v * gw;
         }
     }
@@ -723,7 +763,8 @@ int orc_moe_add_shared(const orc_moe_weights* w, const float* x, int64_t n_token
     const int64_t H = w->hidden, I = w->inter;
     float* sh = (float*)malloc(sizeof(float) * (size_t)n_tokens * (size_t)H);
     if (!sh) return -2;
-    int rc = orc_ffn_swiglu_q4k(w->sh_gate, w->sh_up, w->sh_down, H, I, x, n_tokens, sh, order, ORC_SILU_FAST_FMA, NULL);
+    int rc = orc_ffn_swiglu_typed(w->sh_gu_type, w->sh_down_type, w->sh_gate, w->sh_up, w->sh_down, H, I, x, n_tokens, sh,
+                                  order, ORC_SILU_FAST_FMA, NULL);
     for (int64_t t = 0; rc == 0 && t < n_tokens; ++t) {
         float scale = 1.0f;
         if (w->sh_gate_inp) {

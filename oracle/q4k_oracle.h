@@ -157,7 +157,19 @@ typedef struct {
     const void* sh_up;
     const void* sh_down;
     const float* sh_gate_inp; /* [hidden] fp32 scalar-gate vector, may be NULL */
+    /* ggml_type of the stacks: 12 = Q4_K, 13 = Q5_K, 14 = Q6_K; 0 reads as Q4_K.  The loader admits Q4_K / Q5_K gate and
+     * up stacks and Q4_K / Q5_K / Q6_K / Q8_0 down stacks (core/src/llm/moe/native.cpp:4611-4620); one template multiplies
+     * the first two (hwy_moe_quant.cc:145-258), ComputeQ6KQ8K the third (core/src/llm/matmul/q6_small_batch.h:13-92). */
+    int gu_type, down_type, sh_gu_type, sh_down_type;
 } orc_moe_weights;
+
+/* Row product of a K-quant weight row of the given ggml_type (12, 13, 14; 0 = 12) with a Q8_K row, and the bytes of
+ * such a weight row. */
+float orc_dot_typed_q8k(int ggml_type, const void* w_row, const void* q8_row, int64_t cols, int order);
+size_t orc_row_bytes_typed(int ggml_type, int64_t cols);
+/* y = down(silu(gate x) * (up x)) with gate/up of gu_type and down of down_type. */
+int orc_ffn_swiglu_typed(int gu_type, int down_type, const void* gate, const void* up, const void* down, int64_t hidden,
+                         int64_t inter, const float* x, int64_t n, float* y, int order, int silu_mode, float* inter_out);
 
 int orc_moe_gateup_swiglu(const orc_moe_weights* w, const float* x, const int32_t* ids, int64_t n_tokens, int order,
                           int silu_mode, float* hidden /* [n][top_k][inter] */);

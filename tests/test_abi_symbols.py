@@ -18,11 +18,13 @@ def declared_symbols(header="mi355_q4k.h"):
 
 def test_header_and_loader_agree():
     assert declared_symbols() == sorted(_lib.EXPORTS)
+    assert declared_symbols("mi355_q4k_debug.h") == sorted(_lib.DEBUG_EXPORTS)
+    assert not [s for s in declared_symbols() if s.startswith(("mq_debug", "mq_census"))], "instruments belong in the debug header"
 
 
 def test_library_exports_every_declared_symbol():
     L = _lib.load()
-    for name in declared_symbols():
+    for name in declared_symbols() + declared_symbols("mi355_q4k_debug.h"):
         assert hasattr(L, name), name
 
 

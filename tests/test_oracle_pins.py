@@ -630,6 +630,80 @@ def test_q6k_fp32_orders_against_double(cols):
         assert np.max(np.abs(got - ref)[ok] / np.abs(ref)[ok]) < 1e-4
 
 
+# ----------------------------------------------------------------- expert stacks of the sibling types
+def np_dequant_typed(w, cols, t):
+    """Independent numpy dequantization of Q4_K / Q5_K / Q6_K rows in double."""
+    if t == 14:
+        d, sc, q = np_unpack_q6k(w)
+        return (d[:, None, None] * sc.reshape(-1, 16)[:, :, None] * (q - 32).reshape(-1, 16, 16)).reshape(w.shape[0], cols)
+    d, dmin, sc, mn, q = np_unpack_q5k(w) if t == 13 else np_unpack_q4k(w)
+    return (d[:, None, None] * sc[:, :, None] * q.reshape(-1, 8, 32) - dmin[:, None, None] * mn[:, :, None]).reshape(
+        w.shape[0], cols)
+
+
+@pytest.mark.parametrize("types", [(13, 13, 13, 13), (13, 14, 12, 14), (12, 14, 13, 12), (14, 12, 12, 12)])
+def test_tiny_moe_layer_with_typed_stacks_against_double_brute_force(types):
+    """The MoE layer with gate/up, down and shared-expert stacks of Q5_K / Q6_K (what the loader admits,
+    core/src/llm/moe/native.cpp:4611-4620): every stage against numpy's own decode of the blocks in double."""
+    H, I, E, K, n = 256, 512, 5, 3, 4
+    gen = {12: synth.q4k_matrix, 13: synth.q5k_matrix, 14: synth.q6k_matrix}
+    gu, dn, sgu, sdn = types
+    ge = np.stack([gen[gu](synth.tensor_seed("tg", e), I, H) for e in range(E)])
+    ue = np.stack([gen[gu](synth.tensor_seed("tu", e), I, H) for e in range(E)])
+    de = np.stack([gen[dn](synth.tensor_seed("td", e), H, I) for e in range(E)])
+    sh = (gen[sgu](171, I, H), gen[sgu](172, I, H), gen[sdn](173, H, I), synth.normal_f32(174, (H,)) * np.float32(0.05))
+    x = synth.normal_f32(175, (n, H))
+    logits = synth.normal_f32(176, (n, E))
+    r = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=sh, silu=orc.SILU_EXACT, types=types)
+    ids, wts = orc.route_topk(logits, K, 0)
+    assert np.array_equal(r["ids"], ids)
+    hid = orc.moe_gateup_swiglu(ge, ue, H, I, x, ids, silu=orc.SILU_EXACT, gu_type=gu)
+    assert np.array_equal(hid.view(np.uint32), r["hidden"].view(np.uint32))
+    xq = np_q8_dequant(x)
+    y = np.zeros((n, H))
+    for t in range(n):
+        for k in range(K):
+            e = ids[t, k]
+            g = np_dequant_typed(ge[e], H, gu) @ xq[t]
+            u = np_dequant_typed(ue[e], H, gu) @ xq[t]
+            h = g / (1 + np.exp(-g)) * u
+            assert np.allclose(hid[t, k], h, rtol=2e-4, atol=1e-5 * np.abs(h).max())
+            hq = np_q8_dequant(hid[t, k][None, :])[0]
+            y[t] += wts[t, k] * (np_dequant_typed(de[e], I, dn) @ hq)
+    routed = orc.moe_down_weighted(de, H, I, hid, ids, wts, down_type=dn)
+    assert np.max(np.abs(routed - y)) < 1e-5 * np.abs(y).max()
+    r2 = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=None, silu=orc.SILU_EXACT, types=types)
+    assert np.array_equal(r2["y"].view(np.uint32), routed.view(np.uint32))
+    # shared expert: the typed dense FFN against the same decode
+    ysh, mid = orc.ffn_swiglu_typed(sgu, sdn, sh[0], sh[1], sh[2], H, I, x, silu=orc.SILU_EXACT, want_inter=True)
+    g = xq @ np_dequant_typed(sh[0], H, sgu).T
+    u = xq @ np_dequant_typed(sh[1], H, sgu).T
+    hs = g / (1 + np.exp(-g)) * u
+    assert np.allclose(mid, hs, rtol=2e-4, atol=1e-5 * np.abs(hs).max())
+    want_sh = np_q8_dequant(mid) @ np_dequant_typed(sh[2], I, sdn).T
+    assert np.max(np.abs(ysh - want_sh)) < 1e-5 * np.abs(want_sh).max()
+    # the layer's own shared expert uses the fast-exp SiLU (~1e-3 off the exact one): looser end to end
+    gate = 1 / (1 + np.exp(-(x.astype(np.float64) @ sh[3].astype(np.float64))))
+    y_full = y + (np_q8_dequant(hs.astype(np.float32)) @ np_dequant_typed(sh[2], I, sdn).T) * gate[:, None]
+    assert np.max(np.abs(r["y"] - y_full)) < 5e-3 * np.abs(y_full).max()
+
+
+def test_typed_layer_with_q4k_types_is_bitwise_the_q4k_layer():
+    """Stacks declared Q4_K go through the typed row product and the typed shared-expert FFN: the same bits as the
+    plain Q4_K functions they stand beside."""
+    H, I, E, K, n = 256, 256, 4, 2, 3
+    ge, ue, de = (np.stack([synth.q4k_matrix(synth.tensor_seed(nm, e), r, c) for e in range(E)])
+                  for nm, r, c in (("g", I, H), ("u", I, H), ("d", H, I)))
+    sh = (synth.q4k_matrix(71, I, H), synth.q4k_matrix(72, I, H), synth.q4k_matrix(73, H, I), None)
+    x = synth.normal_f32(75, (n, H))
+    logits = synth.normal_f32(76, (n, E))
+    want = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=sh, silu=orc.SILU_FAST)["y"]
+    routed = orc.moe_layer(ge, ue, de, H, I, K, x, logits, shared=None, silu=orc.SILU_FAST)["y"]
+    shy = orc.ffn_swiglu(sh[0], sh[1], sh[2], H, I, x, silu=orc.SILU_FAST_FMA)
+    assert np.array_equal((routed + shy).view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(orc.ffn_swiglu_typed(12, 12, sh[0], sh[1], sh[2], H, I, x).view(np.uint32), shy.view(np.uint32))
+
+
 # ---------------------------------------------------------------- Q8_0 x Q8_0 (core/src/llm/matmul/q8_small_batch.h)
 def np_unpack_q80(rows_u8: np.ndarray):
     """-> (d float64 [rows, blocks], codes int64 [rows, blocks, 32]) by an independent numpy decode."""
