@@ -1498,11 +1498,14 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
 
 // The expert-grouped GEMM pays from a dozen routed rows per expert on average (its workgroups multiply 16-row tiles, up to
 // eight of an expert at a time): 256 experts, top-8, 2048 x 512: 242 against 250 us per block at 384 tokens, 262 against
-// 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.  Q4_K stacks.
-static bool moe_gemm_applies(const mq_moe_layer_desc* L, const SharedExpert& sh, int64_t n) {
+// 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.
+// Decided per product: gate / up (one type) and down each run on it when their type is one it takes; a Q4_K_M-style
+// layer (Q4_K or Q5_K gate / up with a Q6_K or Q8_0 down stack, core/src/llm/moe/native.cpp:4611-4620) keeps its two
+// large products on the matrix cores and sends the fp32 hidden rows through the expert-grouped decode launches.
+static bool moe_gemm_takes(const mq_weight* w) { return w->type == kTypeQ4K || w->type == kTypeQ5K; }
+static bool moe_gemm_applies(const mq_moe_layer_desc* L, int64_t n) {
     const mq_weight* ge = L->gate_exps;
-    auto takes = [](const mq_weight* w) { return w->type == kTypeQ4K || w->type == kTypeQ5K; };
-    if (!takes(ge) || !takes(L->up_exps) || !takes(L->down_exps)) return false;  // the shared expert has the stacks' types
+    if (!moe_gemm_takes(ge) || !moe_gemm_takes(L->up_exps)) return false;  // the shared expert has the stacks' types
     if (ge->n_experts > 4096 || (ge->rows & 3) || (ge->cols & 3)) return false;
     return n >= 256 && n * L->top_k >= 12 * ge->n_experts;
 }
@@ -1567,7 +1570,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
     }
     // one arrival counter, kept apart from the quantization counters (last slot of that buffer)
     if (int rc = reserve_counters(4096)) return rc;
-    if (moe_gemm_applies(L, sh, n)) {
+    if (moe_gemm_applies(L, n)) {
         // Prefill widths: the three expert products on the matrix-core GEMM in its expert-grouped form, the shared
         // expert as a dense FFN on it; per-(token, slot) rows and the combine as at the other widths.
         // The shared expert rides along as one more group of all tokens (its own weights, its own SiLU form, output slot K).
@@ -1595,6 +1598,15 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->type, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, G, plan, false, ubuf, inter, s));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
+        if (!moe_gemm_takes(L->down_exps)) {
+            // a down stack of a type the GEMM does not take: the SwiGLU rows leave the quantizer as fp32 at their
+            // (token, slot) places as well, and the expert-grouped decode launches take them from there (their own
+            // quantizer -- Q8_K, or Q8_0 for Q8_0 experts -- and the same combine)
+            MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
+            MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, G, plan, (uint8_t*)g.ap2.ptr,
+                                                      (float*)g.mid.ptr, inter, s));
+            return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, false, n, K, slots, r, ids, wts, L->sh_gate_inp_dev, x_dev, y_dev, s);
+        }
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, G, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
         MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->type, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
                                            (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
