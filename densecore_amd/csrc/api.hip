@@ -538,7 +538,7 @@ constexpr int64_t kPrefillMinRows = 48;
 constexpr int64_t kPrefillMinRowsLarge = 17;
 constexpr int64_t kPrefillLargeBytes = 24ll << 20;
 static bool prefill_applies(const mq_weight* w, int64_t n) {
-    if (w->type != kTypeQ4K && w->type != kTypeQ5K) return false;
+    if (w->type != kTypeQ4K && w->type != kTypeQ5K && w->type != kTypeQ6K) return false;
     return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->type == kTypeQ4K && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
 }
 constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
@@ -616,8 +616,8 @@ int mq_gemm_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, 
     if (int rc = check_ready()) return rc;
     if (int rc = check_weight(w, "mq_gemm_q4k")) return rc;
     if (w->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: weight is an expert stack");
-    if (w->type != kTypeQ4K && w->type != kTypeQ5K)
-        return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K and Q5_K weights only");
+    if (w->type != kTypeQ4K && w->type != kTypeQ5K && w->type != kTypeQ6K)
+        return fail(MQ_ERR_UNSUPPORTED, "mq_gemm_q4k: the matrix-core GEMM takes Q4_K, Q5_K and Q6_K weights only");
     if (int rc = check_x(x_dev, n, ldx, w->cols, "mq_gemm_q4k")) return rc;
     if (n == 0) return MQ_OK;
     if (!y_dev || ldy < w->rows) return fail(MQ_ERR_INVALID, "mq_gemm_q4k: null output or ldy < rows");
@@ -998,7 +998,7 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
 
 // Widths at which an expert product runs on the matrix-core GEMM in its expert-grouped form (see moe_gemm_applies).
 static bool moe_gemm_width(const mq_weight* w, int64_t n, int top_k) {
-    return (w->type == kTypeQ4K || w->type == kTypeQ5K) && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
+    return (w->type == kTypeQ4K || w->type == kTypeQ5K || w->type == kTypeQ6K) && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
            !(w->cols & 3);
 }
 
@@ -1499,10 +1499,10 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
 // The expert-grouped GEMM pays from a dozen routed rows per expert on average (its workgroups multiply 16-row tiles, up to
 // eight of an expert at a time): 256 experts, top-8, 2048 x 512: 242 against 250 us per block at 384 tokens, 262 against
 // 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.
-// Decided per product: gate / up (one type) and down each run on it when their type is one it takes; a Q4_K_M-style
-// layer (Q4_K or Q5_K gate / up with a Q6_K or Q8_0 down stack, core/src/llm/moe/native.cpp:4611-4620) keeps its two
-// large products on the matrix cores and sends the fp32 hidden rows through the expert-grouped decode launches.
-static bool moe_gemm_takes(const mq_weight* w) { return w->type == kTypeQ4K || w->type == kTypeQ5K; }
+// Decided per product: gate / up (one type) and down each run on it when their type is one it takes; a layer with
+// a Q8_0 down stack (core/src/llm/moe/native.cpp:4611-4620; its activations are Q8_0 as well) keeps its two large
+// products on the matrix cores and sends the fp32 hidden rows through the Q8_0 launches.
+static bool moe_gemm_takes(const mq_weight* w) { return w->type == kTypeQ4K || w->type == kTypeQ5K || w->type == kTypeQ6K; }
 static bool moe_gemm_applies(const mq_moe_layer_desc* L, int64_t n) {
     const mq_weight* ge = L->gate_exps;
     if (!moe_gemm_takes(ge) || !moe_gemm_takes(L->up_exps)) return false;  // the shared expert has the stacks' types

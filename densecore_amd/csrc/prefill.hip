@@ -129,6 +129,93 @@ __device__ __forceinline__ void expand_tile(const v4u seg0, const v4u seg1, cons
     t.dmin = half_bits_to_float(hdr.x >> 16);
 }
 
+// ---- Q6_K on the matrix cores ---------------------------------------------------------------------------------
+// weight = d * scale_g * (code - 32): sixteen signed 8-bit scales per super-block, one per 16 weights, six-bit codes
+// (core/src/llm/matmul/q6_small_batch.h:13-92).  scale * (code - 32) reaches 4096, so both factors are cut in two:
+//     scale + 128 = u = 16 u1 + u0   (u1, u0 in 0..15)          code - 32 = c = 8 c1 + c0   (c0 in 0..7, c1 in -4..3)
+//     sum_g scale_g sum_i c_i q_i = 128 P11 + 16 P10 + 8 P01 + P00 - 128 R,
+//     Pjk = sum_i (u_j c_k)_i q_i,  R = sum_i c_i q_i
+// exactly, in int32: every byte u_j * c_k lies in [-60, 105] and c itself in [-32, 31] (the chain R multiplies
+// 4 c, the tile's own bytes, and enters with -32).  Five chains of four K = 64 MFMAs per 16 x 16 outputs and
+// super-block, no term from the activations' block sums, so the activation tiles are the Q4_K kernel's: the tile
+// keeps each 64-byte run of low / high nibbles as two 32-weight sub-blocks (4 j + z and 4 j + z + 2 for the low and
+// high nibbles of one byte), the pairs the P-major layout puts side by side.
+// u_j * c1 for a signed c1 comes bytewise from the unsigned product with d1 = c1 + 4 = code >> 3:
+//     u c1 = u d1 - 4 u,   ((u d1 | 0x80) - 4 u) ^ 0x80 per byte (u d1 <= 105 < 128, 4 u <= 60: no borrow).
+struct WTile6 {
+    v4i p11[4], p10[4], p01[4], p00[4], r4[4];
+    float d;
+};
+
+__device__ __forceinline__ uint32_t signed_digit_bytes(uint32_t prod, uint32_t four_u) {
+    return ((prod | 0x80808080u) - four_u) ^ 0x80808080u;
+}
+
+__device__ __forceinline__ void expand_tile6(const v4u ql0, const v4u ql1, const v4u qh, const v4u sc, uint32_t dw, int kq, WTile6& t) {
+    const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+    uint32_t u1w[4], u0w[4], f1w[4], f0w[4];  // digits of the sixteen scales, and four times the digits
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t u = scw[w] ^ 0x80808080u;  // scale + 128, bytewise
+        u1w[w] = (u >> 4) & 0x0f0f0f0fu;
+        u0w[w] = u & 0x0f0f0f0fu;
+        f1w[w] = u1w[w] << 2;
+        f0w[w] = u0w[w] << 2;
+    }
+    // weights 128 j + 32 z + l, l = 8 kq .. 8 kq + 7, have scale 8 j + 2 z + (kq >> 1): byte 2 (z & 1) + (kq >> 1) of
+    // scale word 2 j + (z >> 1)
+    const uint32_t sel = (uint32_t)(kq >> 1);
+    const v4u qlw[2] = {ql0, ql1};
+    const uint32_t qhw[4] = {qh.x, qh.y, qh.z, qh.w};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int zp = 0; zp < 2; ++zp) {  // B operand jj = 2 j + zp: sub-blocks z = zp (dwords 0, 1) and z = zp + 2 (dwords 2, 3)
+            const int jj = 2 * j + zp;
+            const uint32_t k = 2u * (uint32_t)zp + sel;
+            // the two sub-blocks' digits as 16-bit numbers side by side (low half: z = zp, high half: z = zp + 2)
+            const uint32_t pick = 0x0c040c00u + k * 0x00010001u;
+            const uint32_t d1p = __builtin_amdgcn_perm(u1w[2 * j + 1], u1w[2 * j], pick);
+            const uint32_t d0p = __builtin_amdgcn_perm(u0w[2 * j + 1], u0w[2 * j], pick);
+            const uint32_t spread = k * 0x01010101u;  // byte k in all four bytes
+            const uint32_t f1[2] = {__builtin_amdgcn_perm(0u, f1w[2 * j], spread), __builtin_amdgcn_perm(0u, f1w[2 * j + 1], spread)};
+            const uint32_t f0[2] = {__builtin_amdgcn_perm(0u, f0w[2 * j], spread), __builtin_amdgcn_perm(0u, f0w[2 * j + 1], spread)};
+            const uint32_t src[2] = {zp ? qlw[j].z : qlw[j].x, zp ? qlw[j].w : qlw[j].y};
+            uint32_t r4[4], p11[4], p10[4], p01[4], p00[4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {      // h = 0: z = zp (low nibbles), h = 1: z = zp + 2 (high nibbles)
+                const int z = zp + 2 * h;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {  // the lane's eight weights of the sub-block, four to a word
+                    const uint32_t nib = (h ? src[i] >> 2 : src[i] << 2) & 0x3c3c3c3cu;
+                    const uint32_t hi = qhw[2 * j + i];
+                    const uint32_t top = (z == 3 ? hi : hi << (6 - 2 * z)) & 0xc0c0c0c0u;
+                    const uint32_t b4 = top | nib;              // 4 (code - 32) as signed bytes
+                    const uint32_t code4 = b4 ^ 0x80808080u;    // 4 code
+                    const uint32_t d1 = (code4 >> 5) & 0x07070707u, c0 = (code4 >> 2) & 0x07070707u;
+                    const int o = 2 * h + i;
+                    r4[o] = b4;
+                    if (h == 0) {
+                        p10[o] = scale_bytes<0>(c0, d1p), p00[o] = scale_bytes<0>(c0, d0p);
+                        p11[o] = signed_digit_bytes(scale_bytes<0>(d1, d1p), f1[0]);
+                        p01[o] = signed_digit_bytes(scale_bytes<0>(d1, d0p), f0[0]);
+                    } else {
+                        p10[o] = scale_bytes<1>(c0, d1p), p00[o] = scale_bytes<1>(c0, d0p);
+                        p11[o] = signed_digit_bytes(scale_bytes<1>(d1, d1p), f1[1]);
+                        p01[o] = signed_digit_bytes(scale_bytes<1>(d1, d0p), f0[1]);
+                    }
+                }
+            }
+            t.r4[jj] = v4i{(int)r4[0], (int)r4[1], (int)r4[2], (int)r4[3]};
+            t.p11[jj] = v4i{(int)p11[0], (int)p11[1], (int)p11[2], (int)p11[3]};
+            t.p10[jj] = v4i{(int)p10[0], (int)p10[1], (int)p10[2], (int)p10[3]};
+            t.p01[jj] = v4i{(int)p01[0], (int)p01[1], (int)p01[2], (int)p01[3]};
+            t.p00[jj] = v4i{(int)p00[0], (int)p00[1], (int)p00[2], (int)p00[3]};
+        }
+    }
+    t.d = half_bits_to_float(dw & 0xffffu);
+}
+
 typedef __attribute__((address_space(1))) const void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -157,7 +244,7 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
 
 // kWTilesPerWave = 2: the 128 x 128 workgroup tile above.  1: 64 weight rows per workgroup, for launches whose
 // 128-row workgroups would leave compute units without their two workgroups (M up to a few hundred).
-template <int kWTilesPerWave, bool Q5 = false>
+template <int kWTilesPerWave, int WT = kWtQ4>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
@@ -166,6 +253,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                                                            const uint8_t* __restrict__ w_shared) {
     extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
+    constexpr bool Q5 = WT == kWtQ5, Q6 = WT == kWtQ6;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -207,15 +295,23 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     // registers.  One workgroup barrier per super-block.
     v4u seg0[kWTilesPerWave], seg1[kWTilesPerWave], hdr[kWTilesPerWave];
     v2u qh[kWTilesPerWave];
+    v4u qh6[kWTilesPerWave];      // Q6_K: the top two bits of the codes; seg0 / seg1 hold its nibbles, hdr its sixteen scales
+    uint32_t d6[kWTilesPerWave];  // Q6_K: fp16 d
     auto request_w = [&](int64_t b) {
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
-            const uint8_t* tile = w + tile_offset(rt[t], b, nb, Q5 ? kTile5Bytes : kTileBytes);
+            const uint8_t* tile = w + tile_offset(rt[t], b, nb, tile_stride<WT>());
             seg0[t] = load16(tile + lane * 16);
             seg1[t] = load16(tile + 1024 + lane * 16);
-            hdr[t] = load16(tile + kTileQBytes + r * 16);
-            if (Q5) qh[t] = *reinterpret_cast<const v2u*>(tile + kTileHBytes + lane * 8);
-            else qh[t] = v2u{0u, 0u};
+            if constexpr (Q6) {
+                qh6[t] = load16(tile + kTile6HOff + lane * 16);
+                hdr[t] = load16(tile + kTile6SOff + r * 16);
+                d6[t] = *reinterpret_cast<const uint32_t*>(tile + kTile6DOff + r * 4);
+            } else {
+                hdr[t] = load16(tile + kTileQBytes + r * 16);
+                if (Q5) qh[t] = *reinterpret_cast<const v2u*>(tile + kTileHBytes + lane * 8);
+                else qh[t] = v2u{0u, 0u};
+            }
         }
     };
     // K split over grid.z: this workgroup multiplies the super-blocks [b_begin, b_end) and writes its sums to
@@ -232,9 +328,12 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         // ... and after the barrier so has everybody else's share of the activation tiles; every wave
         // is also done reading the other buffer (super-block b-1), which the next requests overwrite
         __syncthreads();
-        WTile wt[kWTilesPerWave];
+        std::conditional_t<Q6, WTile6, WTile> wt[kWTilesPerWave];
 #pragma unroll
-        for (int t = 0; t < kWTilesPerWave; ++t) expand_tile<Q5>(seg0[t], seg1[t], hdr[t], qh[t], kq, wt[t]);
+        for (int t = 0; t < kWTilesPerWave; ++t) {
+            if constexpr (Q6) expand_tile6(seg0[t], seg1[t], qh6[t], hdr[t], d6[t], kq, wt[t]);
+            else expand_tile<Q5>(seg0[t], seg1[t], hdr[t], qh[t], kq, wt[t]);
+        }
         if (b + 1 < b_end) {
             request_a_tiles(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
             request_w(b + 1);
@@ -248,38 +347,69 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                 v4i a[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
-                const v8h dg = *reinterpret_cast<const v8h*>(at + digit_off);
                 const float4 yd = *reinterpret_cast<const float4*>(at + kPScaleOff + kq * 16);
                 const v4i zero = {0, 0, 0, 0};
-                const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
-                v4i hi[kWTilesPerWave], lo[kWTilesPerWave], fb[kWTilesPerWave];
-                v4f mn[kWTilesPerWave];
-#pragma unroll
-                for (int t = 0; t < kWTilesPerWave; ++t) {
-                    hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].hi[0], zero, 0, 0, 0);
-                    lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].lo[0], zero, 0, 0, 0);
-                    if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].b5[0], zero, 0, 0, 0);
-                    mn[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt[t].mins, zero_f, 0, 0, 0);
-                }
-#pragma unroll
-                for (int j = 1; j < 4; ++j)
+                const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+                if constexpr (Q6) {
+                    v4i p11[kWTilesPerWave], p10[kWTilesPerWave], p01[kWTilesPerWave], p00[kWTilesPerWave], r4[kWTilesPerWave];
 #pragma unroll
                     for (int t = 0; t < kWTilesPerWave; ++t) {
-                        hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].hi[j], hi[t], 0, 0, 0);
-                        lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].lo[j], lo[t], 0, 0, 0);
-                        if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].b5[j], fb[t], 0, 0, 0);
+                        p11[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].p11[0], zero, 0, 0, 0);
+                        p10[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].p10[0], zero, 0, 0, 0);
+                        p01[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].p01[0], zero, 0, 0, 0);
+                        p00[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].p00[0], zero, 0, 0, 0);
+                        r4[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].r4[0], zero, 0, 0, 0);
                     }
-                const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
 #pragma unroll
-                for (int t = 0; t < kWTilesPerWave; ++t)
+                    for (int j = 1; j < 4; ++j)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        int dot = hi[t][i] * 8 + lo[t][i];
-                        if (Q5) dot += fb[t][i] * 16;
-                        // yd * (d * dot - dmin * min_dot): three fp32 operations per output and super-block
-                        const float v = __fmaf_rn(-wt[t].dmin, mn[t][i], __fmul_rn(wt[t].d, (float)dot));
-                        acc[t][m][i] = __fmaf_rn(ydv[i], v, acc[t][m][i]);
+                        for (int t = 0; t < kWTilesPerWave; ++t) {
+                            p11[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].p11[j], p11[t], 0, 0, 0);
+                            p10[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].p10[j], p10[t], 0, 0, 0);
+                            p01[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].p01[j], p01[t], 0, 0, 0);
+                            p00[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].p00[j], p00[t], 0, 0, 0);
+                            r4[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].r4[j], r4[t], 0, 0, 0);
+                        }
+#pragma unroll
+                    for (int t = 0; t < kWTilesPerWave; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            // sum_g scale_g sum (code - 32) q8, the integer of the reference's kernel, then its one fused
+                            // multiply-add per block (core/src/llm/matmul/q6_small_batch.h:84-86)
+                            const int isum = p11[t][i] * 128 + p10[t][i] * 16 + p01[t][i] * 8 + p00[t][i] - r4[t][i] * 32;
+                            acc[t][m][i] = __fmaf_rn(__fmul_rn(ydv[i], wt[t].d), (float)isum, acc[t][m][i]);
+                        }
+                } else {
+                    const v8h dg = *reinterpret_cast<const v8h*>(at + digit_off);
+                    const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
+                    v4i hi[kWTilesPerWave], lo[kWTilesPerWave], fb[kWTilesPerWave];
+                    v4f mn[kWTilesPerWave];
+#pragma unroll
+                    for (int t = 0; t < kWTilesPerWave; ++t) {
+                        hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].hi[0], zero, 0, 0, 0);
+                        lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].lo[0], zero, 0, 0, 0);
+                        if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], wt[t].b5[0], zero, 0, 0, 0);
+                        mn[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt[t].mins, zero_f, 0, 0, 0);
                     }
+#pragma unroll
+                    for (int j = 1; j < 4; ++j)
+#pragma unroll
+                        for (int t = 0; t < kWTilesPerWave; ++t) {
+                            hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].hi[j], hi[t], 0, 0, 0);
+                            lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].lo[j], lo[t], 0, 0, 0);
+                            if (Q5) fb[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], wt[t].b5[j], fb[t], 0, 0, 0);
+                        }
+#pragma unroll
+                    for (int t = 0; t < kWTilesPerWave; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            int dot = hi[t][i] * 8 + lo[t][i];
+                            if (Q5) dot += fb[t][i] * 16;
+                            // yd * (d * dot - dmin * min_dot): three fp32 operations per output and super-block
+                            const float v = __fmaf_rn(-wt[t].dmin, mn[t][i], __fmul_rn(wt[t].d, (float)dot));
+                            acc[t][m][i] = __fmaf_rn(ydv[i], v, acc[t][m][i]);
+                        }
+                }
             }
         }
     }
@@ -415,14 +545,14 @@ struct PrefillShape {
     int splits, sb_split;
     unsigned row_wgs, groups;
 };
-PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n, bool q5 = false) {
+PrefillShape prefill_shape(int64_t rows, int64_t nb, int64_t n, bool one_tile_per_wave = false) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
     PrefillShape ps;
     ps.groups = (unsigned)((m_tiles + kMTilesPerGroup - 1) / kMTilesPerGroup);
     // two workgroups fit a compute unit: while the 128-row workgroups would not even give every unit one, 64-row
     // ones fill the chip better (14336 rows on 256 units: up to M = 256; 52 -> 40 us at M = 128, 55 -> 51 at 256,
     // and 76 -> 79, 78 -> 91 at M = 384, 512, where the wide ones stay)
-    ps.narrow = q5 || ((rowtiles + 7) / 8) * (int64_t)ps.groups <= (int64_t)compute_units();  // Q5_K: its third operand set only fits the registers of 64-row workgroups
+    ps.narrow = one_tile_per_wave || ((rowtiles + 7) / 8) * (int64_t)ps.groups <= (int64_t)compute_units();  // Q5_K, Q6_K: their operand sets only fit the registers of 64-row workgroups
     ps.row_wgs = (unsigned)(ps.narrow ? (rowtiles + 3) / 4 : (rowtiles + 7) / 8);
     const int64_t wgs = (int64_t)ps.row_wgs * ps.groups;
     int splits = (int)(2 * (int64_t)compute_units() / (wgs > 0 ? wgs : 1));
@@ -580,7 +710,7 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
 hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows,
                                        int64_t nb, const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan,
                                        bool scatter, float* y, int64_t ldy, hipStream_t stream) {
-    if (wtype != kTypeQ4K && wtype != kTypeQ5K) return hipErrorInvalidValue;
+    if (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t items = moe_gemm_items_max(entries, groups_max);
     if (rowtiles == 0 || items == 0) return hipSuccess;
@@ -588,15 +718,19 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expe
     static bool raised = false;
     if (!raised) {
         for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>),
-                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, true>)}) {
+                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, kWtQ5>), reinterpret_cast<const void*>(&prefill_gemm_kernel<1, kWtQ6>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
             if (e != hipSuccess) return e;
         }
         raised = true;
     }
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
-    if (wtype == kTypeQ5K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, true>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+    if (wtype == kTypeQ6K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ6>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
+                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+    } else if (wtype == kTypeQ5K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ5>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
                            2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
                            (int64_t)0, plan, expert_bytes, out_row, w_shared);
     } else {
@@ -608,7 +742,7 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expe
 }
 
 size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype) {
-    const PrefillShape ps = prefill_shape(rows, nb, n, wtype == kTypeQ5K);
+    const PrefillShape ps = prefill_shape(rows, nb, n, wtype != kTypeQ4K);
     return ps.splits > 1 ? (size_t)ps.splits * (size_t)n * (size_t)rows * sizeof(float) : 0;
 }
 
@@ -640,14 +774,14 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
                                int64_t ldy, float* part, hipStream_t stream) {
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
     if (rowtiles == 0 || m_tiles == 0) return hipSuccess;
-    if (wtype != kTypeQ4K && wtype != kTypeQ5K) return hipErrorInvalidValue;
-    const PrefillShape ps = prefill_shape(rows, nb, n, wtype == kTypeQ5K);
+    if (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K) return hipErrorInvalidValue;
+    const PrefillShape ps = prefill_shape(rows, nb, n, wtype != kTypeQ4K);
     if (ps.groups > 65535u) return hipErrorInvalidValue;
     if (ps.splits > 1 && !part) return hipErrorInvalidValue;
     static bool raised = false;  // two activation buffers: more than the default 64 KB of dynamic LDS
     if (!raised) {
         for (const void* k : {reinterpret_cast<const void*>(&prefill_gemm_kernel<1>), reinterpret_cast<const void*>(&prefill_gemm_kernel<2>),
-                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, true>)}) {
+                              reinterpret_cast<const void*>(&prefill_gemm_kernel<1, kWtQ5>), reinterpret_cast<const void*>(&prefill_gemm_kernel<1, kWtQ6>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
             if (e != hipSuccess) return e;
         }
@@ -658,8 +792,12 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
     const int64_t ld = split ? rows : ldy;
     const int64_t stride = split ? n * rows : 0;
     const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
-    if (wtype == kTypeQ5K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, true>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+    if (wtype == kTypeQ6K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ6>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+                           ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
+                           (const uint8_t*)nullptr);
+    } else if (wtype == kTypeQ5K) {
+        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ5>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);
     } else if (ps.narrow) {

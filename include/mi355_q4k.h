@@ -72,8 +72,9 @@ int mq_weight_upload(const void* q4k_host, int64_t rows, int64_t cols, int64_t n
  * (core/src/llm/matmul/q6_small_batch.h:13-92): one integer sum_g scale_g * sum (code - 32) * q8 per
  * super-block (what mq_debug_block_sums returns as dot_scaled; min_dot is 0), one fused multiply-add per block.
  * Every product entry point accepts handles of any of the three types (gate and up of one call must share
- * theirs); the matrix-core GEMM (mq_gemm_q4k) and its expert-grouped form take Q4_K and Q5_K (the one-launch decoder
- * Q4_K only), wide Q6_K products run through the decode kernel in passes of 16 rows.
+ * theirs), the matrix-core GEMM (mq_gemm_q4k) and its expert-grouped form included -- the reference serves Q6_K at
+ * every width through its batched machinery as well (core/src/llm/matmul/batched_exec.cpp:933,1280); the one-launch
+ * decoder takes Q4_K only.
  * 8 = Q8_0 (fp16 d + 32 int8 codes, 34 bytes per 32 weights; core/src/llm/matmul/q8_small_batch.h:9-14): dense
  * matrices only (n_experts == 1, cols % 256 == 0, row_bytes >= cols / 32 * 34), taken by mq_mul_mat_q4k (and
  * mq_mul_mat_q4k_host, mq_debug_block_sums, the handle queries) and refused by every other entry point.  As in
@@ -197,7 +198,7 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
  * [n][top_k]; entries outside [0, n_experts) produce zeros.  Tokens are grouped
  * by expert on the device; nothing returns to the host.  y_dev fp32
  * [n][top_k][rows].  (ggml_mul_mat_id as emitted at
- * core/src/llm/moe/native_gemma.cpp:1509-1559.)  Prefill widths (Q4_K, 256 tokens
+ * core/src/llm/moe/native_gemma.cpp:1509-1559.)  Prefill widths (256 tokens
  * and more with a dozen rows per expert on average) run on the int8 matrix-core
  * GEMM in its expert-grouped form, as do mq_moe_gateup_swiglu_q4k and
  * mq_moe_down_weighted_q4k below. */
@@ -229,9 +230,9 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  * Up to eight tokens (and 512 experts) two launches: gate/up + SwiGLU with the router and the Q8_K of x inside,
  * down with the Q8_K of the hidden rows and the weighted combine inside.  Above: router + expert grouping + Q8_K
  * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way.
- * Prefill widths (Q4_K stacks, 256 tokens and more with a dozen routed rows per expert on average): the expert
- * products run on the int8 matrix-core GEMM in an expert-grouped form (entries in 16-row tiles per expert), the
- * shared expert as one more group of all tokens; same routing, results within the fp32 tolerance of the other form (the
+ * Prefill widths (256 tokens and more with a dozen routed rows per expert on average): the expert products run on the
+ * int8 matrix-core GEMM in an expert-grouped form (entries in 16-row tiles per expert), the shared expert as one more
+ * group of all tokens; a Q8_0 down stack takes the fp32 hidden rows of that gate/up through its own launches; same routing, results within the fp32 tolerance of the other form (the
  * summation order differs), and mq_debug_moe_hidden does not apply. */
 typedef struct {
     const mq_weight* gate_exps; /* n_experts x [inter][hidden]  */

@@ -64,7 +64,10 @@ def test_q6k_matmul_integer_sums_exact_and_fp32_within_tolerance(ops, rows, cols
     assert np.array_equal(ds.cpu().numpy(), orc.q6k_matrix_block_sums(w_np, cols, q8)), "block sums differ"
     assert not md.cpu().numpy().any()
     y = y.cpu().numpy()
-    assert np.array_equal(y_dbg.cpu().numpy().view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    if n < 48:
+        assert np.array_equal(y_dbg.cpu().numpy().view(np.uint32), y.view(np.uint32)), "debug and production kernels disagree"
+    else:  # from 48 rows the product runs on the matrix-core GEMM: the same integers, another summation order
+        assert np.max(np.abs(y_dbg.cpu().numpy() - y)) <= 1e-5 * np.max(np.abs(y))
     mag = orc.q6k_dot_dequant_f64(w_np, cols, q8, magnitude=True)
     for name, order in Q6_ORDERS.items():
         assert_fp32_parity(y, orc.mul_mat_q6k_q8k(w_np, cols, q8, order), mag, f"order={name}")
@@ -158,9 +161,79 @@ def test_q6k_rejections(ops):
     import torch
     from densecore_amd._lib import MqError
     w6 = ops.Q4KWeight.from_ggml(synth.q6k_matrix(1, 64, 512), 512, Q6)
+    w8 = ops.Q4KWeight.from_ggml(synth.q80_matrix(1, 64, 512), 512, synth.GGML_TYPE_Q8_0)
     x = torch.zeros((64, 512), device="cuda")
     with pytest.raises(MqError):
-        ops.gemm(w6, x)                                                 # the matrix-core GEMM takes Q4_K and Q5_K only
+        ops.gemm(w8, x)                                                 # the matrix-core GEMM takes the three K-quant types only
+    w8.free()
     with pytest.raises(MqError):
         ops.Q4KWeight.from_ggml(np.zeros((4, 176), np.uint8), 256, Q6)  # a Q6_K row needs 210 bytes
     w6.free()
+
+
+# ----------------------------------------------------------------------------- matrix-core GEMM (prefill widths)
+@pytest.mark.parametrize("rows,cols,n", [(96, 768, 64), (80, 4096, 50), (272, 2048, 130), (1000, 1024, 300)])
+def test_q6k_gemm_matches_oracle_and_decode_kernel(ops, rows, cols, n):
+    """48 rows and more of Q6_K: the int8 matrix-core GEMM with both factors of scale * (code - 32) cut in two digits
+    (five MFMA chains; the second shape splits K into runs, the last has a ragged last row tile).  Against the oracle,
+    against 16-row passes of the decode kernel, and through mq_mul_mat_q4k."""
+    import torch
+    w_np = synth.q6k_matrix(synth.tensor_seed("pf6-w", rows, cols), rows, cols)
+    x = synth.normal_f32(synth.tensor_seed("pf6-x", rows, cols, n), (n, cols))
+    W = ops.Q4KWeight.from_ggml(w_np, cols, Q6)
+    got = ops.gemm(W, cu(x))
+    assert torch.equal(ops.mul_mat(W, cu(x)), got)
+    small = torch.cat([ops.mul_mat(W, cu(x[i:i + 16])) for i in range(0, n, 16)])
+    assert (got - small).abs().max().item() <= 1e-5 * small.abs().max().item()
+    q8 = orc.quantize_rows_q8k(x)
+    mag = orc.q6k_dot_dequant_f64(w_np, cols, q8, magnitude=True)
+    assert_fp32_parity(got.cpu().numpy(), orc.mul_mat_q6k_q8k(w_np, cols, q8, orc.ORDER_DOTPROD), mag, "Q6_K GEMM")
+    W.free()
+
+
+def test_q6k_gemm_integer_sums_are_exact(ops):
+    """d = 1 and integer activations with a +-127 in every block: the output equals the sum of the oracle's integers,
+    so one wrong unit in any of the five chains, in any digit of any scale or code, changes it."""
+    rows, cols, n = 48, 768, 70
+    nb = cols // 256
+    w = synth.q6k_matrix(synth.tensor_seed("pf6-int", rows), rows, cols).reshape(rows, nb, 210).copy()
+    w[:, :, 208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[1::2, :, 208:210] = np.frombuffer(np.float16(-1.0).tobytes(), np.uint8)
+    w = w.reshape(rows, nb * 210)
+    rng = np.random.default_rng(12)
+    x = rng.integers(-7, 8, size=(n, cols)).astype(np.float32)
+    x.reshape(n, nb, 256)[:, :, 9] = rng.choice([-127.0, 127.0], size=(n, nb))
+    q8 = orc.quantize_rows_q8k(x)
+    d, _, _ = orc.split_q8k(q8)
+    assert np.all(np.abs(d) == 1.0)
+    isum = orc.q6k_matrix_block_sums(w, cols, q8).astype(np.int64)            # [rows, n, nb]
+    sign = np.where(np.arange(rows) % 2 == 0, 1, -1)[:, None, None]
+    want = (isum * sign * d.astype(np.int64)[None]).sum(axis=2).T
+    assert np.abs(isum).sum(axis=2).max() < 2 ** 24
+    W = ops.Q4KWeight.from_ggml(w, cols, Q6)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    assert np.array_equal(got, want.astype(np.float32))
+    W.free()
+
+
+@pytest.mark.parametrize("scale,code", [(-128, 0), (-128, 63), (127, 0), (127, 63), (-1, 31), (15, 40), (16, 24), (-16, 7)])
+def test_q6k_gemm_extreme_blocks(ops, scale, code):
+    """One scale and one code everywhere -- the corners of both digit pairs (scale + 128 = 0, 255, 143, 144, 112;
+    code = 0, 63 and both sides of the digit boundaries) -- with activations at +-full scale."""
+    rows, cols, n = 32, 512, 48
+    w_np = np.zeros((rows, cols // 256 * 210), np.uint8)
+    blocks = w_np.reshape(rows, -1, 210)
+    blocks[:, :, 0:128] = (code & 15) | ((code & 15) << 4)
+    top = code >> 4
+    blocks[:, :, 128:192] = top | (top << 2) | (top << 4) | (top << 6)
+    blocks[:, :, 192:208] = np.int8(scale).view(np.uint8)
+    blocks[:, :, 208:210] = np.array([0.01], np.float16).view(np.uint8)
+    x = np.ones((n, cols), np.float32)
+    x[1::2] *= -1.0
+    x[2, ::2] *= -1.0
+    W = ops.Q4KWeight.from_ggml(w_np, cols, Q6)
+    got = ops.gemm(W, cu(x)).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    assert_fp32_parity(got, orc.mul_mat_q6k_q8k(w_np, cols, q8, orc.ORDER_DOTPROD),
+                       orc.q6k_dot_dequant_f64(w_np, cols, q8, magnitude=True), "Q6_K extremes")
+    W.free()
