@@ -1205,12 +1205,19 @@ int run_moe_down(const mq_weight* down, const SharedExpert& sh, const float* hid
         q.n = mid_rows;
         q.y = (float*)g.part.ptr;
         q.ldy = hidden_dim;
-        q.pair_ids = ids;
         q.top_k = top_k;
         q.slots = slots;
         q.n_experts = (int)down->n_experts;
         q.expert_bytes = down->expert_bytes;
         q.sh_w = sh.down ? sh.down->data : nullptr;
+        if (r.direct_ids) {  // few tokens: nothing was grouped, every pair is a column of its own
+            q.pair_ids = ids;
+        } else {             // an expert's rows together, eight to a pass
+            q.group_expert = r.group_expert, q.group_begin = r.group_begin, q.n_groups = r.n_groups;
+            q.entry_token = r.entry_token, q.entry_k = r.entry_k;
+            q.max_groups = (int)(pairs < down->n_experts ? pairs : down->n_experts);
+            q.sh_tokens = sh.down ? (int)n : 0;
+        }
         MQ_HIP(launch_q80_matmul(q, s));
         MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, slots, hidden_dim, weights, ids, down->n_experts,
                                   sh.down ? 1 : 0, sh_gate_inp, x, y, s));

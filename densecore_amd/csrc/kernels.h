@@ -137,6 +137,17 @@ struct Q80MatmulArgs {
     int top_k = 0, slots = 0, n_experts = 0;
     size_t expert_bytes = 0;
     const uint8_t* sh_w = nullptr;
+    // expert-grouped mode (the same node above eight tokens, where the pairs were sorted by expert): workgroup column g
+    // is group g of the work list -- its expert's weights against the group's rows in passes of eight, so an expert is
+    // streamed once per eight of its rows instead of once per row; columns past the groups are passes of the shared
+    // expert (sh_w) over all tokens.  Rows as above: token * slots + slot.  pair_ids stays null.
+    const int32_t* group_expert = nullptr;
+    const int32_t* group_begin = nullptr;
+    const int32_t* n_groups = nullptr;
+    const int32_t* entry_token = nullptr;
+    const int32_t* entry_k = nullptr;
+    int max_groups = 0;
+    int sh_tokens = 0;
 };
 size_t q80_scale_bytes(int64_t n, int64_t nb);
 // x rows 16-byte aligned (ldx % 4 == 0), cols % 256 == 0

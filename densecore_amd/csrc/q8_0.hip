@@ -86,7 +86,10 @@ __global__ void __launch_bounds__(512) q80_matmul_kernel(const Q80MatmulArgs p) 
     int64_t rt = blockIdx.x;
     const int nb = (int)p.nb;
     const uint8_t* w = p.w;
-    int first = 0, last = (int)p.n;  // activation rows this workgroup multiplies
+    int first = 0, last = (int)p.n;  // activation rows this workgroup multiplies (dense, pairs), or entries of its group
+    int g_begin = 0;                 // expert-grouped: first entry of the group (or first token of a shared-expert pass)
+    bool g_shared = false;
+    const bool grouped = p.group_begin != nullptr;
     if (p.pair_ids) {
         // expert-routed: the grid is flat, workgroup = column g * rowtiles + row tile (a grid's second dimension ends
         // at 65535, a prefill-width block has more pairs); column g is hidden row g = token * slots + slot alone,
@@ -104,21 +107,44 @@ __global__ void __launch_bounds__(512) q80_matmul_kernel(const Q80MatmulArgs p) 
         }
         first = g;
         last = g + 1;
+    } else if (grouped) {
+        const int g = blockIdx.y, ng = *p.n_groups;
+        const int gi = g < p.max_groups ? g : 0;  // columns of the shared expert read group 0's entries and drop them
+        const int g_expert = p.group_expert[gi], b0 = p.group_begin[gi], b1 = p.group_begin[gi + 1];
+        if (g < ng) {
+            w += (size_t)g_expert * p.expert_bytes;
+            g_begin = b0;
+            last = b1 - b0;
+        } else if (g - ng < (p.sh_tokens + kTokTile - 1) / kTokTile) {
+            g_shared = true;
+            w = p.sh_w;
+            g_begin = (g - ng) * kTokTile;
+            last = p.sh_tokens - g_begin < kTokTile ? p.sh_tokens - g_begin : kTokTile;
+        } else {
+            return;  // the whole workgroup, before any barrier
+        }
     }
+    // hidden / output row of entry e of the group
+    auto group_row = [&](int e) {
+        if (g_shared) return (g_begin + e) * p.slots + p.top_k;
+        return p.entry_token[g_begin + e] * p.slots + p.entry_k[g_begin + e];
+    };
     const uint8_t* tiles = w + tile_offset(rt, 0, nb, kTile80Bytes);
     const int cnt = wave < nb ? (nb - wave + n_waves - 1) / n_waves : 0;  // 256-weight groups wave, wave + W, ...
 
     for (int chunk = first; chunk < last; chunk += kTokTile) {
         const int count = last - chunk < kTokTile ? last - chunk : kTokTile;
         // a dead slot reads a live row of the pass and stores nothing
-        const int arow = chunk + ((slot >> 1) < count ? (slot >> 1) : count - 1);
+        const int a_ent = chunk + ((slot >> 1) < count ? (slot >> 1) : count - 1);
+        const int arow = grouped ? group_row(a_ent) : a_ent;
         const size_t a_off = aq_row_offset(arow, nb) + (size_t)kq * 256 + (size_t)(slot & 1) * 16;
         int yrow[2];
         size_t s_off[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const bool live = 2 * kq + j < count;
-            const int r = chunk + (live ? 2 * kq + j : count - 1);
+            const int ent = chunk + (live ? 2 * kq + j : count - 1);
+            const int r = grouped ? group_row(ent) : ent;
             yrow[j] = live ? r : -1;
             s_off[j] = ad_index(r, 0, nb) * 8;  // + b * 64 halves per group
         }
@@ -210,9 +236,19 @@ hipError_t launch_quantize_q80(const float* x, int64_t n, int64_t ldx, int64_t c
 
 hipError_t launch_q80_matmul(const Q80MatmulArgs& a, hipStream_t stream) {
     if (a.rows <= 0 || a.nb <= 0 || a.n <= 0 || !a.w || !a.aq || !a.ah || !a.y || a.ldy < a.rows) return hipErrorInvalidValue;
-    if (a.pair_ids && (a.top_k <= 0 || a.slots < a.top_k || a.n % a.slots || a.dbg_sum || (a.slots > a.top_k && !a.sh_w)))
+    const bool grouped = a.group_begin != nullptr;
+    if ((a.pair_ids || grouped) && (a.top_k <= 0 || a.slots < a.top_k || a.n % a.slots || a.dbg_sum || (a.slots > a.top_k && !a.sh_w)))
         return hipErrorInvalidValue;
+    if (grouped && (a.pair_ids || !a.group_expert || !a.n_groups || !a.entry_token || !a.entry_k || a.max_groups <= 0)) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
+    if (grouped) {
+        const int64_t columns = (int64_t)a.max_groups + (a.sh_tokens + kTokTile - 1) / kTokTile;
+        if (columns > 65535) return hipErrorInvalidValue;
+        const int waves = pick_waves(a.nb, rowtiles * columns);
+        hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)rowtiles, (unsigned)columns), dim3(64 * waves),
+                           waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0, stream, a);
+        return hipGetLastError();
+    }
     const int64_t columns = a.pair_ids ? a.n : 1;
     if (rowtiles * columns >= (int64_t)1 << 31) return hipErrorInvalidValue;
     const int waves = pick_waves(a.nb, rowtiles * columns);

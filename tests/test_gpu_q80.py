@@ -106,10 +106,12 @@ def test_q80_is_refused_where_it_is_not_supported(ops):
     w.free()
 
 
-@pytest.mark.parametrize("n", [1, 3, 9, 24])
+@pytest.mark.parametrize("n", [1, 3, 9, 24, 100, 300])
 def test_moe_layer_with_q80_down_experts_and_shared_expert(ops, n):
     """Q4_K gate/up experts with Q8_0 down experts (an accepted pairing, core/src/llm/moe/native.cpp:4611-4616) through
-    the whole MoE layer, shared expert included: the layer must equal its own gate/up node followed by the Q8_0 down
+    the whole MoE layer, shared expert included (up to eight tokens a workgroup column per pair, above that the pairs
+    grouped by expert, eight rows to a pass; at 300 tokens gate and up run on the expert-grouped matrix-core GEMM and
+    hand their fp32 rows to the same Q8_0 launches): the layer must equal its own gate/up node followed by the Q8_0 down
     arithmetic of the reference (hidden row -> Q8_0 -> dot -> += value * weight in k order, :3239-3286) and the
     sigmoid-gated shared expert."""
     import torch
