@@ -18,7 +18,7 @@ EXPORTS = [
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
     "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k",
     "mq_acts_create", "mq_acts_free", "mq_acts_quantize", "mq_mul_mat_q4k_acts", "mq_swiglu_mul_mat_q4k_acts",
-    "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
+    "mq_silu_mul_f32", "mq_scale_rows_sigmoid_f32", "mq_add_rmsnorm_f32", "mq_add_rmsnorm_q8k", "mq_router_logits_f32", "mq_add_rmsnorm_router_f32", "mq_rmsnorm_mul_mat_q4k",
     "mq_decoder_create", "mq_decoder_step", "mq_decoder_status", "mq_decoder_set_patience", "mq_decoder_free",
     "mq_device_malloc", "mq_device_free", "mq_memcpy_h2d", "mq_memcpy_d2h", "mq_host_malloc", "mq_host_free", "mq_memcpy_h2d_async", "mq_memcpy_d2h_async", "mq_stream_synchronize",
 ]
@@ -92,6 +92,8 @@ def load() -> C.CDLL:
     L.mq_debug_moe_groups.argtypes = [vp, vp, i64, i64, ci, vp, vp, vp]
     L.mq_debug_moe_hidden.argtypes = [vp, sz, vp]
     L.mq_debug_decoder_buffers.argtypes = [vp] + [C.POINTER(vp)] * 5
+    L.mq_silu_mul_f32.argtypes = [vp, vp, i64, i64, i64, i64, vp, i64, ci, vp]
+    L.mq_scale_rows_sigmoid_f32.argtypes = [vp, i64, i64, i64, vp, i64, vp, i64, vp]
     L.mq_add_rmsnorm_f32.argtypes = [vp, vp, vp, i64, i64, C.c_float, vp, vp, vp]
     L.mq_add_rmsnorm_q8k.argtypes = [vp, vp, vp, i64, i64, C.c_float, vp, vp, vp, vp]
     L.mq_router_logits_f32.argtypes = [vp, i64, i64, vp, i64, i64, vp, vp]

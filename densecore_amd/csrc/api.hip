@@ -984,6 +984,27 @@ int mq_add_rmsnorm_router_f32(const float* x_dev, const float* delta_dev, const 
     return MQ_OK;
 }
 
+int mq_silu_mul_f32(const float* gate_dev, const float* up_dev, int64_t n, int64_t cols, int64_t ld_gate, int64_t ld_up, float* out_dev,
+                    int64_t ld_out, int silu_mode, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (n == 0 || cols == 0) return MQ_OK;
+    if (!gate_dev || !up_dev || !out_dev || n < 0 || cols < 0 || ld_gate < cols || ld_up < cols || ld_out < cols)
+        return fail(MQ_ERR_INVALID, "mq_silu_mul_f32: null pointer, negative size or a row stride below cols");
+    if (silu_mode < 0 || silu_mode > 2) return fail(MQ_ERR_INVALID, "mq_silu_mul_f32: silu_mode %d", silu_mode);
+    MQ_HIP(launch_silu_mul(gate_dev, up_dev, n, cols, ld_gate, ld_up, out_dev, ld_out, silu_mode, (hipStream_t)stream));
+    return MQ_OK;
+}
+
+int mq_scale_rows_sigmoid_f32(const float* src_dev, int64_t n, int64_t cols, int64_t ld_src, const float* logit_dev, int64_t ld_logit,
+                              float* out_dev, int64_t ld_out, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (n == 0 || cols == 0) return MQ_OK;
+    if (!src_dev || !logit_dev || !out_dev || n < 0 || cols < 0 || ld_src < cols || ld_out < cols || ld_logit < 1)
+        return fail(MQ_ERR_INVALID, "mq_scale_rows_sigmoid_f32: null pointer, negative size or a row stride too small");
+    MQ_HIP(launch_scale_rows_sigmoid(src_dev, n, cols, ld_src, logit_dev, ld_logit, out_dev, ld_out, (hipStream_t)stream));
+    return MQ_OK;
+}
+
 int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64_t n, const int32_t* ids_dev, int top_k,
                                float* weights_dev, void* stream) {
     if (int rc = check_ready()) return rc;

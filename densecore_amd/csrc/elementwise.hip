@@ -309,6 +309,36 @@ __global__ void __launch_bounds__(256) add_rmsnorm_router_kernel(const float* __
     }
 }
 
+// out = silu(gate) * up, element by element over [n][cols] with their own row strides: the node between the gate / up
+// products and the down product of a dense FFN (cb_silu_mul_fused, core/src/llm/graph/fused_ops.cpp:317-366).
+__global__ void __launch_bounds__(256) silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up, int64_t n,
+                                                       int64_t cols, int64_t ld_gate, int64_t ld_up, float* __restrict__ out,
+                                                       int64_t ld_out, int mode) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * cols) return;
+    const uint32_t row = (uint32_t)i / (uint32_t)cols, c = (uint32_t)i - row * (uint32_t)cols;  // n * cols < 2^31 (launcher)
+    out[(size_t)row * ld_out + c] = silu_mul(gate[(size_t)row * ld_gate + c], up[(size_t)row * ld_up + c], mode);
+}
+
+// out[t] = sigmoid(logit[t]) * src[t] with the two-sided sigmoid of core/src/llm/graph/fused_ops.cpp:451-458
+// (cb_apply_shared_scalar_gate, :437-475): the scalar gate of the shared expert.
+__global__ void __launch_bounds__(256) scale_rows_sigmoid_kernel(const float* __restrict__ src, int64_t n, int64_t cols, int64_t ld_src,
+                                                                 const float* __restrict__ logit, int64_t ld_logit,
+                                                                 float* __restrict__ out, int64_t ld_out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * cols) return;
+    const uint32_t row = (uint32_t)i / (uint32_t)cols, c = (uint32_t)i - row * (uint32_t)cols;
+    const float x = logit[(size_t)row * ld_logit];
+    float g;
+    if (x >= 0.0f) {
+        g = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-x)));
+    } else {
+        const float z = expf(x);
+        g = __fdiv_rn(z, __fadd_rn(1.0f, z));
+    }
+    out[(size_t)row * ld_out + c] = __fmul_rn(src[(size_t)row * ld_src + c], g);
+}
+
 }  // namespace
 
 hipError_t launch_add_rmsnorm_router(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols, float eps,
@@ -349,6 +379,24 @@ hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols,
     if (n > 65535) return hipErrorInvalidValue;
     hipLaunchKernelGGL(router_logits_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256), 0, stream, w,
                        n_experts, cols, x, ldx, logits);
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const float* gate, const float* up, int64_t n, int64_t cols, int64_t ld_gate, int64_t ld_up, float* out,
+                           int64_t ld_out, int mode, hipStream_t stream) {
+    if (n * cols == 0) return hipSuccess;
+    if (n * cols >= (int64_t)1 << 31) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, gate, up, n, cols, ld_gate, ld_up,
+                       out, ld_out, mode);
+    return hipGetLastError();
+}
+
+hipError_t launch_scale_rows_sigmoid(const float* src, int64_t n, int64_t cols, int64_t ld_src, const float* logit, int64_t ld_logit,
+                                     float* out, int64_t ld_out, hipStream_t stream) {
+    if (n * cols == 0) return hipSuccess;
+    if (n * cols >= (int64_t)1 << 31) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(scale_rows_sigmoid_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, src, n, cols, ld_src,
+                       logit, ld_logit, out, ld_out);
     return hipGetLastError();
 }
 

@@ -212,6 +212,11 @@ hipError_t launch_add_rmsnorm_router(const float* x, const float* delta, const f
                                      hipStream_t stream);
 hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols, const float* x, int64_t n, int64_t ldx,
                                 float* logits, hipStream_t stream);
+// out = silu(gate) * up over [n][cols] (mode: MQ_SILU_*), and out[t] = sigmoid(logit[t * ld_logit]) * src[t]
+hipError_t launch_silu_mul(const float* gate, const float* up, int64_t n, int64_t cols, int64_t ld_gate, int64_t ld_up, float* out,
+                           int64_t ld_out, int mode, hipStream_t stream);
+hipError_t launch_scale_rows_sigmoid(const float* src, int64_t n, int64_t cols, int64_t ld_src, const float* logit, int64_t ld_logit,
+                                     float* out, int64_t ld_out, hipStream_t stream);
 
 // ---- router.hip ------------------------------------------------------------------------------
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,

@@ -20,8 +20,9 @@ CALLBACKS = [
     "mq_cb_gemv_custom", "mq_cb_gemv_batched_custom", "mq_cb_moe_gateup_swiglu", "mq_cb_moe_down_weighted_logits",
     "mq_cb_moe_fused_router", "mq_cb_moe_topk_weights_from_logits", "mq_cb_mul_mat_id",
 ]
-EXPORTS = CALLBACKS + [
-    "mq_ggml_last_status", "mq_ggml_weight_cache_clear", "mq_ggml_weight_cache_size", "mq_ggml_weight_fingerprint",
+CALLBACKS2 = ["mq_cb_silu_mul_fused", "mq_cb_apply_shared_scalar_gate"]   # ggml_custom2_op_t: (dst, a, b, ith, nth, userdata)
+EXPORTS = CALLBACKS + CALLBACKS2 + [
+    "mq_ggml_graph_begin", "mq_ggml_tensor_to_host", "mq_ggml_last_status", "mq_ggml_weight_cache_clear", "mq_ggml_weight_cache_size", "mq_ggml_weight_fingerprint",
     "mq_matmul_ggml_quantized_transb",
 ]
 
@@ -59,7 +60,7 @@ _handle = None
 def lib():
     global _handle
     if _handle is None:
-        _lib.load()  # the C ABI library first: the adapter library links against it
+        _lib.lib()  # the C ABI library first (loaded and initialised on device 0): the adapter library links against it
         if not os.path.exists(LIB_PATH):
             raise _lib.MqError(f"{LIB_PATH} is missing: run `make -C densecore_amd/host`")
         L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
@@ -67,6 +68,11 @@ def lib():
         for name in CALLBACKS:
             getattr(L, name).argtypes = cb
             getattr(L, name).restype = None
+        for name in CALLBACKS2:
+            getattr(L, name).argtypes = [C.POINTER(GgmlTensor), C.POINTER(GgmlTensor), C.POINTER(GgmlTensor), C.c_int, C.c_int, C.c_void_p]
+            getattr(L, name).restype = None
+        L.mq_ggml_graph_begin.restype = None
+        L.mq_ggml_tensor_to_host.argtypes = [C.POINTER(GgmlTensor)]
         L.mq_ggml_weight_cache_size.restype = C.c_int64
         L.mq_ggml_weight_fingerprint.argtypes = [C.c_void_p, C.c_size_t]
         L.mq_ggml_weight_fingerprint.restype = C.c_uint64

@@ -7,6 +7,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -203,10 +204,86 @@ thread_local bool t_unsettled = false;
 
 // Every node but the down node of a hand-over starts here: if the previous node left copies queued, wait for them
 // before this node writes the same pinned twins (a graph whose gate/up node is not followed by its down node).
+// Dense nodes and the element-wise nodes upload through a ring of four pinned twins, so that a short run of nodes that
+// leave their results on the device (gate, up, silu * up, down of a dense FFN) queues its uploads without waiting for
+// one another; a twin is written again only after a synchronisation has passed since its last upload.
+constexpr int kInRing = 4;
+struct InRing {
+    Staging slot[kInRing];
+    bool dirty[kInRing] = {false, false, false, false};
+    int next = 0;
+};
+thread_local InRing t_ring;
+
 void settle() {
-    if (!t_unsettled) return;
+    bool any = t_unsettled;
+    for (int i = 0; i < kInRing; ++i) any = any || t_ring.dirty[i];
+    if (!any) return;
     (void)mq_stream_synchronize(nullptr);
     t_unsettled = false;
+    for (int i = 0; i < kInRing; ++i) t_ring.dirty[i] = false;
+}
+void settled_by_sync() {  // the caller has just synchronised the null stream
+    t_unsettled = false;
+    for (int i = 0; i < kInRing; ++i) t_ring.dirty[i] = false;
+}
+// the next twin of the ring, free to be written (waits for the queued copies only when the ring has gone round)
+Staging* ring_slot(size_t bytes) {
+    const int i = t_ring.next;
+    t_ring.next = (i + 1) % kInRing;
+    if (t_ring.dirty[i] || bytes > t_ring.slot[i].cap) settle();  // growing a twin frees it: nothing may still read it
+    if (!t_ring.slot[i].get(bytes)) return nullptr;
+    t_ring.dirty[i] = true;
+    return &t_ring.slot[i];
+}
+
+// ---- tensors left on the device between the nodes of one graph -----------------------------------------------
+// A node whose userdata asks for it (mq_ggml_userdata::keep_hidden_on_device) leaves its result in HBM and does not
+// write dst->data; a later node of the same graph that names that tensor as an operand (the same ggml_tensor, or a
+// view of all of it) reads it there.  Keyed by the tensor object, not by its data pointer: graph allocators give the
+// memory of a dead tensor to a later one, tensor objects are one per node.  mq_ggml_graph_begin() forgets everything.
+struct KeptTensor {
+    const ggml_tensor* tensor = nullptr;
+    int64_t rows = 0, cols = 0;  // dense fp32 [rows][cols]
+    Staging buf;
+};
+thread_local std::vector<KeptTensor*> t_kept;
+
+const ggml_tensor* whole_view_base(const ggml_tensor* t) {
+    // a reshape / view of a whole contiguous tensor stands for the same rows
+    while (t && t->view_src && t->view_offs == 0) t = t->view_src;
+    return t;
+}
+KeptTensor* kept_find(const ggml_tensor* t, int64_t rows, int64_t cols) {
+    const ggml_tensor* base = whole_view_base(t);
+    for (KeptTensor* k : t_kept)
+        if (k->tensor && (k->tensor == t || k->tensor == base) && k->rows * k->cols == rows * cols) return k;
+    return nullptr;
+}
+void kept_forget(const ggml_tensor* t) {
+    for (KeptTensor* k : t_kept)
+        if (k->tensor == t) k->tensor = nullptr;
+}
+KeptTensor* kept_slot(const ggml_tensor* t, int64_t rows, int64_t cols) {
+    KeptTensor* pick = nullptr;
+    for (KeptTensor* k : t_kept)
+        if (k->tensor == t) pick = k;
+    if (!pick)
+        for (KeptTensor* k : t_kept)
+            if (!k->tensor) pick = k;
+    if (!pick) {
+        pick = new KeptTensor;
+        t_kept.push_back(pick);
+    }
+    const size_t bytes = (size_t)rows * (size_t)cols * 4;
+    if (bytes > pick->buf.cap) settle();  // growing frees the old buffer: queued work may still use it
+    if (!pick->buf.get(bytes)) {
+        pick->tensor = nullptr;
+        return nullptr;
+    }
+    pick->tensor = t;
+    pick->rows = rows, pick->cols = cols;
+    return pick;
 }
 
 // Gathers a strided host matrix [rows][cols] of 4-byte elements (row stride in bytes) into the pinned twin and queues
@@ -264,8 +341,7 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
     const ggml_tensor* src = dst->src[0];
     const ggml_tensor* weight = dst->src[1];
     Options o = options_for(userdata, 1);
-    settle();
-    t_resident = Resident{};
+    t_resident = Resident{};  // (no wait here: this node uploads through the ring, whose twins wait for themselves)
     if (!src || !weight || !src->data || !dst->data) return finish(o, MQ_ERR_INVALID);
     if ((!is_kquant_matrix(weight) && !is_q80_matrix(weight)) || weight->ne[2] != 1) return finish(o, MQ_ERR_UNSUPPORTED);
     const int64_t k_in = weight->ne[0], n_out = weight->ne[1];
@@ -281,14 +357,62 @@ void dense_node(ggml_tensor* dst, int ith, void* userdata) {
         return finish(o, MQ_ERR_UNSUPPORTED);
     const mq_weight* w = device_weight(weight);
     if (!w) return finish(o, t_status);
-    Staging &in = t_stage.in, &out = t_stage.out;
-    if (!in.get((size_t)m * k_in * 4) || !out.get((size_t)m * n_out * 4)) return finish(o, t_status);
-    int rc = upload_rows(in, 0, src->data, m, k_in, src->nb[1]);
-    if (rc == MQ_OK) rc = mq_mul_mat_q4k(w, (const float*)in.dev, m, k_in, (float*)out.dev, n_out, nullptr);
+    // the input: left on the device by an earlier node of this graph, or uploaded through the ring of pinned twins
+    const float* x_dev = nullptr;
+    int64_t ldx = k_in;
+    if (KeptTensor* kin = kept_find(src, m, k_in)) {
+        x_dev = (const float*)kin->buf.dev;
+    } else {
+        Staging* in = ring_slot((size_t)m * k_in * 4);
+        if (!in) return finish(o, t_status);
+        if (int rc = upload_rows(*in, 0, src->data, m, k_in, src->nb[1])) return finish(o, rc);
+        x_dev = (const float*)in->dev;
+    }
+    if (o.keep_hidden) {  // the result stays in HBM for the nodes that read this tensor; nothing is waited for
+        KeptTensor* kout = kept_slot(dst, m, n_out);
+        if (!kout) return finish(o, t_status);
+        return finish(o, mq_mul_mat_q4k(w, x_dev, m, ldx, (float*)kout->buf.dev, n_out, nullptr));
+    }
+    kept_forget(dst);
+    Staging& out = t_stage.out;
+    if (!out.get((size_t)m * n_out * 4)) return finish(o, t_status);
+    int rc = mq_mul_mat_q4k(w, x_dev, m, ldx, (float*)out.dev, n_out, nullptr);
     if (rc == MQ_OK) rc = download_rows(out, (size_t)m * n_out * 4);
     if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);  // the node's one synchronisation
+    if (rc == MQ_OK) settled_by_sync();
     if (rc == MQ_OK) scatter_rows(dst->data, out, 0, m, n_out, dst->nb[1]);
     finish(o, rc);
+}
+
+// An fp32 operand [rows][cols] of an element-wise node: on the device already, or uploaded through the ring.
+const float* operand_rows(const ggml_tensor* t, int64_t rows, int64_t cols, int* rc) {
+    if (KeptTensor* k = kept_find(t, rows, cols)) return (const float*)k->buf.dev;
+    Staging* in = ring_slot((size_t)rows * cols * 4);
+    if (!in) {
+        *rc = t_status;
+        return nullptr;
+    }
+    *rc = upload_rows(*in, 0, t->data, rows, cols, t->nb[1]);
+    return *rc == MQ_OK ? (const float*)in->dev : nullptr;
+}
+
+// Ends an element-wise node: the rows stay on the device (kept) or travel to dst->data after one synchronisation.
+void deliver_rows(const Options& o, ggml_tensor* dst, KeptTensor* kout, const Staging* out, int64_t rows, int64_t cols, int rc) {
+    if (rc != MQ_OK || kout) return finish(o, rc);
+    rc = mq_memcpy_d2h_async(out->pin, out->dev, (size_t)rows * cols * 4, nullptr);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (rc == MQ_OK) settled_by_sync();
+    if (rc == MQ_OK) scatter_rows(dst->data, *out, 0, rows, cols, dst->nb[1]);
+    finish(o, rc);
+}
+
+bool rows_layout(const ggml_tensor* t, int64_t* rows, int64_t* cols) {
+    // fp32, unit element stride, rows evenly spaced over the outer dimensions (what upload_rows / scatter_rows walk)
+    if (!t || !t->data || t->type != GGML_TYPE_F32 || t->nb[0] != 4 || t->ne[0] <= 0) return false;
+    *cols = t->ne[0];
+    *rows = t->ne[1] * t->ne[2] * t->ne[3];
+    if (*rows <= 0) return false;
+    return (t->ne[2] <= 1 || t->nb[2] == t->nb[1] * (size_t)t->ne[1]) && (t->ne[3] <= 1 || t->nb[3] == t->nb[2] * (size_t)t->ne[2]);
 }
 
 // selected_experts I32 ne=[top_k, n_tokens] -> dense device [n_tokens][top_k] (queued, not synchronised)
@@ -520,6 +644,100 @@ void mq_cb_mul_mat_id(struct ggml_tensor* dst, int ith, int /*nth*/, void* userd
     if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
     if (rc == MQ_OK) scatter_pairs(dst, out, n_out, top_k, n);
     finish(o, rc);
+}
+
+void mq_cb_silu_mul_fused(struct ggml_tensor* dst, const struct ggml_tensor* a, const struct ggml_tensor* b, int ith, int /*nth*/,
+                          void* userdata) {
+    if (ith != 0) return;
+    Options o = options_for(userdata, 1);
+    t_resident = Resident{};
+    // the checks of cb_silu_mul_fused (core/src/llm/graph/fused_ops.cpp:317-340): anything else leaves dst untouched
+    int64_t rows = 0, cols = 0, rb = 0, cb = 0, rd = 0, cd = 0;
+    if (!dst || !rows_layout(a, &rows, &cols) || !rows_layout(b, &rb, &cb) || !rows_layout(dst, &rd, &cd) || rows != rb || cols != cb ||
+        rows != rd || cols != cd)
+        return finish(o, MQ_ERR_INVALID);
+    // contiguous tensors take the reference's SIMD routine (fused-multiply-add polynomial), strided ones its scalar
+    // loop with the exact exponential (fused_ops.cpp:342-365)
+    const bool contiguous = a->nb[1] == (size_t)cols * 4 && b->nb[1] == (size_t)cols * 4 && dst->nb[1] == (size_t)cols * 4;
+    const int mode = (o.ud && !o.ud->use_defaults) ? o.silu_mode : (contiguous ? MQ_SILU_FAST_FMA : MQ_SILU_EXACT);
+    int rc = MQ_OK;
+    const float* g_dev = operand_rows(a, rows, cols, &rc);
+    const float* u_dev = g_dev ? operand_rows(b, rows, cols, &rc) : nullptr;
+    if (!g_dev || !u_dev) return finish(o, rc);
+    KeptTensor* kout = nullptr;
+    Staging* out = &t_stage.out;
+    if (o.keep_hidden) {
+        kout = kept_slot(dst, rows, cols);
+        if (!kout) return finish(o, t_status);
+        out = &kout->buf;
+    } else {
+        kept_forget(dst);
+        if (!out->get((size_t)rows * cols * 4)) return finish(o, t_status);
+    }
+    rc = mq_silu_mul_f32(g_dev, u_dev, rows, cols, cols, cols, (float*)out->dev, cols, mode, nullptr);
+    deliver_rows(o, dst, kout, out, rows, cols, rc);
+}
+
+void mq_cb_apply_shared_scalar_gate(struct ggml_tensor* dst, const struct ggml_tensor* src, const struct ggml_tensor* gate_logits_scalar,
+                                    int ith, int /*nth*/, void* userdata) {
+    if (ith != 0) return;
+    Options o = options_for(userdata, 1);
+    t_resident = Resident{};
+    // the checks of cb_apply_shared_scalar_gate (core/src/llm/graph/fused_ops.cpp:437-449): hidden = src->ne[0], tokens =
+    // max(1, src->ne[1]), one logit per token at gate_logits_scalar row stride nb[1]
+    int64_t rows = 0, cols = 0, rd = 0, cd = 0;
+    if (!dst || !gate_logits_scalar || !gate_logits_scalar->data || gate_logits_scalar->type != GGML_TYPE_F32 ||
+        !rows_layout(src, &rows, &cols) || !rows_layout(dst, &rd, &cd) || rows != rd || cols != cd || src->ne[2] * src->ne[3] != 1)
+        return finish(o, MQ_ERR_INVALID);
+    const int64_t scalar_elems = gate_logits_scalar->ne[0] * gate_logits_scalar->ne[1] * gate_logits_scalar->ne[2] * gate_logits_scalar->ne[3];
+    if (scalar_elems < rows) return finish(o, MQ_ERR_INVALID);
+    int rc = MQ_OK;
+    const float* s_dev = operand_rows(src, rows, cols, &rc);
+    if (!s_dev) return finish(o, rc);
+    // the logits: one per token, gate_logits_scalar->nb[1] apart
+    const float* l_dev = nullptr;
+    if (KeptTensor* kl = kept_find(gate_logits_scalar, rows, gate_logits_scalar->ne[0])) {
+        l_dev = (const float*)kl->buf.dev;
+    } else {
+        Staging* lg = ring_slot((size_t)rows * 4);
+        if (!lg) return finish(o, t_status);
+        for (int64_t t = 0; t < rows; ++t) std::memcpy((char*)lg->pin + t * 4, (const char*)gate_logits_scalar->data + t * gate_logits_scalar->nb[1], 4);
+        rc = mq_memcpy_h2d_async(lg->dev, lg->pin, (size_t)rows * 4, nullptr);
+        if (rc != MQ_OK) return finish(o, rc);
+        l_dev = (const float*)lg->dev;
+    }
+    const int64_t ld_logit = kept_find(gate_logits_scalar, rows, gate_logits_scalar->ne[0]) ? gate_logits_scalar->ne[0] : 1;
+    KeptTensor* kout = nullptr;
+    Staging* out = &t_stage.out;
+    if (o.keep_hidden) {
+        kout = kept_slot(dst, rows, cols);
+        if (!kout) return finish(o, t_status);
+        out = &kout->buf;
+    } else {
+        kept_forget(dst);
+        if (!out->get((size_t)rows * cols * 4)) return finish(o, t_status);
+    }
+    rc = mq_scale_rows_sigmoid_f32(s_dev, rows, cols, cols, l_dev, ld_logit, (float*)out->dev, cols, nullptr);
+    deliver_rows(o, dst, kout, out, rows, cols, rc);
+}
+
+void mq_ggml_graph_begin(void) {
+    settle();
+    for (KeptTensor* k : t_kept) k->tensor = nullptr;
+    t_resident = Resident{};
+}
+
+int mq_ggml_tensor_to_host(struct ggml_tensor* t) {
+    int64_t rows = 0, cols = 0;
+    if (!rows_layout(t, &rows, &cols)) return 0;
+    KeptTensor* k = kept_find(t, rows, cols);
+    if (!k) return 0;
+    int rc = mq_memcpy_d2h_async(k->buf.pin, k->buf.dev, (size_t)rows * cols * 4, nullptr);
+    if (rc == MQ_OK) rc = mq_stream_synchronize(nullptr);
+    if (note(rc) != MQ_OK) return 0;
+    settled_by_sync();
+    scatter_rows(t->data, k->buf, 0, rows, cols, t->nb[1]);
+    return 1;
 }
 
 int mq_ggml_last_status(void) { return t_status; }

@@ -322,6 +322,18 @@ int mq_add_rmsnorm_router_f32(const float* x_dev, const float* delta_dev, const 
                               float eps, float* sum_out_dev, float* normed_out_dev, const float* router_dev, int64_t n_experts,
                               float* logits_dev, void* stream);
 
+/* ---- the two element-wise nodes of a dense FFN / shared expert as the graph emits them ---------------
+ * out[t][c] = silu(gate[t][c]) * up[t][c] over [n][cols] fp32 with row strides in floats: cb_silu_mul_fused
+ * (core/src/llm/graph/fused_ops.cpp:317-366).  The reference runs MQ_SILU_FAST_FMA on contiguous tensors
+ * (SiLUMulParallel, core/src/kernels/hwy/hwy_activation.cc:153-167) and MQ_SILU_EXACT on strided ones (:364). */
+int mq_silu_mul_f32(const float* gate_dev, const float* up_dev, int64_t n, int64_t cols, int64_t ld_gate, int64_t ld_up, float* out_dev,
+                    int64_t ld_out, int silu_mode, void* stream);
+/* out[t][c] = sigmoid(logit[t * ld_logit]) * src[t][c], the sigmoid two-sided (1 / (1 + e^-x) for x >= 0, e^x / (1 + e^x)
+ * below): cb_apply_shared_scalar_gate (core/src/llm/graph/fused_ops.cpp:437-475), the scalar gate on the shared expert's
+ * output. */
+int mq_scale_rows_sigmoid_f32(const float* src_dev, int64_t n, int64_t cols, int64_t ld_src, const float* logit_dev, int64_t ld_logit,
+                              float* out_dev, int64_t ld_out, void* stream);
+
 /* Verification hooks (per-super-block integer sums, work lists, intermediates), the launch census and the kernel
  * selection switch are declared in mi355_q4k_debug.h: test and measurement instruments, not part of what a host binds. */
 

@@ -55,6 +55,13 @@ typedef struct {
      * nothing but the down node reads the gate/up node's output (true of the native MoE graph); any other consumer
      * would read stale host memory. */
     int keep_hidden_on_device;
+    /* The same flag on a dense node (mq_cb_gemv_custom, mq_cb_gemv_batched_custom) or on one of the two element-wise
+     * nodes below: the node's result stays in HBM, dst->data is not written, nothing is waited for, and any later
+     * dense or element-wise node of the graph that names the tensor (or a view of all of it) as an operand reads it
+     * there -- gate -> up -> silu * up -> down -> scalar gate of a dense FFN or shared expert
+     * (core/src/llm/graph/decoder.cpp:2426-2600) cost one synchronisation, at the node that does not set the flag.
+     * Tensors are remembered by their ggml_tensor object for the calling thread until mq_ggml_graph_begin();
+     * mq_ggml_tensor_to_host() brings one back for a consumer that is not one of these nodes. */
 } mq_ggml_userdata;
 
 /* dst F32 ne=[N_out, M]; src[0] = input F32 ne=[K_in, M] (column stride nb[1]); src[1] = weight
@@ -96,6 +103,23 @@ void mq_cb_moe_topk_weights_from_logits(struct ggml_tensor* dst, int ith, int nt
  * The nodes emitted at core/src/llm/moe/native_gemma.cpp:1509-1559 (gate, up, gate_up and down of the routed
  * experts); rows whose id is outside [0, n_expert) come back as zeros. */
 void mq_cb_mul_mat_id(struct ggml_tensor* dst, int ith, int nth, void* userdata);
+
+/* The element-wise nodes between the products of a dense FFN / shared expert, with ggml_custom2_op_t's shape
+ * (ggml_map_custom2): void fn(dst, a, b, ith, nth, userdata); userdata NULL or mq_ggml_userdata*.
+ * dst = silu(a) * b, all F32 of one shape with unit element stride: cb_silu_mul_fused
+ * (core/src/llm/graph/fused_ops.cpp:317-366; contiguous tensors take MQ_SILU_FAST_FMA as SiLUMulParallel does,
+ * strided ones MQ_SILU_EXACT, unless userdata names a mode). */
+void mq_cb_silu_mul_fused(struct ggml_tensor* dst, const struct ggml_tensor* a, const struct ggml_tensor* b, int ith, int nth,
+                          void* userdata);
+/* dst[:, t] = sigmoid(gate_logits_scalar[t]) * src[:, t], src / dst F32 ne=[hidden, tokens], one logit per token at
+ * row stride nb[1]: cb_apply_shared_scalar_gate (core/src/llm/graph/fused_ops.cpp:437-475). */
+void mq_cb_apply_shared_scalar_gate(struct ggml_tensor* dst, const struct ggml_tensor* src, const struct ggml_tensor* gate_logits_scalar,
+                                    int ith, int nth, void* userdata);
+/* Forgets every tensor the calling thread's nodes left on the device (call where a graph compute starts: a tensor
+ * whose producer did not run through these adapters this time must not be answered from an old device copy). */
+void mq_ggml_graph_begin(void);
+/* Copies a tensor that a node left on the device into t->data (one synchronisation); 1 when it was there, else 0. */
+int mq_ggml_tensor_to_host(struct ggml_tensor* t);
 
 /* Status of the calling thread's last adapter call (MQ_OK / MQ_ERR_*). */
 int mq_ggml_last_status(void);
