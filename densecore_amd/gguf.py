@@ -13,6 +13,7 @@ from . import _lib, ggml_adapter, ops
 EXPORTS = [
     "mq_gguf_open", "mq_gguf_last_error", "mq_gguf_close", "mq_gguf_tensor_count", "mq_gguf_tensor_at",
     "mq_gguf_find_tensor", "mq_gguf_get_int", "mq_gguf_get_string", "mq_gguf_load_q4k", "mq_gguf_load_weight",
+    "mq_gguf_load_moe_layer", "mq_gguf_free_moe_layer",
 ]
 
 GGML_F32, GGML_F16, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_I32 = 0, 1, 12, 13, 14, 26
@@ -22,6 +23,57 @@ GGML_Q8_0 = 8
 class TensorInfo(C.Structure):
     _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_int32), ("n_dims", C.c_int32), ("ne", C.c_int64 * 4),
                 ("offset", C.c_uint64), ("nbytes", C.c_uint64), ("data", C.c_void_p)]
+
+
+class MoELayerStruct(C.Structure):
+    """mq_gguf_moe_layer (include/mi355_q4k_gguf.h)."""
+    _fields_ = [("desc", _lib.MoELayerDesc), ("owned", C.c_void_p * 6), ("router_dev", C.c_void_p), ("sh_gate_inp_dev", C.c_void_p),
+                ("n_experts", C.c_int64), ("hidden", C.c_int64), ("inter", C.c_int64)]
+
+
+class MoELayer:
+    """A layer loaded by mq_gguf_load_moe_layer: .desc for mq_moe_layer_q4k, .weights as ops.Q4KWeight views (not owning)."""
+
+    def __init__(self, raw: MoELayerStruct, types):
+        self.raw = raw
+        self.n_experts, self.hidden, self.inter = raw.n_experts, raw.hidden, raw.inter
+        self.top_k = raw.desc.top_k
+        shapes = [(self.inter, self.hidden, self.n_experts)] * 2 + [(self.hidden, self.inter, self.n_experts)] + \
+                 [(self.inter, self.hidden, 1)] * 2 + [(self.hidden, self.inter, 1)]
+        self.weights = [ops.Q4KWeight(raw.owned[i], r, c, e, types[i]) if raw.owned[i] else None
+                        for i, (r, c, e) in enumerate(shapes)]
+        self._freed = False
+
+    def run(self, x, logits, silu: int = ops.SILU_EXACT, route_mode: int = ops.ROUTE_FUSED, top_k: int = 0):
+        """mq_moe_layer_q4k on the loaded layer: returns (y, ids, weights)."""
+        import torch
+        self.raw.desc.top_k = top_k or self.top_k
+        self.raw.desc.silu_mode, self.raw.desc.route_mode = silu, route_mode
+        n, K = x.shape[0], self.raw.desc.top_k
+        y = torch.empty((n, self.hidden), dtype=torch.float32, device="cuda")
+        ids = torch.empty((n, K), dtype=torch.int32, device="cuda")
+        wts = torch.empty((n, K), dtype=torch.float32, device="cuda")
+        p = lambda t: C.c_void_p(t.data_ptr())
+        _lib.check(_lib.lib().mq_moe_layer_q4k(C.byref(self.raw.desc), p(x), p(logits), n, p(y), p(ids), p(wts),
+                                               C.c_void_p(torch.cuda.current_stream().cuda_stream)), "mq_moe_layer_q4k")
+        return y, ids, wts
+
+    def free(self):
+        """Frees the layer's device memory; its weight views stop being usable."""
+        if self._freed:
+            return
+        self._freed = True
+        for w in self.weights:           # views: the layer owns the handles, a view must not free its own
+            if w is not None:
+                w._h = C.c_void_p()
+        self.weights = []
+        lib().mq_gguf_free_moe_layer(C.byref(self.raw))
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
 
 
 _handle = None
@@ -45,6 +97,8 @@ def lib(need_gpu: bool = False):
         L.mq_gguf_get_string.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(C.c_size_t)]
         L.mq_gguf_load_q4k.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
         L.mq_gguf_load_weight.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+        L.mq_gguf_load_moe_layer.argtypes = [C.c_void_p, C.c_int, C.POINTER(MoELayerStruct)]
+        L.mq_gguf_free_moe_layer.argtypes = [C.POINTER(MoELayerStruct)]
         _handle = L
     if need_gpu:
         _lib.lib()
@@ -100,6 +154,23 @@ class GgufFile:
     def load_weight(self, name: str) -> "ops.Q4KWeight":
         """Upload a GGML_TYPE_Q4_K, Q5_K or Q6_K tensor ([K, N] or [K, N, E]) or a dense Q8_0 matrix to the GPU."""
         return self._load(name, "mq_gguf_load_weight")
+
+    def load_moe_layer(self, layer: int) -> MoELayer:
+        """Bind blk.<layer>'s expert stacks, shared expert, router and scalar gate to a MoE layer descriptor."""
+        lib(need_gpu=True)
+        raw = MoELayerStruct()
+        rc = lib().mq_gguf_load_moe_layer(self._h, layer, C.byref(raw))
+        if rc != 0:
+            _lib.check(rc, f"mq_gguf_load_moe_layer({layer}): {lib().mq_gguf_last_error().decode()}")
+        by_name = {t["name"]: t["type"] for t in self.tensors()}
+        pick = lambda *sfx: next((by_name[f"blk.{layer}.{s}"] for s in sfx if f"blk.{layer}.{s}" in by_name), 12)
+        types = [pick("ffn_gate_exps.weight", "ffn_gate_exps", "experts.gate_proj.weight"),
+                 pick("ffn_up_exps.weight", "ffn_up_exps", "experts.up_proj.weight"),
+                 pick("ffn_down_exps.weight", "ffn_down_exps", "experts.down_proj.weight"),
+                 pick("ffn_gate.weight", "ffn_gate_shexp.weight", "shared_expert.gate_proj.weight", "mlp.gate_proj.weight", "gate_proj.weight"),
+                 pick("ffn_up.weight", "ffn_up_shexp.weight", "shared_expert.up_proj.weight", "mlp.up_proj.weight", "up_proj.weight"),
+                 pick("ffn_down.weight", "ffn_down_shexp.weight", "shared_expert.down_proj.weight", "mlp.down_proj.weight", "down_proj.weight")]
+        return MoELayer(raw, types)
 
     def _load(self, name: str, entry: str) -> "ops.Q4KWeight":
         lib(need_gpu=True)

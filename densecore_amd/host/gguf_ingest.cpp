@@ -8,6 +8,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <initializer_list>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -294,5 +295,129 @@ int load_kquant(const mq_gguf* g, const char* name, bool q4k_only, mq_weight** o
 int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out) { return load_kquant(g, name, true, out); }
 
 int mq_gguf_load_weight(const mq_gguf* g, const char* name, mq_weight** out) { return load_kquant(g, name, false, out); }
+
+namespace {
+
+// The first of the reference's alternative names for a per-layer tensor that the file holds: "blk.<layer>.<suffix>"
+// (get_layer_tensor_any, core/src/models/model_loader.cpp:3802-3811).
+const mq_gguf_tensor* layer_tensor_any(const mq_gguf* g, int layer, std::initializer_list<const char*> suffixes) {
+    for (const char* suffix : suffixes) {
+        const std::string name = "blk." + std::to_string(layer) + "." + suffix;
+        const int64_t idx = mq_gguf_find_tensor(g, name.c_str());
+        if (idx >= 0) return &g->tensors[(size_t)idx];
+    }
+    return nullptr;
+}
+
+float half_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {  // subnormal: normalise
+            int e = -1;
+            uint32_t m = man;
+            do {
+                ++e;
+                m <<= 1;
+            } while (!(m & 0x400u));
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+
+// An F32 or F16 tensor of `count` elements as fp32 on the device.
+int upload_f32(const mq_gguf_tensor* t, int64_t count, float** out_dev) {
+    if (t->ggml_type != 0 && t->ggml_type != 1) return fail(std::string("tensor ") + t->name + " is neither F32 nor F16");
+    if (t->ne[0] * t->ne[1] * t->ne[2] * t->ne[3] != count) return fail(std::string("tensor ") + t->name + " has an unexpected shape");
+    std::vector<float> host((size_t)count);
+    if (t->ggml_type == 0) {
+        std::memcpy(host.data(), t->data, (size_t)count * 4);
+    } else {
+        const uint16_t* h = static_cast<const uint16_t*>(t->data);
+        for (int64_t i = 0; i < count; ++i) host[(size_t)i] = half_to_float(h[i]);
+    }
+    void* dev = nullptr;
+    if (int rc = mq_device_malloc(&dev, (size_t)count * 4)) return rc;
+    if (int rc = mq_memcpy_h2d(dev, host.data(), (size_t)count * 4)) {
+        mq_device_free(dev);
+        return rc;
+    }
+    *out_dev = static_cast<float*>(dev);
+    return MQ_OK;
+}
+
+}  // namespace
+
+int mq_gguf_free_moe_layer(mq_gguf_moe_layer* L) {
+    if (!L) return MQ_OK;
+    for (mq_weight*& w : L->owned) {
+        if (w) mq_weight_free(w);
+        w = nullptr;
+    }
+    if (L->router_dev) mq_device_free(L->router_dev);
+    if (L->sh_gate_inp_dev) mq_device_free(L->sh_gate_inp_dev);
+    *L = mq_gguf_moe_layer{};
+    return MQ_OK;
+}
+
+int mq_gguf_load_moe_layer(const mq_gguf* g, int layer_index, mq_gguf_moe_layer* out) {
+    if (!g || !out || layer_index < 0) return fail("null argument or negative layer");
+    *out = mq_gguf_moe_layer{};
+    // the stacked expert tensors (core/src/models/model_loader.cpp:231-235,4429-4440) ...
+    const mq_gguf_tensor* ge = layer_tensor_any(g, layer_index, {"ffn_gate_exps.weight", "ffn_gate_exps", "experts.gate_proj.weight"});
+    const mq_gguf_tensor* ue = layer_tensor_any(g, layer_index, {"ffn_up_exps.weight", "ffn_up_exps", "experts.up_proj.weight"});
+    const mq_gguf_tensor* de = layer_tensor_any(g, layer_index, {"ffn_down_exps.weight", "ffn_down_exps", "experts.down_proj.weight"});
+    if (!ge || !ue || !de) return fail("layer " + std::to_string(layer_index) + " holds no stacked ffn_{gate,up,down}_exps tensors");
+    // ... the shared expert, the router and the shared expert's scalar gate (:3961-4001)
+    const mq_gguf_tensor* sg = layer_tensor_any(g, layer_index, {"ffn_gate.weight", "ffn_gate_shexp.weight", "shared_expert.gate_proj.weight", "mlp.gate_proj.weight", "gate_proj.weight"});
+    const mq_gguf_tensor* su = layer_tensor_any(g, layer_index, {"ffn_up.weight", "ffn_up_shexp.weight", "shared_expert.up_proj.weight", "mlp.up_proj.weight", "up_proj.weight"});
+    const mq_gguf_tensor* sd = layer_tensor_any(g, layer_index, {"ffn_down.weight", "ffn_down_shexp.weight", "shared_expert.down_proj.weight", "mlp.down_proj.weight", "down_proj.weight"});
+    const mq_gguf_tensor* sgi = layer_tensor_any(g, layer_index, {"ffn_gate_inp_shexp.weight", "shared_expert_gate.weight"});
+    const mq_gguf_tensor* router = layer_tensor_any(g, layer_index, {"moe_gate.weight", "router.proj.weight", "mlp.gate.weight", "ffn_gate_inp.weight", "ffn_gate_inp"});
+    // layout facts of the stacks (core/src/llm/moe/native.cpp:4546-4548,4589-4597): gate / up [n_embd, n_ff, n_expert],
+    // down [n_ff, n_embd, n_expert]
+    const int64_t hidden = ge->ne[0], inter = ge->ne[1], E = ge->ne[2];
+    if (ue->ne[0] != hidden || ue->ne[1] != inter || ue->ne[2] != E || de->ne[0] != inter || de->ne[1] != hidden || de->ne[2] != E)
+        return fail("layer " + std::to_string(layer_index) + ": the expert stacks do not fit each other");
+    if ((sg || su || sd) && !(sg && su && sd)) return fail("layer " + std::to_string(layer_index) + ": an incomplete shared expert");
+    if (sg && (sg->ne[0] != hidden || sg->ne[1] != inter || su->ne[0] != hidden || su->ne[1] != inter || sd->ne[0] != inter || sd->ne[1] != hidden))
+        return fail("layer " + std::to_string(layer_index) + ": the shared expert does not have the routed experts' shape");
+    int rc = load_kquant(g, ge->name, false, &out->owned[0]);
+    if (rc == MQ_OK) rc = load_kquant(g, ue->name, false, &out->owned[1]);
+    if (rc == MQ_OK) rc = load_kquant(g, de->name, false, &out->owned[2]);
+    if (rc == MQ_OK && sg) rc = load_kquant(g, sg->name, false, &out->owned[3]);
+    if (rc == MQ_OK && sg) rc = load_kquant(g, su->name, false, &out->owned[4]);
+    if (rc == MQ_OK && sg) rc = load_kquant(g, sd->name, false, &out->owned[5]);
+    if (rc == MQ_OK && router) {
+        if (router->ne[0] != hidden || router->ne[1] != E) rc = fail(std::string("tensor ") + router->name + " is not [n_embd, n_expert]");
+        else rc = upload_f32(router, hidden * E, &out->router_dev);
+    }
+    if (rc == MQ_OK && sgi) rc = upload_f32(sgi, hidden, &out->sh_gate_inp_dev);
+    if (rc != MQ_OK) {
+        mq_gguf_free_moe_layer(out);
+        return rc;
+    }
+    out->desc.gate_exps = out->owned[0], out->desc.up_exps = out->owned[1], out->desc.down_exps = out->owned[2];
+    out->desc.shared_gate = out->owned[3], out->desc.shared_up = out->owned[4], out->desc.shared_down = out->owned[5];
+    out->desc.sh_gate_inp_dev = out->sh_gate_inp_dev;
+    out->n_experts = E, out->hidden = hidden, out->inter = inter;
+    // experts per token: "<architecture>.expert_used_count" (the key ggml model files carry)
+    const char* arch = nullptr;
+    size_t arch_len = 0;
+    int64_t used = 0;
+    if (mq_gguf_get_string(g, "general.architecture", &arch, &arch_len) == MQ_OK &&
+        mq_gguf_get_int(g, (std::string(arch, arch_len) + ".expert_used_count").c_str(), &used) == MQ_OK && used > 0 && used <= 8)
+        out->desc.top_k = (int)used;
+    return MQ_OK;
+}
 
 }  // extern "C"

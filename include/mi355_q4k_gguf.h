@@ -58,6 +58,24 @@ int mq_gguf_load_q4k(const mq_gguf* g, const char* name, mq_weight** out);
  * Q6_K. */
 int mq_gguf_load_weight(const mq_gguf* g, const char* name, mq_weight** out);
 
+/* One MoE layer of a model file bound to the descriptor mq_moe_layer_q4k takes: the stacked expert tensors
+ * blk.<layer>.ffn_{gate,up,down}_exps [K, N, E] (any type the product entry points multiply), the shared expert
+ * blk.<layer>.ffn_{gate,up,down}_shexp.weight when the layer has one, its scalar gate ffn_gate_inp_shexp.weight and the
+ * router ffn_gate_inp.weight (F32 or F16, uploaded as fp32) -- each under the alternative names the reference's loader
+ * tries, in its order (core/src/models/model_loader.cpp:231-235, 3961-4001, 4429-4440; stack layout
+ * core/src/llm/moe/native.cpp:4546-4548,4589-4597).  desc.top_k comes from "<general.architecture>.expert_used_count"
+ * when the file has it (else 0: the caller sets it); silu_mode and route_mode are left 0 for the caller.
+ * Everything is owned by the struct until mq_gguf_free_moe_layer. */
+typedef struct {
+    mq_moe_layer_desc desc;
+    mq_weight* owned[6];     /* gate_exps, up_exps, down_exps, shared gate / up / down (NULL without a shared expert) */
+    float* router_dev;       /* fp32 [n_experts][hidden] on the device, or NULL when the file has no router tensor */
+    float* sh_gate_inp_dev;  /* fp32 [hidden] or NULL */
+    int64_t n_experts, hidden, inter;
+} mq_gguf_moe_layer;
+int mq_gguf_load_moe_layer(const mq_gguf* g, int layer_index, mq_gguf_moe_layer* out);
+int mq_gguf_free_moe_layer(mq_gguf_moe_layer* layer);
+
 #ifdef __cplusplus
 }
 #endif
