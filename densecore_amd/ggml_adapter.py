@@ -60,7 +60,10 @@ _handle = None
 def lib():
     global _handle
     if _handle is None:
-        _lib.lib()  # the C ABI library first (loaded and initialised on device 0): the adapter library links against it
+        try:
+            _lib.lib()   # the C ABI library first, initialised on device 0: the adapter library links against it
+        except _lib.MqError:
+            _lib.load()  # no GPU: the host-only helpers (fingerprint, GGUF reader) still work, every node reports MQ_ERR_STATE
         if not os.path.exists(LIB_PATH):
             raise _lib.MqError(f"{LIB_PATH} is missing: run `make -C densecore_amd/host`")
         L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
