@@ -77,8 +77,30 @@ def lib() -> C.CDLL:
     return _lib
 
 
-def simd() -> C.CDLL:
-    global _simd
+def host_has_vnni() -> bool:
+    """AVX-512 VNNI with 256-bit vectors on this host (what liboracle_simd_vnni.so needs)."""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("flags"):
+                flags = set(line.split(":", 1)[1].split())
+                return {"avx512_vnni", "avx512vl", "avx512f", "avx512bw"} <= flags
+    except OSError:
+        pass
+    return False
+
+
+_simd_vnni = None
+
+
+def simd(isa: str = "avx2") -> C.CDLL:
+    """The threaded SIMD build: "avx2", "vnni" (AVX-512 VNNI; only load it where host_has_vnni()), or "best"."""
+    global _simd, _simd_vnni
+    if isa == "best":
+        isa = "vnni" if host_has_vnni() else "avx2"
+    if isa == "vnni":
+        if _simd_vnni is None:
+            _simd_vnni = _load("liboracle_simd_vnni.so")
+        return _simd_vnni
     if _simd is None:
         _simd = _load("liboracle_simd.so")
     return _simd
@@ -509,12 +531,12 @@ def moe_layer(gate_exps, up_exps, down_exps, hidden, inter, top_k, x, logits, sh
 
 
 # ---------------------------------------------------------------- timed SIMD baseline
-def simd_mul_mat_q4k_q8k(w, cols: int, q8, threads: int) -> np.ndarray:
+def simd_mul_mat_q4k_q8k(w, cols: int, q8, threads: int, isa: str = "avx2") -> np.ndarray:
     w = _c(w, np.uint8)
     q8 = _c(q8, np.uint8)
     rows, n = w.shape[0], q8.shape[0]
     out = np.zeros((n, rows), np.float32)
-    rc = simd().orc_simd_mul_mat_q4k_q8k(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
+    rc = simd(isa).orc_simd_mul_mat_q4k_q8k(_p(w), C.c_int64(rows), C.c_int64(cols), C.c_size_t(w.shape[1]), _p(q8),
                                          C.c_int64(n), C.c_size_t(q8.shape[1]), _p(out), C.c_int64(rows),
                                          C.c_int(threads))
     if rc:
@@ -522,11 +544,11 @@ def simd_mul_mat_q4k_q8k(w, cols: int, q8, threads: int) -> np.ndarray:
     return out
 
 
-def simd_ffn_swiglu(gate, up, down, hidden: int, inter: int, x, threads: int, silu=SILU_FAST_FMA) -> np.ndarray:
+def simd_ffn_swiglu(gate, up, down, hidden: int, inter: int, x, threads: int, silu=SILU_FAST_FMA, isa: str = "avx2") -> np.ndarray:
     gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
     x = _c(x, np.float32)
     y = np.zeros((x.shape[0], hidden), np.float32)
-    rc = simd().orc_simd_ffn_swiglu_q4k(_p(gate), _p(up), _p(down), C.c_int64(hidden), C.c_int64(inter), _p(x),
+    rc = simd(isa).orc_simd_ffn_swiglu_q4k(_p(gate), _p(up), _p(down), C.c_int64(hidden), C.c_int64(inter), _p(x),
                                         C.c_int64(x.shape[0]), _p(y), C.c_int(threads), C.c_int(silu))
     if rc:
         raise ValueError(f"orc_simd_ffn_swiglu_q4k rc={rc}")

@@ -9,6 +9,12 @@
  * the thread partition of core/src/llm/matmul/gemv_exec.cpp:376-380
  * (rows [ith*ceil(N/nth), ...) per thread, one thread quantizes first).
  * fp32 order = ORC_ORDER_AVX2 of the scalar oracle, bit for bit.
+ *
+ * Built a second time with -mavx512vnni -mavx512vl (liboracle_simd_vnni.so): the block product then is the
+ * reference's VNNI kernel's, _mm256_dpbusd_epi32 on the nibbles and the codes and a 32-bit multiply by the scale
+ * (ComputeMoEQ4KQ8KBatchedRowVnni, core/src/backend/cpu_backend_moe_raw_batched.inl:562-616).  Lane i of its eight
+ * sums holds the same four products of every 32-weight sub-block as the AVX2 form's, so the results are the same
+ * bits; it is the build the CPU baseline is timed with where the host has the instructions.
  */
 #define _GNU_SOURCE
 #include "q4k_oracle.h"
@@ -51,12 +57,17 @@ static void row_times_tile(const orc_block_q4k* w, int64_t nb, const uint8_t* q8
         uint8_t sc[8], mn[8];
         unpack_scales(w[b].scales, sc, mn);
         __m256i lo[4], hi[4], slo[4], shi[4];
+#if defined(__AVX512VNNI__) && defined(__AVX512VL__)
+        __m256i slo32[4], shi32[4];
+        for (int c = 0; c < 4; ++c) slo32[c] = _mm256_set1_epi32(sc[2 * c]), shi32[c] = _mm256_set1_epi32(sc[2 * c + 1]);
+#endif
         for (int c = 0; c < 4; ++c) {
             const __m256i bytes = _mm256_loadu_si256((const __m256i*)(w[b].qs + 32 * c));
             lo[c] = _mm256_and_si256(bytes, nib);
             hi[c] = _mm256_and_si256(_mm256_srli_epi16(bytes, 4), nib);
             slo[c] = _mm256_set1_epi16(sc[2 * c]);
             shi[c] = _mm256_set1_epi16(sc[2 * c + 1]);
+            (void)slo[c], (void)shi[c];  /* the VNNI build multiplies by the 32-bit copies */
         }
         const float wd = half_to_float(w[b].d), wm = half_to_float(w[b].dmin);
         for (int t = 0; t < m; ++t) {
@@ -67,8 +78,13 @@ static void row_times_tile(const orc_block_q4k* w, int64_t nb, const uint8_t* q8
             for (int c = 0; c < 4; ++c) {
                 const __m256i ya = _mm256_loadu_si256((const __m256i*)(y->qs + 64 * c));
                 const __m256i yb = _mm256_loadu_si256((const __m256i*)(y->qs + 64 * c + 32));
+#if defined(__AVX512VNNI__) && defined(__AVX512VL__)
+                const __m256i pa = _mm256_mullo_epi32(_mm256_dpbusd_epi32(_mm256_setzero_si256(), lo[c], ya), slo32[c]);
+                const __m256i pb = _mm256_mullo_epi32(_mm256_dpbusd_epi32(_mm256_setzero_si256(), hi[c], yb), shi32[c]);
+#else
                 const __m256i pa = _mm256_madd_epi16(slo[c], _mm256_maddubs_epi16(lo[c], ya));
                 const __m256i pb = _mm256_madd_epi16(shi[c], _mm256_maddubs_epi16(hi[c], yb));
+#endif
                 sum = _mm256_add_epi32(sum, _mm256_add_epi32(pa, pb));
             }
             const float d = wd * y->d;
@@ -78,6 +94,15 @@ static void row_times_tile(const orc_block_q4k* w, int64_t nb, const uint8_t* q8
         }
     }
     memcpy(out, acc, sizeof(float) * (size_t)m);
+}
+
+/* 2: this build multiplies with AVX-512 VNNI (256-bit), 1: with AVX2. */
+int orc_simd_isa(void) {
+#if defined(__AVX512VNNI__) && defined(__AVX512VL__)
+    return 2;
+#else
+    return 1;
+#endif
 }
 
 typedef struct {

@@ -272,6 +272,25 @@ def test_simd_baseline_is_bitwise_the_avx2_order():
         assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
 
 
+@pytest.mark.skipif(not orc.host_has_vnni(), reason="this host has no AVX-512 VNNI")
+def test_vnni_build_of_the_baseline_is_bitwise_the_avx2_build():
+    """The reference's VNNI kernel (cpu_backend_moe_raw_batched.inl:562-616) keeps the AVX2 kernel's eight lanes: the
+    two builds of the baseline must agree bit for bit, for a product and for the whole FFN."""
+    assert orc.simd("vnni").orc_simd_isa() == 2 and orc.simd("avx2").orc_simd_isa() == 1
+    cols, rows = 2048, 96
+    w = synth.q4k_matrix(271, rows, cols)
+    q8 = orc.quantize_rows_q8k(synth.normal_f32(272, (5, cols)))
+    a = orc.simd_mul_mat_q4k_q8k(w, cols, q8, 3, isa="avx2")
+    b = orc.simd_mul_mat_q4k_q8k(w, cols, q8, 3, isa="vnni")
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(a.view(np.uint32), orc.mul_mat_q4k_q8k(w, cols, q8, orc.ORDER_AVX2).view(np.uint32))
+    H, I = 512, 768
+    g, u, d = synth.q4k_matrix(273, I, H), synth.q4k_matrix(274, I, H), synth.q4k_matrix(275, H, I)
+    x = synth.normal_f32(276, (3, H))
+    assert np.array_equal(orc.simd_ffn_swiglu(g, u, d, H, I, x, 2, isa="vnni").view(np.uint32),
+                          orc.simd_ffn_swiglu(g, u, d, H, I, x, 2, isa="avx2").view(np.uint32))
+
+
 def test_simd_ffn_baseline_matches_scalar_oracle():
     H, I, n = 512, 768, 3
     g, u, d = synth.q4k_matrix(55, I, H), synth.q4k_matrix(56, I, H), synth.q4k_matrix(57, H, I)
