@@ -99,10 +99,13 @@ __device__ __forceinline__ void a_codes_from_lane_codes(ACodes& a, const Q8Lane&
 }
 
 __device__ __forceinline__ void a_from_codes(ARegs<1>& a, const ACodes& s, int lane) {
-    const int slot = lane & 15;
+    // Slot 0 holds the codes in its first half and zeros in the second, slot 1 the other way round (the lanes of odd
+    // slots fetched the odd sub-block's codes).  Slots 2..15 belong to rows nobody stores, and every output row of
+    // the product depends on its own operand row only: they take the same pattern by slot parity, which costs two
+    // masks instead of a three-way choice per register.
+    const uint32_t even = (lane & 1) ? 0u : 0xffffffffu, odd = ~even;
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-        a.q[0][c] = slot == 0 ? v4u{s.lo[c], s.hi[c], 0u, 0u} : (slot == 1 ? v4u{0u, 0u, s.lo[c], s.hi[c]} : v4u{0u, 0u, 0u, 0u});
+    for (int c = 0; c < 4; ++c) a.q[0][c] = v4u{s.lo[c] & even, s.hi[c] & even, s.lo[c] & odd, s.hi[c] & odd};
     a.yd[0][0] = s.d;
     a.yd[0][1] = 0.0f;
 }
