@@ -71,6 +71,10 @@ def main() -> int:
                     help="only run the 14336x4096 prefill GEMM at M = 2048 ten times (for counter passes) and exit")
     ap.add_argument("--decode-step-only", type=int, default=0, metavar="N",
                     help="only replay the 40-layer decoder step at N tokens ten times, one launch per graph node (for kernel traces), and exit")
+    ap.add_argument("--skeleton", action="store_true",
+                    help="with --decode-step-only: time the step's graph, then the same graph captured with every kernel body "
+                         "compiled out (mq_debug_set_skeleton: empty kernels of the same grid, block and LDS size) -- the "
+                         "cost of the dependent launches alone")
     ap.add_argument("--moe-layer-only", type=int, default=0, metavar="N",
                     help="only run the cfg3 MoE layer (256 + 1 experts, 2048 x 512, top-8) at N tokens forty times over a ring "
                          "of 4 layers (for kernel traces), and exit")
@@ -123,7 +127,36 @@ def main() -> int:
         for _ in range(10):
             st.replay()
         torch.cuda.synchronize()
-        print(json.dumps({"decode_step_only": n, "layers": cfg.n_layers, "replays": 10}))
+        out = {"decode_step_only": n, "layers": cfg.n_layers, "replays": 10}
+        if args.skeleton:
+            from densecore_amd import _lib
+
+            def timed(step):
+                best = float("inf")
+                for _ in range(5):
+                    t = time.perf_counter()
+                    for _ in range(10):
+                        step.replay()
+                    torch.cuda.synchronize()
+                    best = min(best, (time.perf_counter() - t) / 10)
+                return best
+
+            full = timed(st)
+            _lib.lib().mq_debug_set_skeleton(1)
+            try:
+                sk = decode_step.DecodeStep(cfg, n, layers=st.layers)
+                sk.x.copy_(x)
+                sk.capture()
+            finally:
+                _lib.lib().mq_debug_set_skeleton(0)
+            sk.replay()
+            torch.cuda.synchronize()
+            floor = timed(sk)
+            out.update({"ms_per_step": round(full * 1e3, 3), "skeleton_ms_per_step": round(floor * 1e3, 3),
+                        "us_per_layer": round(full * 1e6 / cfg.n_layers, 2),
+                        "skeleton_us_per_layer": round(floor * 1e6 / cfg.n_layers, 2),
+                        "note": "skeleton = the same graph with empty kernels of the same grid, block and LDS size"})
+        print(json.dumps(out))
         return 0
 
     if args.moe_layer_only:

@@ -25,7 +25,7 @@ EXPORTS = [
 # every symbol include/mi355_q4k_debug.h declares (verification hooks and measurement instruments)
 DEBUG_EXPORTS = [
     "mq_debug_block_sums", "mq_debug_moe_groups", "mq_debug_moe_hidden", "mq_debug_decoder_buffers",
-    "mq_census_enable", "mq_census_reset", "mq_census_read", "mq_debug_set_dense_lds",
+    "mq_census_enable", "mq_census_reset", "mq_census_read", "mq_debug_set_dense_lds", "mq_debug_set_skeleton",
 ]
 
 
@@ -111,6 +111,7 @@ def load() -> C.CDLL:
     L.mq_mul_mat_q4k_acts.argtypes = [vp, vp, vp, i64, vp]
     L.mq_swiglu_mul_mat_q4k_acts.argtypes = [vp, vp, vp, vp, i64, ci, vp]
     L.mq_census_enable.argtypes = [ci]
+    L.mq_debug_set_skeleton.argtypes = [ci]
     L.mq_census_read.argtypes = [ci, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)]
     L.mq_device_malloc.argtypes = [C.POINTER(vp), sz]
     L.mq_device_free.argtypes = [vp]

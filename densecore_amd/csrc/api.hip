@@ -1873,6 +1873,13 @@ int mq_debug_set_dense_lds(int on) {
     return before;
 }
 
+int mq_debug_set_skeleton(int on) {
+    std::lock_guard<std::recursive_mutex> lock(g.mu);
+    const int before = g_skeleton;
+    g_skeleton = on != 0;
+    return before;
+}
+
 int mq_census_enable(int on) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     census.on = on != 0;

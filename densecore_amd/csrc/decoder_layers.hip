@@ -609,7 +609,7 @@ hipError_t launch_decoder_layers(const DecoderArgs& a, int n_workgroups, hipStre
         a.hidden <= 0 || (a.hidden % kQK) || a.inter <= 0 || (a.inter % kQK) || a.inter > kMaxInterBlocks * kQK ||
         n_workgroups < 1 || a.n_q <= 0 || (a.n_q % kQK))
         return hipErrorInvalidValue;
-    hipLaunchKernelGGL(decoder_layers_kernel, dim3((unsigned)n_workgroups), dim3(kThreads), decoder_layers_lds_bytes(a),
+    MQ_LAUNCH(decoder_layers_kernel, dim3((unsigned)n_workgroups), dim3(kThreads), decoder_layers_lds_bytes(a),
                        stream, a);
     return hipGetLastError();
 }

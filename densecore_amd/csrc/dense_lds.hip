@@ -263,7 +263,7 @@ hipError_t launch_odd(const DenseLdsArgs& a, hipStream_t stream, hipEvent_t star
     constexpr int RPW = 8 / WPR;
     const dim3 grid((unsigned)((rowtiles + RPW - 1) / RPW));
     if (start && stop) hipExtLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, start, stop, 0, a);
-    else hipLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, a);
+    else MQ_LAUNCH(kernel, grid, dim3(512), lds, stream, a);
     return hipGetLastError();
 }
 

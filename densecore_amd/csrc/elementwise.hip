@@ -346,7 +346,7 @@ hipError_t launch_add_rmsnorm_router(const float* x, const float* delta, const f
                                      hipStream_t stream) {
     if (n == 0) return hipSuccess;
     if ((cols % kQK) || cols > 4 * 4 * kQK || n > 65535 || n_experts <= 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(add_rmsnorm_router_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256),
+    MQ_LAUNCH(add_rmsnorm_router_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256),
                        (size_t)cols * sizeof(float), stream, x, delta, weight, cols, eps, sum_out, normed_out, w_router, n_experts,
                        logits);
     return hipGetLastError();
@@ -361,13 +361,13 @@ hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* w
                                             reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(sum_out) |
                                             reinterpret_cast<uintptr_t>(normed_out)) & 15u) == 0;
     if (vec && cols <= 4 * 4 * kQK) {
-        hipLaunchKernelGGL(add_rmsnorm_blocks_kernel<4>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
+        MQ_LAUNCH(add_rmsnorm_blocks_kernel<4>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
                            sum_out, normed_out, q_aq, q_ad);
     } else if (vec) {
-        hipLaunchKernelGGL(add_rmsnorm_blocks_kernel<0>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
+        MQ_LAUNCH(add_rmsnorm_blocks_kernel<0>, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps,
                            sum_out, normed_out, q_aq, q_ad);
     } else {
-        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
+        MQ_LAUNCH(add_rmsnorm_kernel, dim3((unsigned)n), dim3(256), 0, stream, x, delta, weight, cols, eps, sum_out,
                            normed_out, q_aq, q_ad);
     }
     return hipGetLastError();
@@ -377,7 +377,7 @@ hipError_t launch_router_logits(const float* w, int64_t n_experts, int64_t cols,
                                 float* logits, hipStream_t stream) {
     if (n == 0) return hipSuccess;
     if (n > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(router_logits_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256), 0, stream, w,
+    MQ_LAUNCH(router_logits_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n), dim3(256), 0, stream, w,
                        n_experts, cols, x, ldx, logits);
     return hipGetLastError();
 }
@@ -386,7 +386,7 @@ hipError_t launch_silu_mul(const float* gate, const float* up, int64_t n, int64_
                            int64_t ld_out, int mode, hipStream_t stream) {
     if (n * cols == 0) return hipSuccess;
     if (n * cols >= (int64_t)1 << 31) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, gate, up, n, cols, ld_gate, ld_up,
+    MQ_LAUNCH(silu_mul_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, gate, up, n, cols, ld_gate, ld_up,
                        out, ld_out, mode);
     return hipGetLastError();
 }
@@ -395,7 +395,7 @@ hipError_t launch_scale_rows_sigmoid(const float* src, int64_t n, int64_t cols, 
                                      float* out, int64_t ld_out, hipStream_t stream) {
     if (n * cols == 0) return hipSuccess;
     if (n * cols >= (int64_t)1 << 31) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(scale_rows_sigmoid_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, src, n, cols, ld_src,
+    MQ_LAUNCH(scale_rows_sigmoid_kernel, dim3((unsigned)((n * cols + 255) / 256)), dim3(256), 0, stream, src, n, cols, ld_src,
                        logit, ld_logit, out, ld_out);
     return hipGetLastError();
 }

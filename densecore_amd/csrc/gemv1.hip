@@ -360,7 +360,7 @@ hipError_t launch_gemvn_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
     const int64_t rowtiles = (rows + 15) / 16;
     const size_t lds = (size_t)waves * (8 * 256 + 32) + (waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0);
 #define MQ_GEMVN(NORM, RMAX)                                                                                                 \
-    hipLaunchKernelGGL((gemvn_fused_kernel<NORM, RMAX>), dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx, \
+    MQ_LAUNCH((gemvn_fused_kernel<NORM, RMAX>), dim3((unsigned)rowtiles), dim3(64 * waves), lds, stream, w, rows, nb, x, ldx, \
                        delta, weight, eps, sum_out, y, ldy, n)
     if (norm) {
         if (n <= 2) MQ_GEMVN(true, 2);
@@ -379,7 +379,7 @@ hipError_t launch_gemv1_norm_fused(const uint8_t* w, int64_t rows, int64_t nb, c
                                    const float* weight, float eps, float* sum_out, float* y, int waves, hipStream_t stream) {
     if (!gemv1_fused_applies(nb, waves) || rows <= 0) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16;
-    hipLaunchKernelGGL(gemv1_norm_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
+    MQ_LAUNCH(gemv1_norm_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 64 * sizeof(float) : 0, stream, w, rows, nb, x, delta, weight, eps, sum_out,
                        y);
     return hipGetLastError();
@@ -391,7 +391,7 @@ hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
                               hipStream_t stream) {
     if (!gemv1_fused_applies(nb, waves) || rows <= 0) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16;
-    hipLaunchKernelGGL(gemv1_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
+    MQ_LAUNCH(gemv1_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 64 * sizeof(float) : 0, stream, w, rows, nb, x, y);
     return hipGetLastError();
 }

@@ -271,7 +271,7 @@ hipError_t launch_wt(const MatmulArgs& a, dim3 grid, hipStream_t stream, hipEven
         raised = true;
     }
     if (start && stop) hipExtLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, start, stop, 0, a);
-    else hipLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, a);
+    else MQ_LAUNCH(kernel, grid, dim3(512), lds, stream, a);
     return hipGetLastError();
 }
 

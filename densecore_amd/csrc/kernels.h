@@ -238,6 +238,18 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,
                               const float* x, float* y, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream);
+// A measurement instrument (mq_debug_set_skeleton): while it is on, every launch of the compute and routing kernels
+// is replaced by a kernel with an empty body and the same grid, block and LDS size -- a captured graph then has the
+// dependent launches of the real one and none of their work, which is what the launches alone cost.  Weight set-up
+// and launches that carry timing events are not replaced.
+extern int g_skeleton;
+hipError_t launch_skeleton(dim3 grid, dim3 block, size_t lds, hipStream_t stream);
+#define MQ_LAUNCH(kernel, grid, block, lds, stream, ...)                            \
+    do {                                                                            \
+        if (::mq::g_skeleton) (void)::mq::launch_skeleton(grid, block, lds, stream); \
+        else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);     \
+    } while (0)
+
 // The work list written out as (expert, token, k) triples in list order, and the number of entries.
 hipError_t launch_flatten_groups(const int32_t* group_expert, const int32_t* group_begin, const int32_t* n_groups,
                                  const int32_t* entry_token, const int32_t* entry_k, int max_entries, int32_t* triples,

@@ -383,7 +383,7 @@ hipError_t launch_one(const MatmulArgs& a, int waves, dim3 grid, hipStream_t str
         hipExtLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ, REUSE_A, BM>), grid, dim3(64 * waves), lds, stream, start, stop,
                               0, a);
     } else {
-        hipLaunchKernelGGL((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ, REUSE_A, BM>), grid, dim3(64 * waves), lds, stream, a);
+        MQ_LAUNCH((matmul_kernel<NMAT, TT, GROUPED, DEBUG, WT, J, XQ, REUSE_A, BM>), grid, dim3(64 * waves), lds, stream, a);
     }
     return hipGetLastError();
 }

@@ -345,17 +345,17 @@ hipError_t launch_moe_down_token(const MoeDownTokenArgs& a, hipStream_t stream) 
             b.rt_per_wg = r_wg;
             b.inv_items = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)n_items) + 1u;
             const dim3 grid_rows((unsigned)(rowtiles / r_wg), (unsigned)a.n);
-            if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_down_rows_kernel<kWtQ6>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
-            else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_down_rows_kernel<kWtQ5>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
-            else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_down_rows_kernel<kWtQ4>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
+            if (a.wtype == kTypeQ6K) MQ_LAUNCH(moe_down_rows_kernel<kWtQ6>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
+            else if (a.wtype == kTypeQ5K) MQ_LAUNCH(moe_down_rows_kernel<kWtQ5>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
+            else if (a.wtype == kTypeQ4K) MQ_LAUNCH(moe_down_rows_kernel<kWtQ4>, grid_rows, dim3(kWaves * 64), lds_rows, stream, b);
             else return hipErrorInvalidValue;
             return hipGetLastError();
         }
     }
 #define MQ_DOWN_TOKEN(WT)                                                                                              \
     do {                                                                                                               \
-        if (a.hidden) hipLaunchKernelGGL((moe_down_token_kernel<WT, true>), grid, dim3(kWaves * 64), lds, stream, b);  \
-        else hipLaunchKernelGGL((moe_down_token_kernel<WT, false>), grid, dim3(kWaves * 64), lds, stream, b);          \
+        if (a.hidden) MQ_LAUNCH((moe_down_token_kernel<WT, true>), grid, dim3(kWaves * 64), lds, stream, b);  \
+        else MQ_LAUNCH((moe_down_token_kernel<WT, false>), grid, dim3(kWaves * 64), lds, stream, b);          \
     } while (0)
     if (a.wtype == kTypeQ6K) MQ_DOWN_TOKEN(kWtQ6);
     else if (a.wtype == kTypeQ5K) MQ_DOWN_TOKEN(kWtQ5);

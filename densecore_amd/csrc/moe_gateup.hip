@@ -346,9 +346,9 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
             const dim3 grid((unsigned)((a.rows + 15) / 16), (unsigned)runs, (unsigned)a.n);
             const size_t lds = (size_t)a.nb * 256 + (size_t)((a.nb + 63) & ~(int64_t)63) * 4 + (size_t)per_wg * (a.waves - 1) * 2 * 64 * 4;
             const dim3 block(64 * per_wg * a.waves);
-            if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ6>, grid, block, lds, stream, b);
-            else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ5>, grid, block, lds, stream, b);
-            else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_slots_kernel<kWtQ4>, grid, block, lds, stream, b);
+            if (a.wtype == kTypeQ6K) MQ_LAUNCH(moe_gateup_slots_kernel<kWtQ6>, grid, block, lds, stream, b);
+            else if (a.wtype == kTypeQ5K) MQ_LAUNCH(moe_gateup_slots_kernel<kWtQ5>, grid, block, lds, stream, b);
+            else if (a.wtype == kTypeQ4K) MQ_LAUNCH(moe_gateup_slots_kernel<kWtQ4>, grid, block, lds, stream, b);
             else return hipErrorInvalidValue;
             return hipGetLastError();
         }
@@ -357,9 +357,9 @@ hipError_t launch_moe_gateup_token(const MoeGateupTokenArgs& a, hipStream_t stre
     MoeGateupTokenArgs b = a;
     b.stages = (int)(a.nb / a.waves);
     const size_t lds = a.waves > 1 ? (size_t)(a.waves - 1) * 2 * 64 * sizeof(float) : 0;
-    if (a.wtype == kTypeQ6K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ6>, grid, dim3(64 * a.waves), lds, stream, b);
-    else if (a.wtype == kTypeQ5K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ5>, grid, dim3(64 * a.waves), lds, stream, b);
-    else if (a.wtype == kTypeQ4K) hipLaunchKernelGGL(moe_gateup_token_kernel<kWtQ4>, grid, dim3(64 * a.waves), lds, stream, b);
+    if (a.wtype == kTypeQ6K) MQ_LAUNCH(moe_gateup_token_kernel<kWtQ6>, grid, dim3(64 * a.waves), lds, stream, b);
+    else if (a.wtype == kTypeQ5K) MQ_LAUNCH(moe_gateup_token_kernel<kWtQ5>, grid, dim3(64 * a.waves), lds, stream, b);
+    else if (a.wtype == kTypeQ4K) MQ_LAUNCH(moe_gateup_token_kernel<kWtQ4>, grid, dim3(64 * a.waves), lds, stream, b);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

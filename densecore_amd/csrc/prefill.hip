@@ -677,7 +677,7 @@ hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_ex
     int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
     const int64_t rows_max = 16 * moe_gemm_tiles_max(entries, groups_max);
     const unsigned wgs = (unsigned)(rows_max / 1024 < 1 ? 1 : (rows_max / 1024 > 64 ? 64 : rows_max / 1024));
-    hipLaunchKernelGGL(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 2) * sizeof(int32_t), stream, n_groups,
+    MQ_LAUNCH(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 2) * sizeof(int32_t), stream, n_groups,
                        group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, (int)sh_tokens,
                        slots - 1, sh_silu_mode, plan, row_src, out_row);
     return hipGetLastError();
@@ -694,11 +694,11 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
     const int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     if (swiglu) {
-        hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x, x2, silu_mode,
+        MQ_LAUNCH(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x, x2, silu_mode,
                            h_out, ldh, m_tiles * 16, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr,
                            row_src + 16 * m_tiles);
     } else {
-        hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
+        MQ_LAUNCH(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
                            (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, m_tiles * 16, ldx, nb, m_tiles, ap, plan, row_src,
                            (const int32_t*)nullptr);
     }
@@ -726,15 +726,15 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expe
     }
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
     if (wtype == kTypeQ6K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ6>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ6>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
                            2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
                            (int64_t)0, plan, expert_bytes, out_row, w_shared);
     } else if (wtype == kTypeQ5K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ5>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ5>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
                            2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
                            (int64_t)0, plan, expert_bytes, out_row, w_shared);
     } else {
-        hipLaunchKernelGGL(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
+        MQ_LAUNCH(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
                            2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
                            (int64_t)0, plan, expert_bytes, out_row, w_shared);
     }
@@ -753,7 +753,7 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
     if (m_tiles == 0 || nb == 0) return hipSuccess;
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
+    MQ_LAUNCH(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
                        (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr,
                        (const int32_t*)nullptr, (const int32_t*)nullptr);
     return hipGetLastError();
@@ -764,7 +764,7 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
     const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
     if (m_tiles == 0 || nb == 0) return hipSuccess;
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, gate, up,
+    MQ_LAUNCH(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, gate, up,
                        silu_mode, h_out, ldh, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr, (const int32_t*)nullptr,
                        (const int32_t*)nullptr);
     return hipGetLastError();
@@ -793,26 +793,26 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
     const int64_t stride = split ? n * rows : 0;
     const dim3 grid(ps.row_wgs, ps.groups, (unsigned)ps.splits);
     if (wtype == kTypeQ6K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ6>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ6>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);
     } else if (wtype == kTypeQ5K) {
-        hipLaunchKernelGGL((prefill_gemm_kernel<1, kWtQ5>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ5>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);
     } else if (ps.narrow) {
-        hipLaunchKernelGGL(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+        MQ_LAUNCH(prefill_gemm_kernel<1>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);
     } else {
-        hipLaunchKernelGGL(prefill_gemm_kernel<2>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
+        MQ_LAUNCH(prefill_gemm_kernel<2>, grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb,
                            ap, m_tiles, n, out, ld, ps.sb_split, stride, (const int32_t*)nullptr, (int64_t)0, (const int32_t*)nullptr,
                            (const uint8_t*)nullptr);
     }
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     if (split) {
         const int64_t units = n * (rows >> 2);
-        hipLaunchKernelGGL(prefill_sum_planes_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, part, ps.splits, n,
+        MQ_LAUNCH(prefill_sum_planes_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, part, ps.splits, n,
                            rows, y, ldy);
     }
     return hipGetLastError();

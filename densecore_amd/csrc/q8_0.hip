@@ -230,7 +230,7 @@ hipError_t launch_quantize_q80(const float* x, int64_t n, int64_t ldx, int64_t c
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     if ((cols % kQK) || ldx < cols || (ldx & 3) || (reinterpret_cast<uintptr_t>(x) & 15u)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(quantize_q80_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx, nb, aq, ah);
+    MQ_LAUNCH(quantize_q80_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, ldx, nb, aq, ah);
     return hipGetLastError();
 }
 
@@ -245,14 +245,14 @@ hipError_t launch_q80_matmul(const Q80MatmulArgs& a, hipStream_t stream) {
         const int64_t columns = (int64_t)a.max_groups + (a.sh_tokens + kTokTile - 1) / kTokTile;
         if (columns > 65535) return hipErrorInvalidValue;
         const int waves = pick_waves(a.nb, rowtiles * columns);
-        hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)rowtiles, (unsigned)columns), dim3(64 * waves),
+        MQ_LAUNCH(q80_matmul_kernel, dim3((unsigned)rowtiles, (unsigned)columns), dim3(64 * waves),
                            waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0, stream, a);
         return hipGetLastError();
     }
     const int64_t columns = a.pair_ids ? a.n : 1;
     if (rowtiles * columns >= (int64_t)1 << 31) return hipErrorInvalidValue;
     const int waves = pick_waves(a.nb, rowtiles * columns);
-    hipLaunchKernelGGL(q80_matmul_kernel, dim3((unsigned)(rowtiles * columns)), dim3(64 * waves),
+    MQ_LAUNCH(q80_matmul_kernel, dim3((unsigned)(rowtiles * columns)), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 2 * 64 * sizeof(float) : 0, stream, a);
     return hipGetLastError();
 }

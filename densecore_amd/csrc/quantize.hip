@@ -56,7 +56,7 @@ hipError_t launch_quantize_q8k(const float* x, int64_t n, int64_t ldx, int64_t k
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     const unsigned grid = (unsigned)((units + 3) / 4);
-    hipLaunchKernelGGL(quantize_q8k_kernel, dim3(grid), dim3(256), 0, stream, x, n, ldx, nb, (uint8_t*)q8_std,
+    MQ_LAUNCH(quantize_q8k_kernel, dim3(grid), dim3(256), 0, stream, x, n, ldx, nb, (uint8_t*)q8_std,
                        q8_row_bytes, aq, ad);
     return hipGetLastError();
 }
@@ -68,7 +68,7 @@ hipError_t launch_q8k_to_amajor(const void* q8_std, int64_t n, size_t q8_row_byt
     if (units == 0) return hipSuccess;
     if (units >= (int64_t)1 << 31) return hipErrorInvalidValue;  // split_unit divides in 32 bits
     const unsigned grid = (unsigned)((units + 3) / 4);
-    hipLaunchKernelGGL(q8k_to_amajor_kernel, dim3(grid), dim3(256), 0, stream, (const uint8_t*)q8_std, n, q8_row_bytes,
+    MQ_LAUNCH(q8k_to_amajor_kernel, dim3(grid), dim3(256), 0, stream, (const uint8_t*)q8_std, n, q8_row_bytes,
                        nb, aq, ad);
     return hipGetLastError();
 }

@@ -442,13 +442,28 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, s
     for (; i < count; i += stride) p[i] = 0.0f;
 }
 
+__global__ void __launch_bounds__(1024) skeleton_kernel() {}
+
 }  // namespace
+
+int g_skeleton = 0;
+
+hipError_t launch_skeleton(dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skeleton_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(skeleton_kernel, grid, block, lds, stream);
+    return hipGetLastError();
+}
 
 hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, int top_k, int mode, int32_t* ids,
                              float* weights, hipStream_t stream) {
     if (n_experts > kMaxExperts || top_k > 8) return hipErrorInvalidValue;
     const size_t lds = (size_t)(n_experts > kRouteScratch ? n_experts : kRouteScratch) * 8 + 64;
-    hipLaunchKernelGGL(route_topk_kernel, dim3((unsigned)n), dim3(256), lds, stream, logits, (int)n_experts, top_k, mode,
+    MQ_LAUNCH(route_topk_kernel, dim3((unsigned)n), dim3(256), lds, stream, logits, (int)n_experts, top_k, mode,
                        ids, weights);
     return hipGetLastError();
 }
@@ -456,7 +471,7 @@ hipError_t launch_route_topk(const float* logits, int64_t n_experts, int64_t n, 
 hipError_t launch_weights_from_ids(const float* logits, int64_t n_experts, int64_t n, const int32_t* ids, int top_k,
                                    float* weights, hipStream_t stream) {
     if (top_k > 8 || top_k <= 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(weights_from_ids_kernel, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, stream, logits,
+    MQ_LAUNCH(weights_from_ids_kernel, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, stream, logits,
                        (int)n_experts, (int)n, ids, top_k, weights);
     return hipGetLastError();
 }
@@ -488,7 +503,7 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     // placing a pair is a population count over its expert's mask words and two scattered stores: beyond a few thousand
     // pairs several workgroups share that part (each repeats the cheap counting): 43 -> 16 us at 16384 pairs
     const unsigned parts = entries >= 3072 ? 8u : 1u;
-    hipLaunchKernelGGL(build_groups_kernel, dim3(parts), dim3(threads), lds, stream, ids, (int)entries, top_k,
+    MQ_LAUNCH(build_groups_kernel, dim3(parts), dim3(threads), lds, stream, ids, (int)entries, top_k,
                        (int)n_experts, use_lds, mask_words, group_expert, group_begin, n_groups, entry_token, entry_k);
     return hipGetLastError();
 }
@@ -523,7 +538,7 @@ hipError_t launch_route_and_group(const float* logits, int64_t n_experts, int64_
     const int64_t per_block = block / 64;
     const int64_t quant_blocks = qx ? (n * q_nb + per_block - 1) / per_block : 0;
     const size_t lds = wave_parallel ? lds_wave : (lds_route > lds_group ? lds_route : lds_group);
-    hipLaunchKernelGGL(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(block), lds, stream, logits,
+    MQ_LAUNCH(route_and_group_kernel, dim3((unsigned)(route_blocks + quant_blocks)), dim3(block), lds, stream, logits,
                        (int)n_experts, (int)n, top_k, mode, ids, weights, arrivals, group_expert, group_begin, n_groups,
                        entry_token, entry_k, build_groups ? 1 : 0, route_blocks, mask_words, wave_parallel ? 1 : 0, qx, q_ldx,
                        q_nb, q_aq, q_ad);
@@ -534,7 +549,7 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
                               const int32_t* ids, int64_t n_experts, int has_shared, const float* sh_gate_inp,
                               const float* x, float* y, hipStream_t stream) {
     if (top_k < 0 || top_k > 8) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((rows + 255) / 256), (unsigned)n), dim3(256), 0, stream, part,
+    MQ_LAUNCH(moe_combine_kernel, dim3((unsigned)((rows + 255) / 256), (unsigned)n), dim3(256), 0, stream, part,
                        top_k, slots, rows, weights, ids, (int)n_experts, has_shared, sh_gate_inp, x, y);
     return hipGetLastError();
 }
@@ -542,7 +557,7 @@ hipError_t launch_moe_combine(const float* part, int64_t n, int top_k, int slots
 hipError_t launch_flatten_groups(const int32_t* group_expert, const int32_t* group_begin, const int32_t* n_groups,
                                  const int32_t* entry_token, const int32_t* entry_k, int max_entries, int32_t* triples,
                                  int32_t* count, hipStream_t stream) {
-    hipLaunchKernelGGL(flatten_groups_kernel, dim3(1), dim3(256), 0, stream, group_expert, group_begin, n_groups, entry_token,
+    MQ_LAUNCH(flatten_groups_kernel, dim3(1), dim3(256), 0, stream, group_expert, group_begin, n_groups, entry_token,
                        entry_k, max_entries, triples, count);
     return hipGetLastError();
 }
@@ -551,7 +566,7 @@ hipError_t launch_fill_zero(float* p, size_t count, hipStream_t stream) {
     if (count == 0) return hipSuccess;
     size_t blocks = (count + 255) / 256;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, count);
+    MQ_LAUNCH(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, count);
     return hipGetLastError();
 }
 

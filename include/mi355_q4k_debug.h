@@ -63,6 +63,13 @@ int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int
  * previous setting of bit 0.  No counterpart in the reference. */
 int mq_debug_set_dense_lds(int on);
 
+/* Measurement instrument: while on != 0 every compute and routing launch of the library is replaced by a kernel with
+ * an empty body and the same grid, block and LDS size (weight set-up and launches that carry timing events are
+ * not).  A graph captured in this state has the launches of the real one and none of their work: its replay time
+ * is what the launches alone cost.  Outputs are not written while it is on.  Returns the previous setting.  No
+ * counterpart in the reference. */
+int mq_debug_set_skeleton(int on);
+
 #ifdef __cplusplus
 }
 #endif
