@@ -412,6 +412,17 @@ def side_measurements(ops, synth, torch, np, dev):
     # the same launch on ONE matrix over and over (9.4 MB: it stays in the last-level cache) -- not the roofline claim
     dt = time_graph(lambda: [ops.mul_mat(ring[0], x1) for _ in range(64)], 20) / 64
     res["gemv_4096x4096_n1"]["cache_hot_single_matrix_us"] = round(dt * 1e6, 2)
+    res["gemv_4096x4096_n1"]["note"] = ("one launch per 9.4 MB: an empty launch in a graph costs 1.6 us and the first bytes of cold weights "
+                                        "arrive 2 us after the workgroups start, so the single-matrix call is bound by its launch, not "
+                                        "by the memory pipes; gemv_4096x4096_n1_four_per_launch is the same work with four matrices "
+                                        "handed over together (mq_mul_mat_q4k_multi)")
+    # four matrices of the ring per launch on the same activation row (a layer's projections handed over together)
+    outs = [torch.empty((4096,), dtype=torch.float32, device=dev) for _ in range(4)]
+    dt = time_graph(lambda: [ops.mul_mat_multi(ring[i:i + 4], x1, outs) for i in range(0, len(ring), 4)], 20) / (len(ring) // 4)
+    b4 = 4 * 4096 * 16 * 144 + (1 + 4) * 4096 * 4
+    res["gemv_4096x4096_n1_four_per_launch"] = {"us": round(dt * 1e6, 2), "us_per_matrix": round(dt * 1e6 / 4, 2),
+                                                "GBps": round(b4 / dt / 1e9, 1),
+                                                "pct_hbm_peak": round(b4 / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
     for w in ring:
         w.free()
 

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libmi355q4k.so")
 EXPORTS = [
     "mq_init", "mq_shutdown", "mq_last_error", "mq_device_info",
     "mq_weight_upload", "mq_weight_upload_typed", "mq_weight_synthetic", "mq_weight_synthetic_typed", "mq_weight_type", "mq_weight_download", "mq_weight_shape", "mq_weight_free",
-    "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_mul_mat_q4k_noalloc", "mq_gemm_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
+    "mq_quantize_q8k", "mq_mul_mat_q4k", "mq_mul_mat_q4k_multi", "mq_mul_mat_q4k_noalloc", "mq_gemm_q4k", "mq_mul_mat_q4k_q8k", "mq_mul_mat_q4k_host", "mq_swiglu_mul_mat_q4k",
     "mq_ffn_swiglu_q4k", "mq_moe_gateup_swiglu_q4k", "mq_moe_down_weighted_q4k",
     "mq_moe_route_topk", "mq_moe_weights_from_logits", "mq_mul_mat_id_q4k", "mq_moe_layer_q4k",
     "mq_acts_create", "mq_acts_free", "mq_acts_quantize", "mq_mul_mat_q4k_acts", "mq_swiglu_mul_mat_q4k_acts",
@@ -76,6 +76,7 @@ def load() -> C.CDLL:
     L.mq_weight_free.argtypes = [vp]
     L.mq_quantize_q8k.argtypes = [vp, i64, i64, i64, vp, vp]
     L.mq_mul_mat_q4k.argtypes = [vp, vp, i64, i64, vp, i64, vp]
+    L.mq_mul_mat_q4k_multi.argtypes = [C.POINTER(vp), ci, vp, C.POINTER(vp), vp]
     L.mq_mul_mat_q4k_noalloc.argtypes = [vp, vp, i64, i64, vp, i64, vp]
     L.mq_gemm_q4k.argtypes = [vp, vp, i64, i64, vp, i64, vp]
     L.mq_mul_mat_q4k_q8k.argtypes = [vp, vp, i64, sz, vp, i64, vp]

@@ -672,6 +672,48 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }
 
+int mq_mul_mat_q4k_multi(const mq_weight* const* w, int count, const float* x_dev, float* const* y_dev, void* stream) {
+    if (int rc = check_ready()) return rc;
+    if (count < 0 || count > kGemvMultiMax) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_multi: count %d is outside [0, %d]", count, kGemvMultiMax);
+    if (count == 0) return MQ_OK;
+    if (!w || !y_dev) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_multi: null weight or output list");
+    for (int i = 0; i < count; ++i) {
+        if (int rc = check_weight(w[i], "mq_mul_mat_q4k_multi", true)) return rc;
+        if (w[i]->n_experts != 1) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_multi: weight %d is an expert stack", i);
+        if (w[i]->cols != w[0]->cols) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_multi: weight %d has %lld columns, weight 0 has %lld", i, (long long)w[i]->cols, (long long)w[0]->cols);
+        if (!y_dev[i]) return fail(MQ_ERR_INVALID, "mq_mul_mat_q4k_multi: output %d is null", i);
+    }
+    if (int rc = check_x(x_dev, 1, w[0]->cols, w[0]->cols, "mq_mul_mat_q4k_multi")) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    // Matrices that take the single-row kernel with the quantizer inside share launches, one per wave split (a launch
+    // has one workgroup shape, and every matrix keeps the split -- so the bits -- of a launch of its own); the others
+    // (another type, long rows, a misaligned x) go through mq_mul_mat_q4k one by one.
+    bool taken[kGemvMultiMax] = {};
+    for (int i = 0; i < count; ++i) {
+        if (taken[i]) continue;
+        const int waves = pick_waves(w[i]->nb, w[i]->rowtiles);
+        const bool fused = w[i]->type == kTypeQ4K && gemv1_fused_applies(w[i]->nb, waves);
+        if (!fused) {
+            taken[i] = true;
+            if (int rc = mq_mul_mat_q4k(w[i], x_dev, 1, w[i]->cols, y_dev[i], w[i]->rows, stream)) return rc;
+            continue;
+        }
+        Gemv1MultiArgs a;
+        a.nb = w[i]->nb;
+        a.x = x_dev;
+        for (int j = i; j < count; ++j) {
+            if (taken[j] || w[j]->type != kTypeQ4K || pick_waves(w[j]->nb, w[j]->rowtiles) != waves) continue;
+            taken[j] = true;
+            a.w[a.count] = w[j]->data, a.y[a.count] = y_dev[j], a.rows[a.count] = w[j]->rows;
+            ++a.count;
+        }
+        Entry entry(s);
+        if (entry.rc) return entry.rc;
+        MQ_HIP(launch_gemv1_multi(a, waves, s));
+    }
+    return MQ_OK;
+}
+
 int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                            void* stream) {
     if (int rc = check_ready()) return rc;

@@ -19,14 +19,12 @@ namespace {
 
 constexpr int kMaxStages = 2;
 
-__global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restrict__ w, int64_t rows, int64_t nb,
-                                                          const float* __restrict__ x, float* __restrict__ y) {
-    extern __shared__ float red[];  // [W-1][64]
+__device__ __forceinline__ void gemv1_fused_body(const uint8_t* __restrict__ w, int64_t rows, int64_t nb, const float* __restrict__ x,
+                                                 float* __restrict__ y, int64_t rt, float* red) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
     const int slot = lane & 15, kq = lane >> 4;
-    const int64_t rt = blockIdx.x;
     const uint8_t* tiles = w + tile_offset(rt, 0, nb);
     const int cnt = (wave < nb ? 1 : 0) + (wave + n_waves < nb ? 1 : 0);  // super-blocks wave, wave + W (at most kMaxStages, host-checked; no division)
 
@@ -66,6 +64,85 @@ __global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restr
         if (n_waves > 1) v = add_wave_partials(v, n_waves, [&](int wv) { return red[(wv - 1) * 64 + lane]; });
         const int64_t row = rt * 16 + slot;
         if (kq == 0 && row < rows) y[row] = v;
+    }
+}
+
+__global__ void __launch_bounds__(512) gemv1_fused_kernel(const uint8_t* __restrict__ w, int64_t rows, int64_t nb,
+                                                          const float* __restrict__ x, float* __restrict__ y) {
+    extern __shared__ float red[];  // [W-1][64]
+    gemv1_fused_body(w, rows, nb, x, y, blockIdx.x, red);
+}
+
+// Several matrices against ONE activation row in one launch (the q, k and v projections of a layer, the gate and up
+// projections of an FFN: core/src/llm/graph/decoder.cpp:1092-1099, :2662-2663 emit them as separate nodes on the same
+// input).  The grid is the matrices' row tiles one after the other, RT consecutive row tiles of one matrix to a
+// workgroup; per row tile the arithmetic, the wave split and the reduction order are the single-matrix kernel's, so the
+// bits are those of one launch per matrix -- whose dispatch and first trip to memory are paid once here, and whose
+// quantization of x (every workgroup repeats it) once per RT row tiles: with a thousand workgroups that repetition,
+// not memory, is what a launch costs.
+template <int RT>
+__global__ void __launch_bounds__(512) gemv1_multi_kernel(const Gemv1MultiArgs p) {
+    extern __shared__ float red[];  // [RT][W-1][64]
+    const int g = blockIdx.x;
+    int m = 0;
+#pragma unroll
+    for (int i = 1; i < kGemvMultiMax; ++i) m += (i < p.count && g >= p.rt_begin[i]) ? 1 : 0;  // begins ascend: a count, no search
+    const uint8_t* w = p.w[m];
+    const int64_t rows = p.rows[m], nb = p.nb;
+    const int64_t rowtiles = (rows + 15) >> 4;
+    const int64_t rt0 = (int64_t)(g - p.rt_begin[m]) * RT;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;
+    const int slot = lane & 15, kq = lane >> 4;
+    const int cnt = (wave < nb ? 1 : 0) + (wave + n_waves < nb ? 1 : 0);
+    TileRegs t[RT][kMaxStages];
+    float4 xv[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) xv[i] = *reinterpret_cast<const float4*>(p.x + (size_t)(i < cnt ? wave + i * n_waves : 0) * kQK + lane * 4);
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        // a row tile past the matrix's last streams the last one again and stores nothing
+        const uint8_t* tiles = w + tile_offset(rt0 + r < rowtiles ? rt0 + r : rowtiles - 1, 0, nb);
+#pragma unroll
+        for (int i = 0; i < kMaxStages; ++i) load_tile(t[r][i], tiles + (size_t)(i < cnt ? wave + i * n_waves : 0) * kTileBytes, lane);
+    }
+    ACodes codes[kMaxStages];
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        const float e[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+        a_codes_from_lane_codes(codes[i], quantize_block_q8k(e, lane), lane);
+    }
+    float acc[RT][1][2];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[r][0][0] = acc[r][0][1] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kMaxStages; ++i) {
+        if (i < cnt) {
+            ARegs<1> a;
+            a_from_codes(a, codes[i], lane);
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+                int32_t dsum[1][2], msum[1][2];
+                compute_tile<1, false, 1>(t[r][i], a, acc[r], dsum, msum);
+            }
+        }
+    }
+    if (n_waves > 1) {
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r) red[(r * (n_waves - 1) + wave - 1) * 64 + lane] = acc[r][0][0];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            float v = acc[r][0][0];
+            if (n_waves > 1) v = add_wave_partials(v, n_waves, [&](int wv) { return red[(r * (n_waves - 1) + wv - 1) * 64 + lane]; });
+            const int64_t row = (rt0 + r) * 16 + slot;
+            if (kq == 0 && rt0 + r < rowtiles && row < rows) p.y[m][row] = v;
+        }
     }
 }
 
@@ -393,6 +470,30 @@ hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
     const int64_t rowtiles = (rows + 15) / 16;
     MQ_LAUNCH(gemv1_fused_kernel, dim3((unsigned)rowtiles), dim3(64 * waves),
                        waves > 1 ? (size_t)(waves - 1) * 64 * sizeof(float) : 0, stream, w, rows, nb, x, y);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv1_multi(const Gemv1MultiArgs& a, int waves, hipStream_t stream) {
+    if (a.count < 1 || a.count > kGemvMultiMax || !gemv1_fused_applies(a.nb, waves) || !a.x) return hipErrorInvalidValue;
+    int64_t all_tiles = 0;
+    for (int i = 0; i < a.count; ++i) {
+        if (!a.w[i] || !a.y[i] || a.rows[i] <= 0) return hipErrorInvalidValue;
+        all_tiles += (a.rows[i] + 15) / 16;
+    }
+    // row tiles per workgroup: as many as leave every compute unit a workgroup (at most four)
+    const int64_t per_cu = all_tiles / compute_units();
+    const int rt = per_cu >= 4 ? 4 : per_cu >= 2 ? 2 : 1;
+    Gemv1MultiArgs b = a;
+    int total = 0;
+    for (int i = 0; i < a.count; ++i) {
+        b.rt_begin[i] = total;
+        total += (int)(((a.rows[i] + 15) / 16 + rt - 1) / rt);
+    }
+    for (int i = a.count; i <= kGemvMultiMax; ++i) b.rt_begin[i] = total;
+    const size_t lds = waves > 1 ? (size_t)rt * (waves - 1) * 64 * sizeof(float) : 0;
+    if (rt == 4) MQ_LAUNCH(gemv1_multi_kernel<4>, dim3((unsigned)total), dim3(64 * waves), lds, stream, b);
+    else if (rt == 2) MQ_LAUNCH(gemv1_multi_kernel<2>, dim3((unsigned)total), dim3(64 * waves), lds, stream, b);
+    else MQ_LAUNCH(gemv1_multi_kernel<1>, dim3((unsigned)total), dim3(64 * waves), lds, stream, b);
     return hipGetLastError();
 }
 

@@ -165,6 +165,19 @@ hipError_t launch_gemvn_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
 // The same with the residual add and the RMSNorm of the row inside (sum_out apart from x and delta).
 hipError_t launch_gemv1_norm_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, const float* delta,
                                    const float* weight, float eps, float* sum_out, float* y, int waves, hipStream_t stream);
+// Several single-row GEMVs of one activation row in one launch (gemv1.hip): matrices of one column count, each
+// with the wave split a launch of its own would take.
+constexpr int kGemvMultiMax = 8;
+struct Gemv1MultiArgs {
+    const uint8_t* w[kGemvMultiMax] = {};
+    float* y[kGemvMultiMax] = {};
+    int64_t rows[kGemvMultiMax] = {};
+    int rt_begin[kGemvMultiMax + 1] = {};  // filled by the launcher: first workgroup of matrix i
+    int count = 0;
+    int64_t nb = 0;
+    const float* x = nullptr;
+};
+hipError_t launch_gemv1_multi(const Gemv1MultiArgs& a, int waves, hipStream_t stream);
 hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const float* x, float* y, int waves,
                               hipStream_t stream);
 

@@ -112,6 +112,17 @@ def mul_mat(w: Q4KWeight, x: torch.Tensor, out: torch.Tensor = None) -> torch.Te
     return y
 
 
+def mul_mat_multi(ws, x: torch.Tensor, outs=None):
+    """Several products of one activation row in one launch (mq_mul_mat_q4k_multi): the q, k and v projections of a
+    layer as the graph emits them on one input (core/src/llm/graph/decoder.cpp:1092-1099).  Returns the list of y."""
+    x = _f32(x).reshape(-1)
+    ys = outs if outs is not None else [torch.empty((w.rows,), dtype=torch.float32, device=x.device) for w in ws]
+    wl = (C.c_void_p * len(ws))(*[w._h for w in ws])
+    yl = (C.c_void_p * len(ws))(*[y.data_ptr() for y in ys])
+    _lib.check(_lib.lib().mq_mul_mat_q4k_multi(wl, len(ws), _ptr(x), yl, _stream()), "mq_mul_mat_q4k_multi")
+    return ys
+
+
 def gemm(w: Q4KWeight, x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     """The same product through the int8 matrix-core GEMM kernel at any n (RunQ4KRawBatchedDenseGemm,
     core/src/backend/cpu_backend_q4k_dense.cpp:57-101)."""

@@ -116,6 +116,15 @@ int mq_quantize_q8k(const float* x_dev, int64_t n, int64_t ldx, int64_t k, void*
  * (core/include/densecore/backend/cpu_backend.h:293-300, any n). */
 int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                    void* stream);
+/* Several products of ONE activation row in one launch: y_dev[i][r] = w[i][r] . q8k(x), i < count <= 8, all
+ * weights dense with the same number of columns (x_dev fp32 [cols]; y_dev[i] fp32 [rows of w[i]]).  The graph
+ * emits the q, k and v projections of a layer, and the gate and up projections of an FFN, as separate nodes on the
+ * same input (core/src/llm/graph/decoder.cpp:1092-1099, :2662-2663; one fused tensor at :630); a caller that holds
+ * them together hands them over together.  Q4_K matrices whose rows are short enough for the single-row kernel
+ * with the quantizer inside share a launch -- the same bits as mq_mul_mat_q4k on each -- and pay the dispatch and
+ * the first trip to memory once; any other weight in the list goes through mq_mul_mat_q4k.  An error leaves the
+ * outputs of the list undefined. */
+int mq_mul_mat_q4k_multi(const mq_weight* const* w, int count, const float* x_dev, float* const* y_dev, void* stream);
 /* mq_mul_mat_q4k for callers that cannot allocate (code under HIP-graph capture, serving loops and harnesses that
  * forbid hipMalloc): the same product, bit for bit, for n <= 16 rows of cols <= 16384 (MQ_ERR_UNSUPPORTED beyond
  * that), Q4_K / Q5_K / Q6_K weights.  It calls no allocating routine: the quantized activations go to a fixed
