@@ -500,6 +500,23 @@ def side_measurements(ops, synth, torch, np, dev):
                           "tokens_per_s": round(n / dt, 1)}
     moe_pf["note"] = "useful ops 2 * tokens * (top_k + shared) * 3 matrices * 2048 * 512 over the whole block (routing, gather, combine included)"
     res["moe_layer_prefill"] = moe_pf
+    # the layer a Q4_K_M file holds: Q4_K gate/up stacks with Q6_K down experts (the shared expert's down Q6_K too)
+    down6 = [(ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "down6"), H, I, E, synth.GGML_TYPE_Q6_K),
+              ops.Q4KWeight.synthetic(synth.tensor_seed("cfg3", r, "sd6"), H, I, 1, synth.GGML_TYPE_Q6_K)) for r in range(len(layers))]
+    moe_pf6 = {}
+    for n in (512, 2048):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-x", n), (n, H))).to(dev)
+        lg = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg3-l", n), (n, E))).to(dev)
+        dt = time_graph(lambda: [ops.moe_layer(ge, ue, d6, x, lg, K, shared=(sh[0], sh[1], sd6, sh[3]), silu=ops.SILU_FAST)
+                                 for (ge, ue, de, sh), (d6, sd6) in zip(layers, down6)], 5) / len(layers)
+        tops = 2.0 * n * (K + 1) * 3 * H * I / dt / 1e12
+        moe_pf6[str(n)] = {"us": round(dt * 1e6, 1), "TOPs": round(tops, 1), "pct_int8_mfma_peak": round(tops / INT8_PEAK_TOPS * 100, 2),
+                           "tokens_per_s": round(n / dt, 1)}
+    moe_pf6["note"] = "the same block with Q6_K down experts (gate/up Q4_K): all three expert products on the matrix-core GEMM"
+    res["moe_layer_prefill_q6k_down"] = moe_pf6
+    for d6, sd6 in down6:
+        d6.free()
+        sd6.free()
     for ge, ue, de, sh in layers:
         for w in (ge, ue, de) + sh[:3]:
             w.free()

@@ -471,7 +471,7 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
         if (T == 1 && a.n == 1) return launch_one<NM, 1, false, false, W, 1>(b, waves, grid, stream, start, stop); \
         return launch_one<NM, T, false, false, W>(b, waves, grid, stream, start, stop);                   \
     } while (0)
-#define MQ_LAUNCH(NM, T)                                 \
+#define MQ_LAUNCH_NT(NM, T)                               \
     do {                                                 \
         if (a.wtype == kTypeQ6K) MQ_LAUNCH_WT(NM, T, kWtQ6); \
         if (a.wtype == kTypeQ5K) MQ_LAUNCH_WT(NM, T, kWtQ5); \
@@ -479,13 +479,13 @@ hipError_t launch_matmul(const MatmulArgs& a, hipStream_t stream, hipEvent_t sta
     } while (0)
 
     if (nmat == 1) {
-        if (tt == 1) MQ_LAUNCH(1, 1);
-        MQ_LAUNCH(1, 2);
+        if (tt == 1) MQ_LAUNCH_NT(1, 1);
+        MQ_LAUNCH_NT(1, 2);
     } else {
-        if (tt == 1) MQ_LAUNCH(2, 1);
-        MQ_LAUNCH(2, 2);
+        if (tt == 1) MQ_LAUNCH_NT(2, 1);
+        MQ_LAUNCH_NT(2, 2);
     }
-#undef MQ_LAUNCH
+#undef MQ_LAUNCH_NT
 #undef MQ_LAUNCH_WT
     return hipSuccess;
 }

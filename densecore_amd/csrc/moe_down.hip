@@ -262,6 +262,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_rows_kernel(const MoeDow
 #pragma unroll
     for (int st = 0; st < kItems - 1; ++st) issue(st, st);
     const int src = 8 * (slot & 1) + 2 * kq;  // this lane's words of a block's operand (a_codes_from_lane_codes)
+    const uint32_t even_slot = (slot & 1) ? 0u : 0xffffffffu, odd_slot = ~even_slot;
     for (int q0 = 0; q0 < cnt; q0 += kItems) {
 #pragma unroll
         for (int st = 0; st < kItems; ++st) {
@@ -276,7 +277,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_rows_kernel(const MoeDow
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         const v2u v = *reinterpret_cast<const v2u*>(codes + i * 64 + 16 * c + src);
-                        a.q[0][c] = slot == 0 ? v4u{v.x, v.y, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, v.x, v.y} : v4u{0u, 0u, 0u, 0u});
+                        a.q[0][c] = v4u{v.x & even_slot, v.y & even_slot, v.x & odd_slot, v.y & odd_slot};  // as a_from_codes (q8k_block.h)
                     }
                     a.yd[0][0] = scales[i];
                     a.yd[0][1] = 0.0f;

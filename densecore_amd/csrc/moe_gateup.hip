@@ -217,6 +217,7 @@ __global__ void __launch_bounds__(WT == kWtQ4 ? 1024 : 512) moe_gateup_slots_ker
         for (int st = 0; st < kStages - 1; ++st) issue_t(st, st);
         // this lane's words of a block's operand (a_codes_from_lane_codes): codes 64c + 32(slot & 1) + 8kq .. +7 of chunk c
         const int src = 8 * (slot & 1) + 2 * kq;
+        const uint32_t even_slot = (slot & 1) ? 0u : 0xffffffffu, odd_slot = ~even_slot;
         for (int base = 0; base < cnt; base += kStages) {
 #pragma unroll
             for (int st = 0; st < kStages; ++st) {
@@ -228,7 +229,7 @@ __global__ void __launch_bounds__(WT == kWtQ4 ? 1024 : 512) moe_gateup_slots_ker
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         const v2u v = *reinterpret_cast<const v2u*>(codes + b * 64 + 16 * c + src);
-                        a.q[0][c] = slot == 0 ? v4u{v.x, v.y, 0u, 0u} : (slot == 1 ? v4u{0u, 0u, v.x, v.y} : v4u{0u, 0u, 0u, 0u});
+                        a.q[0][c] = v4u{v.x & even_slot, v.y & even_slot, v.x & odd_slot, v.y & odd_slot};  // as a_from_codes (q8k_block.h)
                     }
                     a.yd[0][0] = scales[b];
                     a.yd[0][1] = 0.0f;
