@@ -101,7 +101,9 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_token_kernel(const MoeDo
             const int e = __builtin_amdgcn_readlane(id_lane, sl & 7);
             live[j] = i < n_items && (shared || (e >= 0 && e < p.n_experts));
             const uint8_t* m = shared ? p.sh_w : p.w + (size_t)(live[j] ? e : 0) * p.expert_bytes;
-            tile_ptr[j] = m + (live[j] ? tile_offset(rt, b, nb, kTileStride) : 0);
+            // (a harmless tile of this workgroup's own row tile: were it one fixed place for the whole launch, every
+            // wavefront's spare requests would queue at the one memory channel that holds it)
+            tile_ptr[j] = m + tile_offset(rt, live[j] ? b : 0, nb, kTileStride);
         }
 #pragma unroll
         for (int j = 0; j < kItems; ++j) load_tile_wt<WT>(tiles[j], tile_ptr[j], lane);
@@ -257,7 +259,7 @@ __global__ void __launch_bounds__(kWaves * 64) moe_down_rows_kernel(const MoeDow
         const int e = __builtin_amdgcn_readlane(id_lane, sl & 7);
         live[st] = q < cnt && (shared || (e >= 0 && e < p.n_experts));
         const uint8_t* m = shared ? p.sh_w : p.w + (size_t)(live[st] ? e : 0) * p.expert_bytes;
-        load_tile_wt<WT>(ring[st], m + (live[st] ? tile_offset(rt0 + r, b, nb, kTileStride) : 0), lane);
+        load_tile_wt<WT>(ring[st], m + tile_offset(rt0 + r, live[st] ? b : 0, nb, kTileStride), lane);  // dead: a tile of this workgroup's own rows, not one place for all
     };
 #pragma unroll
     for (int st = 0; st < kItems - 1; ++st) issue(st, st);
