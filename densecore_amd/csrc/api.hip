@@ -135,6 +135,7 @@ struct State {
     std::recursive_mutex mu;  // recursive: the host-pointer entry points call the device-pointer ones while holding it
     Buffer aq, ad;        // A-major activations of the op input
     Buffer ap, ap2;       // P-major activations of the prefill GEMM (input; FFN intermediate)
+    Buffer ap_rows;       // the distinct rows of an expert-grouped GEMM's input, quantized once, before they are copied to their groups
     Buffer mid2;          // gate and up products of a wide FFN, fp32
     Buffer kpart;         // planes of partial sums of a prefill GEMM whose K is split
     Buffer plan;          // tile plan of the expert-grouped GEMM
@@ -374,7 +375,7 @@ int mq_shutdown(void) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     if (!g.ready) return MQ_OK;
     (void)hipDeviceSynchronize();
-    for (Buffer* b : {&g.aq, &g.ad, &g.ap, &g.ap2, &g.mid, &g.mid2, &g.kpart, &g.plan, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
+    for (Buffer* b : {&g.aq, &g.ad, &g.ap, &g.ap2, &g.ap_rows, &g.mid, &g.mid2, &g.kpart, &g.plan, &g.aq2, &g.ad2, &g.part, &g.counters, &g.route, &g.stage_in, &g.stage_out}) b->release();
     g.pin_in.release();
     g.pin_out.release();
     if (g.order_event) (void)hipEventDestroy(g.order_event);
@@ -1093,8 +1094,11 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, x_slots != 1, entries, E,
                                     0, 0, (int32_t*)g.plan.ptr, s));
         MQ_HIP(g.ap.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, w->nb)));
+        // one row per token (b broadcast over the slots): the rows repeat top_k times -- quantize each once
+        if (x_slots == 1) MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, w->nb)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, w->cols, w->cols, entries, E, (const int32_t*)g.plan.ptr,
-                                                  (uint8_t*)g.ap.ptr, nullptr, 0, s));
+                                                  (uint8_t*)g.ap.ptr, nullptr, 0, s, x_slots == 1 ? n : 0,
+                                                  x_slots == 1 ? (uint8_t*)g.ap_rows.ptr : nullptr));
         MQ_HIP(launch_prefill_gemm_grouped(w->data, w->type, w->expert_bytes, nullptr, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
                                            (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s));
         return MQ_OK;
@@ -1490,7 +1494,9 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
                                     0, 0, (int32_t*)g.plan.ptr, s));
         const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
+        MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, hidden / kQK)));  // every token is a row of top_k experts: quantized once
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s,
+                                                  n, (uint8_t*)g.ap_rows.ptr));
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
@@ -1656,7 +1662,9 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
                                     sh.gate ? n : 0, MQ_SILU_FAST_FMA, (int32_t*)g.plan.ptr, s));
         const int64_t rows_max = moe_gemm_tiles_max(entries, G) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
-        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, G, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s));
+        MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, hidden / kQK)));  // every token is a row of top_k (+ the shared) experts: quantized once
+        MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, G, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s,
+                                                  n, (uint8_t*)g.ap_rows.ptr));
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;

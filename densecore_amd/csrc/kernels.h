@@ -210,7 +210,8 @@ hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_ex
                                 int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream);
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
                                               int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
-                                              int64_t ldh, hipStream_t stream);
+                                              int64_t ldh, hipStream_t stream, int64_t distinct_rows = 0,
+                                              uint8_t* ap_rows = nullptr);
 hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows,
                                        int64_t nb, const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan,
                                        bool scatter, float* y, int64_t ldy, hipStream_t stream);

@@ -518,6 +518,42 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     for (int i = tid; i < kPTileWords; i += 256) dst[i] = reinterpret_cast<const v4u*>(img)[i];
 }
 
+// The expert-grouped tiles of rows that repeat (a token is a row of top_k experts, and of the shared one): the distinct
+// rows are quantized ONCE into tiles in their own order (quantize_q8k_pmajor_kernel on x as it is), and this kernel
+// copies row row_src[m] of those tiles to row m of the plan's tiles -- sixteen 16-byte pieces of codes, two of digits
+// and a scale per row and super-block, the same bytes the gathering quantizer writes (at top-8 it ran the block
+// quantizer eight or nine times per token: 35 of the block's 406 us at 2048 tokens).  A workgroup per (tile,
+// super-block); -1 in row_src: padding, zeros.
+__global__ void __launch_bounds__(256) gather_pmajor_tiles_kernel(const uint8_t* __restrict__ ap_src, int64_t src_tiles,
+                                                                  int64_t m_tiles, uint8_t* __restrict__ ap,
+                                                                  const int32_t* __restrict__ plan,
+                                                                  const int32_t* __restrict__ row_src) {
+    const int tid = threadIdx.x;
+    const int64_t tile = blockIdx.x, b = blockIdx.y;
+    if (tile >= (int64_t)plan[1]) return;
+    const uint8_t* from = ap_src + (size_t)b * (size_t)src_tiles * kPTileBytes;
+    uint8_t* dst = ap + ((size_t)b * (size_t)m_tiles + (size_t)tile) * kPTileBytes;
+    const int r = tid & 15, piece = tid >> 4;  // piece j * 4 + kq of row r: bytes j * 1024 + (kq * 16 + r) * 16
+    const int t = row_src[tile * 16 + r];
+    const uint8_t* st = from + (size_t)(t >= 0 ? t >> 4 : 0) * kPTileBytes;
+    const int tr = t >= 0 ? (t & 15) : 0;
+    const int j = piece >> 2, kq = piece & 3;
+    v4u codes = *reinterpret_cast<const v4u*>(st + j * 1024 + (kq * 16 + tr) * 16);
+    if (t < 0) codes = v4u{0u, 0u, 0u, 0u};
+    *reinterpret_cast<v4u*>(dst + j * 1024 + (kq * 16 + r) * 16) = codes;
+    if (tid < 32) {  // the row's sixteen fp16 digits: two pieces
+        v4u d = *reinterpret_cast<const v4u*>(st + kPDigitOff + tr * 32 + piece * 16);
+        if (t < 0) d = v4u{0u, 0u, 0u, 0u};
+        *reinterpret_cast<v4u*>(dst + kPDigitOff + r * 32 + piece * 16) = d;
+    } else if (tid < 48) {
+        float sc = *reinterpret_cast<const float*>(st + kPScaleOff + tr * 4);
+        if (t < 0) sc = 0.0f;
+        *reinterpret_cast<float*>(dst + kPScaleOff + r * 4) = sc;
+    } else if (tid < 52) {
+        *reinterpret_cast<uint32_t*>(dst + kPZeroOff + (tid - 48) * 4) = 0u;
+    }
+}
+
 // y[tok][row] = plane 0 + plane 1 + ... in that order; four rows per thread (rows % 4 == 0)
 __global__ void __launch_bounds__(256) prefill_sum_planes_kernel(const float* __restrict__ part, int splits, int64_t n, int64_t rows,
                                                                  float* __restrict__ y, int64_t ldy) {
@@ -688,11 +724,19 @@ hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_ex
 // those rows as fp32 at their per-(token, slot) places).
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
                                               int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
-                                              int64_t ldh, hipStream_t stream) {
+                                              int64_t ldh, hipStream_t stream, int64_t distinct_rows, uint8_t* ap_rows) {
     const int64_t nb = k / kQK, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     if (m_tiles == 0 || nb == 0) return hipSuccess;
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
     const int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
+    if (!swiglu && ap_rows && distinct_rows > 0) {
+        // the plan's rows repeat the distinct_rows rows of x: quantize those once, then copy them to their places
+        hipError_t e = launch_quantize_q8k_pmajor(x, distinct_rows, ldx, k, ap_rows, stream);
+        if (e != hipSuccess) return e;
+        MQ_LAUNCH(gather_pmajor_tiles_kernel, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, (const uint8_t*)ap_rows,
+                  (distinct_rows + 15) / 16, m_tiles, ap, plan, row_src);
+        return hipGetLastError();
+    }
     if (swiglu) {
         MQ_LAUNCH(quantize_q8k_pmajor_kernel<true>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x, x2, silu_mode,
                            h_out, ldh, m_tiles * 16, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr,
