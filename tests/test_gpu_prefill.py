@@ -209,3 +209,33 @@ def test_gemm_full_size_sampled_rows_against_the_oracle(ops, m):
     assert_fp32_parity(y[pick], ref, mag, "sampled rows (AVX2 order)")
     assert_fp32_parity(y[pick[:2]], orc.mul_mat_q4k_q8k(w, cols, q8[:2], orc.ORDER_HWY), mag[:2], "Highway order")
     W.free()
+
+
+@pytest.mark.parametrize("n,E,K", [(400, 16, 4), (300, 10, 8), (1030, 24, 3)])
+def test_rows_quantized_once_and_copied_to_their_groups_give_the_bits_of_rows_quantized_per_slot(ops, n, E, K):
+    """mul_mat_id at a width that takes the expert-grouped GEMM.  With one activation row per token the row is
+    quantized once and its codes are copied to every group it is routed to; with the same rows replicated per slot by
+    the caller every (token, slot) row is quantized by itself.  Same quantizer, same codes: the outputs must agree bit
+    for bit (ragged token counts, a last tile of padding rows, ids outside the expert range)."""
+    import torch
+    rows, cols = 64, 1024
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("once-w", n, E), rows, cols, E)
+    x = synth.normal_f32(synth.tensor_seed("once-x", n, cols), (n, cols))
+    rng = np.random.default_rng(synth.tensor_seed("once-ids", n, E, K) & 0xffffffff)
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(n)]).astype(np.int32)
+    ids[3, 0] = -1
+    ids[n - 1, K - 1] = E + 5
+    xd, idd = cu(x), cu(ids)
+    once = ops.mul_mat_id(W, xd, idd).cpu().numpy()
+    per_slot = ops.mul_mat_id(W, xd[:, None, :].expand(n, K, cols).contiguous(), idd).cpu().numpy()
+    assert np.array_equal(once.view(np.uint32), per_slot.view(np.uint32))
+    assert not np.any(once[3, 0]) and not np.any(once[n - 1, K - 1])
+    # and against the oracle on a sample of pairs
+    w_np = W.to_ggml()
+    q8 = orc.quantize_rows_q8k(x)
+    for t, k in ((0, 0), (7, K - 1), (n - 2, 1), (n // 2, 0)):
+        e = int(ids[t, k])
+        ref = orc.mul_mat_q4k_q8k(w_np[e], cols, q8[t:t + 1], orc.ORDERS["avx2"])
+        mag = orc.dot_magnitude_f64(w_np[e], cols, q8[t:t + 1])
+        assert_fp32_parity(once[t, k][None], ref, mag, f"pair ({t}, {k})")
+    W.free()
