@@ -172,6 +172,7 @@ struct Census {
 // Dense products of up to 16 rows go to the kernel that stages the activations in LDS where the shape fits it (the
 // same bits as matmul_kernel on the same operands); mq_debug_set_dense_lds(0) keeps them on matmul_kernel.
 int g_dense_lds = 1;
+int g_gemm_pair = 1;  // prefill widths: Q4_K gate and up in ONE GEMM launch that stores silu(gate) * up (mq_debug_set_dense_lds bit 3 turns it off)
 // Widest product whose fp32 rows the LDS-staged kernel quantizes itself (no quantizer launch).
 int64_t g_dense_xf_rows = 2;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
 
@@ -565,11 +566,23 @@ static int gemm_locked(const mq_weight* w, const float* x_dev, int64_t n, int64_
 static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_weight* down, const float* x_dev, int64_t n,
                            int64_t ldx, int silu_mode, float* h_dev, int64_t ldh, float* y_dev, int64_t ldy, hipStream_t s) {
     const int64_t inter = gate->rows;
+    MQ_HIP(g.ap.reserve(pmajor_bytes(n, gate->nb)));
+    MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, gate->cols, (uint8_t*)g.ap.ptr, s));
+    if (g_gemm_pair && gate->type == kTypeQ4K && up->type == kTypeQ4K && prefill_pair_applies(gate->type, inter, gate->nb, n)) {
+        // gate and up in one launch that stores silu(gate) * up: no fp32 planes, no pass that reads them back
+        MQ_HIP(launch_prefill_gemm_pair(gate->data, up->data, gate->type, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, silu_mode, h_dev, ldh, s));
+        if (!down) return MQ_OK;
+        MQ_HIP(g.ap2.reserve(pmajor_bytes(n, down->nb)));
+        MQ_HIP(launch_quantize_q8k_pmajor(h_dev, n, ldh, inter, (uint8_t*)g.ap2.ptr, s));
+        const size_t part2 = prefill_part_bytes(down->rows, down->nb, n, down->type);
+        if (part2) MQ_HIP(g.kpart.reserve(part2));
+        MQ_HIP(launch_prefill_gemm(down->data, down->type, down->rows, down->nb, (const uint8_t*)g.ap2.ptr, n, y_dev, ldy,
+                                   part2 ? (float*)g.kpart.ptr : nullptr, s));
+        return MQ_OK;
+    }
     MQ_HIP(g.mid2.reserve(2 * (size_t)n * (size_t)inter * sizeof(float)));
     float* gbuf = (float*)g.mid2.ptr;
     float* ubuf = gbuf + (size_t)n * (size_t)inter;
-    MQ_HIP(g.ap.reserve(pmajor_bytes(n, gate->nb)));
-    MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, gate->cols, (uint8_t*)g.ap.ptr, s));
     const size_t part_bytes = prefill_part_bytes(inter, gate->nb, n, gate->type);
     if (part_bytes) MQ_HIP(g.kpart.reserve(part_bytes));
     float* part = part_bytes ? (float*)g.kpart.ptr : nullptr;
@@ -1497,6 +1510,13 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
         MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, hidden / kQK)));  // every token is a row of top_k experts: quantized once
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(x_dev, nullptr, false, 0, hidden, hidden, entries, E, plan, (uint8_t*)g.ap.ptr, nullptr, 0, s,
                                                   n, (uint8_t*)g.ap_rows.ptr));
+        if (g_gemm_pair && gate_exps->type == kTypeQ4K && up_exps->type == kTypeQ4K) {
+            // one launch for gate and up, silu(gate) * up scattered to its (token, slot) place by the epilogue
+            MQ_HIP(launch_prefill_gemm_grouped_pair(gate_exps->data, up_exps->data, gate_exps->type, gate_exps->expert_bytes, nullptr, nullptr,
+                                                    inter, gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, E, plan, true, silu_mode, hidden_dev,
+                                                    inter, s));
+            return MQ_OK;
+        }
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
@@ -1671,6 +1691,24 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         const uint8_t* shg = sh.gate ? sh.gate->data : nullptr;
         const uint8_t* shu = sh.gate ? sh.up->data : nullptr;
         const uint8_t* shd = sh.gate ? sh.down->data : nullptr;
+        if (g_gemm_pair && L->gate_exps->type == kTypeQ4K && L->up_exps->type == kTypeQ4K) {
+            // gate and up in ONE launch whose epilogue stores silu(gate) * up (the shared expert's rows with its own SiLU form)
+            if (!moe_gemm_takes(L->down_exps)) {  // fp32 rows at their (token, slot) places for the down stack's own kernel
+                MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
+                MQ_HIP(launch_prefill_gemm_grouped_pair(L->gate_exps->data, L->up_exps->data, kTypeQ4K, L->gate_exps->expert_bytes, shg, shu, inter,
+                                                        L->gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, G, plan, true, L->silu_mode,
+                                                        (float*)g.mid.ptr, inter, s));
+                return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, false, n, K, slots, r, ids, wts, L->sh_gate_inp_dev, x_dev, y_dev, s);
+            }
+            MQ_HIP(launch_prefill_gemm_grouped_pair(L->gate_exps->data, L->up_exps->data, kTypeQ4K, L->gate_exps->expert_bytes, shg, shu, inter,
+                                                    L->gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, G, plan, false, L->silu_mode, gbuf, inter, s));
+            MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
+            MQ_HIP(launch_quantize_q8k_pmajor(gbuf, rows_max, inter, inter, (uint8_t*)g.ap2.ptr, s, plan));  // rows in the plan's order already
+            MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->type, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
+                                               (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
+            MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
+            return MQ_OK;
+        }
         MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->type, L->gate_exps->expert_bytes, shg, inter, L->gate_exps->nb,
                                            (const uint8_t*)g.ap.ptr, entries, G, plan, false, gbuf, inter, s));
         MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->type, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
@@ -1918,6 +1956,7 @@ int mq_debug_set_dense_lds(int on) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     const int before = g_dense_lds;
     g_dense_lds = on & 1;
+    g_gemm_pair = (on & 8) ? 0 : 1;  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;

@@ -184,8 +184,9 @@ hipError_t launch_gemv1_fused(const uint8_t* w, int64_t rows, int64_t nb, const 
 // ---- prefill.hip -----------------------------------------------------------------------------
 // fp32 rows -> Q8_K in the P-major layout of the prefill GEMM (pmajor_bytes(n, nb) bytes).
 size_t pmajor_bytes(int64_t n, int64_t nb);
+// plan (optional): the rows are an expert-grouped GEMM's tiles in the plan's order; tiles past the plan's count are skipped
 hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
-                                      hipStream_t stream);
+                                      hipStream_t stream, const int32_t* plan = nullptr);
 // The same for the rows silu(gate) * up (both [n][ldx]); h_out (may be null) receives them as fp32 [n][ldh] as well.
 hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up, int64_t n, int64_t ldx, int64_t k,
                                              int silu_mode, float* h_out, int64_t ldh, uint8_t* ap, hipStream_t stream);
@@ -194,6 +195,14 @@ hipError_t launch_swiglu_quantize_q8k_pmajor(const float* gate, const float* up,
 // nothing is split) and are added in order by a second launch.
 // wtype: kTypeQ4K, or kTypeQ5K (a third MFMA chain for the fifth code bits; 64-row workgroups).
 size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype);
+// silu(gate . x) * (up . x) from ONE launch (prefill.hip: the pair form of the GEMM kernel), dense and expert-grouped
+bool prefill_pair_applies(int wtype, int64_t rows, int64_t nb, int64_t n);
+hipError_t launch_prefill_gemm_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t rows, int64_t nb, const uint8_t* ap,
+                                    int64_t n, int silu_mode, float* h, int64_t ldh, hipStream_t stream);
+hipError_t launch_prefill_gemm_grouped_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t expert_bytes,
+                                            const uint8_t* gate_shared, const uint8_t* up_shared, int64_t rows, int64_t nb,
+                                            const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
+                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream);
 hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
                                int64_t ldy, float* part, hipStream_t stream);
 

@@ -244,13 +244,20 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
 
 // kWTilesPerWave = 2: the 128 x 128 workgroup tile above.  1: 64 weight rows per workgroup, for launches whose
 // 128-row workgroups would leave compute units without their two workgroups (M up to a few hundred).
-template <int kWTilesPerWave, int WT = kWtQ4>
+// PAIR (two weight tiles per wavefront, Q4_K): the wavefront's two tiles are the SAME row tile of two matrices, gate
+// (w) and up (w2), and what is stored is silu(gate) * up -- the two fp32 planes a gate launch and an up launch would
+// write, and the pass that reads them back to form the product, never exist (for 2048 rows of a 4096 -> 14336 FFN that
+// is 235 MB written and read).  The same accumulators, the same SiLU function on the same values: the same bits.
+template <int kWTilesPerWave, int WT = kWtQ4, bool PAIR = false>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
                                                            int64_t split_stride, const int32_t* __restrict__ plan,
                                                            int64_t expert_bytes, const int32_t* __restrict__ out_rows,
-                                                           const uint8_t* __restrict__ w_shared) {
+                                                           const uint8_t* __restrict__ w_shared,
+                                                           const uint8_t* __restrict__ w2 = nullptr,
+                                                           const uint8_t* __restrict__ w2_shared = nullptr, int silu_mode = 0) {
+    static_assert(!PAIR || (kWTilesPerWave == 2 && WT == kWtQ4), "the pair form is the two-tile Q4_K kernel");
     extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
     constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
     constexpr bool Q5 = WT == kWtQ5, Q6 = WT == kWtQ6;
@@ -267,14 +274,18 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         if (item >= plan[0]) return;  // the whole workgroup, before any barrier
         const int expert = plan[4 + 3 * item];  // -1: the shared expert's rows
         w = expert < 0 ? w_shared : w + (size_t)expert * (size_t)expert_bytes;
+        if constexpr (PAIR) {
+            w2 = expert < 0 ? w2_shared : w2 + (size_t)expert * (size_t)expert_bytes;
+            if (expert < 0) silu_mode = plan[3];  // the shared expert's rows: its own SiLU form
+        }
         mt0 = plan[5 + 3 * item];
         mt_count = plan[6 + 3 * item];
     }
-    const int64_t rt0 = ((int64_t)blockIdx.x * 4 + wave) * kWTilesPerWave;
+    const int64_t rt0 = ((int64_t)blockIdx.x * 4 + wave) * (PAIR ? 1 : kWTilesPerWave);
     // weight tiles past the end are replaced by the last valid one and simply not stored
     int64_t rt[kWTilesPerWave];
 #pragma unroll
-    for (int t = 0; t < kWTilesPerWave; ++t) rt[t] = rt0 + t < rowtiles ? rt0 + t : rowtiles - 1;
+    for (int t = 0; t < kWTilesPerWave; ++t) rt[t] = rt0 + (PAIR ? 0 : t) < rowtiles ? rt0 + (PAIR ? 0 : t) : rowtiles - 1;
 
     float acc[kWTilesPerWave][kMTilesPerGroup][4];
 #pragma unroll
@@ -300,7 +311,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     auto request_w = [&](int64_t b) {
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
-            const uint8_t* tile = w + tile_offset(rt[t], b, nb, tile_stride<WT>());
+            const uint8_t* tile = (PAIR && t == 1 ? w2 : w) + tile_offset(rt[t], b, nb, tile_stride<WT>());
             seg0[t] = load16(tile + lane * 16);
             seg1[t] = load16(tile + 1024 + lane * 16);
             if constexpr (Q6) {
@@ -414,9 +425,16 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         }
     }
 
+    if constexpr (PAIR) {  // one output per (token, row): silu(gate) * up
+#pragma unroll
+        for (int m = 0; m < kMTilesPerGroup; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[0][m][i] = silu_mul(acc[0][m][i], acc[1][m][i], silu_mode);
+    }
+    constexpr int kStoredTiles = PAIR ? 1 : kWTilesPerWave;
     if (out_rows) {  // grouped down product: row 16 (mt0 + m) + 4 kq + i of the plan goes to row out_rows[..] of y (-1: padding)
 #pragma unroll
-        for (int t = 0; t < kWTilesPerWave; ++t) {
+        for (int t = 0; t < kStoredTiles; ++t) {
             const int64_t row = (rt0 + t) * kTileRows + r;
             if (rt0 + t >= rowtiles || row >= rows) continue;
 #pragma unroll
@@ -435,7 +453,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     // down the token rows (an addition per store, no product).
     const int tok_left = (int)(n_tokens - mt0 * 16) - kq * 4;  // tokens from this lane's first one to the end
 #pragma unroll
-    for (int t = 0; t < kWTilesPerWave; ++t) {
+    for (int t = 0; t < kStoredTiles; ++t) {
         const int64_t row = (rt0 + t) * kTileRows + r;
         if (rt0 + t >= rowtiles || row >= rows) continue;
         float* yp = y + (mt0 * 16 + kq * 4) * ldy + row;
@@ -785,6 +803,58 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expe
     return hipGetLastError();
 }
 
+// The pair form: h[tok][row] = silu(gate[row] . x[tok]) * (up[row] . x[tok]).  It has no K split (SiLU is not linear), so it
+// applies where the two single launches would not split K either; Q4_K only (the other types' operand sets fill the
+// registers with one tile per wavefront).
+bool prefill_pair_applies(int wtype, int64_t rows, int64_t nb, int64_t n) {
+    if (wtype != kTypeQ4K) return false;
+    return prefill_shape(rows, nb, n, true).splits == 1;
+}
+
+hipError_t launch_prefill_gemm_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t rows, int64_t nb, const uint8_t* ap,
+                                    int64_t n, int silu_mode, float* h, int64_t ldh, hipStream_t stream) {
+    const int64_t rowtiles = (rows + 15) / 16, m_tiles = (n + 15) / 16;
+    if (rowtiles == 0 || m_tiles == 0) return hipSuccess;
+    if (!prefill_pair_applies(wtype, rows, nb, n)) return hipErrorInvalidValue;
+    const PrefillShape ps = prefill_shape(rows, nb, n, true);
+    if (ps.groups > 65535u) return hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<2, kWtQ4, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true>), dim3(ps.row_wgs, ps.groups, 1u), dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream,
+              gate, rowtiles, rows, nb, ap, m_tiles, n, h, ldh, (int)nb, (int64_t)0, (const int32_t*)nullptr, (int64_t)0,
+              (const int32_t*)nullptr, (const uint8_t*)nullptr, up, (const uint8_t*)nullptr, silu_mode);
+    return hipGetLastError();
+}
+
+// The expert-grouped pair form: scatter == false: h [tiles * 16][ldh] in the plan's row order; true: row out_row[r] of h.
+hipError_t launch_prefill_gemm_grouped_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t expert_bytes,
+                                            const uint8_t* gate_shared, const uint8_t* up_shared, int64_t rows, int64_t nb,
+                                            const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
+                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream) {
+    if (wtype != kTypeQ4K) return hipErrorInvalidValue;
+    const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
+    const int64_t items = moe_gemm_items_max(entries, groups_max);
+    if (rowtiles == 0 || items == 0) return hipSuccess;
+    if (items > 65535) return hipErrorInvalidValue;
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<2, kWtQ4, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kMTilesPerGroup * kPTileBytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
+    MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
+              2 * kMTilesPerGroup * kPTileBytes, stream, gate, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, h, ldh, (int)nb, (int64_t)0, plan,
+              expert_bytes, out_row, gate_shared, up, up_shared, silu_mode);
+    return hipGetLastError();
+}
+
 size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype) {
     const PrefillShape ps = prefill_shape(rows, nb, n, wtype != kTypeQ4K);
     return ps.splits > 1 ? (size_t)ps.splits * (size_t)n * (size_t)rows * sizeof(float) : 0;
@@ -793,12 +863,12 @@ size_t prefill_part_bytes(int64_t rows, int64_t nb, int64_t n, int wtype) {
 size_t pmajor_bytes(int64_t n, int64_t nb) { return (size_t)((n + 15) / 16) * (size_t)nb * kPTileBytes; }
 
 hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, int64_t k, uint8_t* ap,
-                                      hipStream_t stream) {
+                                      hipStream_t stream, const int32_t* plan) {
     const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
     if (m_tiles == 0 || nb == 0) return hipSuccess;
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
     MQ_LAUNCH(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
-                       (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, (const int32_t*)nullptr,
+                       (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, plan,
                        (const int32_t*)nullptr, (const int32_t*)nullptr);
     return hipGetLastError();
 }

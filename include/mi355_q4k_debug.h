@@ -59,7 +59,8 @@ int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int
  * in LDS once per workgroup (and, for up to four fp32 rows, quantizes them itself), and expert-grouped launches
  * with many groups on the kernel that gathers a group's rows into LDS once per eight wavefronts; on = 0 keeps
  * both on the kernel that reads its operand from global memory at every stage, on = 5 only the expert-grouped
- * ones.  All return the same bits (tests/test_gpu_dense_lds.py, tests/test_gpu_grouped_lds.py); returns the
+ * ones; bit 3 (on = 9) makes Q4_K gate and up at prefill widths two GEMM launches and a SwiGLU pass instead of the
+ * one launch that stores silu(gate) * up.  All return the same bits (tests/test_gpu_dense_lds.py, tests/test_gpu_grouped_lds.py); returns the
  * previous setting of bit 0.  No counterpart in the reference. */
 int mq_debug_set_dense_lds(int on);
 

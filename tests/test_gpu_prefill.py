@@ -239,3 +239,64 @@ def test_rows_quantized_once_and_copied_to_their_groups_give_the_bits_of_rows_qu
         mag = orc.dot_magnitude_f64(w_np[e], cols, q8[t:t + 1])
         assert_fp32_parity(once[t, k][None], ref, mag, f"pair ({t}, {k})")
     W.free()
+
+
+def _with_pair(on):
+    from densecore_amd import _lib
+    _lib.lib().mq_debug_set_dense_lds(1 if on else 9)  # bit 3: gate and up as two GEMM launches and a SwiGLU pass
+
+
+@pytest.mark.parametrize("n", [48, 130, 512, 1000])
+@pytest.mark.parametrize("silu", [0, 1, 2])
+def test_pair_gemm_of_gate_and_up_gives_the_bits_of_two_launches_and_a_swiglu_pass(ops, n, silu):
+    """Dense FFN and SwiGLU product at prefill widths: one GEMM launch whose epilogue stores silu(gate) * up against the
+    two launches + SwiGLU pass it replaces (the same accumulators, the same SiLU function on the same values)."""
+    import torch
+    hidden, inter = 1024, 2560
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("pair-g"), inter, hidden)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("pair-u"), inter, hidden)
+    D = ops.Q4KWeight.synthetic(synth.tensor_seed("pair-d"), hidden, inter)
+    x = cu(synth.normal_f32(synth.tensor_seed("pair-x", n), (n, hidden)))
+    try:
+        _with_pair(True)
+        h1 = ops.swiglu_mul_mat(G, U, x, silu).cpu().numpy()
+        y1 = ops.ffn_swiglu(G, U, D, x, silu).cpu().numpy()
+        _with_pair(False)
+        h0 = ops.swiglu_mul_mat(G, U, x, silu).cpu().numpy()
+        y0 = ops.ffn_swiglu(G, U, D, x, silu).cpu().numpy()
+    finally:
+        _with_pair(True)
+    assert np.array_equal(h1.view(np.uint32), h0.view(np.uint32))
+    assert np.array_equal(y1.view(np.uint32), y0.view(np.uint32))
+    for w in (G, U, D):
+        w.free()
+
+
+@pytest.mark.parametrize("n,down_type", [(300, synth.GGML_TYPE_Q4_K), (520, synth.GGML_TYPE_Q6_K), (300, synth.GGML_TYPE_Q8_0)])
+def test_pair_gemm_in_the_moe_block_gives_the_bits_of_two_launches(ops, n, down_type):
+    """The expert-grouped form, in the MoE layer (rows in the plan's order for a GEMM down product, scattered to their
+    (token, slot) places for a down stack with a kernel of its own) and in the gate/up entry point, shared expert included."""
+    import torch
+    E, H, I, K = 12, 1024, 512, 4
+    ge = ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-g"), I, H, E)
+    ue = ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-u"), I, H, E)
+    de = ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-d", down_type), H, I, E, down_type)
+    sh = (ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-sg"), I, H), ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-su"), I, H),
+          ops.Q4KWeight.synthetic(synth.tensor_seed("pairm-sd", down_type), H, I, 1, down_type),
+          cu(synth.normal_f32(synth.tensor_seed("pairm-gi"), (H,)) * np.float32(0.02)))
+    x = cu(synth.normal_f32(synth.tensor_seed("pairm-x", n), (n, H)))
+    lg = cu(synth.normal_f32(synth.tensor_seed("pairm-l", n), (n, E)))
+    out = {}
+    try:
+        for on in (True, False):
+            _with_pair(on)
+            y, ids, wts = ops.moe_layer(ge, ue, de, x, lg, K, shared=sh, silu=ops.SILU_FAST)
+            h = ops.moe_gateup_swiglu(ge, ue, x, ids, ops.SILU_FAST)
+            out[on] = (y.cpu().numpy(), h.cpu().numpy(), ids.cpu().numpy())
+    finally:
+        _with_pair(True)
+    assert np.array_equal(out[True][2], out[False][2])
+    assert np.array_equal(out[True][1].view(np.uint32), out[False][1].view(np.uint32))
+    assert np.array_equal(out[True][0].view(np.uint32), out[False][0].view(np.uint32))
+    for w in (ge, ue, de) + sh[:3]:
+        w.free()
