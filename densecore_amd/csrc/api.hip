@@ -172,6 +172,7 @@ struct Census {
 // Dense products of up to 16 rows go to the kernel that stages the activations in LDS where the shape fits it (the
 // same bits as matmul_kernel on the same operands); mq_debug_set_dense_lds(0) keeps them on matmul_kernel.
 int g_dense_lds = 1;
+int g_moe_item_tiles = 0;  // 0: chosen per launch (moe_gemm_item_tiles); 2, 4 or 8: forced (mq_debug_set_dense_lds bits 8..11)
 int g_gemm_pair = 1;  // prefill widths: Q4_K gate and up in ONE GEMM launch that stores silu(gate) * up (mq_debug_set_dense_lds bit 3 turns it off)
 // Widest product whose fp32 rows the LDS-staged kernel quantizes itself (no quantizer launch).
 int64_t g_dense_xf_rows = 2;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
@@ -1104,8 +1105,9 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
     if (use_gemm) {
         const int64_t entries = n * top_k, E = w->n_experts;
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int mt = g_moe_item_tiles ? g_moe_item_tiles : moe_gemm_item_tiles(entries, E);  // tiles per item: the plan and every launch reading it
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, x_slots != 1, entries, E,
-                                    0, 0, (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s, mt));
         MQ_HIP(g.ap.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, w->nb)));
         // one row per token (b broadcast over the slots): the rows repeat top_k times -- quantize each once
         if (x_slots == 1) MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, w->nb)));
@@ -1113,7 +1115,7 @@ int mq_mul_mat_id_q4k(const mq_weight* w, const float* x_dev, int64_t n, int x_s
                                                   (uint8_t*)g.ap.ptr, nullptr, 0, s, x_slots == 1 ? n : 0,
                                                   x_slots == 1 ? (uint8_t*)g.ap_rows.ptr : nullptr));
         MQ_HIP(launch_prefill_gemm_grouped(w->data, w->type, w->expert_bytes, nullptr, w->rows, w->nb, (const uint8_t*)g.ap.ptr, entries, E,
-                                           (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s));
+                                           (const int32_t*)g.plan.ptr, true, y_dev, w->rows, s, mt));
         return MQ_OK;
     }
     MatmulArgs a;
@@ -1502,9 +1504,10 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
         // prefill widths: both products on the expert-grouped GEMM, SwiGLU rows scattered to their (token, slot) places
         const int64_t entries = n * top_k, E = gate_exps->n_experts, inter = gate_exps->rows, hidden = gate_exps->cols;
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int mt = g_moe_item_tiles ? g_moe_item_tiles : moe_gemm_item_tiles(entries, E);  // tiles per item: the plan and every launch reading it
         const int32_t* plan = (const int32_t*)g.plan.ptr;
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, false, entries, E,
-                                    0, 0, (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s, mt));
         const int64_t rows_max = moe_gemm_tiles_max(entries, E) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
         MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, hidden / kQK)));  // every token is a row of top_k experts: quantized once
@@ -1514,16 +1517,16 @@ int mq_moe_gateup_swiglu_q4k(const mq_weight* gate_exps, const mq_weight* up_exp
             // one launch for gate and up, silu(gate) * up scattered to its (token, slot) place by the epilogue
             MQ_HIP(launch_prefill_gemm_grouped_pair(gate_exps->data, up_exps->data, gate_exps->type, gate_exps->expert_bytes, nullptr, nullptr,
                                                     inter, gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, E, plan, true, silu_mode, hidden_dev,
-                                                    inter, s));
+                                                    inter, s, mt));
             return MQ_OK;
         }
         MQ_HIP(g.mid2.reserve(2 * (size_t)rows_max * (size_t)inter * sizeof(float)));
         float* gbuf = (float*)g.mid2.ptr;
         float* ubuf = gbuf + (size_t)rows_max * (size_t)inter;
         MQ_HIP(launch_prefill_gemm_grouped(gate_exps->data, gate_exps->type, gate_exps->expert_bytes, nullptr, inter, gate_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s));
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, gbuf, inter, s, mt));
         MQ_HIP(launch_prefill_gemm_grouped(up_exps->data, up_exps->type, up_exps->expert_bytes, nullptr, inter, up_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s));
+                                           (const uint8_t*)g.ap.ptr, entries, E, plan, false, ubuf, inter, s, mt));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, silu_mode, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
                                                   hidden_dev, inter, s));
@@ -1553,15 +1556,16 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
         // prefill widths: the product on the expert-grouped GEMM into the per-(token, slot) rows, then the combine
         const int64_t entries = n * top_k, E = down_exps->n_experts, hidden = down_exps->rows, inter = down_exps->cols;
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, E) * sizeof(int32_t)));
+        const int mt = g_moe_item_tiles ? g_moe_item_tiles : moe_gemm_item_tiles(entries, E);  // tiles per item: the plan and every launch reading it
         const int32_t* plan = (const int32_t*)g.plan.ptr;
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, top_k, true, entries, E,
-                                    0, 0, (int32_t*)g.plan.ptr, s));
+                                    0, 0, (int32_t*)g.plan.ptr, s, mt));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(moe_gemm_tiles_max(entries, E) * 16, inter / kQK)));
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(hidden_dev, nullptr, false, 0, inter, inter, entries, E, plan, (uint8_t*)g.ap2.ptr,
                                                   nullptr, 0, s));
         MQ_HIP(g.part.reserve((size_t)n * top_k * (size_t)hidden * sizeof(float)));
         MQ_HIP(launch_prefill_gemm_grouped(down_exps->data, down_exps->type, down_exps->expert_bytes, nullptr, hidden, down_exps->nb,
-                                           (const uint8_t*)g.ap2.ptr, entries, E, plan, true, (float*)g.part.ptr, hidden, s));
+                                           (const uint8_t*)g.ap2.ptr, entries, E, plan, true, (float*)g.part.ptr, hidden, s, mt));
         MQ_HIP(launch_moe_combine((const float*)g.part.ptr, n, top_k, top_k, hidden, weights_dev, ids_dev, E, 0, nullptr, nullptr, y_dev, s));
         return MQ_OK;
     }
@@ -1677,9 +1681,10 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
                                       r.group_expert, r.group_begin, r.n_groups, r.entry_token, r.entry_k, true, nullptr, 0, 0,
                                       nullptr, nullptr, s));
         MQ_HIP(g.plan.reserve(moe_gemm_plan_ints(entries, G) * sizeof(int32_t)));
+        const int mt = g_moe_item_tiles ? g_moe_item_tiles : moe_gemm_item_tiles(entries, G);  // tiles per item: the plan and every launch reading it
         const int32_t* plan = (const int32_t*)g.plan.ptr;
         MQ_HIP(launch_moe_gemm_plan(r.n_groups, r.group_expert, r.group_begin, r.entry_token, r.entry_k, slots, false, entries, G,
-                                    sh.gate ? n : 0, MQ_SILU_FAST_FMA, (int32_t*)g.plan.ptr, s));
+                                    sh.gate ? n : 0, MQ_SILU_FAST_FMA, (int32_t*)g.plan.ptr, s, mt));
         const int64_t rows_max = moe_gemm_tiles_max(entries, G) * 16;
         MQ_HIP(g.ap.reserve(pmajor_bytes(rows_max, hidden / kQK)));
         MQ_HIP(g.ap_rows.reserve(pmajor_bytes(n, hidden / kQK)));  // every token is a row of top_k (+ the shared) experts: quantized once
@@ -1697,22 +1702,22 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
                 MQ_HIP(g.mid.reserve((size_t)n * slots * (size_t)inter * sizeof(float)));
                 MQ_HIP(launch_prefill_gemm_grouped_pair(L->gate_exps->data, L->up_exps->data, kTypeQ4K, L->gate_exps->expert_bytes, shg, shu, inter,
                                                         L->gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, G, plan, true, L->silu_mode,
-                                                        (float*)g.mid.ptr, inter, s));
+                                                        (float*)g.mid.ptr, inter, s, mt));
                 return run_moe_down(L->down_exps, sh, (const float*)g.mid.ptr, false, n, K, slots, r, ids, wts, L->sh_gate_inp_dev, x_dev, y_dev, s);
             }
             MQ_HIP(launch_prefill_gemm_grouped_pair(L->gate_exps->data, L->up_exps->data, kTypeQ4K, L->gate_exps->expert_bytes, shg, shu, inter,
-                                                    L->gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, G, plan, false, L->silu_mode, gbuf, inter, s));
+                                                    L->gate_exps->nb, (const uint8_t*)g.ap.ptr, entries, G, plan, false, L->silu_mode, gbuf, inter, s, mt));
             MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
             MQ_HIP(launch_quantize_q8k_pmajor(gbuf, rows_max, inter, inter, (uint8_t*)g.ap2.ptr, s, plan));  // rows in the plan's order already
             MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->type, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
-                                               (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
+                                               (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s, mt));
             MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
             return MQ_OK;
         }
         MQ_HIP(launch_prefill_gemm_grouped(L->gate_exps->data, L->gate_exps->type, L->gate_exps->expert_bytes, shg, inter, L->gate_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, gbuf, inter, s));
+                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, gbuf, inter, s, mt));
         MQ_HIP(launch_prefill_gemm_grouped(L->up_exps->data, L->up_exps->type, L->up_exps->expert_bytes, shu, inter, L->up_exps->nb,
-                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, ubuf, inter, s));
+                                           (const uint8_t*)g.ap.ptr, entries, G, plan, false, ubuf, inter, s, mt));
         MQ_HIP(g.ap2.reserve(pmajor_bytes(rows_max, inter / kQK)));
         if (!moe_gemm_takes(L->down_exps)) {
             // a down stack of a type the GEMM does not take: the SwiGLU rows leave the quantizer as fp32 at their
@@ -1725,7 +1730,7 @@ int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float
         }
         MQ_HIP(launch_quantize_q8k_pmajor_grouped(gbuf, ubuf, true, L->silu_mode, inter, inter, entries, G, plan, (uint8_t*)g.ap2.ptr, nullptr, 0, s));
         MQ_HIP(launch_prefill_gemm_grouped(L->down_exps->data, L->down_exps->type, L->down_exps->expert_bytes, shd, hidden, L->down_exps->nb,
-                                           (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s));
+                                           (const uint8_t*)g.ap2.ptr, entries, G, plan, true, part, hidden, s, mt));
         MQ_HIP(launch_moe_combine(part, n, K, slots, hidden, wts, ids, E, sh.gate ? 1 : 0, L->sh_gate_inp_dev, x_dev, y_dev, s));
         return MQ_OK;
     }
@@ -1956,7 +1961,8 @@ int mq_debug_set_dense_lds(int on) {
     std::lock_guard<std::recursive_mutex> lock(g.mu);
     const int before = g_dense_lds;
     g_dense_lds = on & 1;
-    g_gemm_pair = (on & 8) ? 0 : 1;  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
+    g_gemm_pair = (on & 8) ? 0 : 1;
+    g_moe_item_tiles = (on >> 8) & 0xf;      // bits 8..11: activation tiles per item of the expert-grouped GEMM (2, 4 or 8), 0 = by the rows per expert  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;

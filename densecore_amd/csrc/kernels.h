@@ -202,7 +202,7 @@ hipError_t launch_prefill_gemm_pair(const uint8_t* gate, const uint8_t* up, int 
 hipError_t launch_prefill_gemm_grouped_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t expert_bytes,
                                             const uint8_t* gate_shared, const uint8_t* up_shared, int64_t rows, int64_t nb,
                                             const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
-                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream);
+                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream, int mt = 8);
 hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_t nb, const uint8_t* ap, int64_t n, float* y,
                                int64_t ldy, float* part, hipStream_t stream);
 
@@ -214,16 +214,19 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
 int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max);
 int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max);
 size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max);
+// activation tiles per item (2 or 8) of an expert-grouped launch over `entries` rows in `groups` groups: the plan and
+// every launch that reads it take the same value
+int moe_gemm_item_tiles(int64_t entries, int64_t groups);
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
                                 const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
-                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream);
+                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream, int mt = 8);
 hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, bool swiglu, int silu_mode, int64_t ldx, int64_t k,
                                               int64_t entries, int64_t groups_max, const int32_t* plan, uint8_t* ap, float* h_out,
                                               int64_t ldh, hipStream_t stream, int64_t distinct_rows = 0,
                                               uint8_t* ap_rows = nullptr);
 hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows,
                                        int64_t nb, const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan,
-                                       bool scatter, float* y, int64_t ldy, hipStream_t stream);
+                                       bool scatter, float* y, int64_t ldy, hipStream_t stream, int mt = 8);
 
 // ---- elementwise.hip -------------------------------------------------------------------------
 hipError_t launch_add_rmsnorm(const float* x, const float* delta, const float* weight, int64_t n, int64_t cols,

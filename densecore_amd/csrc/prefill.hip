@@ -49,6 +49,8 @@ constexpr int kPTileBytes = 4688;
 constexpr int kPTileWords = kPTileBytes / 16;  // 293
 constexpr int kPDigitOff = 4096, kPScaleOff = 4608, kPZeroOff = 4672;
 constexpr int kMTilesPerGroup = 8;             // activation tiles (of 16 rows) per workgroup
+constexpr int kMTilesSmall = 2;                // ... of an expert-grouped launch whose experts hold a dozen or two rows
+constexpr int kMTilesMid = 4;                  // ... or three or four dozen
 
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -223,6 +225,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // into LDS with global_load_lds_dwordx4: lane l of a request writes its 16 bytes at base + 16*l, so a
 // run of 64-word requests is a linear copy that never touches a register.  The instruction offset must
 // stay 0 (the hardware adds it to the global address as well).
+template <int MT>
 __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src, uint8_t* buf, int copy_words, int wave,
                                                 int lane) {
     // Written as inline assembly on purpose: the compiler then does not know that LDS is written, and so does
@@ -230,9 +233,9 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
     // for them itself, with vmcnt(0) and a barrier, before the buffer is read.  M0 (the LDS base of the request)
     // is used by nothing else in this kernel.
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)buf;
-    static_assert(10 * 4 * 64 >= kMTilesPerGroup * kPTileWords, "ten rounds of requests cover the tiles of a group");
+    constexpr int kRounds = (MT * kPTileWords + 255) / 256;  // 4 waves x 64 words a round: ten rounds for eight tiles of 293 words
 #pragma unroll
-    for (int j = 0; j < 10; ++j) {  // 4 waves x 10 requests x 64 words >= 8 tiles x 293 words
+    for (int j = 0; j < kRounds; ++j) {
         const int first = (j * 4 + wave) * 64;
         if (first + lane < copy_words) {
             const uint8_t* g = src + (size_t)(first + lane) * 16;
@@ -248,7 +251,11 @@ __device__ __forceinline__ void request_a_tiles(const uint8_t* __restrict__ src,
 // (w) and up (w2), and what is stored is silu(gate) * up -- the two fp32 planes a gate launch and an up launch would
 // write, and the pass that reads them back to form the product, never exist (for 2048 rows of a 4096 -> 14336 FFN that
 // is 235 MB written and read).  The same accumulators, the same SiLU function on the same values: the same bits.
-template <int kWTilesPerWave, int WT = kWtQ4, bool PAIR = false>
+// MT: activation tiles (of 16 rows) a workgroup multiplies.  Eight for the dense product; the expert-grouped one also
+// comes with two (items of 32 rows): with a dozen or two routed rows per expert a workgroup has one or two tiles, its
+// accumulators for eight only cost registers and LDS -- and how many workgroups a compute unit holds is what hides the
+// latency of a workgroup that walks eight super-blocks with a barrier each.
+template <int kWTilesPerWave, int WT = kWtQ4, bool PAIR = false, int MT = kMTilesPerGroup>
 __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __restrict__ w, int64_t rowtiles, int64_t rows,
                                                            int64_t nb, const uint8_t* __restrict__ ap, int64_t m_tiles,
                                                            int64_t n_tokens, float* __restrict__ y, int64_t ldy, int sb_split,
@@ -258,8 +265,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
                                                            const uint8_t* __restrict__ w2 = nullptr,
                                                            const uint8_t* __restrict__ w2_shared = nullptr, int silu_mode = 0) {
     static_assert(!PAIR || (kWTilesPerWave == 2 && WT == kWtQ4), "the pair form is the two-tile Q4_K kernel");
-    extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of kMTilesPerGroup * kPTileBytes bytes
-    constexpr int kBufBytes = kMTilesPerGroup * kPTileBytes;
+    extern __shared__ __align__(16) uint8_t a_lds[];  // two buffers of MT * kPTileBytes bytes
+    constexpr int kBufBytes = MT * kPTileBytes;
     constexpr bool Q5 = WT == kWtQ5, Q6 = WT == kWtQ6;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -267,8 +274,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     const int r = lane & 15, kq = lane >> 4;
     // Dense: workgroup column blockIdx.y takes the activation tiles 8 y .. 8 y + 7.  Expert-grouped (plan != null): it
     // takes item blockIdx.y of the plan -- an expert's weights and a run of up to eight tiles of that expert's rows.
-    int64_t mt0 = (int64_t)blockIdx.y * kMTilesPerGroup;
-    int mt_count = (int)(m_tiles - mt0 < kMTilesPerGroup ? m_tiles - mt0 : kMTilesPerGroup);
+    int64_t mt0 = (int64_t)blockIdx.y * MT;
+    int mt_count = (int)(m_tiles - mt0 < MT ? m_tiles - mt0 : MT);
     if (plan) {
         const int item = blockIdx.y;
         if (item >= plan[0]) return;  // the whole workgroup, before any barrier
@@ -287,11 +294,11 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 #pragma unroll
     for (int t = 0; t < kWTilesPerWave; ++t) rt[t] = rt0 + (PAIR ? 0 : t) < rowtiles ? rt0 + (PAIR ? 0 : t) : rowtiles - 1;
 
-    float acc[kWTilesPerWave][kMTilesPerGroup][4];
+    float acc[kWTilesPerWave][MT][4];
 #pragma unroll
     for (int t = 0; t < kWTilesPerWave; ++t)
 #pragma unroll
-        for (int m = 0; m < kMTilesPerGroup; ++m)
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[t][m][i] = 0.0f;
 
@@ -330,7 +337,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     const int64_t b_begin = (int64_t)blockIdx.z * sb_split;
     const int64_t b_end = b_begin + sb_split < nb ? b_begin + sb_split : nb;
     y += (size_t)blockIdx.z * (size_t)split_stride;
-    request_a_tiles(a_src + (size_t)b_begin * a_stride, a_lds + (b_begin & 1) * kBufBytes, copy_words, wave, lane);
+    request_a_tiles<MT>(a_src + (size_t)b_begin * a_stride, a_lds + (b_begin & 1) * kBufBytes, copy_words, wave, lane);
     request_w(b_begin);
 
     for (int64_t b = b_begin; b < b_end; ++b) {
@@ -346,13 +353,13 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
             else expand_tile<Q5>(seg0[t], seg1[t], hdr[t], qh[t], kq, wt[t]);
         }
         if (b + 1 < b_end) {
-            request_a_tiles(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
+            request_a_tiles<MT>(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
             request_w(b + 1);
         }
         const uint8_t* a_buf = a_lds + (b & 1) * kBufBytes;
 
 #pragma unroll
-        for (int m = 0; m < kMTilesPerGroup; ++m) {
+        for (int m = 0; m < MT; ++m) {
             if (m < mt_count) {  // uniform over the workgroup
                 const uint8_t* at = a_buf + m * kPTileBytes;
                 v4i a[4];
@@ -427,7 +434,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 
     if constexpr (PAIR) {  // one output per (token, row): silu(gate) * up
 #pragma unroll
-        for (int m = 0; m < kMTilesPerGroup; ++m)
+        for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[0][m][i] = silu_mul(acc[0][m][i], acc[1][m][i], silu_mode);
     }
@@ -438,7 +445,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
             const int64_t row = (rt0 + t) * kTileRows + r;
             if (rt0 + t >= rowtiles || row >= rows) continue;
 #pragma unroll
-            for (int m = 0; m < kMTilesPerGroup; ++m) {
+            for (int m = 0; m < MT; ++m) {
                 if (m >= mt_count) continue;
                 const int4 dst = *reinterpret_cast<const int4*>(out_rows + (mt0 + m) * 16 + kq * 4);
                 const int dsts[4] = {dst.x, dst.y, dst.z, dst.w};
@@ -458,7 +465,7 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         if (rt0 + t >= rowtiles || row >= rows) continue;
         float* yp = y + (mt0 * 16 + kq * 4) * ldy + row;
 #pragma unroll
-        for (int m = 0; m < kMTilesPerGroup; ++m) {
+        for (int m = 0; m < MT; ++m) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if (m < mt_count && m * 16 + i < tok_left) *yp = acc[t][m][i];
@@ -632,7 +639,7 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
                                                              const int32_t* __restrict__ entry_k, int slots, int src_per_slot,
                                                              int groups_max, int sh_tokens, int sh_slot, int sh_silu_mode,
                                                              int32_t* __restrict__ plan, int32_t* __restrict__ row_src,
-                                                             int32_t* __restrict__ out_row) {
+                                                             int32_t* __restrict__ out_row, int mt) {
     extern __shared__ int32_t plan_sh[];  // begin[g], tile0[g], item0[g]: groups_max + 2 each
     int32_t* begin = plan_sh;
     int32_t* tile0 = begin + groups_max + 2;
@@ -651,7 +658,7 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
         int tiles = 0, items = 0;
         for (int g = g0; g < g0 + per && g < ng; ++g) {
             const int t = (begin[g + 1] - begin[g] + 15) >> 4;
-            tiles += t, items += (t + kMTilesPerGroup - 1) / kMTilesPerGroup;
+            tiles += t, items += (t + mt - 1) / mt;
         }
         int ts = tiles, is = items;  // inclusive scans across the lanes
 #pragma unroll
@@ -664,7 +671,7 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
         for (int g = g0; g < g0 + per && g < ng; ++g) {
             const int t = (begin[g + 1] - begin[g] + 15) >> 4;
             tile0[g] = ts, item0[g] = is;
-            ts += t, is += (t + kMTilesPerGroup - 1) / kMTilesPerGroup;
+            ts += t, is += (t + mt - 1) / mt;
         }
         if (tid == 0) {
             tile0[ng] = all_tiles, item0[ng] = all_items;
@@ -687,10 +694,10 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
     const int first = blockIdx.x * nt + tid, step = gridDim.x * nt;
     for (int i = first; i < items; i += step) {
         const int g = group_of(item0, i);
-        const int t_g = tile0[g + 1] - tile0[g], at = (i - item0[g]) * kMTilesPerGroup;
+        const int t_g = tile0[g + 1] - tile0[g], at = (i - item0[g]) * mt;
         plan[4 + 3 * i] = g < ng_routed ? group_expert[g] : -1;
         plan[5 + 3 * i] = tile0[g] + at;
-        plan[6 + 3 * i] = t_g - at < kMTilesPerGroup ? t_g - at : kMTilesPerGroup;
+        plan[6 + 3 * i] = t_g - at < mt ? t_g - at : mt;
     }
     for (int rr = first; rr < tiles * 16; rr += step) {
         const int g = group_of(tile0, rr >> 4);
@@ -716,8 +723,10 @@ __global__ void __launch_bounds__(1024) moe_gemm_plan_kernel(const int32_t* __re
 // upper bounds: `entries` counts every row of the plan (the routed pairs and, with a shared expert, every token once
 // more), groups_max every group (the experts, + 1 with a shared expert)
 int64_t moe_gemm_tiles_max(int64_t entries, int64_t groups_max) { return (entries + 15) / 16 + groups_max; }
+// (sized for the smallest items a plan may be cut into, so that the lists behind the items lie at one place whatever
+// the item size of a launch)
 int64_t moe_gemm_items_max(int64_t entries, int64_t groups_max) {  // a multiple of four: the row arrays behind the items stay 16-byte aligned
-    return ((entries + 16 * kMTilesPerGroup - 1) / (16 * kMTilesPerGroup) + groups_max + 3) & ~(int64_t)3;
+    return ((entries + 16 * kMTilesSmall - 1) / (16 * kMTilesSmall) + groups_max + 3) & ~(int64_t)3;
 }
 size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max) {
     return 4 + 3 * (size_t)moe_gemm_items_max(entries, groups_max) + 2 * 16 * (size_t)moe_gemm_tiles_max(entries, groups_max);
@@ -725,15 +734,15 @@ size_t moe_gemm_plan_ints(int64_t entries, int64_t groups_max) {
 
 hipError_t launch_moe_gemm_plan(const int32_t* n_groups, const int32_t* group_expert, const int32_t* group_begin,
                                 const int32_t* entry_token, const int32_t* entry_k, int slots, bool src_per_slot, int64_t entries,
-                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream) {
-    if (groups_max > 4097) return hipErrorInvalidValue;
+                                int64_t groups_max, int64_t sh_tokens, int sh_silu_mode, int32_t* plan, hipStream_t stream, int mt) {
+    if (groups_max > 4097 || (mt != kMTilesSmall && mt != kMTilesMid && mt != kMTilesPerGroup)) return hipErrorInvalidValue;
     int32_t* row_src = plan + 4 + 3 * moe_gemm_items_max(entries, groups_max);
     int32_t* out_row = row_src + 16 * moe_gemm_tiles_max(entries, groups_max);
     const int64_t rows_max = 16 * moe_gemm_tiles_max(entries, groups_max);
     const unsigned wgs = (unsigned)(rows_max / 1024 < 1 ? 1 : (rows_max / 1024 > 64 ? 64 : rows_max / 1024));
     MQ_LAUNCH(moe_gemm_plan_kernel, dim3(wgs), dim3(1024), 3 * (size_t)(groups_max + 2) * sizeof(int32_t), stream, n_groups,
                        group_expert, group_begin, entry_token, entry_k, slots, src_per_slot ? 1 : 0, (int)groups_max, (int)sh_tokens,
-                       slots - 1, sh_silu_mode, plan, row_src, out_row);
+                       slots - 1, sh_silu_mode, plan, row_src, out_row, mt);
     return hipGetLastError();
 }
 
@@ -769,10 +778,21 @@ hipError_t launch_quantize_q8k_pmajor_grouped(const float* x, const float* x2, b
 
 // y = the plan's tiles . W_expert^T per item.  scatter == false: y [tiles * 16][ldy] in the plan's row order;
 // true: row out_row[r] of y (the per-(token, slot) rows of the down product).
+int moe_gemm_item_tiles(int64_t entries, int64_t groups) {
+    // An expert with more rows than an item takes several items, each of which expands the expert's weights again; an
+    // item larger than its expert's rows holds accumulators and LDS for tiles that do not exist, and a compute unit
+    // then holds fewer workgroups.  MoE block of 256 + 1 experts, top-8, 2048 x 512, items of 2 / 4 / 8 tiles: 162 / 172 /
+    // 209 us at 384 tokens (13 rows per expert), 173 / 181 / 219 at 512, 195 / 203 / 239 at 768, 236 / 224 / 260 at 1024
+    // (36 rows), 315 / 276 / 311 at 1536, 385 / 356 / 364 at 2048 (72 rows), 686 / 612 / 615 at 4096.
+    if (groups <= 0) return kMTilesPerGroup;
+    return entries <= 30 * groups ? kMTilesSmall : entries <= 160 * groups ? kMTilesMid : kMTilesPerGroup;
+}
+
 hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expert_bytes, const uint8_t* w_shared, int64_t rows,
                                        int64_t nb, const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan,
-                                       bool scatter, float* y, int64_t ldy, hipStream_t stream) {
+                                       bool scatter, float* y, int64_t ldy, hipStream_t stream, int mt) {
     if (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K) return hipErrorInvalidValue;
+    if (mt != kMTilesSmall && mt != kMTilesMid && mt != kMTilesPerGroup) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t items = moe_gemm_items_max(entries, groups_max);
     if (rowtiles == 0 || items == 0) return hipSuccess;
@@ -787,19 +807,27 @@ hipError_t launch_prefill_gemm_grouped(const uint8_t* w, int wtype, int64_t expe
         raised = true;
     }
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
-    if (wtype == kTypeQ6K) {
-        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ6>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
-                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
-                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+    const dim3 narrow((unsigned)((rowtiles + 3) / 4), (unsigned)items), wide((unsigned)((rowtiles + 7) / 8), (unsigned)items);
+#define MQ_GROUPED(KW, WT_, MT_, GRID)                                                                                             \
+    MQ_LAUNCH((prefill_gemm_kernel<KW, WT_, false, MT_>), GRID, dim3(256), 2 * MT_ * kPTileBytes, stream, w, rowtiles, rows, nb, ap, \
+              m_tiles, m_tiles * 16, y, ldy, (int)nb, (int64_t)0, plan, expert_bytes, out_row, w_shared, (const uint8_t*)nullptr,  \
+              (const uint8_t*)nullptr, 0)
+    if (mt == kMTilesSmall) {  // one weight tile per wavefront: few registers, several workgroups to a compute unit
+        if (wtype == kTypeQ6K) MQ_GROUPED(1, kWtQ6, kMTilesSmall, narrow);
+        else if (wtype == kTypeQ5K) MQ_GROUPED(1, kWtQ5, kMTilesSmall, narrow);
+        else MQ_GROUPED(1, kWtQ4, kMTilesSmall, narrow);
+    } else if (mt == kMTilesMid) {
+        if (wtype == kTypeQ6K) MQ_GROUPED(1, kWtQ6, kMTilesMid, narrow);
+        else if (wtype == kTypeQ5K) MQ_GROUPED(1, kWtQ5, kMTilesMid, narrow);
+        else MQ_GROUPED(1, kWtQ4, kMTilesMid, narrow);
+    } else if (wtype == kTypeQ6K) {
+        MQ_GROUPED(1, kWtQ6, kMTilesPerGroup, narrow);
     } else if (wtype == kTypeQ5K) {
-        MQ_LAUNCH((prefill_gemm_kernel<1, kWtQ5>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
-                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
-                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+        MQ_GROUPED(1, kWtQ5, kMTilesPerGroup, narrow);
     } else {
-        MQ_LAUNCH(prefill_gemm_kernel<2>, dim3((unsigned)((rowtiles + 7) / 8), (unsigned)items), dim3(256),
-                           2 * kMTilesPerGroup * kPTileBytes, stream, w, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, y, ldy, (int)nb,
-                           (int64_t)0, plan, expert_bytes, out_row, w_shared);
+        MQ_GROUPED(2, kWtQ4, kMTilesPerGroup, wide);
     }
+#undef MQ_GROUPED
     return hipGetLastError();
 }
 
@@ -835,8 +863,8 @@ hipError_t launch_prefill_gemm_pair(const uint8_t* gate, const uint8_t* up, int 
 hipError_t launch_prefill_gemm_grouped_pair(const uint8_t* gate, const uint8_t* up, int wtype, int64_t expert_bytes,
                                             const uint8_t* gate_shared, const uint8_t* up_shared, int64_t rows, int64_t nb,
                                             const uint8_t* ap, int64_t entries, int64_t groups_max, const int32_t* plan, bool scatter,
-                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream) {
-    if (wtype != kTypeQ4K) return hipErrorInvalidValue;
+                                            int silu_mode, float* h, int64_t ldh, hipStream_t stream, int mt) {
+    if (wtype != kTypeQ4K || (mt != kMTilesSmall && mt != kMTilesMid && mt != kMTilesPerGroup)) return hipErrorInvalidValue;
     const int64_t rowtiles = (rows + 15) / 16, m_tiles = moe_gemm_tiles_max(entries, groups_max);
     const int64_t items = moe_gemm_items_max(entries, groups_max);
     if (rowtiles == 0 || items == 0) return hipSuccess;
@@ -849,9 +877,18 @@ hipError_t launch_prefill_gemm_grouped_pair(const uint8_t* gate, const uint8_t* 
         raised = true;
     }
     const int32_t* out_row = scatter ? plan + 4 + 3 * items + 16 * m_tiles : nullptr;
-    MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true>), dim3((unsigned)((rowtiles + 3) / 4), (unsigned)items), dim3(256),
-              2 * kMTilesPerGroup * kPTileBytes, stream, gate, rowtiles, rows, nb, ap, m_tiles, m_tiles * 16, h, ldh, (int)nb, (int64_t)0, plan,
-              expert_bytes, out_row, gate_shared, up, up_shared, silu_mode);
+    const dim3 grid((unsigned)((rowtiles + 3) / 4), (unsigned)items);
+    if (mt == kMTilesSmall)
+        MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true, kMTilesSmall>), grid, dim3(256), 2 * kMTilesSmall * kPTileBytes, stream, gate, rowtiles,
+                  rows, nb, ap, m_tiles, m_tiles * 16, h, ldh, (int)nb, (int64_t)0, plan, expert_bytes, out_row, gate_shared, up, up_shared,
+                  silu_mode);
+    else if (mt == kMTilesMid)
+        MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true, kMTilesMid>), grid, dim3(256), 2 * kMTilesMid * kPTileBytes, stream, gate, rowtiles,
+                  rows, nb, ap, m_tiles, m_tiles * 16, h, ldh, (int)nb, (int64_t)0, plan, expert_bytes, out_row, gate_shared, up, up_shared,
+                  silu_mode);
+    else
+        MQ_LAUNCH((prefill_gemm_kernel<2, kWtQ4, true>), grid, dim3(256), 2 * kMTilesPerGroup * kPTileBytes, stream, gate, rowtiles, rows, nb,
+                  ap, m_tiles, m_tiles * 16, h, ldh, (int)nb, (int64_t)0, plan, expert_bytes, out_row, gate_shared, up, up_shared, silu_mode);
     return hipGetLastError();
 }
 

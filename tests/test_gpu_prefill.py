@@ -300,3 +300,32 @@ def test_pair_gemm_in_the_moe_block_gives_the_bits_of_two_launches(ops, n, down_
     assert np.array_equal(out[True][0].view(np.uint32), out[False][0].view(np.uint32))
     for w in (ge, ue, de) + sh[:3]:
         w.free()
+
+
+@pytest.mark.parametrize("n,E,K,down_type", [(300, 12, 4, synth.GGML_TYPE_Q4_K), (700, 64, 8, synth.GGML_TYPE_Q6_K), (260, 20, 2, synth.GGML_TYPE_Q5_K)])
+def test_items_of_two_four_and_eight_tiles_give_the_same_bits(ops, n, E, K, down_type):
+    """The expert-grouped GEMM cuts an expert's rows into items of two, four or eight 16-row tiles (chosen by the rows per
+    expert); an output's accumulator walks K the same way in both, so the MoE block must not change by a bit -- gate/up
+    in the pair form and as single products, down of every type, experts with more rows than an item."""
+    from densecore_amd import _lib
+    E_, H, I = E, 1024, 512
+    ge = ops.Q4KWeight.synthetic(synth.tensor_seed("mt-g", E), I, H, E_)
+    ue = ops.Q4KWeight.synthetic(synth.tensor_seed("mt-u", E), I, H, E_)
+    de = ops.Q4KWeight.synthetic(synth.tensor_seed("mt-d", E, down_type), H, I, E_, down_type)
+    x = cu(synth.normal_f32(synth.tensor_seed("mt-x", n), (n, H)))
+    lg = cu(synth.normal_f32(synth.tensor_seed("mt-l", n, E), (n, E_)))
+    out = {}
+    try:
+        for mode in (1 | (2 << 8), 1 | (4 << 8), 1 | (8 << 8), 9 | (2 << 8), 9 | (4 << 8), 1):
+            _lib.lib().mq_debug_set_dense_lds(mode)
+            y, ids, wts = ops.moe_layer(ge, ue, de, x, lg, K, silu=ops.SILU_FAST)
+            yk = ops.mul_mat_id(ge, x, ids)
+            out[mode] = (y.cpu().numpy(), yk.cpu().numpy())
+    finally:
+        _lib.lib().mq_debug_set_dense_lds(1)
+    ref = out[1 | (8 << 8)]
+    for mode, got in out.items():
+        assert np.array_equal(got[0].view(np.uint32), ref[0].view(np.uint32)), f"layer, mode {mode}"
+        assert np.array_equal(got[1].view(np.uint32), ref[1].view(np.uint32)), f"mul_mat_id, mode {mode}"
+    for w in (ge, ue, de):
+        w.free()
