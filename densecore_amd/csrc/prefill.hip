@@ -315,9 +315,10 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     v2u qh[kWTilesPerWave];
     v4u qh6[kWTilesPerWave];      // Q6_K: the top two bits of the codes; seg0 / seg1 hold its nibbles, hdr its sixteen scales
     uint32_t d6[kWTilesPerWave];  // Q6_K: fp16 d
-    auto request_w = [&](int64_t b) {
+    auto request_w = [&](int64_t b, int only = -1) {  // only >= 0: that tile alone
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
+            if (only >= 0 && t != only) continue;
             const uint8_t* tile = (PAIR && t == 1 ? w2 : w) + tile_offset(rt[t], b, nb, tile_stride<WT>());
             seg0[t] = load16(tile + lane * 16);
             seg1[t] = load16(tile + 1024 + lane * 16);
@@ -346,6 +347,49 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
         // ... and after the barrier so has everybody else's share of the activation tiles; every wave
         // is also done reading the other buffer (super-block b-1), which the next requests overwrite
         __syncthreads();
+        if constexpr (PAIR && MT <= 4) {
+            // Few activation tiles: the two weight tiles are expanded and multiplied one after the other, so that one
+            // expanded tile is live at a time (38 registers less: three wavefronts per SIMD instead of two, which is
+            // what a launch of many short workgroups needs); the activation operands are read from LDS once per tile.
+            if (b + 1 < b_end)
+                request_a_tiles<MT>(a_src + (size_t)(b + 1) * a_stride, a_lds + ((b + 1) & 1) * kBufBytes, copy_words, wave, lane);
+            const uint8_t* a_buf = a_lds + (b & 1) * kBufBytes;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                WTile w1;
+                expand_tile<false>(seg0[t], seg1[t], hdr[t], qh[t], kq, w1);
+                if (b + 1 < b_end) request_w(b + 1, t);  // the raw tile's registers are free again
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    if (m < mt_count) {  // uniform over the workgroup
+                        const uint8_t* at = a_buf + m * kPTileBytes;
+                        v4i a[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
+                        const float4 yd = *reinterpret_cast<const float4*>(at + kPScaleOff + kq * 16);
+                        const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
+                        const v8h dg = *reinterpret_cast<const v8h*>(at + digit_off);
+                        const v4i zero = {0, 0, 0, 0};
+                        const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
+                        v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], w1.hi[0], zero, 0, 0, 0);
+                        v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], w1.lo[0], zero, 0, 0, 0);
+                        const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, w1.mins, zero_f, 0, 0, 0);
+#pragma unroll
+                        for (int j = 1; j < 4; ++j) {
+                            hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], w1.hi[j], hi, 0, 0, 0);
+                            lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], w1.lo[j], lo, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {  // the arithmetic of the two-tiles-at-once form below
+                            const int dot = hi[i] * 8 + lo[i];
+                            const float v = __fmaf_rn(-w1.dmin, mn[i], __fmul_rn(w1.d, (float)dot));
+                            acc[t][m][i] = __fmaf_rn(ydv[i], v, acc[t][m][i]);
+                        }
+                    }
+                }
+            }
+            continue;
+        }
         std::conditional_t<Q6, WTile6, WTile> wt[kWTilesPerWave];
 #pragma unroll
         for (int t = 0; t < kWTilesPerWave; ++t) {
