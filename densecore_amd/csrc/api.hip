@@ -1076,7 +1076,7 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
 
 // Widths at which an expert product runs on the matrix-core GEMM in its expert-grouped form (see moe_gemm_applies).
 static bool moe_gemm_width(const mq_weight* w, int64_t n, int top_k) {
-    return (w->type == kTypeQ4K || w->type == kTypeQ5K || w->type == kTypeQ6K) && n >= 256 && n * top_k >= 12 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
+    return (w->type == kTypeQ4K || w->type == kTypeQ5K || w->type == kTypeQ6K) && n >= 192 && n * top_k >= 6 * w->n_experts && w->n_experts <= 4096 && !(w->rows & 3) &&
            !(w->cols & 3);
 }
 
@@ -1596,9 +1596,9 @@ int decoder_grid(size_t lds_bytes, int* n_workgroups, long long* spin_ticks) {
 
 }  // namespace
 
-// The expert-grouped GEMM pays from a dozen routed rows per expert on average (its workgroups multiply 16-row tiles, up to
-// eight of an expert at a time): 256 experts, top-8, 2048 x 512: 242 against 250 us per block at 384 tokens, 262 against
-// 309 at 512, 286 against 374 at 640 -- and 234 against 212 at 320, where the decode kernels' 8-row groups stay.
+// The expert-grouped GEMM pays from six routed rows per expert on average (its workgroups multiply 16-row tiles, two,
+// four or eight of an expert at a time): 256 experts, top-8, 2048 x 512: 152 against 153 us per block at 192 tokens, 158
+// against 186 at 256, 164 against 217 at 320 -- and 141 against 119 at 128, where the decode kernels' 8-row groups stay.
 // Decided per product: gate / up (one type) and down each run on it when their type is one it takes; a layer with
 // a Q8_0 down stack (core/src/llm/moe/native.cpp:4611-4620; its activations are Q8_0 as well) keeps its two large
 // products on the matrix cores and sends the fp32 hidden rows through the Q8_0 launches.
@@ -1607,7 +1607,9 @@ static bool moe_gemm_applies(const mq_moe_layer_desc* L, int64_t n) {
     const mq_weight* ge = L->gate_exps;
     if (!moe_gemm_takes(ge) || !moe_gemm_takes(L->up_exps)) return false;  // the shared expert has the stacks' types
     if (ge->n_experts > 4096 || (ge->rows & 3) || (ge->cols & 3)) return false;
-    return n >= 256 && n * L->top_k >= 12 * ge->n_experts;
+    // (256 + 1 experts, top-8, 2048 x 512, the expert-grouped decode launches against the GEMM with items of two tiles:
+    // 106 / 135 us at 96 tokens, 119 / 141 at 128, 153 / 152 at 192, 186 / 158 at 256, 217 / 164 at 320)
+    return n >= 192 && n * L->top_k >= 6 * ge->n_experts;
 }
 
 int mq_moe_layer_q4k(const mq_moe_layer_desc* L, const float* x_dev, const float* logits_dev, int64_t n, float* y_dev,

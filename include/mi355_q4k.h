@@ -207,8 +207,8 @@ int mq_moe_weights_from_logits(const float* logits_dev, int64_t n_experts, int64
  * [n][top_k]; entries outside [0, n_experts) produce zeros.  Tokens are grouped
  * by expert on the device; nothing returns to the host.  y_dev fp32
  * [n][top_k][rows].  (ggml_mul_mat_id as emitted at
- * core/src/llm/moe/native_gemma.cpp:1509-1559.)  Prefill widths (256 tokens
- * and more with a dozen rows per expert on average) run on the int8 matrix-core
+ * core/src/llm/moe/native_gemma.cpp:1509-1559.)  Prefill widths (192 tokens
+ * and more with six rows per expert on average) run on the int8 matrix-core
  * GEMM in its expert-grouped form, as do mq_moe_gateup_swiglu_q4k and
  * mq_moe_down_weighted_q4k below. */
 int mq_mul_mat_id_q4k(const mq_weight* w_exps, const float* x_dev, int64_t n, int x_slots, const int32_t* ids_dev,
@@ -239,7 +239,7 @@ int mq_moe_down_weighted_q4k(const mq_weight* down_exps, const float* hidden_dev
  * Up to eight tokens (and 512 experts) two launches: gate/up + SwiGLU with the router and the Q8_K of x inside,
  * down with the Q8_K of the hidden rows and the weighted combine inside.  Above: router + expert grouping + Q8_K
  * of x, expert-grouped gate/up leaving its rows in Q8_K, expert-grouped down, combine.  Same bits either way.
- * Prefill widths (256 tokens and more with a dozen routed rows per expert on average): the expert products run on the
+ * Prefill widths (192 tokens and more with six routed rows per expert on average): the expert products run on the
  * int8 matrix-core GEMM in an expert-grouped form (entries in 16-row tiles per expert), the shared expert as one more
  * group of all tokens; a Q8_0 down stack takes the fp32 hidden rows of that gate/up through its own launches; same routing, results within the fp32 tolerance of the other form (the
  * summation order differs), and mq_debug_moe_hidden does not apply. */
