@@ -99,3 +99,26 @@ def test_host_entry_point_from_several_threads(env):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_skeleton_mode_launches_nothing_that_computes_and_restores(env):
+    """mq_debug_set_skeleton: while it is on, a product call queues an empty kernel of the same shape (the output stays as
+    it was); switched off again the same call computes, and the switch reports its previous setting."""
+    import torch
+    from densecore_amd import _lib, ops, synth
+    L = _lib.lib()
+    w = ops.Q4KWeight.synthetic(synth.tensor_seed("skel-w"), 512, 1024)
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("skel-x"), (3, 1024))).cuda()
+    want = ops.mul_mat(w, x).clone()
+    out = torch.full_like(want, 7.0)
+    assert L.mq_debug_set_skeleton(1) == 0
+    try:
+        ops.mul_mat(w, x, out=out)
+        torch.cuda.synchronize()
+        assert torch.all(out == 7.0)
+    finally:
+        assert L.mq_debug_set_skeleton(0) == 1
+    ops.mul_mat(w, x, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    w.free()
