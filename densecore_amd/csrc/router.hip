@@ -134,7 +134,8 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
                                               int32_t* count, int32_t* __restrict__ group_expert,
                                               int32_t* __restrict__ group_begin, int32_t* __restrict__ n_groups,
                                               int32_t* __restrict__ entry_token, int32_t* __restrict__ entry_k,
-                                              uint32_t* token_mask = nullptr, int mask_words = 0, int part = 0, int parts = 1) {
+                                              uint32_t* token_mask = nullptr, int mask_words = 0, int part = 0, int parts = 1,
+                                              uint16_t* mask_prefix = nullptr) {
     const int tid = threadIdx.x, nt = blockDim.x;
     // an expert's mask words are an odd number of words apart: the lanes of a wavefront (consecutive pairs, different
     // experts) walk their experts' words side by side, and an even stride puts them all on one LDS bank (225 us
@@ -202,6 +203,21 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
     }
     __syncthreads();
     const bool by_mask = token_mask && token_mask[n_experts * mask_stride] == 0u;
+    // mask_prefix (LDS, n_experts * mask_stride 16-bit words, or null; at most 65535 tokens): the number of set bits in an
+    // expert's mask words before word w, so that a pair's place costs one look-up and one population count instead of a
+    // walk over all the expert's earlier words (half of them on average: at 2048 tokens 32 LDS reads per pair)
+    if (by_mask && mask_prefix) {
+        for (int e = tid; e < n_experts; e += nt) {
+            const uint32_t* m = token_mask + e * mask_stride;
+            uint16_t* pre = mask_prefix + e * mask_stride;
+            int run = 0;
+            for (int w = 0; w < mask_words; ++w) {
+                pre[w] = (uint16_t)run;
+                run += __popc(m[w]);
+            }
+        }
+        __syncthreads();
+    }
     // several workgroups (parts > 1) all build the counts and masks, each places its share of the pairs
     for (int i = part * nt + tid; i < n_entries; i += parts * nt) {
         const int e = ids[i];
@@ -211,7 +227,9 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
         if (by_mask) {
             const int t = i / top_k;
             const uint32_t* m = token_mask + e * mask_stride;
-            for (int w = 0; w < (t >> 5); ++w) rank += __popc(m[w]);
+            if (mask_prefix) rank = mask_prefix[e * mask_stride + (t >> 5)];
+            else
+                for (int w = 0; w < (t >> 5); ++w) rank += __popc(m[w]);
             rank += __popc(m[t >> 5] & ((1u << (t & 31)) - 1u));
             j = i;  // nothing left to scan
         }
@@ -230,7 +248,7 @@ __device__ __forceinline__ void group_entries(const int32_t* ids, int n_entries,
 }
 
 __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __restrict__ ids, int n_entries,
-                                                            int top_k, int n_experts, int use_lds, int mask_words,
+                                                            int top_k, int n_experts, int use_lds, int mask_words, int with_prefix,
                                                             int32_t* __restrict__ group_expert,
                                                             int32_t* __restrict__ group_begin,
                                                             int32_t* __restrict__ n_groups,
@@ -244,9 +262,10 @@ __global__ void __launch_bounds__(1024) build_groups_kernel(const int32_t* __res
         for (int i = threadIdx.x; i < n_entries; i += blockDim.x) ids_s[i] = ids[i];
         src = ids_s;  // the barrier inside group_entries orders these stores
     }
-    group_entries(src, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k,
-                  mask_words ? reinterpret_cast<uint32_t*>(sh + n_experts + (use_lds ? n_entries : 0)) : nullptr, mask_words,
-                  (int)blockIdx.x, (int)gridDim.x);
+    uint32_t* masks = mask_words ? reinterpret_cast<uint32_t*>(sh + n_experts + (use_lds ? n_entries : 0)) : nullptr;
+    uint16_t* prefix = with_prefix ? reinterpret_cast<uint16_t*>(masks + n_experts * (mask_words | 1) + 1) : nullptr;
+    group_entries(src, n_entries, top_k, n_experts, count, group_expert, group_begin, n_groups, entry_token, entry_k, masks, mask_words,
+                  (int)blockIdx.x, (int)gridDim.x, prefix);
 }
 
 // Router and grouping in one launch (decode widths): a workgroup per token routes it; the last
@@ -489,6 +508,10 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     int mask_words = n <= 4096 ? (int)((n + 31) / 32) : 0;
     if (lds + ((size_t)n_experts * (mask_words | 1) + 1) * 4 > 150 * 1024) mask_words = 0;
     if (mask_words) lds += ((size_t)n_experts * (mask_words | 1) + 1) * 4;
+    // from 512 tokens the prefix counts of the masks join them (where they fit), ahead of the ids
+    const size_t prefix_bytes = ((size_t)n_experts * (mask_words | 1) * 2 + 3) & ~(size_t)3;
+    const int with_prefix = mask_words >= 16 && lds + prefix_bytes <= 150 * 1024;
+    if (with_prefix) lds += prefix_bytes;
     const int use_lds = lds + (size_t)entries * 4 <= 150 * 1024;
     if (use_lds) lds += (size_t)entries * 4;
     if (lds > 64 * 1024) {
@@ -504,7 +527,7 @@ hipError_t launch_build_groups(const int32_t* ids, int64_t n, int top_k, int64_t
     // pairs several workgroups share that part (each repeats the cheap counting): 43 -> 16 us at 16384 pairs
     const unsigned parts = entries >= 3072 ? 8u : 1u;
     MQ_LAUNCH(build_groups_kernel, dim3(parts), dim3(threads), lds, stream, ids, (int)entries, top_k,
-                       (int)n_experts, use_lds, mask_words, group_expert, group_begin, n_groups, entry_token, entry_k);
+                       (int)n_experts, use_lds, mask_words, with_prefix, group_expert, group_begin, n_groups, entry_token, entry_k);
     return hipGetLastError();
 }
 
