@@ -28,8 +28,10 @@ struct mq_weight {
 struct mq_acts {
     void* aq = nullptr;   // A-major codes
     void* ad = nullptr;   // A-major scales
+    void* ap = nullptr;   // handles of more than eight rows: the rows as one P-major tile per super-block as well (written for 9..16 rows)
     int64_t max_rows = 0, cols = 0, nb = 0;
     int64_t n = 0;        // rows quantized by the last mq_acts_quantize
+    bool tile16 = false;  // ap holds those rows (set by the quantizer that wrote both layouts, cleared by one that did not)
 };
 
 // Scratch of mq_mul_mat_q4k_noalloc: the quantized activations (A-major codes, then the scales) of at most
@@ -187,7 +189,28 @@ bool dense_lds_quantizes(const mq_weight* w, const float* x, int64_t n, int64_t 
            dense_lds_applies(w->nb, w->rowtiles, n, swiglu, w->type);
 }
 
+// Nine to sixteen rows of a Q4_K matrix: one activation tile of sixteen rows per weight tile (skinny16_kernel, the same
+// bits as the two tiles of eight of the other decode kernels); mq_debug_set_dense_lds bit 12 turns it off.
+int g_skinny16 = 1;
+bool skinny16_takes(const mq_weight* w, int64_t n, bool swiglu) {
+    return g_skinny16 && g_dense_lds && n > 8 && n <= 16 && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu);
+}
+
 hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
+    if (a.ap) {  // callers ask skinny16_takes first
+        if (a.grouped || a.dbg_dot || a.out_aq || a.wtype != kTypeQ4K) return hipErrorInvalidValue;
+        Skinny16Args k;
+        k.w0 = a.w0;
+        k.w1 = a.swiglu ? a.w1 : nullptr;
+        k.rows = a.rows;
+        k.nb = a.nb;
+        k.ap = a.ap;
+        k.n = a.n;
+        k.y = a.y;
+        k.ldy = a.ldy;
+        k.silu_mode = a.silu_mode;
+        return launch_skinny16(k, s, start, stop);
+    }
     if (!dense_lds_takes(a)) {
         if (a.xf && a.n != 1) return hipErrorInvalidValue;  // callers ask dense_lds_quantizes first
         return launch_matmul(a, s, start, stop);
@@ -291,6 +314,13 @@ int quantize_into(Buffer& aq, Buffer& ad, const float* x, int64_t n, int64_t ldx
     MQ_HIP(aq.reserve(aq_bytes(n, nb)));
     MQ_HIP(ad.reserve(ad_count(n, nb) * sizeof(float)));
     MQ_HIP(launch_quantize_q8k(x, n, ldx, cols, nullptr, 0, (uint8_t*)aq.ptr, (float*)ad.ptr, s));
+    return MQ_OK;
+}
+
+// Quantize up to sixteen rows of x into one P-major tile per super-block (g.ap), the operand of skinny16_kernel.
+int quantize_into_tile16(const float* x, int64_t n, int64_t ldx, int64_t cols, hipStream_t s) {
+    MQ_HIP(g.ap.reserve(pmajor_bytes(n, cols / kQK)));
+    MQ_HIP(launch_quantize_q8k_pmajor(x, n, ldx, cols, (uint8_t*)g.ap.ptr, s));
     return MQ_OK;
 }
 
@@ -683,6 +713,20 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
         MQ_HIP(census_launch(a, s));
         return MQ_OK;
     }
+    if (skinny16_takes(w, n, false)) {  // nine to sixteen rows as one tile of sixteen
+        if (int rc = quantize_into_tile16(x_dev, n, ldx, w->cols, s)) return rc;
+        MatmulArgs a;
+        a.w0 = w->data;
+        a.wtype = w->type;
+        a.rows = w->rows;
+        a.nb = w->nb;
+        a.ap = (const uint8_t*)g.ap.ptr;
+        a.n = n;
+        a.y = y_dev;
+        a.ldy = ldy;
+        MQ_HIP(census_launch(a, s));
+        return MQ_OK;
+    }
     if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, w->cols, s)) return rc;
     return matmul_from_ws(w, n, y_dev, ldy, nullptr, nullptr, s);
 }
@@ -896,8 +940,12 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     // One row: both quantizers run inside the products (two launches instead of four, the same bits).
     const bool one_row = n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u);
     const bool inline_quant = one_row || dense_lds_quantizes(gate, x_dev, n, hidden, true);
-    if (!inline_quant)
+    const bool tile16 = !inline_quant && skinny16_takes(gate, n, true);
+    if (tile16) {
+        if (int rc = quantize_into_tile16(x_dev, n, hidden, hidden, s)) return rc;
+    } else if (!inline_quant) {
         if (int rc = quantize_into(g.aq, g.ad, x_dev, n, hidden, hidden, s)) return rc;
+    }
     MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
     MatmulArgs a;
     a.w0 = gate->data;
@@ -908,6 +956,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (inline_quant) {
         a.xf = x_dev;
         a.ldx = hidden;
+    } else if (tile16) {
+        a.ap = (const uint8_t*)g.ap.ptr;
     } else {
         a.aq = (const uint8_t*)g.aq.ptr;
         a.ad = (const float*)g.ad.ptr;
@@ -921,8 +971,12 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     // The SwiGLU output is re-quantized by a launch of its own: the kernel's fused re-quantization (last
     // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
     const bool inline_quant_down = one_row || dense_lds_quantizes(down, (const float*)g.mid.ptr, n, inter, false);
-    if (!inline_quant_down)
+    const bool tile16_down = !inline_quant_down && skinny16_takes(down, n, false);  // (g.ap again: the gate/up launch ahead on the stream has read it)
+    if (tile16_down) {
+        if (int rc = quantize_into_tile16((const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    } else if (!inline_quant_down) {
         if (int rc = quantize_into(g.aq2, g.ad2, (const float*)g.mid.ptr, n, inter, inter, s)) return rc;
+    }
     MatmulArgs d;
     d.w0 = down->data;
     d.wtype = down->type;
@@ -931,6 +985,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     if (inline_quant_down) {
         d.xf = (const float*)g.mid.ptr;
         d.ldx = inter;
+    } else if (tile16_down) {
+        d.ap = (const uint8_t*)g.ap.ptr;
     } else {
         d.aq = (const uint8_t*)g.aq2.ptr;
         d.ad = (const float*)g.ad2.ptr;
@@ -1008,6 +1064,7 @@ int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* 
     if ((reinterpret_cast<uintptr_t>(x_dev) & 15u) || (normed_out_dev && (reinterpret_cast<uintptr_t>(normed_out_dev) & 15u)))
         return fail(MQ_ERR_INVALID, "mq_add_rmsnorm_q8k: rows must be 16-byte aligned");
     acts->n = n;
+    acts->tile16 = false;  // this producer writes the A-major rows only
     MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, cols, eps, sum_out_dev, normed_out_dev, (uint8_t*)acts->aq,
                               (float*)acts->ad, (hipStream_t)stream));
     return MQ_OK;
@@ -1381,8 +1438,12 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
         return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, 0, s);
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
-    if (!inline_quant)
+    const bool tile16 = !inline_quant && skinny16_takes(gate, n, true);
+    if (tile16) {
+        if (int rc = quantize_into_tile16(x_dev, n, ldx, gate->cols, s)) return rc;
+    } else if (!inline_quant) {
         if (int rc = quantize_into(g.aq, g.ad, x_dev, n, ldx, gate->cols, s)) return rc;
+    }
     MatmulArgs a;
     a.w0 = gate->data;
     a.wtype = gate->type;
@@ -1392,6 +1453,8 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     if (inline_quant) {
         a.xf = x_dev;
         a.ldx = ldx;
+    } else if (tile16) {
+        a.ap = (const uint8_t*)g.ap.ptr;
     } else {
         a.aq = (const uint8_t*)g.aq.ptr;
         a.ad = (const float*)g.ad.ptr;
@@ -1413,8 +1476,10 @@ int mq_acts_create(int64_t max_rows, int64_t cols, mq_acts** out) {
     a->max_rows = max_rows, a->cols = cols, a->nb = cols / kQK;
     hipError_t e = hipMalloc(&a->aq, aq_bytes(max_rows, a->nb));
     if (e == hipSuccess) e = hipMalloc(&a->ad, ad_count(max_rows, a->nb) * sizeof(float));
+    if (e == hipSuccess && max_rows > 8) e = hipMalloc(&a->ap, pmajor_bytes(16, a->nb));
     if (e != hipSuccess) {
         if (a->aq) (void)hipFree(a->aq);
+        if (a->ad) (void)hipFree(a->ad);
         delete a;
         return fail(MQ_ERR_HIP, "mq_acts_create: %s", hipGetErrorString(e));
     }
@@ -1426,6 +1491,7 @@ int mq_acts_free(mq_acts* a) {
     if (!a) return MQ_OK;
     if (a->aq) (void)hipFree(a->aq);
     if (a->ad) (void)hipFree(a->ad);
+    if (a->ap) (void)hipFree(a->ap);
     delete a;
     return MQ_OK;
 }
@@ -1436,8 +1502,12 @@ int mq_acts_quantize(mq_acts* a, const float* x_dev, int64_t n, int64_t ldx, voi
     if (n > a->max_rows) return fail(MQ_ERR_INVALID, "mq_acts_quantize: %lld rows exceed the handle's %lld", (long long)n, (long long)a->max_rows);
     if (int rc = check_x(x_dev, n, ldx, a->cols, "mq_acts_quantize")) return rc;
     a->n = n;
+    a->tile16 = false;
     if (n == 0) return MQ_OK;
     MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, a->cols, nullptr, 0, (uint8_t*)a->aq, (float*)a->ad, (hipStream_t)stream));
+    // nine to sixteen rows: their tile of sixteen as well, for the Q4_K products that take it (skinny16_takes)
+    a->tile16 = n > 8 && n <= 16 && a->ap;
+    if (a->tile16) MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, a->cols, (uint8_t*)a->ap, (hipStream_t)stream));
     return MQ_OK;
 }
 
@@ -1458,8 +1528,12 @@ static int acts_matmul(const mq_weight* w0, const mq_weight* w1, const mq_acts* 
     m.w1 = w1 ? w1->data : nullptr;
     m.rows = w0->rows;
     m.nb = w0->nb;
-    m.aq = (const uint8_t*)a->aq;
-    m.ad = (const float*)a->ad;
+    if (a->tile16 && skinny16_takes(w0, a->n, swiglu != 0)) {
+        m.ap = (const uint8_t*)a->ap;
+    } else {
+        m.aq = (const uint8_t*)a->aq;
+        m.ad = (const float*)a->ad;
+    }
     m.n = a->n;
     m.y = y_dev;
     m.ldy = ldy;
@@ -1966,6 +2040,7 @@ int mq_debug_set_dense_lds(int on) {
     g_gemm_pair = (on & 8) ? 0 : 1;
     g_moe_item_tiles = (on >> 8) & 0xf;      // bits 8..11: activation tiles per item of the expert-grouped GEMM (2, 4 or 8), 0 = by the rows per expert  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
+    g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to sixteen rows stay on the kernels with two token tiles of eight
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;
 }

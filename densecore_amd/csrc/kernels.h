@@ -36,6 +36,8 @@ struct MatmulArgs {
     size_t expert_bytes = 0;       // tiled bytes per expert (grouped mode)
     const uint8_t* aq = nullptr;   // A-major activations
     const float* ad = nullptr;
+    // dense mode, nine to sixteen rows of a Q4_K matrix: the rows as one P-major tile per super-block instead (skinny16_kernel)
+    const uint8_t* ap = nullptr;
     // dense mode, n == 1: the activation row as fp32 instead; every wavefront quantizes the super-blocks it
     // multiplies (same codes and scales as the stand-alone quantizer, so the same result)
     const float* xf = nullptr;
@@ -117,6 +119,23 @@ struct DenseLdsArgs {
 // true when the shape fits the kernel (LDS capacity, wavefront split)
 bool dense_lds_applies(int64_t nb, int64_t rowtiles, int64_t n, bool swiglu, int wtype);
 hipError_t launch_dense_lds(const DenseLdsArgs& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
+
+// Wavefronts per row tile of the LDS-staged dense kernels for a matrix (pick_waves, as a divisor of eight; 0: none)
+int dense_lds_wpr(int64_t nb, int64_t rowtiles);
+
+// ---- prefill.hip: nine to sixteen rows as ONE activation tile against a streamed Q4_K matrix (skinny16_kernel) ----
+struct Skinny16Args {
+    const uint8_t* w0 = nullptr;   // tiled Q4_K weights; gate when w1 is set
+    const uint8_t* w1 = nullptr;   // up weights: y = silu(w0 x) * (w1 x)
+    int64_t rows = 0, nb = 0;
+    const uint8_t* ap = nullptr;   // the rows' P-major tile of every super-block: [nb][4688] (launch_quantize_q8k_pmajor on up to 16 rows)
+    int64_t n = 0;                 // live rows, 1..16
+    float* y = nullptr;
+    int64_t ldy = 0;
+    int silu_mode = 0;
+};
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu);
+hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 // ---- q8_0.hip --------------------------------------------------------------------------------
 // Q8_0 weights (16-row tiles of common.h) x Q8_0 activations, dense, any n (passes of eight rows).

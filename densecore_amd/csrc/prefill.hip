@@ -37,8 +37,11 @@
 //   [tok][32 B] at 4096                  fp16: l_0..l_7, then 128 h_0..128 h_7
 //   [tok] fp32 at 4608                   block scale d
 //   16 zero bytes at 4672                what the lanes of k-groups 2 and 3 feed the min MFMA
+#include <hip/hip_ext.h>
+
 #include "common.h"
 #include "kernels.h"
+#include "decode_tile.h"
 #include "q8k_block.h"
 
 namespace mq {
@@ -520,6 +523,202 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
     }
 }
 
+// ---- nine to sixteen activation rows against a streamed matrix ------------------------------------------------
+// The decode kernels multiply a weight tile with EIGHT activation rows per MFMA (the sixteen operand rows hold a row's
+// two sub-blocks of a 64-weight chunk side by side, the sub-block scales are applied on the vector unit); from nine rows
+// they take two such token tiles per weight tile: 16 MFMAs and ~147 vector instructions.  This kernel multiplies the
+// same rows as ONE tile of sixteen, the way prefill_gemm_kernel does (scale digits folded into the weight operand, the
+// min term as one fp16 MFMA): 9 MFMAs and ~126 vector instructions per weight tile.  Everything else is
+// dense_lds_kernel's (dense_lds.hip): eight wavefronts, WPR of them per row tile taking the super-blocks h, h + WPR, ...
+// in ascending order, partial sums met in wave order, two register stages of raw weight tiles; the rows' quantized
+// activations -- here P-major tiles -- are staged in LDS once per workgroup while the first weight tiles travel, or,
+// where all super-blocks do not fit LDS (GA: the 14336 columns of an FFN's down projection), requested from global
+// memory a stage ahead, beside the weight tile (six loads, all answered by the L2).  The integers of a (row, token,
+// super-block) are the same and so is the fp32 update, (wd * yd) * dot - (wm * yd) * min_dot added to the running
+// sum: the same bits as dense_lds_kernel and matmul_kernel.
+// LDS: [nb][4688] activation tiles (not GA), then the partial sums [8 / WPR][WPR - 1][NMAT][4][64].
+// nb % WPR == 0 (host-checked): every wavefront has nb / WPR stages; ODD: that count is odd.
+struct ATile16 {
+    v4i a[4];   // the four 64-weight chunks of this lane's operand
+    v4f yd;     // the Q8_K scales of rows 4 kq .. 4 kq + 3
+    v8h dg;     // this lane's operand of the min MFMA (fp16 digits of the sub-block sums, or zeros)
+};
+
+template <int NMAT, int WPR, bool ODD, bool GA>
+__global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
+    constexpr int RPW = 8 / WPR;  // row tiles per workgroup
+    extern __shared__ __align__(16) uint8_t lds16[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, kq = lane >> 4;
+    const int nb = (int)p.nb;
+    const int64_t rowtiles = (p.rows + 15) >> 4;
+    const int pair = wave / WPR, h = wave % WPR;
+    int64_t rt = (int64_t)blockIdx.x * RPW + pair;
+    const bool dead = rt >= rowtiles;  // past the last row tile: stream the last one again and store nothing
+    if (dead) rt = rowtiles - 1;
+    float* red = reinterpret_cast<float*>(lds16 + (GA ? (size_t)0 : (size_t)nb * kPTileBytes));
+
+    const uint8_t* tiles[NMAT];
+    tiles[0] = p.w0 + tile_offset(rt, 0, nb, kTileBytes);
+    if (NMAT == 2) tiles[1] = p.w1 + tile_offset(rt, 0, nb, kTileBytes);
+    const int cnt = nb / WPR;  // stages of this wavefront: super-blocks h, h + WPR, ...
+
+    // lane (r, kq): weight row r of the tile, activation rows 4 kq .. 4 kq + 3
+    const int digit_off = kq < 2 ? kPDigitOff + r * 32 + kq * 16 : kPZeroOff;
+    auto read_a = [&](ATile16& t, const uint8_t* at) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t.a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
+        t.yd = *reinterpret_cast<const v4f*>(at + kPScaleOff + kq * 16);
+        t.dg = *reinterpret_cast<const v8h*>(at + digit_off);
+    };
+
+    if constexpr (!GA) {
+        // ---- the activation tiles -> LDS: a linear copy, 1 KB per request, the wavefronts taking the requests in turn ----
+        const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr_t)lds16;
+        const int words = nb * kPTileWords;
+        for (int c = wave; c * 64 < words; c += 8) {
+            const int first = c * 64;
+            if (first + lane < words) {
+                const uint8_t* g = p.ap + (size_t)(first + lane) * 16;
+                const uint32_t dst = base + (uint32_t)first * 16u;
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
+            }
+        }
+    }
+
+    TileRegs ring_t[2][NMAT];
+    ATile16 ring_a[GA ? 2 : 1];
+    auto issue = [&](auto st_c, int i) {  // only ever called for a stage that exists
+        constexpr int st = decltype(st_c)::value;
+        const int b = h + i * WPR;
+        if constexpr (GA) read_a(ring_a[st], p.ap + (size_t)b * kPTileBytes);  // ahead of the tiles: it is needed first
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) load_tile<false>(ring_t[st][m], tiles[m] + (size_t)b * kTileBytes, lane);
+    };
+
+    float acc[NMAT][4];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[m][i] = 0.0f;
+
+    auto consume = [&](auto st_c, int i) {
+        constexpr int st = decltype(st_c)::value;
+        const int b = h + i * WPR;
+        ATile16 from_lds;
+        if constexpr (!GA) read_a(from_lds, lds16 + (size_t)b * kPTileBytes);
+        const ATile16& t = GA ? ring_a[GA ? st : 0] : from_lds;
+        const float ydv[4] = {t.yd.x, t.yd.y, t.yd.z, t.yd.w};
+        const v8h dg = t.dg;
+        const v4i zero = {0, 0, 0, 0};
+        const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            WTile wt;
+            expand_tile<false>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, v2u{0u, 0u}, kq, wt);
+            v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[0], wt.hi[0], zero, 0, 0, 0);
+            v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[0], wt.lo[0], zero, 0, 0, 0);
+            const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt.mins, zero_f, 0, 0, 0);
+#pragma unroll
+            for (int j = 1; j < 4; ++j) {
+                hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[j], wt.hi[j], hi, 0, 0, 0);
+                lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[j], wt.lo[j], lo, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile's update (decode_tile.h); mn[i2] is the integer min_dot, exactly
+                const int dot = hi[i2] * 8 + lo[i2];
+                const float d = __fmul_rn(wt.d, ydv[i2]);
+                const float dm = __fmul_rn(wt.dmin, ydv[i2]);
+                const float term = __fsub_rn(__fmul_rn(d, (float)dot), __fmul_rn(dm, mn[i2]));
+                acc[m][i2] = __fadd_rn(acc[m][i2], term);
+            }
+        }
+    };
+
+    // Two register stages, one in flight while the other is multiplied; written out for an even and for an odd number
+    // of stages (an odd run is one stage followed by an even run with the stages' roles swapped), so that no request
+    // is ever made for a stage that does not exist.
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    const bool single = ODD && cnt == 1;  // wave-uniform
+    issue(S0{}, 0);
+    asm volatile("" ::: "memory");  // requests stay in stage order
+    if (!single) {
+        issue(S1{}, 1);
+        asm volatile("" ::: "memory");
+    }
+    if constexpr (!GA) {
+        // the LDS-direct copies are older than the tile requests: they have landed once at most those are outstanding
+        if (single) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NMAT * 3) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NMAT * 3) : "memory");
+        __builtin_amdgcn_s_barrier();  // no fence: a fence would wait for the outstanding weight tiles as well
+        asm volatile("" ::: "memory");
+    }
+    if constexpr (ODD) {
+        consume(S0{}, 0);
+        if (!single) {
+            issue(S0{}, 2);  // cnt >= 3
+            asm volatile("" ::: "memory");
+            int i = 1;
+            for (; i + 2 < cnt; i += 2) {
+                consume(S1{}, i);
+                issue(S1{}, i + 2);
+                asm volatile("" ::: "memory");
+                consume(S0{}, i + 1);
+                issue(S0{}, i + 3);
+                asm volatile("" ::: "memory");
+            }
+            consume(S1{}, i);
+            consume(S0{}, i + 1);
+        }
+    } else {
+        int i = 0;
+        for (; i + 2 < cnt; i += 2) {
+            consume(S0{}, i);
+            issue(S0{}, i + 2);
+            asm volatile("" ::: "memory");
+            consume(S1{}, i + 1);
+            issue(S1{}, i + 3);
+            asm volatile("" ::: "memory");
+        }
+        consume(S0{}, i);
+        consume(S1{}, i + 1);
+    }
+
+    // ---- the WPR wavefronts of a row tile meet in wave order; the first one stores ----
+    if (WPR > 1) {
+        if (h > 0) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((((pair * (WPR - 1) + (h - 1)) * NMAT + m) * 4 + i) * 64) + lane] = acc[m][i];
+        }
+        __syncthreads();
+    }
+    if (h == 0 && !dead) {
+        for (int wv = 1; wv < WPR; ++wv) {
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[m][i] = __fadd_rn(acc[m][i], red[((((pair * (WPR - 1) + (wv - 1)) * NMAT + m) * 4 + i) * 64) + lane]);
+        }
+        const int64_t row = rt * 16 + r;
+        if (row < p.rows) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int tok = 4 * kq + i;
+                if (tok < p.n) {
+                    float v = acc[0][i];
+                    if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][i], p.silu_mode);
+                    p.y[(size_t)tok * (size_t)p.ldy + (size_t)row] = v;
+                }
+            }
+        }
+    }
+}
+
 // One workgroup per (tile of 16 activation rows, super-block): its four wavefronts quantize four rows each into an
 // image of the tile in LDS, which then leaves as one run of 16-byte stores (a wavefront per row writing straight to
 // the tile scattered its 256 bytes over 32 cache lines: 52 us for the 16384 gathered rows of a MoE block at 2048
@@ -528,8 +727,10 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 // pass of its own; h_out, if given, receives it as fp32 as well.
 // Expert-grouped forms: plan (tiles past plan[1] are skipped), row_src (row m of the tiles is row row_src[m] of x, -1:
 // padding, zeros), h_rows (row m of the tiles is row h_rows[m] of h_out, -1: not written).
-template <bool kSwiglu>
-__global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* __restrict__ x, const float* __restrict__ x2,
+// kRowsPerWave: four (256 threads) in general; one (1024 threads, a wavefront per row) for launches of a few workgroups
+// (sixteen rows: one workgroup per super-block), where the four rows one after the other are the launch's length.
+template <bool kSwiglu, int kRowsPerWave = 4>
+__global__ void __launch_bounds__(64 * 16 / kRowsPerWave) quantize_q8k_pmajor_kernel(const float* __restrict__ x, const float* __restrict__ x2,
                                                                   int silu_mode, float* __restrict__ h_out, int64_t ldh,
                                                                   int64_t n, int64_t ldx, int64_t nb, int64_t m_tiles,
                                                                   uint8_t* __restrict__ ap, const int32_t* __restrict__ plan,
@@ -540,16 +741,17 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     const int64_t tile = blockIdx.x, b = blockIdx.y;
     if (plan && tile >= (int64_t)plan[1]) return;  // the whole workgroup, before the barrier
     if (plan && kSwiglu && tile >= (int64_t)plan[2]) silu_mode = plan[3];  // the shared expert's tiles: its own SiLU form
-    int64_t src[4], hr[4];
-    float4 v[4], u[4];
+    constexpr int kThreads = 64 * 16 / kRowsPerWave;
+    int64_t src[kRowsPerWave], hr[kRowsPerWave];
+    float4 v[kRowsPerWave], u[kRowsPerWave];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int64_t m = tile * 16 + wave * 4 + r;
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        const int64_t m = tile * 16 + wave * kRowsPerWave + r;
         src[r] = row_src ? row_src[m] : (m < n ? m : -1);
         hr[r] = h_rows ? h_rows[m] : src[r];
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {  // all of the wavefront's rows are requested before any is worked on
+    for (int r = 0; r < kRowsPerWave; ++r) {  // all of the wavefront's rows are requested before any is worked on
         const int64_t from = src[r] >= 0 ? src[r] : 0;
         v[r] = *reinterpret_cast<const float4*>(x + from * ldx + b * kQK + lane * 4);
         if (kSwiglu) u[r] = *reinterpret_cast<const float4*>(x2 + from * ldx + b * kQK + lane * 4);
@@ -559,8 +761,8 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     const int j = 2 * (g >> 2) + (g & 1), half = (g >> 1) & 1;
     const int kq = (lane & 7) >> 1;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int tok = wave * 4 + r;
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        const int tok = wave * kRowsPerWave + r;
         float e[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (src[r] >= 0) {  // wave-uniform
             e[0] = v[r].x, e[1] = v[r].y, e[2] = v[r].z, e[3] = v[r].w;
@@ -584,7 +786,7 @@ __global__ void __launch_bounds__(256) quantize_q8k_pmajor_kernel(const float* _
     if (tid < 4) *reinterpret_cast<uint32_t*>(img + kPZeroOff + tid * 4) = 0u;
     __syncthreads();
     v4u* dst = reinterpret_cast<v4u*>(ap + ((size_t)b * (size_t)m_tiles + (size_t)tile) * kPTileBytes);
-    for (int i = tid; i < kPTileWords; i += 256) dst[i] = reinterpret_cast<const v4u*>(img)[i];
+    for (int i = tid; i < kPTileWords; i += kThreads) dst[i] = reinterpret_cast<const v4u*>(img)[i];
 }
 
 // The expert-grouped tiles of rows that repeat (a token is a row of top_k experts, and of the shared one): the distinct
@@ -948,6 +1150,12 @@ hipError_t launch_quantize_q8k_pmajor(const float* x, int64_t n, int64_t ldx, in
     const int64_t nb = k / kQK, m_tiles = (n + 15) / 16;
     if (m_tiles == 0 || nb == 0) return hipSuccess;
     if (nb > 65535 || m_tiles >= (int64_t)1 << 31) return hipErrorInvalidValue;
+    if (m_tiles * nb <= 64 && !plan) {  // a few workgroups (sixteen rows of a decode-width product): a wavefront per row
+        MQ_LAUNCH((quantize_q8k_pmajor_kernel<false, 1>), dim3((unsigned)m_tiles, (unsigned)nb), dim3(1024), 0, stream, x,
+                  (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, plan, (const int32_t*)nullptr,
+                  (const int32_t*)nullptr);
+        return hipGetLastError();
+    }
     MQ_LAUNCH(quantize_q8k_pmajor_kernel<false>, dim3((unsigned)m_tiles, (unsigned)nb), dim3(256), 0, stream, x,
                        (const float*)nullptr, 0, (float*)nullptr, (int64_t)0, n, ldx, nb, m_tiles, ap, plan,
                        (const int32_t*)nullptr, (const int32_t*)nullptr);
@@ -1011,6 +1219,69 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
                            rows, y, ldy);
     }
     return hipGetLastError();
+}
+
+// ---- skinny16 -------------------------------------------------------------------------------------------------
+namespace {
+
+size_t skinny16_lds_bytes(int nmat, int wpr, int64_t nb, bool ga) {
+    return (ga ? (size_t)0 : (size_t)nb * kPTileBytes) + (size_t)(8 / wpr) * (wpr - 1) * nmat * 4 * 64 * sizeof(float);
+}
+bool skinny16_in_lds(int nmat, int wpr, int64_t nb) { return skinny16_lds_bytes(nmat, wpr, nb, false) <= 160 * 1024; }
+
+template <int NMAT, int WPR, bool ODD, bool GA>
+hipError_t launch_skinny16_one(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    const int64_t rowtiles = (a.rows + 15) / 16;
+    const size_t lds = skinny16_lds_bytes(NMAT, WPR, a.nb, GA);
+    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA>;
+    static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    constexpr int RPW = 8 / WPR;
+    const dim3 grid((unsigned)((rowtiles + RPW - 1) / RPW));
+    if (start && stop) hipExtLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, start, stop, 0, a);
+    else MQ_LAUNCH(kernel, grid, dim3(512), lds, stream, a);
+    return hipGetLastError();
+}
+
+template <int NMAT, int WPR>
+hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    const bool odd = ((a.nb / WPR) & 1) != 0, ga = !skinny16_in_lds(NMAT, WPR, a.nb);
+    if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false>(a, stream, start, stop);
+    return ga ? launch_skinny16_one<NMAT, WPR, false, true>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false>(a, stream, start, stop);
+}
+
+template <int NMAT>
+hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    switch (wpr) {
+        case 1: return launch_skinny16_form<NMAT, 1>(a, stream, start, stop);
+        case 2: return launch_skinny16_form<NMAT, 2>(a, stream, start, stop);
+        case 4: return launch_skinny16_form<NMAT, 4>(a, stream, start, stop);
+        case 8: return launch_skinny16_form<NMAT, 8>(a, stream, start, stop);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+// Whether a Q4_K product of nine to sixteen rows runs on skinny16_kernel: the wave split of the other decode kernels
+// must be one of its own (a divisor of eight that divides the super-blocks of a row).
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu) {
+    (void)swiglu;
+    const int wpr = dense_lds_wpr(nb, rowtiles);
+    return wpr && nb % wpr == 0;
+}
+
+hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 16 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
+    const int64_t rowtiles = (a.rows + 15) / 16;
+    if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr)) return hipErrorInvalidValue;
+    const int wpr = dense_lds_wpr(a.nb, rowtiles);
+    if (a.w1) return launch_skinny16_wpr<2>(a, wpr, stream, start, stop);
+    return launch_skinny16_wpr<1>(a, wpr, stream, start, stop);
 }
 
 }  // namespace mq

@@ -1,0 +1,159 @@
+"""Dense Q4_K products of nine to sixteen rows as ONE activation tile of sixteen (skinny16_kernel) against the kernels
+that take the same rows as two token tiles of eight: the same bits for every wave split the kernel has (one, two, four
+and eight wavefronts per row tile), ragged row counts, strided rows, the fused gate/up form and the whole FFN -- and
+within 1e-4 of every fp32 accumulation order the reference has."""
+import numpy as np
+import pytest
+
+from densecore_amd import synth
+from oracle import binding as orc
+from tests._parity import assert_fp32_parity, oracle_all_orders
+
+pytestmark = pytest.mark.gpu
+
+TWO_TILES_OF_EIGHT = 1 | 0x1000   # mq_debug_set_dense_lds: LDS-staged kernels on, the sixteen-row tile off
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from densecore_amd import _lib, ops
+    assert torch.cuda.is_available()
+    yield torch, _lib, ops
+    _lib.lib().mq_debug_set_dense_lds(1)
+
+
+def three_ways(env, fn):
+    """global-operand kernel, LDS-staged kernel with two token tiles, the sixteen-row tile"""
+    torch, _lib, ops = env
+    L = _lib.lib()
+    out = []
+    for mode in (0, TWO_TILES_OF_EIGHT, 1):
+        L.mq_debug_set_dense_lds(mode)
+        out.append(fn().clone())
+    torch.cuda.synchronize()
+    L.mq_debug_set_dense_lds(1)
+    return [o.cpu().numpy() for o in out]
+
+
+# rows, cols: wavefronts per row tile 2 (896 row tiles), 8, 8 with a ragged last tile, 4, 1, 2 with workgroups past the end,
+# 8 with all of LDS in use; then odd stage counts: one stage per wavefront (2048 x 2048, 1000 x 1024), seven with the
+# activation tiles read from global memory (the FFN's down projection: 56 super-blocks do not fit LDS), an even count
+# from global memory, and a wave split the kernel does not have (six: falls back to two token tiles)
+SHAPES = [(14336, 4096), (4096, 4096), (1000, 4096), (6144, 4096), (20480, 1024), (14000, 2048), (2048, 8192),
+          (2048, 2048), (1000, 1024), (4096, 14336), (512, 16384), (2560, 3072)]
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_single_matrix_same_bits(env, rows, cols):
+    torch, _lib, ops = env
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("s16", rows, cols), rows, cols)
+    for n in (9, 11, 16):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-x", rows, cols, n), (n, cols))).cuda()
+        a, b, c = three_ways(env, lambda: ops.mul_mat(W, x))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32)), f"n={n}: against the global-operand kernel"
+        assert np.array_equal(b.view(np.uint32), c.view(np.uint32)), f"n={n}: against two token tiles in LDS"
+    W.free()
+
+
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (1024, 4096), (3000, 2048)])
+@pytest.mark.parametrize("silu", [0, 1, 2])
+def test_gate_up_same_bits(env, rows, cols, silu):
+    torch, _lib, ops = env
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-g", rows, cols), rows, cols)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-u", rows, cols), rows, cols)
+    for n in (9, 13, 16):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-gx", rows, cols, n), (n, cols))).cuda()
+        a, b, c = three_ways(env, lambda: ops.swiglu_mul_mat(G, U, x, silu))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32)), f"n={n}"
+        assert np.array_equal(b.view(np.uint32), c.view(np.uint32)), f"n={n}"
+    G.free(), U.free()
+
+
+def test_strided_rows_and_strided_output(env):
+    torch, _lib, ops = env
+    W = ops.Q4KWeight.synthetic(11, 1024, 4096)
+    n = 14
+    buf = torch.from_numpy(synth.normal_f32(1100 + n, (n, 4096 + 64))).cuda()
+    x = buf[:, :4096]
+
+    def raw():
+        y = torch.full((n, W.rows + 32), 7.0, dtype=torch.float32, device="cuda")
+        _lib.check(_lib.lib().mq_mul_mat_q4k(W._h, x.data_ptr(), n, x.stride(0), y.data_ptr(), y.stride(0), None), "mq_mul_mat_q4k")
+        return y
+    a, b, c = three_ways(env, raw)
+    assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+    assert np.all(c[:, W.rows:] == 7.0)
+    ref = ops.mul_mat(W, x.contiguous()).cpu().numpy()
+    assert np.array_equal(ref.view(np.uint32), c[:, :W.rows].view(np.uint32))
+    W.free()
+
+
+@pytest.mark.parametrize("hidden,inter", [(4096, 14336), (4096, 4096)])
+def test_ffn_same_bits_and_graph_replay(env, hidden, inter):
+    """gate/up on the sixteen-row tile with its rows in LDS; down on it as well, its rows in LDS (inter 4096) or read
+    from global memory a stage ahead (inter 14336)."""
+    torch, _lib, ops = env
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-fg", inter), inter, hidden)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-fu", inter), inter, hidden)
+    D = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-fd", inter), hidden, inter)
+    for n in (10, 16):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-fx", n), (n, hidden))).cuda()
+        a, b, c = three_ways(env, lambda: ops.ffn_swiglu(G, U, D, x, ops.SILU_FAST))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32)), f"n={n}"
+        assert np.array_equal(b.view(np.uint32), c.view(np.uint32)), f"n={n}"
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-fx", 16), (16, hidden))).cuda()
+    eager = ops.ffn_swiglu(G, U, D, x, ops.SILU_FAST).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    out = {}
+    with torch.cuda.graph(g, stream=side):
+        out["y"] = ops.ffn_swiglu(G, U, D, x, ops.SILU_FAST)
+    for _ in range(3):
+        out["y"].fill_(3.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out["y"], eager)
+    G.free(), U.free(), D.free()
+
+
+def test_against_the_oracle(env):
+    torch, _lib, ops = env
+    rows, cols, n = 272, 4096, 13   # 17 row tiles, eight wavefronts per row tile
+    w_np = synth.q4k_matrix(synth.tensor_seed("s16-ow"), rows, cols)
+    W = ops.Q4KWeight.from_ggml(w_np, cols, synth.GGML_TYPE_Q4_K)
+    x = synth.normal_f32(synth.tensor_seed("s16-ox"), (n, cols))
+    y = ops.mul_mat(W, torch.from_numpy(x).cuda()).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(x)
+    mag = orc.dot_magnitude_f64(w_np, cols, q8)
+    for name, ref in oracle_all_orders(w_np, cols, q8).items():
+        assert_fp32_parity(y, ref, mag, f"order={name}")
+    W.free()
+
+
+def test_shared_activation_handle_keeps_its_tile_of_sixteen_current(env):
+    """A handle of more than eight rows carries the rows' tile of sixteen beside the A-major rows: mq_acts_quantize
+    writes both, mq_add_rmsnorm_q8k only the A-major ones -- a product from the handle must then not read the stale
+    tile.  Both ways the product equals the one-shot entry point on the same fp32 rows."""
+    import ctypes as C
+    torch, _lib, ops = env
+    L = _lib.lib()
+    rows, cols, n = 4096, 4096, 12
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-hw"), rows, cols)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s16-hu"), rows, cols)
+    x1 = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-h1"), (n, cols))).cuda()
+    x2 = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s16-h2"), (n, cols))).cuda()
+    acts = ops.Q8KActs(16, cols)
+    acts.quantize(x1)
+    assert torch.equal(acts.mul_mat(W), ops.mul_mat(W, x1))
+    assert torch.equal(acts.swiglu_mul_mat(W, U, 2), ops.swiglu_mul_mat(W, U, x1, 2))
+    p = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    normed = torch.empty_like(x2)
+    _lib.check(L.mq_add_rmsnorm_q8k(p(x2), None, None, n, cols, C.c_float(1e-6), None, p(normed), C.c_void_p(acts._h), None), "norm")
+    acts.n = n
+    assert torch.equal(acts.mul_mat(W), ops.mul_mat(W, normed))
+    acts.quantize(x2[:9])
+    assert torch.equal(acts.mul_mat(W), ops.mul_mat(W, x2[:9]))
+    acts.free(), W.free(), U.free()
