@@ -791,16 +791,23 @@ int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, in
     if (entry.rc) return entry.rc;
     uint8_t* aq = ws;
     float* ad = reinterpret_cast<float*>(ws + kNoAllocAqBytes);
-    // Every byte of the scratch that the product reads is written by this call's quantizer (slots past row n read
-    // row n - 1), so nothing of an earlier call is seen and nothing needs clearing.
-    MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, w->cols, nullptr, 0, aq, ad, s));
     MatmulArgs a;
     a.w0 = w->data;
     a.wtype = w->type;
     a.rows = w->rows;
     a.nb = w->nb;
-    a.aq = aq;
-    a.ad = ad;
+    // Every byte of the scratch that the product reads is written by this call's quantizer (slots past row n read
+    // row n - 1; rows past n of a tile of sixteen are written as zeros), so nothing of an earlier call is seen and
+    // nothing needs clearing.
+    static_assert((kNoAllocMaxCols / mq::kQK) * 4688 <= kNoAllocAqBytes + kNoAllocAdBytes, "the rows' tiles of sixteen fit the scratch as well");
+    if (skinny16_takes(w, n, false)) {  // nine to sixteen rows: one P-major tile per super-block, in the same scratch
+        MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, w->cols, ws, s));
+        a.ap = ws;
+    } else {
+        MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, w->cols, nullptr, 0, aq, ad, s));
+        a.aq = aq;
+        a.ad = ad;
+    }
     a.n = n;
     a.y = y_dev;
     a.ldy = ldy;
