@@ -323,21 +323,20 @@ def main() -> int:
 
     del blocker
     # ---------------------------------------------------------------- per-width detail
-    per_width = {}
-    for n in WIDTHS:
+    def width_detail(n, x):
         for i in range(RING):
-            ops.ffn_swiglu(*sets[i], xs[n], ops.SILU_FAST_FMA)
+            ops.ffn_swiglu(*sets[i], x, ops.SILU_FAST_FMA)
         torch.cuda.synchronize()
         reps = 256
         t1 = time.perf_counter()
         if graphs is None:
             for i in range(reps):
-                ops.ffn_swiglu(*sets[i % RING], xs[n], ops.SILU_FAST_FMA)
+                ops.ffn_swiglu(*sets[i % RING], x, ops.SILU_FAST_FMA)
         else:
             gph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(gph, stream=side_stream):
                 for i in range(RING):
-                    ops.ffn_swiglu(*sets[i], xs[n], ops.SILU_FAST_FMA)
+                    ops.ffn_swiglu(*sets[i], x, ops.SILU_FAST_FMA)
             gph.replay()            # one untimed replay: the first one also uploads the graph
             torch.cuda.synchronize()
             t1 = time.perf_counter()
@@ -345,9 +344,17 @@ def main() -> int:
                 gph.replay()
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t1) / reps
-        per_width[str(n)] = {"us": round(dt * 1e6, 2), "GBps": round(ffn_bytes(n) / dt / 1e9, 1),
-                             "pct_hbm_peak": round(ffn_bytes(n) / dt / 1e9 / HBM_PEAK_GBPS * 100, 1),
-                             "tokens_per_s": round(n / dt, 1)}
+        return {"us": round(dt * 1e6, 2), "GBps": round(ffn_bytes(n) / dt / 1e9, 1),
+                "pct_hbm_peak": round(ffn_bytes(n) / dt / 1e9 / HBM_PEAK_GBPS * 100, 1), "tokens_per_s": round(n / dt, 1)}
+
+    per_width = {str(n): width_detail(n, xs[n]) for n in WIDTHS}
+    # the same FFN pass at widths between the workload's sixteen rows and the GEMM's prefill widths (not part of `value`)
+    wider = {}
+    for n in (24, 32, 48):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg2-x", n), (n, HIDDEN))).to(dev)
+        wider[str(n)] = width_detail(n, x)
+    wider["note"] = ("the cfg2 FFN pass beyond its widths, same cold ring: up to 32 rows on the decode arithmetic "
+                     "(two activation tiles of sixteen per weight tile), from 33 on the matrix-core GEMM")
 
     extras = {}
     if not args.no_extras:
@@ -374,6 +381,7 @@ def main() -> int:
         "pct_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 1),
         "step_spread": step_spread,
         "per_width": per_width,
+        "ffn_pass_wider": wider,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

@@ -189,11 +189,14 @@ bool dense_lds_quantizes(const mq_weight* w, const float* x, int64_t n, int64_t 
            dense_lds_applies(w->nb, w->rowtiles, n, swiglu, w->type);
 }
 
-// Nine to sixteen rows of a Q4_K matrix: one activation tile of sixteen rows per weight tile (skinny16_kernel, the same
-// bits as the two tiles of eight of the other decode kernels); mq_debug_set_dense_lds bit 12 turns it off.
+// Nine to thirty-two rows of a Q4_K matrix: one or two activation tiles of sixteen rows per weight tile
+// (skinny16_kernel, the same bits as the token tiles of eight of the other decode kernels); mq_debug_set_dense_lds
+// bit 12 turns it off.  kSkinnyMaxRows: beyond it the matrix-core GEMM (large matrices) or the 16-row passes of the
+// decode kernels take over.
 int g_skinny16 = 1;
+constexpr int64_t kSkinnyMaxRows = 32;
 bool skinny16_takes(const mq_weight* w, int64_t n, bool swiglu) {
-    return g_skinny16 && g_dense_lds && n > 8 && n <= 16 && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu);
+    return g_skinny16 && g_dense_lds && n > 8 && n <= kSkinnyMaxRows && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu);
 }
 
 hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
@@ -317,7 +320,7 @@ int quantize_into(Buffer& aq, Buffer& ad, const float* x, int64_t n, int64_t ldx
     return MQ_OK;
 }
 
-// Quantize up to sixteen rows of x into one P-major tile per super-block (g.ap), the operand of skinny16_kernel.
+// Quantize up to thirty-two rows of x into one or two P-major tiles per super-block (g.ap), the operand of skinny16_kernel.
 int quantize_into_tile16(const float* x, int64_t n, int64_t ldx, int64_t cols, hipStream_t s) {
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, cols / kQK)));
     MQ_HIP(launch_quantize_q8k_pmajor(x, n, ldx, cols, (uint8_t*)g.ap.ptr, s));
@@ -566,7 +569,9 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
 
 // Activation rows from which the matrix-core GEMM beats re-streaming the weights per 16-row chunk: 48 in general,
 // 17 for matrices of 24 MB and more (14336 x 4096 and 4096 x 14336: 19 against 24 us at 17 rows, 21 against 35-38 us
-// at 47; 4096 x 4096: 17.4 against 14.1 us at 17 rows, 17.9 against 14.6 at 47).
+// at 47; 4096 x 4096: 17.4 against 14.1 us at 17 rows, 17.9 against 14.6 at 47).  Q4_K products of up to 32 rows go to
+// skinny16_kernel ahead of both (skinny16_takes: gate/up of a 4096 -> 14336 FFN 41 -> 22 us at 17 to 32 rows,
+// 4096 x 4096 11.5 -> 9.5 us).
 constexpr int64_t kPrefillMinRows = 48;
 constexpr int64_t kPrefillMinRowsLarge = 17;
 constexpr int64_t kPrefillLargeBytes = 24ll << 20;
@@ -683,7 +688,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
     Entry entry(s);
     if (entry.rc) return entry.rc;
     if (w->type == kTypeQ80) return mul_mat_q80_locked(w, x_dev, n, ldx, y_dev, ldy, nullptr, s);
-    if (prefill_applies(w, n)) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
+    if (prefill_applies(w, n) && !skinny16_takes(w, n, false)) return gemm_locked(w, x_dev, n, ldx, y_dev, ldy, s);
     if (n == 1 && w->type == kTypeQ4K) {  // single row, short K per wave: the quantizer runs inside the GEMV kernel
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
@@ -713,7 +718,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
         MQ_HIP(census_launch(a, s));
         return MQ_OK;
     }
-    if (skinny16_takes(w, n, false)) {  // nine to sixteen rows as one tile of sixteen
+    if (skinny16_takes(w, n, false)) {  // nine to thirty-two rows as one or two tiles of sixteen
         if (int rc = quantize_into_tile16(x_dev, n, ldx, w->cols, s)) return rc;
         MatmulArgs a;
         a.w0 = w->data;
@@ -940,7 +945,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (prefill_applies(gate, n) && prefill_applies(down, n)) {  // wide: the matrix-core GEMM, three times
+    const bool tiles16 = skinny16_takes(gate, n, true) && skinny16_takes(down, n, false);  // up to 32 rows: the decode kernels below
+    if (!tiles16 && prefill_applies(gate, n) && prefill_applies(down, n)) {  // wide: the matrix-core GEMM, three times
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
         return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, hidden, s);
     }
@@ -1441,7 +1447,7 @@ int mq_swiglu_mul_mat_q4k(const mq_weight* gate, const mq_weight* up, const floa
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    if (prefill_applies(gate, n) && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
+    if (prefill_applies(gate, n) && !skinny16_takes(gate, n, true) && !(ldh & 3) && !(reinterpret_cast<uintptr_t>(h_dev) & 15u))
         return ffn_wide_locked(gate, up, nullptr, x_dev, n, ldx, silu_mode, h_dev, ldh, nullptr, 0, s);
     // one row, or a few where the LDS-staged kernel applies: the quantizer runs inside the product
     const bool inline_quant = (n == 1 && !(reinterpret_cast<uintptr_t>(x_dev) & 15u)) || dense_lds_quantizes(gate, x_dev, n, ldx, true);
@@ -2047,7 +2053,7 @@ int mq_debug_set_dense_lds(int on) {
     g_gemm_pair = (on & 8) ? 0 : 1;
     g_moe_item_tiles = (on >> 8) & 0xf;      // bits 8..11: activation tiles per item of the expert-grouped GEMM (2, 4 or 8), 0 = by the rows per expert  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
-    g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to sixteen rows stay on the kernels with two token tiles of eight
+    g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to thirty-two rows stay on the kernels with token tiles of eight (or the GEMM)
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;
 }

@@ -128,8 +128,8 @@ struct Skinny16Args {
     const uint8_t* w0 = nullptr;   // tiled Q4_K weights; gate when w1 is set
     const uint8_t* w1 = nullptr;   // up weights: y = silu(w0 x) * (w1 x)
     int64_t rows = 0, nb = 0;
-    const uint8_t* ap = nullptr;   // the rows' P-major tile of every super-block: [nb][4688] (launch_quantize_q8k_pmajor on up to 16 rows)
-    int64_t n = 0;                 // live rows, 1..16
+    const uint8_t* ap = nullptr;   // the rows' P-major tiles: [nb][tiles][4688], tiles = 1 (up to 16 rows) or 2 (launch_quantize_q8k_pmajor)
+    int64_t n = 0;                 // live rows, 1..32
     float* y = nullptr;
     int64_t ldy = 0;
     int silu_mode = 0;

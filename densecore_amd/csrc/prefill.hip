@@ -544,9 +544,13 @@ struct ATile16 {
     v8h dg;     // this lane's operand of the min MFMA (fp16 digits of the sub-block sums, or zeros)
 };
 
-template <int NMAT, int WPR, bool ODD, bool GA>
+// MT: activation tiles of sixteen rows (one, or two for 17 to 32 rows: the weight tile is expanded once for both, 18
+// MFMAs and ~156 vector instructions against the 32 + 294 of two passes over two token tiles of eight each).  With two
+// tiles the partial sums share LDS with the activation tiles (one more barrier before they are written).
+template <int NMAT, int WPR, bool ODD, bool GA, int MT>
 __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     constexpr int RPW = 8 / WPR;  // row tiles per workgroup
+    constexpr bool kRedShares = MT > 1 && !GA;  // the partial sums reuse the activation tiles' LDS
     extern __shared__ __align__(16) uint8_t lds16[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -557,14 +561,14 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     int64_t rt = (int64_t)blockIdx.x * RPW + pair;
     const bool dead = rt >= rowtiles;  // past the last row tile: stream the last one again and store nothing
     if (dead) rt = rowtiles - 1;
-    float* red = reinterpret_cast<float*>(lds16 + (GA ? (size_t)0 : (size_t)nb * kPTileBytes));
+    float* red = reinterpret_cast<float*>(lds16 + ((GA || kRedShares) ? (size_t)0 : (size_t)nb * MT * kPTileBytes));
 
     const uint8_t* tiles[NMAT];
     tiles[0] = p.w0 + tile_offset(rt, 0, nb, kTileBytes);
     if (NMAT == 2) tiles[1] = p.w1 + tile_offset(rt, 0, nb, kTileBytes);
     const int cnt = nb / WPR;  // stages of this wavefront: super-blocks h, h + WPR, ...
 
-    // lane (r, kq): weight row r of the tile, activation rows 4 kq .. 4 kq + 3
+    // lane (r, kq): weight row r of the tile, activation rows 4 kq .. 4 kq + 3 of every activation tile
     const int digit_off = kq < 2 ? kPDigitOff + r * 32 + kq * 16 : kPZeroOff;
     auto read_a = [&](ATile16& t, const uint8_t* at) {
 #pragma unroll
@@ -574,9 +578,9 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     };
 
     if constexpr (!GA) {
-        // ---- the activation tiles -> LDS: a linear copy, 1 KB per request, the wavefronts taking the requests in turn ----
+        // ---- the activation tiles ([super-block][tile]) -> LDS: a linear copy, 1 KB per request, the wavefronts taking the requests in turn ----
         const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr_t)lds16;
-        const int words = nb * kPTileWords;
+        const int words = nb * MT * kPTileWords;
         for (int c = wave; c * 64 < words; c += 8) {
             const int first = c * 64;
             if (first + lane < words) {
@@ -588,50 +592,57 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     }
 
     TileRegs ring_t[2][NMAT];
-    ATile16 ring_a[GA ? 2 : 1];
+    ATile16 ring_a[GA ? 2 : 1][GA ? MT : 1];
     auto issue = [&](auto st_c, int i) {  // only ever called for a stage that exists
         constexpr int st = decltype(st_c)::value;
         const int b = h + i * WPR;
-        if constexpr (GA) read_a(ring_a[st], p.ap + (size_t)b * kPTileBytes);  // ahead of the tiles: it is needed first
+        if constexpr (GA) {  // ahead of the tiles: they are needed first
+#pragma unroll
+            for (int t = 0; t < MT; ++t) read_a(ring_a[st][t], p.ap + ((size_t)b * MT + t) * kPTileBytes);
+        }
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) load_tile<false>(ring_t[st][m], tiles[m] + (size_t)b * kTileBytes, lane);
     };
 
-    float acc[NMAT][4];
+    float acc[NMAT][MT][4];
 #pragma unroll
     for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[m][i] = 0.0f;
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[m][t][i] = 0.0f;
 
     auto consume = [&](auto st_c, int i) {
         constexpr int st = decltype(st_c)::value;
         const int b = h + i * WPR;
-        ATile16 from_lds;
-        if constexpr (!GA) read_a(from_lds, lds16 + (size_t)b * kPTileBytes);
-        const ATile16& t = GA ? ring_a[GA ? st : 0] : from_lds;
-        const float ydv[4] = {t.yd.x, t.yd.y, t.yd.z, t.yd.w};
-        const v8h dg = t.dg;
         const v4i zero = {0, 0, 0, 0};
         const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) {
             WTile wt;
             expand_tile<false>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, v2u{0u, 0u}, kq, wt);
-            v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[0], wt.hi[0], zero, 0, 0, 0);
-            v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[0], wt.lo[0], zero, 0, 0, 0);
-            const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(dg, wt.mins, zero_f, 0, 0, 0);
 #pragma unroll
-            for (int j = 1; j < 4; ++j) {
-                hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[j], wt.hi[j], hi, 0, 0, 0);
-                lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(t.a[j], wt.lo[j], lo, 0, 0, 0);
-            }
+            for (int t = 0; t < MT; ++t) {
+                ATile16 from_lds;
+                if constexpr (!GA) read_a(from_lds, lds16 + ((size_t)b * MT + t) * kPTileBytes);
+                const ATile16& at = GA ? ring_a[GA ? st : 0][GA ? t : 0] : from_lds;
+                const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
+                v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.hi[0], zero, 0, 0, 0);
+                v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.lo[0], zero, 0, 0, 0);
+                const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.dg, wt.mins, zero_f, 0, 0, 0);
 #pragma unroll
-            for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile's update (decode_tile.h); mn[i2] is the integer min_dot, exactly
-                const int dot = hi[i2] * 8 + lo[i2];
-                const float d = __fmul_rn(wt.d, ydv[i2]);
-                const float dm = __fmul_rn(wt.dmin, ydv[i2]);
-                const float term = __fsub_rn(__fmul_rn(d, (float)dot), __fmul_rn(dm, mn[i2]));
-                acc[m][i2] = __fadd_rn(acc[m][i2], term);
+                for (int j = 1; j < 4; ++j) {
+                    hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[j], wt.hi[j], hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[j], wt.lo[j], lo, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile's update (decode_tile.h); mn[i2] is the integer min_dot, exactly
+                    const int dot = hi[i2] * 8 + lo[i2];
+                    const float d = __fmul_rn(wt.d, ydv[i2]);
+                    const float dm = __fmul_rn(wt.dmin, ydv[i2]);
+                    const float term = __fsub_rn(__fmul_rn(d, (float)dot), __fmul_rn(dm, mn[i2]));
+                    acc[m][t][i2] = __fadd_rn(acc[m][t][i2], term);
+                }
             }
         }
     };
@@ -688,11 +699,15 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
 
     // ---- the WPR wavefronts of a row tile meet in wave order; the first one stores ----
     if (WPR > 1) {
+        if (kRedShares) __syncthreads();  // every wavefront has read its last activation tile
         if (h > 0) {
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) red[((((pair * (WPR - 1) + (h - 1)) * NMAT + m) * 4 + i) * 64) + lane] = acc[m][i];
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        red[(((((pair * (WPR - 1) + (h - 1)) * NMAT + m) * MT + t) * 4 + i) * 64) + lane] = acc[m][t][i];
         }
         __syncthreads();
     }
@@ -701,20 +716,24 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    acc[m][i] = __fadd_rn(acc[m][i], red[((((pair * (WPR - 1) + (wv - 1)) * NMAT + m) * 4 + i) * 64) + lane]);
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[m][t][i] = __fadd_rn(acc[m][t][i], red[(((((pair * (WPR - 1) + (wv - 1)) * NMAT + m) * MT + t) * 4 + i) * 64) + lane]);
         }
         const int64_t row = rt * 16 + r;
         if (row < p.rows) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int tok = 4 * kq + i;
-                if (tok < p.n) {
-                    float v = acc[0][i];
-                    if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][i], p.silu_mode);
-                    p.y[(size_t)tok * (size_t)p.ldy + (size_t)row] = v;
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int tok = 16 * t + 4 * kq + i;
+                    if (tok < p.n) {
+                        float v = acc[0][t][i];
+                        if (NMAT == 2) v = silu_mul(v, acc[NMAT - 1][t][i], p.silu_mode);
+                        p.y[(size_t)tok * (size_t)p.ldy + (size_t)row] = v;
+                    }
                 }
-            }
         }
     }
 }
@@ -1224,16 +1243,20 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
 // ---- skinny16 -------------------------------------------------------------------------------------------------
 namespace {
 
-size_t skinny16_lds_bytes(int nmat, int wpr, int64_t nb, bool ga) {
-    return (ga ? (size_t)0 : (size_t)nb * kPTileBytes) + (size_t)(8 / wpr) * (wpr - 1) * nmat * 4 * 64 * sizeof(float);
+size_t skinny16_red_bytes(int nmat, int wpr, int mt) { return (size_t)(8 / wpr) * (wpr - 1) * nmat * mt * 4 * 64 * sizeof(float); }
+// LDS of the form with the rows' tiles in LDS: with one tile of sixteen the partial sums lie behind the tiles, with two
+// they share the tiles' bytes
+size_t skinny16_lds_bytes(int nmat, int wpr, int64_t nb, int mt) {
+    const size_t tiles = (size_t)nb * mt * kPTileBytes, red = skinny16_red_bytes(nmat, wpr, mt);
+    return mt > 1 ? (tiles > red ? tiles : red) : tiles + red;
 }
-bool skinny16_in_lds(int nmat, int wpr, int64_t nb) { return skinny16_lds_bytes(nmat, wpr, nb, false) <= 160 * 1024; }
+bool skinny16_in_lds(int nmat, int wpr, int64_t nb, int mt) { return skinny16_lds_bytes(nmat, wpr, nb, mt) <= 160 * 1024; }
 
-template <int NMAT, int WPR, bool ODD, bool GA>
+template <int NMAT, int WPR, bool ODD, bool GA, int MT>
 hipError_t launch_skinny16_one(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int64_t rowtiles = (a.rows + 15) / 16;
-    const size_t lds = skinny16_lds_bytes(NMAT, WPR, a.nb, GA);
-    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA>;
+    const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT);
+    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT>;
     static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1247,28 +1270,28 @@ hipError_t launch_skinny16_one(const Skinny16Args& a, hipStream_t stream, hipEve
     return hipGetLastError();
 }
 
-template <int NMAT, int WPR>
+template <int NMAT, int WPR, int MT>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
-    const bool odd = ((a.nb / WPR) & 1) != 0, ga = !skinny16_in_lds(NMAT, WPR, a.nb);
-    if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false>(a, stream, start, stop);
-    return ga ? launch_skinny16_one<NMAT, WPR, false, true>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false>(a, stream, start, stop);
+    const bool odd = ((a.nb / WPR) & 1) != 0, ga = !skinny16_in_lds(NMAT, WPR, a.nb, MT);
+    if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT>(a, stream, start, stop);
+    return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT>(a, stream, start, stop);
 }
 
-template <int NMAT>
+template <int NMAT, int MT>
 hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     switch (wpr) {
-        case 1: return launch_skinny16_form<NMAT, 1>(a, stream, start, stop);
-        case 2: return launch_skinny16_form<NMAT, 2>(a, stream, start, stop);
-        case 4: return launch_skinny16_form<NMAT, 4>(a, stream, start, stop);
-        case 8: return launch_skinny16_form<NMAT, 8>(a, stream, start, stop);
+        case 1: return launch_skinny16_form<NMAT, 1, MT>(a, stream, start, stop);
+        case 2: return launch_skinny16_form<NMAT, 2, MT>(a, stream, start, stop);
+        case 4: return launch_skinny16_form<NMAT, 4, MT>(a, stream, start, stop);
+        case 8: return launch_skinny16_form<NMAT, 8, MT>(a, stream, start, stop);
     }
     return hipErrorInvalidValue;
 }
 
 }  // namespace
 
-// Whether a Q4_K product of nine to sixteen rows runs on skinny16_kernel: the wave split of the other decode kernels
-// must be one of its own (a divisor of eight that divides the super-blocks of a row).
+// Whether a Q4_K product of nine to thirty-two rows runs on skinny16_kernel: the wave split of the other decode
+// kernels must be one of its own (a divisor of eight that divides the super-blocks of a row).
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu) {
     (void)swiglu;
     const int wpr = dense_lds_wpr(nb, rowtiles);
@@ -1276,12 +1299,16 @@ bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu) {
 }
 
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
-    if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 16 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
+    if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 32 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
     if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr)) return hipErrorInvalidValue;
     const int wpr = dense_lds_wpr(a.nb, rowtiles);
-    if (a.w1) return launch_skinny16_wpr<2>(a, wpr, stream, start, stop);
-    return launch_skinny16_wpr<1>(a, wpr, stream, start, stop);
+    if (a.n > 16) {
+        if (a.w1) return launch_skinny16_wpr<2, 2>(a, wpr, stream, start, stop);
+        return launch_skinny16_wpr<1, 2>(a, wpr, stream, start, stop);
+    }
+    if (a.w1) return launch_skinny16_wpr<2, 1>(a, wpr, stream, start, stop);
+    return launch_skinny16_wpr<1, 1>(a, wpr, stream, start, stop);
 }
 
 }  // namespace mq

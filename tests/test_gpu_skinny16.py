@@ -157,3 +157,65 @@ def test_shared_activation_handle_keeps_its_tile_of_sixteen_current(env):
     acts.quantize(x2[:9])
     assert torch.equal(acts.mul_mat(W), ops.mul_mat(W, x2[:9]))
     acts.free(), W.free(), U.free()
+
+
+# ---- seventeen to thirty-two rows: two tiles of sixteen per weight tile ----------------------------------------------
+
+SMALL = [(4096, 4096), (2048, 2048), (1000, 4096), (6144, 4096), (20480, 1024), (2048, 8192), (512, 16384), (2560, 3072)]
+
+
+@pytest.mark.parametrize("rows,cols", SMALL)
+def test_two_tiles_single_matrix_same_bits_as_the_sixteen_row_passes(env, rows, cols):
+    """Matrices below the GEMM's size threshold: the other decode kernel runs 17 to 32 rows as passes of sixteen in one
+    launch (switch 0), the LDS-staged ones do not take them (switch 0x1001 ends on the same kernel)."""
+    torch, _lib, ops = env
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("s32", rows, cols), rows, cols)
+    for n in (17, 25, 32):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s32-x", rows, cols, n), (n, cols))).cuda()
+        a, b, c = three_ways(env, lambda: ops.mul_mat(W, x))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32)), f"n={n}"
+        assert np.array_equal(b.view(np.uint32), c.view(np.uint32)), f"n={n}"
+    W.free()
+
+
+@pytest.mark.parametrize("rows,cols", [(1024, 4096), (3000, 2048), (512, 1024)])
+@pytest.mark.parametrize("silu", [0, 2])
+def test_two_tiles_gate_up_same_bits(env, rows, cols, silu):
+    torch, _lib, ops = env
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("s32-g", rows, cols), rows, cols)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s32-u", rows, cols), rows, cols)
+    for n in (18, 32):
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s32-gx", rows, cols, n), (n, cols))).cuda()
+        a, b, c = three_ways(env, lambda: ops.swiglu_mul_mat(G, U, x, silu))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32)), f"n={n}"
+    G.free(), U.free()
+
+
+@pytest.mark.parametrize("n", [17, 23, 32])
+def test_two_tiles_on_ffn_sized_matrices_equal_the_rows_taken_sixteen_at_a_time(env, n):
+    """Matrices of 24 MB and more used to go to the matrix-core GEMM from 17 rows (another fp32 update, other bits); up to
+    32 rows they now stay on the decode arithmetic.  Every row's result is independent of the rows beside it, so the
+    product and the whole FFN must equal the same rows handed over sixteen at a time, bit for bit -- and the oracle."""
+    torch, _lib, ops = env
+    hidden, inter = 4096, 14336
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("s32-fg"), inter, hidden)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s32-fu"), inter, hidden)
+    D = ops.Q4KWeight.synthetic(synth.tensor_seed("s32-fd"), hidden, inter)
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s32-fx", n), (n, hidden))).cuda()
+    h = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s32-fh", n), (n, inter))).cuda()
+    parts = lambda fn, t: torch.cat([fn(t[:16]), fn(t[16:])], dim=0)
+    for name, fn, t in (("gate", lambda t: ops.mul_mat(G, t), x), ("down (rows read from global memory)", lambda t: ops.mul_mat(D, t), h),
+                        ("gate/up", lambda t: ops.swiglu_mul_mat(G, U, t, 1), x), ("ffn", lambda t: ops.ffn_swiglu(G, U, D, t, ops.SILU_FAST), x)):
+        whole, split = fn(t), parts(fn, t)
+        assert torch.equal(whole, split), name
+    # the oracle on sampled rows of the down projection (K = 14336: 56 super-blocks, seven per wavefront)
+    w_np = synth.q4k_matrix(synth.tensor_seed("s32-ow"), 64, inter)
+    W = ops.Q4KWeight.from_ggml(w_np, inter, synth.GGML_TYPE_Q4_K)
+    hx = h.cpu().numpy()
+    y = ops.mul_mat(W, h).cpu().numpy()
+    q8 = orc.quantize_rows_q8k(hx)
+    mag = orc.dot_magnitude_f64(w_np, inter, q8)
+    for name, ref in oracle_all_orders(w_np, inter, q8).items():
+        assert_fp32_parity(y, ref, mag, f"order={name}")
+    for w in (G, U, D, W):
+        w.free()
