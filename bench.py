@@ -350,11 +350,11 @@ def main() -> int:
     per_width = {str(n): width_detail(n, xs[n]) for n in WIDTHS}
     # the same FFN pass at widths between the workload's sixteen rows and the GEMM's prefill widths (not part of `value`)
     wider = {}
-    for n in (24, 32, 48):
+    for n in (24, 32, 48, 64):
         x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("cfg2-x", n), (n, HIDDEN))).to(dev)
         wider[str(n)] = width_detail(n, x)
-    wider["note"] = ("the cfg2 FFN pass beyond its widths, same cold ring: up to 32 rows on the decode arithmetic "
-                     "(two activation tiles of sixteen per weight tile), from 33 on the matrix-core GEMM")
+    wider["note"] = ("the cfg2 FFN pass beyond its widths, same cold ring: gate/up on the decode arithmetic up to 64 rows (up to four "
+                     "activation tiles of sixteen per weight tile), down likewise up to 32 rows and on the matrix-core GEMM from 33")
 
     extras = {}
     if not args.no_extras:

@@ -189,14 +189,14 @@ bool dense_lds_quantizes(const mq_weight* w, const float* x, int64_t n, int64_t 
            dense_lds_applies(w->nb, w->rowtiles, n, swiglu, w->type);
 }
 
-// Nine to thirty-two rows of a Q4_K matrix: one or two activation tiles of sixteen rows per weight tile
+// Nine to 64 rows of a Q4_K matrix: one to four activation tiles of sixteen rows per weight tile
 // (skinny16_kernel, the same bits as the token tiles of eight of the other decode kernels); mq_debug_set_dense_lds
 // bit 12 turns it off.  kSkinnyMaxRows: beyond it the matrix-core GEMM (large matrices) or the 16-row passes of the
 // decode kernels take over.
 int g_skinny16 = 1;
-constexpr int64_t kSkinnyMaxRows = 32;
+constexpr int64_t kSkinnyMaxRows = 64;
 bool skinny16_takes(const mq_weight* w, int64_t n, bool swiglu) {
-    return g_skinny16 && g_dense_lds && n > 8 && n <= kSkinnyMaxRows && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu);
+    return g_skinny16 && g_dense_lds && n > 8 && n <= kSkinnyMaxRows && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu, n);
 }
 
 hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
@@ -320,7 +320,7 @@ int quantize_into(Buffer& aq, Buffer& ad, const float* x, int64_t n, int64_t ldx
     return MQ_OK;
 }
 
-// Quantize up to thirty-two rows of x into one or two P-major tiles per super-block (g.ap), the operand of skinny16_kernel.
+// Quantize up to 64 rows of x into one to four P-major tiles per super-block (g.ap), the operand of skinny16_kernel.
 int quantize_into_tile16(const float* x, int64_t n, int64_t ldx, int64_t cols, hipStream_t s) {
     MQ_HIP(g.ap.reserve(pmajor_bytes(n, cols / kQK)));
     MQ_HIP(launch_quantize_q8k_pmajor(x, n, ldx, cols, (uint8_t*)g.ap.ptr, s));
@@ -718,7 +718,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
         MQ_HIP(census_launch(a, s));
         return MQ_OK;
     }
-    if (skinny16_takes(w, n, false)) {  // nine to thirty-two rows as one or two tiles of sixteen
+    if (skinny16_takes(w, n, false)) {  // nine to 64 rows as one to four tiles of sixteen
         if (int rc = quantize_into_tile16(x_dev, n, ldx, w->cols, s)) return rc;
         MatmulArgs a;
         a.w0 = w->data;
@@ -945,8 +945,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     hipStream_t s = (hipStream_t)stream;
     Entry entry(s);
     if (entry.rc) return entry.rc;
-    const bool tiles16 = skinny16_takes(gate, n, true) && skinny16_takes(down, n, false);  // up to 32 rows: the decode kernels below
-    if (!tiles16 && prefill_applies(gate, n) && prefill_applies(down, n)) {  // wide: the matrix-core GEMM, three times
+    const bool gateup16 = skinny16_takes(gate, n, true);  // up to 64 rows: gate/up on the decode arithmetic below
+    if (!gateup16 && prefill_applies(gate, n) && prefill_applies(down, n)) {  // wide: the matrix-core GEMM, three times
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)inter * sizeof(float)));
         return ffn_wide_locked(gate, up, down, x_dev, n, hidden, silu_mode, (float*)g.mid.ptr, inter, y_dev, hidden, s);
     }
@@ -985,6 +985,8 @@ int mq_ffn_swiglu_q4k(const mq_weight* gate, const mq_weight* up, const mq_weigh
     // workgroup per 256-row block) serialises n rows per block at the kernel's tail and measures slower here.
     const bool inline_quant_down = one_row || dense_lds_quantizes(down, (const float*)g.mid.ptr, n, inter, false);
     const bool tile16_down = !inline_quant_down && skinny16_takes(down, n, false);  // (g.ap again: the gate/up launch ahead on the stream has read it)
+    // beyond the rows the decode kernels take for this matrix (its rows are too long to pass through LDS): the GEMM on the SwiGLU rows
+    if (!tile16_down && prefill_applies(down, n)) return gemm_locked(down, (const float*)g.mid.ptr, n, inter, y_dev, hidden, s);
     if (tile16_down) {
         if (int rc = quantize_into_tile16((const float*)g.mid.ptr, n, inter, inter, s)) return rc;
     } else if (!inline_quant_down) {
@@ -2053,7 +2055,7 @@ int mq_debug_set_dense_lds(int on) {
     g_gemm_pair = (on & 8) ? 0 : 1;
     g_moe_item_tiles = (on >> 8) & 0xf;      // bits 8..11: activation tiles per item of the expert-grouped GEMM (2, 4 or 8), 0 = by the rows per expert  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
-    g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to thirty-two rows stay on the kernels with token tiles of eight (or the GEMM)
+    g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to 64 rows stay on the kernels with token tiles of eight (or the GEMM)
     if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
     return before;
 }

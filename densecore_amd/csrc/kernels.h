@@ -128,13 +128,14 @@ struct Skinny16Args {
     const uint8_t* w0 = nullptr;   // tiled Q4_K weights; gate when w1 is set
     const uint8_t* w1 = nullptr;   // up weights: y = silu(w0 x) * (w1 x)
     int64_t rows = 0, nb = 0;
-    const uint8_t* ap = nullptr;   // the rows' P-major tiles: [nb][tiles][4688], tiles = 1 (up to 16 rows) or 2 (launch_quantize_q8k_pmajor)
-    int64_t n = 0;                 // live rows, 1..32
+    const uint8_t* ap = nullptr;   // the rows' P-major tiles: [nb][tiles][4688], tiles = ceil(n / 16) (launch_quantize_q8k_pmajor)
+    int64_t n = 0;                 // live rows, 1..64
     float* y = nullptr;
     int64_t ldy = 0;
     int silu_mode = 0;
+    int ranges = 1;                // set by the launcher: runs of super-blocks the tiles pass through LDS in
 };
-bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu);
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n);
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 // ---- q8_0.hip --------------------------------------------------------------------------------

@@ -561,7 +561,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     int64_t rt = (int64_t)blockIdx.x * RPW + pair;
     const bool dead = rt >= rowtiles;  // past the last row tile: stream the last one again and store nothing
     if (dead) rt = rowtiles - 1;
-    float* red = reinterpret_cast<float*>(lds16 + ((GA || kRedShares) ? (size_t)0 : (size_t)nb * MT * kPTileBytes));
+    float* red = reinterpret_cast<float*>(lds16 + ((GA || kRedShares) ? (size_t)0 : (size_t)nb * MT * kPTileBytes));  // (one run when the sums lie behind the tiles)
 
     const uint8_t* tiles[NMAT];
     tiles[0] = p.w0 + tile_offset(rt, 0, nb, kTileBytes);
@@ -577,19 +577,25 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
         t.dg = *reinterpret_cast<const v8h*>(at + digit_off);
     };
 
-    if constexpr (!GA) {
-        // ---- the activation tiles ([super-block][tile]) -> LDS: a linear copy, 1 KB per request, the wavefronts taking the requests in turn ----
+    // ---- the activation tiles ([super-block][tile]) -> LDS: a linear copy, 1 KB per request, the wavefronts taking the
+    // requests in turn.  Rows too long for LDS in one piece come in `ranges` runs of super-blocks, one run at a time:
+    // stage i of every wavefront lies in run i / (cnt / ranges), so the wavefronts change runs together (cnt % ranges == 0,
+    // host-checked).
+    const int sb_per_range = nb / p.ranges, stages_per_range = cnt / p.ranges;
+    auto stage_range = [&](int rg) {
         const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr_t)lds16;
-        const int words = nb * MT * kPTileWords;
+        const int words = sb_per_range * MT * kPTileWords;
+        const uint8_t* src = p.ap + (size_t)rg * (size_t)words * 16;
         for (int c = wave; c * 64 < words; c += 8) {
             const int first = c * 64;
             if (first + lane < words) {
-                const uint8_t* g = p.ap + (size_t)(first + lane) * 16;
+                const uint8_t* g = src + (size_t)(first + lane) * 16;
                 const uint32_t dst = base + (uint32_t)first * 16u;
                 asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(dst) : "memory", "m0");
             }
         }
-    }
+    };
+    if constexpr (!GA) stage_range(0);
 
     TileRegs ring_t[2][NMAT];
     ATile16 ring_a[GA ? 2 : 1][GA ? MT : 1];
@@ -612,6 +618,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[m][t][i] = 0.0f;
 
+    int b_range0 = 0;  // first super-block of the run in LDS
     auto consume = [&](auto st_c, int i) {
         constexpr int st = decltype(st_c)::value;
         const int b = h + i * WPR;
@@ -619,12 +626,15 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
         const v4f zero_f = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) {
+            // three and four tiles: the second matrix reads the activation tiles from LDS again instead of keeping the first
+            // one's copies in registers (they would not fit)
+            if (MT > 2 && m > 0) asm volatile("" ::: "memory");
             WTile wt;
             expand_tile<false>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, v2u{0u, 0u}, kq, wt);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 ATile16 from_lds;
-                if constexpr (!GA) read_a(from_lds, lds16 + ((size_t)b * MT + t) * kPTileBytes);
+                if constexpr (!GA) read_a(from_lds, lds16 + ((size_t)(b - b_range0) * MT + t) * kPTileBytes);
                 const ATile16& at = GA ? ring_a[GA ? st : 0][GA ? t : 0] : from_lds;
                 const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
                 v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.hi[0], zero, 0, 0, 0);
@@ -684,16 +694,30 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             consume(S0{}, i + 1);
         }
     } else {
+        // the next run of super-blocks replaces the one in LDS once every wavefront has multiplied its last stage of it
+        auto next_range = [&](int i) {
+            if (GA || p.ranges == 1 || i == 0 || i % stages_per_range) return;  // wave-uniform, the same i in every wavefront
+            __syncthreads();
+            const int rg = i / stages_per_range;
+            stage_range(rg);
+            b_range0 = rg * sb_per_range;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the copy (and its two stages of weight tiles)
+            __syncthreads();
+        };
         int i = 0;
         for (; i + 2 < cnt; i += 2) {
+            next_range(i);
             consume(S0{}, i);
             issue(S0{}, i + 2);
             asm volatile("" ::: "memory");
+            next_range(i + 1);
             consume(S1{}, i + 1);
             issue(S1{}, i + 3);
             asm volatile("" ::: "memory");
         }
+        next_range(i);
         consume(S0{}, i);
+        next_range(i + 1);
         consume(S1{}, i + 1);
     }
 
@@ -1243,38 +1267,61 @@ hipError_t launch_prefill_gemm(const uint8_t* w, int wtype, int64_t rows, int64_
 // ---- skinny16 -------------------------------------------------------------------------------------------------
 namespace {
 
+constexpr size_t kSkinnyLdsMax = 160 * 1024;
+
 size_t skinny16_red_bytes(int nmat, int wpr, int mt) { return (size_t)(8 / wpr) * (wpr - 1) * nmat * mt * 4 * 64 * sizeof(float); }
-// LDS of the form with the rows' tiles in LDS: with one tile of sixteen the partial sums lie behind the tiles, with two
-// they share the tiles' bytes
-size_t skinny16_lds_bytes(int nmat, int wpr, int64_t nb, int mt) {
-    const size_t tiles = (size_t)nb * mt * kPTileBytes, red = skinny16_red_bytes(nmat, wpr, mt);
+// LDS of the form with the rows' tiles in LDS, `ranges` runs of super-blocks one after the other: with one tile of
+// sixteen the partial sums lie behind the tiles, with more they share the tiles' bytes
+size_t skinny16_lds_bytes(int nmat, int wpr, int64_t nb, int mt, int ranges) {
+    const size_t tiles = (size_t)(nb / ranges) * mt * kPTileBytes, red = skinny16_red_bytes(nmat, wpr, mt);
     return mt > 1 ? (tiles > red ? tiles : red) : tiles + red;
 }
-bool skinny16_in_lds(int nmat, int wpr, int64_t nb, int mt) { return skinny16_lds_bytes(nmat, wpr, nb, mt) <= 160 * 1024; }
+// Runs of super-blocks the rows' tiles need to pass through LDS (1, 2 or 4; every wavefront must have a whole number
+// of stages per run), or 0: they do not fit that way.
+int skinny16_ranges(int nmat, int wpr, int64_t nb, int mt) {
+    for (int ranges = 1; ranges <= 4; ranges *= 2) {
+        if (ranges > 1 && (mt == 1 || nb % ((int64_t)wpr * ranges))) break;
+        if (skinny16_lds_bytes(nmat, wpr, nb, mt, ranges) <= kSkinnyLdsMax) return ranges;
+    }
+    return 0;
+}
 
 template <int NMAT, int WPR, bool ODD, bool GA, int MT>
-hipError_t launch_skinny16_one(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int64_t rowtiles = (a.rows + 15) / 16;
-    const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT);
+    const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT, ranges);
     auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT>;
     static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
         if (e != hipSuccess) return e;
         raised = true;
     }
+    Skinny16Args b = a;
+    b.ranges = GA ? 1 : ranges;
     constexpr int RPW = 8 / WPR;
     const dim3 grid((unsigned)((rowtiles + RPW - 1) / RPW));
-    if (start && stop) hipExtLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, start, stop, 0, a);
-    else MQ_LAUNCH(kernel, grid, dim3(512), lds, stream, a);
+    if (start && stop) hipExtLaunchKernelGGL(kernel, grid, dim3(512), lds, stream, start, stop, 0, b);
+    else MQ_LAUNCH(kernel, grid, dim3(512), lds, stream, b);
     return hipGetLastError();
 }
 
+// MT <= 2: the rows' tiles in LDS (in runs if need be), else from global memory a stage ahead; three and four tiles only
+// from LDS (read a stage ahead they do not fit the registers), an even number of stages per wavefront.
 template <int NMAT, int WPR, int MT>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
-    const bool odd = ((a.nb / WPR) & 1) != 0, ga = !skinny16_in_lds(NMAT, WPR, a.nb, MT);
-    if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT>(a, stream, start, stop);
-    return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT>(a, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT>(a, stream, start, stop);
+    const bool odd = ((a.nb / WPR) & 1) != 0;
+    const int ranges = odd ? (skinny16_lds_bytes(NMAT, WPR, a.nb, MT, 1) <= kSkinnyLdsMax ? 1 : 0) : skinny16_ranges(NMAT, WPR, a.nb, MT);
+    if constexpr (MT <= 2) {
+        const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
+        if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT>(a, 1, stream, start, stop);
+        return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT>(a, 1, stream, start, stop);
+    } else if constexpr (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8)) {
+        return hipErrorInvalidValue;  // (skinny16_applies: not built)
+    } else {
+        if (odd || ranges == 0) return hipErrorInvalidValue;
+        return launch_skinny16_one<NMAT, WPR, false, false, MT>(a, ranges, stream, start, stop);
+    }
 }
 
 template <int NMAT, int MT>
@@ -1288,27 +1335,38 @@ hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t strea
     return hipErrorInvalidValue;
 }
 
+template <int NMAT>
+hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+    switch ((int)((a.n + 15) / 16)) {
+        case 1: return launch_skinny16_wpr<NMAT, 1>(a, wpr, stream, start, stop);
+        case 2: return launch_skinny16_wpr<NMAT, 2>(a, wpr, stream, start, stop);
+        case 3: return launch_skinny16_wpr<NMAT, 3>(a, wpr, stream, start, stop);
+        case 4: return launch_skinny16_wpr<NMAT, 4>(a, wpr, stream, start, stop);
+    }
+    return hipErrorInvalidValue;
+}
+
 }  // namespace
 
-// Whether a Q4_K product of nine to thirty-two rows runs on skinny16_kernel: the wave split of the other decode
-// kernels must be one of its own (a divisor of eight that divides the super-blocks of a row).
-bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu) {
-    (void)swiglu;
+// Whether a Q4_K product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
+// one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
+// (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages, an even number of stages in all.
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
-    return wpr && nb % wpr == 0;
+    if (!wpr || nb % wpr || n < 1 || n > 64) return false;
+    if (n <= 32) return true;
+    if ((nb / wpr) & 1) return false;
+    if (swiglu && n > 48 && (wpr == 1 || wpr == 8)) return false;  // these two forms of the four-tile pair kernel spill registers
+    return skinny16_ranges(swiglu ? 2 : 1, wpr, nb, (int)((n + 15) / 16)) != 0;
 }
 
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
-    if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 32 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
+    if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 64 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
-    if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr)) return hipErrorInvalidValue;
+    if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr, a.n)) return hipErrorInvalidValue;
     const int wpr = dense_lds_wpr(a.nb, rowtiles);
-    if (a.n > 16) {
-        if (a.w1) return launch_skinny16_wpr<2, 2>(a, wpr, stream, start, stop);
-        return launch_skinny16_wpr<1, 2>(a, wpr, stream, start, stop);
-    }
-    if (a.w1) return launch_skinny16_wpr<2, 1>(a, wpr, stream, start, stop);
-    return launch_skinny16_wpr<1, 1>(a, wpr, stream, start, stop);
+    if (a.w1) return launch_skinny16_tiles<2>(a, wpr, stream, start, stop);
+    return launch_skinny16_tiles<1>(a, wpr, stream, start, stop);
 }
 
 }  // namespace mq

@@ -134,8 +134,8 @@ int mq_mul_mat_q4k_multi(const mq_weight* const* w, int count, const float* x_de
 int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, int64_t ldx, float* y_dev, int64_t ldy,
                            void* stream);
 /* The same product computed by the matrix-core GEMM kernel whatever n is (mq_mul_mat_q4k switches to it
- * by itself from 48 rows up, from 33 for Q4_K matrices of 24 MB and more -- up to 32 rows Q4_K products stay on the
- * decode arithmetic): weights are read once per 128 activation rows and the int8 MFMA
+ * by itself from 48 rows up, from 17 for matrices of 24 MB and more; Q4_K products stay on the decode arithmetic up to
+ * 32 rows, up to 64 where their rows pass through LDS in runs of super-blocks): weights are read once per 128 activation rows and the int8 MFMA
  * units do the arithmetic.  RunQ4KRawBatchedDenseGemm (core/src/backend/cpu_backend_q4k_dense.cpp:57-101),
  * the A.shape[0] >= 4 branch of MatMulGgmlQuantizedTransBWithPath
  * (core/src/backend/cpu_backend_quantized_matmul.cpp:164-170).  Same integers per super-block as

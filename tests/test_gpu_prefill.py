@@ -158,22 +158,30 @@ def test_gemm_integer_sums_are_exact_with_k_in_runs(ops):
 
 
 def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(ops):
-    """24 MB of weights and more: Q4_K rows up to 32 stay on the decode arithmetic (two tiles of sixteen per weight tile:
-    a row's result is the one it has when the rows are handed over sixteen at a time, bit for bit); from 33 rows
-    mul_mat hands them to the matrix-core GEMM (smaller matrices and the other weight types from 48)."""
+    """24 MB of weights and more: Q4_K rows up to 64 stay on the decode arithmetic (up to four tiles of sixteen per weight
+    tile: a row's result is the one it has when the rows are handed over sixteen at a time, bit for bit); from 65 rows
+    mul_mat hands them to the matrix-core GEMM (matrices whose rows do not pass through LDS that way from 33, smaller
+    matrices and the other weight types from 48)."""
     import torch
     W = ops.Q4KWeight.synthetic(4, 14336, 4096)
-    x = torch.randn((40, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(20))
-    assert torch.equal(ops.mul_mat(W, x[:20]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:20])]))
+    x = torch.randn((70, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(20))
+    pieces = lambda t: torch.cat([ops.mul_mat(W, t[i:i + 16]) for i in range(0, t.shape[0], 16)])
+    assert torch.equal(ops.mul_mat(W, x[:20]), pieces(x[:20]))
+    assert torch.equal(ops.mul_mat(W, x[:40]), pieces(x[:40]))
     big = ops.gemm(W, x)
     assert torch.equal(ops.mul_mat(W, x), big)
-    small = torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:32]), ops.mul_mat(W, x[32:])])
+    small = pieces(x)
     assert (big - small).abs().max().item() <= 1e-5 * small.abs().max().item()
     W.free()
+    W = ops.Q4KWeight.synthetic(7, 4096, 14336)   # 56 super-blocks, seven per wavefront: two tiles read from global memory, then the GEMM
+    x = torch.randn((40, 14336), device="cuda", generator=torch.Generator(device="cuda").manual_seed(23))
+    assert torch.equal(ops.mul_mat(W, x[:30]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:30])]))
+    assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
+    W.free()
     W = ops.Q4KWeight.synthetic(6, 4096, 4096, ggml_type=synth.GGML_TYPE_Q5_K)   # the other types: 16-row passes up to 47 rows
+    x = torch.randn((48, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(22))
     assert torch.equal(ops.mul_mat(W, x[:20]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:20])]))
-    x48 = torch.randn((48, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(22))
-    assert torch.equal(ops.mul_mat(W, x48), ops.gemm(W, x48))
+    assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
     W.free()
     W = ops.Q4KWeight.synthetic(5, 4096, 4096)
     x = torch.randn((20, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(21))
