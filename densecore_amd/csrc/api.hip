@@ -28,7 +28,7 @@ struct mq_weight {
 struct mq_acts {
     void* aq = nullptr;   // A-major codes
     void* ad = nullptr;   // A-major scales
-    void* ap = nullptr;   // handles of more than eight rows: the rows as one P-major tile per super-block as well (written for 9..16 rows)
+    void* ap = nullptr;   // handles of more than eight rows: the rows as P-major tiles of sixteen as well (written for 9..64 rows)
     int64_t max_rows = 0, cols = 0, nb = 0;
     int64_t n = 0;        // rows quantized by the last mq_acts_quantize
     bool tile16 = false;  // ap holds those rows (set by the quantizer that wrote both layouts, cleared by one that did not)
@@ -1491,7 +1491,7 @@ int mq_acts_create(int64_t max_rows, int64_t cols, mq_acts** out) {
     a->max_rows = max_rows, a->cols = cols, a->nb = cols / kQK;
     hipError_t e = hipMalloc(&a->aq, aq_bytes(max_rows, a->nb));
     if (e == hipSuccess) e = hipMalloc(&a->ad, ad_count(max_rows, a->nb) * sizeof(float));
-    if (e == hipSuccess && max_rows > 8) e = hipMalloc(&a->ap, pmajor_bytes(16, a->nb));
+    if (e == hipSuccess && max_rows > 8) e = hipMalloc(&a->ap, pmajor_bytes(max_rows < kSkinnyMaxRows ? max_rows : kSkinnyMaxRows, a->nb));
     if (e != hipSuccess) {
         if (a->aq) (void)hipFree(a->aq);
         if (a->ad) (void)hipFree(a->ad);
@@ -1520,8 +1520,8 @@ int mq_acts_quantize(mq_acts* a, const float* x_dev, int64_t n, int64_t ldx, voi
     a->tile16 = false;
     if (n == 0) return MQ_OK;
     MQ_HIP(launch_quantize_q8k(x_dev, n, ldx, a->cols, nullptr, 0, (uint8_t*)a->aq, (float*)a->ad, (hipStream_t)stream));
-    // nine to sixteen rows: their tile of sixteen as well, for the Q4_K products that take it (skinny16_takes)
-    a->tile16 = n > 8 && n <= 16 && a->ap;
+    // nine to 64 rows: their tiles of sixteen as well, for the Q4_K products that take them (skinny16_takes)
+    a->tile16 = n > 8 && n <= kSkinnyMaxRows && a->ap;
     if (a->tile16) MQ_HIP(launch_quantize_q8k_pmajor(x_dev, n, ldx, a->cols, (uint8_t*)a->ap, (hipStream_t)stream));
     return MQ_OK;
 }

@@ -303,3 +303,17 @@ def test_three_tiles_against_the_oracle(env):
     for name, ref in oracle_all_orders(w_pick, cols, q8).items():
         assert_fp32_parity(y[:, pick], ref, mag, f"order={name}")
     W.free()
+
+
+def test_shared_activation_handle_up_to_64_rows(env):
+    torch, _lib, ops = env
+    rows, cols = 6144, 4096
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("s64-hw"), rows, cols)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("s64-hu"), rows, cols)
+    acts = ops.Q8KActs(64, cols)
+    for n in (64, 20, 40, 5):      # every later batch reuses the handle
+        x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s64-hx", n), (n, cols))).cuda()
+        acts.quantize(x)
+        assert torch.equal(acts.mul_mat(W), ops.mul_mat(W, x)), f"n={n}"
+        assert torch.equal(acts.swiglu_mul_mat(W, U, 1), ops.swiglu_mul_mat(W, U, x, 1)), f"n={n}"
+    acts.free(), W.free(), U.free()
