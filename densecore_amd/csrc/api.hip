@@ -177,7 +177,8 @@ int g_dense_lds = 1;
 int g_moe_item_tiles = 0;  // 0: chosen per launch (moe_gemm_item_tiles); 2, 4 or 8: forced (mq_debug_set_dense_lds bits 8..11)
 int g_gemm_pair = 1;  // prefill widths: Q4_K gate and up in ONE GEMM launch that stores silu(gate) * up (mq_debug_set_dense_lds bit 3 turns it off)
 // Widest product whose fp32 rows the LDS-staged kernel quantizes itself (no quantizer launch).
-int64_t g_dense_xf_rows = 2;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
+constexpr int64_t kDenseXfRowsDefault = 2;
+int64_t g_dense_xf_rows = kDenseXfRowsDefault;  // measured on the 4096 -> 14336 gate/up pair: two rows 15.4 against 16.5 us with the quantizer launch, four rows 16.9 against 16.4
 
 bool dense_lds_takes(const MatmulArgs& a) {
     return g_dense_lds && !a.grouped && !a.dbg_dot && !a.out_aq && a.n >= 1 && a.n <= 16 &&
@@ -2056,7 +2057,7 @@ int mq_debug_set_dense_lds(int on) {
     g_moe_item_tiles = (on >> 8) & 0xf;      // bits 8..11: activation tiles per item of the expert-grouped GEMM (2, 4 or 8), 0 = by the rows per expert  // bit 3: gate and up as two GEMM launches and a SwiGLU pass instead of the pair form
     set_grouped_lds((on & 1) && !(on & 4));  // bit 2: only the expert-grouped launches go back to matmul_kernel
     g_skinny16 = (on & 0x1000) ? 0 : 1;      // bit 12: nine to 64 rows stay on the kernels with token tiles of eight (or the GEMM)
-    if (on >> 4) g_dense_xf_rows = ((on >> 4) & 0xf) - 1;  // experiments: widest product that quantizes its rows itself, plus one
+    g_dense_xf_rows = ((on >> 4) & 0xf) ? ((on >> 4) & 0xf) - 1 : kDenseXfRowsDefault;  // bits 4..7, experiments: widest product that quantizes its rows itself, plus one (0: the default)
     return before;
 }
 

@@ -61,8 +61,8 @@ int mq_census_read(int kind, double* avg_us, double* min_us, double* max_us, int
  * both on the kernel that reads its operand from global memory at every stage, on = 5 only the expert-grouped
  * ones; bit 3 (on = 9) makes Q4_K gate and up at prefill widths two GEMM launches and a SwiGLU pass instead of the
  * one launch that stores silu(gate) * up; bits 8..11 force the activation tiles per item of the expert-grouped GEMM (2,
- * 4 or 8; 0 = chosen by the rows per expert); bit 12 keeps dense Q4_K products of nine to sixteen rows on the kernels
- * that multiply them as two token tiles of eight instead of the one that takes them as one tile of sixteen.  All
+ * 4 or 8; 0 = chosen by the rows per expert); bit 12 keeps dense Q4_K products of nine to 64 rows on the kernels
+ * that multiply them as token tiles of eight (or on the GEMM) instead of the one that takes them as tiles of sixteen.  All
  * return the same bits (tests/test_gpu_dense_lds.py, tests/test_gpu_grouped_lds.py, tests/test_gpu_prefill.py); returns the
  * previous setting of bit 0.  No counterpart in the reference. */
 int mq_debug_set_dense_lds(int on);
