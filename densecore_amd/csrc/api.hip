@@ -572,13 +572,15 @@ static int matmul_from_ws(const mq_weight* w, int64_t n, float* y, int64_t ldy, 
 // 17 for matrices of 24 MB and more (14336 x 4096 and 4096 x 14336: 19 against 24 us at 17 rows, 21 against 35-38 us
 // at 47; 4096 x 4096: 17.4 against 14.1 us at 17 rows, 17.9 against 14.6 at 47).  Q4_K products of up to 32 rows go to
 // skinny16_kernel ahead of both (skinny16_takes: gate/up of a 4096 -> 14336 FFN 41 -> 22 us at 17 to 32 rows,
-// 4096 x 4096 11.5 -> 9.5 us).
+// 4096 x 4096 11.5 -> 9.5 us).  The 17-row rule holds for Q5_K and Q6_K matrices of that many weights as well (4096 x
+// 14336: Q5_K 28.7 / 30.7 / 42.5 us in 16-row passes against 22.3 / 22.6 / 25.3 on the GEMM at 17 / 32 / 47 rows, Q6_K 30.7 /
+// 33.2 / 46.3 against 28.2 / 28.5 / 32.3; 4096 x 4096 stays: 12.1 against 14.1 us at 17 rows, 16.8 against 15.9 at 47).
 constexpr int64_t kPrefillMinRows = 48;
 constexpr int64_t kPrefillMinRowsLarge = 17;
 constexpr int64_t kPrefillLargeBytes = 24ll << 20;
 static bool prefill_applies(const mq_weight* w, int64_t n) {
     if (w->type != kTypeQ4K && w->type != kTypeQ5K && w->type != kTypeQ6K) return false;
-    return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->type == kTypeQ4K && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
+    return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
 }
 constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
 // Widest product that also runs the residual add and the RMSNorm inside the GEMV kernel: every workgroup repeats the
