@@ -583,6 +583,12 @@ static bool prefill_applies(const mq_weight* w, int64_t n) {
     return n >= kPrefillMinRows || (n >= kPrefillMinRowsLarge && w->rows * w->nb * (int64_t)kQ4Block >= kPrefillLargeBytes);
 }
 constexpr int64_t kGemvFusedMaxRows = 4;  // widest product whose quantizer runs inside the GEMV kernel (measured: 8 loses)
+// At three and four rows the quantizer inside pays only for a small matrix with short rows: 2048x2048 and 2560x2048 take
+// 5.3 / 5.6 us against 5.8 for a quantizer launch and the LDS-staged product; 1024x4096 6.6 / 7.3 against 6.6,
+// 4096x4096 7.5 / 8.3 against 7.2, 8192x2048 7.5 / 8.2 against 7.0.
+static bool gemvn_fused_pays(const mq_weight* w, int64_t n) {
+    return n <= 2 || (w->nb <= 8 && w->rowtiles * w->nb <= 1536);
+}
 // Widest product that also runs the residual add and the RMSNorm inside the GEMV kernel: every workgroup repeats the
 // rows' norm, about 1.25 us per row.  Decoder layer (2048 hidden, 64 experts) with the norm inside / as a launch of
 // its own that emits Q8_K for the LDS-staged product: 36.0 / 36.2 us at two rows, 43.9 / 42.4 at three, 48.6 / 45.7 at four.
@@ -699,7 +705,7 @@ int mq_mul_mat_q4k(const mq_weight* w, const float* x_dev, int64_t n, int64_t ld
             return MQ_OK;
         }
     }
-    if (n <= kGemvFusedMaxRows && w->type == kTypeQ4K) {  // a few rows, short K per wave: the same with the rows' codes going through LDS
+    if (n <= kGemvFusedMaxRows && w->type == kTypeQ4K && gemvn_fused_pays(w, n)) {  // a few rows, short K per wave: the same with the rows' codes going through LDS
         const int waves = pick_waves(w->nb, w->rowtiles);
         if (gemv1_fused_applies(w->nb, waves)) {
             MQ_HIP(launch_gemvn_fused(w->data, w->rows, w->nb, x_dev, ldx, nullptr, nullptr, 0.0f, nullptr, y_dev, ldy, (int)n, false, waves, s));

@@ -1319,7 +1319,8 @@ hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEv
     } else if constexpr (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8)) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
-        if (odd || ranges == 0) return hipErrorInvalidValue;
+        if (ranges == 0) return hipErrorInvalidValue;
+        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
         return launch_skinny16_one<NMAT, WPR, false, false, MT>(a, ranges, stream, start, stop);
     }
 }
@@ -1350,14 +1351,16 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 
 // Whether a Q4_K product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
-// (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages, an even number of stages in all.
+// (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages (in one run where a
+// wavefront's stage count is odd).
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64) return false;
     if (n <= 32) return true;
-    if ((nb / wpr) & 1) return false;
     if (swiglu && n > 48 && (wpr == 1 || wpr == 8)) return false;  // these two forms of the four-tile pair kernel spill registers
-    return skinny16_ranges(swiglu ? 2 : 1, wpr, nb, (int)((n + 15) / 16)) != 0;
+    const int nmat = swiglu ? 2 : 1, mt = (int)((n + 15) / 16);
+    if ((nb / wpr) & 1) return skinny16_lds_bytes(nmat, wpr, nb, mt, 1) <= kSkinnyLdsMax;  // an odd stage count: the tiles in one run
+    return skinny16_ranges(nmat, wpr, nb, mt) != 0;
 }
 
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {

@@ -229,15 +229,16 @@ def _sixteen_at_a_time(fn, t):
 
 
 # wavefronts per row tile 2 (two runs of super-blocks), 4 (two runs), 1 (one run), 4 (one run), 8 (two runs of one stage
-# each), and a shape with a single stage per wavefront (falls back to the 16-row passes or the GEMM)
-WIDE = [(14336, 4096), (6144, 4096), (20480, 1024), (8192, 2048), (4096, 4096), (2048, 2048)]
+# each), a single stage per wavefront whose tiles fit LDS in one run (twice), and three stages per wavefront whose tiles
+# do not (falls back to the 16-row passes or the GEMM)
+WIDE = [(14336, 4096), (6144, 4096), (20480, 1024), (8192, 2048), (4096, 4096), (2048, 2048), (2560, 2048), (2048, 6144)]
 
 
 @pytest.mark.parametrize("rows,cols", WIDE)
 def test_three_and_four_tiles_equal_the_rows_taken_sixteen_at_a_time(env, rows, cols):
     torch, _lib, ops = env
     W = ops.Q4KWeight.synthetic(synth.tensor_seed("s64", rows, cols), rows, cols)
-    takes = (rows, cols) != (2048, 2048)
+    takes = (rows, cols) != (2048, 6144)
     for n in (33, 40, 48, 64):
         x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s64-x", rows, cols, n), (n, cols))).cuda()
         whole, split = ops.mul_mat(W, x), _sixteen_at_a_time(lambda t: ops.mul_mat(W, t), x)
@@ -248,7 +249,7 @@ def test_three_and_four_tiles_equal_the_rows_taken_sixteen_at_a_time(env, rows, 
     W.free()
 
 
-@pytest.mark.parametrize("rows,cols", [(14336, 4096), (8192, 2048)])
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (8192, 2048), (2048, 2048)])
 @pytest.mark.parametrize("n", [40, 64])
 def test_three_and_four_tiles_gate_up(env, rows, cols, n):
     torch, _lib, ops = env
