@@ -256,9 +256,14 @@ def test_three_and_four_tiles_gate_up(env, rows, cols, n):
     G = ops.Q4KWeight.synthetic(synth.tensor_seed("s64-g", rows, cols), rows, cols)
     U = ops.Q4KWeight.synthetic(synth.tensor_seed("s64-u", rows, cols), rows, cols)
     x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s64-gx", rows, cols, n), (n, cols))).cuda()
+    gemm = (rows, cols, n) == (2048, 2048, 64)   # (four tiles of a pair with eight wavefronts per row tile are not built: the GEMM)
     for silu in (0, 1):
         fn = lambda t: ops.swiglu_mul_mat(G, U, t, silu)
-        assert torch.equal(fn(x), _sixteen_at_a_time(fn, x)), f"silu={silu}"
+        whole, split = fn(x), _sixteen_at_a_time(fn, x)
+        if gemm:
+            assert (whole - split).abs().max().item() <= 1e-5 * split.abs().max().item(), f"silu={silu}"
+        else:
+            assert torch.equal(whole, split), f"silu={silu}"
     G.free(), U.free()
 
 
