@@ -633,6 +633,10 @@ static int ffn_wide_locked(const mq_weight* gate, const mq_weight* up, const mq_
     float* part = part_bytes ? (float*)g.kpart.ptr : nullptr;
     MQ_HIP(launch_prefill_gemm(gate->data, gate->type, inter, gate->nb, (const uint8_t*)g.ap.ptr, n, gbuf, inter, part, s));
     MQ_HIP(launch_prefill_gemm(up->data, up->type, inter, up->nb, (const uint8_t*)g.ap.ptr, n, ubuf, inter, part, s));
+    if (!down && inter % kQK) {  // SwiGLU rows that do not divide into super-blocks: nothing to quantize them for
+        MQ_HIP(launch_silu_mul(gbuf, ubuf, n, inter, inter, inter, h_dev, ldh, silu_mode, s));
+        return MQ_OK;
+    }
     if (!down) {  // SwiGLU rows only: the quantizer's fp32 side output is the result
         MQ_HIP(g.ap2.reserve(pmajor_bytes(n, inter / kQK)));
         MQ_HIP(launch_swiglu_quantize_q8k_pmajor(gbuf, ubuf, n, inter, inter, silu_mode, h_dev, ldh, (uint8_t*)g.ap2.ptr, s));
