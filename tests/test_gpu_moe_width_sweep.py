@@ -65,3 +65,52 @@ def test_token_i_of_the_moe_layer_depends_on_token_i_alone(E, H, I, K, shared, g
         assert err.max().item() <= 5e-4 and (err > 2e-5).sum().item() <= max(2, n // 50), f"n={n}"
     for w in (ge, ue, de) + (tuple(sh[:3]) if sh else ()):
         w.free()
+
+
+@pytest.mark.parametrize("E,H,I,K,wtype", [(40, 1024, 512, 4, 12), (7, 512, 256, 3, 12), (40, 1024, 512, 4, 13), (24, 512, 512, 8, 14)])
+def test_expert_nodes_with_given_ids_at_every_width(E, H, I, K, wtype):
+    """mul_mat_id, the gate/up node and the down node with ids handed in -- some outside [0, E) (zero rows, skipped
+    terms), some repeated within a token -- at 1..72 tokens and at prefill widths: (token, slot) rows depend on their
+    own token alone (to rounding: the launches of different widths split a row's super-blocks over wavefronts
+    differently)."""
+    import torch
+    from densecore_amd import ops
+    tag = ("mwi", E, H, I, K, wtype)
+    ge = ops.Q4KWeight.synthetic(synth.tensor_seed(*tag, "g"), I, H, E, ggml_type=wtype)
+    ue = ops.Q4KWeight.synthetic(synth.tensor_seed(*tag, "u"), I, H, E, ggml_type=wtype)
+    de = ops.Q4KWeight.synthetic(synth.tensor_seed(*tag, "d"), H, I, E, ggml_type=wtype)
+    N = 520
+    rng = np.random.default_rng(synth.tensor_seed(*tag, "ids") % (1 << 32))
+    ids_h = rng.integers(0, E, size=(N, K)).astype(np.int32)
+    ids_h[rng.random((N, K)) < 0.06] = -1
+    ids_h[rng.random((N, K)) < 0.03] = E + 3
+    ids_h[5, :] = ids_h[5, 0]           # one expert in every slot of a token
+    ids_h[9, :] = -1                    # a token with no valid slot
+    ids = torch.from_numpy(ids_h).cuda()
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed(*tag, "x"), (N, H))).cuda()
+    hid = torch.from_numpy(synth.normal_f32(synth.tensor_seed(*tag, "h"), (N, K, I))).cuda()
+    wts = torch.from_numpy(np.abs(synth.normal_f32(synth.tensor_seed(*tag, "w"), (N, K)))).cuda()
+    fns = {
+        "mul_mat_id": lambda a, b: ops.mul_mat_id(ge, x[a:b], ids[a:b]),
+        "mul_mat_id per slot": lambda a, b: ops.mul_mat_id(de, hid[a:b], ids[a:b]),
+        "gate/up node": lambda a, b: ops.moe_gateup_swiglu(ge, ue, x[a:b], ids[a:b], ops.SILU_FAST),
+        "down node": lambda a, b: ops.moe_down_weighted(de, hid[a:b], ids[a:b], wts[a:b]),
+    }
+    invalid = torch.from_numpy((ids_h < 0) | (ids_h >= E)).cuda()
+    for name, fn in fns.items():
+        one = torch.cat([fn(i, i + 1) for i in range(72)], dim=0)
+        if one.dim() == 3:
+            assert (one[invalid[:72]] == 0).all(), f"{name}: rows of invalid ids are zero"
+        scale = one.abs().max().item()
+        for n in range(1, 73):
+            y = fn(0, n)
+            assert (y - one[:n]).abs().max().item() <= 2e-6 * scale, f"{name} n={n}"
+            if y.dim() == 3:
+                assert (y[invalid[:n]] == 0).all(), f"{name} n={n}: rows of invalid ids are zero"
+        for n in (200, 333, N):
+            whole = fn(0, n)
+            parts = torch.cat([fn(a, min(a + 40, n)) for a in range(0, n, 40)], dim=0)
+            assert (whole - parts).abs().max().item() <= 2e-6 * parts.abs().max().item(), f"{name} n={n}"
+            if whole.dim() == 3:
+                assert (whole[invalid[:n]] == 0).all(), f"{name} n={n}: rows of invalid ids are zero"
+    ge.free(), ue.free(), de.free()
