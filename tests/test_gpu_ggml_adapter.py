@@ -202,3 +202,30 @@ def test_library_level_matmul(ga):
     # a type other than Q4_K, Q5_K, Q6_K and Q8_0 is rejected like an unsupported ggml type
     assert ga.lib().mq_matmul_ggml_quantized_transb(a.ctypes.data, m, cols, cols, w.ctypes.data, 2, rows, cols,
                                                     144 * (cols // 256), c.ctypes.data, rows) == 0
+
+
+@pytest.mark.parametrize("rows,cols", [(1000, 1024), (2048, 2048)])
+def test_dense_node_at_every_width_equals_the_device_entry_point(ga, rows, cols):
+    """The batched callback on host tensors with strided rows (NaN in the gaps of src, a sentinel in those of dst) at
+    1..40 rows and three wider ones: the bits of mq_mul_mat_q4k on the same rows, nothing written outside them."""
+    import torch
+    from densecore_amd import ops
+    w = synth.q4k_matrix(synth.tensor_seed("ga-w", rows, cols), rows, cols)
+    W = ops.Q4KWeight.from_ggml(w, cols)
+    tw = ga.tensor(w, ga.GGML_TYPE_Q4_K, [cols, rows], name=b"blk.1.attn_output.weight")
+    xs = synth.normal_f32(synth.tensor_seed("ga-x", rows, cols), (130, cols))
+    for m in list(range(1, 41)) + [49, 70, 130]:
+        pad = 32 if m % 2 else 0
+        xbuf = np.full((m, cols + pad), np.nan, np.float32)
+        xbuf[:, :cols] = xs[:m]
+        ybuf = np.full((m + 1, rows + pad), 7.0, np.float32)
+        tx = ga.tensor(xbuf, ga.GGML_TYPE_F32, [cols, m], nb=[4, 4 * (cols + pad)])
+        ty = ga.tensor(ybuf, ga.GGML_TYPE_F32, [rows, m], nb=[4, 4 * (rows + pad)])
+        ga.set_src(ty, tx, tw)
+        fn = ga.lib().mq_cb_gemv_custom if m == 1 else ga.lib().mq_cb_gemv_batched_custom
+        fn(C.byref(ty), 0, 1, None)
+        assert ga.lib().mq_ggml_last_status() == 0, f"m={m}"
+        want = ops.mul_mat(W, torch.from_numpy(np.ascontiguousarray(xs[:m])).cuda()).cpu().numpy()
+        assert np.array_equal(ybuf[:m, :rows].view(np.uint32), want.view(np.uint32)), f"m={m}"
+        assert np.all(ybuf[:m, rows:] == 7.0) and np.all(ybuf[m] == 7.0), f"m={m}: written outside the rows"
+    W.free()
