@@ -89,3 +89,29 @@ def test_wide_gate_up_and_product_on_row_counts_that_are_no_multiple_of_a_super_
             split = torch.cat([fn(x[i:i + 16]) for i in range(0, n, 16)], dim=0)
             assert (whole - split).abs().max().item() <= 2e-5 * split.abs().max().item(), f"n={n}"
     G.free(), U.free()
+
+
+@pytest.mark.parametrize("hidden,inter,gu_type,down_type", [(1024, 3072, 12, 13), (1024, 3072, 12, 14), (2048, 512, 13, 13),
+                                                           (2048, 512, 14, 14), (4096, 14336, 12, 14)])
+def test_ffn_with_sibling_types_equals_its_two_nodes_at_every_width(hidden, inter, gu_type, down_type):
+    """mq_ffn_swiglu_q4k against the gate/up entry point followed by the down product, as a graph that keeps the three
+    nodes apart would run them: bit for bit up to sixteen rows (every kernel there shares one arithmetic and the
+    quantizers one block routine); beyond, the fused entry point may take other launches (the matrix-core GEMM, the
+    SwiGLU product formed in its quantizer), whose last-bit differences in a hidden row can move a code of the down
+    product's quantizer in a few rows."""
+    import torch
+    from densecore_amd import ops
+    G = ops.Q4KWeight.synthetic(synth.tensor_seed("fs-g", hidden, inter, gu_type), inter, hidden, ggml_type=gu_type)
+    U = ops.Q4KWeight.synthetic(synth.tensor_seed("fs-u", hidden, inter, gu_type), inter, hidden, ggml_type=gu_type)
+    D = ops.Q4KWeight.synthetic(synth.tensor_seed("fs-d", hidden, inter, down_type), hidden, inter, ggml_type=down_type)
+    xs = torch.from_numpy(synth.normal_f32(synth.tensor_seed("fs-x", hidden, inter), (300, hidden))).cuda()
+    for n in list(range(1, 73)) + [130, 300]:
+        x = xs[:n]
+        y = ops.ffn_swiglu(G, U, D, x, ops.SILU_FAST_FMA)
+        want = ops.mul_mat(D, ops.swiglu_mul_mat(G, U, x, ops.SILU_FAST_FMA))
+        if n <= 16:
+            assert torch.equal(y, want), f"n={n}"
+        else:
+            err = (y - want).abs().max(dim=1).values / want.abs().max().item()
+            assert err.max().item() <= 5e-4 and (err > 2e-5).sum().item() <= max(2, n // 40), f"n={n}: {err.max().item()}"
+    G.free(), U.free(), D.free()
