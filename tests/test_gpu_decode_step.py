@@ -40,7 +40,7 @@ def small_cfg(ds, n_layers):
     return ds.StepConfig(n_layers=n_layers, hidden=512, n_experts=16, inter=256, top_k=4, n_q=512, n_kv=128, seed=7)
 
 
-@pytest.mark.parametrize("n", [1, 4, 8])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 24, 33, 50, 70])
 def test_single_layer_stagewise(ds, n):
     import torch
     cfg = small_cfg(ds, 1)
@@ -50,9 +50,10 @@ def test_single_layer_stagewise(ds, n):
     r = ref_step.layer_forward(host_weights(step.layers[0]), x.cpu().numpy(), None, cfg, step.silu_mode())
     close(step.qkv.cpu().numpy(), r["qkv"], STAGE_REL, "qkv")
     close(step.o.cpu().numpy(), r["o"], STAGE_REL, "wo")
-    close(step.logits.cpu().numpy(), r["logits"], 1e-5, "router logits")
+    # (the router reads the residual stream behind wo: at many rows one of them has a flipped code upstream)
+    close(step.logits.cpu().numpy(), r["logits"], 1e-5 if n <= 8 else STAGE_REL, "router logits")
     assert np.array_equal(step.ids[0].cpu().numpy(), r["ids"])
-    close(step.wts[0].cpu().numpy(), r["weights"], 1e-5, "routing weights")
+    close(step.wts[0].cpu().numpy(), r["weights"], 1e-5 if n <= 8 else STAGE_REL, "routing weights")
     close(step.y.cpu().numpy(), r["y"], 2e-3, "moe layer")
     close(out, r["x"] + r["y"], 2e-3, "layer output")
     step.free()
