@@ -197,12 +197,12 @@ bool dense_lds_quantizes(const mq_weight* w, const float* x, int64_t n, int64_t 
 int g_skinny16 = 1;
 constexpr int64_t kSkinnyMaxRows = 64;
 bool skinny16_takes(const mq_weight* w, int64_t n, bool swiglu) {
-    return g_skinny16 && g_dense_lds && n > 8 && n <= kSkinnyMaxRows && w->type == kTypeQ4K && skinny16_applies(w->nb, w->rowtiles, swiglu, n);
+    return g_skinny16 && g_dense_lds && n > 8 && n <= kSkinnyMaxRows && skinny16_applies(w->nb, w->rowtiles, swiglu, n, w->type);
 }
 
 hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
     if (a.ap) {  // callers ask skinny16_takes first
-        if (a.grouped || a.dbg_dot || a.out_aq || a.wtype != kTypeQ4K) return hipErrorInvalidValue;
+        if (a.grouped || a.dbg_dot || a.out_aq) return hipErrorInvalidValue;
         Skinny16Args k;
         k.w0 = a.w0;
         k.w1 = a.swiglu ? a.w1 : nullptr;
@@ -213,6 +213,7 @@ hipError_t dense_launch(const MatmulArgs& a, hipStream_t s, hipEvent_t start = n
         k.y = a.y;
         k.ldy = a.ldy;
         k.silu_mode = a.silu_mode;
+        k.wtype = a.wtype;
         return launch_skinny16(k, s, start, stop);
     }
     if (!dense_lds_takes(a)) {

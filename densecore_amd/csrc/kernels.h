@@ -133,9 +133,10 @@ struct Skinny16Args {
     float* y = nullptr;
     int64_t ldy = 0;
     int silu_mode = 0;
+    int wtype = kTypeQ4K;          // kTypeQ4K or kTypeQ5K (one and two tiles)
     int ranges = 1;                // set by the launcher: runs of super-blocks the tiles pass through LDS in
 };
-bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n);
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype = kTypeQ4K);
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
 // ---- q8_0.hip --------------------------------------------------------------------------------

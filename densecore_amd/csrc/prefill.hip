@@ -547,9 +547,11 @@ struct ATile16 {
 // MT: activation tiles of sixteen rows (one, or two for 17 to 32 rows: the weight tile is expanded once for both, 18
 // MFMAs and ~156 vector instructions against the 32 + 294 of two passes over two token tiles of eight each).  With two
 // tiles the partial sums share LDS with the activation tiles (one more barrier before they are written).
-template <int NMAT, int WPR, bool ODD, bool GA, int MT>
+template <int NMAT, int WPR, bool ODD, bool GA, int MT, bool Q5 = false>
 __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     constexpr int RPW = 8 / WPR;  // row tiles per workgroup
+    constexpr int kStride = Q5 ? kTile5Bytes : kTileBytes;
+    constexpr int kTileLoads = Q5 ? 4 : 3;  // requests of a weight tile (load_tile)
     constexpr bool kRedShares = MT > 1 && !GA;  // the partial sums reuse the activation tiles' LDS
     extern __shared__ __align__(16) uint8_t lds16[];
     const int lane = threadIdx.x & 63;
@@ -564,8 +566,8 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     float* red = reinterpret_cast<float*>(lds16 + ((GA || kRedShares) ? (size_t)0 : (size_t)nb * MT * kPTileBytes));  // (one run when the sums lie behind the tiles)
 
     const uint8_t* tiles[NMAT];
-    tiles[0] = p.w0 + tile_offset(rt, 0, nb, kTileBytes);
-    if (NMAT == 2) tiles[1] = p.w1 + tile_offset(rt, 0, nb, kTileBytes);
+    tiles[0] = p.w0 + tile_offset(rt, 0, nb, kStride);
+    if (NMAT == 2) tiles[1] = p.w1 + tile_offset(rt, 0, nb, kStride);
     const int cnt = nb / WPR;  // stages of this wavefront: super-blocks h, h + WPR, ...
 
     // lane (r, kq): weight row r of the tile, activation rows 4 kq .. 4 kq + 3 of every activation tile
@@ -607,7 +609,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             for (int t = 0; t < MT; ++t) read_a(ring_a[st][t], p.ap + ((size_t)b * MT + t) * kPTileBytes);
         }
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m) load_tile<false>(ring_t[st][m], tiles[m] + (size_t)b * kTileBytes, lane);
+        for (int m = 0; m < NMAT; ++m) load_tile<Q5>(ring_t[st][m], tiles[m] + (size_t)b * kStride, lane);
     };
 
     float acc[NMAT][MT][4];
@@ -630,7 +632,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             // one's copies in registers (they would not fit)
             if (MT > 2 && m > 0) asm volatile("" ::: "memory");
             WTile wt;
-            expand_tile<false>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, v2u{0u, 0u}, kq, wt);
+            expand_tile<Q5>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, Q5 ? ring_t[st][m].qh : v2u{0u, 0u}, kq, wt);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 ATile16 from_lds;
@@ -639,15 +641,19 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
                 const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
                 v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.hi[0], zero, 0, 0, 0);
                 v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.lo[0], zero, 0, 0, 0);
+                v4i fb = zero;  // Q5_K: the fifth code bits times the whole scale
+                if constexpr (Q5) fb = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[0], wt.b5[0], zero, 0, 0, 0);
                 const v4f mn = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.dg, wt.mins, zero_f, 0, 0, 0);
 #pragma unroll
                 for (int j = 1; j < 4; ++j) {
                     hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[j], wt.hi[j], hi, 0, 0, 0);
                     lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[j], wt.lo[j], lo, 0, 0, 0);
+                    if constexpr (Q5) fb = __builtin_amdgcn_mfma_i32_16x16x64_i8(at.a[j], wt.b5[j], fb, 0, 0, 0);
                 }
 #pragma unroll
                 for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile's update (decode_tile.h); mn[i2] is the integer min_dot, exactly
-                    const int dot = hi[i2] * 8 + lo[i2];
+                    int dot = hi[i2] * 8 + lo[i2];
+                    if constexpr (Q5) dot += fb[i2] * 16;
                     const float d = __fmul_rn(wt.d, ydv[i2]);
                     const float dm = __fmul_rn(wt.dmin, ydv[i2]);
                     const float term = __fsub_rn(__fmul_rn(d, (float)dot), __fmul_rn(dm, mn[i2]));
@@ -671,8 +677,8 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     }
     if constexpr (!GA) {
         // the LDS-direct copies are older than the tile requests: they have landed once at most those are outstanding
-        if (single) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NMAT * 3) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NMAT * 3) : "memory");
+        if (single) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NMAT * kTileLoads) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NMAT * kTileLoads) : "memory");
         __builtin_amdgcn_s_barrier();  // no fence: a fence would wait for the outstanding weight tiles as well
         asm volatile("" ::: "memory");
     }
@@ -1286,11 +1292,11 @@ int skinny16_ranges(int nmat, int wpr, int64_t nb, int mt) {
     return 0;
 }
 
-template <int NMAT, int WPR, bool ODD, bool GA, int MT>
+template <int NMAT, int WPR, bool ODD, bool GA, int MT, bool Q5>
 hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int64_t rowtiles = (a.rows + 15) / 16;
     const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT, ranges);
-    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT>;
+    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT, Q5>;
     static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
@@ -1308,54 +1314,70 @@ hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t st
 
 // MT <= 2: the rows' tiles in LDS (in runs if need be), else from global memory a stage ahead; three and four tiles only
 // from LDS (read a stage ahead they do not fit the registers), an even number of stages per wavefront.
-template <int NMAT, int WPR, int MT>
+template <int NMAT, int WPR, int MT, bool Q5>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const bool odd = ((a.nb / WPR) & 1) != 0;
     const int ranges = odd ? (skinny16_lds_bytes(NMAT, WPR, a.nb, MT, 1) <= kSkinnyLdsMax ? 1 : 0) : skinny16_ranges(NMAT, WPR, a.nb, MT);
     if constexpr (MT <= 2) {
         const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
-        if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT>(a, 1, stream, start, stop);
-        return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT>(a, 1, stream, start, stop);
-    } else if constexpr (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8)) {
+        if constexpr (Q5 && NMAT == 2 && MT == 2) {  // (read a stage ahead, two tiles of a Q5_K pair spill registers: skinny16_applies)
+            if (ga) return hipErrorInvalidValue;
+            if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, Q5>(a, 1, stream, start, stop);
+            return launch_skinny16_one<NMAT, WPR, false, false, MT, Q5>(a, 1, stream, start, stop);
+        } else {
+            if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, Q5>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, Q5>(a, 1, stream, start, stop);
+            return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, Q5>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, Q5>(a, 1, stream, start, stop);
+        }
+    } else if constexpr (Q5 || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
-        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
-        return launch_skinny16_one<NMAT, WPR, false, false, MT>(a, ranges, stream, start, stop);
+        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, false>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
+        return launch_skinny16_one<NMAT, WPR, false, false, MT, false>(a, ranges, stream, start, stop);
     }
 }
 
-template <int NMAT, int MT>
+template <int NMAT, int MT, bool Q5>
 hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     switch (wpr) {
-        case 1: return launch_skinny16_form<NMAT, 1, MT>(a, stream, start, stop);
-        case 2: return launch_skinny16_form<NMAT, 2, MT>(a, stream, start, stop);
-        case 4: return launch_skinny16_form<NMAT, 4, MT>(a, stream, start, stop);
-        case 8: return launch_skinny16_form<NMAT, 8, MT>(a, stream, start, stop);
+        case 1: return launch_skinny16_form<NMAT, 1, MT, Q5>(a, stream, start, stop);
+        case 2: return launch_skinny16_form<NMAT, 2, MT, Q5>(a, stream, start, stop);
+        case 4: return launch_skinny16_form<NMAT, 4, MT, Q5>(a, stream, start, stop);
+        case 8: return launch_skinny16_form<NMAT, 8, MT, Q5>(a, stream, start, stop);
     }
     return hipErrorInvalidValue;
 }
 
 template <int NMAT>
 hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
-    switch ((int)((a.n + 15) / 16)) {
-        case 1: return launch_skinny16_wpr<NMAT, 1>(a, wpr, stream, start, stop);
-        case 2: return launch_skinny16_wpr<NMAT, 2>(a, wpr, stream, start, stop);
-        case 3: return launch_skinny16_wpr<NMAT, 3>(a, wpr, stream, start, stop);
-        case 4: return launch_skinny16_wpr<NMAT, 4>(a, wpr, stream, start, stop);
+    const int mt = (int)((a.n + 15) / 16);
+    if (a.wtype == kTypeQ5K) {  // one and two tiles (the third chain's operands leave no registers for more)
+        if (mt == 1) return launch_skinny16_wpr<NMAT, 1, true>(a, wpr, stream, start, stop);
+        if (mt == 2) return launch_skinny16_wpr<NMAT, 2, true>(a, wpr, stream, start, stop);
+        return hipErrorInvalidValue;
+    }
+    switch (mt) {
+        case 1: return launch_skinny16_wpr<NMAT, 1, false>(a, wpr, stream, start, stop);
+        case 2: return launch_skinny16_wpr<NMAT, 2, false>(a, wpr, stream, start, stop);
+        case 3: return launch_skinny16_wpr<NMAT, 3, false>(a, wpr, stream, start, stop);
+        case 4: return launch_skinny16_wpr<NMAT, 4, false>(a, wpr, stream, start, stop);
     }
     return hipErrorInvalidValue;
 }
 
 }  // namespace
 
-// Whether a Q4_K product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
+// Whether a Q4_K product of n rows (nine to 64; Q5_K: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
 // (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages (in one run where a
 // wavefront's stage count is odd).
-bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n) {
+bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
-    if (!wpr || nb % wpr || n < 1 || n > 64) return false;
+    if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K)) return false;
+    if (wtype != kTypeQ4K) {  // Q5_K: up to two tiles, those of a gate/up pair only from LDS
+        if (n > 32) return false;
+        return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
+    }
     if (n <= 32) return true;
     if (swiglu && n > 48 && (wpr == 1 || wpr == 8)) return false;  // these two forms of the four-tile pair kernel spill registers
     const int nmat = swiglu ? 2 : 1, mt = (int)((n + 15) / 16);
@@ -1366,7 +1388,7 @@ bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n) {
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     if (a.rows <= 0 || a.nb <= 0 || a.n < 1 || a.n > 64 || !a.y || !a.w0 || !a.ap) return hipErrorInvalidValue;
     const int64_t rowtiles = (a.rows + 15) / 16;
-    if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr, a.n)) return hipErrorInvalidValue;
+    if (!skinny16_applies(a.nb, rowtiles, a.w1 != nullptr, a.n, a.wtype)) return hipErrorInvalidValue;
     const int wpr = dense_lds_wpr(a.nb, rowtiles);
     if (a.w1) return launch_skinny16_tiles<2>(a, wpr, stream, start, stop);
     return launch_skinny16_tiles<1>(a, wpr, stream, start, stop);
