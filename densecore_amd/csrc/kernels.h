@@ -133,7 +133,7 @@ struct Skinny16Args {
     float* y = nullptr;
     int64_t ldy = 0;
     int silu_mode = 0;
-    int wtype = kTypeQ4K;          // kTypeQ4K or kTypeQ5K (one and two tiles)
+    int wtype = kTypeQ4K;          // kTypeQ4K, or kTypeQ5K / kTypeQ6K (one and two tiles)
     int ranges = 1;                // set by the launcher: runs of super-blocks the tiles pass through LDS in
 };
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype = kTypeQ4K);

@@ -547,11 +547,12 @@ struct ATile16 {
 // MT: activation tiles of sixteen rows (one, or two for 17 to 32 rows: the weight tile is expanded once for both, 18
 // MFMAs and ~156 vector instructions against the 32 + 294 of two passes over two token tiles of eight each).  With two
 // tiles the partial sums share LDS with the activation tiles (one more barrier before they are written).
-template <int NMAT, int WPR, bool ODD, bool GA, int MT, bool Q5 = false>
+template <int NMAT, int WPR, bool ODD, bool GA, int MT, int WT = kWtQ4>
 __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     constexpr int RPW = 8 / WPR;  // row tiles per workgroup
-    constexpr int kStride = Q5 ? kTile5Bytes : kTileBytes;
-    constexpr int kTileLoads = Q5 ? 4 : 3;  // requests of a weight tile (load_tile)
+    constexpr bool Q5 = WT == kWtQ5, Q6 = WT == kWtQ6;
+    constexpr int kStride = tile_stride<WT>();
+    constexpr int kTileLoads = Q6 ? 5 : Q5 ? 4 : 3;  // requests of a weight tile (load_tile, load_tile6)
     constexpr bool kRedShares = MT > 1 && !GA;  // the partial sums reuse the activation tiles' LDS
     extern __shared__ __align__(16) uint8_t lds16[];
     const int lane = threadIdx.x & 63;
@@ -576,7 +577,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) t.a[j] = *reinterpret_cast<const v4i*>(at + j * 1024 + lane * 16);
         t.yd = *reinterpret_cast<const v4f*>(at + kPScaleOff + kq * 16);
-        t.dg = *reinterpret_cast<const v8h*>(at + digit_off);
+        if constexpr (!Q6) t.dg = *reinterpret_cast<const v8h*>(at + digit_off);  // (Q6_K has no min term)
     };
 
     // ---- the activation tiles ([super-block][tile]) -> LDS: a linear copy, 1 KB per request, the wavefronts taking the
@@ -599,7 +600,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
     };
     if constexpr (!GA) stage_range(0);
 
-    TileRegs ring_t[2][NMAT];
+    typename TileOf<WT>::Regs ring_t[2][NMAT];
     ATile16 ring_a[GA ? 2 : 1][GA ? MT : 1];
     auto issue = [&](auto st_c, int i) {  // only ever called for a stage that exists
         constexpr int st = decltype(st_c)::value;
@@ -609,7 +610,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             for (int t = 0; t < MT; ++t) read_a(ring_a[st][t], p.ap + ((size_t)b * MT + t) * kPTileBytes);
         }
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m) load_tile<Q5>(ring_t[st][m], tiles[m] + (size_t)b * kStride, lane);
+        for (int m = 0; m < NMAT; ++m) load_tile_wt<WT>(ring_t[st][m], tiles[m] + (size_t)b * kStride, lane);
     };
 
     float acc[NMAT][MT][4];
@@ -631,6 +632,75 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             // three and four tiles: the second matrix reads the activation tiles from LDS again instead of keeping the first
             // one's copies in registers (they would not fit)
             if (MT > 2 && m > 0) asm volatile("" ::: "memory");
+            if constexpr (Q6) {
+                // Q6_K the way compute_tile6 multiplies it (decode_tile.h): the B bytes are 4 * (code - 32), a scale per
+                // 16 weights.  B operand jj = 2 j + zp holds the lane's eight weights of sub-block z = zp (dwords 0, 1)
+                // and of z = zp + 2 (dwords 2, 3) of half j -- the pair the activation tile's word jj holds --, and the
+                // k-groups 0, 1 / 2, 3 are the two 16-weight groups of each: four MFMAs per word, every one with the
+                // bytes of one group alone, sixteen group sums per (row, token) and super-block, each times its scale.
+                const TileRegs6& tr = ring_t[st][m];
+                const uint32_t qlw[2][4] = {{tr.ql0.x, tr.ql0.y, tr.ql0.z, tr.ql0.w}, {tr.ql1.x, tr.ql1.y, tr.ql1.z, tr.ql1.w}};
+                const uint32_t qhw[4] = {tr.qh.x, tr.qh.y, tr.qh.z, tr.qh.w};
+                const uint32_t scw[4] = {tr.sc.x, tr.sc.y, tr.sc.z, tr.sc.w};
+                const uint32_t keep_lo = kq < 2 ? 0xffffffffu : 0u, keep_hi = ~keep_lo;
+                // (K = 32 MFMAs: a lane's eight bytes of one sub-block are the whole operand, no zero halves)
+                long bg[4][4];  // [jj][group within the operand: (z = zp, first 16), (zp, last 16), (zp + 2, first), (zp + 2, last)]
+                int sg[4][4];   // their scales
+                auto two = [](uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); };
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int zp = 0; zp < 2; ++zp) {
+                        const int jj = 2 * j + zp;
+                        uint32_t b4[2][2];  // [h][i]
+#pragma unroll
+                        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                            for (int i2 = 0; i2 < 2; ++i2) {
+                                const int z = zp + 2 * hh;
+                                const uint32_t src = qlw[j][2 * zp + i2];
+                                const uint32_t nib = (hh ? src >> 2 : src << 2) & 0x3c3c3c3cu;
+                                const uint32_t hi = qhw[2 * j + i2];
+                                const uint32_t top = (z == 3 ? hi : hi << (6 - 2 * z)) & 0xc0c0c0c0u;
+                                b4[hh][i2] = top | nib;
+                            }
+                        bg[jj][0] = two(b4[0][0] & keep_lo, b4[0][1] & keep_lo);
+                        bg[jj][1] = two(b4[0][0] & keep_hi, b4[0][1] & keep_hi);
+                        bg[jj][2] = two(b4[1][0] & keep_lo, b4[1][1] & keep_lo);
+                        bg[jj][3] = two(b4[1][0] & keep_hi, b4[1][1] & keep_hi);
+                        // group 8 j + 2 z + half: byte 2 (z & 1) + half of scale word 2 j + (z >> 1)
+#pragma unroll
+                        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                            for (int half = 0; half < 2; ++half) {
+                                const int z = zp + 2 * hh;
+                                sg[jj][2 * hh + half] = (int)(int8_t)((scw[2 * j + (z >> 1)] >> (8 * (2 * (z & 1) + half))) & 0xffu);
+                            }
+                    }
+                const float wd = half_bits_to_float(tr.d & 0xffffu);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    ATile16 from_lds;
+                    if constexpr (!GA) read_a(from_lds, lds16 + ((size_t)(b - b_range0) * MT + t) * kPTileBytes);
+                    const ATile16& at = GA ? ring_a[GA ? st : 0][GA ? t : 0] : from_lds;
+                    const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
+                    int dot[4] = {0, 0, 0, 0};
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            const long a8 = gq < 2 ? two((uint32_t)at.a[jj].x, (uint32_t)at.a[jj].y) : two((uint32_t)at.a[jj].z, (uint32_t)at.a[jj].w);
+                            const v4i pg = __builtin_amdgcn_mfma_i32_16x16x32_i8(a8, bg[jj][gq], zero, 0, 0, 0);
+#pragma unroll
+                            for (int i2 = 0; i2 < 4; ++i2) dot[i2] += __mul24(pg[i2], sg[jj][gq]);
+                        }
+#pragma unroll
+                    for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile6's update
+                        const int isum = dot[i2] >> 2;  // the B bytes carried a factor 4
+                        acc[m][t][i2] = __fmaf_rn(__fmul_rn(ydv[i2], wd), (float)isum, acc[m][t][i2]);
+                    }
+                }
+            } else {
             WTile wt;
             expand_tile<Q5>(ring_t[st][m].q0, ring_t[st][m].q1, ring_t[st][m].hdr, Q5 ? ring_t[st][m].qh : v2u{0u, 0u}, kq, wt);
 #pragma unroll
@@ -659,6 +729,7 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
                     const float term = __fsub_rn(__fmul_rn(d, (float)dot), __fmul_rn(dm, mn[i2]));
                     acc[m][t][i2] = __fadd_rn(acc[m][t][i2], term);
                 }
+            }
             }
         }
     };
@@ -1292,11 +1363,11 @@ int skinny16_ranges(int nmat, int wpr, int64_t nb, int mt) {
     return 0;
 }
 
-template <int NMAT, int WPR, bool ODD, bool GA, int MT, bool Q5>
+template <int NMAT, int WPR, bool ODD, bool GA, int MT, int WT>
 hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int64_t rowtiles = (a.rows + 15) / 16;
     const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT, ranges);
-    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT, Q5>;
+    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT, WT>;
     static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
@@ -1314,36 +1385,38 @@ hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t st
 
 // MT <= 2: the rows' tiles in LDS (in runs if need be), else from global memory a stage ahead; three and four tiles only
 // from LDS (read a stage ahead they do not fit the registers), an even number of stages per wavefront.
-template <int NMAT, int WPR, int MT, bool Q5>
+template <int NMAT, int WPR, int MT, int WT>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const bool odd = ((a.nb / WPR) & 1) != 0;
     const int ranges = odd ? (skinny16_lds_bytes(NMAT, WPR, a.nb, MT, 1) <= kSkinnyLdsMax ? 1 : 0) : skinny16_ranges(NMAT, WPR, a.nb, MT);
-    if constexpr (MT <= 2) {
+    if constexpr (WT == kWtQ6 && (WPR == 1 || (NMAT == 2 && MT == 2))) {
+        return hipErrorInvalidValue;  // (these Q6_K forms spill registers: skinny16_applies)
+    } else if constexpr (MT <= 2) {
         const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
-        if constexpr (Q5 && NMAT == 2 && MT == 2) {  // (read a stage ahead, two tiles of a Q5_K pair spill registers: skinny16_applies)
+        if constexpr (WT != kWtQ4 && NMAT == 2 && MT == 2) {  // (read a stage ahead, two tiles of a Q5_K or Q6_K pair spill registers: skinny16_applies)
             if (ga) return hipErrorInvalidValue;
-            if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, Q5>(a, 1, stream, start, stop);
-            return launch_skinny16_one<NMAT, WPR, false, false, MT, Q5>(a, 1, stream, start, stop);
+            if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
+            return launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
         } else {
-            if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, Q5>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, Q5>(a, 1, stream, start, stop);
-            return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, Q5>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, Q5>(a, 1, stream, start, stop);
+            if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
+            return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
         }
-    } else if constexpr (Q5 || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
+    } else if constexpr (WT != kWtQ4 || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
-        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, false>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
-        return launch_skinny16_one<NMAT, WPR, false, false, MT, false>(a, ranges, stream, start, stop);
+        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, kWtQ4>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
+        return launch_skinny16_one<NMAT, WPR, false, false, MT, kWtQ4>(a, ranges, stream, start, stop);
     }
 }
 
-template <int NMAT, int MT, bool Q5>
+template <int NMAT, int MT, int WT>
 hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     switch (wpr) {
-        case 1: return launch_skinny16_form<NMAT, 1, MT, Q5>(a, stream, start, stop);
-        case 2: return launch_skinny16_form<NMAT, 2, MT, Q5>(a, stream, start, stop);
-        case 4: return launch_skinny16_form<NMAT, 4, MT, Q5>(a, stream, start, stop);
-        case 8: return launch_skinny16_form<NMAT, 8, MT, Q5>(a, stream, start, stop);
+        case 1: return launch_skinny16_form<NMAT, 1, MT, WT>(a, stream, start, stop);
+        case 2: return launch_skinny16_form<NMAT, 2, MT, WT>(a, stream, start, stop);
+        case 4: return launch_skinny16_form<NMAT, 4, MT, WT>(a, stream, start, stop);
+        case 8: return launch_skinny16_form<NMAT, 8, MT, WT>(a, stream, start, stop);
     }
     return hipErrorInvalidValue;
 }
@@ -1352,30 +1425,36 @@ template <int NMAT>
 hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int mt = (int)((a.n + 15) / 16);
     if (a.wtype == kTypeQ5K) {  // one and two tiles (the third chain's operands leave no registers for more)
-        if (mt == 1) return launch_skinny16_wpr<NMAT, 1, true>(a, wpr, stream, start, stop);
-        if (mt == 2) return launch_skinny16_wpr<NMAT, 2, true>(a, wpr, stream, start, stop);
+        if (mt == 1) return launch_skinny16_wpr<NMAT, 1, kWtQ5>(a, wpr, stream, start, stop);
+        if (mt == 2) return launch_skinny16_wpr<NMAT, 2, kWtQ5>(a, wpr, stream, start, stop);
+        return hipErrorInvalidValue;
+    }
+    if (a.wtype == kTypeQ6K) {
+        if (mt == 1) return launch_skinny16_wpr<NMAT, 1, kWtQ6>(a, wpr, stream, start, stop);
+        if (mt == 2) return launch_skinny16_wpr<NMAT, 2, kWtQ6>(a, wpr, stream, start, stop);
         return hipErrorInvalidValue;
     }
     switch (mt) {
-        case 1: return launch_skinny16_wpr<NMAT, 1, false>(a, wpr, stream, start, stop);
-        case 2: return launch_skinny16_wpr<NMAT, 2, false>(a, wpr, stream, start, stop);
-        case 3: return launch_skinny16_wpr<NMAT, 3, false>(a, wpr, stream, start, stop);
-        case 4: return launch_skinny16_wpr<NMAT, 4, false>(a, wpr, stream, start, stop);
+        case 1: return launch_skinny16_wpr<NMAT, 1, kWtQ4>(a, wpr, stream, start, stop);
+        case 2: return launch_skinny16_wpr<NMAT, 2, kWtQ4>(a, wpr, stream, start, stop);
+        case 3: return launch_skinny16_wpr<NMAT, 3, kWtQ4>(a, wpr, stream, start, stop);
+        case 4: return launch_skinny16_wpr<NMAT, 4, kWtQ4>(a, wpr, stream, start, stop);
     }
     return hipErrorInvalidValue;
 }
 
 }  // namespace
 
-// Whether a Q4_K product of n rows (nine to 64; Q5_K: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
+// Whether a Q4_K product of n rows (nine to 64; Q5_K, Q6_K: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
 // (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages (in one run where a
 // wavefront's stage count is odd).
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
-    if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K)) return false;
-    if (wtype != kTypeQ4K) {  // Q5_K: up to two tiles, those of a gate/up pair only from LDS
+    if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
+    if (wtype != kTypeQ4K) {  // Q5_K, Q6_K: up to two tiles, those of a gate/up pair only from LDS
         if (n > 32) return false;
+        if (wtype == kTypeQ6K && (wpr == 1 || (swiglu && n > 16))) return false;  // (forms that spill registers)
         return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
     }
     if (n <= 32) return true;
