@@ -434,14 +434,15 @@ def side_measurements(ops, synth, torch, np, dev):
     for w in ring:
         w.free()
 
-    # the sibling K-quant types through the same decode kernel: the FFN down projection 14336 -> 4096 at n = 1 and 8
-    # on a ring of 12 matrices per type (Q4_K 396 MB, Q5_K 484 MB, Q6_K 578 MB)
+    # the sibling K-quant types through the same decode kernels: the FFN down projection 14336 -> 4096 at n = 1 and 8,
+    # and at 16 and 32 rows (one and two activation tiles of sixteen), on a ring of 12 matrices per type
+    # (Q4_K 396 MB, Q5_K 484 MB, Q6_K 578 MB)
     sib = {}
     for name, gtype, bb in (("Q4_K", synth.GGML_TYPE_Q4_K, 144), ("Q5_K", synth.GGML_TYPE_Q5_K, 176),
                             ("Q6_K", synth.GGML_TYPE_Q6_K, 210)):
         ring = [ops.Q4KWeight.synthetic(synth.tensor_seed("sib", name, r), 4096, 14336, 1, gtype) for r in range(12)]
         per = {}
-        for n in (1, 8):
+        for n in (1, 8, 16, 32):
             acts = ops.Q8KActs(n, 14336).quantize(torch.from_numpy(synth.normal_f32(synth.tensor_seed("sib-x", n), (n, 14336))).to(dev))
             y = torch.empty((n, 4096), dtype=torch.float32, device=dev)
             dt = time_graph(lambda: [acts.mul_mat(w, out=y) for w in ring], 20) / len(ring)
