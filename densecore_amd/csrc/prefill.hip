@@ -221,6 +221,74 @@ __device__ __forceinline__ void expand_tile6(const v4u ql0, const v4u ql1, const
     t.d = half_bits_to_float(dw & 0xffffu);
 }
 
+// Q6_K the way compute_tile6 multiplies it (decode_tile.h), for activation tiles of sixteen rows: the B bytes are
+// 4 * (code - 32), a scale per 16 weights.  Word jj = 2 j + zp of a P-major activation tile holds a lane's eight values
+// of sub-block z = zp (bytes 0..7) and of z = zp + 2 (bytes 8..15) of half j, and the k-groups 0, 1 / 2, 3 of a K = 32
+// MFMA over one of those runs are the two 16-weight scale groups of the sub-block: four MFMAs per word, each with the
+// bytes of one group alone (the others' lanes zero), sixteen group sums per (row, token) and super-block, each times
+// its scale in integers -- dot = sum_g scale_g * sum (code - 32) * q8 exactly (core/src/llm/matmul/q6_small_batch.h:56-83),
+// carrying the bytes' factor 4.
+struct WTile6G {
+    long bg[4][4];  // [word jj][(z = zp, first 16), (zp, last 16), (zp + 2, first 16), (zp + 2, last 16)]
+    int sg[4][4];   // their scales
+    float d;
+};
+
+__device__ __forceinline__ long two_words(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+
+__device__ __forceinline__ void expand_tile6g(const v4u ql0, const v4u ql1, const v4u qh, const v4u sc, uint32_t dw, int kq, WTile6G& t) {
+    const uint32_t qlw[2][4] = {{ql0.x, ql0.y, ql0.z, ql0.w}, {ql1.x, ql1.y, ql1.z, ql1.w}};
+    const uint32_t qhw[4] = {qh.x, qh.y, qh.z, qh.w};
+    const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+    const uint32_t keep_lo = kq < 2 ? 0xffffffffu : 0u, keep_hi = ~keep_lo;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int zp = 0; zp < 2; ++zp) {
+            const int jj = 2 * j + zp;
+            uint32_t b4[2][2];  // [nibble side h][word i]: 4 * (code - 32) of z = zp + 2 h
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int z = zp + 2 * h;
+                    const uint32_t src = qlw[j][2 * zp + i];
+                    const uint32_t nib = (h ? src >> 2 : src << 2) & 0x3c3c3c3cu;
+                    const uint32_t hi = qhw[2 * j + i];
+                    const uint32_t top = (z == 3 ? hi : hi << (6 - 2 * z)) & 0xc0c0c0c0u;
+                    b4[h][i] = top | nib;
+                }
+            t.bg[jj][0] = two_words(b4[0][0] & keep_lo, b4[0][1] & keep_lo);
+            t.bg[jj][1] = two_words(b4[0][0] & keep_hi, b4[0][1] & keep_hi);
+            t.bg[jj][2] = two_words(b4[1][0] & keep_lo, b4[1][1] & keep_lo);
+            t.bg[jj][3] = two_words(b4[1][0] & keep_hi, b4[1][1] & keep_hi);
+            // group 8 j + 2 z + half: byte 2 (z & 1) + half of scale word 2 j + (z >> 1)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int z = zp + 2 * h;
+                    t.sg[jj][2 * h + half] = (int)(int8_t)((scw[2 * j + (z >> 1)] >> (8 * (2 * (z & 1) + half))) & 0xffu);
+                }
+        }
+    t.d = half_bits_to_float(dw & 0xffffu);
+}
+
+// one activation tile of sixteen rows (its four words a[]) against the expanded tile: dot[i] += the lane's four
+// (token 4 kq + i, weight row r) sums, times 4
+__device__ __forceinline__ void mul_tile6g(const v4i (&a)[4], const WTile6G& w, int (&dot)[4]) {
+    const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            const long a8 = gq < 2 ? two_words((uint32_t)a[jj].x, (uint32_t)a[jj].y) : two_words((uint32_t)a[jj].z, (uint32_t)a[jj].w);
+            const v4i pg = __builtin_amdgcn_mfma_i32_16x16x32_i8(a8, w.bg[jj][gq], zero, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dot[i] += __mul24(pg[i], w.sg[jj][gq]);
+        }
+}
+
 typedef __attribute__((address_space(1))) const void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -633,51 +701,9 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             // one's copies in registers (they would not fit)
             if (MT > 2 && m > 0) asm volatile("" ::: "memory");
             if constexpr (Q6) {
-                // Q6_K the way compute_tile6 multiplies it (decode_tile.h): the B bytes are 4 * (code - 32), a scale per
-                // 16 weights.  B operand jj = 2 j + zp holds the lane's eight weights of sub-block z = zp (dwords 0, 1)
-                // and of z = zp + 2 (dwords 2, 3) of half j -- the pair the activation tile's word jj holds --, and the
-                // k-groups 0, 1 / 2, 3 are the two 16-weight groups of each: four MFMAs per word, every one with the
-                // bytes of one group alone, sixteen group sums per (row, token) and super-block, each times its scale.
                 const TileRegs6& tr = ring_t[st][m];
-                const uint32_t qlw[2][4] = {{tr.ql0.x, tr.ql0.y, tr.ql0.z, tr.ql0.w}, {tr.ql1.x, tr.ql1.y, tr.ql1.z, tr.ql1.w}};
-                const uint32_t qhw[4] = {tr.qh.x, tr.qh.y, tr.qh.z, tr.qh.w};
-                const uint32_t scw[4] = {tr.sc.x, tr.sc.y, tr.sc.z, tr.sc.w};
-                const uint32_t keep_lo = kq < 2 ? 0xffffffffu : 0u, keep_hi = ~keep_lo;
-                // (K = 32 MFMAs: a lane's eight bytes of one sub-block are the whole operand, no zero halves)
-                long bg[4][4];  // [jj][group within the operand: (z = zp, first 16), (zp, last 16), (zp + 2, first), (zp + 2, last)]
-                int sg[4][4];   // their scales
-                auto two = [](uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); };
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-#pragma unroll
-                    for (int zp = 0; zp < 2; ++zp) {
-                        const int jj = 2 * j + zp;
-                        uint32_t b4[2][2];  // [h][i]
-#pragma unroll
-                        for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-                            for (int i2 = 0; i2 < 2; ++i2) {
-                                const int z = zp + 2 * hh;
-                                const uint32_t src = qlw[j][2 * zp + i2];
-                                const uint32_t nib = (hh ? src >> 2 : src << 2) & 0x3c3c3c3cu;
-                                const uint32_t hi = qhw[2 * j + i2];
-                                const uint32_t top = (z == 3 ? hi : hi << (6 - 2 * z)) & 0xc0c0c0c0u;
-                                b4[hh][i2] = top | nib;
-                            }
-                        bg[jj][0] = two(b4[0][0] & keep_lo, b4[0][1] & keep_lo);
-                        bg[jj][1] = two(b4[0][0] & keep_hi, b4[0][1] & keep_hi);
-                        bg[jj][2] = two(b4[1][0] & keep_lo, b4[1][1] & keep_lo);
-                        bg[jj][3] = two(b4[1][0] & keep_hi, b4[1][1] & keep_hi);
-                        // group 8 j + 2 z + half: byte 2 (z & 1) + half of scale word 2 j + (z >> 1)
-#pragma unroll
-                        for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-                            for (int half = 0; half < 2; ++half) {
-                                const int z = zp + 2 * hh;
-                                sg[jj][2 * hh + half] = (int)(int8_t)((scw[2 * j + (z >> 1)] >> (8 * (2 * (z & 1) + half))) & 0xffu);
-                            }
-                    }
-                const float wd = half_bits_to_float(tr.d & 0xffffu);
+                WTile6G w6;
+                expand_tile6g(tr.ql0, tr.ql1, tr.qh, tr.sc, tr.d, kq, w6);
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
                     ATile16 from_lds;
@@ -685,19 +711,11 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
                     const ATile16& at = GA ? ring_a[GA ? st : 0][GA ? t : 0] : from_lds;
                     const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
                     int dot[4] = {0, 0, 0, 0};
-#pragma unroll
-                    for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-                        for (int gq = 0; gq < 4; ++gq) {
-                            const long a8 = gq < 2 ? two((uint32_t)at.a[jj].x, (uint32_t)at.a[jj].y) : two((uint32_t)at.a[jj].z, (uint32_t)at.a[jj].w);
-                            const v4i pg = __builtin_amdgcn_mfma_i32_16x16x32_i8(a8, bg[jj][gq], zero, 0, 0, 0);
-#pragma unroll
-                            for (int i2 = 0; i2 < 4; ++i2) dot[i2] += __mul24(pg[i2], sg[jj][gq]);
-                        }
+                    mul_tile6g(at.a, w6, dot);
 #pragma unroll
                     for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile6's update
                         const int isum = dot[i2] >> 2;  // the B bytes carried a factor 4
-                        acc[m][t][i2] = __fmaf_rn(__fmul_rn(ydv[i2], wd), (float)isum, acc[m][t][i2]);
+                        acc[m][t][i2] = __fmaf_rn(__fmul_rn(ydv[i2], w6.d), (float)isum, acc[m][t][i2]);
                     }
                 }
             } else {
