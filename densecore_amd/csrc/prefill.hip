@@ -276,10 +276,14 @@ __device__ __forceinline__ void expand_tile6g(const v4u ql0, const v4u ql1, cons
 
 // one activation tile of sixteen rows (its four words a[]) against the expanded tile: dot[i] += the lane's four
 // (token 4 kq + i, weight row r) sums, times 4
+template <bool kFenced = false>
 __device__ __forceinline__ void mul_tile6g(const v4i (&a)[4], const WTile6G& w, int (&dot)[4]) {
     const v4i zero = {0, 0, 0, 0};
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj)
+    for (int jj = 0; jj < 4; ++jj) {
+        // kFenced: the scheduler keeps each word's four MFMAs and their sums together instead of sixteen results in
+        // flight (kernels with many accumulators: registers)
+        if (kFenced && jj > 0) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
             const long a8 = gq < 2 ? two_words((uint32_t)a[jj].x, (uint32_t)a[jj].y) : two_words((uint32_t)a[jj].z, (uint32_t)a[jj].w);
@@ -287,6 +291,7 @@ __device__ __forceinline__ void mul_tile6g(const v4i (&a)[4], const WTile6G& w, 
 #pragma unroll
             for (int i = 0; i < 4; ++i) dot[i] += __mul24(pg[i], w.sg[jj][gq]);
         }
+    }
 }
 
 typedef __attribute__((address_space(1))) const void* global_ptr_t;
@@ -706,12 +711,13 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
                 expand_tile6g(tr.ql0, tr.ql1, tr.qh, tr.sc, tr.d, kq, w6);
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
+                    if (MT > 2 && t > 0) asm volatile("" ::: "memory");  // a tile's LDS reads stay behind the tile before (registers)
                     ATile16 from_lds;
                     if constexpr (!GA) read_a(from_lds, lds16 + ((size_t)(b - b_range0) * MT + t) * kPTileBytes);
                     const ATile16& at = GA ? ring_a[GA ? st : 0][GA ? t : 0] : from_lds;
                     const float ydv[4] = {at.yd.x, at.yd.y, at.yd.z, at.yd.w};
                     int dot[4] = {0, 0, 0, 0};
-                    mul_tile6g(at.a, w6, dot);
+                    mul_tile6g<(MT > 2)>(at.a, w6, dot);
 #pragma unroll
                     for (int i2 = 0; i2 < 4; ++i2) {  // compute_tile6's update
                         const int isum = dot[i2] >> 2;  // the B bytes carried a factor 4
@@ -1419,12 +1425,13 @@ hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEv
             if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
             return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
         }
-    } else if constexpr (WT != kWtQ4 || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
+    } else if constexpr ((WT != kWtQ4 && (NMAT == 2 || WPR == 1)) || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
-        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, kWtQ4>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
-        return launch_skinny16_one<NMAT, WPR, false, false, MT, kWtQ4>(a, ranges, stream, start, stop);
+        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
+        if constexpr (WT == kWtQ6) return hipErrorInvalidValue;  // (its forms for an even count spill registers: skinny16_applies)
+        else return launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, ranges, stream, start, stop);
     }
 }
 
@@ -1442,14 +1449,18 @@ hipError_t launch_skinny16_wpr(const Skinny16Args& a, int wpr, hipStream_t strea
 template <int NMAT>
 hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int mt = (int)((a.n + 15) / 16);
-    if (a.wtype == kTypeQ5K) {  // one and two tiles (the third chain's operands leave no registers for more)
+    if (a.wtype == kTypeQ5K) {
         if (mt == 1) return launch_skinny16_wpr<NMAT, 1, kWtQ5>(a, wpr, stream, start, stop);
         if (mt == 2) return launch_skinny16_wpr<NMAT, 2, kWtQ5>(a, wpr, stream, start, stop);
+        if (mt == 3) return launch_skinny16_wpr<NMAT, 3, kWtQ5>(a, wpr, stream, start, stop);
+        if (mt == 4) return launch_skinny16_wpr<NMAT, 4, kWtQ5>(a, wpr, stream, start, stop);
         return hipErrorInvalidValue;
     }
     if (a.wtype == kTypeQ6K) {
         if (mt == 1) return launch_skinny16_wpr<NMAT, 1, kWtQ6>(a, wpr, stream, start, stop);
         if (mt == 2) return launch_skinny16_wpr<NMAT, 2, kWtQ6>(a, wpr, stream, start, stop);
+        if (mt == 3) return launch_skinny16_wpr<NMAT, 3, kWtQ6>(a, wpr, stream, start, stop);
+        if (mt == 4) return launch_skinny16_wpr<NMAT, 4, kWtQ6>(a, wpr, stream, start, stop);
         return hipErrorInvalidValue;
     }
     switch (mt) {
@@ -1463,7 +1474,7 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 
 }  // namespace
 
-// Whether a Q4_K product of n rows (nine to 64; Q5_K, Q6_K: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
+// Whether a Q4_K product of n rows (nine to 64; a Q5_K or Q6_K pair: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
 // (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages (in one run where a
 // wavefront's stage count is odd).
@@ -1471,8 +1482,13 @@ bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int 
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
     if (wtype != kTypeQ4K) {  // Q5_K, Q6_K: up to two tiles, those of a gate/up pair only from LDS
-        if (n > 32) return false;
         if (wtype == kTypeQ6K && (wpr == 1 || (swiglu && n > 16))) return false;  // (forms that spill registers)
+        if (n > 32) {  // three and four tiles: single matrices, from LDS
+            if (swiglu || wpr == 1) return false;
+            const int mt = (int)((n + 15) / 16);
+            if ((nb / wpr) & 1) return skinny16_lds_bytes(1, wpr, nb, mt, 1) <= kSkinnyLdsMax;
+            return wtype != kTypeQ6K && skinny16_ranges(1, wpr, nb, mt) != 0;  // (Q6_K: the forms for an even stage count spill registers)
+        }
         return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
     }
     if (n <= 32) return true;

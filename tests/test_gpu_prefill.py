@@ -160,9 +160,9 @@ def test_gemm_integer_sums_are_exact_with_k_in_runs(ops):
 def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(ops):
     """24 MB of weights and more: Q4_K rows up to 64 stay on the decode arithmetic (up to four tiles of sixteen per weight
     tile: a row's result is the one it has when the rows are handed over sixteen at a time, bit for bit); from 65 rows
-    mul_mat hands them to the matrix-core GEMM (matrices whose rows do not pass through LDS that way from 33; Q5_K and
-    Q6_K matrices of that size from 33 -- up to 32 rows they are one and two tiles of sixteen --, smaller matrices from
-    48)."""
+    mul_mat hands them to the matrix-core GEMM (matrices whose rows do not pass through LDS that way from 33; Q5_K
+    matrices as Q4_K ones; Q6_K matrices of that size from 33 -- up to 32 rows they are one and two tiles of sixteen --,
+    smaller ones from 48)."""
     import torch
     W = ops.Q4KWeight.synthetic(4, 14336, 4096)
     x = torch.randn((70, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(20))
@@ -179,18 +179,26 @@ def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(op
     assert torch.equal(ops.mul_mat(W, x[:30]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:30])]))
     assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
     W.free()
-    W = ops.Q4KWeight.synthetic(6, 4096, 4096, ggml_type=synth.GGML_TYPE_Q5_K)   # the other types, smaller matrices: 16-row passes up to 47 rows
-    x = torch.randn((48, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(22))
-    assert torch.equal(ops.mul_mat(W, x[:20]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:20])]))
-    assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
-    W.free()
-    # ... and of 24 MB of Q4_K's size and more: the GEMM from 33 rows (one and two tiles of sixteen before)
-    for wtype in (synth.GGML_TYPE_Q5_K, synth.GGML_TYPE_Q6_K):
-        W = ops.Q4KWeight.synthetic(8, 14336, 4096, ggml_type=wtype)
-        assert torch.equal(ops.mul_mat(W, x[:33]), ops.gemm(W, x[:33]))
-        assert torch.equal(ops.mul_mat(W, x[:30]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:30])]))
+    # the other types: Q5_K like Q4_K (up to four tiles of sixteen, then the GEMM); Q6_K two tiles, then 16-row passes up to
+    # 47 rows on smaller matrices, the GEMM from 33 on those of 24 MB of Q4_K's size and more
+    x = torch.randn((70, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(22))
+    pieces = lambda t: torch.cat([ops.mul_mat(W, t[i:i + 16]) for i in range(0, t.shape[0], 16)])
+    for rows in (4096, 14336):
+        W = ops.Q4KWeight.synthetic(6, rows, 4096, ggml_type=synth.GGML_TYPE_Q5_K)
+        assert torch.equal(ops.mul_mat(W, x[:20]), pieces(x[:20]))
+        assert torch.equal(ops.mul_mat(W, x[:48]), pieces(x[:48]))
+        assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
         assert torch.equal(ops.mul_mat(W, x[:16]), torch.cat([ops.mul_mat(W, x[:8]), ops.mul_mat(W, x[8:16])]))
         W.free()
+    W = ops.Q4KWeight.synthetic(6, 4096, 4096, ggml_type=synth.GGML_TYPE_Q6_K)
+    assert torch.equal(ops.mul_mat(W, x[:40]), pieces(x[:40]))
+    assert torch.equal(ops.mul_mat(W, x[:48]), ops.gemm(W, x[:48]))
+    W.free()
+    W = ops.Q4KWeight.synthetic(8, 14336, 4096, ggml_type=synth.GGML_TYPE_Q6_K)
+    assert torch.equal(ops.mul_mat(W, x[:33]), ops.gemm(W, x[:33]))
+    assert torch.equal(ops.mul_mat(W, x[:30]), pieces(x[:30]))
+    assert torch.equal(ops.mul_mat(W, x[:16]), torch.cat([ops.mul_mat(W, x[:8]), ops.mul_mat(W, x[8:16])]))
+    W.free()
     W = ops.Q4KWeight.synthetic(5, 4096, 4096)
     x = torch.randn((20, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(21))
     assert torch.equal(ops.mul_mat(W, x), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:])]))
