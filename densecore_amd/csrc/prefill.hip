@@ -609,6 +609,10 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 // memory a stage ahead, beside the weight tile (six loads, all answered by the L2).  The integers of a (row, token,
 // super-block) are the same and so is the fp32 update, (wd * yd) * dot - (wm * yd) * min_dot added to the running
 // sum: the same bits as dense_lds_kernel and matmul_kernel.
+// WT: Q4_K; Q5_K with a third MFMA chain for the fifth code bits times the whole scale (expand_tile<true>), the decode
+// kernels' integers (scale * (nibble + 16 bit)) and update; Q6_K with the arithmetic of compute_tile6 carried over to
+// tiles of sixteen (expand_tile6g, mul_tile6g above): sixteen K = 32 MFMAs per activation tile and super-block, one per
+// 16-weight scale group, the group sums times their scales in integers, one fused multiply-add per super-block.
 // LDS: [nb][4688] activation tiles (not GA), then the partial sums [8 / WPR][WPR - 1][NMAT][4][64].
 // nb % WPR == 0 (host-checked): every wavefront has nb / WPR stages; ODD: that count is odd.
 struct ATile16 {
