@@ -1478,14 +1478,20 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 
 }  // namespace
 
-// Whether a Q4_K product of n rows (nine to 64; a Q5_K or Q6_K pair: to 32) runs on skinny16_kernel: the wave split of the other decode kernels must be
-// one of its own (a divisor of eight that divides the super-blocks of a row); up to 32 rows that is all, 33 to 64 rows
-// (three and four tiles of sixteen) must also pass through LDS in at most four runs of whole stages (in one run where a
-// wavefront's stage count is odd).
+// Whether a product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
+// one of its own (a divisor of eight that divides the super-blocks of a row), and the form must be built
+// (launch_skinny16_form returns an error for the others: those whose registers spill).
+//   Q4_K  one and two tiles (up to 32 rows) always; three and four where the tiles pass through LDS in at most four runs
+//         of whole stages (in one run where a wavefront's stage count is odd); a gate/up pair of four tiles not with one
+//         or eight wavefronts per row tile.
+//   Q5_K  single matrices as Q4_K, three and four tiles not with one wavefront per row tile; a pair one tile, two where
+//         they fit LDS in one run.
+//   Q6_K  not with one wavefront per row tile; single matrices one and two tiles, three and four only where a
+//         wavefront's stage count is odd; a pair one tile.
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
-    if (wtype != kTypeQ4K) {  // Q5_K, Q6_K: up to two tiles, those of a gate/up pair only from LDS
+    if (wtype != kTypeQ4K) {
         if (wtype == kTypeQ6K && (wpr == 1 || (swiglu && n > 16))) return false;  // (forms that spill registers)
         if (n > 32) {  // three and four tiles: single matrices, from LDS
             if (swiglu || wpr == 1) return false;
