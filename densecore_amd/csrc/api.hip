@@ -864,11 +864,27 @@ int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* 
             return MQ_OK;
         }
     }
-    if (prefill_applies(w, n)) {
-        // prefill widths: the normalised rows as fp32, then the matrix-core GEMM (its quantizer reads them)
+    // Seventeen to 64 rows where mq_mul_mat_q4k takes them as tiles of sixteen: the normalised rows as fp32, their
+    // quantizer, the same launch (up to sixteen rows the norm's own Q8_K output and the kernels with token tiles of
+    // eight below cost a launch less; the bits are the same)
+    const bool tiles16 = n > 16 && skinny16_takes(w, n, false);
+    if (tiles16 || prefill_applies(w, n)) {
+        // ... and prefill widths: the normalised rows as fp32, then the matrix-core GEMM (its quantizer reads them)
         MQ_HIP(g.mid.reserve((size_t)n * (size_t)w->cols * sizeof(float)));
         MQ_HIP(launch_add_rmsnorm(x_dev, delta_dev, weight_dev, n, w->cols, eps, sum_out_dev, (float*)g.mid.ptr, nullptr, nullptr, s));
-        return gemm_locked(w, (const float*)g.mid.ptr, n, w->cols, y_dev, ldy, s);
+        if (!tiles16) return gemm_locked(w, (const float*)g.mid.ptr, n, w->cols, y_dev, ldy, s);
+        if (int rc = quantize_into_tile16((const float*)g.mid.ptr, n, w->cols, w->cols, s)) return rc;
+        MatmulArgs a;
+        a.w0 = w->data;
+        a.wtype = w->type;
+        a.rows = w->rows;
+        a.nb = w->nb;
+        a.ap = (const uint8_t*)g.ap.ptr;
+        a.n = n;
+        a.y = y_dev;
+        a.ldy = ldy;
+        MQ_HIP(census_launch(a, s));
+        return MQ_OK;
     }
     const int64_t nb = w->cols / kQK;
     MQ_HIP(g.aq.reserve(aq_bytes(n, nb)));

@@ -317,7 +317,8 @@ int mq_add_rmsnorm_q8k(const float* x_dev, const float* delta_dev, const float* 
  * weight (weight_dev may be NULL), y[t] = W . q8k(h[t]); x/delta/sum fp32 [n][cols] dense, y fp32 [n][ldy].  Up to
  * four rows of input against Q4_K weights with short rows run as ONE launch (norm and quantizer inside the GEMV),
  * otherwise two; the same bits either way.  sum_out_dev (may be NULL) must be neither x_dev nor delta_dev.  At the
- * widths where mq_mul_mat_q4k takes the matrix-core GEMM the normalised rows are written as fp32 and go through it. */
+ * widths where mq_mul_mat_q4k takes the matrix-core GEMM the normalised rows are written as fp32 and go through it, and
+ * likewise, from seventeen rows, where it takes the rows as tiles of sixteen. */
 int mq_rmsnorm_mul_mat_q4k(const mq_weight* w, const float* x_dev, const float* delta_dev, const float* weight_dev, int64_t n,
                            float eps, float* sum_out_dev, float* y_dev, int64_t ldy, void* stream);
 /* logits[t][e] = w[e] . x[t] in fp32: the ffn_gate_inp router projection

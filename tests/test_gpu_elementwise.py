@@ -137,10 +137,10 @@ def test_rmsnorm_mul_mat_equals_norm_then_product(n, rows, cols, with_delta, wit
     W.free()
 
 
-@pytest.mark.parametrize("n,rows,cols", [(64, 2560, 2048), (20, 14336, 4096)])
+@pytest.mark.parametrize("n,rows,cols", [(70, 2560, 2048), (40, 4096, 14336)])
 def test_rmsnorm_mul_mat_at_prefill_widths_is_norm_then_gemm(n, rows, cols):
-    """Where mq_mul_mat_q4k takes the matrix-core GEMM (48 rows; 17 for 24 MB and more) the fused entry does too: the
-    bits of mq_add_rmsnorm_f32 followed by mq_gemm_q4k on the normalised rows."""
+    """Where mq_mul_mat_q4k takes the matrix-core GEMM (65 rows; 33 where the rows do not pass through LDS as tiles of
+    sixteen) the fused entry does too: the bits of mq_add_rmsnorm_f32 followed by mq_gemm_q4k on the normalised rows."""
     import torch
     from densecore_amd import _lib, ops
     g = torch.Generator(device="cuda").manual_seed(rows + cols + n)
