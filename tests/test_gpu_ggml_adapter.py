@@ -70,7 +70,7 @@ def test_dense_node_rejects_mismatch(ga):
     assert ud.last_status != 0 and np.all(ty2._keep == 3.0)
 
 
-@pytest.mark.parametrize("n", [1, 6])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 6, 8, 9, 12, 16, 17, 33, 70, 200, 333])
 def test_moe_nodes(ga, n):
     hidden, inter, n_exp, top_k = 512, 256, 8, 2
     gate = np.stack([synth.q4k_matrix(2010 + e, inter, hidden) for e in range(n_exp)])
