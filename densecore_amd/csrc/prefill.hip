@@ -1417,7 +1417,7 @@ template <int NMAT, int WPR, int MT, int WT>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const bool odd = ((a.nb / WPR) & 1) != 0;
     const int ranges = odd ? (skinny16_lds_bytes(NMAT, WPR, a.nb, MT, 1) <= kSkinnyLdsMax ? 1 : 0) : skinny16_ranges(NMAT, WPR, a.nb, MT);
-    if constexpr (WT == kWtQ6 && (WPR == 1 || (NMAT == 2 && MT == 2))) {
+    if constexpr (WT == kWtQ6 && (NMAT == 2 && (MT == 2 || WPR == 1))) {
         return hipErrorInvalidValue;  // (these Q6_K forms spill registers: skinny16_applies)
     } else if constexpr (MT <= 2) {
         const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
@@ -1429,7 +1429,7 @@ hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEv
             if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
             return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
         }
-    } else if constexpr ((WT != kWtQ4 && (NMAT == 2 || WPR == 1)) || (NMAT == 2 && MT == 4 && (WPR == 1 || WPR == 8))) {
+    } else if constexpr (WPR == 1 || (WT != kWtQ4 && NMAT == 2) || (NMAT == 2 && MT == 4 && WPR == 8)) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
@@ -1481,18 +1481,18 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 // Whether a product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row), and the form must be built
 // (launch_skinny16_form returns an error for the others: those whose registers spill).
-//   Q4_K  one and two tiles (up to 32 rows) always; three and four where the tiles pass through LDS in at most four runs
-//         of whole stages (in one run where a wavefront's stage count is odd); a gate/up pair of four tiles not with one
-//         or eight wavefronts per row tile.
-//   Q5_K  single matrices as Q4_K, three and four tiles not with one wavefront per row tile; a pair one tile, two where
-//         they fit LDS in one run.
-//   Q6_K  not with one wavefront per row tile; single matrices one and two tiles, three and four only where a
-//         wavefront's stage count is odd; a pair one tile.
+//   Q4_K  one and two tiles (up to 32 rows) always; three and four not with one wavefront per row tile (more than 1,024
+//         row tiles: the GEMM is faster there) and where the tiles pass through LDS in at most four runs of whole stages
+//         (in one run where a wavefront's stage count is odd); a gate/up pair of four tiles not with eight wavefronts per
+//         row tile.
+//   Q5_K  single matrices as Q4_K; a pair one tile, two where they fit LDS in one run.
+//   Q6_K  single matrices one and two tiles, three and four only where a wavefront's stage count is odd; a pair one
+//         tile, not with one wavefront per row tile.
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
     if (wtype != kTypeQ4K) {
-        if (wtype == kTypeQ6K && (wpr == 1 || (swiglu && n > 16))) return false;  // (forms that spill registers)
+        if (wtype == kTypeQ6K && swiglu && (wpr == 1 || n > 16)) return false;  // (forms that spill registers)
         if (n > 32) {  // three and four tiles: single matrices, from LDS
             if (swiglu || wpr == 1) return false;
             const int mt = (int)((n + 15) / 16);
@@ -1502,7 +1502,10 @@ bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int 
         return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
     }
     if (n <= 32) return true;
-    if (swiglu && n > 48 && (wpr == 1 || wpr == 8)) return false;  // these two forms of the four-tile pair kernel spill registers
+    // more than 1,024 row tiles (a wavefront per row tile): the matrix-core GEMM is faster from 33 rows (128256 x 4096 at
+    // 33 / 64 rows: 93 / 108 us against 102 / 126 as three and four tiles)
+    if (wpr == 1) return false;
+    if (swiglu && n > 48 && wpr == 8) return false;  // this form of the four-tile pair kernel spills registers
     const int nmat = swiglu ? 2 : 1, mt = (int)((n + 15) / 16);
     if ((nb / wpr) & 1) return skinny16_lds_bytes(nmat, wpr, nb, mt, 1) <= kSkinnyLdsMax;  // an odd stage count: the tiles in one run
     return skinny16_ranges(nmat, wpr, nb, mt) != 0;

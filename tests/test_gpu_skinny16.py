@@ -228,7 +228,7 @@ def _sixteen_at_a_time(fn, t):
     return torch.cat([fn(t[i:i + 16]) for i in range(0, t.shape[0], 16)], dim=0)
 
 
-# wavefronts per row tile 2 (two runs of super-blocks), 4 (two runs), 1 (one run), 4 (one run), 8 (two runs of one stage
+# wavefronts per row tile 2 (two runs of super-blocks), 4 (two runs), 1 (not taken: 16-row passes or the GEMM), 4 (one run), 8 (two runs of one stage
 # each), a single stage per wavefront whose tiles fit LDS in one run (twice), and three stages per wavefront whose tiles
 # do not (falls back to the 16-row passes or the GEMM)
 WIDE = [(14336, 4096), (6144, 4096), (20480, 1024), (8192, 2048), (4096, 4096), (2048, 2048), (2560, 2048), (2048, 6144)]
@@ -238,7 +238,7 @@ WIDE = [(14336, 4096), (6144, 4096), (20480, 1024), (8192, 2048), (4096, 4096), 
 def test_three_and_four_tiles_equal_the_rows_taken_sixteen_at_a_time(env, rows, cols):
     torch, _lib, ops = env
     W = ops.Q4KWeight.synthetic(synth.tensor_seed("s64", rows, cols), rows, cols)
-    takes = (rows, cols) != (2048, 6144)
+    takes = (rows, cols) not in ((2048, 6144), (20480, 1024))   # (... and more than 1,024 row tiles: the GEMM from 33 rows)
     for n in (33, 40, 48, 64):
         x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("s64-x", rows, cols, n), (n, cols))).cuda()
         whole, split = ops.mul_mat(W, x), _sixteen_at_a_time(lambda t: ops.mul_mat(W, t), x)
@@ -400,4 +400,23 @@ def test_sibling_types_against_the_oracle(env, wtype):
         mag = mag_of(w, cols, q8, magnitude=True)
         for order in orc.ORDERS.values():
             assert_fp32_parity(got, mul(w, cols, q8, order), mag, f"n={n} order {order}")
+    W.free()
+
+
+@pytest.mark.parametrize("wtype", [12, 14])
+def test_output_projection_sized_matrix(env, wtype):
+    """128,256 x 4,096 (a vocabulary's output projection, Q6_K in a Q4_K_M file): more than 1,024 row tiles, a wavefront
+    per row tile.  Nine to 32 rows are one and two tiles of sixteen -- the bits of the passes of eight --, from 33 the GEMM."""
+    torch, _lib, ops = env
+    L = _lib.lib()
+    rows, cols = 128256, 4096
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("lmhead", wtype), rows, cols, ggml_type=wtype)
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("lmhead-x"), (40, cols))).cuda()
+    for n in (12, 16, 27):
+        got = ops.mul_mat(W, x[:n])
+        L.mq_debug_set_dense_lds(TWO_TILES_OF_EIGHT)
+        want = torch.cat([ops.mul_mat(W, x[i:min(i + 8, n)]) for i in range(0, n, 8)], dim=0)
+        L.mq_debug_set_dense_lds(1)
+        assert torch.equal(got, want), f"n={n}"
+    assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
     W.free()
