@@ -79,3 +79,35 @@ def test_norm_fused_router_equals_norm_then_router(cols, n_experts):
         if n in (1, 9, 72):
             want = h_ref.double().cpu().numpy() @ router.double().cpu().numpy().T
             assert np.abs(lg_ref.cpu().numpy() - want).max() <= 2e-6 * max(np.abs(want).max(), 1e-30), f"n={n}: router"
+
+
+@pytest.mark.parametrize("n", [3, 12, 24, 50, 100])
+def test_norm_fused_projection_replayed_from_a_graph(n):
+    """Every width's launch sequence (norm inside the GEMV, norm + Q8_K + decode kernel, norm + quantizer + tiles of
+    sixteen, norm + GEMM) captured into a HIP graph: three replays with eager work in between equal the eager result."""
+    import torch
+    from densecore_amd import _lib, ops
+    L = _lib.lib()
+    rows, cols = 2560, 2048
+    W = ops.Q4KWeight.synthetic(synth.tensor_seed("nwg", rows, cols), rows, cols)
+    x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("nwg-x", n), (n, cols))).cuda()
+    d = torch.from_numpy(synth.normal_f32(synth.tensor_seed("nwg-d", n), (n, cols))).cuda()
+    s_out, y = torch.empty_like(x), torch.empty((n, rows), dtype=torch.float32, device="cuda")
+    def run():
+        st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(L.mq_rmsnorm_mul_mat_q4k(W._h, _p(x), _p(d), None, n, C.c_float(EPS), _p(s_out), _p(y), rows, st), "mq_rmsnorm_mul_mat_q4k")
+    run()
+    torch.cuda.synchronize()
+    eager = y.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run()
+    for rep in range(3):
+        y.fill_(0.0)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {rep}"
+        other = torch.from_numpy(synth.normal_f32(synth.tensor_seed("nwg-o", rep), (7 + rep, cols))).cuda()
+        ops.mul_mat(W, other)          # eager work on the same workspaces between the replays
+        torch.cuda.synchronize()
+    W.free()
