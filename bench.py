@@ -472,6 +472,25 @@ def side_measurements(ops, synth, torch, np, dev):
     for w in ring:
         w.free()
 
+    # the same entry point on the largest matrix of a model, the output projection (a 128,256-token vocabulary, hidden
+    # 4096; Q6_K in a Q4_K_M file): what the kernels reach on a launch of several hundred MB, quantizer included
+    outp = {}
+    for name, gtype, bb in (("Q4_K", synth.GGML_TYPE_Q4_K, 144), ("Q6_K", synth.GGML_TYPE_Q6_K, 210)):
+        ring = [ops.Q4KWeight.synthetic(synth.tensor_seed("outp", name, r), 128256, 4096, 1, gtype) for r in range(2)]
+        per = {}
+        for n in (1, 8, 16):
+            x = torch.from_numpy(synth.normal_f32(synth.tensor_seed("outp-x", n), (n, 4096))).to(dev)
+            y = torch.empty((n, 128256), dtype=torch.float32, device=dev)
+            dt = time_graph(lambda: [ops.mul_mat(w, x, out=y) for w in ring], 10) / len(ring)
+            b = 128256 * 16 * bb + n * (4096 + 128256) * 4
+            per[str(n)] = {"us": round(dt * 1e6, 1), "GBps": round(b / dt / 1e9, 1),
+                           "pct_hbm_peak": round(b / dt / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+        outp[name] = per
+        for w in ring:
+            w.free()
+    outp["note"] = "mq_mul_mat_q4k (quantizer included), 128256 x 4096 weights, two matrices alternating, bytes = ggml bytes of the type + fp32 in/out"
+    res["output_projection_128256x4096"] = outp
+
     # cfg3: MoE layer, hidden 2048, 256 + 1 experts, inter 512, top-8; ring of 4 layers (1.8 GB)
     E, H, I, K = 256, 2048, 512, 8
     layers = []
