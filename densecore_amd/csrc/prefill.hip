@@ -614,7 +614,8 @@ __global__ void __launch_bounds__(256, 2) prefill_gemm_kernel(const uint8_t* __r
 // tiles of sixteen (expand_tile6g, mul_tile6g above): sixteen K = 32 MFMAs per activation tile and super-block, one per
 // 16-weight scale group, the group sums times their scales in integers, one fused multiply-add per super-block.
 // LDS: [nb][4688] activation tiles (not GA), then the partial sums [8 / WPR][WPR - 1][NMAT][4][64].
-// nb % WPR == 0 (host-checked): every wavefront has nb / WPR stages; ODD: that count is odd.
+// nb % WPR == 0 (host-checked): every wavefront has nb / WPR stages; FLOW 1: that count is odd (a single run); 0: even, a
+// single run or runs of an even number of stages; 2: even, runs of an odd number of stages.
 struct ATile16 {
     v4i a[4];   // the four 64-weight chunks of this lane's operand
     v4f yd;     // the Q8_K scales of rows 4 kq .. 4 kq + 3
@@ -624,8 +625,9 @@ struct ATile16 {
 // MT: activation tiles of sixteen rows (one, or two for 17 to 32 rows: the weight tile is expanded once for both, 18
 // MFMAs and ~156 vector instructions against the 32 + 294 of two passes over two token tiles of eight each).  With two
 // tiles the partial sums share LDS with the activation tiles (one more barrier before they are written).
-template <int NMAT, int WPR, bool ODD, bool GA, int MT, int WT = kWtQ4>
+template <int NMAT, int WPR, int FLOW, bool GA, int MT, int WT = kWtQ4>
 __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
+    constexpr bool ODD = FLOW == 1;  // (FLOW: the shape of the stage loop, below)
     constexpr int RPW = 8 / WPR;  // row tiles per workgroup
     constexpr bool Q5 = WT == kWtQ5, Q6 = WT == kWtQ6;
     constexpr int kStride = tile_stride<WT>();
@@ -799,31 +801,61 @@ __global__ void __launch_bounds__(512) skinny16_kernel(const Skinny16Args p) {
             consume(S0{}, i + 1);
         }
     } else {
-        // the next run of super-blocks replaces the one in LDS once every wavefront has multiplied its last stage of it
-        auto next_range = [&](int i) {
-            if (GA || p.ranges == 1 || i == 0 || i % stages_per_range) return;  // wave-uniform, the same i in every wavefront
-            __syncthreads();
-            const int rg = i / stages_per_range;
-            stage_range(rg);
-            b_range0 = rg * sb_per_range;
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the copy (and its two stages of weight tiles)
-            __syncthreads();
-        };
-        int i = 0;
-        for (; i + 2 < cnt; i += 2) {
+        // The next run of super-blocks replaces the one in LDS once every wavefront has multiplied its last stage of it
+        // (the weight tiles of the next run's first two stages are already on their way: they do not depend on LDS).
+        if constexpr (FLOW == 0) {
+            // A single run, or runs of an even number of stages: run by run, the change of runs between two inner loops
+            // (a conditional change inside the pipelined loop, as below, costs the Q6_K forms their registers: 256 and
+            // spills against 120-130).  The last pair of stages of the launch is peeled off: no request past the end.
+            const int runs = GA ? 1 : p.ranges;
+            int i = 0;
+            for (int rg = 0; rg < runs; ++rg) {
+                if (rg > 0) {  // wave-uniform, the same in every wavefront
+                    __syncthreads();
+                    stage_range(rg);
+                    b_range0 = rg * sb_per_range;
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the copy (and its two stages of weight tiles)
+                    __syncthreads();
+                }
+                const int i_stop = (rg + 1) * (cnt / runs) - (rg == runs - 1 ? 2 : 0);
+                for (; i < i_stop; i += 2) {
+                    consume(S0{}, i);
+                    issue(S0{}, i + 2);
+                    asm volatile("" ::: "memory");
+                    consume(S1{}, i + 1);
+                    issue(S1{}, i + 3);
+                    asm volatile("" ::: "memory");
+                }
+            }
+            consume(S0{}, i);
+            consume(S1{}, i + 1);
+        } else {
+            // FLOW == 2: runs of an odd number of stages begin at either stage of a pair
+            auto next_range = [&](int i) {
+                if (GA || p.ranges == 1 || i == 0 || i % stages_per_range) return;  // wave-uniform, the same i in every wavefront
+                __syncthreads();
+                const int rg = i / stages_per_range;
+                stage_range(rg);
+                b_range0 = rg * sb_per_range;
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the copy (and its two stages of weight tiles)
+                __syncthreads();
+            };
+            int i = 0;
+            for (; i + 2 < cnt; i += 2) {
+                next_range(i);
+                consume(S0{}, i);
+                issue(S0{}, i + 2);
+                asm volatile("" ::: "memory");
+                next_range(i + 1);
+                consume(S1{}, i + 1);
+                issue(S1{}, i + 3);
+                asm volatile("" ::: "memory");
+            }
             next_range(i);
             consume(S0{}, i);
-            issue(S0{}, i + 2);
-            asm volatile("" ::: "memory");
             next_range(i + 1);
             consume(S1{}, i + 1);
-            issue(S1{}, i + 3);
-            asm volatile("" ::: "memory");
         }
-        next_range(i);
-        consume(S0{}, i);
-        next_range(i + 1);
-        consume(S1{}, i + 1);
     }
 
     // ---- the WPR wavefronts of a row tile meet in wave order; the first one stores ----
@@ -1391,11 +1423,11 @@ int skinny16_ranges(int nmat, int wpr, int64_t nb, int mt) {
     return 0;
 }
 
-template <int NMAT, int WPR, bool ODD, bool GA, int MT, int WT>
+template <int NMAT, int WPR, int FLOW, bool GA, int MT, int WT>
 hipError_t launch_skinny16_one(const Skinny16Args& a, int ranges, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const int64_t rowtiles = (a.rows + 15) / 16;
     const size_t lds = GA ? skinny16_red_bytes(NMAT, WPR, MT) : skinny16_lds_bytes(NMAT, WPR, a.nb, MT, ranges);
-    auto* kernel = &skinny16_kernel<NMAT, WPR, ODD, GA, MT, WT>;
+    auto* kernel = &skinny16_kernel<NMAT, WPR, FLOW, GA, MT, WT>;
     static bool raised = false;  // per instantiation; the attribute belongs to the function, not to a launch
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSkinnyLdsMax);
@@ -1423,19 +1455,20 @@ hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEv
         const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
         if constexpr (WT != kWtQ4 && NMAT == 2 && MT == 2) {  // (read a stage ahead, two tiles of a Q5_K or Q6_K pair spill registers: skinny16_applies)
             if (ga) return hipErrorInvalidValue;
-            if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
-            return launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
+            if (odd) return launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);
+            return launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, 1, stream, start, stop);
         } else {
-            if (odd) return ga ? launch_skinny16_one<NMAT, WPR, true, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);
-            return ga ? launch_skinny16_one<NMAT, WPR, false, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, 1, stream, start, stop);
+            if (odd) return ga ? launch_skinny16_one<NMAT, WPR, 1, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);
+            return ga ? launch_skinny16_one<NMAT, WPR, 0, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, 1, stream, start, stop);
         }
     } else if constexpr (WPR == 1 || (WT != kWtQ4 && NMAT == 2) || (NMAT == 2 && MT == 4 && WPR == 8)) {
         return hipErrorInvalidValue;  // (skinny16_applies: not built)
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
-        if (odd) return launch_skinny16_one<NMAT, WPR, true, false, MT, WT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
-        if constexpr (WT == kWtQ6) return hipErrorInvalidValue;  // (its forms for an even count spill registers: skinny16_applies)
-        else return launch_skinny16_one<NMAT, WPR, false, false, MT, WT>(a, ranges, stream, start, stop);
+        if (odd) return launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
+        if ((((a.nb / WPR) / ranges) & 1) == 0) return launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, ranges, stream, start, stop);
+        if constexpr (WT == kWtQ6) return hipErrorInvalidValue;  // (runs of an odd stage count: this form spills registers, skinny16_applies)
+        else return launch_skinny16_one<NMAT, WPR, 2, false, MT, WT>(a, ranges, stream, start, stop);
     }
 }
 
@@ -1486,8 +1519,8 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 //         (in one run where a wavefront's stage count is odd); a gate/up pair of four tiles not with eight wavefronts per
 //         row tile.
 //   Q5_K  single matrices as Q4_K; a pair one tile, two where they fit LDS in one run.
-//   Q6_K  single matrices one and two tiles, three and four only where a wavefront's stage count is odd; a pair one
-//         tile, not with one wavefront per row tile.
+//   Q6_K  single matrices as Q4_K, three and four tiles not in runs of an odd number of stages; a pair one tile, not
+//         with one wavefront per row tile.
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
@@ -1497,7 +1530,8 @@ bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int 
             if (swiglu || wpr == 1) return false;
             const int mt = (int)((n + 15) / 16);
             if ((nb / wpr) & 1) return skinny16_lds_bytes(1, wpr, nb, mt, 1) <= kSkinnyLdsMax;
-            return wtype != kTypeQ6K && skinny16_ranges(1, wpr, nb, mt) != 0;  // (Q6_K: the forms for an even stage count spill registers)
+            const int ranges = skinny16_ranges(1, wpr, nb, mt);
+            return ranges != 0 && (wtype != kTypeQ6K || (((nb / wpr) / ranges) & 1) == 0);  // (Q6_K: not with runs of an odd stage count, whose form spills registers)
         }
         return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
     }

@@ -161,8 +161,7 @@ def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(op
     """24 MB of weights and more: Q4_K rows up to 64 stay on the decode arithmetic (up to four tiles of sixteen per weight
     tile: a row's result is the one it has when the rows are handed over sixteen at a time, bit for bit); from 65 rows
     mul_mat hands them to the matrix-core GEMM (matrices whose rows do not pass through LDS that way from 33; Q5_K
-    matrices as Q4_K ones; Q6_K matrices of that size from 33 -- up to 32 rows they are one and two tiles of sixteen --,
-    smaller ones from 48)."""
+    and Q6_K matrices as Q4_K ones, Q6_K not in runs of an odd number of stages)."""
     import torch
     W = ops.Q4KWeight.synthetic(4, 14336, 4096)
     x = torch.randn((70, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(20))
@@ -179,8 +178,8 @@ def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(op
     assert torch.equal(ops.mul_mat(W, x[:30]), torch.cat([ops.mul_mat(W, x[:16]), ops.mul_mat(W, x[16:30])]))
     assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
     W.free()
-    # the other types: Q5_K like Q4_K (up to four tiles of sixteen, then the GEMM); Q6_K two tiles, then 16-row passes up to
-    # 47 rows on smaller matrices, the GEMM from 33 on those of 24 MB of Q4_K's size and more
+    # the other types: Q5_K like Q4_K (up to four tiles of sixteen, then the GEMM); Q6_K likewise except where the tiles would
+    # pass through LDS in runs of an odd number of stages (4096 x 4096: runs of one): two tiles, then 16-row passes up to 47 rows
     x = torch.randn((70, 4096), device="cuda", generator=torch.Generator(device="cuda").manual_seed(22))
     pieces = lambda t: torch.cat([ops.mul_mat(W, t[i:i + 16]) for i in range(0, t.shape[0], 16)])
     for rows in (4096, 14336):
@@ -194,9 +193,10 @@ def test_large_matrices_take_the_gemm_beyond_the_widths_of_the_decode_kernels(op
     assert torch.equal(ops.mul_mat(W, x[:40]), pieces(x[:40]))
     assert torch.equal(ops.mul_mat(W, x[:48]), ops.gemm(W, x[:48]))
     W.free()
-    W = ops.Q4KWeight.synthetic(8, 14336, 4096, ggml_type=synth.GGML_TYPE_Q6_K)
-    assert torch.equal(ops.mul_mat(W, x[:33]), ops.gemm(W, x[:33]))
-    assert torch.equal(ops.mul_mat(W, x[:30]), pieces(x[:30]))
+    W = ops.Q4KWeight.synthetic(8, 14336, 4096, ggml_type=synth.GGML_TYPE_Q6_K)   # (runs of four stages: up to four tiles)
+    assert torch.equal(ops.mul_mat(W, x[:33]), pieces(x[:33]))
+    assert torch.equal(ops.mul_mat(W, x[:64]), pieces(x[:64]))
+    assert torch.equal(ops.mul_mat(W, x), ops.gemm(W, x))
     assert torch.equal(ops.mul_mat(W, x[:16]), torch.cat([ops.mul_mat(W, x[:8]), ops.mul_mat(W, x[8:16])]))
     W.free()
     W = ops.Q4KWeight.synthetic(5, 4096, 4096)
