@@ -1449,11 +1449,12 @@ template <int NMAT, int WPR, int MT, int WT>
 hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
     const bool odd = ((a.nb / WPR) & 1) != 0;
     const int ranges = odd ? (skinny16_lds_bytes(NMAT, WPR, a.nb, MT, 1) <= kSkinnyLdsMax ? 1 : 0) : skinny16_ranges(NMAT, WPR, a.nb, MT);
-    if constexpr (WT == kWtQ6 && (NMAT == 2 && (MT == 2 || WPR == 1))) {
-        return hipErrorInvalidValue;  // (these Q6_K forms spill registers: skinny16_applies)
+    // (the forms left out below spill registers -- skinny16_applies knows them)
+    if constexpr (WT == kWtQ6 && NMAT == 2 && WPR == 1) {
+        return hipErrorInvalidValue;
     } else if constexpr (MT <= 2) {
         const bool ga = ranges != 1;  // (two tiles could also come in runs; read a stage ahead they cost no barrier)
-        if constexpr (WT != kWtQ4 && NMAT == 2 && MT == 2) {  // (read a stage ahead, two tiles of a Q5_K or Q6_K pair spill registers: skinny16_applies)
+        if constexpr (WT != kWtQ4 && NMAT == 2 && MT == 2) {  // two tiles of a Q5_K or Q6_K pair: not read a stage ahead
             if (ga) return hipErrorInvalidValue;
             if (odd) return launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);
             return launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, 1, stream, start, stop);
@@ -1461,13 +1462,13 @@ hipError_t launch_skinny16_form(const Skinny16Args& a, hipStream_t stream, hipEv
             if (odd) return ga ? launch_skinny16_one<NMAT, WPR, 1, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);
             return ga ? launch_skinny16_one<NMAT, WPR, 0, true, MT, WT>(a, 1, stream, start, stop) : launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, 1, stream, start, stop);
         }
-    } else if constexpr (WPR == 1 || (WT != kWtQ4 && NMAT == 2) || (NMAT == 2 && MT == 4 && WPR == 8)) {
-        return hipErrorInvalidValue;  // (skinny16_applies: not built)
+    } else if constexpr (WPR == 1 || (NMAT == 2 && MT == 4 && WPR == 8)) {
+        return hipErrorInvalidValue;
     } else {
         if (ranges == 0) return hipErrorInvalidValue;
         if (odd) return launch_skinny16_one<NMAT, WPR, 1, false, MT, WT>(a, 1, stream, start, stop);  // (an odd stage count: one run only)
         if ((((a.nb / WPR) / ranges) & 1) == 0) return launch_skinny16_one<NMAT, WPR, 0, false, MT, WT>(a, ranges, stream, start, stop);
-        if constexpr (WT == kWtQ6) return hipErrorInvalidValue;  // (runs of an odd stage count: this form spills registers, skinny16_applies)
+        if constexpr (WT == kWtQ6 || (WT == kWtQ5 && NMAT == 2 && MT == 4)) return hipErrorInvalidValue;  // (runs of an odd stage count)
         else return launch_skinny16_one<NMAT, WPR, 2, false, MT, WT>(a, ranges, stream, start, stop);
     }
 }
@@ -1514,35 +1515,24 @@ hipError_t launch_skinny16_tiles(const Skinny16Args& a, int wpr, hipStream_t str
 // Whether a product of n rows (nine to 64) runs on skinny16_kernel: the wave split of the other decode kernels must be
 // one of its own (a divisor of eight that divides the super-blocks of a row), and the form must be built
 // (launch_skinny16_form returns an error for the others: those whose registers spill).
-//   Q4_K  one and two tiles (up to 32 rows) always; three and four not with one wavefront per row tile (more than 1,024
-//         row tiles: the GEMM is faster there) and where the tiles pass through LDS in at most four runs of whole stages
-//         (in one run where a wavefront's stage count is odd); a gate/up pair of four tiles not with eight wavefronts per
-//         row tile.
-//   Q5_K  single matrices as Q4_K; a pair one tile, two where they fit LDS in one run.
-//   Q6_K  single matrices as Q4_K, three and four tiles not in runs of an odd number of stages; a pair one tile, not
-//         with one wavefront per row tile.
+//   One and two tiles (up to 32 rows): always; the two tiles of a Q5_K or Q6_K gate/up pair only where they fit LDS in
+//   one run; a Q6_K pair not with one wavefront per row tile.
+//   Three and four tiles: not with one wavefront per row tile (more than 1,024 row tiles: the GEMM is faster from 33
+//   rows -- 128256 x 4096 at 33 / 64 rows: 93 / 108 us against 102 / 126); the tiles must pass through LDS in at most four
+//   runs of whole stages (in one run where a wavefront's stage count is odd); a pair of four tiles not with eight
+//   wavefronts per row tile; in runs of an odd number of stages no Q6_K form and no Q5_K pair of four tiles.
 bool skinny16_applies(int64_t nb, int64_t rowtiles, bool swiglu, int64_t n, int wtype) {
     const int wpr = dense_lds_wpr(nb, rowtiles);
     if (!wpr || nb % wpr || n < 1 || n > 64 || (wtype != kTypeQ4K && wtype != kTypeQ5K && wtype != kTypeQ6K)) return false;
-    if (wtype != kTypeQ4K) {
-        if (wtype == kTypeQ6K && swiglu && (wpr == 1 || n > 16)) return false;  // (forms that spill registers)
-        if (n > 32) {  // three and four tiles: single matrices, from LDS
-            if (swiglu || wpr == 1) return false;
-            const int mt = (int)((n + 15) / 16);
-            if ((nb / wpr) & 1) return skinny16_lds_bytes(1, wpr, nb, mt, 1) <= kSkinnyLdsMax;
-            const int ranges = skinny16_ranges(1, wpr, nb, mt);
-            return ranges != 0 && (wtype != kTypeQ6K || (((nb / wpr) / ranges) & 1) == 0);  // (Q6_K: not with runs of an odd stage count, whose form spills registers)
-        }
-        return !(swiglu && n > 16) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
-    }
-    if (n <= 32) return true;
-    // more than 1,024 row tiles (a wavefront per row tile): the matrix-core GEMM is faster from 33 rows (128256 x 4096 at
-    // 33 / 64 rows: 93 / 108 us against 102 / 126 as three and four tiles)
-    if (wpr == 1) return false;
-    if (swiglu && n > 48 && wpr == 8) return false;  // this form of the four-tile pair kernel spills registers
     const int nmat = swiglu ? 2 : 1, mt = (int)((n + 15) / 16);
+    if (wtype == kTypeQ6K && swiglu && wpr == 1) return false;
+    if (mt <= 2) return !(wtype != kTypeQ4K && swiglu && mt == 2) || skinny16_lds_bytes(2, wpr, nb, 2, 1) <= kSkinnyLdsMax;
+    if (wpr == 1 || (swiglu && mt == 4 && wpr == 8)) return false;
     if ((nb / wpr) & 1) return skinny16_lds_bytes(nmat, wpr, nb, mt, 1) <= kSkinnyLdsMax;  // an odd stage count: the tiles in one run
-    return skinny16_ranges(nmat, wpr, nb, mt) != 0;
+    const int ranges = skinny16_ranges(nmat, wpr, nb, mt);
+    if (!ranges) return false;
+    const bool odd_runs = (((nb / wpr) / ranges) & 1) != 0;
+    return !odd_runs || !(wtype == kTypeQ6K || (wtype == kTypeQ5K && swiglu && mt == 4));
 }
 
 hipError_t launch_skinny16(const Skinny16Args& a, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {

@@ -135,7 +135,7 @@ int mq_mul_mat_q4k_noalloc(const mq_weight* w, const float* x_dev, int64_t n, in
                            void* stream);
 /* The same product computed by the matrix-core GEMM kernel whatever n is (mq_mul_mat_q4k switches to it
  * by itself from 48 rows up, from 17 for matrices of 24 MB and more; Q4_K products stay on the decode arithmetic up to
- * 32 rows, up to 64 where their rows pass through LDS in runs of super-blocks, Q5_K products likewise, Q6_K products up to 32 rows): weights are read once per 128 activation rows and the int8 MFMA
+ * 32 rows, up to 64 where their rows pass through LDS in runs of super-blocks, Q5_K and Q6_K products likewise): weights are read once per 128 activation rows and the int8 MFMA
  * units do the arithmetic.  RunQ4KRawBatchedDenseGemm (core/src/backend/cpu_backend_q4k_dense.cpp:57-101),
  * the A.shape[0] >= 4 branch of MatMulGgmlQuantizedTransBWithPath
  * (core/src/backend/cpu_backend_quantized_matmul.cpp:164-170).  Same integers per super-block as
