@@ -65,6 +65,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a 256 MiB device-to-device copy kernel 20 times (the known-size reference for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
+    ap.add_argument("--kernel-only-n16", action="store_true",
+                    help="the same for the n = 16 form of the launch (skinny16_kernel<2,2,...>: the rows as one tile of sixteen)")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only run the back-to-back launches of the dominant kernel (for counter passes) and exit")
     ap.add_argument("--prefill-only", action="store_true",
@@ -219,6 +221,10 @@ def main() -> int:
             a.free()
         return e0.elapsed_time(e1) * 1e3 / (reps * count)     # us per launch
 
+    if args.kernel_only_n16:
+        us = kernel_leg((16,), 5)
+        print(json.dumps({"kernel_only": "skinny16_kernel<2,2,...>", "avg_us": round(us, 3), "widths": (16,)}))
+        return 0
     if args.kernel_only:
         narrow = tuple(n for n in WIDTHS if n <= 8)
         us = kernel_leg(narrow, 5)
